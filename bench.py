@@ -1,0 +1,282 @@
+#!/usr/bin/env python3
+"""Benchmark of the matmul hot path on one MI355X.
+
+Headline workload (BASELINE.json configs[2], the one the north-star target is quoted on):
+  uint8 [4096,4096] (zero-point 128) x int8 [4096,4096] (symmetric) -> int32 accumulate ->
+  requantize to uint8 with scale 1/(K*64), zero-point 128, through the fused kernel
+  (tfcc_rocm_gemm_u8s8s32_requant_u8, int32 accumulators not written).
+One step = one such product with inputs resident in HBM.  value = 2*M*N*K / time, in TOP/s.
+
+The same JSON line carries
+  roofline      the dominant kernel against the int8 MFMA peak (5.0 POP/s dense)
+  cpu_baseline  the reference's own AVX2 quantized matmul + requantize (oracle/_ref, kind
+                "reference") or, where that library is absent, the scalar C oracle (kind "port"),
+                timed on this host's cores on a bounded sample
+  other         the remaining BASELINE configs (fp32 GEMM + bias, attention-shaped batched fp32,
+                skinny int8 decode GEMV, int32-writing variant), each with its own roofline figure
+
+usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-other]
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA
+PEAK_FP32_TFLOPS = 157.3  # MI355X fp32 MFMA
+PEAK_HBM_GBS = 8000.0     # MI355X HBM3E
+
+
+def time_launches(torch, fn, steps, warmup):
+    """Average duration of one call in ms, measured with HIP events on the stream fn launches on."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / steps
+
+
+def c3_setup(torch, pkg, dev, seed=0, size=4096):
+    rng = np.random.default_rng(seed)
+    a = rng.integers(0, 256, (size, size), dtype=np.uint8)
+    b = rng.integers(-127, 128, (size, size), dtype=np.int8)
+    ta, tb = torch.from_numpy(a).to(dev), torch.from_numpy(b).to(dev)
+    rs, cs = pkg.reduce_sum(ta, True), pkg.reduce_sum(tb, False)
+    f1 = lambda v: torch.tensor([v], dtype=torch.float32, device=dev)
+    ranges = [f1(-128.0), f1(127.0), f1(-128.0), f1(127.0)]
+    out_range = [f1(-128.0 * size * 64.0), f1(127.0 * size * 64.0)]
+    return a, b, ta, tb, rs, cs, ranges, out_range
+
+
+def make_c3_step(torch, pkg, ta, tb, rs, cs, ranges, out_range, want_acc):
+    """A closure that launches exactly one fused product into preallocated outputs."""
+    m, k = ta.shape
+    n = tb.shape[1]
+    d = pkg.QGemmDesc()
+    d.a, d.b, d.rowsum_a, d.colsum_b = ta.data_ptr(), tb.data_ptr(), rs.data_ptr(), cs.data_ptr()
+    d.m, d.n, d.k, d.batch, d.stride_c = m, n, k, 1, m * n
+    d.min_a, d.max_a, d.min_b, d.max_b = [r.data_ptr() for r in ranges]
+    mn_c = torch.empty(1, dtype=torch.float32, device=ta.device)
+    mx_c = torch.empty(1, dtype=torch.float32, device=ta.device)
+    d.min_c, d.max_c = mn_c.data_ptr(), mx_c.data_ptr()
+    q = torch.empty((m, n), dtype=torch.uint8, device=ta.device)
+    acc = torch.empty((m, n), dtype=torch.int32, device=ta.device) if want_acc else None
+    lib = pkg.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+    acc_ptr = None if acc is None else acc.data_ptr()
+    keep = (d, mn_c, mx_c, q, acc)
+
+    def step():
+        st = lib.tfcc_rocm_gemm_u8s8s32_requant_u8(stream, C.byref(d), acc_ptr, q.data_ptr(), 0.0, 0.0, 0.0, 0,
+                                                   out_range[0].data_ptr(), out_range[1].data_ptr())
+        if st != 0:
+            pkg.check(st)
+    step.keep = keep
+    step.q = q
+    step.acc = acc
+    return step
+
+
+def cpu_baseline(a, b, size):
+    """The reference's CPU path on this host: its AVX2 quantized matmul (offset matrix + kernel) followed
+    by its AVX2 requantize, both from oracle/_ref; falls back to the scalar C oracle on a smaller sample."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_lib as O
+    cores = len(os.sched_getaffinity(0))
+    threads = int(os.environ.get("OMP_NUM_THREADS", cores))
+    ref = O.ref()
+    ranges = (-128.0, 127.0, -128.0, 127.0)
+    if ref is not None:
+        rs, cs = O.reduce_sum(a, True), O.reduce_sum(b, False)
+        oa, ob = O.qmatmul_offsets(*ranges, lib=ref)
+        mn_c, mx_c = O.qmatmul_range(*ranges, lib=ref)
+        q = np.empty((size, size), np.uint8)
+        O.qgemm(a[:256], b, oa, ob, rs[:256], cs, lib=ref)  # warm the thread pool
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            c = O.qgemm(a, b, oa, ob, rs, cs, lib=ref)
+            ref.ref_requantize_s32_u8(c.reshape(-1), c.size, mn_c, mx_c, -128.0 * size * 64.0, 127.0 * size * 64.0, 1,
+                                      q.reshape(-1))
+            reps += 1
+            dt = time.perf_counter() - t0
+            if dt > 10.0 or reps >= 8:
+                break
+        tops = 2.0 * size ** 3 * reps / dt / 1e12
+        return {"value": round(tops, 4), "unit": "TOP/s", "cores": min(threads, cores), "kind": "reference",
+                "sample": "%d full %d^3 products + requantize through the reference's AVX2 kernels (oracle/_ref), "
+                          "%.1f s, OMP threads %d" % (reps, size, dt, threads)}
+    sub = 1024
+    sa, sb = np.ascontiguousarray(a[:sub, :sub]), np.ascontiguousarray(b[:sub, :sub])
+    t0 = time.perf_counter()
+    c = O.qgemm(sa, sb, -128, 0)
+    O.requantize_s32_u8(c, -2147483648.0, 2147483648.0, -128.0 * sub * 64.0, 127.0 * sub * 64.0)
+    dt = time.perf_counter() - t0
+    return {"value": round(2.0 * sub ** 3 / dt / 1e12, 5), "unit": "TOP/s", "cores": 1, "kind": "port",
+            "sample": "one %d^3 product + requantize through the scalar C oracle, %.1f s" % (sub, dt)}
+
+
+def bench_other(torch, pkg, dev, steps, warmup, c3):
+    """Remaining BASELINE configs; each entry: ms, achieved rate, bound, fraction of the bounding peak."""
+    out = {}
+    rng = np.random.default_rng(1)
+    t = lambda x: torch.from_numpy(np.ascontiguousarray(x)).to(dev)
+    lib = pkg.lib()
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def sgemm_case(name, shape_a, shape_b, bias, sets=4):
+        p = pkg.matmul_plan(shape_a, shape_b, None if not bias else (shape_b[-1],))
+        # several buffer sets so that a small working set does not simply sit in the caches
+        bufs = []
+        for _ in range(sets):
+            a = torch.randn(shape_a, device=dev, dtype=torch.float32)
+            b = torch.randn(shape_b, device=dev, dtype=torch.float32)
+            bi = torch.randn(shape_b[-1], device=dev, dtype=torch.float32) if bias else None
+            c = torch.empty(p["shape"], device=dev, dtype=torch.float32)
+            bufs.append((a, b, bi, c))
+        idx = [0]
+
+        def step():
+            a, b, bi, c = bufs[idx[0] % sets]
+            idx[0] += 1
+            st = lib.tfcc_rocm_sgemm_strided_batched(stream, a.data_ptr(), p["stride_a"], b.data_ptr(), p["stride_b"],
+                                                     None if bi is None else bi.data_ptr(), c.data_ptr(), p["stride_c"],
+                                                     p["m"], p["n"], p["k"], p["batch"])
+            if st != 0:
+                pkg.check(st)
+        ms = time_launches(torch, step, steps, warmup)
+        flop = 2.0 * p["m"] * p["n"] * p["k"] * p["batch"] + (p["m"] * p["n"] * p["batch"] if bias else 0)
+        nbytes = 4.0 * (int(np.prod(shape_a)) + int(np.prod(shape_b)) + int(np.prod(p["shape"])) + (shape_b[-1] if bias else 0))
+        tflops, gbs = flop / ms / 1e9, nbytes / ms / 1e6
+        out[name] = {"ms": round(ms, 5), "tflops": round(tflops, 3), "frac_fp32_mfma": round(tflops / PEAK_FP32_TFLOPS, 4),
+                     "gbs": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4)}
+
+    sgemm_case("c1_fp32_128x768x3072_bias", (128, 768), (768, 3072), True)
+    sgemm_case("c2_fp32_qk_16x12x128x64x128", (16, 12, 128, 64), (16, 12, 64, 128), False)
+    sgemm_case("c2_fp32_pv_16x12x128x128x64", (16, 12, 128, 128), (16, 12, 128, 64), False)
+    sgemm_case("c4_fp32_ffn_up_1024x768x3072_bias", (8, 128, 768), (768, 3072), True)
+    sgemm_case("fp32_4096x4096x4096", (4096, 4096), (4096, 4096), False, sets=1)
+
+    # C3 with the int32 accumulators also written (67 MB more traffic)
+    a, b, ta, tb, rs, cs, ranges, out_range = c3
+    step = make_c3_step(torch, pkg, ta, tb, rs, cs, ranges, out_range, want_acc=True)
+    ms = time_launches(torch, step, steps, warmup)
+    tops = 2.0 * 4096 ** 3 / ms / 1e9
+    out["c3_int8_4096_requant_plus_int32_out"] = {"ms": round(ms, 5), "tops": round(tops, 2),
+                                                  "frac_int8_mfma": round(tops / PEAK_INT8_TOPS, 4)}
+
+    # C5: skinny decode shapes, B streamed once; rotate B buffers larger than the last-level cache
+    n, k = 11008, 4096
+    sets = 8
+    bs = [t(rng.integers(-127, 128, (k, n), dtype=np.int8)) for _ in range(sets)]
+    css = [pkg.reduce_sum(x, False) for x in bs]
+    scale_b = t(rng.uniform(0.001, 0.01, n).astype(np.float32))
+    for m in (1, 4, 8):
+        am = t(rng.integers(0, 256, (m, k), dtype=np.uint8))
+        rsm = pkg.reduce_sum(am, True)
+        acc = torch.empty((m, n), dtype=torch.int32, device=dev)
+        f32 = torch.empty((m, n), dtype=torch.float32, device=dev)
+        idx = [0]
+
+        def step():
+            i = idx[0] % sets
+            idx[0] += 1
+            st = lib.tfcc_rocm_gemv_u8s8s32(stream, am.data_ptr(), bs[i].data_ptr(), rsm.data_ptr(), css[i].data_ptr(),
+                                            -128, 0, m, n, k, acc.data_ptr(), 0.02, scale_b.data_ptr(), f32.data_ptr())
+            if st != 0:
+                pkg.check(st)
+        ms = time_launches(torch, step, max(steps, 50), warmup)
+        nbytes = k * n + m * k + 4 * n + 4 * m * n  # B + A + scales + fp32 out (algorithmic)
+        gbs = nbytes / ms / 1e6
+        out["c5_int8_gemv_m%d_4096x11008" % m] = {"ms": round(ms, 5), "gbs": round(gbs, 1),
+                                                   "frac_hbm": round(gbs / PEAK_HBM_GBS, 4),
+                                                   "gops": round(2.0 * m * n * k / ms / 1e6, 1)}
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-other", action="store_true", help="skip the secondary configs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: the matmul path has no multi-GPU part (run with --gpus 1)")
+
+    import torch
+    from __graft_entry__ import load_package
+    pkg = load_package()
+    pkg.lib()
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    size = 4096
+    c3 = c3_setup(torch, pkg, dev, seed=0, size=size)
+    a, b, ta, tb, rs, cs, ranges, out_range = c3
+    step = make_c3_step(torch, pkg, ta, tb, rs, cs, ranges, out_range, want_acc=False)
+
+    # warmup, then exactly K timed steps between synchronisation points
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for _ in range(args.steps):
+        step()
+    stop.record()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    kernel_ms = start.elapsed_time(stop) / args.steps  # HIP events on the launch stream
+    ops = 2.0 * size ** 3
+    tops = ops / wall_ms / 1e9
+    kernel_tops = ops / kernel_ms / 1e9
+
+    result = {
+        "metric": "int8 matmul TOPS (u8 x s8 -> s32 -> requantized u8, M=N=K=4096)",
+        "value": round(tops, 2),
+        "unit": "TOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8 (int32 accumulate, fp64 requantize)",
+        "data": "synthetic (seeded uniform uint8 / int8, resident in HBM)",
+        "config": {"workload": "BASELINE configs[2]: A u8[4096,4096] zp 128 x B s8[4096,4096] symmetric -> "
+                               "int32 -> requantize u8, scale 1/(K*64), zp 128; fused kernel, uint8 output only",
+                   "m": size, "n": size, "k": size},
+        "roofline": {"bound": "mfma", "achieved": round(kernel_tops, 2), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
+                     "frac": round(kernel_tops / PEAK_INT8_TOPS, 4), "traffic": None,
+                     "kernel": "qgemm_kernel<256,256,64,aligned,requant>", "kernel_ms": round(kernel_ms, 5),
+                     "algorithmic_ops_per_launch": ops},
+    }
+    traffic_file = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(traffic_file):
+        result["roofline"]["traffic"] = json.load(open(traffic_file)).get("qgemm_c3_bytes_per_launch")
+    if not args.no_other:
+        result["other"] = bench_other(torch, pkg, dev, max(10, args.steps // 2), args.warmup, c3)
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(a, b, size)
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,194 @@
+/*
+ * tfcc_rocm.h -- C ABI of the MI355X (gfx950) matmul backend for TFCC.
+ *
+ * This is the only boundary between the host side (the C++ TFCC device/interface layer, or any
+ * FFI: ctypes, cgo, JNI) and the hand-written HIP kernels in libtfcc_rocm.so.  Plain pointers and
+ * sizes only.  All tensor pointers are DEVICE pointers to row-major, contiguous data unless a
+ * parameter says "host".  `stream` is a hipStream_t passed as void* (NULL = the default stream);
+ * every compute entry point only enqueues work on it and returns.
+ *
+ * Return value: 0 on success, otherwise a TFCC_ROCM_* code; tfcc_rocm_last_error_string() gives
+ * the text of the last failure on the calling thread.
+ *
+ * Each entry point names the reference function (file:line under the reference root) it replaces.
+ */
+#ifndef TFCC_ROCM_H_
+#define TFCC_ROCM_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  TFCC_ROCM_OK = 0,
+  TFCC_ROCM_INVALID_ARGUMENT = 1, /* bad pointer / size / type code: nothing was launched */
+  TFCC_ROCM_HIP_ERROR = 2,        /* a HIP runtime call failed */
+  TFCC_ROCM_OUT_OF_MEMORY = 3,    /* device allocation failed */
+  TFCC_ROCM_NO_DEVICE = 4,        /* no usable GPU */
+};
+
+/* element type codes for the type-generic quantization entry points */
+enum {
+  TFCC_ROCM_S8 = 0,
+  TFCC_ROCM_U8 = 1,
+  TFCC_ROCM_S16 = 2,
+  TFCC_ROCM_U16 = 3,
+  TFCC_ROCM_S32 = 4,
+  TFCC_ROCM_U32 = 5,
+};
+
+const char* tfcc_rocm_last_error_string(void);
+/* "tfcc_rocm <version> gfx950" */
+const char* tfcc_rocm_version(void);
+
+/* ---------------------------------------------------------------------------------------------
+ * Device, stream and memory plumbing.  Replaces what the reference's GPU device/session do with
+ * the CUDA runtime: tfcc/cuda/framework/tfcc_cudadevice.cpp:30-55 (memory limit, allocator
+ * hooks), tfcc/cuda/framework/tfcc_cudasession.cpp:36-63 (stream), and the copies of
+ * tfcc/cuda/interfaces/tfcc_cudadatainterface.cu:62-97.
+ * ------------------------------------------------------------------------------------------- */
+int tfcc_rocm_device_count(int* count);
+int tfcc_rocm_set_device(int device);
+int tfcc_rocm_mem_info(size_t* free_bytes, size_t* total_bytes);
+int tfcc_rocm_device_name(char* buf, size_t len);
+int tfcc_rocm_malloc(void** ptr, size_t bytes);
+int tfcc_rocm_free(void* ptr);
+int tfcc_rocm_stream_create(void** stream);
+int tfcc_rocm_stream_destroy(void* stream);
+int tfcc_rocm_stream_synchronize(void* stream);
+/* host<->device copies: synchronise the stream, then copy synchronously (reference semantics) */
+int tfcc_rocm_memcpy_h2d(void* stream, void* dst_device, const void* src_host, size_t bytes);
+int tfcc_rocm_memcpy_d2h(void* stream, void* dst_host, const void* src_device, size_t bytes);
+int tfcc_rocm_memcpy_d2d_async(void* stream, void* dst, const void* src, size_t bytes);
+/* fill `count` elements of `elem_size` (1, 2, 4 or 8) bytes with the bit pattern `value` */
+int tfcc_rocm_fill_async(void* stream, void* dst, uint64_t value, int elem_size, size_t count);
+
+/* ---------------------------------------------------------------------------------------------
+ * fp32 matmul.
+ * Replaces _call_matmul_wrapper / _call_matmul_with_beta_wrapper + _mkl_set_bias_wrapper,
+ * tfcc/mkl/interfaces/tfcc_mklblasinterface.cpp:41-67, 69-78, 87-118 (same argument meaning:
+ * batch strides in elements, 0 = operand shared by every batch; bias[n] or NULL).
+ *   C[b] (m x n) = A[b] (m x k) * B[b] (k x n) (+ bias broadcast over rows)
+ * ------------------------------------------------------------------------------------------- */
+int tfcc_rocm_sgemm_strided_batched(void* stream, const float* a, uint64_t stride_a,
+                                    const float* b, uint64_t stride_b, const float* bias, float* c,
+                                    uint64_t stride_c, unsigned m, unsigned n, unsigned k,
+                                    unsigned batch);
+
+/* ---------------------------------------------------------------------------------------------
+ * Quantized uint8 x int8 -> int32 matmul.
+ * Replaces _mkl_create_offset_matrix + _MKLQuantizationMatmulAVX256::quantizedMatmulColMajor,
+ * tfcc/mkl/operations/tfcc_mklquantization.cpp:33-69,176-201 and
+ * tfcc/mkl/kernel/tfcc_mklquantizationmatmul.avx256.h:27-29:
+ *   C[b][i][j] = k*oA*oB + rowsum_a[b][i]*oB + colsum_b[b][j]*oA + sum_p A[b][i][p]*B[b][p][j]
+ * in wrap-around int32.  rowsum_a / colsum_b are the caller's tensors (as in the reference they
+ * are used as given); strides in elements, 0 = shared by all batches.
+ * ------------------------------------------------------------------------------------------- */
+typedef struct tfcc_rocm_qgemm_desc {
+  const uint8_t* a;        /* [batch] m x k */
+  const int8_t* b;         /* [batch] k x n */
+  const int32_t* rowsum_a; /* [batch] m */
+  const int32_t* colsum_b; /* [batch] n */
+  uint64_t stride_a, stride_b, stride_rowsum_a, stride_colsum_b, stride_c;
+  unsigned m, n, k, batch;
+  /* Offsets: either immediate ... */
+  int32_t offset_a, offset_b;
+  /* ... or derived on the device from float ranges in device memory (all four non-NULL), exactly
+   * as tfcc/mkl/operations/tfcc_mklquantization.cpp:181-186 does; then min_c / max_c (device,
+   * may be NULL) receive the int32 result's range (tfcc/core/utils/tfcc_quantizationutils.h:30-43). */
+  const float *min_a, *max_a, *min_b, *max_b;
+  float *min_c, *max_c;
+} tfcc_rocm_qgemm_desc;
+
+/* int32 result only */
+int tfcc_rocm_gemm_u8s8s32(void* stream, const tfcc_rocm_qgemm_desc* desc, int32_t* c);
+
+/*
+ * Same product with the requantize step fused into the tile store: replaces the separate pass
+ * _MKLRequantizationKernelAVX256<int32_t, uint8_t>::requantize
+ * (tfcc/mkl/kernel/tfcc_mklquantizationkernel.avx256.cpp:120-145; fused multiply-add and
+ * round-to-nearest-even as that kernel is built).  acc_out may be NULL (int32 not written).
+ * Scalars as _requantize_helper computes them (tfcc/mkl/interfaces/tfcc_mklquantizationinterface.cpp:125-130):
+ *   in_scale, in_min = get_dequantized_scale_info<int32_t>(minC, maxC)
+ *   out_scale, out_offset = get_quantized_scale_info<uint8_t>(minOut, maxOut)
+ * If min_out / max_out (device pointers) are both non-NULL the four scalars are instead derived
+ * on the device from the result range and *min_out / *max_out; this form needs the desc's float
+ * ranges.  Degenerate ranges follow tfcc_mklquantizationinterface.cpp:121-139.
+ */
+int tfcc_rocm_gemm_u8s8s32_requant_u8(void* stream, const tfcc_rocm_qgemm_desc* desc,
+                                      int32_t* acc_out, uint8_t* q_out, double in_scale,
+                                      double in_min, double out_scale, int64_t out_offset,
+                                      const float* min_out, const float* max_out);
+
+/*
+ * Skinny (m <= 8) product for decode shapes, HBM-bandwidth bound; single B shared by the batch of
+ * rows (batch folded into m as tfcc_mklquantization.cpp:140-145 does).  Same int32 arithmetic as
+ * above; the reference has no dedicated kernel for this shape (it takes the general path).
+ * Optional fused per-output-channel dequantize (no counterpart in the reference, which only has
+ * per-tensor ranges): f32_out[i][j] = (float)((double)acc[i][j] * ((double)scale_a * (double)scale_b[j])).
+ * acc_out and f32_out may each be NULL, not both.
+ */
+int tfcc_rocm_gemv_u8s8s32(void* stream, const uint8_t* a, const int8_t* b,
+                           const int32_t* rowsum_a, const int32_t* colsum_b, int32_t offset_a,
+                           int32_t offset_b, unsigned m, unsigned n, unsigned k, int32_t* acc_out,
+                           float scale_a, const float* scale_b, float* f32_out);
+
+/*
+ * Row sums (out [batch][row]) and column sums (out [batch][col]) in int32.
+ * Replaces _mkl_reduce_sum_row / _mkl_reduce_sum_column,
+ * tfcc/mkl/operations/tfcc_mklquantization.cpp:205-237, 239-282.  type: TFCC_ROCM_S8 / U8 / S16.
+ */
+int tfcc_rocm_reduce_sum_rows(void* stream, const void* a, int type, unsigned batch, unsigned row,
+                              unsigned col, int32_t* out);
+int tfcc_rocm_reduce_sum_cols(void* stream, const void* a, int type, unsigned batch, unsigned row,
+                              unsigned col, int32_t* out);
+
+/* ---------------------------------------------------------------------------------------------
+ * Range-based quantize / requantize / dequantize (per tensor).
+ * Replaces _MKLRequantizationKernelAVX256::requantize, _MKLQuantizationKernelAVX256::quantize /
+ * dequantize (tfcc/mkl/kernel/tfcc_mklquantizationkernel.avx256.cpp:55-145) and the range logic of
+ * tfcc/mkl/interfaces/tfcc_mklquantizationinterface.cpp:47-69, 72-147, 150-240, 284-333.
+ * All ranges are float scalars in DEVICE memory (as the reference passes them as tensors); the
+ * scale/offset arithmetic (tfcc/core/utils/tfcc_quantizationutils.h:45-70) runs on the device in
+ * double, so nothing synchronises with the host.
+ * ------------------------------------------------------------------------------------------- */
+int tfcc_rocm_requantize(void* stream, const void* in, int in_type, void* out, int out_type,
+                         uint64_t total, const float* min_in, const float* max_in,
+                         const float* min_out, const float* max_out);
+int tfcc_rocm_dequantize(void* stream, const void* in, int in_type, uint64_t total,
+                         const float* min_v, const float* max_v, float* out);
+int tfcc_rocm_quantize(void* stream, const float* in, uint64_t total, const float* min_v,
+                       const float* max_v, void* out, int out_type);
+/* quantize with the range taken from the data: writes *min_v / *max_v (device) first */
+int tfcc_rocm_quantize_minmax(void* stream, const float* in, uint64_t total, void* out,
+                              int out_type, float* min_v, float* max_v);
+
+/* ---------------------------------------------------------------------------------------------
+ * The element-wise neighbours of matmul inside one transformer encoder layer (fp32).
+ * ------------------------------------------------------------------------------------------- */
+/* softmax over the last axis: _MKLActivationKernel::softmaxV2, tfcc/mkl/kernel/tfcc_mklactivationkernel.hpp:137-155 */
+int tfcc_rocm_softmax_f32(void* stream, const float* in, uint64_t rows, unsigned cols, float* out);
+/* _mkl_layer_normalize, tfcc/mkl/interfaces/tfcc_mklnormalizationinterface.cpp:29-62 */
+int tfcc_rocm_layer_norm_f32(void* stream, const float* in, const float* gamma, const float* beta,
+                             float epsilon, uint64_t rows, unsigned cols, float* out);
+/* _MKLActivationKernel::geluAccurate, tfcc/mkl/kernel/tfcc_mklactivationkernel.hpp:213-220 */
+int tfcc_rocm_gelu_accurate_f32(void* stream, const float* in, uint64_t total, float* out);
+/* out = a * alpha + beta: TransformationInterface::transform, tfcc/core/operations/tfcc_operator.cpp:78-95 */
+int tfcc_rocm_transform_f32(void* stream, const float* in, uint64_t total, float alpha, float beta,
+                            float* out);
+/* out[i] = a[i] + b[i % period] (period == total: plain add; period < total: trailing-dims
+ * broadcast of b).  ArithmeticInterface::add, tfcc/core/interfaces/tfcc_arithmeticinterface.h:34-49 */
+int tfcc_rocm_add_f32(void* stream, const float* a, const float* b, uint64_t total,
+                      uint64_t period, float* out);
+/* rank <= 6 permutation: BasicInterface::transpose, tfcc/core/operations/tfcc_base.cpp:124-134.
+ * shape / perm are HOST arrays of length rank. */
+int tfcc_rocm_transpose_f32(void* stream, const float* in, const unsigned* shape,
+                            const unsigned* perm, int rank, float* out);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TFCC_ROCM_H_ */

@@ -1,0 +1,363 @@
+"""GPU parity tests: every compute entry point of the C ABI against the CPU oracle and the committed
+outputs of the reference's own kernels.  Integer and byte results must be bit-exact; fp32 matmul
+must be within a relative Frobenius error of 1e-5 of the float64 result."""
+import hashlib
+import json
+import os
+
+import numpy as np
+import pytest
+
+import oracle_lib as O
+from golden.make_golden import BENCH_RANGES, SMALL_CASES, bench_out_range, gen_inputs
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+FP32_TOL = 1e-5  # relative Frobenius error allowed for fp32 matmul
+
+
+def wrap32(x):
+    return (np.asarray(x, np.int64) & 0xFFFFFFFF).astype(np.uint32).view(np.int32)
+
+
+@pytest.fixture(scope="module")
+def T(dev):
+    import torch
+
+    class Helper:
+        def t(self, x):
+            return torch.from_numpy(np.ascontiguousarray(x)).to(dev)
+
+        def f1(self, v):
+            return torch.tensor([v], dtype=torch.float32, device=dev)
+
+        def n(self, x):
+            torch.cuda.synchronize()
+            return x.cpu().numpy()
+    return Helper()
+
+
+def rel_fro(got, want64):
+    return np.linalg.norm(got.astype(np.float64) - want64) / max(np.linalg.norm(want64), 1e-300)
+
+
+# ---- quantized matmul ----------------------------------------------------------------------------
+
+@pytest.mark.parametrize("seed,shape_a,shape_b", SMALL_CASES)
+def test_qgemm_golden_vectors(pkg, T, seed, shape_a, shape_b):
+    """All shape families (matrix, batched x batched, batched x matrix, matrix x batched, N == 1)
+    with float ranges in device memory, against the reference kernel's stored outputs."""
+    print("case", seed, shape_a, shape_b, flush=True)
+    z = np.load(os.path.join(GOLDEN, "qgemm_ref_vectors.npz"))
+    p = "case%d/" % seed
+    a, b = z[p + "a"], z[p + "b"]
+    ranges = [float(v) for v in z[p + "ranges"]]
+    rs, cs = O.reduce_sum(a, True), O.reduce_sum(b, False)
+    r = [T.f1(v) for v in ranges]
+    c, mn_c, mx_c = pkg.quantization_matmul(T.t(a), T.t(rs), r[0], r[1], T.t(b), T.t(cs), r[2], r[3])
+    assert np.array_equal(T.n(c), z[p + "c"])
+    assert (float(T.n(mn_c)[0]), float(T.n(mx_c)[0])) == O.qmatmul_range(*ranges)
+    mn_o, mx_o = [float(v) for v in z[p + "out_range"]]
+    q, c2, _, _ = pkg.quantization_matmul_requantize(T.t(a), T.t(rs), r[0], r[1], T.t(b), T.t(cs), r[2], r[3],
+                                                     T.f1(mn_o), T.f1(mx_o), want_acc=True)
+    assert np.array_equal(T.n(c2), z[p + "c"])
+    assert np.array_equal(T.n(q), z[p + "q"])
+    q_only, none, _, _ = pkg.quantization_matmul_requantize(T.t(a), T.t(rs), r[0], r[1], T.t(b), T.t(cs), r[2],
+                                                            r[3], T.f1(mn_o), T.f1(mx_o), want_acc=False)
+    assert none is None and np.array_equal(T.n(q_only), z[p + "q"])
+    # the stand-alone requantize pass gives the same bytes
+    q_sep = pkg.requantize(c, mn_c, mx_c, T.f1(mn_o), T.f1(mx_o), __import__("torch").uint8)
+    assert np.array_equal(T.n(q_sep), z[p + "q"])
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 1, 1), (1, 16, 16), (5, 7, 3), (31, 33, 15), (64, 64, 64), (100, 260, 72),
+                                   (257, 129, 130), (128, 128, 2048), (300, 516, 1040), (512, 768, 256),
+                                   (1000, 1012, 1040), (2048, 2048, 512), (768, 4096, 1024)])
+def test_qgemm_shapes_against_oracle(pkg, T, m, n, k):
+    """Ragged, unaligned, tail-in-K and multi-tile shapes; both tile configurations and the
+    unaligned path are exercised.  Offsets wrap around int32 on purpose in one case."""
+    print("shape", m, n, k, flush=True)
+    rng = np.random.default_rng(m * 7 + n * 3 + k)
+    a = rng.integers(0, 256, (m, k), dtype=np.uint8)
+    b = rng.integers(-128, 128, (k, n), dtype=np.int8)
+    rs, cs = O.reduce_sum(a, True), O.reduce_sum(b, False)
+    for oa, ob in ((-128, 0), (-57, 93), (70000, -90000)):
+        want = O.qgemm(a, b, oa, ob, rs, cs)
+        got = pkg.quantization_matmul_offsets(T.t(a), T.t(rs), T.t(b), T.t(cs), oa, ob)
+        assert np.array_equal(T.n(got), want), (oa, ob)
+
+
+def test_qgemm_uses_caller_sums_as_given(pkg, T):
+    """rowsum / colsum tensors that are NOT the true sums, and a rank-1 sum shared by a batch."""
+    rng = np.random.default_rng(5)
+    a = rng.integers(0, 256, (3, 70, 48), dtype=np.uint8)
+    b = rng.integers(-128, 128, (3, 48, 36), dtype=np.int8)
+    rs = rng.integers(-10000, 10000, 70).astype(np.int32)      # rank 1: shared by the batch
+    cs = rng.integers(-10000, 10000, (3, 36)).astype(np.int32)
+    oa, ob = -31, 17
+    want = wrap32(48 * oa * ob + rs[None, :, None].astype(np.int64) * ob + cs[:, None, :].astype(np.int64) * oa +
+                  np.matmul(a.astype(np.int64), b.astype(np.int64)))
+    assert np.array_equal(O.qgemm(a, b, oa, ob, rs, cs), want)
+    got = pkg.quantization_matmul_offsets(T.t(a), T.t(rs), T.t(b), T.t(cs), oa, ob)
+    assert np.array_equal(T.n(got), want)
+
+
+@pytest.mark.parametrize("name", ["c3_1024_ragged", "c3_4096"])
+def test_qgemm_full_size_hash(pkg, T, name):
+    """The benchmark configuration at full size: SHA-256 of the int32 accumulators and of the fused
+    uint8 output against the reference kernel's (int32 matmul + AVX2 requantize) on the same seeded inputs."""
+    print("hash case", name, flush=True)
+    h = json.load(open(os.path.join(GOLDEN, "qgemm_ref_hashes.json")))[name]
+    a, b = gen_inputs(h["seed"], h["shape_a"], h["shape_b"])
+    rs, cs = O.reduce_sum(a, True), O.reduce_sum(b, False)
+    r = [T.f1(v) for v in h["ranges"]]
+    mn_o, mx_o = h["out_range"]
+    q, c, _, _ = pkg.quantization_matmul_requantize(T.t(a), T.t(rs), r[0], r[1], T.t(b), T.t(cs), r[2], r[3],
+                                                    T.f1(mn_o), T.f1(mx_o), want_acc=True)
+    assert hashlib.sha256(T.n(c).tobytes()).hexdigest() == h["sha256_c"]
+    assert hashlib.sha256(T.n(q).tobytes()).hexdigest() == h["sha256_q"]
+    q2, _, _, _ = pkg.quantization_matmul_requantize(T.t(a), T.t(rs), r[0], r[1], T.t(b), T.t(cs), r[2], r[3],
+                                                     T.f1(mn_o), T.f1(mx_o), want_acc=False)
+    assert hashlib.sha256(T.n(q2).tobytes()).hexdigest() == h["sha256_q"]
+    # sums computed on the device equal the oracle's
+    assert np.array_equal(T.n(pkg.reduce_sum(T.t(a), True)), rs)
+    assert np.array_equal(T.n(pkg.reduce_sum(T.t(b), False)), cs)
+
+
+def test_qgemm_requant_immediate_scalars(pkg, T):
+    """The fused kernel with host-computed scalars (the kernel-level form of the C ABI)."""
+    import ctypes as C
+    import torch
+    rng = np.random.default_rng(6)
+    m, n, k = 300, 260, 200
+    a = rng.integers(0, 256, (m, k), dtype=np.uint8)
+    b = rng.integers(-128, 128, (k, n), dtype=np.int8)
+    rs, cs = O.reduce_sum(a, True), O.reduce_sum(b, False)
+    oa, ob = O.qmatmul_offsets(*BENCH_RANGES)
+    want_c = O.qgemm(a, b, oa, ob, rs, cs)
+    mn_c, mx_c = O.qmatmul_range(*BENCH_RANGES)
+    mn_o, mx_o = bench_out_range(k)
+    want_q = O.requantize_s32_u8(want_c, mn_c, mx_c, mn_o, mx_o)
+    in_s, in_m = O.dequantized_scale_info(32, mn_c, mx_c)
+    out_s, out_o = O.quantized_scale_info(8, mn_o, mx_o)
+    ta, tb, trs, tcs = T.t(a), T.t(b), T.t(rs), T.t(cs)
+    d = pkg.QGemmDesc()
+    d.a, d.b, d.rowsum_a, d.colsum_b = ta.data_ptr(), tb.data_ptr(), trs.data_ptr(), tcs.data_ptr()
+    d.m, d.n, d.k, d.batch, d.stride_c = m, n, k, 1, m * n
+    d.offset_a, d.offset_b = oa, ob
+    q = torch.empty((m, n), dtype=torch.uint8, device=ta.device)
+    pkg.check(pkg.lib().tfcc_rocm_gemm_u8s8s32_requant_u8(torch.cuda.current_stream().cuda_stream, C.byref(d), None,
+                                                           q.data_ptr(), in_s, in_m, out_s, out_o, None, None))
+    assert np.array_equal(T.n(q), want_q)
+
+
+# ---- skinny (decode) shapes -------------------------------------------------------------------------
+
+@pytest.mark.parametrize("m", [1, 4, 8])
+@pytest.mark.parametrize("n,k", [(11008, 4096), (128, 64), (260, 80), (4096, 4000)])
+def test_gemv_against_oracle(pkg, T, m, n, k):
+    print("gemv", m, n, k, flush=True)
+    rng = np.random.default_rng(m + n + k)
+    a = rng.integers(0, 256, (m, k), dtype=np.uint8)
+    b = rng.integers(-127, 128, (k, n), dtype=np.int8)
+    rs, cs = O.reduce_sum(a, True), O.reduce_sum(b, False)
+    scale_b = rng.uniform(0.001, 0.01, n).astype(np.float32)
+    scale_a = float(np.float32(0.02))
+    for oa, ob in ((-128, 0), (-57, 93)):
+        want = O.qgemm(a, b, oa, ob, rs, cs)
+        out, acc = pkg.gemv_dequant(T.t(a), T.t(b), T.t(rs), T.t(cs), oa, ob, scale_a, T.t(scale_b))
+        assert np.array_equal(T.n(acc), want), (oa, ob)
+        assert np.array_equal(T.n(out), O.dequant_per_channel(want, scale_a, scale_b))
+        # second call in a row reuses the workspace and the tickets
+        out2, _ = pkg.gemv_dequant(T.t(a), T.t(b), T.t(rs), T.t(cs), oa, ob, scale_a, T.t(scale_b), want_acc=False)
+        assert np.array_equal(T.n(out2), T.n(out))
+    # the general entry point routes these shapes to the same kernel
+    got = pkg.quantization_matmul_offsets(T.t(a), T.t(rs), T.t(b), T.t(cs), -128, 0)
+    assert np.array_equal(T.n(got), O.qgemm(a, b, -128, 0, rs, cs))
+
+
+def test_gemv_full_size_hash(pkg, T):
+    h = json.load(open(os.path.join(GOLDEN, "qgemm_ref_hashes.json")))["c5_m8"]
+    a, b = gen_inputs(h["seed"], h["shape_a"], h["shape_b"])
+    rs, cs = O.reduce_sum(a, True), O.reduce_sum(b, False)
+    _, acc = pkg.gemv_dequant(T.t(a), T.t(b), T.t(rs), T.t(cs), h["offsets"][0], h["offsets"][1], 1.0, None)
+    assert hashlib.sha256(T.n(acc).tobytes()).hexdigest() == h["sha256_c"]
+
+
+# ---- sums, quantize, requantize, dequantize ----------------------------------------------------------
+
+@pytest.mark.parametrize("shape", [(1, 1), (17, 29), (3, 64, 256), (2, 100, 1000), (4096, 512), (5, 7, 16)])
+def test_reduce_sum(pkg, T, shape):
+    rng = np.random.default_rng(sum(shape))
+    for x in (rng.integers(0, 256, shape, dtype=np.uint8), rng.integers(-128, 128, shape, dtype=np.int8)):
+        assert np.array_equal(T.n(pkg.reduce_sum(T.t(x), True)), O.reduce_sum(x, True))
+        assert np.array_equal(T.n(pkg.reduce_sum(T.t(x), False)), O.reduce_sum(x, False))
+
+
+def test_requantize_known_answer_and_fma_cases(pkg, T):
+    import torch
+    # tfcc/test/quantization.cpp:88-101 (int8 -> uint16; torch has no uint16 arithmetic: use int16 storage)
+    a = np.array([23, -115, -128, 127, -20, -11], np.int8)
+    ta = T.t(a)
+    out = torch.empty(6, dtype=torch.int16, device=ta.device)
+    pkg.check(pkg.lib().tfcc_rocm_requantize(torch.cuda.current_stream().cuda_stream, ta.data_ptr(), pkg.S8,
+                                              out.data_ptr(), pkg.U16, 6, T.f1(-2.5).data_ptr(), T.f1(3.4).data_ptr(),
+                                              T.f1(-12.7).data_ptr(), T.f1(24.5).data_ptr()))
+    assert T.n(out).view(np.uint16).tolist() == [24125, 18500, 17970, 28364, 22372, 22739]
+    # inputs on which the fused multiply-add decides: outputs of the reference's AVX2 kernel
+    for c in json.load(open(os.path.join(GOLDEN, "requantize_fma_cases.json")))["cases"]:
+        acc = np.asarray(c["acc"], np.int32)
+        got = pkg.requantize(T.t(acc), T.f1(c["minIn"]), T.f1(c["maxIn"]), T.f1(c["minOut"]), T.f1(c["maxOut"]),
+                             torch.uint8)
+        assert T.n(got).tolist() == c["ref_avx2"]
+
+
+def test_requantize_against_oracle(pkg, T):
+    import torch
+    rng = np.random.default_rng(40)
+    for total in (1, 3, 4, 1000, 4099, 1 << 16):
+        acc = rng.integers(-2 ** 31, 2 ** 31, total).astype(np.int32)
+        for (mi, ma, mo, mxo) in ((-1000.0, 1000.0, -300.0, 310.0), (-2147483648.0, 2147483648.0, -33554432.0, 33292288.0),
+                                  (-1.0, 1.0, 2.0, 2.0), (1.5, 1.5, -4.0, 4.0), (-3.0, 5.0, 0.5, -0.5)):
+            got = pkg.requantize(T.t(acc), T.f1(mi), T.f1(ma), T.f1(mo), T.f1(mxo), torch.uint8)
+            assert np.array_equal(T.n(got), O.requantize_s32_u8(acc, mi, ma, mo, mxo)), (total, mi, ma, mo, mxo)
+    # ties: nearest-even like the reference's AVX2 kernel
+    a8 = np.arange(-128, 128).astype(np.int8)
+    out = torch.empty(256, dtype=torch.int16, device=T.t(a8).device)
+    ta = T.t(a8)
+    pkg.check(pkg.lib().tfcc_rocm_requantize(torch.cuda.current_stream().cuda_stream, ta.data_ptr(), pkg.S8,
+                                              out.data_ptr(), pkg.U16, 256, T.f1(-128.0).data_ptr(),
+                                              T.f1(127.0).data_ptr(), T.f1(-65535.0).data_ptr(), T.f1(65535.0).data_ptr()))
+    assert np.array_equal(T.n(out).view(np.uint16), O.requantize_s8_u16(a8, -128.0, 127.0, -65535.0, 65535.0))
+
+
+def test_dequantize_and_quantize_against_oracle(pkg, T):
+    import torch
+    rng = np.random.default_rng(41)
+    a = np.array([23, -115, -128, 127, -20, -11], np.int8)
+    got = T.n(pkg.dequantize(T.t(a), T.f1(-2.5), T.f1(3.4)))
+    assert np.array_equal(got, O.dequantize(a, -2.5, 3.4))
+    q = rng.integers(-2 ** 31, 2 ** 31, 5000).astype(np.int32)
+    assert np.array_equal(T.n(pkg.dequantize(T.t(q), T.f1(-3.25), T.f1(7.5))), O.dequantize(q, -3.25, 7.5))
+    assert np.array_equal(T.n(pkg.dequantize(T.t(q), T.f1(3.0), T.f1(3.0))), np.full(5000, 3.0, np.float32))
+    u = rng.integers(0, 256, 777, dtype=np.uint8)
+    assert np.array_equal(T.n(pkg.dequantize(T.t(u), T.f1(-1.0), T.f1(2.0))), O.dequantize(u, -1.0, 2.0))
+    x = rng.uniform(-5, 5, 4097).astype(np.float32)
+    x[:50] = np.float32(np.arange(50) * 0.5 - 12)
+    for dtype, tdt in ((np.uint8, torch.uint8), (np.int8, torch.int8)):
+        for mn, mx in ((-5.0, 5.0), (-8.0, 7.9375), (3.0, 3.0)):
+            got = pkg.quantize(T.t(x), tdt, T.f1(mn), T.f1(mx))
+            assert np.array_equal(T.n(got), O.quantize(x, mn, mx, dtype))
+        got, mn_t, mx_t = pkg.quantize(T.t(x), tdt)
+        mn, mx = float(x.min()), float(x.max())
+        assert (float(T.n(mn_t)[0]), float(T.n(mx_t)[0])) == (mn, mx)
+        assert np.array_equal(T.n(got), O.quantize(x, mn, mx, dtype))
+    const = np.full(100, 1.25, np.float32)
+    got, _, _ = pkg.quantize(T.t(const), torch.int8)
+    assert np.array_equal(T.n(got), np.full(100, -128, np.int8))
+
+
+def test_quantized_matmul_round_trip(pkg, T):
+    """tfcc/test/quantization.cpp:105-189: quantize -> reduce_sum -> matmul -> dequantize gives 5, 11, 17."""
+    import torch
+    for shape_a, shape_b in (((2, 3, 2), (2, 2, 1)), ((3, 2), (2, 2, 1)), ((2, 3, 2), (2, 1))):
+        v1 = np.array([1, 2, 3, 4, 5, 6] * (2 if len(shape_a) == 3 else 1), np.float32).reshape(shape_a)
+        v2 = np.array([1, 2] * (2 if len(shape_b) == 3 else 1), np.float32).reshape(shape_b)
+        qa, mn_a, mx_a = pkg.quantize(T.t(v1), torch.uint8)
+        qb, mn_b, mx_b = pkg.quantize(T.t(v2), torch.int8)
+        ra, rb = pkg.reduce_sum(qa, True), pkg.reduce_sum(qb, False)
+        qc, mn_c, mx_c = pkg.quantization_matmul(qa, ra, mn_a, mx_a, qb, rb, mn_b, mx_b)
+        out = T.n(pkg.dequantize(qc, mn_c, mx_c))
+        assert out.astype(np.int64).reshape(-1).tolist() == [5, 11, 17, 5, 11, 17]
+
+
+# ---- fp32 matmul -------------------------------------------------------------------------------------
+
+def test_sgemm_config_c1(pkg, T):
+    """[128,768] x [768,3072] + bias[3072], U[-1,1) / U[-0.1,0.1): relative Frobenius error <= 1e-5."""
+    rng = np.random.default_rng(0)
+    a = rng.uniform(-1, 1, (128, 768)).astype(np.float32)
+    b = rng.uniform(-1, 1, (768, 3072)).astype(np.float32)
+    bias = rng.uniform(-0.1, 0.1, 3072).astype(np.float32)
+    _, want = O.sgemm(a, b, bias, want64=True)
+    got = T.n(pkg.blas_matmul(T.t(a), T.t(b), T.t(bias)))
+    assert got.shape == (128, 3072) and rel_fro(got, want) <= FP32_TOL
+    _, want2 = O.sgemm(a, b, want64=True)
+    assert rel_fro(T.n(pkg.blas_matmul(T.t(a), T.t(b))), want2) <= FP32_TOL
+
+
+def test_sgemm_exact_cases(pkg, T):
+    rng = np.random.default_rng(20)
+    a = rng.uniform(-1, 1, (137, 253)).astype(np.float32)
+    eye = np.eye(253, dtype=np.float32)
+    mm = lambda x, y, *b: T.n(pkg.blas_matmul(T.t(x), T.t(y), *[T.t(v) for v in b]))
+    assert np.array_equal(mm(a, eye), a)
+    perm = rng.permutation(253)
+    assert np.array_equal(mm(a, eye[:, perm]), a[:, perm])
+    assert np.array_equal(mm(eye[perm], a.T.copy()), a.T[perm])
+    assert np.array_equal(mm(np.ones((5, 64), np.float32), np.ones((64, 7), np.float32)), np.full((5, 7), 64, np.float32))
+    assert np.array_equal(mm(a * 4, eye * 0.5), a * 2)
+    x = np.arange(6, dtype=np.float32).reshape(2, 3)
+    y = np.arange(12, dtype=np.float32).reshape(3, 4)
+    assert mm(x, y).tolist() == [[20, 23, 26, 29], [56, 68, 80, 92]]
+    assert mm(x, y, np.array([1, 2, 3, 4], np.float32)).tolist() == [[21, 25, 29, 33], [57, 70, 83, 96]]
+
+
+@pytest.mark.parametrize("shape_a,shape_b", [
+    ((1, 1), (1, 1)), ((5, 7), (7, 3)), ((33, 65), (65, 31)), ((99, 98), (98, 97)),
+    ((3, 50, 20), (3, 20, 30)), ((4, 25, 40), (40, 24)), ((31, 48), (2, 48, 52)), ((2, 3, 17, 9), (2, 3, 9, 33)),
+    ((16, 12, 128, 64), (16, 12, 64, 128)),      # attention scores Q.K^T
+    ((16, 12, 128, 128), (16, 12, 128, 64)),     # attention P.V
+    ((8, 128, 768), (768, 3072)), ((8, 128, 3072), (3072, 768)),   # BERT-base FFN
+    ((1024, 1024), (1024, 4096)),                # enough tiles for the 128x128 configuration
+    ((130, 36), (36, 516)), ((257, 100), (100, 260)),
+])
+def test_sgemm_shapes_against_oracle(pkg, T, shape_a, shape_b):
+    """The four shape families of tfcc/test/blas.cpp:34-61 plus the benchmark's batched shapes."""
+    print("sgemm", shape_a, shape_b, flush=True)
+    rng = np.random.default_rng(sum(shape_a) + sum(shape_b))
+    a = rng.normal(0, 1, shape_a).astype(np.float32)
+    b = rng.normal(0, 1, shape_b).astype(np.float32)
+    bias = rng.uniform(-1, 1, shape_b[-1]).astype(np.float32)
+    want = np.matmul(a.astype(np.float64), b.astype(np.float64))
+    got = T.n(pkg.blas_matmul(T.t(a), T.t(b)))
+    assert got.shape == want.shape and rel_fro(got, want) <= FP32_TOL
+    got_b = T.n(pkg.blas_matmul(T.t(a), T.t(b), T.t(bias)))
+    assert rel_fro(got_b, want + bias) <= FP32_TOL
+    # the reference's own tolerance (tfcc/core/utils/tfcc_debugutils.cpp:102-111) against a float32 product
+    ref32 = O.sgemm(a, b)
+    assert np.all((np.abs(got - ref32) < 1e-3 * np.abs(got + ref32)) | (np.abs(got - ref32) < 1e-5))
+
+
+def test_matmul_validation_and_empty(pkg, T):
+    """Error behaviour of tfcc::blas::matmul (tfcc/core/operations/tfcc_blas.cpp:26-54)."""
+    z = lambda *s: T.t(np.zeros(s, np.float32))
+    with pytest.raises(pkg.InvalidArgumentError, match="two or more dimensions"):
+        pkg.blas_matmul(z(3), z(3, 4))
+    for sa, sb in (((2, 3, 4), (5, 6, 4, 7)), ((3, 4), (5, 6)), ((2, 3, 4), (1, 4, 5))):
+        with pytest.raises(pkg.InvalidArgumentError, match="shape invalid"):
+            pkg.blas_matmul(z(*sa), z(*sb))
+    with pytest.raises(pkg.InvalidArgumentError, match="shape invalid"):
+        pkg.blas_matmul(z(3, 4), z(4, 5), z(4))
+    assert tuple(pkg.blas_matmul(z(2, 0, 4), z(2, 4, 5)).shape) == (2, 0, 5)
+    assert tuple(pkg.blas_matmul(z(6, 3, 4), z(4, 5)).shape) == (6, 3, 5)
+
+
+# ---- element-wise neighbours --------------------------------------------------------------------------
+
+def test_elementwise_against_oracle(pkg, T):
+    rng = np.random.default_rng(50)
+    for shape in ((8, 12, 128, 128), (7, 33), (5, 1000)):
+        x = rng.normal(0, 2, shape).astype(np.float32)
+        assert np.allclose(T.n(pkg.softmax(T.t(x))), O.softmax(x), rtol=2e-6, atol=1e-8)
+    x = rng.normal(0, 1, (1024, 768)).astype(np.float32)
+    g, b = rng.normal(1, 0.1, 768).astype(np.float32), rng.normal(0, 0.1, 768).astype(np.float32)
+    assert np.allclose(T.n(pkg.layer_norm(T.t(x), T.t(g), T.t(b), 1e-12)), O.layer_norm(x, g, b, 1e-12), rtol=1e-5, atol=1e-5)
+    assert np.allclose(T.n(pkg.gelu_accurate(T.t(x))), O.gelu_accurate(x), rtol=1e-6, atol=1e-7)
+    assert np.array_equal(T.n(pkg.transform(T.t(x), 0.125, 0.0)), x * np.float32(0.125))
+    assert np.array_equal(T.n(pkg.add(T.t(x), T.t(g))), x + g)
+    assert np.array_equal(T.n(pkg.add(T.t(x), T.t(x))), x + x)
+    y = rng.normal(0, 1, (8, 128, 12, 64)).astype(np.float32)
+    for perm in ((0, 2, 1, 3), (0, 1, 3, 2), (3, 2, 1, 0), (0, 2, 3, 1)):
+        assert np.array_equal(T.n(pkg.transpose(T.t(y), perm)), np.transpose(y, perm))
+    assert np.array_equal(T.n(pkg.transpose(T.t(x), (1, 0))), x.T)

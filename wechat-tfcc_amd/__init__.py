@@ -1,0 +1,382 @@
+"""ctypes binding of libtfcc_rocm.so (the C ABI of include/tfcc_rocm.h) for the Python test and
+benchmark harness.  PyTorch is used only as the owner of device memory and of the HIP stream; every
+computation goes through the C ABI into the hand-written gfx950 kernels.  There is no fallback: a
+missing library or a failing call raises.
+
+The functions mirror the reference's operator interface for this path:
+  blas_matmul            tfcc::blas::matmul                   (tfcc/core/operations/tfcc_blas.cpp:26-96)
+  quantization_matmul    tfcc::mkl::quantization::matmul      (tfcc/mkl/operations/tfcc_mklquantization.h:39-42)
+  reduce_sum             tfcc::mkl::quantization::reduce_sum  (tfcc/mkl/operations/tfcc_mklquantization.h:50-51)
+  quantize / requantize / dequantize   tfcc::quantization::*  (tfcc/core/operations/tfcc_quantization.cpp:26-98)
+"""
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libtfcc_rocm.so")
+CSRC_DIR = os.path.join(_HERE, "csrc")
+
+S8, U8, S16, U16, S32, U32 = range(6)
+
+
+class TfccRocmError(RuntimeError):
+    pass
+
+
+class InvalidArgumentError(ValueError):
+    """tfcc::InvalidArgumentError"""
+
+
+class QGemmDesc(C.Structure):
+    _fields_ = [
+        ("a", C.c_void_p), ("b", C.c_void_p), ("rowsum_a", C.c_void_p), ("colsum_b", C.c_void_p),
+        ("stride_a", C.c_uint64), ("stride_b", C.c_uint64), ("stride_rowsum_a", C.c_uint64),
+        ("stride_colsum_b", C.c_uint64), ("stride_c", C.c_uint64),
+        ("m", C.c_uint), ("n", C.c_uint), ("k", C.c_uint), ("batch", C.c_uint),
+        ("offset_a", C.c_int32), ("offset_b", C.c_int32),
+        ("min_a", C.c_void_p), ("max_a", C.c_void_p), ("min_b", C.c_void_p), ("max_b", C.c_void_p),
+        ("min_c", C.c_void_p), ("max_c", C.c_void_p),
+    ]
+
+
+# name -> (restype, argtypes): every symbol include/tfcc_rocm.h declares
+_VP, _U64, _U, _I, _F, _D, _I64 = C.c_void_p, C.c_uint64, C.c_uint, C.c_int, C.c_float, C.c_double, C.c_int64
+SYMBOLS = {
+    "tfcc_rocm_last_error_string": (C.c_char_p, []),
+    "tfcc_rocm_version": (C.c_char_p, []),
+    "tfcc_rocm_device_count": (_I, [C.POINTER(C.c_int)]),
+    "tfcc_rocm_set_device": (_I, [_I]),
+    "tfcc_rocm_mem_info": (_I, [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
+    "tfcc_rocm_device_name": (_I, [C.c_char_p, C.c_size_t]),
+    "tfcc_rocm_malloc": (_I, [C.POINTER(C.c_void_p), C.c_size_t]),
+    "tfcc_rocm_free": (_I, [_VP]),
+    "tfcc_rocm_stream_create": (_I, [C.POINTER(C.c_void_p)]),
+    "tfcc_rocm_stream_destroy": (_I, [_VP]),
+    "tfcc_rocm_stream_synchronize": (_I, [_VP]),
+    "tfcc_rocm_memcpy_h2d": (_I, [_VP, _VP, _VP, C.c_size_t]),
+    "tfcc_rocm_memcpy_d2h": (_I, [_VP, _VP, _VP, C.c_size_t]),
+    "tfcc_rocm_memcpy_d2d_async": (_I, [_VP, _VP, _VP, C.c_size_t]),
+    "tfcc_rocm_fill_async": (_I, [_VP, _VP, _U64, _I, C.c_size_t]),
+    "tfcc_rocm_sgemm_strided_batched": (_I, [_VP, _VP, _U64, _VP, _U64, _VP, _VP, _U64, _U, _U, _U, _U]),
+    "tfcc_rocm_gemm_u8s8s32": (_I, [_VP, C.POINTER(QGemmDesc), _VP]),
+    "tfcc_rocm_gemm_u8s8s32_requant_u8": (_I, [_VP, C.POINTER(QGemmDesc), _VP, _VP, _D, _D, _D, _I64, _VP, _VP]),
+    "tfcc_rocm_gemv_u8s8s32": (_I, [_VP, _VP, _VP, _VP, _VP, C.c_int32, C.c_int32, _U, _U, _U, _VP, _F, _VP, _VP]),
+    "tfcc_rocm_reduce_sum_rows": (_I, [_VP, _VP, _I, _U, _U, _U, _VP]),
+    "tfcc_rocm_reduce_sum_cols": (_I, [_VP, _VP, _I, _U, _U, _U, _VP]),
+    "tfcc_rocm_requantize": (_I, [_VP, _VP, _I, _VP, _I, _U64, _VP, _VP, _VP, _VP]),
+    "tfcc_rocm_dequantize": (_I, [_VP, _VP, _I, _U64, _VP, _VP, _VP]),
+    "tfcc_rocm_quantize": (_I, [_VP, _VP, _U64, _VP, _VP, _VP, _I]),
+    "tfcc_rocm_quantize_minmax": (_I, [_VP, _VP, _U64, _VP, _I, _VP, _VP]),
+    "tfcc_rocm_softmax_f32": (_I, [_VP, _VP, _U64, _U, _VP]),
+    "tfcc_rocm_layer_norm_f32": (_I, [_VP, _VP, _VP, _VP, _F, _U64, _U, _VP]),
+    "tfcc_rocm_gelu_accurate_f32": (_I, [_VP, _VP, _U64, _VP]),
+    "tfcc_rocm_transform_f32": (_I, [_VP, _VP, _U64, _F, _F, _VP]),
+    "tfcc_rocm_add_f32": (_I, [_VP, _VP, _VP, _U64, _U64, _VP]),
+    "tfcc_rocm_transpose_f32": (_I, [_VP, _VP, C.POINTER(C.c_uint), C.POINTER(C.c_uint), _I, _VP]),
+}
+
+_lib = None
+
+
+def lib():
+    """The loaded library.  Raises if it has not been built (see csrc/Makefile)."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise TfccRocmError("%s is missing: build it with `make -C %s`" % (LIB_PATH, CSRC_DIR))
+        handle = C.CDLL(LIB_PATH)
+        for name, (res, args) in SYMBOLS.items():
+            f = getattr(handle, name)  # AttributeError if the symbol is not exported
+            f.restype = res
+            f.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def check(status):
+    if status != 0:
+        raise TfccRocmError("tfcc_rocm error %d: %s" % (status, lib().tfcc_rocm_last_error_string().decode()))
+
+
+# ---------------------------------------------------------------------------------------------
+# torch-tensor convenience layer
+# ---------------------------------------------------------------------------------------------
+
+def _stream():
+    import torch
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t):
+    return None if t is None else t.data_ptr()
+
+
+def _type_code(dtype):
+    import torch
+    return {torch.int8: S8, torch.uint8: U8, torch.int16: S16, torch.int32: S32}[dtype]
+
+
+def matmul_plan(shape_a, shape_b, shape_bias=None):
+    """Validation and stride rules of tfcc::blas::matmul / MKLBlasInterface::matmul
+    (tfcc/core/operations/tfcc_blas.cpp:26-96, tfcc/mkl/interfaces/tfcc_mklblasinterface.cpp:127-151)."""
+    ra, rb = len(shape_a), len(shape_b)
+    if ra < 2 or rb < 2:
+        raise InvalidArgumentError("matmul require tensors with two or more dimensions")
+    if ra != rb and ra != 2 and rb != 2:
+        raise InvalidArgumentError("shape invalid")
+    if shape_a[-1] != shape_b[-2]:
+        raise InvalidArgumentError("shape invalid")
+    if shape_bias is not None and (len(shape_bias) != 1 or shape_bias[0] != shape_b[-1]):
+        raise InvalidArgumentError("shape invalid")
+    if ra == rb and tuple(shape_a[:-2]) != tuple(shape_b[:-2]):
+        raise InvalidArgumentError("shape invalid")
+    m, n, k = shape_a[-2], shape_b[-1], shape_a[-1]
+    lead = tuple(shape_a[:-2]) if ra > rb else tuple(shape_b[:-2])
+    batch = 1
+    for d in lead:
+        batch *= d
+    stride_a, stride_b = m * k, n * k
+    if ra != rb:
+        if ra == 2:
+            stride_a = 0
+        if rb == 2:
+            stride_b = 0
+    return dict(m=m, n=n, k=k, batch=batch, shape=lead + (m, n), stride_a=stride_a, stride_b=stride_b,
+                stride_c=m * n)
+
+
+def blas_matmul(a, b, bias=None):
+    """tfcc::blas::matmul(a, b[, bias]) on fp32 device tensors."""
+    import torch
+    for t in (a, b) + (() if bias is None else (bias,)):
+        if t.dtype != torch.float32:
+            raise NotImplementedError("matmul is implemented for float32 only, like the reference's MKL device")
+    p = matmul_plan(tuple(a.shape), tuple(b.shape), None if bias is None else tuple(bias.shape))
+    out = torch.empty(p["shape"], dtype=torch.float32, device=a.device)
+    if a.numel() == 0 or b.numel() == 0:
+        return out  # uninitialised, as the reference returns it
+    a, b = a.contiguous(), b.contiguous()
+    bias = None if bias is None else bias.contiguous()
+    check(lib().tfcc_rocm_sgemm_strided_batched(_stream(), _ptr(a), p["stride_a"], _ptr(b), p["stride_b"],
+                                                 _ptr(bias), _ptr(out), p["stride_c"], p["m"], p["n"], p["k"],
+                                                 p["batch"]))
+    return out
+
+
+def reduce_sum(a, row):
+    """tfcc::mkl::quantization::reduce_sum: int32 sums over the last (row=True) or the
+    second-to-last (row=False) dimension."""
+    import torch
+    if a.numel() == 0 or a.dim() < 2:
+        raise InvalidArgumentError("invalid input tensor a")
+    a = a.contiguous()
+    r, c = a.shape[-2], a.shape[-1]
+    batch = a.numel() // (r * c)
+    out = torch.empty(tuple(a.shape[:-2]) + ((r,) if row else (c,)), dtype=torch.int32, device=a.device)
+    f = lib().tfcc_rocm_reduce_sum_rows if row else lib().tfcc_rocm_reduce_sum_cols
+    check(f(_stream(), _ptr(a), _type_code(a.dtype), batch, r, c, _ptr(out)))
+    return out
+
+
+def _qdesc(a, reduce_a, b, reduce_b):
+    if a.numel() == 0 or a.dim() < 2:
+        raise InvalidArgumentError("invalid input tensor a")
+    if reduce_a.numel() == 0:
+        raise InvalidArgumentError("invalid tensor reduceSumA")
+    if b.numel() == 0 or b.dim() < 2:
+        raise InvalidArgumentError("invalid input tensor b")
+    if reduce_b.numel() == 0:
+        raise InvalidArgumentError("invalid tensor reduceSumB")
+    if a.shape[-1] != b.shape[-2]:
+        raise InvalidArgumentError("tensor a and b don't match")
+    if a.dim() != b.dim() and a.dim() != 2 and b.dim() != 2:
+        raise InvalidArgumentError("tensor a and b don't match")
+    if a.shape[-2] != reduce_a.shape[-1]:
+        raise InvalidArgumentError("tensor a and reduceSumA don't match")
+    if b.shape[-1] != reduce_b.shape[-1]:
+        raise InvalidArgumentError("tensor b and reduceSumB don't match")
+    if a.dim() == b.dim() and tuple(a.shape[:-2]) != tuple(b.shape[:-2]):
+        raise InvalidArgumentError("tensor a and b don't match")
+    m, k, n = a.shape[-2], a.shape[-1], b.shape[-1]
+    shape = tuple(a.shape[:-2] if a.dim() > b.dim() else b.shape[:-2]) + (m, n)
+    batch = 1
+    for d in shape[:-2]:
+        batch *= d
+    d = QGemmDesc()
+    d.a, d.b, d.rowsum_a, d.colsum_b = _ptr(a), _ptr(b), _ptr(reduce_a), _ptr(reduce_b)
+    d.stride_rowsum_a = 0 if reduce_a.dim() == 1 else m
+    d.stride_colsum_b = 0 if reduce_b.dim() == 1 else n
+    d.stride_a = 0 if a.dim() == 2 else m * k
+    d.stride_b = 0 if b.dim() == 2 else k * n
+    if b.dim() == 2:  # single B: the batch folds into M (tfcc_mklquantization.cpp:140-145)
+        m, d.stride_rowsum_a, d.stride_a, batch = m * batch, d.stride_rowsum_a * batch, d.stride_a * batch, 1
+    d.stride_c = m * n
+    d.m, d.n, d.k, d.batch = m, n, k, batch
+    return d, shape
+
+
+def _check_scalar(t, name):
+    if t.numel() != 1 or t.dim() != 1:
+        raise InvalidArgumentError("invalid tensor " + name)
+
+
+def quantization_matmul(a, reduce_a, min_a, max_a, b, reduce_b, min_b, max_b):
+    """tfcc::mkl::quantization::matmul: returns (int32 C, minC, maxC); ranges are 1-element device tensors."""
+    import torch
+    a, b, reduce_a, reduce_b = a.contiguous(), b.contiguous(), reduce_a.contiguous(), reduce_b.contiguous()
+    for t, nm in ((min_a, "minA"), (max_a, "maxA"), (min_b, "minB"), (max_b, "maxB")):
+        _check_scalar(t, nm)
+    d, shape = _qdesc(a, reduce_a, b, reduce_b)
+    c = torch.empty(shape, dtype=torch.int32, device=a.device)
+    min_c = torch.empty(1, dtype=torch.float32, device=a.device)
+    max_c = torch.empty(1, dtype=torch.float32, device=a.device)
+    d.min_a, d.max_a, d.min_b, d.max_b = _ptr(min_a), _ptr(max_a), _ptr(min_b), _ptr(max_b)
+    d.min_c, d.max_c = _ptr(min_c), _ptr(max_c)
+    check(lib().tfcc_rocm_gemm_u8s8s32(_stream(), C.byref(d), _ptr(c)))
+    return c, min_c, max_c
+
+
+def quantization_matmul_offsets(a, reduce_a, b, reduce_b, offset_a, offset_b):
+    """The same product with immediate integer offsets (kernel-level form)."""
+    import torch
+    a, b, reduce_a, reduce_b = a.contiguous(), b.contiguous(), reduce_a.contiguous(), reduce_b.contiguous()
+    d, shape = _qdesc(a, reduce_a, b, reduce_b)
+    d.offset_a, d.offset_b = offset_a, offset_b
+    c = torch.empty(shape, dtype=torch.int32, device=a.device)
+    check(lib().tfcc_rocm_gemm_u8s8s32(_stream(), C.byref(d), _ptr(c)))
+    return c
+
+
+def quantization_matmul_requantize(a, reduce_a, min_a, max_a, b, reduce_b, min_b, max_b, min_out, max_out,
+                                   want_acc=False):
+    """matmul followed by requantize<uint8_t> in one kernel.  Returns (uint8 Q, int32 C or None, minC, maxC)."""
+    import torch
+    a, b, reduce_a, reduce_b = a.contiguous(), b.contiguous(), reduce_a.contiguous(), reduce_b.contiguous()
+    for t, nm in ((min_a, "minA"), (max_a, "maxA"), (min_b, "minB"), (max_b, "maxB"), (min_out, "minOutput"),
+                  (max_out, "maxOutput")):
+        _check_scalar(t, nm)
+    d, shape = _qdesc(a, reduce_a, b, reduce_b)
+    q = torch.empty(shape, dtype=torch.uint8, device=a.device)
+    c = torch.empty(shape, dtype=torch.int32, device=a.device) if want_acc else None
+    min_c = torch.empty(1, dtype=torch.float32, device=a.device)
+    max_c = torch.empty(1, dtype=torch.float32, device=a.device)
+    d.min_a, d.max_a, d.min_b, d.max_b = _ptr(min_a), _ptr(max_a), _ptr(min_b), _ptr(max_b)
+    d.min_c, d.max_c = _ptr(min_c), _ptr(max_c)
+    check(lib().tfcc_rocm_gemm_u8s8s32_requant_u8(_stream(), C.byref(d), _ptr(c), _ptr(q), 0.0, 0.0, 0.0, 0,
+                                                   _ptr(min_out), _ptr(max_out)))
+    return q, c, min_c, max_c
+
+
+def gemv_dequant(a, b, reduce_a, reduce_b, offset_a, offset_b, scale_a, scale_b, want_acc=True):
+    """Skinny (M <= 8) product with optional fused per-channel dequantize.  Returns (f32 or None, int32 or None)."""
+    import torch
+    a, b = a.contiguous(), b.contiguous()
+    m, k, n = a.shape[0], a.shape[1], b.shape[1]
+    acc = torch.empty((m, n), dtype=torch.int32, device=a.device) if want_acc else None
+    out = torch.empty((m, n), dtype=torch.float32, device=a.device) if scale_b is not None else None
+    check(lib().tfcc_rocm_gemv_u8s8s32(_stream(), _ptr(a), _ptr(b), _ptr(reduce_a), _ptr(reduce_b), offset_a,
+                                        offset_b, m, n, k, _ptr(acc), float(scale_a), _ptr(scale_b), _ptr(out)))
+    return out, acc
+
+
+def requantize(a, min_in, max_in, min_out, max_out, out_dtype):
+    """tfcc::quantization::requantize<T>(a, minInput, maxInput, minOutput, maxOutput)"""
+    import torch
+    if a.numel() == 0:
+        raise InvalidArgumentError("invalid tensor")
+    for t, nm in ((min_in, "minInput"), (max_in, "maxInput"), (min_out, "minOutput"), (max_out, "maxOutput")):
+        if t.numel() != 1 or t.dim() != 1:
+            raise InvalidArgumentError("invalid " + nm)
+    a = a.contiguous()
+    out = torch.empty(a.shape, dtype=out_dtype, device=a.device)
+    check(lib().tfcc_rocm_requantize(_stream(), _ptr(a), _type_code(a.dtype), _ptr(out), _type_code(out_dtype),
+                                      a.numel(), _ptr(min_in), _ptr(max_in), _ptr(min_out), _ptr(max_out)))
+    return out
+
+
+def dequantize(a, min_v, max_v):
+    """tfcc::quantization::dequantize(a, minValue, maxValue)"""
+    import torch
+    if a.numel() == 0:
+        raise InvalidArgumentError("invalid tensor")
+    for t, nm in ((min_v, "minValue"), (max_v, "maxValue")):
+        if t.numel() != 1 or t.dim() != 1:
+            raise InvalidArgumentError("invalid " + nm)
+    a = a.contiguous()
+    out = torch.empty(a.shape, dtype=torch.float32, device=a.device)
+    check(lib().tfcc_rocm_dequantize(_stream(), _ptr(a), _type_code(a.dtype), a.numel(), _ptr(min_v), _ptr(max_v),
+                                      _ptr(out)))
+    return out
+
+
+def quantize(a, out_dtype, min_v=None, max_v=None):
+    """tfcc::quantization::quantize<T>(a) -> (q, min, max), or quantize<T>(a, min, max) -> q"""
+    import torch
+    if a.numel() == 0:
+        raise InvalidArgumentError("invalid tensor")
+    a = a.contiguous()
+    out = torch.empty(a.shape, dtype=out_dtype, device=a.device)
+    if min_v is None:
+        mn = torch.empty(1, dtype=torch.float32, device=a.device)
+        mx = torch.empty(1, dtype=torch.float32, device=a.device)
+        check(lib().tfcc_rocm_quantize_minmax(_stream(), _ptr(a), a.numel(), _ptr(out), _type_code(out_dtype),
+                                               _ptr(mn), _ptr(mx)))
+        return out, mn, mx
+    for t, nm in ((min_v, "minValue"), (max_v, "maxValue")):
+        if t.numel() != 1 or t.dim() != 1:
+            raise InvalidArgumentError("invalid " + nm)
+    check(lib().tfcc_rocm_quantize(_stream(), _ptr(a), a.numel(), _ptr(min_v), _ptr(max_v), _ptr(out),
+                                    _type_code(out_dtype)))
+    return out
+
+
+def softmax(a):
+    import torch
+    a = a.contiguous()
+    out = torch.empty_like(a)
+    check(lib().tfcc_rocm_softmax_f32(_stream(), _ptr(a), a.numel() // a.shape[-1], a.shape[-1], _ptr(out)))
+    return out
+
+
+def layer_norm(a, gamma, beta, eps):
+    import torch
+    a = a.contiguous()
+    out = torch.empty_like(a)
+    check(lib().tfcc_rocm_layer_norm_f32(_stream(), _ptr(a), _ptr(gamma.contiguous()), _ptr(beta.contiguous()),
+                                          eps, a.numel() // a.shape[-1], a.shape[-1], _ptr(out)))
+    return out
+
+
+def gelu_accurate(a):
+    import torch
+    a = a.contiguous()
+    out = torch.empty_like(a)
+    check(lib().tfcc_rocm_gelu_accurate_f32(_stream(), _ptr(a), a.numel(), _ptr(out)))
+    return out
+
+
+def transform(a, alpha, beta):
+    import torch
+    a = a.contiguous()
+    out = torch.empty_like(a)
+    check(lib().tfcc_rocm_transform_f32(_stream(), _ptr(a), a.numel(), alpha, beta, _ptr(out)))
+    return out
+
+
+def add(a, b):
+    """a + b where b's shape equals the trailing dims of a's."""
+    import torch
+    a, b = a.contiguous(), b.contiguous()
+    out = torch.empty_like(a)
+    check(lib().tfcc_rocm_add_f32(_stream(), _ptr(a), _ptr(b), a.numel(), b.numel(), _ptr(out)))
+    return out
+
+
+def transpose(a, perm):
+    import torch
+    a = a.contiguous()
+    shape = (C.c_uint * a.dim())(*a.shape)
+    p = (C.c_uint * a.dim())(*perm)
+    out = torch.empty([a.shape[i] for i in perm], dtype=a.dtype, device=a.device)
+    check(lib().tfcc_rocm_transpose_f32(_stream(), _ptr(a), shape, p, a.dim(), _ptr(out)))
+    return out

@@ -1,0 +1,156 @@
+// Shared plumbing of the HIP translation units: error reporting behind the C ABI and the
+// range arithmetic of the quantization path evaluated on the device in double.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "tfcc_rocm.h"
+
+namespace tfcc_rocm {
+
+// Records the text returned by tfcc_rocm_last_error_string() for the calling thread.
+int set_error(int code, const char* fmt, ...);
+
+#define TFCC_HIP_CHECK(expr)                                                                  \
+  do {                                                                                        \
+    hipError_t _e = (expr);                                                                   \
+    if (_e != hipSuccess)                                                                     \
+      return ::tfcc_rocm::set_error(                                                          \
+          _e == hipErrorOutOfMemory ? TFCC_ROCM_OUT_OF_MEMORY : TFCC_ROCM_HIP_ERROR,          \
+          "%s failed: %s", #expr, hipGetErrorString(_e));                                     \
+  } while (0)
+
+#define TFCC_REQUIRE(cond, ...)                                                               \
+  do {                                                                                        \
+    if (!(cond)) return ::tfcc_rocm::set_error(TFCC_ROCM_INVALID_ARGUMENT, __VA_ARGS__);      \
+  } while (0)
+
+// Checks the launch that has just been enqueued.
+static inline int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return set_error(TFCC_ROCM_HIP_ERROR, "%s launch failed: %s", what, hipGetErrorString(e));
+  return TFCC_ROCM_OK;
+}
+
+static inline hipStream_t as_stream(void* s) { return reinterpret_cast<hipStream_t>(s); }
+
+// ---- range arithmetic (tfcc/core/utils/tfcc_quantizationutils.h:23-70), host and device ----
+
+struct IntRange {
+  long long lowest, highest;
+  int bits;
+};
+
+__host__ __device__ static inline IntRange int_range(int type) {
+  switch (type) {
+    case TFCC_ROCM_S8: return {-128, 127, 8};
+    case TFCC_ROCM_U8: return {0, 255, 8};
+    case TFCC_ROCM_S16: return {-32768, 32767, 16};
+    case TFCC_ROCM_U16: return {0, 65535, 16};
+    case TFCC_ROCM_S32: return {-2147483648LL, 2147483647LL, 32};
+    default: return {0, 4294967295LL, 32};
+  }
+}
+
+// get_quantized_scale_info<T>: scale = stepCnt / range, offset = round(min * scale)
+__host__ __device__ static inline void quantized_scale_info(int bits, float mn, float mx,
+                                                            double* scale, long long* offset) {
+  double step = (double)(1LL << bits);
+  double adjust = step / (step - 1.0);
+  float span = mx - mn;  // float subtraction, as in the reference
+  double range = (double)span * adjust;
+  double s = step / range;
+  *scale = s;
+  *offset = (long long)round((double)mn * s);
+}
+
+// get_dequantized_scale_info<T>: scale = range / stepCnt, minRounded = min
+__host__ __device__ static inline void dequantized_scale_info(int bits, float mn, float mx,
+                                                              double* scale, double* minRounded) {
+  double step = (double)(1LL << bits);
+  double adjust = step / (step - 1.0);
+  float span = mx - mn;
+  double range = (double)span * adjust;
+  *scale = range / step;
+  *minRounded = (double)mn;
+}
+
+// get_quantization_range_for_multiplication<uint8_t, int8_t, int32_t>
+__host__ __device__ static inline void qmatmul_range(float minA, float maxA, float minB, float maxB,
+                                                     float* minC, float* maxC) {
+  float aLevel = (maxA - minA) / 255.0f;
+  float bLevel = (maxB - minB) / 255.0f;
+  float cLevel = aLevel * bLevel;
+  *minC = cLevel * -2147483648.0f;
+  *maxC = cLevel * 2147483648.0f;  // (float)INT32_MAX rounds to 2^31
+}
+
+// offsets of the quantized matmul: tfcc/mkl/operations/tfcc_mklquantization.cpp:181-186
+__host__ __device__ static inline void qmatmul_offsets(float minA, float maxA, float minB, float maxB,
+                                                       int* offsetA, int* offsetB) {
+  double s;
+  long long oa, ob;
+  quantized_scale_info(8, minA, maxA, &s, &oa);
+  quantized_scale_info(8, minB, maxB, &s, &ob);
+  *offsetA = (int)oa;          // - lowest(uint8) = 0
+  *offsetB = (int)(ob + 128);  // - lowest(int8) = -128
+}
+
+// double -> int64 the way x86 cvttsd2si does it (out of range and NaN give INT64_MIN)
+__host__ __device__ static inline long long to_int64_x86(double v) {
+  if (!(v > -9223372036854775808.0 && v < 9223372036854775808.0)) return (long long)0x8000000000000000ULL;
+  return (long long)v;
+}
+
+// One requantize step, AVX2 flavour of the reference: fused multiply-add, nearest-even.
+// tfcc/mkl/kernel/tfcc_mklquantizationkernel.avx256.cpp:128-138
+struct RequantScalars {
+  double inScale, inMin, outScale;
+  long long outOffset;
+  long long inLowest, outLowest, outHighest;
+  int mode;            // 0: per-element arithmetic, 1: fill with fillValue (degenerate ranges)
+  long long fillValue;
+};
+
+__device__ static inline long long requantize_one(long long x, const RequantScalars& s) {
+  double off = (double)x - (double)s.inLowest;
+  double real = fma(off, s.inScale, s.inMin);
+  long long q = to_int64_x86(rint(real * s.outScale));
+  q = (long long)((unsigned long long)q - (unsigned long long)s.outOffset + (unsigned long long)s.outLowest);
+  q = q < s.outLowest ? s.outLowest : q;
+  q = q > s.outHighest ? s.outHighest : q;
+  return q;
+}
+
+// The branches of _requantize_helper (tfcc/mkl/interfaces/tfcc_mklquantizationinterface.cpp:121-141)
+__host__ __device__ static inline RequantScalars make_requant_scalars(int inType, int outType, float minIn,
+                                                                      float maxIn, float minOut, float maxOut) {
+  RequantScalars s;
+  IntRange ri = int_range(inType), ro = int_range(outType);
+  s.inLowest = ri.lowest;
+  s.outLowest = ro.lowest;
+  s.outHighest = ro.highest;
+  s.mode = 0;
+  s.fillValue = 0;
+  s.inScale = s.inMin = s.outScale = 0.0;
+  s.outOffset = 0;
+  if (minOut >= maxOut) {
+    s.mode = 1;
+    s.fillValue = ro.lowest;
+    return s;
+  }
+  dequantized_scale_info(ri.bits, minIn, maxIn, &s.inScale, &s.inMin);
+  quantized_scale_info(ro.bits, minOut, maxOut, &s.outScale, &s.outOffset);
+  if (minIn >= maxIn) {
+    long long q = to_int64_x86(round((double)minIn * s.outScale));
+    q = (long long)((unsigned long long)q - (unsigned long long)s.outOffset + (unsigned long long)ro.lowest);
+    q = q < ro.lowest ? ro.lowest : q;
+    q = q > ro.highest ? ro.highest : q;
+    s.mode = 1;
+    s.fillValue = q;
+  }
+  return s;
+}
+
+}  // namespace tfcc_rocm

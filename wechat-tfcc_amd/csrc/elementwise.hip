@@ -1,0 +1,266 @@
+// The fp32 element-wise / row-wise neighbours of matmul in one transformer encoder layer, so that
+// the layer's tensors stay resident on the GPU between the matrix products.  All are bandwidth
+// bound: one pass over the data, a wavefront (or workgroup) per row for the row-wise ones.
+//
+// Numerics follow the reference's scalar MKL kernels:
+//   softmax     tfcc/mkl/kernel/tfcc_mklactivationkernel.hpp:137-155  exp(x - max) / sum
+//   layer norm  tfcc/mkl/interfaces/tfcc_mklnormalizationinterface.cpp:29-62  two-pass mean / variance,
+//               1/sqrt(var + eps), (x - mean) * (inv * gamma) + beta
+//   gelu        tfcc/mkl/kernel/tfcc_mklactivationkernel.hpp:213-220  0.5 x (1 + erf(x / sqrt 2))
+//   transform   tfcc/core/operations/tfcc_operator.cpp:78-95  a * alpha + beta
+//   add         tfcc/core/operations/tfcc_math.cpp:38-104 (trailing-dims broadcast only)
+//   transpose   tfcc/core/operations/tfcc_base.cpp:124-134
+#include "common.hpp"
+
+namespace tfcc_rocm {
+namespace {
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+// block-wide reductions for rows handled by a whole workgroup
+template <bool MAX>
+__device__ __forceinline__ float block_reduce(float v, float* sh) {
+  v = MAX ? wave_max(v) : wave_sum(v);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+  __syncthreads();
+  if (lane == 0) sh[wave] = v;
+  __syncthreads();
+  float r = sh[0];
+  for (int i = 1; i < nw; ++i) r = MAX ? fmaxf(r, sh[i]) : r + sh[i];
+  return r;
+}
+
+// one workgroup of 256 threads per row
+__global__ __launch_bounds__(256) void softmax_kernel(const float* in, unsigned cols, float* out) {
+  __shared__ float sh[4];
+  const float* a = in + (size_t)blockIdx.x * cols;
+  float* o = out + (size_t)blockIdx.x * cols;
+  float mx = -3.402823466e+38f;
+  for (unsigned i = threadIdx.x; i < cols; i += 256) mx = fmaxf(mx, a[i]);
+  mx = block_reduce<true>(mx, sh);
+  float s = 0.f;
+  for (unsigned i = threadIdx.x; i < cols; i += 256) {
+    float e = expf(a[i] - mx);
+    o[i] = e;
+    s += e;
+  }
+  s = block_reduce<false>(s, sh);
+  for (unsigned i = threadIdx.x; i < cols; i += 256) o[i] = o[i] / s;
+}
+
+// rows of at most 256 columns: one wavefront per row, values stay in registers
+__global__ __launch_bounds__(256) void softmax_small_kernel(const float* in, size_t rows, unsigned cols, float* out) {
+  const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  const int lane = threadIdx.x & 63;
+  if (row >= rows) return;
+  const float* a = in + row * cols;
+  float* o = out + row * cols;
+  float v[4];
+  float mx = -3.402823466e+38f;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    unsigned i = lane + 64 * q;
+    v[q] = i < cols ? a[i] : -3.402823466e+38f;
+    mx = fmaxf(mx, v[q]);
+  }
+  mx = wave_max(mx);
+  float s = 0.f;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    unsigned i = lane + 64 * q;
+    v[q] = i < cols ? expf(v[q] - mx) : 0.f;
+    s += v[q];
+  }
+  s = wave_sum(s);
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    unsigned i = lane + 64 * q;
+    if (i < cols) o[i] = v[q] / s;
+  }
+}
+
+__global__ __launch_bounds__(256) void layer_norm_kernel(const float* in, const float* gamma, const float* beta,
+                                                         float eps, unsigned cols, float* out) {
+  __shared__ float sh[4];
+  const float* a = in + (size_t)blockIdx.x * cols;
+  float* o = out + (size_t)blockIdx.x * cols;
+  float s = 0.f;
+  for (unsigned i = threadIdx.x; i < cols; i += 256) s += a[i];
+  const float mean = block_reduce<false>(s, sh) / (float)cols;
+  float v = 0.f;
+  for (unsigned i = threadIdx.x; i < cols; i += 256) {
+    float t = a[i] - mean;
+    v += t * t;
+  }
+  const float var = block_reduce<false>(v, sh) / (float)cols;
+  const float inv = 1.0f / sqrtf(var + eps);
+  for (unsigned i = threadIdx.x; i < cols; i += 256) o[i] = (a[i] - mean) * (inv * gamma[i]) + beta[i];
+}
+
+__global__ __launch_bounds__(256) void gelu_kernel(const float* in, size_t total, float* out) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t step = (size_t)gridDim.x * blockDim.x;
+  for (; i < total; i += step) {
+    float v = in[i];
+    out[i] = (float)(0.5 * (double)v * (double)(1.0f + erff(v / 1.4142135623730951f)));
+  }
+}
+
+__global__ __launch_bounds__(256) void transform_kernel(const float* in, size_t total, float alpha, float beta,
+                                                        float* out) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t step = (size_t)gridDim.x * blockDim.x;
+  for (; i < total; i += step) out[i] = in[i] * alpha + beta;
+}
+
+__global__ __launch_bounds__(256) void add_kernel(const float* a, const float* b, size_t total, size_t period,
+                                                  float* out) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t step = (size_t)gridDim.x * blockDim.x;
+  for (; i < total; i += step) out[i] = a[i] + b[period == total ? i : i % period];
+}
+
+struct TransposeParams {
+  unsigned outShape[6];
+  unsigned long long inStride[6];  // input stride of each OUTPUT dim
+  int rank;
+};
+
+__global__ __launch_bounds__(256) void transpose_kernel(const float* in, size_t total, TransposeParams p, float* out) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t step = (size_t)gridDim.x * blockDim.x;
+  for (; i < total; i += step) {
+    size_t rem = i, src = 0;
+    for (int d = p.rank - 1; d >= 0; --d) {
+      size_t c = rem % p.outShape[d];
+      rem /= p.outShape[d];
+      src += c * p.inStride[d];
+    }
+    out[i] = in[src];
+  }
+}
+
+// batched 2-D transpose of the last two dims through LDS (both sides coalesced)
+__global__ __launch_bounds__(256) void transpose_last2_kernel(const float* in, unsigned rows, unsigned cols, float* out) {
+  __shared__ float tile[32][33];
+  const size_t b = blockIdx.z;
+  const float* a = in + b * (size_t)rows * cols;
+  float* o = out + b * (size_t)rows * cols;
+  const unsigned c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
+  const unsigned tx = threadIdx.x & 31, ty = threadIdx.x >> 5;  // 32 x 8
+  for (unsigned y = ty; y < 32; y += 8)
+    if (r0 + y < rows && c0 + tx < cols) tile[y][tx] = a[(size_t)(r0 + y) * cols + c0 + tx];
+  __syncthreads();
+  for (unsigned y = ty; y < 32; y += 8)
+    if (c0 + y < cols && r0 + tx < rows) o[(size_t)(c0 + y) * rows + r0 + tx] = tile[tx][y];
+}
+
+unsigned grid_for(size_t total) {
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 256u * 32u) blocks = 256u * 32u;
+  if (blocks < 1) blocks = 1;
+  return (unsigned)blocks;
+}
+
+}  // namespace
+}  // namespace tfcc_rocm
+
+using namespace tfcc_rocm;
+
+extern "C" {
+
+int tfcc_rocm_softmax_f32(void* stream, const float* in, uint64_t rows, unsigned cols, float* out) {
+  TFCC_REQUIRE(in && out, "softmax: null argument");
+  TFCC_REQUIRE(rows > 0 && cols > 0, "softmax: empty tensor");
+  TFCC_REQUIRE(rows < (1ull << 31), "softmax: too many rows");
+  if (cols <= 256)
+    hipLaunchKernelGGL(softmax_small_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, as_stream(stream), in,
+                       (size_t)rows, cols, out);
+  else
+    hipLaunchKernelGGL(softmax_kernel, dim3((unsigned)rows), dim3(256), 0, as_stream(stream), in, cols, out);
+  return check_launch("softmax");
+}
+
+int tfcc_rocm_layer_norm_f32(void* stream, const float* in, const float* gamma, const float* beta,
+                             float epsilon, uint64_t rows, unsigned cols, float* out) {
+  TFCC_REQUIRE(in && gamma && beta && out, "layer_norm: null argument");
+  TFCC_REQUIRE(rows > 0 && cols > 0, "layer_norm: empty tensor");
+  TFCC_REQUIRE(rows < (1ull << 31), "layer_norm: too many rows");
+  hipLaunchKernelGGL(layer_norm_kernel, dim3((unsigned)rows), dim3(256), 0, as_stream(stream), in, gamma, beta,
+                     epsilon, cols, out);
+  return check_launch("layer_norm");
+}
+
+int tfcc_rocm_gelu_accurate_f32(void* stream, const float* in, uint64_t total, float* out) {
+  TFCC_REQUIRE(in && out, "gelu: null argument");
+  TFCC_REQUIRE(total > 0, "gelu: empty tensor");
+  hipLaunchKernelGGL(gelu_kernel, dim3(grid_for(total)), dim3(256), 0, as_stream(stream), in, (size_t)total, out);
+  return check_launch("gelu");
+}
+
+int tfcc_rocm_transform_f32(void* stream, const float* in, uint64_t total, float alpha, float beta, float* out) {
+  TFCC_REQUIRE(in && out, "transform: null argument");
+  TFCC_REQUIRE(total > 0, "transform: empty tensor");
+  hipLaunchKernelGGL(transform_kernel, dim3(grid_for(total)), dim3(256), 0, as_stream(stream), in, (size_t)total,
+                     alpha, beta, out);
+  return check_launch("transform");
+}
+
+int tfcc_rocm_add_f32(void* stream, const float* a, const float* b, uint64_t total, uint64_t period, float* out) {
+  TFCC_REQUIRE(a && b && out, "add: null argument");
+  TFCC_REQUIRE(total > 0 && period > 0 && period <= total && total % period == 0, "add: bad broadcast period");
+  hipLaunchKernelGGL(add_kernel, dim3(grid_for(total)), dim3(256), 0, as_stream(stream), a, b, (size_t)total,
+                     (size_t)period, out);
+  return check_launch("add");
+}
+
+int tfcc_rocm_transpose_f32(void* stream, const float* in, const unsigned* shape, const unsigned* perm,
+                            int rank, float* out) {
+  TFCC_REQUIRE(in && out && shape && perm, "transpose: null argument");
+  TFCC_REQUIRE(rank >= 1 && rank <= 6, "transpose: rank %d (1..6)", rank);
+  bool seen[6] = {};
+  size_t total = 1;
+  for (int d = 0; d < rank; ++d) {
+    TFCC_REQUIRE(perm[d] < (unsigned)rank && !seen[perm[d]], "transpose: perm is not a permutation");
+    seen[perm[d]] = true;
+    total *= shape[d];
+  }
+  TFCC_REQUIRE(total > 0, "transpose: empty tensor");
+  // identity up to the last two dims swapped: tiled kernel
+  bool last2 = rank >= 2 && perm[rank - 1] == (unsigned)rank - 2 && perm[rank - 2] == (unsigned)rank - 1;
+  for (int d = 0; d + 2 < rank && last2; ++d) last2 = perm[d] == (unsigned)d;
+  if (last2) {
+    unsigned rows = shape[rank - 2], cols = shape[rank - 1];
+    size_t batch = total / ((size_t)rows * cols);
+    if (batch <= 65535 && (rows + 31) / 32 <= 65535) {
+      hipLaunchKernelGGL(transpose_last2_kernel, dim3((cols + 31) / 32, (rows + 31) / 32, (unsigned)batch), dim3(256),
+                         0, as_stream(stream), in, rows, cols, out);
+      return check_launch("transpose");
+    }
+  }
+  TransposeParams p{};
+  p.rank = rank;
+  unsigned long long stride[6];
+  unsigned long long s = 1;
+  for (int d = rank - 1; d >= 0; --d) {
+    stride[d] = s;
+    s *= shape[d];
+  }
+  for (int d = 0; d < rank; ++d) {
+    p.outShape[d] = shape[perm[d]];
+    p.inStride[d] = stride[perm[d]];
+  }
+  hipLaunchKernelGGL(transpose_kernel, dim3(grid_for(total)), dim3(256), 0, as_stream(stream), in, total, p, out);
+  return check_launch("transpose");
+}
+
+}  // extern "C"

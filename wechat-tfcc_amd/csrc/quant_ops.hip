@@ -1,0 +1,368 @@
+// Bandwidth-bound companions of the quantized matmul: int32 row / column sums, and the
+// range-based quantize / requantize / dequantize steps with their scale arithmetic evaluated on
+// the device in double (the ranges are float scalars in device memory, as the reference passes
+// them as tensors).
+//
+// Replaces tfcc/mkl/operations/tfcc_mklquantization.cpp:205-318 (reduce_sum),
+// tfcc/mkl/kernel/tfcc_mklquantizationkernel.avx256.cpp:55-145 (the AVX2 kernels: nearest-even
+// rounding, fused multiply-add) and the branches of
+// tfcc/mkl/interfaces/tfcc_mklquantizationinterface.cpp:47-69,72-147,191-240,284-333.
+#include "common.hpp"
+
+namespace tfcc_rocm {
+namespace {
+
+template <class T>
+__device__ __forceinline__ long long load_as_i64(const void* p, size_t i) {
+  return (long long)static_cast<const T*>(p)[i];
+}
+
+__device__ __forceinline__ long long load_typed(const void* p, int type, size_t i) {
+  switch (type) {
+    case TFCC_ROCM_S8: return load_as_i64<int8_t>(p, i);
+    case TFCC_ROCM_U8: return load_as_i64<uint8_t>(p, i);
+    case TFCC_ROCM_S16: return load_as_i64<int16_t>(p, i);
+    case TFCC_ROCM_U16: return load_as_i64<uint16_t>(p, i);
+    case TFCC_ROCM_S32: return load_as_i64<int32_t>(p, i);
+    default: return load_as_i64<uint32_t>(p, i);
+  }
+}
+
+__device__ __forceinline__ void store_typed(void* p, int type, size_t i, long long v) {
+  switch (type) {
+    case TFCC_ROCM_S8: static_cast<int8_t*>(p)[i] = (int8_t)v; break;
+    case TFCC_ROCM_U8: static_cast<uint8_t*>(p)[i] = (uint8_t)v; break;
+    case TFCC_ROCM_S16: static_cast<int16_t*>(p)[i] = (int16_t)v; break;
+    case TFCC_ROCM_U16: static_cast<uint16_t*>(p)[i] = (uint16_t)v; break;
+    case TFCC_ROCM_S32: static_cast<int32_t*>(p)[i] = (int32_t)v; break;
+    default: static_cast<uint32_t*>(p)[i] = (uint32_t)v; break;
+  }
+}
+
+// ---- row sums: one wavefront per row, 128-bit loads when the row allows it ------------------
+template <class T>
+__global__ __launch_bounds__(256) void reduce_rows_kernel(const T* a, unsigned rows, unsigned col, int* out) {
+  const unsigned wave = (blockIdx.x * 256 + threadIdx.x) >> 6, lane = threadIdx.x & 63;
+  if (wave >= rows) return;
+  const T* p = a + (size_t)wave * col;
+  unsigned s = 0;
+  constexpr unsigned PER = 16 / sizeof(T);
+  if (col % PER == 0 && ((uintptr_t)a % 16 == 0)) {
+    const uint4* v = reinterpret_cast<const uint4*>(p);
+    for (unsigned i = lane; i < col / PER; i += 64) {
+      uint4 q = v[i];
+      unsigned w[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        if (sizeof(T) == 1) {
+#pragma unroll
+          for (int b = 0; b < 4; ++b) s += (unsigned)(int)(T)(w[d] >> (8 * b));
+        } else {
+#pragma unroll
+          for (int b = 0; b < 2; ++b) s += (unsigned)(int)(T)(w[d] >> (16 * b));
+        }
+      }
+    }
+  } else {
+    for (unsigned i = lane; i < col; i += 64) s += (unsigned)(int)p[i];
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) s += __shfl_down(s, off, 64);
+  if (lane == 0) out[wave] = (int)s;
+}
+
+// ---- column sums: a workgroup owns 256 x (4 bytes) columns of one batch entry and a slab of rows;
+// slabs are combined with integer atomics (exact and order independent) into a zeroed result.
+template <class T>
+__global__ __launch_bounds__(256) void reduce_cols_kernel(const T* a, unsigned row, unsigned col,
+                                                          unsigned rowsPerSlab, int* out) {
+  const unsigned b = blockIdx.z;
+  const unsigned c = blockIdx.x * 256 + threadIdx.x;
+  const unsigned r0 = blockIdx.y * rowsPerSlab;
+  const unsigned r1 = min(r0 + rowsPerSlab, row);
+  if (c >= col) return;
+  const T* p = a + (size_t)b * row * col + c;
+  unsigned s = 0;
+  for (unsigned r = r0; r < r1; ++r) s += (unsigned)(int)p[(size_t)r * col];
+  atomicAdd(reinterpret_cast<unsigned*>(out) + (size_t)b * col + c, s);
+}
+
+template <class T>
+__global__ __launch_bounds__(256) void reduce_cols_vec_kernel(const T* a, unsigned row, unsigned col,
+                                                              unsigned rowsPerSlab, int* out) {
+  // col % 4 == 0 and 4-byte aligned rows (1-byte types): one dword = 4 columns per thread
+  const unsigned b = blockIdx.z;
+  const unsigned c4 = blockIdx.x * 256 + threadIdx.x;
+  const unsigned r0 = blockIdx.y * rowsPerSlab;
+  const unsigned r1 = min(r0 + rowsPerSlab, row);
+  if (c4 * 4 >= col) return;
+  const unsigned* p = reinterpret_cast<const unsigned*>(a + (size_t)b * row * col) + c4;
+  const unsigned pitch = col / 4;
+  unsigned s[4] = {0, 0, 0, 0};
+  for (unsigned r = r0; r < r1; ++r) {
+    unsigned w = p[(size_t)r * pitch];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) s[e] += (unsigned)(int)(T)(w >> (8 * e));
+  }
+  unsigned* o = reinterpret_cast<unsigned*>(out) + (size_t)b * col + c4 * 4;
+#pragma unroll
+  for (int e = 0; e < 4; ++e) atomicAdd(o + e, s[e]);
+}
+
+__global__ void zero_kernel(int* p, size_t n) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0;
+}
+
+// ---- requantize / dequantize / quantize -----------------------------------------------------
+__global__ __launch_bounds__(256) void requantize_kernel(const void* in, int inType, void* out, int outType,
+                                                         size_t total, const float* minIn, const float* maxIn,
+                                                         const float* minOut, const float* maxOut) {
+  const RequantScalars s = make_requant_scalars(inType, outType, *minIn, *maxIn, *minOut, *maxOut);
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t step = (size_t)gridDim.x * blockDim.x;
+  for (; i < total; i += step) {
+    long long q = s.mode ? s.fillValue : requantize_one(load_typed(in, inType, i), s);
+    store_typed(out, outType, i, q);
+  }
+}
+
+// int32 -> uint8, the matmul epilogue's type pair, four elements per thread
+__global__ __launch_bounds__(256) void requantize_s32_u8_vec_kernel(const int4* in, unsigned* out, size_t total4,
+                                                                    const float* minIn, const float* maxIn,
+                                                                    const float* minOut, const float* maxOut) {
+  const RequantScalars s = make_requant_scalars(TFCC_ROCM_S32, TFCC_ROCM_U8, *minIn, *maxIn, *minOut, *maxOut);
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t step = (size_t)gridDim.x * blockDim.x;
+  for (; i < total4; i += step) {
+    int4 v = in[i];
+    unsigned q0, q1, q2, q3;
+    if (s.mode) {
+      q0 = q1 = q2 = q3 = (unsigned)s.fillValue;
+    } else {
+      q0 = (unsigned)requantize_one(v.x, s);
+      q1 = (unsigned)requantize_one(v.y, s);
+      q2 = (unsigned)requantize_one(v.z, s);
+      q3 = (unsigned)requantize_one(v.w, s);
+    }
+    out[i] = q0 | (q1 << 8) | (q2 << 16) | (q3 << 24);
+  }
+}
+
+__global__ __launch_bounds__(256) void dequantize_kernel(const void* in, int inType, size_t total,
+                                                         const float* minV, const float* maxV, float* out) {
+  const float mn = *minV, mx = *maxV;
+  const IntRange r = int_range(inType);
+  double scale = 0, minRounded = 0;
+  const bool constant = mn >= mx;  // tfcc_mklquantizationinterface.cpp:321-324
+  if (!constant) dequantized_scale_info(r.bits, mn, mx, &scale, &minRounded);
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t step = (size_t)gridDim.x * blockDim.x;
+  for (; i < total; i += step) {
+    if (constant) {
+      out[i] = mn;
+    } else {
+      double off = (double)load_typed(in, inType, i) - (double)r.lowest;
+      out[i] = (float)fma(off, scale, minRounded);
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void quantize_kernel(const float* in, size_t total, const float* minV,
+                                                       const float* maxV, void* out, int outType, int fromData) {
+  const float mn = *minV, mx = *maxV;
+  const IntRange r = int_range(outType);
+  // given range: min >= max fills with lowest (tfcc_mklquantizationinterface.cpp:229-232);
+  // range taken from the data: min == max fills with lowest (:58-61)
+  const bool fillLowest = fromData ? (mn == mx) : (mn >= mx);
+  double scale = 0;
+  long long offset = 0;
+  if (!fillLowest) quantized_scale_info(r.bits, mn, mx, &scale, &offset);
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t step = (size_t)gridDim.x * blockDim.x;
+  for (; i < total; i += step) {
+    long long q = r.lowest;
+    if (!fillLowest) {
+      q = to_int64_x86(rint((double)in[i] * scale));
+      q = (long long)((unsigned long long)q - (unsigned long long)offset + (unsigned long long)r.lowest);
+      q = q < r.lowest ? r.lowest : q;
+      q = q > r.highest ? r.highest : q;
+    }
+    store_typed(out, outType, i, q);
+  }
+}
+
+// min / max of a float tensor.  Monotone uint encoding so that unsigned atomics order floats.
+__device__ __forceinline__ unsigned enc(float f) {
+  unsigned u = __float_as_uint(f);
+  return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float dec(unsigned u) {
+  return __uint_as_float((u & 0x80000000u) ? (u & 0x7fffffffu) : ~u);
+}
+
+__global__ void minmax_init_kernel(unsigned* scratch) {
+  scratch[0] = 0xffffffffu;  // min
+  scratch[1] = 0u;           // max
+}
+
+__global__ __launch_bounds__(256) void minmax_kernel(const float* in, size_t total, unsigned* scratch) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t step = (size_t)gridDim.x * blockDim.x;
+  float mn = 3.402823466e+38f, mx = -3.402823466e+38f;
+  for (; i < total; i += step) {
+    float v = in[i];
+    mn = fminf(mn, v);
+    mx = fmaxf(mx, v);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    mn = fminf(mn, __shfl_down(mn, off, 64));
+    mx = fmaxf(mx, __shfl_down(mx, off, 64));
+  }
+  if ((threadIdx.x & 63) == 0) {
+    atomicMin(&scratch[0], enc(mn));
+    atomicMax(&scratch[1], enc(mx));
+  }
+}
+
+__global__ void minmax_finish_kernel(const unsigned* scratch, float* mn, float* mx) {
+  *mn = dec(scratch[0]);
+  *mx = dec(scratch[1]);
+}
+
+unsigned grid_for(size_t total, unsigned perThread = 1) {
+  size_t blocks = (total + 256ull * perThread - 1) / (256ull * perThread);
+  if (blocks > 256u * 32u) blocks = 256u * 32u;
+  if (blocks < 1) blocks = 1;
+  return (unsigned)blocks;
+}
+
+bool valid_type(int t) { return t >= TFCC_ROCM_S8 && t <= TFCC_ROCM_U32; }
+
+template <class T>
+int reduce_rows(hipStream_t s, const void* a, unsigned batch, unsigned row, unsigned col, int* out) {
+  unsigned long long rows = (unsigned long long)batch * row;
+  if (rows >= (1ull << 31)) return set_error(TFCC_ROCM_INVALID_ARGUMENT, "reduce_sum: too many rows");
+  unsigned blocks = (unsigned)((rows + 3) / 4);
+  hipLaunchKernelGGL(reduce_rows_kernel<T>, dim3(blocks), dim3(256), 0, s, static_cast<const T*>(a),
+                     (unsigned)rows, col, out);
+  return check_launch("reduce_sum rows");
+}
+
+template <class T>
+int reduce_cols(hipStream_t s, const void* a, unsigned batch, unsigned row, unsigned col, int* out) {
+  size_t n = (size_t)batch * col;
+  hipLaunchKernelGGL(zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, out, n);
+  if (int e = check_launch("reduce_sum cols (zero)")) return e;
+  const bool vec = sizeof(T) == 1 && col % 4 == 0 && (uintptr_t)a % 4 == 0;
+  const unsigned colBlocks = vec ? (col / 4 + 255) / 256 : (col + 255) / 256;
+  // enough row slabs for ~2048 workgroups
+  unsigned slabs = (2048 + colBlocks * batch - 1) / (colBlocks * batch);
+  if (slabs > (row + 31) / 32) slabs = (row + 31) / 32;
+  if (slabs < 1) slabs = 1;
+  if (slabs > 65535) slabs = 65535;
+  if (batch > 65535) return set_error(TFCC_ROCM_INVALID_ARGUMENT, "reduce_sum: batch too large");
+  const unsigned rowsPerSlab = (row + slabs - 1) / slabs;
+  slabs = (row + rowsPerSlab - 1) / rowsPerSlab;
+  if (vec)
+    hipLaunchKernelGGL(reduce_cols_vec_kernel<T>, dim3(colBlocks, slabs, batch), dim3(256), 0, s,
+                       static_cast<const T*>(a), row, col, rowsPerSlab, out);
+  else
+    hipLaunchKernelGGL(reduce_cols_kernel<T>, dim3(colBlocks, slabs, batch), dim3(256), 0, s,
+                       static_cast<const T*>(a), row, col, rowsPerSlab, out);
+  return check_launch("reduce_sum cols");
+}
+
+// scratch for quantize_minmax: two words per device, allocated once
+unsigned* g_minmax[16] = {};
+
+}  // namespace
+}  // namespace tfcc_rocm
+
+using namespace tfcc_rocm;
+
+extern "C" {
+
+int tfcc_rocm_reduce_sum_rows(void* stream, const void* a, int type, unsigned batch, unsigned row,
+                              unsigned col, int32_t* out) {
+  TFCC_REQUIRE(a && out, "reduce_sum: null argument");
+  TFCC_REQUIRE(batch > 0 && row > 0 && col > 0, "reduce_sum: empty tensor");
+  switch (type) {
+    case TFCC_ROCM_S8: return reduce_rows<int8_t>(as_stream(stream), a, batch, row, col, out);
+    case TFCC_ROCM_U8: return reduce_rows<uint8_t>(as_stream(stream), a, batch, row, col, out);
+    case TFCC_ROCM_S16: return reduce_rows<int16_t>(as_stream(stream), a, batch, row, col, out);
+  }
+  return set_error(TFCC_ROCM_INVALID_ARGUMENT, "reduce_sum: type %d (int8, uint8 or int16)", type);
+}
+
+int tfcc_rocm_reduce_sum_cols(void* stream, const void* a, int type, unsigned batch, unsigned row,
+                              unsigned col, int32_t* out) {
+  TFCC_REQUIRE(a && out, "reduce_sum: null argument");
+  TFCC_REQUIRE(batch > 0 && row > 0 && col > 0, "reduce_sum: empty tensor");
+  switch (type) {
+    case TFCC_ROCM_S8: return reduce_cols<int8_t>(as_stream(stream), a, batch, row, col, out);
+    case TFCC_ROCM_U8: return reduce_cols<uint8_t>(as_stream(stream), a, batch, row, col, out);
+    case TFCC_ROCM_S16: return reduce_cols<int16_t>(as_stream(stream), a, batch, row, col, out);
+  }
+  return set_error(TFCC_ROCM_INVALID_ARGUMENT, "reduce_sum: type %d (int8, uint8 or int16)", type);
+}
+
+int tfcc_rocm_requantize(void* stream, const void* in, int in_type, void* out, int out_type,
+                         uint64_t total, const float* min_in, const float* max_in,
+                         const float* min_out, const float* max_out) {
+  TFCC_REQUIRE(in && out && min_in && max_in && min_out && max_out, "requantize: null argument");
+  TFCC_REQUIRE(total > 0, "requantize: empty tensor");
+  TFCC_REQUIRE(valid_type(in_type) && valid_type(out_type), "requantize: bad type code");
+  hipStream_t s = as_stream(stream);
+  if (in_type == TFCC_ROCM_S32 && out_type == TFCC_ROCM_U8 && total % 4 == 0 && (uintptr_t)in % 16 == 0 &&
+      (uintptr_t)out % 4 == 0) {
+    hipLaunchKernelGGL(requantize_s32_u8_vec_kernel, dim3(grid_for(total / 4)), dim3(256), 0, s,
+                       static_cast<const int4*>(in), static_cast<unsigned*>(out), (size_t)(total / 4), min_in,
+                       max_in, min_out, max_out);
+  } else {
+    hipLaunchKernelGGL(requantize_kernel, dim3(grid_for(total)), dim3(256), 0, s, in, in_type, out, out_type,
+                       (size_t)total, min_in, max_in, min_out, max_out);
+  }
+  return check_launch("requantize");
+}
+
+int tfcc_rocm_dequantize(void* stream, const void* in, int in_type, uint64_t total,
+                         const float* min_v, const float* max_v, float* out) {
+  TFCC_REQUIRE(in && out && min_v && max_v, "dequantize: null argument");
+  TFCC_REQUIRE(total > 0, "dequantize: empty tensor");
+  TFCC_REQUIRE(valid_type(in_type), "dequantize: bad type code");
+  hipLaunchKernelGGL(dequantize_kernel, dim3(grid_for(total)), dim3(256), 0, as_stream(stream), in, in_type,
+                     (size_t)total, min_v, max_v, out);
+  return check_launch("dequantize");
+}
+
+int tfcc_rocm_quantize(void* stream, const float* in, uint64_t total, const float* min_v,
+                       const float* max_v, void* out, int out_type) {
+  TFCC_REQUIRE(in && out && min_v && max_v, "quantize: null argument");
+  TFCC_REQUIRE(total > 0, "quantize: empty tensor");
+  TFCC_REQUIRE(valid_type(out_type), "quantize: bad type code");
+  hipLaunchKernelGGL(quantize_kernel, dim3(grid_for(total)), dim3(256), 0, as_stream(stream), in, (size_t)total,
+                     min_v, max_v, out, out_type, 0);
+  return check_launch("quantize");
+}
+
+int tfcc_rocm_quantize_minmax(void* stream, const float* in, uint64_t total, void* out,
+                              int out_type, float* min_v, float* max_v) {
+  TFCC_REQUIRE(in && out && min_v && max_v, "quantize: null argument");
+  TFCC_REQUIRE(total > 0, "quantize: empty tensor");
+  TFCC_REQUIRE(valid_type(out_type), "quantize: bad type code");
+  int dev = 0;
+  TFCC_HIP_CHECK(hipGetDevice(&dev));
+  TFCC_REQUIRE(dev >= 0 && dev < 16, "quantize: device index %d", dev);
+  if (!g_minmax[dev]) TFCC_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&g_minmax[dev]), 2 * sizeof(unsigned)));
+  hipStream_t s = as_stream(stream);
+  hipLaunchKernelGGL(minmax_init_kernel, dim3(1), dim3(1), 0, s, g_minmax[dev]);
+  hipLaunchKernelGGL(minmax_kernel, dim3(grid_for(total, 4)), dim3(256), 0, s, in, (size_t)total, g_minmax[dev]);
+  hipLaunchKernelGGL(minmax_finish_kernel, dim3(1), dim3(1), 0, s, g_minmax[dev], min_v, max_v);
+  hipLaunchKernelGGL(quantize_kernel, dim3(grid_for(total)), dim3(256), 0, s, in, (size_t)total, min_v, max_v, out,
+                     out_type, 1);
+  return check_launch("quantize");
+}
+
+}  // extern "C"

@@ -1,0 +1,289 @@
+// fp32 strided-batched matrix product on the gfx950 fp32 matrix cores with the bias add fused
+// into the tile store.
+//
+// Replaces the oneDNN calls of tfcc/mkl/interfaces/tfcc_mklblasinterface.cpp:41-67 (matmul) and
+// :69-78,87-118 (bias pre-fill + accumulate), with the same argument meaning: row-major operands,
+// batch strides in elements, stride 0 = operand shared by every batch.
+//
+// A workgroup of four wavefronts owns a BM x BN tile of one batch entry and walks K in slabs of
+// BK = 32.  Both slabs are kept in LDS with k contiguous (As[row][k], Bs[col][k]) so that a lane
+// fetches the operands of four v_mfma_f32_32x32x2_f32 steps with one 128-bit LDS read: lane
+// (i, g) holds k = 8*kb + 4*g + s of row/column i for step s, for A and B alike.  B is row-major
+// [K,N] in HBM: every thread loads a 4(k) x 4(n) block as four 128-bit rows, transposes it by
+// register renaming and writes four 128-bit chunks.  16-byte chunks are xor-swizzled by the row
+// index, and tile columns are stored interleaved (LDS row j*32+i holds tile column NI*i+j of the
+// wavefront's column range) so that a lane owns NI consecutive output columns.
+#include "common.hpp"
+
+namespace tfcc_rocm {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+namespace {
+
+struct SgemmParams {
+  const float* A;
+  const float* B;
+  const float* bias;
+  float* C;
+  unsigned long long strideA, strideB, strideC;
+  unsigned M, N, K, batch;
+  unsigned tilesM, tilesN, tilesTotal, chunk;
+};
+
+constexpr int kThreads = 256;
+constexpr int BK = 32;
+constexpr int CH = BK / 4;  // 16-byte chunks per LDS row
+
+__device__ __forceinline__ int swz(int row, int chunk) { return chunk ^ ((row >> 1) & (CH - 1)); }
+
+// WGM x WGN wavefronts, each owning an (MI*32) x (NI*32) sub-tile
+template <int WGM, int WGN, int MI, int NI, bool VEC>
+__global__ __launch_bounds__(kThreads) void sgemm_kernel(const SgemmParams p) {
+  static_assert(WGM * WGN == 4, "four wavefronts");
+  constexpr int BM = WGM * MI * 32, BN = WGN * NI * 32;
+  constexpr int WM = MI * 32, WN = NI * 32;
+  constexpr int A_TOTAL = BM * CH, B_TOTAL = (BN / 4) * CH;    // 128-bit chunks of A, 4x4 blocks of B
+  constexpr int A_ITEMS = (A_TOTAL + kThreads - 1) / kThreads;  // per thread
+  constexpr int B_ITEMS = (B_TOTAL + kThreads - 1) / kThreads;
+
+  extern __shared__ __align__(16) float smemf[];
+  float* As = smemf;                 // [2][BM][BK]
+  float* Bs = smemf + 2 * BM * BK;   // [2][BN][BK]
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave / WGN, wn = wave % WGN;
+
+  unsigned tm, tn, bi;
+  {
+    // consecutive workgroup ids land on different XCDs: hand each XCD a contiguous run of tiles
+    const unsigned wg = blockIdx.x;
+    const unsigned xcd = wg & 7u, slot = wg >> 3;
+    const unsigned L = xcd * p.chunk + slot;
+    if (slot >= p.chunk || L >= p.tilesTotal) return;
+    const unsigned perBatch = p.tilesM * p.tilesN;
+    bi = L / perBatch;
+    unsigned t = L - bi * perBatch;
+    const unsigned band = 4u * p.tilesN;
+    unsigned g = t / band;
+    unsigned rowsInBand = min(4u, p.tilesM - g * 4u);
+    unsigned r = t - g * band;
+    tm = g * 4u + r % rowsInBand;
+    tn = r / rowsInBand;
+  }
+  const unsigned m0 = tm * BM, n0 = tn * BN;
+  const unsigned M = p.M, N = p.N, K = p.K;
+  const float* __restrict__ A = p.A + (size_t)bi * p.strideA;
+  const float* __restrict__ B = p.B + (size_t)bi * p.strideB;
+
+  v16f acc[MI][NI];
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int j = 0; j < NI; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  v4f aReg[A_ITEMS];
+  v4f bReg[B_ITEMS][4];
+
+  // Vector path: raw buffer loads, an offset past the end of the operand reads zero (rows >= M of
+  // A, rows >= K of B).  The k tail of an A row is zeroed explicitly: it would otherwise meet the
+  // zero rows of B as garbage that may be Inf/NaN.
+  const __amdgpu_buffer_rsrc_t rsrcA =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(A), 0, VEC ? (int)(M * K * 4u) : 0, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrcB =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(B), 0, VEC ? (int)(K * N * 4u) : 0, 0x00020000);
+
+  auto loadA = [&](unsigned k0) {
+#pragma unroll
+    for (int it = 0; it < A_ITEMS; ++it) {
+      const int w = tid + it * kThreads;
+      if (A_TOTAL % kThreads != 0 && w >= A_TOTAL) break;
+      const int row = w / CH, ch = w % CH;
+      const unsigned gr = m0 + row, gk = k0 + ch * 4;
+      v4f v = {0.f, 0.f, 0.f, 0.f};
+      if constexpr (VEC) {
+        v4f t = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rsrcA, (gr * K + gk) * 4u, 0, 0));
+        v = gk < K ? t : v;
+      } else {
+        if (gr < M) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            if (gk + q < K) v[q] = A[(size_t)gr * K + gk + q];
+        }
+      }
+      aReg[it] = v;
+    }
+  };
+  auto loadB = [&](unsigned k0) {
+#pragma unroll
+    for (int it = 0; it < B_ITEMS; ++it) {
+      const int w = tid + it * kThreads;
+      if (B_TOTAL % kThreads != 0 && w >= B_TOTAL) break;
+      const int nq = w % (BN / 4), kq = w / (BN / 4);
+      const unsigned gn = n0 + nq * 4, gk = k0 + kq * 4;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        v4f v = {0.f, 0.f, 0.f, 0.f};
+        if constexpr (VEC) {
+          v = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rsrcB, ((gk + q) * N + gn) * 4u, 0, 0));
+        } else {
+          if (gk + q < K) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+              if (gn + e < N) v[e] = B[(size_t)(gk + q) * N + gn + e];
+          }
+        }
+        bReg[it][q] = v;
+      }
+    }
+  };
+  auto storeTiles = [&](int buf) {
+    float* as = As + buf * BM * BK;
+    float* bs = Bs + buf * BN * BK;
+#pragma unroll
+    for (int it = 0; it < A_ITEMS; ++it) {
+      const int w = tid + it * kThreads;
+      if (A_TOTAL % kThreads != 0 && w >= A_TOTAL) break;
+      const int row = w / CH, ch = w % CH;
+      *reinterpret_cast<v4f*>(as + row * BK + swz(row, ch) * 4) = aReg[it];
+    }
+#pragma unroll
+    for (int it = 0; it < B_ITEMS; ++it) {
+      const int w = tid + it * kThreads;
+      if (B_TOTAL % kThreads != 0 && w >= B_TOTAL) break;
+      const int nq = w % (BN / 4), kq = w / (BN / 4);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int n = nq * 4 + j;
+        const int wnn = n / WN, within = n % WN;
+        const int row = wnn * WN + (within % NI) * 32 + within / NI;
+        v4f v = {bReg[it][0][j], bReg[it][1][j], bReg[it][2][j], bReg[it][3][j]};
+        *reinterpret_cast<v4f*>(bs + row * BK + swz(row, kq) * 4) = v;
+      }
+    }
+  };
+
+  const unsigned KT = (K + BK - 1) / BK;
+  loadA(0);
+  loadB(0);
+  storeTiles(0);
+  __syncthreads();
+
+  const int lrow = lane & 31, g = lane >> 5;
+  for (unsigned kt = 0; kt < KT; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < KT) {
+      loadA((kt + 1) * BK);
+      loadB((kt + 1) * BK);
+    }
+    const float* as = As + buf * BM * BK + (wm * WM) * BK;
+    const float* bs = Bs + buf * BN * BK + (wn * WN) * BK;
+#pragma unroll
+    for (int kb = 0; kb < BK / 8; ++kb) {
+      v4f af[MI], bf[NI];
+#pragma unroll
+      for (int i = 0; i < MI; ++i) {
+        const int row = i * 32 + lrow;
+        af[i] = *reinterpret_cast<const v4f*>(as + row * BK + swz(row, kb * 2 + g) * 4);
+      }
+#pragma unroll
+      for (int j = 0; j < NI; ++j) {
+        const int row = j * 32 + lrow;
+        bf[j] = *reinterpret_cast<const v4f*>(bs + row * BK + swz(row, kb * 2 + g) * 4);
+      }
+#pragma unroll
+      for (int s = 0; s < 4; ++s)
+#pragma unroll
+        for (int i = 0; i < MI; ++i)
+#pragma unroll
+          for (int j = 0; j < NI; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[i][s], bf[j][s], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < KT) storeTiles(buf ^ 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue: + bias, store.  Lane (i, g) owns columns NI*i .. NI*i+NI-1 of the wavefront's
+  // column range and rows 8*(r/4) + 4*g + r%4 of each 32-row block.
+  float* __restrict__ C = p.C + (size_t)bi * p.strideC;
+  const unsigned gcol = n0 + wn * WN + NI * lrow;
+  float bv[NI];
+#pragma unroll
+  for (int j = 0; j < NI; ++j) bv[j] = (p.bias && gcol + j < N) ? p.bias[gcol + j] : 0.f;
+  const bool vecOK = VEC && (gcol + NI <= N);
+#pragma unroll
+  for (int i = 0; i < MI; ++i) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const unsigned grow = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * g + (r & 3);
+      if (grow >= M) continue;
+      float v[NI];
+#pragma unroll
+      for (int j = 0; j < NI; ++j) v[j] = acc[i][j][r] + bv[j];
+      const size_t off = (size_t)grow * N + gcol;
+      if (vecOK) {
+        if constexpr (NI == 4) *reinterpret_cast<v4f*>(C + off) = v4f{v[0], v[1], v[2], v[3]};
+        else if constexpr (NI == 2) *reinterpret_cast<float2*>(C + off) = make_float2(v[0], v[1]);
+        else C[off] = v[0];
+      } else {
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+          if (gcol + j < N) C[off + j] = v[j];
+      }
+    }
+  }
+}
+
+template <int WGM, int WGN, int MI, int NI, bool VEC>
+int launch(hipStream_t stream, SgemmParams p) {
+  constexpr int BM = WGM * MI * 32, BN = WGN * NI * 32;
+  p.tilesM = (p.M + BM - 1) / BM;
+  p.tilesN = (p.N + BN - 1) / BN;
+  unsigned long long total = (unsigned long long)p.tilesM * p.tilesN * p.batch;
+  if (total > 0x7fffffffull) return set_error(TFCC_ROCM_INVALID_ARGUMENT, "sgemm: too many tiles");
+  p.tilesTotal = (unsigned)total;
+  p.chunk = (p.tilesTotal + 7) / 8;
+  constexpr size_t lds = 2 * (size_t)(BM + BN) * BK * sizeof(float);
+  auto kern = sgemm_kernel<WGM, WGN, MI, NI, VEC>;
+  static bool attrSet = false;
+  if (!attrSet) {
+    TFCC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attrSet = true;
+  }
+  hipLaunchKernelGGL(kern, dim3(p.chunk * 8), dim3(kThreads), lds, stream, p);
+  return check_launch("sgemm");
+}
+
+}  // namespace
+}  // namespace tfcc_rocm
+
+using namespace tfcc_rocm;
+
+extern "C" int tfcc_rocm_sgemm_strided_batched(void* stream, const float* a, uint64_t stride_a,
+                                               const float* b, uint64_t stride_b, const float* bias,
+                                               float* c, uint64_t stride_c, unsigned m, unsigned n,
+                                               unsigned k, unsigned batch) {
+  TFCC_REQUIRE(a && b && c, "sgemm: null operand");
+  TFCC_REQUIRE(m > 0 && n > 0 && k > 0 && batch > 0, "sgemm: empty operand");
+  SgemmParams p{};
+  p.A = a; p.B = b; p.bias = bias; p.C = c;
+  p.strideA = stride_a; p.strideB = stride_b; p.strideC = stride_c;
+  p.M = m; p.N = n; p.K = k; p.batch = batch;
+  const bool vec = (k % 4 == 0) && (n % 4 == 0) && ((uintptr_t)a % 16 == 0) && ((uintptr_t)b % 16 == 0) &&
+                   ((uintptr_t)c % 16 == 0) && (stride_a % 4 == 0) && (stride_b % 4 == 0) && (stride_c % 4 == 0) &&
+                   ((unsigned long long)m * k < (1ull << 30)) && (((unsigned long long)k + 64) * n + 1024 < (1ull << 30));
+  hipStream_t s = as_stream(stream);
+  // 128x128 tiles once there are enough of them to fill the 256 CUs twice over, else 64x64
+  const unsigned long long big = (unsigned long long)((m + 127) / 128) * ((n + 127) / 128) * batch;
+  if (vec) {
+    if (big >= 512) return launch<4, 1, 1, 4, true>(s, p);
+    return launch<2, 2, 1, 1, true>(s, p);
+  }
+  TFCC_REQUIRE((unsigned long long)m * n < (1ull << 32) && (unsigned long long)m * k < (1ull << 32) &&
+               (unsigned long long)k * n < (1ull << 32), "sgemm: operand larger than 2^32 elements");
+  return launch<2, 2, 1, 1, false>(s, p);
+}
