@@ -111,9 +111,21 @@ struct RequantScalars {
   long long inLowest, outLowest, outHighest;
   int mode;            // 0: per-element arithmetic, 1: fill with fillValue (degenerate ranges)
   long long fillValue;
+  double offsetMinusLowest;  // (double)(outOffset - outLowest), exact when fastOK
+  int fastOK;
 };
 
-__device__ static inline long long requantize_one(long long x, const RequantScalars& s) {
+// offMax = highest - lowest of the input type (its largest x - inLowest)
+__host__ __device__ static inline void finish_requant_scalars(RequantScalars& s, double offMax) {
+  const long long d = (long long)((unsigned long long)s.outOffset - (unsigned long long)s.outLowest);
+  s.offsetMinusLowest = (double)d;
+  // real = inMin + off * inScale is monotone in off, so its extremes are at off = 0 and off = offMax
+  const double r0 = fabs(s.inMin), r1 = fabs(fma(offMax, s.inScale, s.inMin));
+  const double bound = (r0 > r1 ? r0 : r1) * fabs(s.outScale);
+  s.fastOK = (d > -(1LL << 52) && d < (1LL << 52) && bound < 1125899906842624.0) ? 1 : 0;  // NaN compares false
+}
+
+__device__ static inline long long requantize_one_exact(long long x, const RequantScalars& s) {
   double off = (double)x - (double)s.inLowest;
   double real = fma(off, s.inScale, s.inMin);
   long long q = to_int64_x86(rint(real * s.outScale));
@@ -121,6 +133,17 @@ __device__ static inline long long requantize_one(long long x, const RequantScal
   q = q < s.outLowest ? s.outLowest : q;
   q = q > s.outHighest ? s.outHighest : q;
   return q;
+}
+
+// Same result with the integer tail evaluated in double, valid when RequantScalars::fastOK: then
+// |y| < 2^50 for every possible input and |outOffset - outLowest| < 2^52, so rint(y), the
+// subtraction and the clamp are exact in double.  `off` = x - inLowest as a double.
+__device__ static inline int requantize_one_fast(double off, const RequantScalars& s) {
+  const double y = fma(off, s.inScale, s.inMin) * s.outScale;
+  double q = rint(y) - s.offsetMinusLowest;
+  q = fmax(q, (double)s.outLowest);
+  q = fmin(q, (double)s.outHighest);
+  return (int)q;
 }
 
 // The branches of _requantize_helper (tfcc/mkl/interfaces/tfcc_mklquantizationinterface.cpp:121-141)
@@ -135,6 +158,8 @@ __host__ __device__ static inline RequantScalars make_requant_scalars(int inType
   s.fillValue = 0;
   s.inScale = s.inMin = s.outScale = 0.0;
   s.outOffset = 0;
+  s.fastOK = 0;
+  s.offsetMinusLowest = 0.0;
   if (minOut >= maxOut) {
     s.mode = 1;
     s.fillValue = ro.lowest;
@@ -150,6 +175,7 @@ __host__ __device__ static inline RequantScalars make_requant_scalars(int inType
     s.mode = 1;
     s.fillValue = q;
   }
+  finish_requant_scalars(s, (double)(ri.highest - ri.lowest));
   return s;
 }
 

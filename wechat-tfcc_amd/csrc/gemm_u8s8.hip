@@ -25,8 +25,11 @@
 // where rowsumA / colsumB are the caller's tensors (used as given, like the reference) and
 // colsum(B) is the true column sum, accumulated on the fly from the transposed B registers with
 // v_dot4_i32_i8 so that no assumption about the caller's tensors is needed.
+#include <type_traits>
+
 #include "common.hpp"
 #include "gemv.hpp"
+#include "qgemm_dma.hpp"
 #include "qgemm_params.hpp"
 
 namespace tfcc_rocm {
@@ -289,6 +292,7 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(const QGemmParams p) {
     } else {
       rq.inScale = p.inScale; rq.inMin = p.inMin; rq.outScale = p.outScale; rq.outOffset = p.outOffset;
       rq.inLowest = -2147483648LL; rq.outLowest = 0; rq.outHighest = 255; rq.mode = 0; rq.fillValue = 0;
+      finish_requant_scalars(rq, 4294967295.0);
     }
   }
 
@@ -301,40 +305,61 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(const QGemmParams p) {
   for (int j = 0; j < NI; ++j) ct[j] = colTerm[colBase + j];
   const bool vecOK = ALIGNED && (gcol + NI <= N);     // N % 4 == 0 and base pointers aligned when ALIGNED
 
+  // FLAVOUR 0: int32 only; 1: requantize, fast double path; 2: requantize, exact int64 path; 3: constant fill
+  auto storeTile = [&](auto flavour) {
+    constexpr int FLAVOUR = decltype(flavour)::value;
 #pragma unroll
-  for (int i = 0; i < MI; ++i) {
+    for (int i = 0; i < MI; ++i) {
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int trow = wm * WM + i * 32 + 8 * (r / 4) + 4 * khalf + (r & 3);
-      const unsigned grow = m0 + trow;
-      if (grow >= M) continue;
-      const int rt = rowTerm[trow];
-      int v[NI];
+      for (int r = 0; r < 16; ++r) {
+        const int trow = wm * WM + i * 32 + 8 * (r / 4) + 4 * khalf + (r & 3);
+        const unsigned grow = m0 + trow;
+        if (grow >= M) continue;
+        const int rt = rowTerm[trow];
+        int v[NI];
 #pragma unroll
-      for (int j = 0; j < NI; ++j) v[j] = (int)((unsigned)acc[i][j][r] + (unsigned)rt + (unsigned)ct[j]);
-      const size_t off = (size_t)grow * N + gcol;
-      if (C) {
-        if (vecOK) {
-          if constexpr (NI == 4) *reinterpret_cast<v4i*>(C + off) = v4i{v[0], v[1], v[2], v[3]};
-          else *reinterpret_cast<int2*>(C + off) = make_int2(v[0], v[1]);
-        } else {
+        for (int j = 0; j < NI; ++j) v[j] = (int)((unsigned)acc[i][j][r] + (unsigned)rt + (unsigned)ct[j]);
+        const size_t off = (size_t)grow * N + gcol;
+        if (C) {
+          if (vecOK) {
+            if constexpr (NI == 4) *reinterpret_cast<v4i*>(C + off) = v4i{v[0], v[1], v[2], v[3]};
+            else *reinterpret_cast<int2*>(C + off) = make_int2(v[0], v[1]);
+          } else {
 #pragma unroll
-          for (int j = 0; j < NI; ++j) if (gcol + j < N) C[off + j] = v[j];
+            for (int j = 0; j < NI; ++j) if (gcol + j < N) C[off + j] = v[j];
+          }
         }
-      }
-      if (REQUANT) {
-        unsigned q[NI];
+        if constexpr (FLAVOUR != 0) {
+          unsigned q[NI];
 #pragma unroll
-        for (int j = 0; j < NI; ++j) q[j] = rq.mode ? (unsigned)rq.fillValue : (unsigned)requantize_one((long long)v[j], rq);
-        if (vecOK) {
-          if constexpr (NI == 4) *reinterpret_cast<unsigned*>(Q + off) = q[0] | (q[1] << 8) | (q[2] << 16) | (q[3] << 24);
-          else *reinterpret_cast<unsigned short*>(Q + off) = (unsigned short)(q[0] | (q[1] << 8));
-        } else {
+          for (int j = 0; j < NI; ++j) {
+            if constexpr (FLAVOUR == 1) {
+              // (double)(v - INT32_MIN) without a 64-bit integer: flip the sign bit, convert as unsigned
+              q[j] = (unsigned)requantize_one_fast((double)((unsigned)v[j] ^ 0x80000000u), rq);
+            } else if constexpr (FLAVOUR == 2) {
+              q[j] = (unsigned)requantize_one_exact((long long)v[j], rq);
+            } else {
+              q[j] = (unsigned)rq.fillValue;
+            }
+          }
+          if (vecOK) {
+            if constexpr (NI == 4) *reinterpret_cast<unsigned*>(Q + off) = q[0] | (q[1] << 8) | (q[2] << 16) | (q[3] << 24);
+            else *reinterpret_cast<unsigned short*>(Q + off) = (unsigned short)(q[0] | (q[1] << 8));
+          } else {
 #pragma unroll
-          for (int j = 0; j < NI; ++j) if (gcol + j < N) Q[off + j] = (unsigned char)q[j];
+            for (int j = 0; j < NI; ++j) if (gcol + j < N) Q[off + j] = (unsigned char)q[j];
+          }
         }
       }
     }
+  };
+  if constexpr (!REQUANT) {
+    storeTile(std::integral_constant<int, 0>{});
+  } else {
+    // uniform over the whole launch: every wavefront takes the same branch
+    if (rq.mode) storeTile(std::integral_constant<int, 3>{});
+    else if (rq.fastOK) storeTile(std::integral_constant<int, 1>{});
+    else storeTile(std::integral_constant<int, 2>{});
   }
 }
 
@@ -361,6 +386,7 @@ int launch(hipStream_t stream, QGemmParams p) {
 
 template <bool REQUANT>
 int dispatch(hipStream_t stream, const QGemmParams& p) {
+  if (qgemm_dma_supported(p, REQUANT)) return qgemm_dma_launch(stream, p, REQUANT);
   const bool aligned = (p.K % 16 == 0) && (p.N % 4 == 0) && ((uintptr_t)p.A % 16 == 0) &&
                        ((uintptr_t)p.B % 4 == 0) && (p.strideA % 16 == 0) && (p.strideB % 4 == 0) &&
                        (p.C == nullptr || ((uintptr_t)p.C % 16 == 0 && p.strideC % 4 == 0)) &&
@@ -409,7 +435,7 @@ extern "C" int tfcc_rocm_gemm_u8s8s32(void* stream, const tfcc_rocm_qgemm_desc* 
     const float* ranges[4] = {p.minA, p.maxA, p.minB, p.maxB};
     float* rangeOut[2] = {p.minC, p.maxC};
     return gemv_launch(as_stream(stream), p.A, p.B, p.rowsumA, p.colsumB, p.offsetA, p.offsetB, ranges, rangeOut,
-                       p.M, p.N, p.K, c, 0.f, nullptr, nullptr, 0);
+                       p.M, p.N, p.K, c, 0.f, nullptr, nullptr);
   }
   return dispatch<false>(as_stream(stream), p);
 }

@@ -1,0 +1,373 @@
+// uint8 x int8 -> int32 matrix product for large aligned shapes: the gfx950-specific pipeline.
+//
+// Same arithmetic as the kernel in gemm_u8s8.hip (which stays the path for unaligned and small
+// shapes); replaces tfcc/mkl/operations/tfcc_mklquantization.cpp:33-69,176-201 and the blocked CPU
+// GEMM below it (tfcc/mkl/gemm/tfcc_mklsinglethreadgemm.h:93-141, tfcc_mklmatmulkernel.h:142-260).
+//
+// Data path of one BM x BN tile (four wavefronts, 2 x 2):
+//   HBM -> LDS  buffer_load_dwordx4 ... lds (asynchronous, no VGPRs): every K slab of 64 bytes is
+//               copied as it lies in memory, A rows as As[row][64] and B rows as Bs[k][BN], into a
+//               ring of STAGES LDS buffers, STAGES-1 slabs ahead of the matrix cores.  Out-of-range
+//               rows read zero through the buffer descriptor.  The 16-byte chunk a lane copies is
+//               chosen so that the LDS image is xor-swizzled (the DMA writes lanes contiguously).
+//   LDS -> VGPR A: ds_read_b128 (16 consecutive k of a row), xor 0x80 turns uint8 into int8.
+//               B: k is the strided dimension of Bs, and the matrix core wants 16 consecutive k
+//               per lane: ds_read_b64_tr_b8 transposes 8(k) x 16(n) byte blocks on the way out of
+//               LDS, two of them give a lane its 16 k for one column.
+//   MFMA        v_mfma_i32_32x32x32_i8 with the operands swapped (D = B^T A^T), so that a lane owns
+//               four consecutive columns of one row of C in each accumulator quad.
+//   epilogue    offset terms (see gemm_u8s8.hip), then either 128-bit int32 stores or the fused
+//               requantize: four uint8 packed per lane, staged through LDS, written as whole
+//               256-byte row segments.
+// The true column sums of B (needed because a' = a - 128) are accumulated from the B operands with
+// v_dot4_i32_i8 by the two wavefronts of the first tile row.
+#include <type_traits>
+
+#include "common.hpp"
+#include "qgemm_dma.hpp"
+
+namespace tfcc_rocm {
+
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int BK = 64;
+
+// One asynchronous 16-byte-per-lane copy HBM -> LDS.  The LDS address of lane i is ldsBase + 16*i
+// (ldsBase wave-uniform, goes through M0); voffset is the lane's byte offset into the buffer.
+// Inline asm on purpose: the outstanding-copy count is managed by hand (s_waitcnt vmcnt) so that
+// several slabs stay in flight across iterations.
+__device__ __forceinline__ v4i make_rsrc(const void* base, unsigned bytes) {
+  const unsigned long long a = reinterpret_cast<unsigned long long>(base);
+  v4i r;
+  r[0] = __builtin_amdgcn_readfirstlane((int)(unsigned)a);
+  r[1] = __builtin_amdgcn_readfirstlane((int)((unsigned)(a >> 32) & 0xffffu));
+  r[2] = __builtin_amdgcn_readfirstlane((int)bytes);
+  r[3] = 0x00020000;
+  return r;
+}
+
+__device__ __forceinline__ void dma16(v4i rsrc, unsigned ldsBase, unsigned voffset) {
+  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+               :
+               : "s"(ldsBase), "v"(voffset), "s"(rsrc)
+               : "memory", "m0");
+}
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  // s_waitcnt simm16: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt_hi[15:14]; leave the others at max
+  static_assert(N >= 0 && N < 64, "vmcnt range");
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0f70);
+}
+
+__device__ __forceinline__ int swzA(int row) { return ((row >> 1) & 3) ^ ((row >> 3) & 1); }
+
+template <int BM, int BN, int STAGES, bool REQUANT>
+__global__ __launch_bounds__(kThreads) void qgemm_dma_kernel(const QGemmParams p) {
+  constexpr int WM = BM / 2, WN = BN / 2;
+  constexpr int MI = WM / 32, NI = WN / 32;
+  constexpr int A_BYTES = BM * BK, B_BYTES = BK * BN, STAGE_BYTES = A_BYTES + B_BYTES;
+  constexpr int A_COPIES = A_BYTES / 16 / kThreads, B_COPIES = B_BYTES / 16 / kThreads;
+  constexpr int COPIES = A_COPIES + B_COPIES;  // per thread per slab
+  constexpr int BCH = BN / 16;                 // 16-byte chunks per B row
+  static_assert(BCH >= 8 && (BCH & (BCH - 1)) == 0, "B swizzle needs at least 8 chunks per row");
+  static_assert(COPIES * (STAGES - 1) < 64, "vmcnt range");
+
+  extern __shared__ __align__(16) unsigned char smem[];
+  const unsigned ldsBase = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)smem;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept in an SGPR
+  const int wm = wave >> 1, wn = wave & 1;
+
+  unsigned tm, tn, bi;
+  {
+    // consecutive workgroup ids go to different XCDs: each XCD gets a contiguous run of tiles,
+    // ordered in bands of 4 tile rows
+    const unsigned wg = blockIdx.x;
+    const unsigned xcd = wg & 7u, slot = wg >> 3;
+    const unsigned L = xcd * p.chunk + slot;
+    if (slot >= p.chunk || L >= p.tilesTotal) return;
+    const unsigned perBatch = p.tilesM * p.tilesN;
+    bi = L / perBatch;
+    unsigned t = L - bi * perBatch;
+    const unsigned band = 4u * p.tilesN;
+    unsigned g = t / band;
+    unsigned rowsInBand = min(4u, p.tilesM - g * 4u);
+    unsigned r = t - g * band;
+    tm = g * 4u + r % rowsInBand;
+    tn = r / rowsInBand;
+  }
+  const unsigned m0 = tm * BM, n0 = tn * BN;
+  const unsigned M = p.M, N = p.N, K = p.K;
+  const unsigned char* A = p.A + (size_t)bi * p.strideA;
+  const signed char* B = p.B + (size_t)bi * p.strideB;
+  // buffer descriptors: base, 0 stride, size in bytes, raw 32-bit format; held in SGPRs
+  const v4i rsrcA = make_rsrc(A, M * K);
+  const v4i rsrcB = make_rsrc(B, K * N);
+
+  int offA = p.offsetA, offB = p.offsetB;
+  float minC = 0.f, maxC = 0.f;
+  if (p.minA) {
+    float mnA = *p.minA, mxA = *p.maxA, mnB = *p.minB, mxB = *p.maxB;
+    qmatmul_offsets(mnA, mxA, mnB, mxB, &offA, &offB);
+    qmatmul_range(mnA, mxA, mnB, mxB, &minC, &maxC);
+    if (blockIdx.x == 0 && tid == 0) {
+      if (p.minC) *p.minC = minC;
+      if (p.maxC) *p.maxC = maxC;
+    }
+  }
+
+  // ---- per-thread copy descriptors: which 16 bytes of the slab this lane moves in each copy.
+  // LDS slot s (16 bytes) of the A image holds row s/4, physical chunk s%4 = logical chunk ^ swzA(row).
+  unsigned aOff[A_COPIES], bOff[B_COPIES];  // byte offsets into A / B for slab 0
+#pragma unroll
+  for (int c = 0; c < A_COPIES; ++c) {
+    const int s = c * kThreads + tid;
+    const int row = s >> 2, phys = s & 3;
+    aOff[c] = (m0 + row) * K + ((phys ^ swzA(row)) << 4);
+  }
+  // LDS slot s of the B image holds k row s/BCH, physical chunk s%BCH = logical chunk ^ (k & 7).
+#pragma unroll
+  for (int c = 0; c < B_COPIES; ++c) {
+    const int s = c * kThreads + tid;
+    const int k = s / BCH, phys = s % BCH;
+    bOff[c] = k * N + n0 + ((phys ^ (k & 7)) << 4);
+  }
+  auto issueSlab = [&](unsigned slab) {
+    const unsigned stage = slab % STAGES;
+    const unsigned base = __builtin_amdgcn_readfirstlane(ldsBase + stage * STAGE_BYTES + wave * 1024);
+    const unsigned k0 = slab * BK;
+#pragma unroll
+    for (int c = 0; c < A_COPIES; ++c) dma16(rsrcA, base + c * (kThreads * 16), aOff[c] + k0);
+#pragma unroll
+    for (int c = 0; c < B_COPIES; ++c) dma16(rsrcB, base + A_BYTES + c * (kThreads * 16), bOff[c] + k0 * N);
+  };
+
+  v16i acc[MI][NI];
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int j = 0; j < NI; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+  int colsum[NI];
+#pragma unroll
+  for (int j = 0; j < NI; ++j) colsum[j] = 0;
+
+  // ---- operand addresses inside a stage
+  const int l32 = lane & 31, g = lane >> 5;
+  // A: row wm*WM + 32*i + l32, logical chunk 2*ks + g
+  int aAddr[MI][2];
+#pragma unroll
+  for (int i = 0; i < MI; ++i)
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      const int row = wm * WM + 32 * i + l32;
+      aAddr[i][ks] = row * BK + (((2 * ks + g) ^ swzA(row)) << 4);
+    }
+  // B: transposing read.  Within a block of 16 lanes, lane s points at k row (s >> 1) and 8-byte
+  // column half (s & 1); the lane then receives, for column 8*(l&8 ? 1 : 0) + (l & 7) of the 16, the
+  // bytes of k rows 0..7.  Lane blocks: (lane >> 4) & 1 selects the 16-column half of the 32-column
+  // MFMA block, lane >> 5 the k half (g).
+  const int s16 = lane & 15, colHalf = (lane >> 4) & 1;
+  const int trK = s16 >> 1;           // k row within a group of 8
+  const int trByte = (s16 & 1) << 3;  // 0 or 8 within the 16-byte chunk
+  int bChunk[NI];                     // logical 16-byte chunk index of this lane's columns
+#pragma unroll
+  for (int j = 0; j < NI; ++j) bChunk[j] = (wn * WN + 32 * j + 16 * colHalf) >> 4;
+
+  const unsigned KT = (K + BK - 1) / BK;
+#pragma unroll
+  for (int s = 0; s < STAGES - 1; ++s) issueSlab(s);
+
+  for (unsigned kt = 0; kt < KT; ++kt) {
+    // slab kt has landed once at most the copies of the STAGES-2 younger slabs are outstanding
+    wait_vmcnt<COPIES*(STAGES - 2)>();
+    __syncthreads();
+    // every wavefront is past slab kt-1, whose stage is the one refilled now (copies past the end of
+    // K read zeros or unused bytes; issuing them keeps the outstanding-copy count uniform)
+    issueSlab(kt + STAGES - 1);
+
+    const unsigned char* as = smem + (kt % STAGES) * STAGE_BYTES;
+    const unsigned char* bs = as + A_BYTES;
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      v4i af[MI], bf[NI];
+#pragma unroll
+      for (int i = 0; i < MI; ++i) {
+        v4i v = *reinterpret_cast<const v4i*>(as + aAddr[i][ks]);
+        af[i] = v ^ (int)0x80808080;
+      }
+#pragma unroll
+      for (int j = 0; j < NI; ++j) {
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          const int k = 32 * ks + 16 * g + 8 * half + trK;  // (k & 7) == trK
+          const unsigned char* ptr = bs + k * BN + ((bChunk[j] ^ trK) << 4) + trByte;
+          v2i t = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+              (__attribute__((address_space(3))) v2i*)(const_cast<unsigned char*>(ptr)));
+          bf[j][2 * half] = t[0];
+          bf[j][2 * half + 1] = t[1];
+        }
+      }
+      if (wm == 0) {
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+#pragma unroll
+          for (int q = 0; q < 4; ++q) colsum[j] = __builtin_amdgcn_sdot4(bf[j][q], 0x01010101, colsum[j], false);
+      }
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[i], acc[i][j], 0, 0, 0);
+    }
+  }
+  wait_vmcnt<0>();
+  __syncthreads();
+
+  // ---- epilogue.  Accumulator layout (operands swapped): lane (l32, g) holds row l32 of the 32-row
+  // block and columns 8*(r/4) + 4*g + r%4 of the 32-column block, r = 0..15.
+  int* colTerm = reinterpret_cast<int*>(smem);  // [BN]
+  int* rowTerm = colTerm + BN;                  // [BM]
+  unsigned char* stageQ = smem + (BM + BN) * 4; // [BM][BN + 4] bytes, requantized tile
+  constexpr int QPITCH = BN + 4;
+  if (wm == 0) {
+    // lanes l and l+32 hold the two k halves of the same column
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      int s = colsum[j] + __shfl_xor(colsum[j], 32, 64);
+      // tr-read column order: lane (colHalf, s16) -> column 16*colHalf + 8*(s16>>3) + (s16&7) = 16*colHalf + s16
+      if (g == 0) colTerm[wn * WN + 32 * j + 16 * colHalf + s16] = s;
+    }
+  }
+  __syncthreads();
+  const int* rsA = p.rowsumA + (size_t)bi * p.strideRA;
+  const int* csB = p.colsumB + (size_t)bi * p.strideRB;
+  const unsigned global = (unsigned)offA * (unsigned)offB * K;
+  for (int i = tid; i < BN; i += kThreads) {
+    unsigned gn = n0 + i;
+    unsigned cs = gn < N ? (unsigned)csB[gn] : 0u;
+    colTerm[i] = (int)(128u * (unsigned)colTerm[i] + cs * (unsigned)offA);
+  }
+  for (int i = tid; i < BM; i += kThreads) {
+    unsigned gm = m0 + i;
+    unsigned rs = gm < M ? (unsigned)rsA[gm] : 0u;
+    rowTerm[i] = (int)(global + rs * (unsigned)offB);
+  }
+  __syncthreads();
+
+  RequantScalars rq;
+  if (REQUANT) {
+    if (p.minOut) {
+      rq = make_requant_scalars(TFCC_ROCM_S32, TFCC_ROCM_U8, minC, maxC, *p.minOut, *p.maxOut);
+    } else {
+      rq.inScale = p.inScale; rq.inMin = p.inMin; rq.outScale = p.outScale; rq.outOffset = p.outOffset;
+      rq.inLowest = -2147483648LL; rq.outLowest = 0; rq.outHighest = 255; rq.mode = 0; rq.fillValue = 0;
+      finish_requant_scalars(rq, 4294967295.0);
+    }
+  }
+
+  int* C = p.C ? p.C + (size_t)bi * p.strideC : nullptr;
+  unsigned char* Q = REQUANT ? p.Q + (size_t)bi * p.strideC : nullptr;
+
+  auto storeTile = [&](auto flavour) {
+    constexpr int FLAVOUR = decltype(flavour)::value;  // 0 int32 only, 1 fast requantize, 2 exact, 3 fill
+#pragma unroll
+    for (int i = 0; i < MI; ++i) {
+      const int trow = wm * WM + 32 * i + l32;
+      const unsigned grow = m0 + trow;
+      const int rt = rowTerm[trow];
+#pragma unroll
+      for (int j = 0; j < NI; ++j) {
+#pragma unroll
+        for (int rq4 = 0; rq4 < 4; ++rq4) {
+          const int tcol = wn * WN + 32 * j + 8 * rq4 + 4 * g;  // first of 4 consecutive columns
+          const v4i ct = *reinterpret_cast<const v4i*>(colTerm + tcol);
+          int v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = (int)((unsigned)acc[i][j][4 * rq4 + e] + (unsigned)rt + (unsigned)ct[e]);
+          if (C && grow < M && n0 + tcol < N)  // N % 16 == 0: the four columns are in or out together
+            *reinterpret_cast<v4i*>(C + (size_t)grow * N + n0 + tcol) = v4i{v[0], v[1], v[2], v[3]};
+          if constexpr (FLAVOUR != 0) {
+            unsigned q[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              if constexpr (FLAVOUR == 1) q[e] = (unsigned)requantize_one_fast((double)((unsigned)v[e] ^ 0x80000000u), rq);
+              else if constexpr (FLAVOUR == 2) q[e] = (unsigned)requantize_one_exact((long long)v[e], rq);
+              else q[e] = (unsigned)rq.fillValue;
+            }
+            *reinterpret_cast<unsigned*>(stageQ + trow * QPITCH + tcol) = q[0] | (q[1] << 8) | (q[2] << 16) | (q[3] << 24);
+          }
+        }
+      }
+    }
+  };
+  if constexpr (!REQUANT) {
+    storeTile(std::integral_constant<int, 0>{});
+  } else {
+    if (rq.mode) storeTile(std::integral_constant<int, 3>{});
+    else if (rq.fastOK) storeTile(std::integral_constant<int, 1>{});
+    else storeTile(std::integral_constant<int, 2>{});
+    __syncthreads();
+    // staged tile -> HBM: 16 lanes write one 256-byte row segment
+    constexpr int CHUNKS = BN / 16;
+    for (int idx = tid; idx < BM * CHUNKS; idx += kThreads) {
+      const int row = idx / CHUNKS, ch = idx % CHUNKS;
+      const unsigned grow = m0 + row, gcol = n0 + ch * 16;
+      if (grow >= M || gcol >= N) continue;
+      const unsigned* src = reinterpret_cast<const unsigned*>(stageQ + row * QPITCH + ch * 16);
+      v4i v = {(int)src[0], (int)src[1], (int)src[2], (int)src[3]};
+      *reinterpret_cast<v4i*>(Q + (size_t)grow * N + gcol) = v;
+    }
+  }
+}
+
+template <int BM, int BN, int STAGES, bool REQUANT>
+int launch(hipStream_t stream, QGemmParams p) {
+  p.tilesM = (p.M + BM - 1) / BM;
+  p.tilesN = (p.N + BN - 1) / BN;
+  unsigned long long total = (unsigned long long)p.tilesM * p.tilesN * p.batch;
+  if (total > 0x7fffffffull) return set_error(TFCC_ROCM_INVALID_ARGUMENT, "quantized matmul: too many tiles");
+  p.tilesTotal = (unsigned)total;
+  p.chunk = (p.tilesTotal + 7) / 8;
+  constexpr size_t ring = (size_t)STAGES * (BM + BN) * BK;
+  constexpr size_t epi = (size_t)(BM + BN) * 4 + (size_t)BM * (BN + 4);
+  constexpr size_t lds = ring > epi ? ring : epi;
+  static_assert(lds <= 160 * 1024, "LDS budget");
+  auto kern = qgemm_dma_kernel<BM, BN, STAGES, REQUANT>;
+  static bool attrSet = false;
+  if (!attrSet) {
+    TFCC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+    attrSet = true;
+  }
+  hipLaunchKernelGGL(kern, dim3(p.chunk * 8), dim3(kThreads), lds, stream, p);
+  return check_launch("quantized matmul (dma)");
+}
+
+}  // namespace
+
+bool qgemm_dma_supported(const QGemmParams& p, bool requant) {
+  return (p.K % 16 == 0) && (p.N % 16 == 0) && ((uintptr_t)p.A % 16 == 0) && ((uintptr_t)p.B % 16 == 0) &&
+         (p.strideA % 16 == 0) && (p.strideB % 16 == 0) &&
+         (p.C == nullptr || ((uintptr_t)p.C % 16 == 0 && p.strideC % 4 == 0)) &&
+         (!requant || ((uintptr_t)p.Q % 16 == 0 && p.strideC % 16 == 0)) &&
+         ((unsigned long long)p.M + 512) * p.K < (1ull << 32) && ((unsigned long long)p.K + 1024) * p.N + 1024 < (1ull << 32);
+}
+
+int qgemm_dma_launch(hipStream_t stream, const QGemmParams& p, bool requant) {
+  const unsigned long long big = (unsigned long long)((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batch;
+  if (big >= 192) {
+    return requant ? launch<256, 256, 4, true>(stream, p) : launch<256, 256, 4, false>(stream, p);
+  }
+  return requant ? launch<128, 128, 4, true>(stream, p) : launch<128, 128, 4, false>(stream, p);
+}
+
+}  // namespace tfcc_rocm

@@ -11,6 +11,6 @@ bool gemv_supported(const void* a, const void* b, unsigned m, unsigned n, unsign
 int gemv_launch(hipStream_t stream, const unsigned char* a, const signed char* b, const int* rowsumA,
                 const int* colsumB, int offsetA, int offsetB, const float* const ranges[4],
                 float* const rangeOut[2], unsigned m, unsigned n, unsigned k, int* accOut,
-                float scaleA, const float* scaleB, float* f32Out, unsigned kslabsHint);
+                float scaleA, const float* scaleB, float* f32Out);
 
 }  // namespace tfcc_rocm

@@ -4,17 +4,16 @@
 // Same arithmetic as the general quantized matmul (tfcc/mkl/operations/tfcc_mklquantization.cpp:
 // 33-69,176-201); the reference has no dedicated kernel for this shape.
 //
-// Work split: a wavefront owns 128 consecutive columns and walks a K range in steps of 64 rows.
-// Per step every lane loads a 16(k) x 4(n) byte block of B for two column blocks (32 dword loads;
-// a wavefront reads four 128-byte row segments per instruction), transposes the blocks in registers
-// with v_perm_b32 so that it holds 16 consecutive k for each of its columns, and feeds them to
-// v_mfma_i32_16x16x64_i8 as the B operand.  The A operand holds the (up to 8) rows of A, xor 0x80
-// (a' = a - 128), zero rows, and one row of ones in row 15 whose product is the true column sum of
-// B, needed to undo the -128 shift: sum a*b = sum a'*b + 128*colsum(B).
-// The four wavefronts of a workgroup split the workgroup's K slab and reduce through LDS; the K
-// slabs of different workgroups are combined through a workspace: every workgroup writes its
-// partial sums, the last one to arrive for a column group (atomic ticket) adds them up in slab
-// order, applies the offset terms and the optional per-channel dequantize, and resets the ticket.
+// Work split: a workgroup of 16 wavefronts owns 64 consecutive columns over the whole of K, so no
+// partial sums ever leave the CU.  The wavefronts deal the 64-row steps of K among themselves.
+// Per step every lane loads a 16(k) x 4(n) byte block of B as 16 dwords (a wavefront reads four
+// 64-byte row segments per instruction; the neighbouring column group, which shares the 128-byte
+// lines, is placed on the same XCD), transposes it in registers with v_perm_b32 so that it holds
+// 16 consecutive k for each of its four columns, and feeds them to v_mfma_i32_16x16x64_i8 as the
+// B operand.  The A operand holds the (up to 8) rows of A, xor 0x80 (a' = a - 128), zero rows, and
+// one row of ones in row 15 whose product is the true column sum of B, needed to undo the -128
+// shift: sum a*b = sum a'*b + 128*colsum(B).  The 16 partial tiles are added through LDS, the
+// offset terms and the optional per-channel dequantize are applied in the store.
 #include <stdlib.h>
 
 #include "common.hpp"
@@ -26,11 +25,12 @@ typedef int v4i __attribute__((ext_vector_type(4)));
 
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kCols = 128;    // columns per workgroup
+constexpr int kWaves = 16;
+constexpr int kThreads = kWaves * 64;
+constexpr int kCols = 64;     // columns per workgroup
 constexpr int kMaxM = 8;
 constexpr int kRows = 16;     // MFMA rows: kMaxM data rows, zeros, ones in row 15
-constexpr int kPartRows = 9;  // rows kept per partial: 8 data rows + the column-sum row
+constexpr int kPartRows = 9;  // rows kept per wavefront: 8 data rows + the column-sum row
 
 struct GemvParams {
   const unsigned char* A;
@@ -45,9 +45,7 @@ struct GemvParams {
   const float *minA, *maxA, *minB, *maxB;  // optional ranges in device memory (override the offsets)
   float *minC, *maxC;
   unsigned M, N, K;
-  unsigned kslabs, stepsPerSlab;  // K split over workgroups, 64-row steps per slab
-  int* partial;                   // [colGroups][kslabs][kPartRows][kCols]
-  unsigned* tickets;              // [colGroups], zero between launches
+  unsigned colGroups, groupsPerXcd;
 };
 
 __device__ __forceinline__ void transpose4x4(const unsigned r[4], unsigned c[4]) {
@@ -62,11 +60,12 @@ __device__ __forceinline__ void transpose4x4(const unsigned r[4], unsigned c[4])
 }
 
 __global__ __launch_bounds__(kThreads) void gemv_kernel(const GemvParams p) {
-  __shared__ int red[4][kPartRows][kCols];
-  __shared__ unsigned lastFlag;
+  __shared__ int red[kWaves][kPartRows][kCols];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const unsigned cg = blockIdx.x / p.kslabs, slab = blockIdx.x % p.kslabs;
+  // consecutive workgroup ids go to different XCDs: give each XCD a run of adjacent column groups
+  const unsigned cg = (blockIdx.x & 7u) * p.groupsPerXcd + (blockIdx.x >> 3);
+  if ((blockIdx.x >> 3) >= p.groupsPerXcd || cg >= p.colGroups) return;
   const unsigned n0 = cg * kCols;
   const unsigned M = p.M, N = p.N, K = p.K;
   const int j = lane & 15, kg = lane >> 4;
@@ -76,85 +75,61 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(const GemvParams p) {
   const __amdgpu_buffer_rsrc_t rsrcA =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(p.A), 0, (int)(M * K), 0x00020000);
 
-  v4i acc[2][4];
+  v4i acc[4];
 #pragma unroll
-  for (int b = 0; b < 2; ++b)
-#pragma unroll
-    for (int e = 0; e < 4; ++e) acc[b][e] = v4i{0, 0, 0, 0};
+  for (int e = 0; e < 4; ++e) acc[e] = v4i{0, 0, 0, 0};
 
-  // steps of this workgroup's slab are dealt round-robin to its four wavefronts
-  const unsigned stepBegin = slab * p.stepsPerSlab;
-  const unsigned stepEnd = min(stepBegin + p.stepsPerSlab, (K + 63) / 64);
-  for (unsigned step = stepBegin + wave; step < stepEnd; step += 4) {
-    const unsigned k0 = step * 64 + kg * 16;  // this lane's 16 rows
+  const unsigned steps = (K + 63) / 64;
+  for (unsigned step = wave; step < steps; step += 2 * kWaves) {
+    // two steps in flight per wavefront (the second may lie past K: it then reads zeros)
     unsigned braw[2][16];
+    v4i a[2];
 #pragma unroll
-    for (int b = 0; b < 2; ++b)
+    for (int u = 0; u < 2; ++u) {
+      const unsigned k0 = (step + u * kWaves) * 64 + kg * 16;  // this lane's 16 rows
 #pragma unroll
       for (int q = 0; q < 16; ++q)
-        braw[b][q] = __builtin_amdgcn_raw_buffer_load_b32(rsrcB, (k0 + q) * N + n0 + (b * 16 + j) * 4, 0, 0);
-    // A operand: row j of A, 16 consecutive k
-    v4i a = {0, 0, 0, 0};
-    if ((unsigned)j < M) {
-      a = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrcA, (unsigned)j * K + k0, 0, 0));
-      a = a ^ (int)0x80808080;
-    } else if (j == kRows - 1) {
-      a = v4i{0x01010101, 0x01010101, 0x01010101, 0x01010101};
+        braw[u][q] = __builtin_amdgcn_raw_buffer_load_b32(rsrcB, (k0 + q) * N + n0 + j * 4, 0, 0);
+      a[u] = v4i{0, 0, 0, 0};
+      if ((unsigned)j < M) {
+        a[u] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrcA, (unsigned)j * K + k0, 0, 0));
+        a[u] = a[u] ^ (int)0x80808080;
+      } else if (j == kRows - 1) {
+        a[u] = v4i{0x01010101, 0x01010101, 0x01010101, 0x01010101};
+      }
     }
 #pragma unroll
-    for (int b = 0; b < 2; ++b) {
+    for (int u = 0; u < 2; ++u) {
       unsigned col[4][4];
 #pragma unroll
       for (int kq = 0; kq < 4; ++kq) {
         unsigned c4[4];
-        transpose4x4(&braw[b][4 * kq], c4);
+        transpose4x4(&braw[u][4 * kq], c4);
 #pragma unroll
         for (int e = 0; e < 4; ++e) col[e][kq] = c4[e];
       }
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         v4i bv = {(int)col[e][0], (int)col[e][1], (int)col[e][2], (int)col[e][3]};
-        acc[b][e] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a, bv, acc[b][e], 0, 0, 0);
+        acc[e] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[u], bv, acc[e], 0, 0, 0);
       }
     }
   }
 
   // D layout of the 16x16 block: lane (j, kg) holds rows 4*kg + r, column j.
-  // Keep rows 0..7 and row 15 (stored as partial row 8).
+  // Keep rows 0..7 and row 15 (stored as row 8).
 #pragma unroll
-  for (int b = 0; b < 2; ++b)
+  for (int e = 0; e < 4; ++e) {
+    const int col = j * 4 + e;
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const int col = (b * 16 + j) * 4 + e;
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const int row = 4 * kg + r;
-        if (row < kMaxM) red[wave][row][col] = acc[b][e][r];
-        else if (row == kRows - 1) red[wave][kMaxM][col] = acc[b][e][r];
-      }
+    for (int r = 0; r < 4; ++r) {
+      const int row = 4 * kg + r;
+      if (row < kMaxM) red[wave][row][col] = acc[e][r];
+      else if (row == kRows - 1) red[wave][kMaxM][col] = acc[e][r];
     }
-  __syncthreads();
-
-  const unsigned rowsKept = M + 1;  // data rows + column-sum row
-  int* part = p.partial + ((size_t)cg * p.kslabs + slab) * kPartRows * kCols;
-  for (unsigned idx = tid; idx < rowsKept * kCols; idx += kThreads) {
-    unsigned r = idx / kCols, c = idx % kCols;
-    unsigned srcRow = r < M ? r : kMaxM;
-    int v = red[0][srcRow][c] + red[1][srcRow][c] + red[2][srcRow][c] + red[3][srcRow][c];
-    part[r * kCols + c] = v;
-  }
-  // publish the partial, then take a ticket: the last workgroup of this column group finishes it
-  __threadfence();
-  __syncthreads();
-  if (tid == 0) {
-    unsigned t = __hip_atomic_fetch_add(&p.tickets[cg], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-    lastFlag = (t == p.kslabs - 1) ? 1u : 0u;
   }
   __syncthreads();
-  if (!lastFlag) return;
-  __threadfence();
 
-  const int* base = p.partial + (size_t)cg * p.kslabs * kPartRows * kCols;
   int oA = p.offsetA, oB = p.offsetB;
   if (p.minA) {
     float mnA = *p.minA, mxA = *p.maxA, mnB = *p.minB, mxB = *p.maxB;
@@ -169,60 +144,19 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(const GemvParams p) {
   const unsigned offA = (unsigned)oA, offB = (unsigned)oB;
   const unsigned global = offA * offB * K;
   for (unsigned idx = tid; idx < M * kCols; idx += kThreads) {
-    unsigned r = idx / kCols, c = idx % kCols;
-    unsigned gn = n0 + c;
+    const unsigned r = idx / kCols, c = idx % kCols;
+    const unsigned gn = n0 + c;
     if (gn >= N) continue;
     unsigned sum = 0, cs = 0;
-    for (unsigned s = 0; s < p.kslabs; ++s) {
-      const int* ps = base + (size_t)s * kPartRows * kCols;
-      sum += (unsigned)__builtin_nontemporal_load(ps + r * kCols + c);
-      cs += (unsigned)__builtin_nontemporal_load(ps + M * kCols + c);
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      sum += (unsigned)red[w][r][c];
+      cs += (unsigned)red[w][kMaxM][c];
     }
-    unsigned v = sum + 128u * cs + global + (unsigned)p.rowsumA[r] * offB + (unsigned)p.colsumB[gn] * offA;
+    const unsigned v = sum + 128u * cs + global + (unsigned)p.rowsumA[r] * offB + (unsigned)p.colsumB[gn] * offA;
     if (p.accOut) p.accOut[(size_t)r * N + gn] = (int)v;
     if (p.f32Out) p.f32Out[(size_t)r * N + gn] = (float)((double)(int)v * ((double)p.scaleA * (double)p.scaleB[gn]));
   }
-  if (tid == 0) __hip_atomic_store(&p.tickets[cg], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// per-device workspace, allocated on first use and kept
-struct Workspace {
-  int* partial = nullptr;
-  unsigned* tickets = nullptr;
-  size_t partialBytes = 0, ticketCount = 0;
-};
-constexpr int kMaxDevices = 16;
-Workspace g_ws[kMaxDevices];
-
-int get_workspace(hipStream_t stream, size_t partialBytes, size_t ticketCount, Workspace** out) {
-  int dev = 0;
-  TFCC_HIP_CHECK(hipGetDevice(&dev));
-  if (dev < 0 || dev >= kMaxDevices) return set_error(TFCC_ROCM_INVALID_ARGUMENT, "gemv: device index %d", dev);
-  Workspace& w = g_ws[dev];
-  if (w.partialBytes < partialBytes) {
-    if (w.partial) {
-      TFCC_HIP_CHECK(hipDeviceSynchronize());
-      TFCC_HIP_CHECK(hipFree(w.partial));
-      w.partial = nullptr;
-      w.partialBytes = 0;
-    }
-    TFCC_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&w.partial), partialBytes));
-    w.partialBytes = partialBytes;
-  }
-  if (w.ticketCount < ticketCount) {
-    if (w.tickets) {
-      TFCC_HIP_CHECK(hipDeviceSynchronize());
-      TFCC_HIP_CHECK(hipFree(w.tickets));
-      w.tickets = nullptr;
-      w.ticketCount = 0;
-    }
-    TFCC_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&w.tickets), ticketCount * sizeof(unsigned)));
-    TFCC_HIP_CHECK(hipMemset(w.tickets, 0, ticketCount * sizeof(unsigned)));
-    w.ticketCount = ticketCount;
-  }
-  (void)stream;
-  *out = &w;
-  return TFCC_ROCM_OK;
 }
 
 }  // namespace
@@ -230,13 +164,13 @@ int get_workspace(hipStream_t stream, size_t partialBytes, size_t ticketCount, W
 // Whether the skinny kernel can take this shape (else the caller uses the general kernel).
 bool gemv_supported(const void* a, const void* b, unsigned m, unsigned n, unsigned k) {
   return m >= 1 && m <= (unsigned)kMaxM && n % 4 == 0 && k % 16 == 0 && (uintptr_t)a % 16 == 0 &&
-         (uintptr_t)b % 4 == 0 && ((unsigned long long)k + 64) * n + 512 < (1ull << 31);
+         (uintptr_t)b % 4 == 0 && ((unsigned long long)k + 2048) * n + 512 < (1ull << 31);
 }
 
 int gemv_launch(hipStream_t stream, const unsigned char* a, const signed char* b, const int* rowsumA,
                 const int* colsumB, int offsetA, int offsetB, const float* const ranges[4],
                 float* const rangeOut[2], unsigned m, unsigned n, unsigned k, int* accOut,
-                float scaleA, const float* scaleB, float* f32Out, unsigned kslabsHint) {
+                float scaleA, const float* scaleB, float* f32Out) {
   GemvParams p{};
   if (ranges && ranges[0]) {
     p.minA = ranges[0]; p.maxA = ranges[1]; p.minB = ranges[2]; p.maxB = ranges[3];
@@ -246,24 +180,11 @@ int gemv_launch(hipStream_t stream, const unsigned char* a, const signed char* b
   p.accOut = accOut; p.f32Out = f32Out; p.scaleA = scaleA; p.scaleB = scaleB;
   p.offsetA = offsetA; p.offsetB = offsetB;
   p.M = m; p.N = n; p.K = k;
-  const unsigned colGroups = (n + kCols - 1) / kCols;
-  const unsigned steps = (k + 63) / 64;
-  // enough workgroups for about four per CU, at least four steps (one per wavefront) each
-  unsigned kslabs = kslabsHint ? kslabsHint : (1024 + colGroups - 1) / colGroups;
-  unsigned maxSlabs = (steps + 3) / 4;
-  if (kslabs > maxSlabs) kslabs = maxSlabs;
-  if (kslabs < 1) kslabs = 1;
-  p.stepsPerSlab = (steps + kslabs - 1) / kslabs;
-  p.kslabs = (steps + p.stepsPerSlab - 1) / p.stepsPerSlab;
-  Workspace* w = nullptr;
-  size_t partialBytes = (size_t)colGroups * p.kslabs * kPartRows * kCols * sizeof(int);
-  if (int e = get_workspace(stream, partialBytes, colGroups, &w)) return e;
-  p.partial = w->partial;
-  p.tickets = w->tickets;
-  hipLaunchKernelGGL(gemv_kernel, dim3(colGroups * p.kslabs), dim3(kThreads), 0, stream, p);
+  p.colGroups = (n + kCols - 1) / kCols;
+  p.groupsPerXcd = (p.colGroups + 7) / 8;
+  hipLaunchKernelGGL(gemv_kernel, dim3(p.groupsPerXcd * 8), dim3(kThreads), 0, stream, p);
   return check_launch("skinny quantized matmul");
 }
-
 
 namespace {
 
@@ -279,17 +200,6 @@ __global__ void dequant_per_channel_kernel(const int* acc, unsigned m, unsigned 
 
 using namespace tfcc_rocm;
 
-// environment override of the K split, for tuning runs only
-static unsigned kslabs_hint() {
-  static int cached = -1;
-  if (cached < 0) {
-    const char* e = getenv("TFCC_ROCM_GEMV_KSLABS");
-    cached = e ? atoi(e) : 0;
-    if (cached < 0) cached = 0;
-  }
-  return (unsigned)cached;
-}
-
 extern "C" int tfcc_rocm_gemv_u8s8s32(void* stream, const uint8_t* a, const int8_t* b,
                                       const int32_t* rowsum_a, const int32_t* colsum_b,
                                       int32_t offset_a, int32_t offset_b, unsigned m, unsigned n,
@@ -302,8 +212,7 @@ extern "C" int tfcc_rocm_gemv_u8s8s32(void* stream, const uint8_t* a, const int8
   hipStream_t s = as_stream(stream);
   if (gemv_supported(a, b, m, n, k))
     return gemv_launch(s, a, reinterpret_cast<const signed char*>(b), rowsum_a, colsum_b, offset_a,
-                       offset_b, nullptr, nullptr, m, n, k, acc_out, scale_a, scale_b, f32_out,
-                       kslabs_hint());
+                       offset_b, nullptr, nullptr, m, n, k, acc_out, scale_a, scale_b, f32_out);
   // shapes the skinny kernel does not take (m > 8, unaligned): general kernel, then dequantize
   TFCC_REQUIRE(acc_out != nullptr, "skinny quantized matmul: this shape needs acc_out (m > 8 or unaligned operands)");
   tfcc_rocm_qgemm_desc d{};

@@ -122,7 +122,11 @@ __global__ __launch_bounds__(256) void requantize_kernel(const void* in, int inT
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   const size_t step = (size_t)gridDim.x * blockDim.x;
   for (; i < total; i += step) {
-    long long q = s.mode ? s.fillValue : requantize_one(load_typed(in, inType, i), s);
+    long long q = s.fillValue;
+    if (!s.mode) {
+      const long long x = load_typed(in, inType, i);
+      q = s.fastOK ? (long long)requantize_one_fast((double)(x - s.inLowest), s) : requantize_one_exact(x, s);
+    }
     store_typed(out, outType, i, q);
   }
 }
@@ -139,11 +143,16 @@ __global__ __launch_bounds__(256) void requantize_s32_u8_vec_kernel(const int4* 
     unsigned q0, q1, q2, q3;
     if (s.mode) {
       q0 = q1 = q2 = q3 = (unsigned)s.fillValue;
+    } else if (s.fastOK) {
+      q0 = (unsigned)requantize_one_fast((double)((unsigned)v.x ^ 0x80000000u), s);
+      q1 = (unsigned)requantize_one_fast((double)((unsigned)v.y ^ 0x80000000u), s);
+      q2 = (unsigned)requantize_one_fast((double)((unsigned)v.z ^ 0x80000000u), s);
+      q3 = (unsigned)requantize_one_fast((double)((unsigned)v.w ^ 0x80000000u), s);
     } else {
-      q0 = (unsigned)requantize_one(v.x, s);
-      q1 = (unsigned)requantize_one(v.y, s);
-      q2 = (unsigned)requantize_one(v.z, s);
-      q3 = (unsigned)requantize_one(v.w, s);
+      q0 = (unsigned)requantize_one_exact(v.x, s);
+      q1 = (unsigned)requantize_one_exact(v.y, s);
+      q2 = (unsigned)requantize_one_exact(v.z, s);
+      q3 = (unsigned)requantize_one_exact(v.w, s);
     }
     out[i] = q0 | (q1 << 8) | (q2 << 16) | (q3 << 24);
   }
