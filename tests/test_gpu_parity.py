@@ -228,7 +228,9 @@ def test_requantize_against_oracle(pkg, T):
         for (mi, ma, mo, mxo) in ((-1000.0, 1000.0, -300.0, 310.0), (-2147483648.0, 2147483648.0, -33554432.0, 33292288.0),
                                   (-1.0, 1.0, 2.0, 2.0), (1.5, 1.5, -4.0, 4.0), (-3.0, 5.0, 0.5, -0.5),
                                   # output scale so large that the int64 conversion overflows: exact integer path
-                                  (-1000.0, 1000.0, 0.0, 1e-30), (-1e30, 1e30, -1e-3, 1e-3)):
+                                  (-1000.0, 1000.0, 0.0, 1e-30), (-1e30, 1e30, -1e-3, 1e-3),
+                                  # output offset near 2^31: the double shortcut, not the int32 one
+                                  (8388607.5, 8388610.0, 8388608.0, 8388609.0)):
             got = pkg.requantize(T.t(acc), T.f1(mi), T.f1(ma), T.f1(mo), T.f1(mxo), torch.uint8)
             assert np.array_equal(T.n(got), O.requantize_s32_u8(acc, mi, ma, mo, mxo)), (total, mi, ma, mo, mxo)
     # ties: nearest-even like the reference's AVX2 kernel

@@ -112,7 +112,9 @@ struct RequantScalars {
   int mode;            // 0: per-element arithmetic, 1: fill with fillValue (degenerate ranges)
   long long fillValue;
   double offsetMinusLowest;  // (double)(outOffset - outLowest), exact when fastOK
-  int fastOK;
+  int fastOK;                // the double shortcut is exact for every input
+  int fast32OK;              // ... and rint(y), rint(y) - (outOffset - outLowest) stay inside int32
+  int offsetMinusLowest32;
 };
 
 // offMax = highest - lowest of the input type (its largest x - inLowest)
@@ -123,6 +125,20 @@ __host__ __device__ static inline void finish_requant_scalars(RequantScalars& s,
   const double r0 = fabs(s.inMin), r1 = fabs(fma(offMax, s.inScale, s.inMin));
   const double bound = (r0 > r1 ? r0 : r1) * fabs(s.outScale);
   s.fastOK = (d > -(1LL << 52) && d < (1LL << 52) && bound < 1125899906842624.0) ? 1 : 0;  // NaN compares false
+  const double dAbs = d < 0 ? -(double)d : (double)d;
+  s.fast32OK = (s.fastOK && bound + dAbs < 2147483000.0) ? 1 : 0;
+  s.offsetMinusLowest32 = s.fast32OK ? (int)d : 0;
+}
+
+// Valid when RequantScalars::fast32OK.  Adding 1.5 * 2^52 rounds y to the nearest integer (ties to
+// even, the default rounding mode) in the low mantissa bits: the low dword of the sum is rint(y) as a
+// two's-complement int32.  The subtraction cannot overflow because |rint(y)| + |offset| < 2^31.
+__device__ static inline int requantize_one_fast32(double off, const RequantScalars& s) {
+  const double y = fma(off, s.inScale, s.inMin) * s.outScale;
+  const int r = (int)(unsigned)__double_as_longlong(y + 6755399441055744.0);
+  const int q = r - s.offsetMinusLowest32;
+  const int lo = (int)s.outLowest, hi = (int)s.outHighest;
+  return q < lo ? lo : (q > hi ? hi : q);
 }
 
 __device__ static inline long long requantize_one_exact(long long x, const RequantScalars& s) {
@@ -159,6 +175,8 @@ __host__ __device__ static inline RequantScalars make_requant_scalars(int inType
   s.inScale = s.inMin = s.outScale = 0.0;
   s.outOffset = 0;
   s.fastOK = 0;
+  s.fast32OK = 0;
+  s.offsetMinusLowest32 = 0;
   s.offsetMinusLowest = 0.0;
   if (minOut >= maxOut) {
     s.mode = 1;

@@ -305,7 +305,7 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(const QGemmParams p) {
   for (int j = 0; j < NI; ++j) ct[j] = colTerm[colBase + j];
   const bool vecOK = ALIGNED && (gcol + NI <= N);     // N % 4 == 0 and base pointers aligned when ALIGNED
 
-  // FLAVOUR 0: int32 only; 1: requantize, fast double path; 2: requantize, exact int64 path; 3: constant fill
+  // FLAVOUR 0: int32 only; 1: requantize, double shortcut; 2: exact int64 path; 3: constant fill; 4: int32 shortcut
   auto storeTile = [&](auto flavour) {
     constexpr int FLAVOUR = decltype(flavour)::value;
 #pragma unroll
@@ -338,6 +338,8 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(const QGemmParams p) {
               q[j] = (unsigned)requantize_one_fast((double)((unsigned)v[j] ^ 0x80000000u), rq);
             } else if constexpr (FLAVOUR == 2) {
               q[j] = (unsigned)requantize_one_exact((long long)v[j], rq);
+            } else if constexpr (FLAVOUR == 4) {
+              q[j] = (unsigned)requantize_one_fast32((double)((unsigned)v[j] ^ 0x80000000u), rq);
             } else {
               q[j] = (unsigned)rq.fillValue;
             }
@@ -358,6 +360,7 @@ __global__ __launch_bounds__(kThreads) void qgemm_kernel(const QGemmParams p) {
   } else {
     // uniform over the whole launch: every wavefront takes the same branch
     if (rq.mode) storeTile(std::integral_constant<int, 3>{});
+    else if (rq.fast32OK) storeTile(std::integral_constant<int, 4>{});
     else if (rq.fastOK) storeTile(std::integral_constant<int, 1>{});
     else storeTile(std::integral_constant<int, 2>{});
   }

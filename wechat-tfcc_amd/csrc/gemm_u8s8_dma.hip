@@ -4,7 +4,8 @@
 // shapes); replaces tfcc/mkl/operations/tfcc_mklquantization.cpp:33-69,176-201 and the blocked CPU
 // GEMM below it (tfcc/mkl/gemm/tfcc_mklsinglethreadgemm.h:93-141, tfcc_mklmatmulkernel.h:142-260).
 //
-// Data path of one BM x BN tile (four wavefronts, 2 x 2):
+// Data path of one BM x BN tile (WGM x WGN wavefronts; eight for the 256 x 256 tile, so that every
+// SIMD holds two: one wavefront's LDS reads, waits and VALU work overlap the other's matrix ops):
 //   HBM -> LDS  buffer_load_dwordx4 ... lds (asynchronous, no VGPRs): every K slab of 64 bytes is
 //               copied as it lies in memory, A rows as As[row][64] and B rows as Bs[k][BN], into a
 //               ring of STAGES LDS buffers, STAGES-1 slabs ahead of the matrix cores.  Out-of-range
@@ -34,7 +35,6 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 
 namespace {
 
-constexpr int kThreads = 256;
 constexpr int BK = 64;
 
 // One asynchronous 16-byte-per-lane copy HBM -> LDS.  The LDS address of lane i is ldsBase + 16*i
@@ -67,23 +67,27 @@ __device__ __forceinline__ void wait_vmcnt() {
 
 __device__ __forceinline__ int swzA(int row) { return ((row >> 1) & 3) ^ ((row >> 3) & 1); }
 
-template <int BM, int BN, int STAGES, bool REQUANT>
-__global__ __launch_bounds__(kThreads) void qgemm_dma_kernel(const QGemmParams p) {
-  constexpr int WM = BM / 2, WN = BN / 2;
+template <int BM, int BN, int WGM, int WGN, int STAGES, bool REQUANT>
+__global__ __launch_bounds__(WGM * WGN * 64) void qgemm_dma_kernel(const QGemmParams p) {
+  constexpr int kThreads = WGM * WGN * 64;
+  constexpr int WM = BM / WGM, WN = BN / WGN;
   constexpr int MI = WM / 32, NI = WN / 32;
+  static_assert(MI + 2 * NI <= 2 * MI * NI, "operand reads are issued two per matrix op");
+  static_assert(NI % WGM == 0, "every 32-column block needs a wavefront row in charge of its column sums");
+  static_assert(MI >= 1 && NI >= 1 && (BM * BK / 16) % kThreads == 0 && (BK * BN / 16) % kThreads == 0, "tile shape");
   constexpr int A_BYTES = BM * BK, B_BYTES = BK * BN, STAGE_BYTES = A_BYTES + B_BYTES;
   constexpr int A_COPIES = A_BYTES / 16 / kThreads, B_COPIES = B_BYTES / 16 / kThreads;
   constexpr int COPIES = A_COPIES + B_COPIES;  // per thread per slab
   constexpr int BCH = BN / 16;                 // 16-byte chunks per B row
   static_assert(BCH >= 8 && (BCH & (BCH - 1)) == 0, "B swizzle needs at least 8 chunks per row");
-  static_assert(COPIES * (STAGES - 1) < 64, "vmcnt range");
+  static_assert(COPIES * STAGES < 64, "vmcnt range");
 
   extern __shared__ __align__(16) unsigned char smem[];
   const unsigned ldsBase = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)smem;
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept in an SGPR
-  const int wm = wave >> 1, wn = wave & 1;
+  const int wm = wave / WGN, wn = wave % WGN;
 
   unsigned tm, tn, bi;
   {
@@ -139,14 +143,17 @@ __global__ __launch_bounds__(kThreads) void qgemm_dma_kernel(const QGemmParams p
     const int k = s / BCH, phys = s % BCH;
     bOff[c] = k * N + n0 + ((phys ^ (k & 7)) << 4);
   }
-  auto issueSlab = [&](unsigned slab) {
+  // copy c (0 .. COPIES-1) of a slab: A chunks first, then B
+  auto issueCopy = [&](unsigned slab, int c) {
     const unsigned stage = slab % STAGES;
     const unsigned base = __builtin_amdgcn_readfirstlane(ldsBase + stage * STAGE_BYTES + wave * 1024);
     const unsigned k0 = slab * BK;
+    if (c < A_COPIES) dma16(rsrcA, base + c * (kThreads * 16), aOff[c] + k0);
+    else dma16(rsrcB, base + A_BYTES + (c - A_COPIES) * (kThreads * 16), bOff[c - A_COPIES] + k0 * N);
+  };
+  auto issueSlab = [&](unsigned slab) {
 #pragma unroll
-    for (int c = 0; c < A_COPIES; ++c) dma16(rsrcA, base + c * (kThreads * 16), aOff[c] + k0);
-#pragma unroll
-    for (int c = 0; c < B_COPIES; ++c) dma16(rsrcB, base + A_BYTES + c * (kThreads * 16), bOff[c] + k0 * N);
+    for (int c = 0; c < COPIES; ++c) issueCopy(slab, c);
   };
 
   v16i acc[MI][NI];
@@ -182,52 +189,84 @@ __global__ __launch_bounds__(kThreads) void qgemm_dma_kernel(const QGemmParams p
 #pragma unroll
   for (int j = 0; j < NI; ++j) bChunk[j] = (wn * WN + 32 * j + 16 * colHalf) >> 4;
 
-  const unsigned KT = (K + BK - 1) / BK;
-#pragma unroll
-  for (int s = 0; s < STAGES - 1; ++s) issueSlab(s);
-
-  for (unsigned kt = 0; kt < KT; ++kt) {
-    // slab kt has landed once at most the copies of the STAGES-2 younger slabs are outstanding
-    wait_vmcnt<COPIES*(STAGES - 2)>();
-    __syncthreads();
-    // every wavefront is past slab kt-1, whose stage is the one refilled now (copies past the end of
-    // K read zeros or unused bytes; issuing them keeps the outstanding-copy count uniform)
-    issueSlab(kt + STAGES - 1);
-
-    const unsigned char* as = smem + (kt % STAGES) * STAGE_BYTES;
+  // raw operand loads of one 32-deep k step of a stage (no arithmetic: nothing here waits for LDS);
+  // load q of a step: first two transposing reads per B block (the next step needs B first), then
+  // the A operand of each row block
+  constexpr int NLOAD = MI + 2 * NI, NMFMA = MI * NI;
+  auto loadOne = [&](const unsigned char* as, const unsigned char* bs, int ks, int q, v4i (&af)[MI], v4i (&bf)[NI]) {
+    if (q >= 2 * NI) {
+      af[q - 2 * NI] = *reinterpret_cast<const v4i*>(as + aAddr[q - 2 * NI][ks]);
+    } else {
+      const int j = q >> 1, half = q & 1;
+      const int k = 32 * ks + 16 * g + 8 * half + trK;  // (k & 7) == trK
+      const unsigned char* ptr = bs + k * BN + ((bChunk[j] ^ trK) << 4) + trByte;
+      v2i t = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+          (__attribute__((address_space(3))) v2i*)(const_cast<unsigned char*>(ptr)));
+      bf[j][2 * half] = t[0];
+      bf[j][2 * half + 1] = t[1];
+    }
+  };
+  // One k step: the matrix ops on operands (ua, ub) that were read during the previous step, with the
+  // LDS reads of the next step's operands (la, lb) issued two at a time between the first half of
+  // them: spread out enough not to queue up behind the other wavefronts' reads (all wavefronts run in
+  // phase, one barrier per slab), early enough to have returned when the step ends.
+  // uint8 -> int8 is the xor on the A operands; block j's column sums belong to wavefront row j % WGM.
+  // When `refill` is set the copies of slab `refillSlab` are issued as well, spread over the step for
+  // the same reason.
+  auto step = [&](v4i (&ua)[MI], v4i (&ub)[NI], v4i (&la)[MI], v4i (&lb)[NI], unsigned stage, int ks,
+                  auto refill, unsigned refillSlab) {
+    constexpr bool REFILL = decltype(refill)::value;
+    constexpr int DMA_EVERY = NMFMA / COPIES > 0 ? NMFMA / COPIES : 1;
+    const unsigned char* as = smem + stage * STAGE_BYTES;
     const unsigned char* bs = as + A_BYTES;
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      v4i af[MI], bf[NI];
+    for (int j = 0; j < NI; ++j) {
+      if (j % WGM == wm) {
+        asm volatile("" ::: "memory");  // keep this a wave-uniform branch, not a select over both blocks
 #pragma unroll
-      for (int i = 0; i < MI; ++i) {
-        v4i v = *reinterpret_cast<const v4i*>(as + aAddr[i][ks]);
-        af[i] = v ^ (int)0x80808080;
+        for (int q = 0; q < 4; ++q) colsum[j] = __builtin_amdgcn_sdot4(ub[j][q], 0x01010101, colsum[j], false);
       }
+    }
+    v4i ax = {0, 0, 0, 0};
 #pragma unroll
-      for (int j = 0; j < NI; ++j) {
+    for (int m = 0; m < NMFMA; ++m) {
+      const int i = m / NI, j = m % NI;
 #pragma unroll
-        for (int half = 0; half < 2; ++half) {
-          const int k = 32 * ks + 16 * g + 8 * half + trK;  // (k & 7) == trK
-          const unsigned char* ptr = bs + k * BN + ((bChunk[j] ^ trK) << 4) + trByte;
-          v2i t = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-              (__attribute__((address_space(3))) v2i*)(const_cast<unsigned char*>(ptr)));
-          bf[j][2 * half] = t[0];
-          bf[j][2 * half + 1] = t[1];
+      for (int q = 2 * m; q < 2 * m + 2 && q < NLOAD; ++q) loadOne(as, bs, ks, q, la, lb);
+      if constexpr (REFILL) {
+        if (m % DMA_EVERY == 0 && m / DMA_EVERY < COPIES) issueCopy(refillSlab, m / DMA_EVERY);
+        if (m == NMFMA - 1) {
+#pragma unroll
+          for (int c = NMFMA / DMA_EVERY; c < COPIES; ++c) issueCopy(refillSlab, c);  // more copies than matrix ops
         }
       }
-      if (wm == 0) {
-#pragma unroll
-        for (int j = 0; j < NI; ++j)
-#pragma unroll
-          for (int q = 0; q < 4; ++q) colsum[j] = __builtin_amdgcn_sdot4(bf[j][q], 0x01010101, colsum[j], false);
-      }
-#pragma unroll
-      for (int i = 0; i < MI; ++i)
-#pragma unroll
-        for (int j = 0; j < NI; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(bf[j], af[i], acc[i][j], 0, 0, 0);
+      if (j == 0) ax = ua[i] ^ (int)0x80808080;
+      acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ub[j], ax, acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
+  };
+
+  // Software pipeline.  The ring holds STAGES slabs.  One barrier per slab, in the middle of it:
+  //   before it: this wavefront's copies of slab kt+1 have landed and its reads of slab kt are done
+  //   after it : slab kt+1 is complete and visible, slab kt's stage is free and is refilled with
+  //              slab kt+STAGES (copies past the end of K read zeros or unused bytes; they are issued
+  //              anyway to keep the outstanding-copy count uniform)
+  const unsigned KT = (K + BK - 1) / BK;
+#pragma unroll
+  for (int s = 0; s < STAGES; ++s) issueSlab(s);
+  wait_vmcnt<COPIES*(STAGES - 1)>();
+  __syncthreads();
+  v4i fa[2][MI], fb[2][NI];
+#pragma unroll
+  for (int q = 0; q < NLOAD; ++q) loadOne(smem, smem + A_BYTES, 0, q, fa[0], fb[0]);
+  for (unsigned kt = 0; kt < KT; ++kt) {
+    const unsigned cur = kt % STAGES, nxt = (kt + 1) % STAGES;
+    step(fa[0], fb[0], fa[1], fb[1], cur, 1, std::false_type{}, 0u);   // k step 0 of slab kt; reads k step 1
+    wait_vmcnt<COPIES*(STAGES - 2)>();
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the reads of slab kt have returned
+    __syncthreads();
+    // k step 1 of slab kt; reads k step 0 of slab kt+1; refills the stage of slab kt
+    step(fa[1], fb[1], fa[0], fb[0], nxt, 0, std::true_type{}, kt + STAGES);
   }
   wait_vmcnt<0>();
   __syncthreads();
@@ -238,12 +277,12 @@ __global__ __launch_bounds__(kThreads) void qgemm_dma_kernel(const QGemmParams p
   int* rowTerm = colTerm + BN;                  // [BM]
   unsigned char* stageQ = smem + (BM + BN) * 4; // [BM][BN + 4] bytes, requantized tile
   constexpr int QPITCH = BN + 4;
-  if (wm == 0) {
-    // lanes l and l+32 hold the two k halves of the same column
+  // lanes l and l+32 hold the two k halves of the same column; the transposing read hands lane
+  // (colHalf, s16) column 16*colHalf + s16 of the 32-column block
 #pragma unroll
-    for (int j = 0; j < NI; ++j) {
+  for (int j = 0; j < NI; ++j) {
+    if (j % WGM == wm) {
       int s = colsum[j] + __shfl_xor(colsum[j], 32, 64);
-      // tr-read column order: lane (colHalf, s16) -> column 16*colHalf + 8*(s16>>3) + (s16&7) = 16*colHalf + s16
       if (g == 0) colTerm[wn * WN + 32 * j + 16 * colHalf + s16] = s;
     }
   }
@@ -278,7 +317,7 @@ __global__ __launch_bounds__(kThreads) void qgemm_dma_kernel(const QGemmParams p
   unsigned char* Q = REQUANT ? p.Q + (size_t)bi * p.strideC : nullptr;
 
   auto storeTile = [&](auto flavour) {
-    constexpr int FLAVOUR = decltype(flavour)::value;  // 0 int32 only, 1 fast requantize, 2 exact, 3 fill
+    constexpr int FLAVOUR = decltype(flavour)::value;  // 0 int32 only, 1 double shortcut, 2 exact int64, 3 fill, 4 int32 shortcut
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
       const int trow = wm * WM + 32 * i + l32;
@@ -301,6 +340,7 @@ __global__ __launch_bounds__(kThreads) void qgemm_dma_kernel(const QGemmParams p
             for (int e = 0; e < 4; ++e) {
               if constexpr (FLAVOUR == 1) q[e] = (unsigned)requantize_one_fast((double)((unsigned)v[e] ^ 0x80000000u), rq);
               else if constexpr (FLAVOUR == 2) q[e] = (unsigned)requantize_one_exact((long long)v[e], rq);
+              else if constexpr (FLAVOUR == 4) q[e] = (unsigned)requantize_one_fast32((double)((unsigned)v[e] ^ 0x80000000u), rq);
               else q[e] = (unsigned)rq.fillValue;
             }
             *reinterpret_cast<unsigned*>(stageQ + trow * QPITCH + tcol) = q[0] | (q[1] << 8) | (q[2] << 16) | (q[3] << 24);
@@ -313,6 +353,7 @@ __global__ __launch_bounds__(kThreads) void qgemm_dma_kernel(const QGemmParams p
     storeTile(std::integral_constant<int, 0>{});
   } else {
     if (rq.mode) storeTile(std::integral_constant<int, 3>{});
+    else if (rq.fast32OK) storeTile(std::integral_constant<int, 4>{});
     else if (rq.fastOK) storeTile(std::integral_constant<int, 1>{});
     else storeTile(std::integral_constant<int, 2>{});
     __syncthreads();
@@ -329,8 +370,9 @@ __global__ __launch_bounds__(kThreads) void qgemm_dma_kernel(const QGemmParams p
   }
 }
 
-template <int BM, int BN, int STAGES, bool REQUANT>
+template <int BM, int BN, int WGM, int WGN, int STAGES, bool REQUANT>
 int launch(hipStream_t stream, QGemmParams p) {
+  constexpr int kThreads = WGM * WGN * 64;
   p.tilesM = (p.M + BM - 1) / BM;
   p.tilesN = (p.N + BN - 1) / BN;
   unsigned long long total = (unsigned long long)p.tilesM * p.tilesN * p.batch;
@@ -341,7 +383,7 @@ int launch(hipStream_t stream, QGemmParams p) {
   constexpr size_t epi = (size_t)(BM + BN) * 4 + (size_t)BM * (BN + 4);
   constexpr size_t lds = ring > epi ? ring : epi;
   static_assert(lds <= 160 * 1024, "LDS budget");
-  auto kern = qgemm_dma_kernel<BM, BN, STAGES, REQUANT>;
+  auto kern = qgemm_dma_kernel<BM, BN, WGM, WGN, STAGES, REQUANT>;
   static bool attrSet = false;
   if (!attrSet) {
     TFCC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -365,9 +407,9 @@ bool qgemm_dma_supported(const QGemmParams& p, bool requant) {
 int qgemm_dma_launch(hipStream_t stream, const QGemmParams& p, bool requant) {
   const unsigned long long big = (unsigned long long)((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batch;
   if (big >= 192) {
-    return requant ? launch<256, 256, 4, true>(stream, p) : launch<256, 256, 4, false>(stream, p);
+    return requant ? launch<256, 256, 2, 4, 4, true>(stream, p) : launch<256, 256, 2, 4, 4, false>(stream, p);
   }
-  return requant ? launch<128, 128, 4, true>(stream, p) : launch<128, 128, 4, false>(stream, p);
+  return requant ? launch<128, 128, 2, 2, 4, true>(stream, p) : launch<128, 128, 2, 2, 4, false>(stream, p);
 }
 
 }  // namespace tfcc_rocm

@@ -143,6 +143,11 @@ __global__ __launch_bounds__(256) void requantize_s32_u8_vec_kernel(const int4* 
     unsigned q0, q1, q2, q3;
     if (s.mode) {
       q0 = q1 = q2 = q3 = (unsigned)s.fillValue;
+    } else if (s.fast32OK) {
+      q0 = (unsigned)requantize_one_fast32((double)((unsigned)v.x ^ 0x80000000u), s);
+      q1 = (unsigned)requantize_one_fast32((double)((unsigned)v.y ^ 0x80000000u), s);
+      q2 = (unsigned)requantize_one_fast32((double)((unsigned)v.z ^ 0x80000000u), s);
+      q3 = (unsigned)requantize_one_fast32((double)((unsigned)v.w ^ 0x80000000u), s);
     } else if (s.fastOK) {
       q0 = (unsigned)requantize_one_fast((double)((unsigned)v.x ^ 0x80000000u), s);
       q1 = (unsigned)requantize_one_fast((double)((unsigned)v.y ^ 0x80000000u), s);
