@@ -212,6 +212,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-other", action="store_true", help="skip the secondary configs")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="instead of the benchmark, run a plain streaming kernel of known size (reads and writes "
+                         "256 MiB each per launch) to calibrate the FETCH_SIZE / WRITE_SIZE counters against")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the matmul path has no multi-GPU part (run with --gpus 1)")
@@ -224,6 +227,18 @@ def main():
         sys.exit("bench.py needs a GPU")
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.copy_calibration:
+        n = 64 * 1024 * 1024  # floats: 256 MiB in, 256 MiB out
+        src = torch.ones(n, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        stream = torch.cuda.current_stream().cuda_stream
+        for _ in range(args.warmup + args.steps):
+            pkg.check(pkg.lib().tfcc_rocm_transform_f32(stream, src.data_ptr(), n, 1.0, 0.0, dst.data_ptr()))
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration_kernel": "transform_kernel", "read_bytes_per_launch": 4 * n,
+                          "write_bytes_per_launch": 4 * n, "launches": args.warmup + args.steps}))
+        return
 
     size = 4096
     c3 = c3_setup(torch, pkg, dev, seed=0, size=size)

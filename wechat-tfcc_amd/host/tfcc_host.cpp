@@ -1,0 +1,655 @@
+// Implementation of the host-side framework (allocators, device / session bookkeeping) and of the
+// ROCm device: every GPU action goes through the C ABI of libtfcc_rocm.so.
+#include <algorithm>
+#include <cstdlib>
+#include <cstring>
+
+#include "tfcc_rocm.h"
+#include "tfcc_rocm_device.h"
+
+namespace tfcc {
+
+// ---------------------------------------------------------------------------------------------
+// framework
+// ---------------------------------------------------------------------------------------------
+thread_local Device* Device::_threadDevice = nullptr;
+thread_local Session* Session::_threadSession = nullptr;
+
+Device::Device(DeviceType type, unsigned index, std::unique_ptr<Allocator> allocator)
+    : _deviceID((static_cast<unsigned>(type) << 24) | (index & 0x00ffffffu)),
+      _allocator(std::move(allocator)),
+      _interfaces(new InterfaceSet()) {}
+
+Device::~Device() {
+  if (_threadDevice == this) _threadDevice = nullptr;
+}
+
+void Session::preRelease() {
+  for (auto& cb : _releaseCallbacks) cb(this);
+  _releaseCallbacks.clear();
+  if (_threadSession == this) _threadSession = nullptr;
+}
+
+namespace detail {
+
+void check_same_area(const Shape& from, const Shape& to) {
+  if (from.area() != to.area()) throw InvalidArgumentError("shape area couldn't be changed");
+}
+
+Shape expand_dims(const Shape& s, size_t axis) {
+  if (axis > s.size()) throw InvalidArgumentError("invalid axis to expand");
+  std::vector<unsigned> dims = s.toVector();
+  dims.insert(dims.begin() + static_cast<std::ptrdiff_t>(axis), 1u);
+  return Shape(std::move(dims));
+}
+
+Shape squeeze_all(const Shape& s) {
+  std::vector<unsigned> dims;
+  for (unsigned d : s.toVector())
+    if (d != 1) dims.push_back(d);
+  Shape r(std::move(dims));
+  check_same_area(s, r);
+  return r;
+}
+
+Shape squeeze_axes(const Shape& s, const std::set<size_t>& axes) {
+  if (!axes.empty() && *axes.rbegin() >= s.size()) throw InvalidArgumentError("invalid axis to squeeze");
+  std::vector<unsigned> dims;
+  for (size_t i = 0; i < s.size(); ++i) {
+    if (axes.count(i)) {
+      if (s[i] != 1) throw InvalidArgumentError("invalid axis to squeeze");
+    } else {
+      dims.push_back(s[i]);
+    }
+  }
+  return Shape(std::move(dims));
+}
+
+}  // namespace detail
+
+// ---- FlexAllocator -------------------------------------------------------------------------------
+
+size_t FlexAllocator::bucket(size_t len) {
+  len += 64;  // header room, part of the accounting the reference's test pins
+  const size_t grain = len < (size_t(4) << 20) ? size_t(4096) : (size_t(1) << 20);
+  return (len + grain - 1) / grain * grain;
+}
+
+FlexAllocator::~FlexAllocator() {
+  // blocks still handed out at this point are a bug of the owner; the cache is returned
+  releaseDownTo(0);
+}
+
+void* FlexAllocator::malloc(size_t len) {
+  if (len == 0) return nullptr;
+  const size_t size = bucket(len);
+  void* p = nullptr;
+  {
+    std::lock_guard<std::mutex> lk(_mtx);
+    auto it = _cached.find(size);
+    if (it != _cached.end()) {
+      p = it->second;
+      _cached.erase(it);
+    }
+  }
+  if (p == nullptr) {
+    if (_limit == 0 || _used.load() + size <= _limit) p = _realMalloc(size);
+    if (p == nullptr) {
+      // over the limit, or the device is out of memory: give the cache back and try once more
+      releaseDownTo(0);
+      if (_limit == 0 || _used.load() + size <= _limit) p = _realMalloc(size);
+    }
+    if (p == nullptr) return nullptr;
+    _used += size;
+  }
+  {
+    std::lock_guard<std::mutex> lk(_mtx);
+    _live[p] = size;
+  }
+  if (_flexLimit != 0 && _used.load() > _flexLimit) releaseDownTo(_flexLimit / 2);
+  return p;
+}
+
+void FlexAllocator::free(void* p) {
+  if (p == nullptr) return;
+  std::lock_guard<std::mutex> lk(_mtx);
+  auto it = _live.find(p);
+  if (it == _live.end()) return;
+  _cached.emplace(it->second, p);
+  _live.erase(it);
+}
+
+void FlexAllocator::releaseDownTo(size_t target) {
+  while (_used.load() > target) {
+    void* p = nullptr;
+    size_t size = 0;
+    {
+      std::lock_guard<std::mutex> lk(_mtx);
+      if (_cached.empty()) return;
+      auto it = _cached.begin();  // smallest bucket first
+      size = it->first;
+      p = it->second;
+      _cached.erase(it);
+    }
+    _realFree(p);
+    _used -= size;
+  }
+}
+
+void* SimpleAllocator::malloc(size_t len) {
+  if (len == 0) return nullptr;
+  if (_limit != 0 && _used.load() + len > _limit) return nullptr;
+  void* p = _realMalloc(len);
+  if (p == nullptr) return nullptr;
+  std::lock_guard<std::mutex> lk(_mtx);
+  _live[p] = len;
+  _used += len;
+  return p;
+}
+
+void SimpleAllocator::free(void* p) {
+  if (p == nullptr) return;
+  {
+    std::lock_guard<std::mutex> lk(_mtx);
+    auto it = _live.find(p);
+    if (it == _live.end()) return;
+    _used -= it->second;
+    _live.erase(it);
+  }
+  _realFree(p);
+}
+
+// ---------------------------------------------------------------------------------------------
+// host device
+// ---------------------------------------------------------------------------------------------
+HostDevice::HostDevice() : Device(DeviceType::HOST, 0, std::unique_ptr<Allocator>(new FlexAllocator())) {
+  _allocator->setRealMalloc([](size_t len) -> void* { return std::aligned_alloc(64, (len + 63) / 64 * 64); });
+  _allocator->setRealFree([](void* p) { std::free(p); });
+}
+
+HostSession::HostSession(HostDevice& device) : Session(std::unique_ptr<Allocator>(new FlexAllocator())), _device(device) {
+  _allocator->setRealMalloc([this](size_t len) { return _device.malloc(len); });
+  _allocator->setRealFree([this](void* p) { _device.free(p); });
+}
+
+HostSession::~HostSession() {
+  preRelease();
+  _allocator->releaseCache();
+}
+
+// ---------------------------------------------------------------------------------------------
+// ROCm device
+// ---------------------------------------------------------------------------------------------
+namespace {
+
+inline void check(int status) {
+  if (status != TFCC_ROCM_OK) throw ROCMRuntimeError(status, tfcc_rocm_last_error_string());
+}
+
+inline void* current_stream() {
+  auto* s = dynamic_cast<ROCMSession*>(Session::getThreadDefault());
+  if (s == nullptr) throw RuntimeError("the thread's default session is not a ROCm session");
+  return s->getStream();
+}
+
+template <class T>
+constexpr int type_code();
+template <> constexpr int type_code<int8_t>() { return TFCC_ROCM_S8; }
+template <> constexpr int type_code<uint8_t>() { return TFCC_ROCM_U8; }
+template <> constexpr int type_code<int16_t>() { return TFCC_ROCM_S16; }
+template <> constexpr int type_code<uint16_t>() { return TFCC_ROCM_U16; }
+template <> constexpr int type_code<int32_t>() { return TFCC_ROCM_S32; }
+template <> constexpr int type_code<uint32_t>() { return TFCC_ROCM_U32; }
+
+inline void require_scalar(const Tensor<float>& t, const char* what) {
+  if (t.size() != 1 || t.shape().size() != 1) throw InvalidArgumentError(what);
+}
+
+// ---- data ------------------------------------------------------------------------------------
+template <class T>
+class ROCMDataInterface : public DataInterface<T> {
+ public:
+  void set(T* dst, const T* data, size_t len) override {
+    check(tfcc_rocm_memcpy_h2d(current_stream(), dst, data, len * sizeof(T)));
+  }
+  void set(Variable<T>& a, const T* data) override { set(a.data(), data, a.size()); }
+  void set(Variable<T>& a, std::vector<T>&& data) override { set(a.data(), data.data(), a.size()); }
+  void get(const Tensor<T>& a, T* data) override {
+    check(tfcc_rocm_memcpy_d2h(current_stream(), data, a.data(), static_cast<size_t>(a.size()) * sizeof(T)));
+  }
+  void zeros(Variable<T>& a) override {
+    check(tfcc_rocm_fill_async(current_stream(), a.data(), 0, sizeof(T), a.size()));
+  }
+  void ones(Variable<T>& a) override {
+    T one = static_cast<T>(1);
+    uint64_t bits = 0;
+    std::memcpy(&bits, &one, sizeof(T));
+    check(tfcc_rocm_fill_async(current_stream(), a.data(), bits, sizeof(T), a.size()));
+  }
+  Variable<T> copy(const Tensor<T>& a) override {
+    Variable<T> r(a.shape());
+    check(tfcc_rocm_memcpy_d2d_async(current_stream(), r.data(), a.data(), static_cast<size_t>(a.size()) * sizeof(T)));
+    return r;
+  }
+};
+
+// ---- blas --------------------------------------------------------------------------------------
+// Stride rules of the reference's blas interface (tfcc/mkl/interfaces/tfcc_mklblasinterface.cpp:127-186):
+// a rank-2 operand against a batched one is shared by the whole batch (stride 0).
+class ROCMBlasInterface : public BlasInterface<float> {
+  static Variable<float> run(const Tensor<float>& a, const Tensor<float>& b, const Tensor<float>* bias) {
+    const size_t ra = a.shape().size(), rb = b.shape().size();
+    const unsigned m = a.shape(ra - 2), n = b.shape(rb - 1), k = a.shape(ra - 1);
+    uint64_t strideA = static_cast<uint64_t>(m) * k, strideB = static_cast<uint64_t>(n) * k;
+    if (ra != rb) {
+      if (ra == 2) strideA = 0;
+      if (rb == 2) strideB = 0;
+    }
+    std::vector<unsigned> s = ra > rb ? a.shape().toVector() : b.shape().toVector();
+    s[s.size() - 2] = m;
+    s[s.size() - 1] = n;
+    Variable<float> result{Shape(std::move(s))};
+    const unsigned batch = result.size() / (m * n);
+    check(tfcc_rocm_sgemm_strided_batched(current_stream(), a.data(), strideA, b.data(), strideB,
+                                          bias ? bias->data() : nullptr, result.data(),
+                                          static_cast<uint64_t>(m) * n, m, n, k, batch));
+    return result;
+  }
+
+ public:
+  Variable<float> matmul(const Tensor<float>& a, const Tensor<float>& b) override { return run(a, b, nullptr); }
+  Variable<float> matmul(const Tensor<float>& a, const Tensor<float>& b, const Tensor<float>& bias) override {
+    return run(a, b, &bias);
+  }
+};
+
+// ---- quantization --------------------------------------------------------------------------------
+template <class T>
+class ROCMQuantizationInterface : public QuantizationInterface<T> {
+  template <class TI>
+  static Variable<T> requantizeImpl(const Tensor<TI>& a, const Tensor<float>& minInput, const Tensor<float>& maxInput,
+                                    const Tensor<float>& minOutput, const Tensor<float>& maxOutput) {
+    if (a.size() == 0) throw InvalidArgumentError("invalid tensor");
+    require_scalar(minInput, "invalid minInput");
+    require_scalar(maxInput, "invalid maxInput");
+    require_scalar(minOutput, "invalid minOutput");
+    require_scalar(maxOutput, "invalid maxOutput");
+    Variable<T> result(a.shape());
+    check(tfcc_rocm_requantize(current_stream(), a.data(), type_code<TI>(), result.data(), type_code<T>(), a.size(),
+                               minInput.data(), maxInput.data(), minOutput.data(), maxOutput.data()));
+    return result;
+  }
+
+ public:
+  std::tuple<Variable<T>, Variable<float>, Variable<float>> quantize(const Tensor<float>& a) override {
+    if (a.size() == 0) throw InvalidArgumentError("invalid tensor");
+    Variable<T> result(a.shape());
+    Variable<float> minValue({1}), maxValue({1});
+    check(tfcc_rocm_quantize_minmax(current_stream(), a.data(), a.size(), result.data(), type_code<T>(),
+                                    minValue.data(), maxValue.data()));
+    return std::make_tuple(std::move(result), std::move(minValue), std::move(maxValue));
+  }
+  Variable<T> quantize(const Tensor<float>& a, const Tensor<float>& minValue, const Tensor<float>& maxValue) override {
+    if (a.size() == 0) throw InvalidArgumentError("invalid tensor");
+    require_scalar(minValue, "invalid minValue");
+    require_scalar(maxValue, "invalid maxValue");
+    Variable<T> result(a.shape());
+    check(tfcc_rocm_quantize(current_stream(), a.data(), a.size(), minValue.data(), maxValue.data(), result.data(),
+                             type_code<T>()));
+    return result;
+  }
+#define TFCC_ROCM_REQUANTIZE(TI)                                                                                \
+  Variable<T> requantize(const Tensor<TI>& a, const Tensor<float>& minInput, const Tensor<float>& maxInput,      \
+                         const Tensor<float>& minOutput, const Tensor<float>& maxOutput) override {             \
+    return requantizeImpl<TI>(a, minInput, maxInput, minOutput, maxOutput);                                     \
+  }
+  TFCC_ROCM_REQUANTIZE(int8_t)
+  TFCC_ROCM_REQUANTIZE(uint8_t)
+  TFCC_ROCM_REQUANTIZE(int16_t)
+  TFCC_ROCM_REQUANTIZE(uint16_t)
+  TFCC_ROCM_REQUANTIZE(int32_t)
+  TFCC_ROCM_REQUANTIZE(uint32_t)
+#undef TFCC_ROCM_REQUANTIZE
+  Variable<float> dequantize(const Tensor<T>& a, const Tensor<float>& minValue, const Tensor<float>& maxValue) override {
+    if (a.size() == 0) throw InvalidArgumentError("invalid tensor");
+    require_scalar(minValue, "invalid minValue");
+    require_scalar(maxValue, "invalid maxValue");
+    Variable<float> result(a.shape());
+    check(tfcc_rocm_dequantize(current_stream(), a.data(), type_code<T>(), a.size(), minValue.data(), maxValue.data(),
+                               result.data()));
+    return result;
+  }
+};
+
+// ---- the element-wise neighbours (float only) ----------------------------------------------------------
+class ROCMActivationInterface : public ActivationInterface<float> {
+ public:
+  Variable<float> softmax(const Tensor<float>& a, size_t axis) override {
+    if (a.size() == 0) throw InvalidArgumentError("invalid tensor");
+    if (axis + 1 != a.shape().size()) throw NotImplementedError("softmax over the last axis only");
+    Variable<float> r(a.shape());
+    const unsigned cols = a.shape(axis);
+    check(tfcc_rocm_softmax_f32(current_stream(), a.data(), a.size() / cols, cols, r.data()));
+    return r;
+  }
+  Variable<float> geluAccurate(const Tensor<float>& a) override {
+    Variable<float> r(a.shape());
+    check(tfcc_rocm_gelu_accurate_f32(current_stream(), a.data(), a.size(), r.data()));
+    return r;
+  }
+};
+
+class ROCMNormalizationInterface : public NormalizationInterface<float> {
+ public:
+  Variable<float> layerNormalize(const Tensor<float>& a, const Tensor<float>& gamma, const Tensor<float>& beta,
+                                 float epsilon, size_t beginNormAxis) override {
+    if (beginNormAxis >= a.shape().size()) throw InvalidArgumentError("invalid beginNormAxis");
+    unsigned cols = 1;
+    for (size_t i = beginNormAxis; i < a.shape().size(); ++i) cols *= a.shape(i);
+    if (gamma.size() != cols || beta.size() != cols) throw InvalidArgumentError("gamma, beta and the normalized dims don't match");
+    if (a.size() == 0) throw InvalidArgumentError("invalid tensor");
+    Variable<float> r(a.shape());
+    check(tfcc_rocm_layer_norm_f32(current_stream(), a.data(), gamma.data(), beta.data(), epsilon, a.size() / cols, cols,
+                                   r.data()));
+    return r;
+  }
+};
+
+class ROCMBasicInterface : public BasicInterface<float> {
+ public:
+  Variable<float> transpose(const Tensor<float>& a, const std::vector<size_t>& perm) override {
+    if (a.size() == 0) throw InvalidArgumentError("invalid tensor");
+    std::vector<unsigned> shape = a.shape().toVector(), p(perm.begin(), perm.end()), out(perm.size());
+    for (size_t i = 0; i < perm.size(); ++i) out[i] = shape[perm[i]];
+    Variable<float> r{Shape(std::move(out))};
+    check(tfcc_rocm_transpose_f32(current_stream(), a.data(), shape.data(), p.data(), static_cast<int>(p.size()), r.data()));
+    return r;
+  }
+};
+
+class ROCMArithmeticInterface : public ArithmeticInterface<float> {
+ public:
+  Variable<float> add(const Tensor<float>& a, const Tensor<float>& b) override {
+    // b equals the trailing dimensions of a (bias / residual forms)
+    const size_t ra = a.shape().size(), rb = b.shape().size();
+    bool ok = rb <= ra && a.size() > 0 && b.size() > 0;
+    for (size_t i = 0; ok && i < rb; ++i) ok = a.shape(ra - rb + i) == b.shape(i);
+    if (!ok) throw NotImplementedError("add: only a trailing-dimension broadcast of the second operand");
+    Variable<float> r(a.shape());
+    check(tfcc_rocm_add_f32(current_stream(), a.data(), b.data(), a.size(), b.size(), r.data()));
+    return r;
+  }
+};
+
+class ROCMTransformationInterface : public TransformationInterface<float> {
+ public:
+  Variable<float> transform(const Tensor<float>& a, float alpha, float beta) override {
+    if (a.size() == 0) throw InvalidArgumentError("invalid tensor");
+    Variable<float> r(a.shape());
+    check(tfcc_rocm_transform_f32(current_stream(), a.data(), a.size(), alpha, beta, r.data()));
+    return r;
+  }
+};
+
+template <class T>
+void install_common(Interface<T>& i) {
+  i.setDataInterface(std::unique_ptr<DataInterface<T>>(new ROCMDataInterface<T>()));
+}
+template <class T>
+void install_quantization(Interface<T>& i) {
+  i.setQuantizationInterface(std::unique_ptr<QuantizationInterface<T>>(new ROCMQuantizationInterface<T>()));
+}
+
+}  // namespace
+
+unsigned ROCMDevice::getDeviceCount() {
+  int n = 0;
+  if (tfcc_rocm_device_count(&n) != TFCC_ROCM_OK) return 0;
+  return n > 0 ? static_cast<unsigned>(n) : 0u;
+}
+
+ROCMDevice::ROCMDevice(unsigned index) : ROCMDevice(index, std::unique_ptr<Allocator>(new FlexAllocator())) {
+  // leave a tenth of the card to the runtime, like the reference's GPU device
+  size_t freeBytes = 0, totalBytes = 0;
+  check(tfcc_rocm_set_device(static_cast<int>(_index)));
+  check(tfcc_rocm_mem_info(&freeBytes, &totalBytes));
+  _allocator->setLimit(totalBytes / 10 * 9);
+}
+
+ROCMDevice::ROCMDevice(unsigned index, std::unique_ptr<Allocator> allocator)
+    : Device(DeviceType::ROCM, index, std::move(allocator)), _index(index) {
+  check(tfcc_rocm_set_device(static_cast<int>(_index)));
+  const int idx = static_cast<int>(_index);
+  _allocator->setRealMalloc([idx](size_t len) -> void* {
+    void* p = nullptr;
+    if (tfcc_rocm_set_device(idx) != TFCC_ROCM_OK) return nullptr;
+    if (tfcc_rocm_malloc(&p, len) != TFCC_ROCM_OK) return nullptr;
+    return p;
+  });
+  _allocator->setRealFree([](void* p) { tfcc_rocm_free(p); });
+
+  install_common(_interfaces->f32);
+  install_common(_interfaces->f64);
+  install_common(_interfaces->s8);
+  install_common(_interfaces->u8);
+  install_common(_interfaces->s16);
+  install_common(_interfaces->u16);
+  install_common(_interfaces->s32);
+  install_common(_interfaces->u32);
+  install_common(_interfaces->s64);
+  install_common(_interfaces->u64);
+  // quantization for the six quantized element types (tfcc/mkl/interfaces/tfcc_mklinterface.cpp:45-50)
+  install_quantization(_interfaces->s8);
+  install_quantization(_interfaces->u8);
+  install_quantization(_interfaces->s16);
+  install_quantization(_interfaces->u16);
+  install_quantization(_interfaces->s32);
+  install_quantization(_interfaces->u32);
+  // matmul is float only, like the reference's MKL device; other types keep the throwing default
+  _interfaces->f32.setBlasInterface(std::unique_ptr<BlasInterface<float>>(new ROCMBlasInterface()));
+  _interfaces->f32.setActivationInterface(std::unique_ptr<ActivationInterface<float>>(new ROCMActivationInterface()));
+  _interfaces->f32.setNormalizationInterface(std::unique_ptr<NormalizationInterface<float>>(new ROCMNormalizationInterface()));
+  _interfaces->f32.setBasicInterface(std::unique_ptr<BasicInterface<float>>(new ROCMBasicInterface()));
+  _interfaces->f32.setArithmeticInterface(std::unique_ptr<ArithmeticInterface<float>>(new ROCMArithmeticInterface()));
+  _interfaces->f32.setTransformationInterface(std::unique_ptr<TransformationInterface<float>>(new ROCMTransformationInterface()));
+}
+
+ROCMDevice::~ROCMDevice() { _allocator->releaseCache(); }
+
+void ROCMDevice::attach() { check(tfcc_rocm_set_device(static_cast<int>(_index))); }
+
+ROCMSession::ROCMSession(ROCMDevice& device) : ROCMSession(device, std::unique_ptr<Allocator>(new FlexAllocator())) {}
+
+ROCMSession::ROCMSession(ROCMDevice& device, std::unique_ptr<Allocator> allocator)
+    : Session(std::move(allocator)), _device(device), _stream(nullptr) {
+  device.attach();
+  check(tfcc_rocm_stream_create(&_stream));
+  // session memory comes from the device allocator; a block only really goes back after the stream
+  // has drained, because kernels still queued may be using it
+  _allocator->setRealMalloc([this](size_t len) { return _device.malloc(len); });
+  _allocator->setRealFree([this](void* p) {
+    this->sync();
+    _device.free(p);
+  });
+}
+
+ROCMSession::~ROCMSession() {
+  preRelease();
+  tfcc_rocm_stream_synchronize(_stream);
+  _allocator->releaseCache();
+  tfcc_rocm_stream_destroy(_stream);
+}
+
+void ROCMSession::sync() const { check(tfcc_rocm_stream_synchronize(_stream)); }
+
+namespace {
+
+struct RocmRuntime {
+  std::mutex mtx;
+  std::vector<std::unique_ptr<ROCMDevice>> devices;
+};
+
+RocmRuntime& runtime() {
+  static RocmRuntime r;
+  return r;
+}
+
+struct ThreadBinding {
+  std::unique_ptr<ROCMSession> session;
+  ~ThreadBinding() {
+    if (session && Session::getThreadDefault() == session.get()) Session::setThreadDefault(nullptr);
+  }
+};
+
+void bind_thread(unsigned deviceID) {
+  thread_local ThreadBinding binding;
+  if (Device::getThreadDefault() != nullptr && Session::getThreadDefault() != nullptr) {
+    Device::getThreadDefault()->attach();
+    return;
+  }
+  RocmRuntime& r = runtime();
+  ROCMDevice* device = nullptr;
+  {
+    std::lock_guard<std::mutex> lk(r.mtx);
+    if (r.devices.empty()) {
+      unsigned n = ROCMDevice::getDeviceCount();
+      if (n == 0) throw RuntimeError("no ROCm device available");
+      for (unsigned i = 0; i < n; ++i) r.devices.emplace_back(new ROCMDevice(i));
+    }
+    if (deviceID >= r.devices.size()) throw InvalidArgumentError("invalid device id");
+    device = r.devices[deviceID].get();
+  }
+  binding.session.reset(new ROCMSession(*device));
+  Device::setThreadDefault(device);
+  Session::setThreadDefault(binding.session.get());
+}
+
+}  // namespace
+
+void initialize_rocm() { bind_thread(0); }
+void initialize_rocm(unsigned deviceID) { bind_thread(deviceID); }
+
+// ---------------------------------------------------------------------------------------------
+// quantized matmul
+// ---------------------------------------------------------------------------------------------
+namespace rocm {
+namespace quantization {
+
+namespace {
+
+struct QPlan {
+  tfcc_rocm_qgemm_desc desc;
+  std::vector<unsigned> shape;
+};
+
+// checks and batch folding of tfcc/mkl/operations/tfcc_mklquantization.cpp:75-145
+QPlan plan(const Tensor<uint8_t>& a, const Tensor<int32_t>& reduceSumA, const Tensor<float>& minA,
+           const Tensor<float>& maxA, const Tensor<int8_t>& b, const Tensor<int32_t>& reduceSumB,
+           const Tensor<float>& minB, const Tensor<float>& maxB) {
+  const size_t ra = a.shape().size(), rb = b.shape().size();
+  if (a.size() == 0 || ra < 2) throw InvalidArgumentError("invalid input tensor a");
+  if (reduceSumA.size() == 0) throw InvalidArgumentError("invalid tensor reduceSumA");
+  require_scalar(minA, "invalid tensor minA");
+  require_scalar(maxA, "invalid tensor maxA");
+  if (b.size() == 0 || rb < 2) throw InvalidArgumentError("invalid input tensor b");
+  if (reduceSumB.size() == 0) throw InvalidArgumentError("invalid tensor reduceSumB");
+  require_scalar(minB, "invalid tensor minB");
+  require_scalar(maxB, "invalid tensor maxB");
+  if (a.shape(ra - 1) != b.shape(rb - 2)) throw InvalidArgumentError("tensor a and b don't match");
+  if (ra != rb && ra != 2 && rb != 2) throw InvalidArgumentError("tensor a and b don't match");
+  if (a.shape(ra - 2) != reduceSumA.shape(reduceSumA.shape().size() - 1))
+    throw InvalidArgumentError("tensor a and reduceSumA don't match");
+  if (b.shape(rb - 1) != reduceSumB.shape(reduceSumB.shape().size() - 1))
+    throw InvalidArgumentError("tensor b and reduceSumB don't match");
+  if (ra == rb)
+    for (size_t i = 0; i + 2 < ra; ++i)
+      if (a.shape(i) != b.shape(i)) throw InvalidArgumentError("tensor a and b don't match");
+
+  QPlan p{};
+  p.shape = ra > rb ? a.shape().toVector() : b.shape().toVector();
+  unsigned m = a.shape(ra - 2), n = b.shape(rb - 1), k = a.shape(ra - 1);
+  p.shape[p.shape.size() - 2] = m;
+  p.shape[p.shape.size() - 1] = n;
+  unsigned batch = 1;
+  for (size_t i = 0; i + 2 < p.shape.size(); ++i) batch *= p.shape[i];
+  uint64_t strideRA = reduceSumA.shape().size() == 1 ? 0 : m;
+  uint64_t strideRB = reduceSumB.shape().size() == 1 ? 0 : n;
+  uint64_t strideA = ra == 2 ? 0 : static_cast<uint64_t>(m) * k;
+  uint64_t strideB = rb == 2 ? 0 : static_cast<uint64_t>(k) * n;
+  if (rb == 2) {  // one B for the whole batch: the batch becomes extra rows
+    m *= batch;
+    strideRA *= batch;
+    strideA *= batch;
+    batch = 1;
+  }
+  tfcc_rocm_qgemm_desc& d = p.desc;
+  d.a = a.data(); d.b = b.data(); d.rowsum_a = reduceSumA.data(); d.colsum_b = reduceSumB.data();
+  d.stride_a = strideA; d.stride_b = strideB; d.stride_rowsum_a = strideRA; d.stride_colsum_b = strideRB;
+  d.stride_c = static_cast<uint64_t>(m) * n;
+  d.m = m; d.n = n; d.k = k; d.batch = batch;
+  d.min_a = minA.data(); d.max_a = maxA.data(); d.min_b = minB.data(); d.max_b = maxB.data();
+  return p;
+}
+
+}  // namespace
+
+std::tuple<Variable<int32_t>, Variable<float>, Variable<float>> matmul(
+    const Tensor<uint8_t>& a, const Tensor<int32_t>& reduceSumA, const Tensor<float>& minA,
+    const Tensor<float>& maxA, const Tensor<int8_t>& b, const Tensor<int32_t>& reduceSumB,
+    const Tensor<float>& minB, const Tensor<float>& maxB) {
+  QPlan p = plan(a, reduceSumA, minA, maxA, b, reduceSumB, minB, maxB);
+  Variable<int32_t> result{Shape(p.shape)};
+  Variable<float> minResult({1}), maxResult({1});
+  p.desc.min_c = minResult.data();
+  p.desc.max_c = maxResult.data();
+  check(tfcc_rocm_gemm_u8s8s32(current_stream(), &p.desc, result.data()));
+  return std::make_tuple(std::move(result), std::move(minResult), std::move(maxResult));
+}
+
+std::tuple<Variable<uint8_t>, Variable<float>, Variable<float>> matmul_requantize(
+    const Tensor<uint8_t>& a, const Tensor<int32_t>& reduceSumA, const Tensor<float>& minA,
+    const Tensor<float>& maxA, const Tensor<int8_t>& b, const Tensor<int32_t>& reduceSumB,
+    const Tensor<float>& minB, const Tensor<float>& maxB, const Tensor<float>& minOutput,
+    const Tensor<float>& maxOutput, Variable<int32_t>* accumulators) {
+  QPlan p = plan(a, reduceSumA, minA, maxA, b, reduceSumB, minB, maxB);
+  require_scalar(minOutput, "invalid minOutput");
+  require_scalar(maxOutput, "invalid maxOutput");
+  Variable<uint8_t> result{Shape(p.shape)};
+  Variable<float> minResult({1}), maxResult({1});
+  p.desc.min_c = minResult.data();
+  p.desc.max_c = maxResult.data();
+  int32_t* acc = nullptr;
+  if (accumulators) {
+    *accumulators = Variable<int32_t>(Shape(p.shape));
+    acc = accumulators->data();
+  }
+  check(tfcc_rocm_gemm_u8s8s32_requant_u8(current_stream(), &p.desc, acc, result.data(), 0.0, 0.0, 0.0, 0,
+                                          minOutput.data(), maxOutput.data()));
+  return std::make_tuple(std::move(result), std::move(minResult), std::move(maxResult));
+}
+
+template <class T>
+Variable<int32_t> reduce_sum(const Tensor<T>& a, bool row) {
+  const size_t rank = a.shape().size();
+  if (a.size() == 0 || rank < 2) throw InvalidArgumentError("invalid input tensor a");
+  std::vector<unsigned> s = a.shape().toVector();
+  const unsigned r = s[rank - 2], c = s[rank - 1];
+  const unsigned batch = a.size() / r / c;
+  s.pop_back();
+  s.pop_back();
+  s.push_back(row ? r : c);
+  Variable<int32_t> result{Shape(std::move(s))};
+  if (row)
+    check(tfcc_rocm_reduce_sum_rows(current_stream(), a.data(), type_code<T>(), batch, r, c, result.data()));
+  else
+    check(tfcc_rocm_reduce_sum_cols(current_stream(), a.data(), type_code<T>(), batch, r, c, result.data()));
+  return result;
+}
+
+template Variable<int32_t> reduce_sum(const Tensor<int8_t>&, bool);
+template Variable<int32_t> reduce_sum(const Tensor<uint8_t>&, bool);
+template Variable<int32_t> reduce_sum(const Tensor<int16_t>&, bool);
+
+}  // namespace quantization
+}  // namespace rocm
+}  // namespace tfcc

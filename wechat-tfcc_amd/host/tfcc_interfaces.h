@@ -1,0 +1,342 @@
+// The plug-in surface a device implements, and the operator functions that dispatch to it.
+//
+// A device owns one Interface<T> per element type; each is a bundle of sub-interfaces whose
+// default implementation throws NotImplementedError, exactly as in the reference
+// (tfcc/core/interfaces/tfcc_interface.h:76-161, tfcc_blasinterface.cpp:23-30).  A backend
+// subclasses the sub-interfaces it supports and installs them with set*Interface from its device
+// constructor (tfcc/cuda/interfaces/tfcc_cudainterface.cpp:38-70).
+//
+// Sub-interfaces present here: the matmul path itself (Blas, Quantization, Data) and the few
+// neighbours one transformer encoder layer needs (Activation: softmax / geluAccurate,
+// Normalization: layerNormalize, Basic: transpose, Arithmetic: add, Transformation: transform).
+//
+// Operator functions (same names and checks as tfcc/core/operations/):
+//   blas::matmul            tfcc_blas.cpp:26-96
+//   data::set/get/...       tfcc_data.cpp
+//   quantization::*         tfcc_quantization.cpp:26-98
+//   math::softmax, gelu_accurate   tfcc_math.cpp:455-461,585-592
+//   nn::layer_normalization tfcc_nn.cpp:755-762
+//   base::transpose         tfcc_base.cpp:124-134
+#pragma once
+
+#include <tuple>
+
+#include "tfcc_core.h"
+
+namespace tfcc {
+
+template <class T>
+class BlasInterface {
+ public:
+  virtual ~BlasInterface() {}
+  // a: [..., m, k], b: [..., k, n]; one operand may be a plain matrix shared by the whole batch
+  virtual Variable<T> matmul(const Tensor<T>&, const Tensor<T>&) { throw NotImplementedError(); }
+  // c = a * b + bias, bias: [n]
+  virtual Variable<T> matmul(const Tensor<T>&, const Tensor<T>&, const Tensor<T>&) { throw NotImplementedError(); }
+};
+
+template <class T>
+class QuantizationInterface {
+ public:
+  virtual ~QuantizationInterface() {}
+  virtual std::tuple<Variable<T>, Variable<float>, Variable<float>> quantize(const Tensor<float>&) {
+    throw NotImplementedError();
+  }
+  virtual Variable<T> quantize(const Tensor<float>&, const Tensor<float>&, const Tensor<float>&) {
+    throw NotImplementedError();
+  }
+#define TFCC_REQUANTIZE_DEFAULT(TI)                                                                        \
+  virtual Variable<T> requantize(const Tensor<TI>&, const Tensor<float>&, const Tensor<float>&,            \
+                                 const Tensor<float>&, const Tensor<float>&) {                             \
+    throw NotImplementedError();                                                                           \
+  }
+  TFCC_REQUANTIZE_DEFAULT(int8_t)
+  TFCC_REQUANTIZE_DEFAULT(uint8_t)
+  TFCC_REQUANTIZE_DEFAULT(int16_t)
+  TFCC_REQUANTIZE_DEFAULT(uint16_t)
+  TFCC_REQUANTIZE_DEFAULT(int32_t)
+  TFCC_REQUANTIZE_DEFAULT(uint32_t)
+#undef TFCC_REQUANTIZE_DEFAULT
+  virtual Variable<float> dequantize(const Tensor<T>&, const Tensor<float>&, const Tensor<float>&) {
+    throw NotImplementedError();
+  }
+};
+
+template <class T>
+class DataInterface {
+ public:
+  virtual ~DataInterface() {}
+  virtual void set(T*, const T*, size_t) { throw NotImplementedError(); }  // host -> device, len elements
+  virtual void set(Variable<T>&, const T*) { throw NotImplementedError(); }
+  virtual void set(Variable<T>&, std::vector<T>&&) { throw NotImplementedError(); }
+  virtual void get(const Tensor<T>&, T*) { throw NotImplementedError(); }  // device -> host, synchronises
+  virtual void zeros(Variable<T>&) { throw NotImplementedError(); }
+  virtual void ones(Variable<T>&) { throw NotImplementedError(); }
+  virtual Variable<T> copy(const Tensor<T>&) { throw NotImplementedError(); }
+};
+
+template <class T>
+class ActivationInterface {
+ public:
+  virtual ~ActivationInterface() {}
+  virtual Variable<T> softmax(const Tensor<T>&, size_t) { throw NotImplementedError(); }
+  virtual Variable<T> geluAccurate(const Tensor<T>&) { throw NotImplementedError(); }
+};
+
+template <class T>
+class NormalizationInterface {
+ public:
+  virtual ~NormalizationInterface() {}
+  virtual Variable<T> layerNormalize(const Tensor<T>&, const Tensor<T>&, const Tensor<T>&, T, size_t) {
+    throw NotImplementedError();
+  }
+};
+
+template <class T>
+class BasicInterface {
+ public:
+  virtual ~BasicInterface() {}
+  virtual Variable<T> transpose(const Tensor<T>&, const std::vector<size_t>&) { throw NotImplementedError(); }
+};
+
+template <class T>
+class ArithmeticInterface {
+ public:
+  virtual ~ArithmeticInterface() {}
+  virtual Variable<T> add(const Tensor<T>&, const Tensor<T>&) { throw NotImplementedError(); }
+};
+
+template <class T>
+class TransformationInterface {
+ public:
+  virtual ~TransformationInterface() {}
+  virtual Variable<T> transform(const Tensor<T>&, T, T) { throw NotImplementedError(); }  // a * alpha + beta
+};
+
+template <class T>
+class Interface {
+#define TFCC_SUB_INTERFACE(NAME)                                                     \
+ private:                                                                            \
+  std::unique_ptr<NAME##Interface<T>> _##NAME{new NAME##Interface<T>()};             \
+                                                                                     \
+ public:                                                                             \
+  NAME##Interface<T>& get##NAME##Interface() { return *_##NAME; }                    \
+  void set##NAME##Interface(std::unique_ptr<NAME##Interface<T>> p) { _##NAME = std::move(p); }
+  TFCC_SUB_INTERFACE(Blas)
+  TFCC_SUB_INTERFACE(Quantization)
+  TFCC_SUB_INTERFACE(Data)
+  TFCC_SUB_INTERFACE(Activation)
+  TFCC_SUB_INTERFACE(Normalization)
+  TFCC_SUB_INTERFACE(Basic)
+  TFCC_SUB_INTERFACE(Arithmetic)
+  TFCC_SUB_INTERFACE(Transformation)
+#undef TFCC_SUB_INTERFACE
+};
+
+// the element types a device carries an Interface for
+struct InterfaceSet {
+  Interface<float> f32;
+  Interface<double> f64;
+  Interface<int8_t> s8;
+  Interface<uint8_t> u8;
+  Interface<int16_t> s16;
+  Interface<uint16_t> u16;
+  Interface<int32_t> s32;
+  Interface<uint32_t> u32;
+  Interface<int64_t> s64;
+  Interface<uint64_t> u64;
+};
+
+namespace detail {
+inline Interface<float>& pick(InterfaceSet& s, float) { return s.f32; }
+inline Interface<double>& pick(InterfaceSet& s, double) { return s.f64; }
+inline Interface<int8_t>& pick(InterfaceSet& s, int8_t) { return s.s8; }
+inline Interface<uint8_t>& pick(InterfaceSet& s, uint8_t) { return s.u8; }
+inline Interface<int16_t>& pick(InterfaceSet& s, int16_t) { return s.s16; }
+inline Interface<uint16_t>& pick(InterfaceSet& s, uint16_t) { return s.u16; }
+inline Interface<int32_t>& pick(InterfaceSet& s, int32_t) { return s.s32; }
+inline Interface<uint32_t>& pick(InterfaceSet& s, uint32_t) { return s.u32; }
+inline Interface<int64_t>& pick(InterfaceSet& s, int64_t) { return s.s64; }
+inline Interface<uint64_t>& pick(InterfaceSet& s, uint64_t) { return s.u64; }
+}  // namespace detail
+
+template <class T>
+Interface<T>& Device::getInterface(T) {
+  return detail::pick(*_interfaces, T());
+}
+
+// tfcc/core/operations/tfcc_operation.cpp:22-26
+template <class T>
+struct Operation {
+  static Interface<T>& getCurrentInterface() {
+    Device* d = Device::getThreadDefault();
+    if (d == nullptr) throw RuntimeError("no default device on this thread: call an initialize function first");
+    return d->getInterface(T());
+  }
+};
+
+// ---------------------------------------------------------------------------------------------
+// operator functions
+// ---------------------------------------------------------------------------------------------
+namespace blas {
+
+namespace detail {
+// the checks shared by both forms; returns the result shape for the empty-operand shortcut
+template <class T>
+std::vector<unsigned> check(const Tensor<T>& a, const Tensor<T>& b, const Tensor<T>* bias) {
+  const size_t ra = a.shape().size(), rb = b.shape().size();
+  if (ra < 2 || rb < 2) throw InvalidArgumentError("matmul require tensors with two or more dimensions");
+  if (ra != rb && ra != 2 && rb != 2) throw InvalidArgumentError("shape invalid");
+  if (a.shape(ra - 1) != b.shape(rb - 2)) throw InvalidArgumentError("shape invalid");
+  if (bias && (bias->shape().size() != 1 || bias->size() != b.shape(rb - 1))) throw InvalidArgumentError("shape invalid");
+  if (ra == rb) {
+    for (size_t i = 0; i + 2 < ra; ++i)
+      if (a.shape(i) != b.shape(i)) throw InvalidArgumentError("shape invalid");
+  }
+  std::vector<unsigned> s = ra > rb ? a.shape().toVector() : b.shape().toVector();
+  s[s.size() - 2] = a.shape(ra - 2);
+  s[s.size() - 1] = b.shape(rb - 1);
+  return s;
+}
+}  // namespace detail
+
+template <class T>
+Variable<T> matmul(const Tensor<T>& a, const Tensor<T>& b) {
+  std::vector<unsigned> s = detail::check<T>(a, b, nullptr);
+  if (a.size() == 0 || b.size() == 0) return Variable<T>(Shape(std::move(s)));  // nothing to compute
+  return Operation<T>::getCurrentInterface().getBlasInterface().matmul(a, b);
+}
+
+template <class T>
+Variable<T> matmul(const Tensor<T>& a, const Tensor<T>& b, const Tensor<T>& c) {
+  std::vector<unsigned> s = detail::check<T>(a, b, &c);
+  if (a.size() == 0 || b.size() == 0) return Variable<T>(Shape(std::move(s)));
+  return Operation<T>::getCurrentInterface().getBlasInterface().matmul(a, b, c);
+}
+
+}  // namespace blas
+
+namespace data {
+
+template <class T>
+void set(Variable<T>& a, const T* values) {
+  Operation<T>::getCurrentInterface().getDataInterface().set(a, values);
+}
+template <class T>
+void set(Variable<T>& a, std::vector<T> values) {
+  if (values.size() != a.size()) throw InvalidArgumentError("the length of vector and variable is unequal");
+  Operation<T>::getCurrentInterface().getDataInterface().set(a, std::move(values));
+}
+template <class T>
+Variable<T> set(std::vector<T> values, Shape shape) {
+  Variable<T> v(std::move(shape));
+  set(v, std::move(values));
+  return v;
+}
+template <class T>
+std::vector<T> get(const Tensor<T>& a) {
+  std::vector<T> out(a.size());
+  if (a.size() > 0) Operation<T>::getCurrentInterface().getDataInterface().get(a, out.data());
+  return out;
+}
+template <class T>
+void zeros(Variable<T>& a) {
+  Operation<T>::getCurrentInterface().getDataInterface().zeros(a);
+}
+template <class T>
+void ones(Variable<T>& a) {
+  Operation<T>::getCurrentInterface().getDataInterface().ones(a);
+}
+template <class T>
+Variable<T> copy(const Tensor<T>& a) {
+  return Operation<T>::getCurrentInterface().getDataInterface().copy(a);
+}
+
+}  // namespace data
+
+namespace quantization {
+
+template <class T>
+std::tuple<Variable<T>, Variable<float>, Variable<float>> quantize(const Tensor<float>& a) {
+  return Operation<T>::getCurrentInterface().getQuantizationInterface().quantize(a);
+}
+template <class T>
+Variable<T> quantize(const Tensor<float>& a, const Tensor<float>& minValue, const Tensor<float>& maxValue) {
+  return Operation<T>::getCurrentInterface().getQuantizationInterface().quantize(a, minValue, maxValue);
+}
+template <class T, class TI>
+Variable<T> requantize(const Tensor<TI>& a, const Tensor<float>& minInput, const Tensor<float>& maxInput,
+                       const Tensor<float>& minOutput, const Tensor<float>& maxOutput) {
+  return Operation<T>::getCurrentInterface().getQuantizationInterface().requantize(a, minInput, maxInput, minOutput,
+                                                                                   maxOutput);
+}
+template <class T>
+Variable<float> dequantize(const Tensor<T>& a, const Tensor<float>& minValue, const Tensor<float>& maxValue) {
+  return Operation<T>::getCurrentInterface().getQuantizationInterface().dequantize(a, minValue, maxValue);
+}
+
+}  // namespace quantization
+
+namespace math {
+
+template <class T>
+Variable<T> softmax(const Tensor<T>& a, size_t axis) {
+  if (axis >= a.shape().size()) throw InvalidArgumentError("invalid axis");
+  return Operation<T>::getCurrentInterface().getActivationInterface().softmax(a, axis);
+}
+template <class T>
+Variable<T> gelu_accurate(const Tensor<T>& a) {
+  if (a.size() == 0) throw InvalidArgumentError("invalid tensor");
+  return Operation<T>::getCurrentInterface().getActivationInterface().geluAccurate(a);
+}
+// a + b with b's shape equal to the trailing dimensions of a's (or the same shape)
+template <class T>
+Variable<T> add(const Tensor<T>& a, const Tensor<T>& b) {
+  return Operation<T>::getCurrentInterface().getArithmeticInterface().add(a, b);
+}
+template <class T>
+Variable<T> transform(const Tensor<T>& a, T alpha, T beta) {
+  return Operation<T>::getCurrentInterface().getTransformationInterface().transform(a, alpha, beta);
+}
+
+}  // namespace math
+
+namespace nn {
+
+template <class T>
+Variable<T> layer_normalization(const Tensor<T>& a, const Tensor<T>& gamma, const Tensor<T>& beta, T epsilon,
+                                size_t beginNormAxis) {
+  return Operation<T>::getCurrentInterface().getNormalizationInterface().layerNormalize(a, gamma, beta, epsilon,
+                                                                                        beginNormAxis);
+}
+
+}  // namespace nn
+
+namespace base {
+
+template <class T>
+Variable<T> transpose(const Tensor<T>& a, const std::vector<size_t>& perm) {
+  if (perm.size() != a.shape().size()) throw InvalidArgumentError("perm and tensor don't match");
+  std::set<size_t> seen(perm.begin(), perm.end());
+  if (seen.size() != perm.size() || (!perm.empty() && *seen.rbegin() >= perm.size()))
+    throw InvalidArgumentError("invalid perm");
+  return Operation<T>::getCurrentInterface().getBasicInterface().transpose(a, perm);
+}
+
+}  // namespace base
+
+// a + b, a * s, a + s  (tfcc/core/operations/tfcc_operator.cpp:34-95)
+template <class T>
+Variable<T> operator+(const Tensor<T>& a, const Tensor<T>& b) {
+  return math::add(a, b);
+}
+template <class T>
+Variable<T> operator*(const Tensor<T>& a, T s) {
+  return math::transform(a, s, static_cast<T>(0));
+}
+template <class T>
+Variable<T> operator+(const Tensor<T>& a, T s) {
+  return math::transform(a, static_cast<T>(1), s);
+}
+
+}  // namespace tfcc

@@ -1,0 +1,100 @@
+// The ROCm device for TFCC: Device / Session subclasses over the C ABI of libtfcc_rocm.so, the
+// interface implementations they install, and the backend-specific quantized matmul operations.
+//
+// Shape of a GPU backend in the reference: tfcc/cuda/framework/tfcc_cudadevice.cpp:36-109 (allocator
+// hooks, 90 % memory limit, interface installation), tfcc/cuda/framework/tfcc_cudasession.cpp:36-63
+// (stream ownership, session allocator chained to the device's with a sync before a real free),
+// tfcc/cuda/utils/tfcc_cudautils.cpp:24-60 (initialize_cuda).  The quantized matmul is not part of
+// Interface<T> in the reference either: it is a public backend header
+// (tfcc/mkl/operations/tfcc_mklquantization.h:39-51), mirrored here as tfcc::rocm::quantization.
+#pragma once
+
+#include <tuple>
+
+#include "tfcc_interfaces.h"
+
+namespace tfcc {
+
+// a failing call into libtfcc_rocm.so; what() carries the library's error text
+class ROCMRuntimeError : public Exception {
+  int _status;
+
+ public:
+  ROCMRuntimeError(int status, const std::string& text) : Exception(text), _status(status) {}
+  int status() const { return _status; }
+};
+
+class ROCMDevice : public Device {
+  unsigned _index;
+
+ public:
+  explicit ROCMDevice(unsigned index);
+  ROCMDevice(unsigned index, std::unique_ptr<Allocator> allocator);
+  ~ROCMDevice() override;
+  void attach() override;
+  unsigned index() const { return _index; }
+  static unsigned getDeviceCount();
+};
+
+class ROCMSession : public Session {
+  ROCMDevice& _device;
+  void* _stream;  // hipStream_t
+
+ public:
+  explicit ROCMSession(ROCMDevice& device);
+  ROCMSession(ROCMDevice& device, std::unique_ptr<Allocator> allocator);
+  ~ROCMSession() override;
+  void sync() const override;
+  Device& getDevice() override { return _device; }
+  const Device& getDevice() const override { return _device; }
+  void* getStream() const { return _stream; }
+};
+
+// Creates (once per process) one ROCMDevice per GPU and gives the calling thread a device and a
+// session of its own as thread defaults.
+void initialize_rocm();
+void initialize_rocm(unsigned deviceID);
+
+// Plain host memory device without any compute interface: lets the framework types (Variable, View,
+// allocators, shape checks) be exercised on machines without a GPU.
+class HostDevice : public Device {
+ public:
+  HostDevice();
+  void attach() override {}
+};
+class HostSession : public Session {
+  HostDevice& _device;
+
+ public:
+  explicit HostSession(HostDevice& device);
+  ~HostSession() override;
+  void sync() const override {}
+  Device& getDevice() override { return _device; }
+  const Device& getDevice() const override { return _device; }
+};
+
+namespace rocm {
+namespace quantization {
+
+// tfcc::mkl::quantization::matmul (tfcc/mkl/operations/tfcc_mklquantization.cpp:71-203): same
+// argument meaning, checks, error texts, batch folding and result ranges.
+std::tuple<Variable<int32_t>, Variable<float>, Variable<float>> matmul(
+    const Tensor<uint8_t>& a, const Tensor<int32_t>& reduceSumA, const Tensor<float>& minA,
+    const Tensor<float>& maxA, const Tensor<int8_t>& b, const Tensor<int32_t>& reduceSumB,
+    const Tensor<float>& minB, const Tensor<float>& maxB);
+
+// The same product with requantize<uint8_t>(c, minC, maxC, minOutput, maxOutput) fused into the
+// kernel's store; `accumulators`, when given, also receives the int32 result.
+std::tuple<Variable<uint8_t>, Variable<float>, Variable<float>> matmul_requantize(
+    const Tensor<uint8_t>& a, const Tensor<int32_t>& reduceSumA, const Tensor<float>& minA,
+    const Tensor<float>& maxA, const Tensor<int8_t>& b, const Tensor<int32_t>& reduceSumB,
+    const Tensor<float>& minB, const Tensor<float>& maxB, const Tensor<float>& minOutput,
+    const Tensor<float>& maxOutput, Variable<int32_t>* accumulators = nullptr);
+
+// tfcc::mkl::quantization::reduce_sum (tfcc_mklquantization.cpp:284-318); T = int8_t, uint8_t, int16_t
+template <class T>
+Variable<int32_t> reduce_sum(const Tensor<T>& a, bool row);
+
+}  // namespace quantization
+}  // namespace rocm
+}  // namespace tfcc
