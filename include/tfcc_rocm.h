@@ -59,6 +59,18 @@ int tfcc_rocm_free(void* ptr);
 int tfcc_rocm_stream_create(void** stream);
 int tfcc_rocm_stream_destroy(void* stream);
 int tfcc_rocm_stream_synchronize(void* stream);
+/* events on a stream, for timing (cf. tfcc::Coster around Session::sync, tfcc_runtime/framework/model.cpp:191-226) */
+int tfcc_rocm_event_create(void** event);
+int tfcc_rocm_event_destroy(void* event);
+int tfcc_rocm_event_record(void* event, void* stream);
+int tfcc_rocm_event_elapsed_ms(void* start_event, void* stop_event, float* ms); /* waits for stop_event */
+/* Recording of everything issued on `stream` between begin and end into an executable graph that
+ * one launch replays.  Stands where the reference assembles a graph's call sequence once and then
+ * calls it per run (tfcc_runtime/framework/graph.cpp:54-59,98-123). */
+int tfcc_rocm_stream_begin_capture(void* stream);
+int tfcc_rocm_stream_end_capture(void* stream, void** graph_exec);
+int tfcc_rocm_graph_launch(void* graph_exec, void* stream);
+int tfcc_rocm_graph_destroy(void* graph_exec);
 /* host<->device copies: synchronise the stream, then copy synchronously (reference semantics) */
 int tfcc_rocm_memcpy_h2d(void* stream, void* dst_device, const void* src_host, size_t bytes);
 int tfcc_rocm_memcpy_d2h(void* stream, void* dst_host, const void* src_device, size_t bytes);
@@ -183,6 +195,13 @@ int tfcc_rocm_transform_f32(void* stream, const float* in, uint64_t total, float
  * broadcast of b).  ArithmeticInterface::add, tfcc/core/interfaces/tfcc_arithmeticinterface.h:34-49 */
 int tfcc_rocm_add_f32(void* stream, const float* a, const float* b, uint64_t total,
                       uint64_t period, float* out);
+/* out = a / alpha + beta: TransformationInterface::transform2 (a / s in tfcc_operator.cpp:78-95) */
+int tfcc_rocm_transform2_f32(void* stream, const float* in, uint64_t total, float alpha, float beta,
+                             float* out);
+/* op: 0 a + b, 1 a - b, 2 a * b, 3 a / b with the same trailing-dims broadcast of b as add:
+ * ArithmeticInterface::add/sub/mul/div, tfcc/core/interfaces/tfcc_arithmeticinterface.h:34-79 */
+int tfcc_rocm_binary_f32(void* stream, int op, const float* a, const float* b, uint64_t total,
+                         uint64_t period, float* out);
 /* rank <= 6 permutation: BasicInterface::transpose, tfcc/core/operations/tfcc_base.cpp:124-134.
  * shape / perm are HOST arrays of length rank. */
 int tfcc_rocm_transpose_f32(void* stream, const float* in, const unsigned* shape,

@@ -1,0 +1,244 @@
+"""The model runtime: archive and message handling, graph building and the operation accept /
+reject rules on the host-memory device (no GPU), and on the GPU one transformer encoder layer
+through the runtime against the CPU oracle, with and without graph replay."""
+import importlib
+import io
+import os
+import re
+import zipfile
+
+import numpy as np
+import pytest
+
+import bert_reference
+import oracle_lib as O
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def mf(pkg):
+    return importlib.import_module("wechat_tfcc_amd.modelfile")
+
+
+@pytest.fixture(scope="module")
+def rt(pkg):
+    return importlib.import_module("wechat_tfcc_amd.runtime_api")
+
+
+def rel_frobenius(got, want):
+    return float(np.linalg.norm(got.astype(np.float64) - want.astype(np.float64)) /
+                 np.linalg.norm(want.astype(np.float64)))
+
+
+def passthrough_graph(mf, dtype, shape, dims):
+    g = mf.GraphBuilder("g")
+    x = g.input("x", dtype, shape)
+    r = g.reshape(x, dims)
+    out = g._symbol("y", dtype, mf.VARIABLE)
+    g.node("base.Identity", [r], [out])
+    g.output(out)
+    return g
+
+
+# ---- no GPU: header, loading, building, host-side steps ----------------------------------------------
+def test_runtime_header_and_binding_agree(rt):
+    text = open(os.path.join(ROOT, "include", "tfcc_rocm_runtime.h")).read()
+    declared = sorted(set(re.findall(r"\b(tfcc_rocm_runtime_\w+)\s*\(", text)))
+    assert declared == sorted(rt.SYMBOLS)
+    rt.lib()  # resolves every symbol
+
+
+def test_reshape_identity_on_host(mf, rt):
+    rng = np.random.default_rng(1)
+    a = rng.normal(size=(2, 3, 4)).astype(np.float32)
+    for dims, want in (([0, -1], (2, 12)), ([-1], (24,)), ([4, 0, 2], (4, 3, 2)), ([0, 0, 2, 2], (2, 3, 2, 2))):
+        m = rt.Model(mf.write_model([passthrough_graph(mf, mf.FLOAT, [2, 3, 4], dims)], "g"), host=True)
+        out = m.run({"x": a})["y"]
+        assert out.shape == want and np.array_equal(out.ravel(), a.ravel())
+        m.close()
+    m = rt.Model(mf.write_model([passthrough_graph(mf, mf.FLOAT, [2, 3, 4], [-1, -1])], "g"), host=True)
+    with pytest.raises(rt.RuntimeError_, match="Reshape: invalid shape"):
+        m.run({"x": a})
+    with pytest.raises(rt.RuntimeError_, match="Invalid data size"):
+        m.run_serialized(mf.f_bytes(1, mf.f_bytes(1, "x") + mf.f_varint(2, mf.FLOAT) + mf.f_packed(3, [2, 3, 4]) +
+                                    mf.f_bytes(4, b"\0" * 8)))
+
+
+@pytest.mark.parametrize("compress", [False, True])
+def test_constants_from_npz(mf, rt, compress):
+    """element conversion, Fortran order, 0-d arrays, stored and deflated members"""
+    rng = np.random.default_rng(2)
+    g = mf.GraphBuilder("main")
+    c_f64 = rng.normal(size=(3, 5))                        # f8 on disk, read as FLOAT
+    c_fortran = np.asfortranarray(rng.normal(size=(4, 3, 2)).astype(np.float32))
+    c_scalar = np.array(7, dtype=np.int64)                 # 0-d -> shape [1]
+    g.constants["main/w64"] = c_f64
+    g._symbol("w64", mf.FLOAT, mf.CONSTANT_TENSOR, [3, 5], "w64")
+    g.constants["main/wf"] = c_fortran
+    g._symbol("wf", mf.FLOAT, mf.CONSTANT_TENSOR, [4, 3, 2], "wf")
+    g.constants["main/s"] = c_scalar
+    g._symbol("s", mf.INT32, mf.CONSTANT_TENSOR, [1], "s")
+    for src, dst, dt in (("w64", "o64", mf.FLOAT), ("wf", "of", mf.FLOAT), ("s", "os", mf.INT32)):
+        g._symbol(dst, dt, mf.VARIABLE)
+        g.node("base.Identity", [src], [dst])
+        g.output(dst)
+    m = rt.Model(mf.write_model([g], "main", compress=compress), host=True)
+    out = m.run({})
+    assert np.array_equal(out["o64"], c_f64.astype(np.float32))
+    assert np.array_equal(out["of"], np.ascontiguousarray(c_fortran))
+    assert out["os"].dtype == np.int32 and out["os"].tolist() == [7]
+
+
+def test_value_arithmetic_and_vectors_on_host(mf, rt):
+    g = mf.GraphBuilder("g")
+    a = g.value_input("a", mf.FLOAT)
+    b = g.value_input("b", mf.FLOAT)
+    results = {}
+    for op in ("Add", "Sub", "Mul", "Div"):
+        out = g._symbol("r_" + op, mf.FLOAT, mf.VALUE)
+        g.node("math." + op, [a, b], [out])
+        g.output(out)
+    m = rt.Model(mf.write_model([g], "g"), host=True)
+    res = m.run({"a": np.array([6.0], np.float32), "b": np.array([1.5], np.float32)})
+    assert [float(res["r_" + op][0]) for op in ("Add", "Sub", "Mul", "Div")] == [7.5, 4.5, 9.0, 4.0]
+
+
+def test_archive_and_graph_errors(mf, rt):
+    g = passthrough_graph(mf, mf.FLOAT, [2], [0])
+    blob = mf.write_model([g], "g")
+    # a member missing
+    out = io.BytesIO()
+    with zipfile.ZipFile(io.BytesIO(blob)) as zin, zipfile.ZipFile(out, "w") as zout:
+        zout.writestr("model.pb", zin.read("model.pb"))
+    with pytest.raises(rt.RuntimeError_, match="Invalid model data"):
+        rt.Model(out.getvalue(), host=True)
+    with pytest.raises(rt.RuntimeError_, match="invalid zip format"):
+        rt.Model(b"not a zip archive at all.........", host=True)
+    # the entrance graph is not among the graphs
+    with pytest.raises(rt.RuntimeError_, match="Invalid model proto"):
+        rt.Model(mf.write_model([g], "other"), host=True).run({})
+    # a node nobody accepts: unknown message, wrong version, wrong input count
+    for op, inputs, version in (("math.NoSuchOp", ["x"], 1), ("math.Gelu", ["x"], 2), ("math.Matmul", ["x"], 1)):
+        bad = mf.GraphBuilder("g")
+        x = bad.input("x", mf.FLOAT, [2])
+        y = bad.variable("y")
+        bad.node(op, inputs, [y], version=version, name="the_node")
+        bad.output(y)
+        with pytest.raises(rt.RuntimeError_) as e:
+            rt.Model(mf.write_model([bad], "g"), host=True).run({"x": np.zeros(2, np.float32)})
+        assert str(e.value) == ("Unknow node: the_node operation: type.googleapis.com/tfcc.runtime.operations.%s "
+                                "version: %d" % (op, version))
+    # duplicate symbol
+    dup = mf.GraphBuilder("g")
+    dup.input("x", mf.FLOAT, [2])
+    dup._symbol("x", mf.FLOAT, mf.VARIABLE)
+    with pytest.raises(rt.RuntimeError_, match="name x has existed"):
+        rt.Model(mf.write_model([dup], "g"), host=True).run({})
+
+
+def test_compute_is_not_implemented_on_the_host_device(mf, rt):
+    rng = np.random.default_rng(3)
+    w = mf.bert_layer_weights(rng, 32, 64)
+    g = mf.bert_encoder_layer(w, 2, 4, 4)
+    m = rt.Model(mf.write_model([g], g.name), host=True)  # loads and builds
+    with pytest.raises(rt.RuntimeError_, match="not implemented"):
+        m.run({"hidden_states": np.zeros((2, 4, 32), np.float32)})
+
+
+def test_oracle_encoder_layer_against_numpy_float64(mf):
+    """pins the oracle composition itself: same layer in straight numpy float64"""
+    from scipy.special import erf
+    rng = np.random.default_rng(4)
+    batch, seq, hidden, heads, ffn = 2, 16, 64, 4, 128
+    w = mf.bert_layer_weights(rng, hidden, ffn)
+    x = rng.normal(size=(batch, seq, hidden)).astype(np.float32)
+    got = bert_reference.encoder_layer(x, w, heads)
+
+    W = {k: v.astype(np.float64) for k, v in w.items()}
+    X = x.astype(np.float64)
+
+    def ln(t, gamma, beta):
+        mu = t.mean(-1, keepdims=True)
+        var = ((t - mu) ** 2).mean(-1, keepdims=True)
+        return (t - mu) / np.sqrt(var + 1e-12) * gamma + beta
+
+    def split(t):
+        return t.reshape(batch, seq, heads, hidden // heads).transpose(0, 2, 1, 3)
+
+    q, k, v = (split(X @ W["w" + n] + W["b" + n]) for n in "qkv")
+    s = q @ k.transpose(0, 1, 3, 2) / np.sqrt(hidden // heads)
+    p = np.exp(s - s.max(-1, keepdims=True))
+    p /= p.sum(-1, keepdims=True)
+    ctx = (p @ v).transpose(0, 2, 1, 3).reshape(batch, seq, hidden)
+    att = ln(ctx @ W["wo"] + W["bo"] + X, W["ln1_gamma"], W["ln1_beta"])
+    h = att @ W["w1"] + W["b1"]
+    h = 0.5 * h * (1 + erf(h / np.sqrt(2)))
+    want = ln(h @ W["w2"] + W["b2"] + att, W["ln2_gamma"], W["ln2_beta"])
+    assert rel_frobenius(got, want) < 2e-6
+
+
+# ---- GPU ----------------------------------------------------------------------------------------------
+@pytest.mark.gpu
+@pytest.mark.parametrize("batch,seq,hidden,heads,ffn", [(2, 16, 64, 4, 128), (3, 7, 96, 3, 200), (8, 128, 768, 12, 3072)])
+def test_encoder_layer_matches_oracle(mf, rt, dev, batch, seq, hidden, heads, ffn):
+    """fp32 tolerance: relative Frobenius error <= 1e-5 against the double-accumulating oracle"""
+    rng = np.random.default_rng(5)
+    w = mf.bert_layer_weights(rng, hidden, ffn)
+    g = mf.bert_encoder_layer(w, batch, seq, heads)
+    m = rt.Model(mf.write_model([g], g.name))
+    x = rng.normal(size=(batch, seq, hidden)).astype(np.float32)
+    got = m.run({"hidden_states": x})["layer_output"]
+    want = bert_reference.encoder_layer(x, w, heads)
+    assert got.shape == want.shape
+    assert rel_frobenius(got, want) <= 1e-5
+    # Model::test on an .npz holding inputs and expected outputs
+    npz = io.BytesIO()
+    np.savez(npz, hidden_states=x, layer_output=want)
+    passed, report = m.test(npz.getvalue())
+    assert passed, report
+    npz = io.BytesIO()
+    np.savez(npz, hidden_states=x, layer_output=want + 1)
+    passed, report = m.test(npz.getvalue())
+    assert not passed and "DIFFERENT" in report
+    m.close()
+
+
+@pytest.mark.gpu
+def test_replay_reproduces_step_by_step_results(mf, rt, dev):
+    """every replay is checked against the step-by-step result of the same input, with ordinary
+    runs and synchronisations of the process in between"""
+    rng = np.random.default_rng(6)
+    batch, seq, hidden, heads, ffn = 4, 32, 128, 4, 256
+    w = mf.bert_layer_weights(rng, hidden, ffn)
+    g = mf.bert_encoder_layer(w, batch, seq, heads)
+    blob = mf.write_model([g], g.name)
+    eager, replay = rt.Model(blob), rt.Model(blob)
+    replay.set_replay(True)
+    for i in range(6):
+        x = rng.normal(size=(batch, seq, hidden)).astype(np.float32)
+        want = eager.run({"hidden_states": x})["layer_output"]
+        got = replay.run({"hidden_states": x})["layer_output"]
+        assert np.array_equal(got, want), "run %d" % i
+    # a new input shape drops the recording and records again
+    x = rng.normal(size=(batch, seq, hidden)).astype(np.float32)
+    assert np.array_equal(replay.run({"hidden_states": x})["layer_output"], eager.run({"hidden_states": x})["layer_output"])
+    replay.set_replay(False)
+    assert np.array_equal(replay.run({"hidden_states": x})["layer_output"], eager.run({"hidden_states": x})["layer_output"])
+    us = replay.time({"hidden_states": x}, warmup=2, iters=5)
+    assert us > 0
+
+
+@pytest.mark.gpu
+def test_matmul_nodes_of_other_dtypes_fail_at_run_time(mf, rt, dev):
+    """accepted when the graph is built, NotImplementedError when run - as on the reference's
+    backends, where only float has a blas implementation"""
+    g = mf.GraphBuilder("g")
+    a = g.input("a", mf.INT32, [2, 3])
+    b = g.input("b", mf.INT32, [3, 2])
+    y = g.variable("y", mf.INT32)
+    g.node("math.Matmul", [a, b], [y])
+    g.output(y)
+    m = rt.Model(mf.write_model([g], "g"))
+    with pytest.raises(rt.RuntimeError_, match="not implemented"):
+        m.run({"a": np.ones((2, 3), np.int32), "b": np.ones((3, 2), np.int32)})

@@ -72,6 +72,16 @@ SYMBOLS = {
     "tfcc_rocm_gelu_accurate_f32": (_I, [_VP, _VP, _U64, _VP]),
     "tfcc_rocm_transform_f32": (_I, [_VP, _VP, _U64, _F, _F, _VP]),
     "tfcc_rocm_add_f32": (_I, [_VP, _VP, _VP, _U64, _U64, _VP]),
+    "tfcc_rocm_event_create": (_I, [C.POINTER(_VP)]),
+    "tfcc_rocm_event_destroy": (_I, [_VP]),
+    "tfcc_rocm_event_record": (_I, [_VP, _VP]),
+    "tfcc_rocm_event_elapsed_ms": (_I, [_VP, _VP, C.POINTER(C.c_float)]),
+    "tfcc_rocm_stream_begin_capture": (_I, [_VP]),
+    "tfcc_rocm_stream_end_capture": (_I, [_VP, C.POINTER(_VP)]),
+    "tfcc_rocm_graph_launch": (_I, [_VP, _VP]),
+    "tfcc_rocm_graph_destroy": (_I, [_VP]),
+    "tfcc_rocm_transform2_f32": (_I, [_VP, _VP, _U64, _F, _F, _VP]),
+    "tfcc_rocm_binary_f32": (_I, [_VP, _I, _VP, _VP, _U64, _U64, _VP]),
     "tfcc_rocm_transpose_f32": (_I, [_VP, _VP, C.POINTER(C.c_uint), C.POINTER(C.c_uint), _I, _VP]),
 }
 
@@ -369,6 +379,27 @@ def add(a, b):
     a, b = a.contiguous(), b.contiguous()
     out = torch.empty_like(a)
     check(lib().tfcc_rocm_add_f32(_stream(), _ptr(a), _ptr(b), a.numel(), b.numel(), _ptr(out)))
+    return out
+
+
+def transform2(a, alpha, beta):
+    """a / alpha + beta"""
+    import torch
+    a = a.contiguous()
+    out = torch.empty_like(a)
+    check(lib().tfcc_rocm_transform2_f32(_stream(), _ptr(a), a.numel(), alpha, beta, _ptr(out)))
+    return out
+
+
+BINARY_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3}
+
+
+def binary(op, a, b):
+    """a (op) b where b's shape equals the trailing dims of a's; op in BINARY_OPS."""
+    import torch
+    a, b = a.contiguous(), b.contiguous()
+    out = torch.empty_like(a)
+    check(lib().tfcc_rocm_binary_f32(_stream(), BINARY_OPS[op], _ptr(a), _ptr(b), a.numel(), b.numel(), _ptr(out)))
     return out
 
 

@@ -106,6 +106,65 @@ int tfcc_rocm_stream_synchronize(void* stream) {
   return TFCC_ROCM_OK;
 }
 
+int tfcc_rocm_event_create(void** event) {
+  TFCC_REQUIRE(event != nullptr, "event_create: null argument");
+  hipEvent_t e;
+  TFCC_HIP_CHECK(hipEventCreate(&e));
+  *event = e;
+  return TFCC_ROCM_OK;
+}
+
+int tfcc_rocm_event_destroy(void* event) {
+  TFCC_HIP_CHECK(hipEventDestroy(static_cast<hipEvent_t>(event)));
+  return TFCC_ROCM_OK;
+}
+
+int tfcc_rocm_event_record(void* event, void* stream) {
+  TFCC_REQUIRE(event != nullptr, "event_record: null argument");
+  TFCC_HIP_CHECK(hipEventRecord(static_cast<hipEvent_t>(event), as_stream(stream)));
+  return TFCC_ROCM_OK;
+}
+
+int tfcc_rocm_event_elapsed_ms(void* start, void* stop, float* ms) {
+  TFCC_REQUIRE(start && stop && ms, "event_elapsed_ms: null argument");
+  TFCC_HIP_CHECK(hipEventSynchronize(static_cast<hipEvent_t>(stop)));
+  TFCC_HIP_CHECK(hipEventElapsedTime(ms, static_cast<hipEvent_t>(start), static_cast<hipEvent_t>(stop)));
+  return TFCC_ROCM_OK;
+}
+
+int tfcc_rocm_stream_begin_capture(void* stream) {
+  TFCC_REQUIRE(stream != nullptr, "begin_capture: the default stream cannot be captured");
+  // relaxed: a cache miss in the caller's allocator may still reach hipMalloc while recording
+  TFCC_HIP_CHECK(hipStreamBeginCapture(as_stream(stream), hipStreamCaptureModeRelaxed));
+  return TFCC_ROCM_OK;
+}
+
+int tfcc_rocm_stream_end_capture(void* stream, void** graph_exec) {
+  TFCC_REQUIRE(stream && graph_exec, "end_capture: null argument");
+  *graph_exec = nullptr;
+  hipGraph_t graph = nullptr;
+  TFCC_HIP_CHECK(hipStreamEndCapture(as_stream(stream), &graph));
+  TFCC_REQUIRE(graph != nullptr, "end_capture: the capture was invalidated");
+  hipGraphExec_t exec = nullptr;
+  hipError_t e = hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0);
+  (void)hipGraphDestroy(graph);
+  TFCC_HIP_CHECK(e);
+  *graph_exec = exec;
+  return TFCC_ROCM_OK;
+}
+
+int tfcc_rocm_graph_launch(void* graph_exec, void* stream) {
+  TFCC_REQUIRE(graph_exec != nullptr, "graph_launch: null argument");
+  TFCC_HIP_CHECK(hipGraphLaunch(static_cast<hipGraphExec_t>(graph_exec), as_stream(stream)));
+  return TFCC_ROCM_OK;
+}
+
+int tfcc_rocm_graph_destroy(void* graph_exec) {
+  if (graph_exec == nullptr) return TFCC_ROCM_OK;
+  TFCC_HIP_CHECK(hipGraphExecDestroy(static_cast<hipGraphExec_t>(graph_exec)));
+  return TFCC_ROCM_OK;
+}
+
 int tfcc_rocm_memcpy_h2d(void* stream, void* dst_device, const void* src_host, size_t bytes) {
   if (bytes == 0) return TFCC_ROCM_OK;
   TFCC_REQUIRE(dst_device && src_host, "memcpy_h2d: null argument");

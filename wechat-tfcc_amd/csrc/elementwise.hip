@@ -122,11 +122,23 @@ __global__ __launch_bounds__(256) void transform_kernel(const float* in, size_t 
   for (; i < total; i += step) out[i] = in[i] * alpha + beta;
 }
 
-__global__ __launch_bounds__(256) void add_kernel(const float* a, const float* b, size_t total, size_t period,
-                                                  float* out) {
+__global__ __launch_bounds__(256) void transform2_kernel(const float* in, size_t total, float alpha, float beta,
+                                                         float* out) {
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   const size_t step = (size_t)gridDim.x * blockDim.x;
-  for (; i < total; i += step) out[i] = a[i] + b[period == total ? i : i % period];
+  for (; i < total; i += step) out[i] = in[i] / alpha + beta;
+}
+
+// OP: 0 a + b, 1 a - b, 2 a * b, 3 a / b; b repeats with `period`
+template <int OP>
+__global__ __launch_bounds__(256) void binary_kernel(const float* a, const float* b, size_t total, size_t period,
+                                                     float* out) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t step = (size_t)gridDim.x * blockDim.x;
+  for (; i < total; i += step) {
+    const float x = a[i], y = b[period == total ? i : i % period];
+    out[i] = OP == 0 ? x + y : OP == 1 ? x - y : OP == 2 ? x * y : x / y;
+  }
 }
 
 struct TransposeParams {
@@ -215,12 +227,32 @@ int tfcc_rocm_transform_f32(void* stream, const float* in, uint64_t total, float
   return check_launch("transform");
 }
 
+int tfcc_rocm_transform2_f32(void* stream, const float* in, uint64_t total, float alpha, float beta, float* out) {
+  TFCC_REQUIRE(in && out, "transform2: null argument");
+  TFCC_REQUIRE(total > 0, "transform2: empty tensor");
+  hipLaunchKernelGGL(transform2_kernel, dim3(grid_for(total)), dim3(256), 0, as_stream(stream), in, (size_t)total,
+                     alpha, beta, out);
+  return check_launch("transform2");
+}
+
+int tfcc_rocm_binary_f32(void* stream, int op, const float* a, const float* b, uint64_t total, uint64_t period,
+                         float* out) {
+  TFCC_REQUIRE(a && b && out, "binary: null argument");
+  TFCC_REQUIRE(op >= 0 && op <= 3, "binary: unknown op %d", op);
+  TFCC_REQUIRE(total > 0 && period > 0 && period <= total && total % period == 0, "binary: bad broadcast period");
+  const dim3 grid(grid_for(total)), block(256);
+  hipStream_t s = as_stream(stream);
+  switch (op) {
+    case 0: hipLaunchKernelGGL(binary_kernel<0>, grid, block, 0, s, a, b, (size_t)total, (size_t)period, out); break;
+    case 1: hipLaunchKernelGGL(binary_kernel<1>, grid, block, 0, s, a, b, (size_t)total, (size_t)period, out); break;
+    case 2: hipLaunchKernelGGL(binary_kernel<2>, grid, block, 0, s, a, b, (size_t)total, (size_t)period, out); break;
+    default: hipLaunchKernelGGL(binary_kernel<3>, grid, block, 0, s, a, b, (size_t)total, (size_t)period, out); break;
+  }
+  return check_launch("binary");
+}
+
 int tfcc_rocm_add_f32(void* stream, const float* a, const float* b, uint64_t total, uint64_t period, float* out) {
-  TFCC_REQUIRE(a && b && out, "add: null argument");
-  TFCC_REQUIRE(total > 0 && period > 0 && period <= total && total % period == 0, "add: bad broadcast period");
-  hipLaunchKernelGGL(add_kernel, dim3(grid_for(total)), dim3(256), 0, as_stream(stream), a, b, (size_t)total,
-                     (size_t)period, out);
-  return check_launch("add");
+  return tfcc_rocm_binary_f32(stream, 0, a, b, total, period, out);
 }
 
 int tfcc_rocm_transpose_f32(void* stream, const float* in, const unsigned* shape, const unsigned* perm,

@@ -108,6 +108,15 @@ class Allocator {
   virtual void setLimit(size_t limit) = 0;
   virtual size_t used() const = 0;
 
+  // Pinning keeps every block that is freed between beginPinning() and endPinning() out of the
+  // general cache: such a block may be handed out again only while pinning is still on.
+  // endPinning() returns the blocks left over; they stay reserved until given to unpin().  A
+  // recorded kernel sequence that is replayed later relies on this: no other user of the
+  // allocator can be given memory the recording writes to.
+  virtual void beginPinning() {}
+  virtual std::vector<void*> endPinning() { return {}; }
+  virtual void unpin(const std::vector<void*>&) {}
+
   void setRealMalloc(std::function<void*(size_t)> f) { _realMalloc = std::move(f); }
   void setRealFree(std::function<void(void*)> f) { _realFree = std::move(f); }
 };
@@ -123,6 +132,9 @@ class FlexAllocator : public Allocator {
   mutable std::mutex _mtx;
   std::atomic<size_t> _used{0};          // bytes obtained from the real allocator
   size_t _limit = 0, _flexLimit = 0;
+  bool _pinning = false;
+  std::multimap<size_t, void*> _pinnedFree;  // freed while pinning: reusable only while pinning
+  std::map<void*, size_t> _reserved;         // handed to the caller of endPinning()
 
   static size_t bucket(size_t len);
   void releaseDownTo(size_t target);
@@ -137,6 +149,9 @@ class FlexAllocator : public Allocator {
   void setLimit(size_t limit) override { _limit = limit; }
   size_t used() const override { return _used.load(); }
   void setFlexLimit(size_t flexLimit) { _flexLimit = flexLimit; }
+  void beginPinning() override;
+  std::vector<void*> endPinning() override;
+  void unpin(const std::vector<void*>& blocks) override;
 };
 
 // Pass-through allocator (tfcc/core/allocators/tfcc_simpleallocator.*)

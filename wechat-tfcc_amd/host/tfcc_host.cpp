@@ -86,6 +86,13 @@ void* FlexAllocator::malloc(size_t len) {
   void* p = nullptr;
   {
     std::lock_guard<std::mutex> lk(_mtx);
+    auto pinned = _pinning ? _pinnedFree.find(size) : _pinnedFree.end();
+    if (pinned != _pinnedFree.end()) {
+      p = pinned->second;
+      _pinnedFree.erase(pinned);
+      _live[p] = size;
+      return p;
+    }
     auto it = _cached.find(size);
     if (it != _cached.end()) {
       p = it->second;
@@ -115,8 +122,35 @@ void FlexAllocator::free(void* p) {
   std::lock_guard<std::mutex> lk(_mtx);
   auto it = _live.find(p);
   if (it == _live.end()) return;
-  _cached.emplace(it->second, p);
+  (_pinning ? _pinnedFree : _cached).emplace(it->second, p);
   _live.erase(it);
+}
+
+void FlexAllocator::beginPinning() {
+  std::lock_guard<std::mutex> lk(_mtx);
+  _pinning = true;
+}
+
+std::vector<void*> FlexAllocator::endPinning() {
+  std::lock_guard<std::mutex> lk(_mtx);
+  _pinning = false;
+  std::vector<void*> blocks;
+  for (auto& kv : _pinnedFree) {
+    _reserved[kv.second] = kv.first;
+    blocks.push_back(kv.second);
+  }
+  _pinnedFree.clear();
+  return blocks;
+}
+
+void FlexAllocator::unpin(const std::vector<void*>& blocks) {
+  std::lock_guard<std::mutex> lk(_mtx);
+  for (void* p : blocks) {
+    auto it = _reserved.find(p);
+    if (it == _reserved.end()) continue;
+    _cached.emplace(it->second, p);
+    _reserved.erase(it);
+  }
 }
 
 void FlexAllocator::releaseDownTo(size_t target) {
@@ -162,9 +196,50 @@ void SimpleAllocator::free(void* p) {
 // ---------------------------------------------------------------------------------------------
 // host device
 // ---------------------------------------------------------------------------------------------
+namespace {
+// plain memory moves: the only interface the host device offers
+template <class T>
+class HostDataInterface : public DataInterface<T> {
+ public:
+  void set(T* dst, const T* data, size_t len) override { std::memcpy(dst, data, len * sizeof(T)); }
+  void set(Variable<T>& a, const T* data) override { set(a.data(), data, a.size()); }
+  void set(Variable<T>& a, std::vector<T>&& data) override { set(a.data(), data.data(), a.size()); }
+  void get(const Tensor<T>& a, T* data) override { std::memcpy(data, a.data(), static_cast<size_t>(a.size()) * sizeof(T)); }
+  void zeros(Variable<T>& a) override { std::fill(a.data(), a.data() + a.size(), static_cast<T>(0)); }
+  void ones(Variable<T>& a) override { std::fill(a.data(), a.data() + a.size(), static_cast<T>(1)); }
+  Variable<T> copy(const Tensor<T>& a) override {
+    Variable<T> r(a.shape());
+    std::memcpy(r.data(), a.data(), static_cast<size_t>(a.size()) * sizeof(T));
+    return r;
+  }
+};
+template <class T>
+void install_host(Interface<T>& i) {
+  i.setDataInterface(std::unique_ptr<DataInterface<T>>(new HostDataInterface<T>()));
+}
+}  // namespace
+
 HostDevice::HostDevice() : Device(DeviceType::HOST, 0, std::unique_ptr<Allocator>(new FlexAllocator())) {
   _allocator->setRealMalloc([](size_t len) -> void* { return std::aligned_alloc(64, (len + 63) / 64 * 64); });
   _allocator->setRealFree([](void* p) { std::free(p); });
+  install_host(_interfaces->f32);
+  install_host(_interfaces->f64);
+  install_host(_interfaces->s8);
+  install_host(_interfaces->u8);
+  install_host(_interfaces->s16);
+  install_host(_interfaces->u16);
+  install_host(_interfaces->s32);
+  install_host(_interfaces->u32);
+  install_host(_interfaces->s64);
+  install_host(_interfaces->u64);
+}
+
+void initialize_host() {
+  static HostDevice device;
+  thread_local std::unique_ptr<HostSession> session;
+  if (!session) session.reset(new HostSession(device));
+  Device::setThreadDefault(&device);
+  Session::setThreadDefault(session.get());
 }
 
 HostSession::HostSession(HostDevice& device) : Session(std::unique_ptr<Allocator>(new FlexAllocator())), _device(device) {
@@ -368,17 +443,31 @@ class ROCMBasicInterface : public BasicInterface<float> {
 };
 
 class ROCMArithmeticInterface : public ArithmeticInterface<float> {
- public:
-  Variable<float> add(const Tensor<float>& a, const Tensor<float>& b) override {
-    // b equals the trailing dimensions of a (bias / residual forms)
-    const size_t ra = a.shape().size(), rb = b.shape().size();
+  // b equals the trailing dimensions of a once leading 1s are dropped (bias / residual forms)
+  static bool trailing(const Tensor<float>& a, const Tensor<float>& b) {
+    const size_t ra = a.shape().size();
+    size_t skip = 0;
+    while (skip + 1 < b.shape().size() && b.shape(skip) == 1) ++skip;
+    const size_t rb = b.shape().size() - skip;
     bool ok = rb <= ra && a.size() > 0 && b.size() > 0;
-    for (size_t i = 0; ok && i < rb; ++i) ok = a.shape(ra - rb + i) == b.shape(i);
-    if (!ok) throw NotImplementedError("add: only a trailing-dimension broadcast of the second operand");
+    for (size_t i = 0; ok && i < rb; ++i) ok = a.shape(ra - rb + i) == b.shape(skip + i);
+    return ok;
+  }
+  static Variable<float> run(int op, const Tensor<float>& a, const Tensor<float>& b) {
+    if (!trailing(a, b)) {
+      if ((op == 0 || op == 2) && trailing(b, a)) return run(op, b, a);  // commutative: swap
+      throw NotImplementedError("element-wise operation: only a trailing-dimension broadcast of one operand");
+    }
     Variable<float> r(a.shape());
-    check(tfcc_rocm_add_f32(current_stream(), a.data(), b.data(), a.size(), b.size(), r.data()));
+    check(tfcc_rocm_binary_f32(current_stream(), op, a.data(), b.data(), a.size(), b.size(), r.data()));
     return r;
   }
+
+ public:
+  Variable<float> add(const Tensor<float>& a, const Tensor<float>& b) override { return run(0, a, b); }
+  Variable<float> sub(const Tensor<float>& a, const Tensor<float>& b) override { return run(1, a, b); }
+  Variable<float> mul(const Tensor<float>& a, const Tensor<float>& b) override { return run(2, a, b); }
+  Variable<float> div(const Tensor<float>& a, const Tensor<float>& b) override { return run(3, a, b); }
 };
 
 class ROCMTransformationInterface : public TransformationInterface<float> {
@@ -387,6 +476,12 @@ class ROCMTransformationInterface : public TransformationInterface<float> {
     if (a.size() == 0) throw InvalidArgumentError("invalid tensor");
     Variable<float> r(a.shape());
     check(tfcc_rocm_transform_f32(current_stream(), a.data(), a.size(), alpha, beta, r.data()));
+    return r;
+  }
+  Variable<float> transform2(const Tensor<float>& a, float alpha, float beta) override {
+    if (a.size() == 0) throw InvalidArgumentError("invalid tensor");
+    Variable<float> r(a.shape());
+    check(tfcc_rocm_transform2_f32(current_stream(), a.data(), a.size(), alpha, beta, r.data()));
     return r;
   }
 };

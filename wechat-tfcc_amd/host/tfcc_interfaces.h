@@ -104,13 +104,17 @@ class ArithmeticInterface {
  public:
   virtual ~ArithmeticInterface() {}
   virtual Variable<T> add(const Tensor<T>&, const Tensor<T>&) { throw NotImplementedError(); }
+  virtual Variable<T> sub(const Tensor<T>&, const Tensor<T>&) { throw NotImplementedError(); }
+  virtual Variable<T> mul(const Tensor<T>&, const Tensor<T>&) { throw NotImplementedError(); }
+  virtual Variable<T> div(const Tensor<T>&, const Tensor<T>&) { throw NotImplementedError(); }
 };
 
 template <class T>
 class TransformationInterface {
  public:
   virtual ~TransformationInterface() {}
-  virtual Variable<T> transform(const Tensor<T>&, T, T) { throw NotImplementedError(); }  // a * alpha + beta
+  virtual Variable<T> transform(const Tensor<T>&, T, T) { throw NotImplementedError(); }   // a * alpha + beta
+  virtual Variable<T> transform2(const Tensor<T>&, T, T) { throw NotImplementedError(); }  // a / alpha + beta
 };
 
 template <class T>
@@ -295,8 +299,24 @@ Variable<T> add(const Tensor<T>& a, const Tensor<T>& b) {
   return Operation<T>::getCurrentInterface().getArithmeticInterface().add(a, b);
 }
 template <class T>
+Variable<T> sub(const Tensor<T>& a, const Tensor<T>& b) {
+  return Operation<T>::getCurrentInterface().getArithmeticInterface().sub(a, b);
+}
+template <class T>
+Variable<T> mul(const Tensor<T>& a, const Tensor<T>& b) {
+  return Operation<T>::getCurrentInterface().getArithmeticInterface().mul(a, b);
+}
+template <class T>
+Variable<T> div(const Tensor<T>& a, const Tensor<T>& b) {
+  return Operation<T>::getCurrentInterface().getArithmeticInterface().div(a, b);
+}
+template <class T>
 Variable<T> transform(const Tensor<T>& a, T alpha, T beta) {
   return Operation<T>::getCurrentInterface().getTransformationInterface().transform(a, alpha, beta);
+}
+template <class T>
+Variable<T> transform2(const Tensor<T>& a, T alpha, T beta) {
+  return Operation<T>::getCurrentInterface().getTransformationInterface().transform2(a, alpha, beta);
 }
 
 }  // namespace math
@@ -337,6 +357,38 @@ Variable<T> operator*(const Tensor<T>& a, T s) {
 template <class T>
 Variable<T> operator+(const Tensor<T>& a, T s) {
   return math::transform(a, static_cast<T>(1), s);
+}
+template <class T>
+Variable<T> operator-(const Tensor<T>& a, T s) {
+  return math::transform(a, static_cast<T>(1), static_cast<T>(-s));
+}
+template <class T>
+Variable<T> operator/(const Tensor<T>& a, T s) {
+  return math::transform2(a, s, static_cast<T>(0));
+}
+template <class T>
+Variable<T> operator+(T s, const Tensor<T>& a) {
+  return math::transform(a, static_cast<T>(1), s);
+}
+template <class T>
+Variable<T> operator*(T s, const Tensor<T>& a) {
+  return math::transform(a, s, static_cast<T>(0));
+}
+template <class T>
+Variable<T> operator-(T s, const Tensor<T>& a) {
+  return math::transform(a, static_cast<T>(-1), s);
+}
+template <class T>
+Variable<T> operator-(const Tensor<T>& a, const Tensor<T>& b) {
+  return math::sub(a, b);
+}
+template <class T>
+Variable<T> operator*(const Tensor<T>& a, const Tensor<T>& b) {
+  return math::mul(a, b);
+}
+template <class T>
+Variable<T> operator/(const Tensor<T>& a, const Tensor<T>& b) {
+  return math::div(a, b);
 }
 
 }  // namespace tfcc

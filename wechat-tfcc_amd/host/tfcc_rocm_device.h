@@ -55,8 +55,9 @@ class ROCMSession : public Session {
 void initialize_rocm();
 void initialize_rocm(unsigned deviceID);
 
-// Plain host memory device without any compute interface: lets the framework types (Variable, View,
-// allocators, shape checks) be exercised on machines without a GPU.
+// Plain host memory device whose only interface is Data (memory moves): lets the framework types
+// (Variable, View, allocators, shape checks) and the runtime's loading and graph building be
+// exercised on machines without a GPU.  Every compute interface keeps the throwing default.
 class HostDevice : public Device {
  public:
   HostDevice();
@@ -72,6 +73,9 @@ class HostSession : public Session {
   Device& getDevice() override { return _device; }
   const Device& getDevice() const override { return _device; }
 };
+
+// gives the calling thread the process-wide host device and a host session of its own
+void initialize_host();
 
 namespace rocm {
 namespace quantization {

@@ -1,0 +1,419 @@
+// The operations this runtime knows.  Each follows the accept/reject rules of the reference's
+// operation of the same name (tfcc_runtime/operations/<package>/<name>.cpp): input and output
+// counts, the Any's message type, and the element types of the symbols involved; a rejected node
+// is offered to the next registered operation and ends as UnknowNodeError when nobody takes it.
+//
+//   math.Matmul, math.MatmulWithBias    operations/math/matmul.cpp:52-81, matmulwithbias.cpp:52-88
+//   math.Add / Sub / Mul / Div          operations/math/add.cpp:80-126 (tensor and value operand forms)
+//   math.Gelu, math.Softmax             operations/math/gelu.cpp, softmax.cpp
+//   nn.LayerNormalization               operations/nn/layernormalization.cpp:52-88
+//   base.Transpose, base.Reshape, base.Identity, base.CreateVector
+//                                       operations/base/transpose.cpp, reshape.cpp:27-59,74-104,
+//                                       identity.cpp, createvector.cpp:63-121
+#include <map>
+
+#include "runtime.h"
+
+namespace tfcc {
+namespace runtime {
+
+namespace {
+
+bool same_dtype(Graph& g, const std::vector<std::string>& names, DataType dtype) {
+  for (const std::string& n : names)
+    if (g.getSymbolManager().getSymbolInfo(n).dtype != dtype) return false;
+  return true;
+}
+
+SymbolType stype_of(Graph& g, const std::string& name) { return g.getSymbolManager().getSymbolInfo(name).stype; }
+
+template <class T>
+class TypedOperation : public Operation {
+ protected:
+  static constexpr DataType DTYPE = DataTypeOf<T>::value;
+  std::string _url;
+
+ public:
+  explicit TypedOperation(const std::string& message) : _url(type_url(message)) {}
+  std::string getOperationTypeUrl() const override { return _url; }
+};
+
+// ---- math.Matmul / math.MatmulWithBias ------------------------------------------------------------------
+template <class T>
+class Matmul : public TypedOperation<T> {
+ public:
+  Matmul() : TypedOperation<T>("math.Matmul") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 2 || node.outputs.size() != 1) return false;
+    if (!same_dtype(graph, node.outputs, this->DTYPE) || !same_dtype(graph, node.inputs, this->DTYPE)) return false;
+    auto& sm = graph.getSymbolManager();
+    const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+    const Tensor<T>* b = sm.getTensor(node.inputs[1], T());
+    Variable<T>* out = sm.getVariable(node.outputs[0], T());
+    graph.addStep([a, b, out] { *out = blas::matmul(*a, *b); });
+    return true;
+  }
+};
+
+template <class T>
+class MatmulWithBias : public TypedOperation<T> {
+ public:
+  MatmulWithBias() : TypedOperation<T>("math.MatmulWithBias") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 3 || node.outputs.size() != 1) return false;
+    if (!same_dtype(graph, node.outputs, this->DTYPE) || !same_dtype(graph, node.inputs, this->DTYPE)) return false;
+    auto& sm = graph.getSymbolManager();
+    const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+    const Tensor<T>* b = sm.getTensor(node.inputs[1], T());
+    const Tensor<T>* bias = sm.getTensor(node.inputs[2], T());
+    Variable<T>* out = sm.getVariable(node.outputs[0], T());
+    graph.addStep([a, b, bias, out] { *out = blas::matmul(*a, *b, *bias); });
+    return true;
+  }
+};
+
+// ---- math.Add / Sub / Mul / Div -------------------------------------------------------------------------
+enum class Arith { ADD, SUB, MUL, DIV };
+
+template <Arith OP, class T>
+class Arithmetic : public TypedOperation<T> {
+  static const char* message() {
+    return OP == Arith::ADD ? "math.Add" : OP == Arith::SUB ? "math.Sub" : OP == Arith::MUL ? "math.Mul" : "math.Div";
+  }
+  static Variable<T> tt(const Tensor<T>& a, const Tensor<T>& b) {
+    return OP == Arith::ADD ? a + b : OP == Arith::SUB ? a - b : OP == Arith::MUL ? a * b : a / b;
+  }
+  static Variable<T> tv(const Tensor<T>& a, T b) {
+    return OP == Arith::ADD ? a + b : OP == Arith::SUB ? a - b : OP == Arith::MUL ? a * b : a / b;
+  }
+  static Variable<T> vt(T a, const Tensor<T>& b) {
+    if (OP == Arith::ADD) return a + b;
+    if (OP == Arith::SUB) return a - b;
+    if (OP == Arith::MUL) return a * b;
+    throw NotImplementedError("value / tensor");
+  }
+  static T vv(T a, T b) {
+    return OP == Arith::ADD ? a + b : OP == Arith::SUB ? a - b : OP == Arith::MUL ? a * b : a / b;
+  }
+
+ public:
+  Arithmetic() : TypedOperation<T>(message()) {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 2 || node.outputs.size() != 1) return false;
+    if (!same_dtype(graph, node.outputs, this->DTYPE) || !same_dtype(graph, node.inputs, this->DTYPE)) return false;
+    auto& sm = graph.getSymbolManager();
+    const SymbolType s0 = stype_of(graph, node.inputs[0]), s1 = stype_of(graph, node.inputs[1]);
+    if (is_tensor(s0) && is_tensor(s1)) {
+      const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+      const Tensor<T>* b = sm.getTensor(node.inputs[1], T());
+      Variable<T>* out = sm.getVariable(node.outputs[0], T());
+      graph.addStep([a, b, out] { *out = tt(*a, *b); });
+    } else if (is_tensor(s0) && is_value(s1)) {
+      const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+      const T* b = sm.getValue(node.inputs[1], T());
+      Variable<T>* out = sm.getVariable(node.outputs[0], T());
+      graph.addStep([a, b, out] { *out = tv(*a, *b); });
+    } else if (is_value(s0) && is_tensor(s1)) {
+      const T* a = sm.getValue(node.inputs[0], T());
+      const Tensor<T>* b = sm.getTensor(node.inputs[1], T());
+      Variable<T>* out = sm.getVariable(node.outputs[0], T());
+      graph.addStep([a, b, out] { *out = vt(*a, *b); });
+    } else if (is_value(s0) && is_value(s1)) {
+      const T* a = sm.getValue(node.inputs[0], T());
+      const T* b = sm.getValue(node.inputs[1], T());
+      T* out = sm.getValue(node.outputs[0], T());
+      graph.addStep([a, b, out] { *out = vv(*a, *b); });
+    } else {
+      return false;
+    }
+    return true;
+  }
+};
+
+// ---- math.Gelu / math.Softmax -----------------------------------------------------------------------------
+template <class T>
+class Gelu : public TypedOperation<T> {
+ public:
+  Gelu() : TypedOperation<T>("math.Gelu") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 1 || node.outputs.size() != 1) return false;
+    if (!same_dtype(graph, node.outputs, this->DTYPE) || !same_dtype(graph, node.inputs, this->DTYPE)) return false;
+    auto& sm = graph.getSymbolManager();
+    const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+    Variable<T>* out = sm.getVariable(node.outputs[0], T());
+    graph.addStep([a, out] { *out = math::gelu_accurate(*a); });
+    return true;
+  }
+};
+
+template <class T>
+class Softmax : public TypedOperation<T> {
+ public:
+  Softmax() : TypedOperation<T>("math.Softmax") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 1 || node.outputs.size() != 1) return false;
+    if (!same_dtype(graph, node.outputs, this->DTYPE) || !same_dtype(graph, node.inputs, this->DTYPE)) return false;
+    size_t axis = 0;
+    wire::Reader r(node.operation);
+    uint32_t f, t;
+    while (r.next(f, t)) {
+      if (f == 1 && t == 0) axis = static_cast<size_t>(r.varint());
+      else r.skip(t);
+    }
+    auto& sm = graph.getSymbolManager();
+    const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+    Variable<T>* out = sm.getVariable(node.outputs[0], T());
+    graph.addStep([a, out, axis] { *out = math::softmax(*a, axis); });
+    return true;
+  }
+};
+
+// ---- nn.LayerNormalization --------------------------------------------------------------------------------
+template <class T>
+class LayerNormalization : public TypedOperation<T> {
+ public:
+  LayerNormalization() : TypedOperation<T>("nn.LayerNormalization") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 3 || node.outputs.size() != 1) return false;
+    if (!same_dtype(graph, node.outputs, this->DTYPE) || !same_dtype(graph, node.inputs, this->DTYPE)) return false;
+    proto::Value eps;
+    wire::Reader r(node.operation);
+    uint32_t f, t;
+    while (r.next(f, t)) {
+      if (f == 1 && t == 2) eps = proto::parse_value(r.sub());
+      else r.skip(t);
+    }
+    T epsilon = static_cast<T>(0);
+    if (!eps.get(epsilon)) return false;
+    auto& sm = graph.getSymbolManager();
+    const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+    const Tensor<T>* gamma = sm.getTensor(node.inputs[1], T());
+    const Tensor<T>* beta = sm.getTensor(node.inputs[2], T());
+    Variable<T>* out = sm.getVariable(node.outputs[0], T());
+    graph.addStep([a, gamma, beta, epsilon, out] {
+      *out = nn::layer_normalization(*a, *gamma, *beta, epsilon, a->shape().size() - 1);
+    });
+    return true;
+  }
+};
+
+// ---- base.Transpose ------------------------------------------------------------------------------------------
+template <class T>
+class Transpose : public TypedOperation<T> {
+ public:
+  Transpose() : TypedOperation<T>("base.Transpose") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 1 || node.outputs.size() != 1) return false;
+    if (!same_dtype(graph, node.outputs, this->DTYPE) || !same_dtype(graph, node.inputs, this->DTYPE)) return false;
+    std::vector<size_t> perm;
+    wire::Reader r(node.operation);
+    uint32_t f, t;
+    while (r.next(f, t)) {
+      if (f == 1) r.repeatedVarint(t, perm);
+      else r.skip(t);
+    }
+    auto& sm = graph.getSymbolManager();
+    const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+    Variable<T>* out = sm.getVariable(node.outputs[0], T());
+    graph.addStep([a, out, perm] { *out = base::transpose(*a, perm); });
+    return true;
+  }
+};
+
+// ---- base.Reshape: output is a View of the input; 0 keeps a dimension, one negative entry is inferred ----------
+template <class T, class SHAPE>
+class Reshape : public TypedOperation<T> {
+ public:
+  Reshape() : TypedOperation<T>("base.Reshape") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 2 || node.outputs.size() != 1) return false;
+    auto& sm = graph.getSymbolManager();
+    if (sm.getSymbolInfo(node.outputs[0]).dtype != this->DTYPE || sm.getSymbolInfo(node.inputs[0]).dtype != this->DTYPE)
+      return false;
+    if (sm.getSymbolInfo(node.inputs[1]).dtype != DataTypeOf<SHAPE>::value) return false;
+    const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+    const std::vector<SHAPE>* shape = sm.getVector(node.inputs[1], SHAPE());
+    View<T>* out = sm.getView(node.outputs[0], T());
+    graph.addStep([a, shape, out] {
+      int inferred = -1;
+      unsigned area = 1;
+      std::vector<unsigned> real(shape->size());
+      for (size_t i = 0; i < shape->size(); ++i) {
+        const SHAPE d = (*shape)[i];
+        if (d == 0) {
+          if (i >= a->shape().size()) throw RuntimeError("Reshape: invalid shape");
+          real[i] = a->shape(i);
+          area *= real[i];
+        } else if (d < 0) {
+          if (inferred >= 0) throw RuntimeError("Reshape: invalid shape");
+          inferred = static_cast<int>(i);
+        } else {
+          real[i] = static_cast<unsigned>(d);
+          area *= real[i];
+        }
+      }
+      if (inferred >= 0) {
+        if (area == 0) throw RuntimeError("Reshape: invalid shape");
+        real[inferred] = a->size() / area;
+      }
+      *out = View<T>(*a, Shape(std::move(real)));
+    });
+    return true;
+  }
+};
+
+// ---- base.Identity -----------------------------------------------------------------------------------------------
+template <class T>
+class Identity : public TypedOperation<T> {
+ public:
+  Identity() : TypedOperation<T>("base.Identity") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 1 || node.outputs.size() != 1) return false;
+    if (!same_dtype(graph, node.outputs, this->DTYPE) || !same_dtype(graph, node.inputs, this->DTYPE)) return false;
+    auto& sm = graph.getSymbolManager();
+    const SymbolType si = stype_of(graph, node.inputs[0]), so = stype_of(graph, node.outputs[0]);
+    if (is_tensor(si) && so == SymbolType::VARIABLE) {
+      const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+      Variable<T>* out = sm.getVariable(node.outputs[0], T());
+      graph.addStep([a, out] { *out = data::copy(*a); });
+    } else if (is_value(si) && so == SymbolType::VALUE) {
+      const T* a = sm.getValue(node.inputs[0], T());
+      T* out = sm.getValue(node.outputs[0], T());
+      graph.addStep([a, out] { *out = *a; });
+    } else if (is_vector(si) && so == SymbolType::VECTOR) {
+      const std::vector<T>* a = sm.getVector(node.inputs[0], T());
+      std::vector<T>* out = sm.getVector(node.outputs[0], T());
+      graph.addStep([a, out] { *out = *a; });
+    } else {
+      return false;
+    }
+    return true;
+  }
+};
+
+// ---- base.CreateVector: literal entries, or `pos` entries that splice in an input value / vector ---------------
+template <class T>
+class CreateVector : public TypedOperation<T> {
+  struct Entry {
+    bool fromInput = false;
+    unsigned pos = 0;
+    T literal = T();
+  };
+
+  template <class S>
+  static bool splice(Graph& graph, const std::string& name, std::vector<T>* out) {
+    auto& sm = graph.getSymbolManager();
+    const SymbolInfo& info = sm.getSymbolInfo(name);
+    if (info.dtype != DataTypeOf<S>::value) return false;
+    if (is_value(info.stype)) {
+      const S* v = sm.getValue(name, S());
+      graph.addStep([v, out] { out->push_back(static_cast<T>(*v)); });
+    } else if (is_vector(info.stype)) {
+      const std::vector<S>* v = sm.getVector(name, S());
+      graph.addStep([v, out] {
+        for (S x : *v) out->push_back(static_cast<T>(x));
+      });
+    } else {
+      return false;
+    }
+    return true;
+  }
+
+ public:
+  CreateVector() : TypedOperation<T>("base.CreateVector") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.outputs.size() != 1) return false;
+    auto& sm = graph.getSymbolManager();
+    if (sm.getSymbolInfo(node.outputs[0]).dtype != this->DTYPE) return false;
+    std::vector<Entry> entries;
+    DataType declared = UNKNOW;
+    wire::Reader r(node.operation);
+    uint32_t f, t;
+    while (r.next(f, t)) {
+      if (f == 1 && t == 2) {
+        Entry e;
+        bool known = false;
+        wire::Reader v = r.sub();
+        uint32_t vf, vt;
+        while (v.next(vf, vt)) {
+          if (vf == 1 && vt == 0) { e.literal = static_cast<T>(static_cast<int64_t>(v.varint())); known = true; }
+          else if (vf == 2 && vt == 0) { e.literal = static_cast<T>(v.varint()); known = true; }
+          else if (vf == 3 && vt == 5) { e.literal = static_cast<T>(v.float32()); known = true; }
+          else if (vf == 4 && vt == 1) { e.literal = static_cast<T>(v.float64()); known = true; }
+          else if (vf == 5 && vt == 0) { e.fromInput = true; e.pos = static_cast<unsigned>(v.varint()); known = true; }
+          else v.skip(vt);
+        }
+        if (!known) return false;
+        entries.push_back(e);
+      } else if (f == 2 && t == 0) {
+        declared = static_cast<DataType>(r.varint());
+      } else {
+        r.skip(t);
+      }
+    }
+    if (declared != this->DTYPE) return false;
+    std::vector<T>* out = sm.getVector(node.outputs[0], T());
+    graph.addStep([out] { out->clear(); });
+    for (const Entry& e : entries) {
+      if (!e.fromInput) {
+        const T literal = e.literal;
+        graph.addStep([out, literal] { out->push_back(literal); });
+        continue;
+      }
+      if (e.pos >= node.inputs.size()) return false;
+      const std::string& name = node.inputs[e.pos];
+      bool ok = false;
+#define TFCC_RUNTIME_SPLICE(S, E) ok = ok || splice<S>(graph, name, out);
+      TFCC_RUNTIME_FOR_ALL_TYPES(TFCC_RUNTIME_SPLICE)
+#undef TFCC_RUNTIME_SPLICE
+      if (!ok) return false;
+    }
+    return true;
+  }
+};
+
+class Collector {
+  std::map<std::string, std::vector<std::unique_ptr<Operation>>> _operations;
+
+  void add(Operation* op) { _operations[op->getOperationTypeUrl()].emplace_back(op); }
+
+  template <class T>
+  void addForType() {
+    add(new Matmul<T>());
+    add(new MatmulWithBias<T>());
+    add(new Arithmetic<Arith::ADD, T>());
+    add(new Arithmetic<Arith::SUB, T>());
+    add(new Arithmetic<Arith::MUL, T>());
+    add(new Arithmetic<Arith::DIV, T>());
+    add(new Gelu<T>());
+    add(new Softmax<T>());
+    add(new LayerNormalization<T>());
+    add(new Transpose<T>());
+    add(new Reshape<T, int32_t>());
+    add(new Reshape<T, int64_t>());
+    add(new Identity<T>());
+    add(new CreateVector<T>());
+  }
+
+ public:
+  Collector() {
+#define TFCC_RUNTIME_ADD(T, E) addForType<T>();
+    TFCC_RUNTIME_FOR_ALL_TYPES(TFCC_RUNTIME_ADD)
+#undef TFCC_RUNTIME_ADD
+  }
+  const std::vector<std::unique_ptr<Operation>>& get(const std::string& url) const {
+    static const std::vector<std::unique_ptr<Operation>> empty;
+    auto it = _operations.find(url);
+    return it == _operations.end() ? empty : it->second;
+  }
+};
+
+}  // namespace
+
+const std::vector<std::unique_ptr<Operation>>& operations_for(const std::string& typeUrl) {
+  static const Collector collector;
+  return collector.get(typeUrl);
+}
+
+}  // namespace runtime
+}  // namespace tfcc
