@@ -111,7 +111,7 @@ def cpu_baseline(a, b, size):
                                       q.reshape(-1))
             reps += 1
             dt = time.perf_counter() - t0
-            if dt > 10.0 or reps >= 8:
+            if dt > 10.0 or reps >= 400:
                 break
         tops = 2.0 * size ** 3 * reps / dt / 1e12
         return {"value": round(tops, 4), "unit": "TOP/s", "cores": min(threads, cores), "kind": "reference",
@@ -202,6 +202,29 @@ def bench_other(torch, pkg, dev, steps, warmup, c3):
         out["c5_int8_gemv_m%d_4096x11008" % m] = {"ms": round(ms, 5), "gbs": round(gbs, 1),
                                                    "frac_hbm": round(gbs / PEAK_HBM_GBS, 4),
                                                    "gops": round(2.0 * m * n * k / ms / 1e6, 1)}
+
+    # C4: one BERT-base encoder layer through the model runtime (fp32, batch 8, seq 128); the entrance
+    # graph alone is timed with events on the runtime's stream, tensors resident in HBM
+    import importlib
+    mf = importlib.import_module("wechat_tfcc_amd.modelfile")
+    rt = importlib.import_module("wechat_tfcc_amd.runtime_api")
+    batch, seq, hidden, heads, ffn = 8, 128, 768, 12, 3072
+    w = mf.bert_layer_weights(rng, hidden, ffn)
+    graph = mf.bert_encoder_layer(w, batch, seq, heads)
+    model = rt.Model(mf.write_model([graph], graph.name))
+    x = {"hidden_states": rng.normal(size=(batch, seq, hidden)).astype(np.float32)}
+    rows = batch * seq
+    gemm_flop = 2.0 * rows * hidden * (4 * hidden + 2 * ffn) + 2 * 2.0 * batch * heads * seq * seq * (hidden // heads)
+    entry = {"gemm_flop": gemm_flop, "nodes": len(graph.nodes)}
+    for label, replay in (("step_by_step", False), ("graph_replay", True)):
+        model.set_replay(replay)
+        us = model.time(x, warmup=max(3, warmup), iters=max(steps, 20))
+        entry[label + "_us"] = round(us, 2)
+        entry[label + "_tflops"] = round(gemm_flop / us / 1e6, 2)
+        entry[label + "_frac_fp32_mfma"] = round(gemm_flop / us / 1e6 / PEAK_FP32_TFLOPS, 4)
+    model.set_replay(False)
+    model.close()
+    out["c4_bert_base_layer_b8_s128_runtime"] = entry
     return out
 
 
@@ -280,7 +303,7 @@ def main():
                    "m": size, "n": size, "k": size},
         "roofline": {"bound": "mfma", "achieved": round(kernel_tops, 2), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                      "frac": round(kernel_tops / PEAK_INT8_TOPS, 4), "traffic": None,
-                     "kernel": "qgemm_kernel<256,256,64,aligned,requant>", "kernel_ms": round(kernel_ms, 5),
+                     "kernel": "qgemm_dma_kernel<256,256,2,4,4,requant>", "kernel_ms": round(kernel_ms, 5),
                      "algorithmic_ops_per_launch": ops},
     }
     traffic_file = os.path.join(ROOT, "profiles", "traffic.json")
