@@ -6,9 +6,10 @@
 //
 // Data path of one BM x BN tile (WGM x WGN wavefronts; eight for the 256 x 256 tile, so that every
 // SIMD holds two: one wavefront's LDS reads, waits and VALU work overlap the other's matrix ops):
-//   HBM -> LDS  buffer_load_dwordx4 ... lds (asynchronous, no VGPRs): every K slab of 64 bytes is
-//               copied as it lies in memory, A rows as As[row][64] and B rows as Bs[k][BN], into a
-//               ring of STAGES LDS buffers, STAGES-1 slabs ahead of the matrix cores.  Out-of-range
+//   HBM -> LDS  buffer_load_dwordx4 ... lds (asynchronous, no VGPRs): every K slab of 128 bytes is
+//               copied as it lies in memory, A rows as As[row][128] (one whole memory line per row
+//               piece) and B rows as Bs[k][BN], into a ring of STAGES LDS buffers, STAGES-1 slabs
+//               ahead of the matrix cores.  Out-of-range
 //               rows read zero through the buffer descriptor.  The 16-byte chunk a lane copies is
 //               chosen so that the LDS image is xor-swizzled (the DMA writes lanes contiguously).
 //   LDS -> VGPR A: ds_read_b128 (16 consecutive k of a row), xor 0x80 turns uint8 into int8.
@@ -35,7 +36,8 @@ typedef int v16i __attribute__((ext_vector_type(16)));
 
 namespace {
 
-constexpr int BK = 64;
+constexpr int BK = 128;      // bytes of k per slab: a row piece of A is one full 128-byte memory line
+constexpr int KS = BK / 32;  // 32-deep matrix-op steps per slab
 
 // One asynchronous 16-byte-per-lane copy HBM -> LDS.  The LDS address of lane i is ldsBase + 16*i
 // (ldsBase wave-uniform, goes through M0); voffset is the lane's byte offset into the buffer.
@@ -65,10 +67,11 @@ __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0f70);
 }
 
-__device__ __forceinline__ int swzA(int row) { return ((row >> 1) & 3) ^ ((row >> 3) & 1); }
+// 16 consecutive rows of one logical chunk fall into 16 different 16-byte slots of the 256-byte bank stripe
+__device__ __forceinline__ int swzA(int row) { return (row >> 1) & 7; }
 
 template <int BM, int BN, int WGM, int WGN, int STAGES, bool REQUANT>
-__global__ __launch_bounds__(WGM * WGN * 64) void qgemm_dma_kernel(const QGemmParams p) {
+__global__ __launch_bounds__(WGM * WGN * 64, 2) void qgemm_dma_kernel(const QGemmParams p) {
   constexpr int kThreads = WGM * WGN * 64;
   constexpr int WM = BM / WGM, WN = BN / WGN;
   constexpr int MI = WM / 32, NI = WN / 32;
@@ -128,12 +131,12 @@ __global__ __launch_bounds__(WGM * WGN * 64) void qgemm_dma_kernel(const QGemmPa
   }
 
   // ---- per-thread copy descriptors: which 16 bytes of the slab this lane moves in each copy.
-  // LDS slot s (16 bytes) of the A image holds row s/4, physical chunk s%4 = logical chunk ^ swzA(row).
+  // LDS slot s (16 bytes) of the A image holds row s/8, physical chunk s%8 = logical chunk ^ swzA(row).
   unsigned aOff[A_COPIES], bOff[B_COPIES];  // byte offsets into A / B for slab 0
 #pragma unroll
   for (int c = 0; c < A_COPIES; ++c) {
     const int s = c * kThreads + tid;
-    const int row = s >> 2, phys = s & 3;
+    const int row = s >> 3, phys = s & 7;
     aOff[c] = (m0 + row) * K + ((phys ^ swzA(row)) << 4);
   }
   // LDS slot s of the B image holds k row s/BCH, physical chunk s%BCH = logical chunk ^ (k & 7).
@@ -163,18 +166,20 @@ __global__ __launch_bounds__(WGM * WGN * 64) void qgemm_dma_kernel(const QGemmPa
     for (int j = 0; j < NI; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
-  int colsum[NI];
+  int colsum[NI][4];  // four independent partial sums per block: a single chain would stall on the dot latency
 #pragma unroll
-  for (int j = 0; j < NI; ++j) colsum[j] = 0;
+  for (int j = 0; j < NI; ++j)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) colsum[j][q] = 0;
 
   // ---- operand addresses inside a stage
   const int l32 = lane & 31, g = lane >> 5;
   // A: row wm*WM + 32*i + l32, logical chunk 2*ks + g
-  int aAddr[MI][2];
+  int aAddr[MI][KS];
 #pragma unroll
   for (int i = 0; i < MI; ++i)
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
+    for (int ks = 0; ks < KS; ++ks) {
       const int row = wm * WM + 32 * i + l32;
       aAddr[i][ks] = row * BK + (((2 * ks + g) ^ swzA(row)) << 4);
     }
@@ -224,7 +229,7 @@ __global__ __launch_bounds__(WGM * WGN * 64) void qgemm_dma_kernel(const QGemmPa
       if (j % WGM == wm) {
         asm volatile("" ::: "memory");  // keep this a wave-uniform branch, not a select over both blocks
 #pragma unroll
-        for (int q = 0; q < 4; ++q) colsum[j] = __builtin_amdgcn_sdot4(ub[j][q], 0x01010101, colsum[j], false);
+        for (int q = 0; q < 4; ++q) colsum[j][q] = __builtin_amdgcn_sdot4(ub[j][q], 0x01010101, colsum[j][q], false);
       }
     }
     v4i ax = {0, 0, 0, 0};
@@ -259,13 +264,17 @@ __global__ __launch_bounds__(WGM * WGN * 64) void qgemm_dma_kernel(const QGemmPa
   v4i fa[2][MI], fb[2][NI];
 #pragma unroll
   for (int q = 0; q < NLOAD; ++q) loadOne(smem, smem + A_BYTES, 0, q, fa[0], fb[0]);
+  static_assert(KS % 2 == 0, "the operand registers alternate per step");
   for (unsigned kt = 0; kt < KT; ++kt) {
     const unsigned cur = kt % STAGES, nxt = (kt + 1) % STAGES;
-    step(fa[0], fb[0], fa[1], fb[1], cur, 1, std::false_type{}, 0u);   // k step 0 of slab kt; reads k step 1
+    // k steps 0 .. KS-2 of slab kt, each reading the operands of the step after it
+#pragma unroll
+    for (int ks = 0; ks < KS - 1; ++ks)
+      step(fa[ks & 1], fb[ks & 1], fa[(ks + 1) & 1], fb[(ks + 1) & 1], cur, ks + 1, std::false_type{}, 0u);
     wait_vmcnt<COPIES*(STAGES - 2)>();
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the reads of slab kt have returned
     __syncthreads();
-    // k step 1 of slab kt; reads k step 0 of slab kt+1; refills the stage of slab kt
+    // last k step of slab kt; reads k step 0 of slab kt+1; refills the stage of slab kt
     step(fa[1], fb[1], fa[0], fb[0], nxt, 0, std::true_type{}, kt + STAGES);
   }
   wait_vmcnt<0>();
@@ -282,7 +291,8 @@ __global__ __launch_bounds__(WGM * WGN * 64) void qgemm_dma_kernel(const QGemmPa
 #pragma unroll
   for (int j = 0; j < NI; ++j) {
     if (j % WGM == wm) {
-      int s = colsum[j] + __shfl_xor(colsum[j], 32, 64);
+      int s = colsum[j][0] + colsum[j][1] + colsum[j][2] + colsum[j][3];
+      s += __shfl_xor(s, 32, 64);
       if (g == 0) colTerm[wn * WN + 32 * j + 16 * colHalf + s16] = s;
     }
   }
@@ -407,9 +417,9 @@ bool qgemm_dma_supported(const QGemmParams& p, bool requant) {
 int qgemm_dma_launch(hipStream_t stream, const QGemmParams& p, bool requant) {
   const unsigned long long big = (unsigned long long)((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batch;
   if (big >= 192) {
-    return requant ? launch<256, 256, 2, 4, 4, true>(stream, p) : launch<256, 256, 2, 4, 4, false>(stream, p);
+    return requant ? launch<256, 256, 2, 4, 2, true>(stream, p) : launch<256, 256, 2, 4, 2, false>(stream, p);
   }
-  return requant ? launch<128, 128, 2, 2, 4, true>(stream, p) : launch<128, 128, 2, 2, 4, false>(stream, p);
+  return requant ? launch<128, 128, 2, 2, 2, true>(stream, p) : launch<128, 128, 2, 2, 2, false>(stream, p);
 }
 
 }  // namespace tfcc_rocm
