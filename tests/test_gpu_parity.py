@@ -324,6 +324,9 @@ def test_sgemm_exact_cases(pkg, T):
     ((8, 128, 768), (768, 3072)), ((8, 128, 3072), (3072, 768)),   # BERT-base FFN
     ((1024, 1024), (1024, 4096)),                # enough tiles for the 128x128 configuration
     ((130, 36), (36, 516)), ((257, 100), (100, 260)),
+    # few tiles and a long K: several K groups per workgroup (x4, x2), with ragged K and edges
+    ((1024, 768), (768, 768)), ((200, 1000), (1000, 300)), ((300, 300), (300, 500)), ((64, 516), (516, 64)),
+    ((3, 70, 1028), (1028, 90)),
 ])
 def test_sgemm_shapes_against_oracle(pkg, T, shape_a, shape_b):
     """The four shape families of tfcc/test/blas.cpp:34-61 plus the benchmark's batched shapes."""

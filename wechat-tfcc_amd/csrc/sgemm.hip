@@ -38,10 +38,14 @@ constexpr int CH = BK / 4;  // 16-byte chunks per LDS row
 
 __device__ __forceinline__ int swz(int row, int chunk) { return chunk ^ ((row >> 1) & (CH - 1)); }
 
-// WGM x WGN wavefronts, each owning an (MI*32) x (NI*32) sub-tile
-template <int WGM, int WGN, int MI, int NI, bool VEC>
-__global__ __launch_bounds__(kThreads) void sgemm_kernel(const SgemmParams p) {
-  static_assert(WGM * WGN == 4, "four wavefronts");
+// WGM x WGN wavefronts, each owning an (MI*32) x (NI*32) sub-tile.  With KSPLIT > 1 the workgroup
+// holds KSPLIT such groups of four wavefronts on the same tile: group q walks the K slabs q,
+// q + KSPLIT, ... through LDS buffers of its own and the partial tiles are added up through LDS in
+// a fixed order at the end.  That is for products with few tiles and a long K, where one group per
+// CU could not hide the memory latency of its own loads.
+template <int WGM, int WGN, int MI, int NI, bool VEC, int KSPLIT>
+__global__ __launch_bounds__(kThreads * KSPLIT) void sgemm_kernel(const SgemmParams p) {
+  static_assert(WGM * WGN == 4, "four wavefronts per group");
   constexpr int BM = WGM * MI * 32, BN = WGN * NI * 32;
   constexpr int WM = MI * 32, WN = NI * 32;
   constexpr int A_TOTAL = BM * CH, B_TOTAL = (BN / 4) * CH;    // 128-bit chunks of A, 4x4 blocks of B
@@ -49,10 +53,11 @@ __global__ __launch_bounds__(kThreads) void sgemm_kernel(const SgemmParams p) {
   constexpr int B_ITEMS = (B_TOTAL + kThreads - 1) / kThreads;
 
   extern __shared__ __align__(16) float smemf[];
-  float* As = smemf;                 // [2][BM][BK]
-  float* Bs = smemf + 2 * BM * BK;   // [2][BN][BK]
+  const int grp = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8));  // K group, wave-uniform
+  float* As = smemf + grp * 2 * (BM + BN) * BK;  // [2][BM][BK]
+  float* Bs = As + 2 * BM * BK;                  // [2][BN][BK]
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WGN, wn = wave % WGN;
 
   unsigned tm, tn, bi;
@@ -166,9 +171,11 @@ __global__ __launch_bounds__(kThreads) void sgemm_kernel(const SgemmParams p) {
     }
   };
 
-  const unsigned KT = (K + BK - 1) / BK;
-  loadA(0);
-  loadB(0);
+  // every group makes the same number of steps (the barriers are workgroup-wide); a slab past the
+  // end of K loads zeros
+  const unsigned KT = ((K + BK - 1) / BK + KSPLIT - 1) / KSPLIT;
+  loadA(grp * BK);
+  loadB(grp * BK);
   storeTiles(0);
   __syncthreads();
 
@@ -176,8 +183,8 @@ __global__ __launch_bounds__(kThreads) void sgemm_kernel(const SgemmParams p) {
   for (unsigned kt = 0; kt < KT; ++kt) {
     const int buf = kt & 1;
     if (kt + 1 < KT) {
-      loadA((kt + 1) * BK);
-      loadB((kt + 1) * BK);
+      loadA(((kt + 1) * KSPLIT + grp) * BK);
+      loadB(((kt + 1) * KSPLIT + grp) * BK);
     }
     const float* as = As + buf * BM * BK + (wm * WM) * BK;
     const float* bs = Bs + buf * BN * BK + (wn * WN) * BK;
@@ -204,6 +211,32 @@ __global__ __launch_bounds__(kThreads) void sgemm_kernel(const SgemmParams p) {
     }
     if (kt + 1 < KT) storeTiles(buf ^ 1);
     __syncthreads();
+  }
+
+  if constexpr (KSPLIT > 1) {
+    // partial tiles of groups 1 .. KSPLIT-1 go through LDS (the slab buffers are free after the last
+    // barrier) and are added by group 0 in group order
+    float* red = smemf;
+    const int slot = ((grp - 1) * 4 + wave) * MI * NI;
+    if (grp > 0) {
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) red[((slot + i * NI + j) * 16 + r) * 64 + lane] = acc[i][j][r];
+    }
+    __syncthreads();
+    if (grp > 0) return;
+#pragma unroll
+    for (int q = 1; q < KSPLIT; ++q)
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            acc[i][j][r] += red[((((q - 1) * 4 + wave) * MI * NI + i * NI + j) * 16 + r) * 64 + lane];
   }
 
   // ---- epilogue: + bias, store.  Lane (i, g) owns columns NI*i .. NI*i+NI-1 of the wavefront's
@@ -237,7 +270,7 @@ __global__ __launch_bounds__(kThreads) void sgemm_kernel(const SgemmParams p) {
   }
 }
 
-template <int WGM, int WGN, int MI, int NI, bool VEC>
+template <int WGM, int WGN, int MI, int NI, bool VEC, int KSPLIT = 1>
 int launch(hipStream_t stream, SgemmParams p) {
   constexpr int BM = WGM * MI * 32, BN = WGN * NI * 32;
   p.tilesM = (p.M + BM - 1) / BM;
@@ -246,15 +279,16 @@ int launch(hipStream_t stream, SgemmParams p) {
   if (total > 0x7fffffffull) return set_error(TFCC_ROCM_INVALID_ARGUMENT, "sgemm: too many tiles");
   p.tilesTotal = (unsigned)total;
   p.chunk = (p.tilesTotal + 7) / 8;
-  constexpr size_t lds = 2 * (size_t)(BM + BN) * BK * sizeof(float);
-  auto kern = sgemm_kernel<WGM, WGN, MI, NI, VEC>;
+  constexpr size_t lds = KSPLIT * 2 * (size_t)(BM + BN) * BK * sizeof(float);
+  static_assert(lds <= 160 * 1024 && (size_t)(KSPLIT - 1) * BM * BN * sizeof(float) <= lds, "LDS budget");
+  auto kern = sgemm_kernel<WGM, WGN, MI, NI, VEC, KSPLIT>;
   static bool attrSet = false;
   if (!attrSet) {
     TFCC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     attrSet = true;
   }
-  hipLaunchKernelGGL(kern, dim3(p.chunk * 8), dim3(kThreads), lds, stream, p);
+  hipLaunchKernelGGL(kern, dim3(p.chunk * 8), dim3(kThreads * KSPLIT), lds, stream, p);
   return check_launch("sgemm");
 }
 
@@ -275,12 +309,16 @@ extern "C" int tfcc_rocm_sgemm_strided_batched(void* stream, const float* a, uin
   p.M = m; p.N = n; p.K = k; p.batch = batch;
   const bool vec = (k % 4 == 0) && (n % 4 == 0) && ((uintptr_t)a % 16 == 0) && ((uintptr_t)b % 16 == 0) &&
                    ((uintptr_t)c % 16 == 0) && (stride_a % 4 == 0) && (stride_b % 4 == 0) && (stride_c % 4 == 0) &&
-                   ((unsigned long long)m * k < (1ull << 30)) && (((unsigned long long)k + 64) * n + 1024 < (1ull << 30));
+                   ((unsigned long long)m * k < (1ull << 30)) && (((unsigned long long)k + 256) * n + 1024 < (1ull << 30));
   hipStream_t s = as_stream(stream);
   // 128x128 tiles once there are enough of them to fill the 256 CUs twice over, else 64x64
   const unsigned long long big = (unsigned long long)((m + 127) / 128) * ((n + 127) / 128) * batch;
   if (vec) {
     if (big >= 512) return launch<4, 1, 1, 4, true>(s, p);
+    // few 64x64 tiles and a long K: several K groups per workgroup keep the CUs that have a tile busy
+    const unsigned long long small = (unsigned long long)((m + 63) / 64) * ((n + 63) / 64) * batch;
+    if (small <= 320 && k >= 512) return launch<2, 2, 1, 1, true, 4>(s, p);
+    if (small <= 640 && k >= 256) return launch<2, 2, 1, 1, true, 2>(s, p);
     return launch<2, 2, 1, 1, true>(s, p);
   }
   TFCC_REQUIRE((unsigned long long)m * n < (1ull << 32) && (unsigned long long)m * k < (1ull << 32) &&
