@@ -90,6 +90,17 @@ int tfcc_rocm_sgemm_strided_batched(void* stream, const float* a, uint64_t strid
                                     uint64_t stride_c, unsigned m, unsigned n, unsigned k,
                                     unsigned batch);
 
+/* The same product with more of the caller's next steps done in the tile store: after the bias,
+ * `residual` (optional; laid out like c, batch stride stride_residual) is added, then `activation`
+ * is applied (0 none, 1 erf-form GELU, tfcc/mkl/kernel/tfcc_mklactivationkernel.hpp:213-220).  Each
+ * step rounds to fp32 exactly as the separate operations would, so fusing changes no bit.  Stands
+ * where the reference's runtime calls matmul, then add / gelu as separate operations
+ * (tfcc_runtime/operations/math/matmulwithbias.cpp:29-40, add.cpp:27-37, gelu.cpp:27-36). */
+int tfcc_rocm_sgemm_fused(void* stream, const float* a, uint64_t stride_a, const float* b,
+                          uint64_t stride_b, const float* bias, const float* residual,
+                          uint64_t stride_residual, float* c, uint64_t stride_c, unsigned m,
+                          unsigned n, unsigned k, unsigned batch, int activation);
+
 /* ---------------------------------------------------------------------------------------------
  * Quantized uint8 x int8 -> int32 matmul.
  * Replaces _mkl_create_offset_matrix + _MKLQuantizationMatmulAVX256::quantizedMatmulColMajor,
@@ -183,6 +194,10 @@ int tfcc_rocm_quantize_minmax(void* stream, const float* in, uint64_t total, voi
  * ------------------------------------------------------------------------------------------- */
 /* softmax over the last axis: _MKLActivationKernel::softmaxV2, tfcc/mkl/kernel/tfcc_mklactivationkernel.hpp:137-155 */
 int tfcc_rocm_softmax_f32(void* stream, const float* in, uint64_t rows, unsigned cols, float* out);
+/* softmax(in / divisor) with the division done in fp32 per element first, i.e. the result of
+ * `a / s` (tfcc/core/operations/tfcc_operator.cpp:78-95) followed by softmax, in one pass */
+int tfcc_rocm_softmax_div_f32(void* stream, const float* in, uint64_t rows, unsigned cols, float divisor,
+                              float* out);
 /* _mkl_layer_normalize, tfcc/mkl/interfaces/tfcc_mklnormalizationinterface.cpp:29-62 */
 int tfcc_rocm_layer_norm_f32(void* stream, const float* in, const float* gamma, const float* beta,
                              float epsilon, uint64_t rows, unsigned cols, float* out);

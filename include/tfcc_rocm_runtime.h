@@ -46,6 +46,15 @@ int tfcc_rocm_runtime_buffer_free(void* buffer);
 int tfcc_rocm_runtime_model_test(void* model, const void* npz, size_t len, int* passed,
                                  char** report);
 
+/* Graphs built after this call on the calling thread fuse node sequences into single kernels
+ * (matmul + gelu, matmul + residual add, div + softmax; the default) or run every node as written.
+ * Results are bit-identical either way.  The reference selects a fused variant of the model per
+ * device instead (model.cpu.pb, tfcc_runtime/framework/model.cpp:311-322). */
+int tfcc_rocm_runtime_set_fusion(int enable);
+
+/* number of bound steps of the entrance graph (builds it if needed); nodes fused together share one */
+int tfcc_rocm_runtime_model_step_count(void* model, size_t* steps);
+
 /* Record the entrance graph's kernel sequence once and replay it with one launch per run from
  * then on (no counterpart in the reference, whose graphs are x86 call sequences). */
 int tfcc_rocm_runtime_model_set_replay(void* model, int enable);

@@ -230,6 +230,43 @@ def test_replay_reproduces_step_by_step_results(mf, rt, dev):
 
 
 @pytest.mark.gpu
+def test_fused_graph_is_bit_identical_to_the_graph_as_written(mf, rt, dev):
+    rng = np.random.default_rng(7)
+    for batch, seq, hidden, heads, ffn in ((2, 16, 64, 4, 128), (3, 7, 96, 3, 200), (4, 128, 256, 4, 1024)):
+        w = mf.bert_layer_weights(rng, hidden, ffn)
+        g = mf.bert_encoder_layer(w, batch, seq, heads)
+        blob = mf.write_model([g], g.name)
+        x = rng.normal(size=(batch, seq, hidden)).astype(np.float32)
+        rt.set_fusion(False)
+        plain = rt.Model(blob)
+        want = plain.run({"hidden_states": x})["layer_output"]
+        rt.set_fusion(True)
+        fused = rt.Model(blob)
+        got = fused.run({"hidden_states": x})["layer_output"]
+        # matmul+gelu, 2 x matmul+add and div+softmax each save one step
+        assert plain.step_count() - fused.step_count() == 4
+        assert np.array_equal(got, want)
+        fused.set_replay(True)
+        for _ in range(3):
+            assert np.array_equal(fused.run({"hidden_states": x})["layer_output"], want)
+    # an Add whose other operand does not have the product's shape runs unfused, same result
+    g = mf.GraphBuilder("g")
+    a = g.input("a", mf.FLOAT, [5, 8])
+    wgt = g.constant("w", rng.normal(size=(8, 6)).astype(np.float32))
+    bias = g.constant("b", rng.normal(size=6).astype(np.float32))
+    row = g.constant("row", rng.normal(size=6).astype(np.float32))
+    y = g.binary("Add", g.matmul(a, wgt, bias), row)
+    g.output(y)
+    av = rng.normal(size=(5, 8)).astype(np.float32)
+    outs = []
+    for enable in (False, True):
+        rt.set_fusion(enable)
+        outs.append(rt.Model(mf.write_model([g], "g")).run({"a": av})[y])
+    rt.set_fusion(True)
+    assert np.array_equal(outs[0], outs[1])
+
+
+@pytest.mark.gpu
 def test_matmul_nodes_of_other_dtypes_fail_at_run_time(mf, rt, dev):
     """accepted when the graph is built, NotImplementedError when run - as on the reference's
     backends, where only float has a blas implementation"""

@@ -80,6 +80,8 @@ SYMBOLS = {
     "tfcc_rocm_stream_end_capture": (_I, [_VP, C.POINTER(_VP)]),
     "tfcc_rocm_graph_launch": (_I, [_VP, _VP]),
     "tfcc_rocm_graph_destroy": (_I, [_VP]),
+    "tfcc_rocm_sgemm_fused": (_I, [_VP, _VP, _U64, _VP, _U64, _VP, _VP, _U64, _VP, _U64, _U, _U, _U, _U, _I]),
+    "tfcc_rocm_softmax_div_f32": (_I, [_VP, _VP, _U64, _U, _F, _VP]),
     "tfcc_rocm_transform2_f32": (_I, [_VP, _VP, _U64, _F, _F, _VP]),
     "tfcc_rocm_binary_f32": (_I, [_VP, _I, _VP, _VP, _U64, _U64, _VP]),
     "tfcc_rocm_transpose_f32": (_I, [_VP, _VP, C.POINTER(C.c_uint), C.POINTER(C.c_uint), _I, _VP]),

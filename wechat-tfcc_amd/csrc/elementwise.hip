@@ -40,16 +40,17 @@ __device__ __forceinline__ float block_reduce(float v, float* sh) {
 }
 
 // one workgroup of 256 threads per row
-__global__ __launch_bounds__(256) void softmax_kernel(const float* in, unsigned cols, float* out) {
+__global__ __launch_bounds__(256) void softmax_kernel(const float* in, unsigned cols, float divisor, bool divide,
+                                                      float* out) {
   __shared__ float sh[4];
   const float* a = in + (size_t)blockIdx.x * cols;
   float* o = out + (size_t)blockIdx.x * cols;
   float mx = -3.402823466e+38f;
-  for (unsigned i = threadIdx.x; i < cols; i += 256) mx = fmaxf(mx, a[i]);
+  for (unsigned i = threadIdx.x; i < cols; i += 256) mx = fmaxf(mx, divide ? a[i] / divisor : a[i]);
   mx = block_reduce<true>(mx, sh);
   float s = 0.f;
   for (unsigned i = threadIdx.x; i < cols; i += 256) {
-    float e = expf(a[i] - mx);
+    float e = expf((divide ? a[i] / divisor : a[i]) - mx);
     o[i] = e;
     s += e;
   }
@@ -58,7 +59,8 @@ __global__ __launch_bounds__(256) void softmax_kernel(const float* in, unsigned 
 }
 
 // rows of at most 256 columns: one wavefront per row, values stay in registers
-__global__ __launch_bounds__(256) void softmax_small_kernel(const float* in, size_t rows, unsigned cols, float* out) {
+__global__ __launch_bounds__(256) void softmax_small_kernel(const float* in, size_t rows, unsigned cols, float divisor,
+                                                            bool divide, float* out) {
   const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   const int lane = threadIdx.x & 63;
   if (row >= rows) return;
@@ -69,7 +71,7 @@ __global__ __launch_bounds__(256) void softmax_small_kernel(const float* in, siz
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
     unsigned i = lane + 64 * q;
-    v[q] = i < cols ? a[i] : -3.402823466e+38f;
+    v[q] = i < cols ? (divide ? a[i] / divisor : a[i]) : -3.402823466e+38f;
     mx = fmaxf(mx, v[q]);
   }
   mx = wave_max(mx);
@@ -190,16 +192,26 @@ using namespace tfcc_rocm;
 
 extern "C" {
 
-int tfcc_rocm_softmax_f32(void* stream, const float* in, uint64_t rows, unsigned cols, float* out) {
+static int softmax_launch(void* stream, const float* in, uint64_t rows, unsigned cols, float divisor, bool divide,
+                          float* out) {
   TFCC_REQUIRE(in && out, "softmax: null argument");
   TFCC_REQUIRE(rows > 0 && cols > 0, "softmax: empty tensor");
   TFCC_REQUIRE(rows < (1ull << 31), "softmax: too many rows");
   if (cols <= 256)
     hipLaunchKernelGGL(softmax_small_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, as_stream(stream), in,
-                       (size_t)rows, cols, out);
+                       (size_t)rows, cols, divisor, divide, out);
   else
-    hipLaunchKernelGGL(softmax_kernel, dim3((unsigned)rows), dim3(256), 0, as_stream(stream), in, cols, out);
+    hipLaunchKernelGGL(softmax_kernel, dim3((unsigned)rows), dim3(256), 0, as_stream(stream), in, cols, divisor, divide,
+                       out);
   return check_launch("softmax");
+}
+
+int tfcc_rocm_softmax_f32(void* stream, const float* in, uint64_t rows, unsigned cols, float* out) {
+  return softmax_launch(stream, in, rows, cols, 1.f, false, out);
+}
+
+int tfcc_rocm_softmax_div_f32(void* stream, const float* in, uint64_t rows, unsigned cols, float divisor, float* out) {
+  return softmax_launch(stream, in, rows, cols, divisor, true, out);
 }
 
 int tfcc_rocm_layer_norm_f32(void* stream, const float* in, const float* gamma, const float* beta,

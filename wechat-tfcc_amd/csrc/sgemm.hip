@@ -26,8 +26,10 @@ struct SgemmParams {
   const float* A;
   const float* B;
   const float* bias;
+  const float* residual;  // optional, laid out like C (batch stride strideR): added after the bias
   float* C;
-  unsigned long long strideA, strideB, strideC;
+  unsigned long long strideA, strideB, strideC, strideR;
+  int act;                // 0 none, 1 erf-form GELU applied last
   unsigned M, N, K, batch;
   unsigned tilesM, tilesN, tilesTotal, chunk;
 };
@@ -110,8 +112,13 @@ __global__ __launch_bounds__(kThreads * KSPLIT) void sgemm_kernel(const SgemmPar
       const unsigned gr = m0 + row, gk = k0 + ch * 4;
       v4f v = {0.f, 0.f, 0.f, 0.f};
       if constexpr (VEC) {
-        v4f t = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rsrcA, (gr * K + gk) * 4u, 0, 0));
-        v = gk < K ? t : v;
+        // Only the slab that crosses the end of K masks its values: a select on every loaded value
+        // would make the compiler wait for the load right here instead of after the matrix ops.
+        v = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rsrcA, (gr * K + gk) * 4u, 0, 0));
+        if (k0 + BK > K) {
+          asm volatile("" ::: "memory");  // keeps this a real (wave-uniform) branch
+          v = gk < K ? v : v4f{0.f, 0.f, 0.f, 0.f};
+        }
       } else {
         if (gr < M) {
 #pragma unroll
@@ -242,6 +249,8 @@ __global__ __launch_bounds__(kThreads * KSPLIT) void sgemm_kernel(const SgemmPar
   // ---- epilogue: + bias, store.  Lane (i, g) owns columns NI*i .. NI*i+NI-1 of the wavefront's
   // column range and rows 8*(r/4) + 4*g + r%4 of each 32-row block.
   float* __restrict__ C = p.C + (size_t)bi * p.strideC;
+  const float* __restrict__ R = p.residual ? p.residual + (size_t)bi * p.strideR : nullptr;
+  const int act = p.act;
   const unsigned gcol = n0 + wn * WN + NI * lrow;
   float bv[NI];
 #pragma unroll
@@ -257,6 +266,17 @@ __global__ __launch_bounds__(kThreads * KSPLIT) void sgemm_kernel(const SgemmPar
 #pragma unroll
       for (int j = 0; j < NI; ++j) v[j] = acc[i][j][r] + bv[j];
       const size_t off = (size_t)grow * N + gcol;
+      if (R) {
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+          if (gcol + j < N) v[j] += R[off + j];
+      }
+      if (act == 1) {
+        // same expression as the stand-alone GELU kernel, so that fusing changes no bit
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+          v[j] = (float)(0.5 * (double)v[j] * (double)(1.0f + erff(v[j] / 1.4142135623730951f)));
+      }
       if (vecOK) {
         if constexpr (NI == 4) *reinterpret_cast<v4f*>(C + off) = v4f{v[0], v[1], v[2], v[3]};
         else if constexpr (NI == 2) *reinterpret_cast<float2*>(C + off) = make_float2(v[0], v[1]);
@@ -301,10 +321,18 @@ extern "C" int tfcc_rocm_sgemm_strided_batched(void* stream, const float* a, uin
                                                const float* b, uint64_t stride_b, const float* bias,
                                                float* c, uint64_t stride_c, unsigned m, unsigned n,
                                                unsigned k, unsigned batch) {
+  return tfcc_rocm_sgemm_fused(stream, a, stride_a, b, stride_b, bias, nullptr, 0, c, stride_c, m, n, k, batch, 0);
+}
+
+extern "C" int tfcc_rocm_sgemm_fused(void* stream, const float* a, uint64_t stride_a, const float* b,
+                                     uint64_t stride_b, const float* bias, const float* residual,
+                                     uint64_t stride_residual, float* c, uint64_t stride_c, unsigned m,
+                                     unsigned n, unsigned k, unsigned batch, int activation) {
   TFCC_REQUIRE(a && b && c, "sgemm: null operand");
   TFCC_REQUIRE(m > 0 && n > 0 && k > 0 && batch > 0, "sgemm: empty operand");
+  TFCC_REQUIRE(activation == 0 || activation == 1, "sgemm: unknown activation %d", activation);
   SgemmParams p{};
-  p.A = a; p.B = b; p.bias = bias; p.C = c;
+  p.A = a; p.B = b; p.bias = bias; p.C = c; p.residual = residual; p.strideR = stride_residual; p.act = activation;
   p.strideA = stride_a; p.strideB = stride_b; p.strideC = stride_c;
   p.M = m; p.N = n; p.K = k; p.batch = batch;
   const bool vec = (k % 4 == 0) && (n % 4 == 0) && ((uintptr_t)a % 16 == 0) && ((uintptr_t)b % 16 == 0) &&

@@ -311,30 +311,35 @@ class ROCMDataInterface : public DataInterface<T> {
 // ---- blas --------------------------------------------------------------------------------------
 // Stride rules of the reference's blas interface (tfcc/mkl/interfaces/tfcc_mklblasinterface.cpp:127-186):
 // a rank-2 operand against a batched one is shared by the whole batch (stride 0).
-class ROCMBlasInterface : public BlasInterface<float> {
-  static Variable<float> run(const Tensor<float>& a, const Tensor<float>& b, const Tensor<float>* bias) {
-    const size_t ra = a.shape().size(), rb = b.shape().size();
-    const unsigned m = a.shape(ra - 2), n = b.shape(rb - 1), k = a.shape(ra - 1);
-    uint64_t strideA = static_cast<uint64_t>(m) * k, strideB = static_cast<uint64_t>(n) * k;
-    if (ra != rb) {
-      if (ra == 2) strideA = 0;
-      if (rb == 2) strideB = 0;
-    }
-    std::vector<unsigned> s = ra > rb ? a.shape().toVector() : b.shape().toVector();
-    s[s.size() - 2] = m;
-    s[s.size() - 1] = n;
-    Variable<float> result{Shape(std::move(s))};
-    const unsigned batch = result.size() / (m * n);
-    check(tfcc_rocm_sgemm_strided_batched(current_stream(), a.data(), strideA, b.data(), strideB,
-                                          bias ? bias->data() : nullptr, result.data(),
-                                          static_cast<uint64_t>(m) * n, m, n, k, batch));
-    return result;
+// shared by the interface and by the fused forms of tfcc::rocm::blas
+Variable<float> rocm_sgemm(const Tensor<float>& a, const Tensor<float>& b, const Tensor<float>* bias,
+                           const Tensor<float>* residual, int activation) {
+  const size_t ra = a.shape().size(), rb = b.shape().size();
+  const unsigned m = a.shape(ra - 2), n = b.shape(rb - 1), k = a.shape(ra - 1);
+  uint64_t strideA = static_cast<uint64_t>(m) * k, strideB = static_cast<uint64_t>(n) * k;
+  if (ra != rb) {
+    if (ra == 2) strideA = 0;
+    if (rb == 2) strideB = 0;
   }
+  std::vector<unsigned> s = ra > rb ? a.shape().toVector() : b.shape().toVector();
+  s[s.size() - 2] = m;
+  s[s.size() - 1] = n;
+  Variable<float> result{Shape(std::move(s))};
+  if (residual && !(residual->shape() == result.shape())) throw InvalidArgumentError("residual and result don't match");
+  const unsigned batch = result.size() / (m * n);
+  check(tfcc_rocm_sgemm_fused(current_stream(), a.data(), strideA, b.data(), strideB, bias ? bias->data() : nullptr,
+                              residual ? residual->data() : nullptr, static_cast<uint64_t>(m) * n, result.data(),
+                              static_cast<uint64_t>(m) * n, m, n, k, batch, activation));
+  return result;
+}
 
+class ROCMBlasInterface : public BlasInterface<float> {
  public:
-  Variable<float> matmul(const Tensor<float>& a, const Tensor<float>& b) override { return run(a, b, nullptr); }
+  Variable<float> matmul(const Tensor<float>& a, const Tensor<float>& b) override {
+    return rocm_sgemm(a, b, nullptr, nullptr, 0);
+  }
   Variable<float> matmul(const Tensor<float>& a, const Tensor<float>& b, const Tensor<float>& bias) override {
-    return run(a, b, &bias);
+    return rocm_sgemm(a, b, &bias, nullptr, 0);
   }
 };
 
@@ -623,6 +628,33 @@ void bind_thread(unsigned deviceID) {
 
 void initialize_rocm() { bind_thread(0); }
 void initialize_rocm(unsigned deviceID) { bind_thread(deviceID); }
+
+// ---------------------------------------------------------------------------------------------
+// fused forms
+// ---------------------------------------------------------------------------------------------
+namespace rocm {
+namespace blas {
+Variable<float> matmul_fused(const Tensor<float>& a, const Tensor<float>& b, const Tensor<float>* bias,
+                             const Tensor<float>* residual, Activation activation) {
+  std::vector<unsigned> s = tfcc::blas::detail::check<float>(a, b, bias);
+  if (a.size() == 0 || b.size() == 0) return Variable<float>(Shape(std::move(s)));
+  if (dynamic_cast<ROCMDevice*>(Device::getThreadDefault()) == nullptr) throw NotImplementedError();
+  return rocm_sgemm(a, b, bias, residual, static_cast<int>(activation));
+}
+}  // namespace blas
+namespace math {
+Variable<float> softmax_div(const Tensor<float>& a, size_t axis, float divisor) {
+  if (axis >= a.shape().size()) throw InvalidArgumentError("invalid axis");
+  if (a.size() == 0) throw InvalidArgumentError("invalid tensor");
+  if (dynamic_cast<ROCMDevice*>(Device::getThreadDefault()) == nullptr) throw NotImplementedError();
+  if (axis + 1 != a.shape().size()) throw NotImplementedError("softmax over the last axis only");
+  Variable<float> r(a.shape());
+  const unsigned cols = a.shape(axis);
+  check(tfcc_rocm_softmax_div_f32(current_stream(), a.data(), a.size() / cols, cols, divisor, r.data()));
+  return r;
+}
+}  // namespace math
+}  // namespace rocm
 
 // ---------------------------------------------------------------------------------------------
 // quantized matmul

@@ -78,6 +78,22 @@ class HostSession : public Session {
 void initialize_host();
 
 namespace rocm {
+
+// Fused forms: what a caller would otherwise issue as consecutive operations, done in one kernel
+// with the same fp32 rounding after every step (results are bit-identical to the separate calls).
+// Backend-specific, like the quantized matmul: they need the ROCm device as the thread default.
+namespace blas {
+enum class Activation { NONE = 0, GELU = 1 };
+// activation(a * b + bias + residual); bias and residual may be null; residual has the result's shape.
+// Checks and shape rules of tfcc::blas::matmul.
+Variable<float> matmul_fused(const Tensor<float>& a, const Tensor<float>& b, const Tensor<float>* bias,
+                             const Tensor<float>* residual, Activation activation);
+}  // namespace blas
+namespace math {
+// softmax(a / divisor, axis)
+Variable<float> softmax_div(const Tensor<float>& a, size_t axis, float divisor);
+}  // namespace math
+
 namespace quantization {
 
 // tfcc::mkl::quantization::matmul (tfcc/mkl/operations/tfcc_mklquantization.cpp:71-203): same

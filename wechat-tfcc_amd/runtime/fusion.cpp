@@ -1,0 +1,166 @@
+// Build-time fusion of node sequences the ROCm backend can run as one kernel.  The reference ships
+// fused graphs as a second, offline-generated model (model.cpu.pb, tfcc_runtime/framework/model.cpp:
+// 74-76,311-322, operations/fusion/); here the plain graph is pattern-matched when it is built:
+//
+//   MatmulWithBias -> Gelu                 one GEMM with the activation in its tile store
+//   MatmulWithBias -> Add(other tensor)    one GEMM that also adds the other tensor (residual)
+//   Div(tensor, value) -> Softmax          one softmax pass that divides first
+//   Identity of a variable nobody else reads: the buffer is handed over instead of copied
+//
+// A producer is absorbed only when its output is a float VARIABLE symbol with exactly one consumer
+// that is not an output of the graph, and when every symbol of the graph has one producer.  Each
+// fused kernel rounds to fp32 after every original step, so results are bit-identical to the
+// unfused graph; when a run-time shape does not fit the fused form the steps run unfused.
+#include <unordered_map>
+
+#include "runtime.h"
+#include "tfcc_rocm_device.h"
+
+namespace tfcc {
+namespace runtime {
+
+namespace {
+
+bool is_op(const proto::Node& n, const char* message, size_t inputs) {
+  return n.version == 1 && n.typeUrl == type_url(message) && n.inputs.size() == inputs && n.outputs.size() == 1;
+}
+
+bool float_tensor(SymbolManager& sm, const std::string& name) {
+  if (!sm.has(name)) return false;
+  const SymbolInfo& info = sm.getSymbolInfo(name);
+  return info.dtype == FLOAT && is_tensor(info.stype);
+}
+
+bool float_variable(SymbolManager& sm, const std::string& name) {
+  if (!sm.has(name)) return false;
+  const SymbolInfo& info = sm.getSymbolInfo(name);
+  return info.dtype == FLOAT && info.stype == SymbolType::VARIABLE;
+}
+
+}  // namespace
+
+std::vector<FusionPlan> plan_fusions(const proto::Graph& g, SymbolManager& sm) {
+  std::vector<FusionPlan> plan(g.nodes.size());
+  std::unordered_map<std::string, size_t> producer;
+  std::unordered_map<std::string, std::vector<size_t>> consumers;
+  for (size_t i = 0; i < g.nodes.size(); ++i) {
+    for (const std::string& o : g.nodes[i].outputs) {
+      if (producer.count(o)) return plan;  // a symbol written twice: leave the graph as it is
+      producer[o] = i;
+    }
+    for (const std::string& in : g.nodes[i].inputs) consumers[in].push_back(i);
+  }
+  std::set<std::string> kept(g.outputs.begin(), g.outputs.end());
+  for (const std::string& in : g.inputs)
+    if (producer.count(in)) return plan;
+
+  // the node that alone produces `name` for node j, if absorbing it is allowed
+  auto sole_producer = [&](const std::string& name, size_t j, size_t& i) {
+    auto p = producer.find(name);
+    if (p == producer.end() || p->second >= j || kept.count(name)) return false;
+    if (consumers[name].size() != 1 || plan[p->second].kind != FusionPlan::NONE) return false;
+    if (!float_variable(sm, name)) return false;
+    i = p->second;
+    return true;
+  };
+  auto all_float_tensors = [&](const proto::Node& n) {
+    for (const std::string& s : n.inputs)
+      if (!float_tensor(sm, s)) return false;
+    return true;
+  };
+
+  for (size_t j = 0; j < g.nodes.size(); ++j) {
+    const proto::Node& n = g.nodes[j];
+    if (plan[j].kind != FusionPlan::NONE) continue;
+    if (!sm.has(n.outputs.empty() ? std::string() : n.outputs[0])) continue;
+    size_t i = 0;
+    if (is_op(n, "math.Gelu", 1) && float_variable(sm, n.outputs[0]) && sole_producer(n.inputs[0], j, i) &&
+        is_op(g.nodes[i], "math.MatmulWithBias", 3) && all_float_tensors(g.nodes[i])) {
+      plan[j] = {FusionPlan::MATMUL_GELU, i, 0};
+      plan[i] = {FusionPlan::ABSORBED, j, 0};
+    } else if (is_op(n, "math.Add", 2) && float_variable(sm, n.outputs[0]) && all_float_tensors(n)) {
+      for (unsigned side = 0; side < 2; ++side) {
+        if (sole_producer(n.inputs[side], j, i) && is_op(g.nodes[i], "math.MatmulWithBias", 3) &&
+            all_float_tensors(g.nodes[i]) && n.inputs[0] != n.inputs[1]) {
+          plan[j] = {FusionPlan::MATMUL_ADD, i, side};
+          plan[i] = {FusionPlan::ABSORBED, j, 0};
+          break;
+        }
+      }
+    } else if (is_op(n, "math.Softmax", 1) && float_variable(sm, n.outputs[0]) && sole_producer(n.inputs[0], j, i) &&
+               is_op(g.nodes[i], "math.Div", 2) && float_tensor(sm, g.nodes[i].inputs[0]) &&
+               sm.has(g.nodes[i].inputs[1]) && sm.getSymbolInfo(g.nodes[i].inputs[1]).dtype == FLOAT &&
+               is_value(sm.getSymbolInfo(g.nodes[i].inputs[1]).stype)) {
+      plan[j] = {FusionPlan::DIV_SOFTMAX, i, 0};
+      plan[i] = {FusionPlan::ABSORBED, j, 0};
+    } else if (is_op(n, "base.Identity", 1) && float_variable(sm, n.outputs[0]) && float_variable(sm, n.inputs[0]) &&
+               producer.count(n.inputs[0]) && producer[n.inputs[0]] < j && consumers[n.inputs[0]].size() == 1 &&
+               !kept.count(n.inputs[0])) {
+      plan[j] = {FusionPlan::MOVE_IDENTITY, j, 0};
+    }
+  }
+  return plan;
+}
+
+void emit_fused(const proto::Graph& g, const FusionPlan& f, size_t j, Graph& graph) {
+  SymbolManager& sm = graph.getSymbolManager();
+  const proto::Node& n = g.nodes[j];
+  Variable<float>* out = sm.getVariable(n.outputs[0], float());
+  if (f.kind == FusionPlan::MOVE_IDENTITY) {
+    Variable<float>* in = sm.getVariable(n.inputs[0], float());
+    graph.addStep([in, out] { *out = std::move(*in); });
+    return;
+  }
+  const proto::Node& p = g.nodes[f.partner];
+  if (f.kind == FusionPlan::DIV_SOFTMAX) {
+    const Tensor<float>* a = sm.getTensor(p.inputs[0], float());
+    const float* divisor = sm.getValue(p.inputs[1], float());
+    size_t axis = 0;
+    wire::Reader r(n.operation);
+    uint32_t field, type;
+    while (r.next(field, type)) {
+      if (field == 1 && type == 0) axis = static_cast<size_t>(r.varint());
+      else r.skip(type);
+    }
+    graph.addStep([a, divisor, axis, out] {
+      if (axis + 1 == a->shape().size()) {
+        *out = rocm::math::softmax_div(*a, axis, *divisor);
+      } else {
+        Variable<float> t = *a / *divisor;
+        *out = math::softmax(t, axis);
+      }
+    });
+    return;
+  }
+  const Tensor<float>* a = sm.getTensor(p.inputs[0], float());
+  const Tensor<float>* b = sm.getTensor(p.inputs[1], float());
+  const Tensor<float>* bias = sm.getTensor(p.inputs[2], float());
+  if (f.kind == FusionPlan::MATMUL_GELU) {
+    graph.addStep([a, b, bias, out] {
+      *out = rocm::blas::matmul_fused(*a, *b, bias, nullptr, rocm::blas::Activation::GELU);
+    });
+    return;
+  }
+  // MATMUL_ADD: the Add's other operand is the residual when it has the product's shape
+  const Tensor<float>* other = sm.getTensor(n.inputs[1 - f.side], float());
+  const bool productFirst = f.side == 0;
+  graph.addStep([a, b, bias, other, productFirst, out] {
+    const size_t ra = a->shape().size(), rb = b->shape().size();
+    bool fits = ra >= 2 && rb >= 2 && a->size() > 0 && b->size() > 0;
+    if (fits) {
+      std::vector<unsigned> s = ra >= rb ? a->shape().toVector() : b->shape().toVector();
+      s[s.size() - 2] = a->shape(ra - 2);
+      s[s.size() - 1] = b->shape(rb - 1);
+      fits = other->shape() == Shape(std::move(s));
+    }
+    if (fits) {
+      *out = rocm::blas::matmul_fused(*a, *b, bias, other, rocm::blas::Activation::NONE);
+    } else {
+      Variable<float> t = blas::matmul(*a, *b, *bias);
+      *out = productFirst ? t + *other : *other + t;
+    }
+  });
+}
+
+}  // namespace runtime
+}  // namespace tfcc

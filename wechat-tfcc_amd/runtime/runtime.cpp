@@ -393,6 +393,7 @@ std::vector<T>* SymbolManager::getVector(const std::string& name, T) {
 // graph
 // ---------------------------------------------------------------------------------------------------
 thread_local bool Graph::_recordDetailError = false;
+thread_local bool Graph::_fusion = true;
 
 namespace {
 void rocm_check(int status) {
@@ -418,9 +419,16 @@ Graph::~Graph() {
 void Graph::buildGraph() {
   if (_built) return;
   _steps.clear();
+  std::vector<FusionPlan> fusion(_proto.nodes.size());
+  if (_fusion && dynamic_cast<ROCMDevice*>(Device::getThreadDefault()) != nullptr) fusion = plan_fusions(_proto, *_symbols);
   for (size_t i = 0; i < _proto.nodes.size(); ++i) {
     const proto::Node& node = _proto.nodes[i];
     _currentNode = i;
+    if (fusion[i].kind == FusionPlan::ABSORBED) continue;
+    if (fusion[i].kind != FusionPlan::NONE) {
+      emit_fused(_proto, fusion[i], i, *this);
+      continue;
+    }
     bool accepted = false;
     for (auto& op : operations_for(node.typeUrl)) {
       if (!op->getOperationVersions().count(node.version)) continue;

@@ -265,6 +265,17 @@ class Operation {
 
 const std::vector<std::unique_ptr<Operation>>& operations_for(const std::string& typeUrl);
 
+// What the build-time fusion pass decided for one node: run it as written (NONE), skip it because a
+// later node runs it as part of a fused step (ABSORBED, partner = that node), or run it fused with
+// the producer `partner` of one of its inputs (side: which input of an Add the product is).
+struct FusionPlan {
+  enum Kind { NONE, ABSORBED, MATMUL_GELU, MATMUL_ADD, DIV_SOFTMAX, MOVE_IDENTITY } kind = NONE;
+  size_t partner = 0;
+  unsigned side = 0;
+};
+std::vector<FusionPlan> plan_fusions(const proto::Graph& graph, SymbolManager& symbols);
+void emit_fused(const proto::Graph& graphProto, const FusionPlan& plan, size_t node, Graph& graph);
+
 class Graph {
   Model& _model;
   const proto::Graph& _proto;
@@ -277,6 +288,7 @@ class Graph {
   size_t _currentNode = 0;
   bool _built = false;
   static thread_local bool _recordDetailError;
+  static thread_local bool _fusion;
 
   // replay state
   bool _replayWanted = false;
@@ -332,9 +344,12 @@ class Graph {
 
   SymbolManager& getSymbolManager() { return *_symbols; }
   Model& getModel() { return _model; }
+  size_t stepCount() const { return _steps.size(); }  // bound steps after building (fused nodes share one)
   // used by operations while the graph is being built
   void addStep(std::function<void()> step) { _steps.push_back(Step{std::move(step), _currentNode}); }
 
+  // graphs built afterwards on this thread fuse node sequences (default) or run every node as written
+  static void setFusionThreadLocal(bool enable) { _fusion = enable; }
   static void setRecordDetailErrorThreadLocal(bool enable) { _recordDetailError = enable; }
   static bool isRecordDetailError() { return _recordDetailError; }
 };

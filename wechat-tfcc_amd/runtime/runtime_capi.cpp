@@ -95,6 +95,17 @@ int tfcc_rocm_runtime_model_test(void* model, const void* npz, size_t len, int* 
   });
 }
 
+int tfcc_rocm_runtime_set_fusion(int enable) {
+  return guarded([&] { tfcc::runtime::Graph::setFusionThreadLocal(enable != 0); });
+}
+
+int tfcc_rocm_runtime_model_step_count(void* model, size_t* steps) {
+  return guarded([&] {
+    if (steps == nullptr) throw tfcc::InvalidArgumentError("null argument");
+    *steps = as_model(model).getEntranceGraph().stepCount();
+  });
+}
+
 int tfcc_rocm_runtime_model_set_replay(void* model, int enable) {
   return guarded([&] { as_model(model).getEntranceGraph().enableReplay(enable != 0); });
 }

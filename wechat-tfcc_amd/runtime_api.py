@@ -18,6 +18,8 @@ SYMBOLS = {
     "tfcc_rocm_runtime_model_run": (C.c_int, [_VP, _VP, C.c_size_t, C.POINTER(_VP), C.POINTER(C.c_size_t)]),
     "tfcc_rocm_runtime_buffer_free": (C.c_int, [_VP]),
     "tfcc_rocm_runtime_model_test": (C.c_int, [_VP, _VP, C.c_size_t, C.POINTER(C.c_int), C.POINTER(_VP)]),
+    "tfcc_rocm_runtime_set_fusion": (C.c_int, [C.c_int]),
+    "tfcc_rocm_runtime_model_step_count": (C.c_int, [_VP, C.POINTER(C.c_size_t)]),
     "tfcc_rocm_runtime_model_set_replay": (C.c_int, [_VP, C.c_int]),
     "tfcc_rocm_runtime_model_time": (C.c_int, [_VP, _VP, C.c_size_t, C.c_int, C.c_int, C.POINTER(C.c_double)]),
 }
@@ -51,6 +53,11 @@ def check(status):
 def initialize(host=False):
     """host=True binds the host-memory device (no compute) instead of the GPU"""
     check(lib().tfcc_rocm_runtime_initialize_host() if host else lib().tfcc_rocm_runtime_initialize())
+
+
+def set_fusion(enable):
+    """graphs built afterwards fuse node sequences (default) or run every node as written"""
+    check(lib().tfcc_rocm_runtime_set_fusion(1 if enable else 0))
 
 
 class Model:
@@ -92,6 +99,11 @@ class Model:
             return bool(passed.value), C.string_at(report).decode(errors="replace")
         finally:
             lib().tfcc_rocm_runtime_buffer_free(report)
+
+    def step_count(self):
+        n = C.c_size_t()
+        check(lib().tfcc_rocm_runtime_model_step_count(self._h, C.byref(n)))
+        return n.value
 
     def set_replay(self, enable):
         check(lib().tfcc_rocm_runtime_model_set_replay(self._h, 1 if enable else 0))
