@@ -161,7 +161,7 @@ def test_qgemm_requant_immediate_scalars(pkg, T):
 # ---- skinny (decode) shapes -------------------------------------------------------------------------
 
 @pytest.mark.parametrize("m", [1, 4, 8])
-@pytest.mark.parametrize("n,k", [(11008, 4096), (128, 64), (260, 80), (4096, 4000)])
+@pytest.mark.parametrize("n,k", [(11008, 4096), (128, 64), (260, 80), (4096, 4000), (176, 272), (1024, 8192), (512, 8320)])
 def test_gemv_against_oracle(pkg, T, m, n, k):
     print("gemv", m, n, k, flush=True)
     rng = np.random.default_rng(m + n + k)
