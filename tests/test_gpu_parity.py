@@ -327,6 +327,7 @@ def test_sgemm_exact_cases(pkg, T):
     # few tiles and a long K: several K groups per workgroup (x4, x2), with ragged K and edges
     ((1024, 768), (768, 768)), ((200, 1000), (1000, 300)), ((300, 300), (300, 500)), ((64, 516), (516, 64)),
     ((3, 70, 1028), (1028, 90)),
+    ((100, 600), (600, 200)), ((128, 768), (768, 3072)),   # 32x96 tiles, ragged edges
 ])
 def test_sgemm_shapes_against_oracle(pkg, T, shape_a, shape_b):
     """The four shape families of tfcc/test/blas.cpp:34-61 plus the benchmark's batched shapes."""

@@ -34,7 +34,6 @@ struct SgemmParams {
   unsigned tilesM, tilesN, tilesTotal, chunk;
 };
 
-constexpr int kThreads = 256;
 constexpr int BK = 32;
 constexpr int CH = BK / 4;  // 16-byte chunks per LDS row
 
@@ -46,8 +45,10 @@ __device__ __forceinline__ int swz(int row, int chunk) { return chunk ^ ((row >>
 // a fixed order at the end.  That is for products with few tiles and a long K, where one group per
 // CU could not hide the memory latency of its own loads.
 template <int WGM, int WGN, int MI, int NI, bool VEC, int KSPLIT>
-__global__ __launch_bounds__(kThreads * KSPLIT) void sgemm_kernel(const SgemmParams p) {
-  static_assert(WGM * WGN == 4, "four wavefronts per group");
+__global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_kernel(const SgemmParams p) {
+  constexpr int GW = WGM * WGN;      // wavefronts per group
+  constexpr int kThreads = GW * 64;  // threads per group
+  static_assert(GW == 4 || GW == 3, "three or four wavefronts per group");
   constexpr int BM = WGM * MI * 32, BN = WGN * NI * 32;
   constexpr int WM = MI * 32, WN = NI * 32;
   constexpr int A_TOTAL = BM * CH, B_TOTAL = (BN / 4) * CH;    // 128-bit chunks of A, 4x4 blocks of B
@@ -55,11 +56,12 @@ __global__ __launch_bounds__(kThreads * KSPLIT) void sgemm_kernel(const SgemmPar
   constexpr int B_ITEMS = (B_TOTAL + kThreads - 1) / kThreads;
 
   extern __shared__ __align__(16) float smemf[];
-  const int grp = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8));  // K group, wave-uniform
+  const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+  const int grp = wv / GW;  // K group, wave-uniform
   float* As = smemf + grp * 2 * (BM + BN) * BK;  // [2][BM][BK]
   float* Bs = As + 2 * BM * BK;                  // [2][BN][BK]
 
-  const int tid = threadIdx.x & 255, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x - grp * kThreads, lane = tid & 63, wave = wv - grp * GW;
   const int wm = wave / WGN, wn = wave % WGN;
 
   unsigned tm, tn, bi;
@@ -224,7 +226,7 @@ __global__ __launch_bounds__(kThreads * KSPLIT) void sgemm_kernel(const SgemmPar
     // partial tiles of groups 1 .. KSPLIT-1 go through LDS (the slab buffers are free after the last
     // barrier) and are added by group 0 in group order
     float* red = smemf;
-    const int slot = ((grp - 1) * 4 + wave) * MI * NI;
+    const int slot = ((grp - 1) * GW + wave) * MI * NI;
     if (grp > 0) {
 #pragma unroll
       for (int i = 0; i < MI; ++i)
@@ -243,7 +245,7 @@ __global__ __launch_bounds__(kThreads * KSPLIT) void sgemm_kernel(const SgemmPar
         for (int j = 0; j < NI; ++j)
 #pragma unroll
           for (int r = 0; r < 16; ++r)
-            acc[i][j][r] += red[((((q - 1) * 4 + wave) * MI * NI + i * NI + j) * 16 + r) * 64 + lane];
+            acc[i][j][r] += red[((((q - 1) * GW + wave) * MI * NI + i * NI + j) * 16 + r) * 64 + lane];
   }
 
   // ---- epilogue: + bias, store.  Lane (i, g) owns columns NI*i .. NI*i+NI-1 of the wavefront's
@@ -308,7 +310,7 @@ int launch(hipStream_t stream, SgemmParams p) {
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
     attrSet = true;
   }
-  hipLaunchKernelGGL(kern, dim3(p.chunk * 8), dim3(kThreads * KSPLIT), lds, stream, p);
+  hipLaunchKernelGGL(kern, dim3(p.chunk * 8), dim3(WGM * WGN * 64 * KSPLIT), lds, stream, p);
   return check_launch("sgemm");
 }
 
@@ -345,6 +347,10 @@ extern "C" int tfcc_rocm_sgemm_fused(void* stream, const float* a, uint64_t stri
     if (big >= 512) return launch<4, 1, 1, 4, true>(s, p);
     // few 64x64 tiles and a long K: several K groups per workgroup keep the CUs that have a tile busy
     const unsigned long long small = (unsigned long long)((m + 63) / 64) * ((n + 63) / 64) * batch;
+    // 32x96 tiles when they cover the 256 CUs in fewer tile-area rounds than 64x64 tiles would
+    const unsigned long long flat = (unsigned long long)((m + 31) / 32) * ((n + 95) / 96) * batch;
+    const bool preferFlat = ((flat + 255) / 256) * (32 * 96) < ((small + 255) / 256) * (64 * 64);
+    if (preferFlat && flat <= 320 && k >= 512) return launch<1, 3, 1, 1, true, 4>(s, p);
     if (small <= 320 && k >= 512) return launch<2, 2, 1, 1, true, 4>(s, p);
     if (small <= 640 && k >= 256) return launch<2, 2, 1, 1, true, 2>(s, p);
     return launch<2, 2, 1, 1, true>(s, p);
