@@ -101,6 +101,31 @@ int tfcc_rocm_sgemm_fused(void* stream, const float* a, uint64_t stride_a, const
                           uint64_t stride_residual, float* c, uint64_t stride_c, unsigned m,
                           unsigned n, unsigned k, unsigned batch, int activation);
 
+/* The general form: operands with their own row strides, a batch that is a grid of outer x inner
+ * entries with a stride each, and B optionally given transposed.  It lets a caller multiply
+ * permuted views of its tensors in place - e.g. the per-head matrices of a [batch, seq, heads, size]
+ * tensor (outer = batch, inner = heads, row stride heads * size), K^T taken straight from K
+ * (trans_b), a result written in [batch, seq, heads, size] order - where the reference materialises
+ * each permutation first with base::transpose (tfcc/core/operations/tfcc_base.cpp:124-134) because
+ * its matmul has no stride or transpose arguments (tfcc/core/operations/tfcc_blas.cpp:26-58).
+ * All strides are in elements.  A residual requires ldc == n and batch_inner == 1. */
+typedef struct tfcc_rocm_sgemm_desc {
+  const float* a;        /* [m, k], row stride lda */
+  const float* b;        /* [k, n], row stride ldb; with trans_b: [n, k], row stride ldb */
+  const float* bias;     /* [n] or NULL */
+  const float* residual; /* dense [batch][m, n] or NULL */
+  float* c;              /* [m, n], row stride ldc */
+  unsigned m, n, k;
+  unsigned lda, ldb, ldc;
+  int trans_b;
+  unsigned batch_outer, batch_inner;
+  uint64_t stride_a, stride_b, stride_c;                   /* between outer batch entries; 0 = shared */
+  uint64_t inner_stride_a, inner_stride_b, inner_stride_c; /* between inner batch entries */
+  uint64_t stride_residual;
+  int activation;        /* 0 none, 1 erf-form GELU */
+} tfcc_rocm_sgemm_desc;
+int tfcc_rocm_sgemm_general(void* stream, const tfcc_rocm_sgemm_desc* desc);
+
 /* ---------------------------------------------------------------------------------------------
  * Quantized uint8 x int8 -> int32 matmul.
  * Replaces _mkl_create_offset_matrix + _MKLQuantizationMatmulAVX256::quantizedMatmulColMajor,

@@ -243,8 +243,9 @@ def test_fused_graph_is_bit_identical_to_the_graph_as_written(mf, rt, dev):
         rt.set_fusion(True)
         fused = rt.Model(blob)
         got = fused.run({"hidden_states": x})["layer_output"]
-        # matmul+gelu, 2 x matmul+add and div+softmax each save one step
-        assert plain.step_count() - fused.step_count() == 4
+        # matmul+gelu, 2 x matmul+add and div+softmax each save one step, the four transposes around the
+        # two batched products are folded into them
+        assert plain.step_count() - fused.step_count() == 8
         assert np.array_equal(got, want)
         fused.set_replay(True)
         for _ in range(3):
@@ -264,6 +265,30 @@ def test_fused_graph_is_bit_identical_to_the_graph_as_written(mf, rt, dev):
         outs.append(rt.Model(mf.write_model([g], "g")).run({"a": av})[y])
     rt.set_fusion(True)
     assert np.array_equal(outs[0], outs[1])
+    # transposes around a batched product in layouts the strided kernel takes (k or n contiguous) and does
+    # not take (A with k strided: falls back to the nodes as written)
+    for perm_a, perm_b, perm_c in (([0, 2, 1, 3], [0, 2, 3, 1], None), ([0, 1, 3, 2], None, [0, 2, 1, 3]),
+                                   (None, [0, 2, 1, 3], [0, 2, 1, 3]), ([0, 2, 1, 3], [0, 2, 1, 3], [1, 0, 2, 3])):
+        g = mf.GraphBuilder("g")
+        shape_a = {None: [2, 3, 10, 8], (0, 2, 1, 3): [2, 10, 3, 8], (0, 1, 3, 2): [2, 3, 8, 10]}[perm_a and tuple(perm_a)]
+        shape_b = {None: [2, 3, 8, 12], (0, 2, 1, 3): [2, 8, 3, 12], (0, 2, 3, 1): [2, 12, 3, 8]}[perm_b and tuple(perm_b)]
+        a = g.input("a", mf.FLOAT, shape_a)
+        b = g.input("b", mf.FLOAT, shape_b)
+        y = g.matmul(g.transpose(a, perm_a) if perm_a else a, g.transpose(b, perm_b) if perm_b else b)
+        if perm_c:
+            y = g.transpose(y, perm_c)
+        g.output(y)
+        av = rng.normal(size=shape_a).astype(np.float32)
+        bv = rng.normal(size=shape_b).astype(np.float32)
+        outs = []
+        for enable in (False, True):
+            rt.set_fusion(enable)
+            outs.append(rt.Model(mf.write_model([g], "g")).run({"a": av, "b": bv})[y])
+        rt.set_fusion(True)
+        want = np.matmul(av.transpose(perm_a) if perm_a else av, bv.transpose(perm_b) if perm_b else bv)
+        want = want.transpose(perm_c) if perm_c else want
+        assert outs[0].shape == want.shape and np.array_equal(outs[0], outs[1])
+        assert rel_frobenius(outs[1], want) <= 1e-5
 
 
 @pytest.mark.gpu

@@ -39,6 +39,21 @@ class QGemmDesc(C.Structure):
     ]
 
 
+class SgemmDesc(C.Structure):
+    """tfcc_rocm_sgemm_desc"""
+    _fields_ = [
+        ("a", C.c_void_p), ("b", C.c_void_p), ("bias", C.c_void_p), ("residual", C.c_void_p), ("c", C.c_void_p),
+        ("m", C.c_uint), ("n", C.c_uint), ("k", C.c_uint),
+        ("lda", C.c_uint), ("ldb", C.c_uint), ("ldc", C.c_uint),
+        ("trans_b", C.c_int),
+        ("batch_outer", C.c_uint), ("batch_inner", C.c_uint),
+        ("stride_a", C.c_uint64), ("stride_b", C.c_uint64), ("stride_c", C.c_uint64),
+        ("inner_stride_a", C.c_uint64), ("inner_stride_b", C.c_uint64), ("inner_stride_c", C.c_uint64),
+        ("stride_residual", C.c_uint64),
+        ("activation", C.c_int),
+    ]
+
+
 # name -> (restype, argtypes): every symbol include/tfcc_rocm.h declares
 _VP, _U64, _U, _I, _F, _D, _I64 = C.c_void_p, C.c_uint64, C.c_uint, C.c_int, C.c_float, C.c_double, C.c_int64
 SYMBOLS = {
@@ -81,6 +96,7 @@ SYMBOLS = {
     "tfcc_rocm_graph_launch": (_I, [_VP, _VP]),
     "tfcc_rocm_graph_destroy": (_I, [_VP]),
     "tfcc_rocm_sgemm_fused": (_I, [_VP, _VP, _U64, _VP, _U64, _VP, _VP, _U64, _VP, _U64, _U, _U, _U, _U, _I]),
+    "tfcc_rocm_sgemm_general": (_I, [_VP, _VP]),
     "tfcc_rocm_softmax_div_f32": (_I, [_VP, _VP, _U64, _U, _F, _VP]),
     "tfcc_rocm_transform2_f32": (_I, [_VP, _VP, _U64, _F, _F, _VP]),
     "tfcc_rocm_binary_f32": (_I, [_VP, _I, _VP, _VP, _U64, _U64, _VP]),
@@ -173,6 +189,21 @@ def blas_matmul(a, b, bias=None):
                                                  _ptr(bias), _ptr(out), p["stride_c"], p["m"], p["n"], p["k"],
                                                  p["batch"]))
     return out
+
+
+def sgemm_general(a, b, c, m, n, k, lda, ldb, ldc, trans_b=False, batch_outer=1, batch_inner=1,
+                  strides=(0, 0, 0), inner_strides=(0, 0, 0), bias=None, activation=0):
+    """tfcc_rocm_sgemm_general on torch tensors used as raw buffers (all strides in elements)."""
+    d = SgemmDesc()
+    d.a, d.b, d.c, d.bias, d.residual = _ptr(a), _ptr(b), _ptr(c), _ptr(bias), None
+    d.m, d.n, d.k, d.lda, d.ldb, d.ldc = m, n, k, lda, ldb, ldc
+    d.trans_b = 1 if trans_b else 0
+    d.batch_outer, d.batch_inner = batch_outer, batch_inner
+    d.stride_a, d.stride_b, d.stride_c = strides
+    d.inner_stride_a, d.inner_stride_b, d.inner_stride_c = inner_strides
+    d.activation = activation
+    check(lib().tfcc_rocm_sgemm_general(_stream(), C.byref(d)))
+    return c
 
 
 def reduce_sum(a, row):

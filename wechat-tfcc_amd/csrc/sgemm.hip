@@ -28,7 +28,10 @@ struct SgemmParams {
   const float* bias;
   const float* residual;  // optional, laid out like C (batch stride strideR): added after the bias
   float* C;
-  unsigned long long strideA, strideB, strideC, strideR;
+  unsigned long long strideA, strideB, strideC, strideR;  // between outer batch entries (elements)
+  unsigned long long innerA, innerB, innerC;              // between inner batch entries
+  unsigned batchInner;    // batch entry bi = (bi / batchInner, bi % batchInner); 1 for a flat batch
+  unsigned lda, ldb, ldc; // row strides of A, of B (of B^T when transposed) and of C, in elements
   int act;                // 0 none, 1 erf-form GELU applied last
   unsigned M, N, K, batch;
   unsigned tilesM, tilesN, tilesTotal, chunk;
@@ -44,14 +47,16 @@ __device__ __forceinline__ int swz(int row, int chunk) { return chunk ^ ((row >>
 // q + KSPLIT, ... through LDS buffers of its own and the partial tiles are added up through LDS in
 // a fixed order at the end.  That is for products with few tiles and a long K, where one group per
 // CU could not hide the memory latency of its own loads.
-template <int WGM, int WGN, int MI, int NI, bool VEC, int KSPLIT>
+// TRANSB: B is given as B^T, an [N, K] row-major matrix (k contiguous), and is staged like A.
+template <int WGM, int WGN, int MI, int NI, bool VEC, int KSPLIT, bool TRANSB>
 __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_kernel(const SgemmParams p) {
   constexpr int GW = WGM * WGN;      // wavefronts per group
   constexpr int kThreads = GW * 64;  // threads per group
   static_assert(GW == 4 || GW == 3, "three or four wavefronts per group");
   constexpr int BM = WGM * MI * 32, BN = WGN * NI * 32;
   constexpr int WM = MI * 32, WN = NI * 32;
-  constexpr int A_TOTAL = BM * CH, B_TOTAL = (BN / 4) * CH;    // 128-bit chunks of A, 4x4 blocks of B
+  constexpr int A_TOTAL = BM * CH;                              // 128-bit chunks of A
+  constexpr int B_TOTAL = TRANSB ? BN * CH : (BN / 4) * CH;     // chunks of B^T, or 4x4 blocks of B
   constexpr int A_ITEMS = (A_TOTAL + kThreads - 1) / kThreads;  // per thread
   constexpr int B_ITEMS = (B_TOTAL + kThreads - 1) / kThreads;
 
@@ -83,8 +88,10 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_kernel(const Sg
   }
   const unsigned m0 = tm * BM, n0 = tn * BN;
   const unsigned M = p.M, N = p.N, K = p.K;
-  const float* __restrict__ A = p.A + (size_t)bi * p.strideA;
-  const float* __restrict__ B = p.B + (size_t)bi * p.strideB;
+  const unsigned bo = bi / p.batchInner, bn = bi - bo * p.batchInner;
+  const float* __restrict__ A = p.A + (size_t)bo * p.strideA + (size_t)bn * p.innerA;
+  const float* __restrict__ B = p.B + (size_t)bo * p.strideB + (size_t)bn * p.innerB;
+  const unsigned lda = p.lda, ldb = p.ldb, ldc = p.ldc;
 
   v16f acc[MI][NI];
 #pragma unroll
@@ -95,15 +102,15 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_kernel(const Sg
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   v4f aReg[A_ITEMS];
-  v4f bReg[B_ITEMS][4];
+  v4f bReg[B_ITEMS][TRANSB ? 1 : 4];
 
   // Vector path: raw buffer loads, an offset past the end of the operand reads zero (rows >= M of
   // A, rows >= K of B).  The k tail of an A row is zeroed explicitly: it would otherwise meet the
   // zero rows of B as garbage that may be Inf/NaN.
   const __amdgpu_buffer_rsrc_t rsrcA =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(A), 0, VEC ? (int)(M * K * 4u) : 0, 0x00020000);
-  const __amdgpu_buffer_rsrc_t rsrcB =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(B), 0, VEC ? (int)(K * N * 4u) : 0, 0x00020000);
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<float*>(A), 0, VEC ? (int)(((M - 1) * lda + K) * 4u) : 0, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rsrcB = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float*>(B), 0, VEC ? (int)((TRANSB ? (N - 1) * ldb + K : (K - 1) * ldb + N) * 4u) : 0, 0x00020000);
 
   auto loadA = [&](unsigned k0) {
 #pragma unroll
@@ -116,7 +123,7 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_kernel(const Sg
       if constexpr (VEC) {
         // Only the slab that crosses the end of K masks its values: a select on every loaded value
         // would make the compiler wait for the load right here instead of after the matrix ops.
-        v = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rsrcA, (gr * K + gk) * 4u, 0, 0));
+        v = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rsrcA, (gr * lda + gk) * 4u, 0, 0));
         if (k0 + BK > K) {
           asm volatile("" ::: "memory");  // keeps this a real (wave-uniform) branch
           v = gk < K ? v : v4f{0.f, 0.f, 0.f, 0.f};
@@ -125,7 +132,7 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_kernel(const Sg
         if (gr < M) {
 #pragma unroll
           for (int q = 0; q < 4; ++q)
-            if (gk + q < K) v[q] = A[(size_t)gr * K + gk + q];
+            if (gk + q < K) v[q] = A[(size_t)gr * lda + gk + q];
         }
       }
       aReg[it] = v;
@@ -136,21 +143,41 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_kernel(const Sg
     for (int it = 0; it < B_ITEMS; ++it) {
       const int w = tid + it * kThreads;
       if (B_TOTAL % kThreads != 0 && w >= B_TOTAL) break;
-      const int nq = w % (BN / 4), kq = w / (BN / 4);
-      const unsigned gn = n0 + nq * 4, gk = k0 + kq * 4;
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
+      if constexpr (TRANSB) {
+        const int row = w / CH, ch = w % CH;
+        const unsigned gn = n0 + row, gk = k0 + ch * 4;
         v4f v = {0.f, 0.f, 0.f, 0.f};
         if constexpr (VEC) {
-          v = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rsrcB, ((gk + q) * N + gn) * 4u, 0, 0));
+          v = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rsrcB, (gn * ldb + gk) * 4u, 0, 0));
+          if (k0 + BK > K) {
+            asm volatile("" ::: "memory");  // as for A: a real branch, taken by the last slab only
+            v = gk < K ? v : v4f{0.f, 0.f, 0.f, 0.f};
+          }
         } else {
-          if (gk + q < K) {
+          if (gn < N) {
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-              if (gn + e < N) v[e] = B[(size_t)(gk + q) * N + gn + e];
+            for (int q = 0; q < 4; ++q)
+              if (gk + q < K) v[q] = B[(size_t)gn * ldb + gk + q];
           }
         }
-        bReg[it][q] = v;
+        bReg[it][0] = v;
+      } else {
+        const int nq = w % (BN / 4), kq = w / (BN / 4);
+        const unsigned gn = n0 + nq * 4, gk = k0 + kq * 4;
+#pragma unroll
+        for (int q = 0; q < (TRANSB ? 1 : 4); ++q) {
+          v4f v = {0.f, 0.f, 0.f, 0.f};
+          if constexpr (VEC) {
+            v = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rsrcB, ((gk + q) * ldb + gn) * 4u, 0, 0));
+          } else {
+            if (gk + q < K) {
+#pragma unroll
+              for (int e = 0; e < 4; ++e)
+                if (gn + e < N) v[e] = B[(size_t)(gk + q) * ldb + gn + e];
+            }
+          }
+          bReg[it][q] = v;
+        }
       }
     }
   };
@@ -168,14 +195,21 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_kernel(const Sg
     for (int it = 0; it < B_ITEMS; ++it) {
       const int w = tid + it * kThreads;
       if (B_TOTAL % kThreads != 0 && w >= B_TOTAL) break;
-      const int nq = w % (BN / 4), kq = w / (BN / 4);
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int n = nq * 4 + j;
+      if constexpr (TRANSB) {
+        const int n = w / CH, ch = w % CH;
         const int wnn = n / WN, within = n % WN;
         const int row = wnn * WN + (within % NI) * 32 + within / NI;
-        v4f v = {bReg[it][0][j], bReg[it][1][j], bReg[it][2][j], bReg[it][3][j]};
-        *reinterpret_cast<v4f*>(bs + row * BK + swz(row, kq) * 4) = v;
+        *reinterpret_cast<v4f*>(bs + row * BK + swz(row, ch) * 4) = bReg[it][0];
+      } else {
+        const int nq = w % (BN / 4), kq = w / (BN / 4);
+#pragma unroll
+        for (int j = 0; j < (TRANSB ? 1 : 4); ++j) {
+          const int n = nq * 4 + j;
+          const int wnn = n / WN, within = n % WN;
+          const int row = wnn * WN + (within % NI) * 32 + within / NI;
+          v4f v = {bReg[it][0][j], bReg[it][TRANSB ? 0 : 1][j], bReg[it][TRANSB ? 0 : 2][j], bReg[it][TRANSB ? 0 : 3][j]};
+          *reinterpret_cast<v4f*>(bs + row * BK + swz(row, kq) * 4) = v;
+        }
       }
     }
   };
@@ -250,8 +284,8 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_kernel(const Sg
 
   // ---- epilogue: + bias, store.  Lane (i, g) owns columns NI*i .. NI*i+NI-1 of the wavefront's
   // column range and rows 8*(r/4) + 4*g + r%4 of each 32-row block.
-  float* __restrict__ C = p.C + (size_t)bi * p.strideC;
-  const float* __restrict__ R = p.residual ? p.residual + (size_t)bi * p.strideR : nullptr;
+  float* __restrict__ C = p.C + (size_t)bo * p.strideC + (size_t)bn * p.innerC;
+  const float* __restrict__ R = p.residual ? p.residual + (size_t)bi * p.strideR : nullptr;  // dense, flat batch
   const int act = p.act;
   const unsigned gcol = n0 + wn * WN + NI * lrow;
   float bv[NI];
@@ -267,11 +301,12 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_kernel(const Sg
       float v[NI];
 #pragma unroll
       for (int j = 0; j < NI; ++j) v[j] = acc[i][j][r] + bv[j];
-      const size_t off = (size_t)grow * N + gcol;
+      const size_t off = (size_t)grow * ldc + gcol;
       if (R) {
+        const size_t roff = (size_t)grow * N + gcol;
 #pragma unroll
         for (int j = 0; j < NI; ++j)
-          if (gcol + j < N) v[j] += R[off + j];
+          if (gcol + j < N) v[j] += R[roff + j];
       }
       if (act == 1) {
         // same expression as the stand-alone GELU kernel, so that fusing changes no bit
@@ -292,7 +327,7 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_kernel(const Sg
   }
 }
 
-template <int WGM, int WGN, int MI, int NI, bool VEC, int KSPLIT = 1>
+template <int WGM, int WGN, int MI, int NI, bool VEC, int KSPLIT = 1, bool TRANSB = false>
 int launch(hipStream_t stream, SgemmParams p) {
   constexpr int BM = WGM * MI * 32, BN = WGN * NI * 32;
   p.tilesM = (p.M + BM - 1) / BM;
@@ -303,7 +338,7 @@ int launch(hipStream_t stream, SgemmParams p) {
   p.chunk = (p.tilesTotal + 7) / 8;
   constexpr size_t lds = KSPLIT * 2 * (size_t)(BM + BN) * BK * sizeof(float);
   static_assert(lds <= 160 * 1024 && (size_t)(KSPLIT - 1) * BM * BN * sizeof(float) <= lds, "LDS budget");
-  auto kern = sgemm_kernel<WGM, WGN, MI, NI, VEC, KSPLIT>;
+  auto kern = sgemm_kernel<WGM, WGN, MI, NI, VEC, KSPLIT, TRANSB>;
   static bool attrSet = false;
   if (!attrSet) {
     TFCC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
@@ -330,17 +365,50 @@ extern "C" int tfcc_rocm_sgemm_fused(void* stream, const float* a, uint64_t stri
                                      uint64_t stride_b, const float* bias, const float* residual,
                                      uint64_t stride_residual, float* c, uint64_t stride_c, unsigned m,
                                      unsigned n, unsigned k, unsigned batch, int activation) {
-  TFCC_REQUIRE(a && b && c, "sgemm: null operand");
-  TFCC_REQUIRE(m > 0 && n > 0 && k > 0 && batch > 0, "sgemm: empty operand");
-  TFCC_REQUIRE(activation == 0 || activation == 1, "sgemm: unknown activation %d", activation);
+  tfcc_rocm_sgemm_desc d{};
+  d.a = a; d.b = b; d.bias = bias; d.residual = residual; d.c = c;
+  d.m = m; d.n = n; d.k = k;
+  d.lda = k; d.ldb = n; d.ldc = n;
+  d.batch_outer = batch; d.batch_inner = 1;
+  d.stride_a = stride_a; d.stride_b = stride_b; d.stride_c = stride_c; d.stride_residual = stride_residual;
+  d.activation = activation;
+  return tfcc_rocm_sgemm_general(stream, &d);
+}
+
+extern "C" int tfcc_rocm_sgemm_general(void* stream, const tfcc_rocm_sgemm_desc* d) {
+  TFCC_REQUIRE(d != nullptr, "sgemm: null descriptor");
+  TFCC_REQUIRE(d->a && d->b && d->c, "sgemm: null operand");
+  TFCC_REQUIRE(d->m > 0 && d->n > 0 && d->k > 0 && d->batch_outer > 0 && d->batch_inner > 0, "sgemm: empty operand");
+  TFCC_REQUIRE(d->activation == 0 || d->activation == 1, "sgemm: unknown activation %d", d->activation);
+  const unsigned m = d->m, n = d->n, k = d->k;
+  TFCC_REQUIRE(d->lda >= k && d->ldc >= n && d->ldb >= (d->trans_b ? k : n), "sgemm: row stride shorter than a row");
+  const unsigned long long batch64 = (unsigned long long)d->batch_outer * d->batch_inner;
+  TFCC_REQUIRE(batch64 < (1ull << 31), "sgemm: too many batch entries");
+  TFCC_REQUIRE(!d->residual || (d->ldc == n && d->batch_inner == 1), "sgemm: a residual needs a dense result");
   SgemmParams p{};
-  p.A = a; p.B = b; p.bias = bias; p.C = c; p.residual = residual; p.strideR = stride_residual; p.act = activation;
-  p.strideA = stride_a; p.strideB = stride_b; p.strideC = stride_c;
-  p.M = m; p.N = n; p.K = k; p.batch = batch;
-  const bool vec = (k % 4 == 0) && (n % 4 == 0) && ((uintptr_t)a % 16 == 0) && ((uintptr_t)b % 16 == 0) &&
-                   ((uintptr_t)c % 16 == 0) && (stride_a % 4 == 0) && (stride_b % 4 == 0) && (stride_c % 4 == 0) &&
-                   ((unsigned long long)m * k < (1ull << 30)) && (((unsigned long long)k + 256) * n + 1024 < (1ull << 30));
+  p.A = d->a; p.B = d->b; p.bias = d->bias; p.C = d->c; p.residual = d->residual; p.strideR = d->stride_residual;
+  p.act = d->activation;
+  p.strideA = d->stride_a; p.strideB = d->stride_b; p.strideC = d->stride_c;
+  p.innerA = d->inner_stride_a; p.innerB = d->inner_stride_b; p.innerC = d->inner_stride_c;
+  p.batchInner = d->batch_inner;
+  p.lda = d->lda; p.ldb = d->ldb; p.ldc = d->ldc;
+  p.M = m; p.N = n; p.K = k; p.batch = (unsigned)batch64;
+  const unsigned batch = p.batch;
+  const bool tb = d->trans_b != 0;
+  const unsigned long long rowsB = tb ? n : k, colsB = tb ? k : n;  // B as stored
+  const bool vec = (k % 4 == 0) && (n % 4 == 0) && ((uintptr_t)d->a % 16 == 0) && ((uintptr_t)d->b % 16 == 0) &&
+                   ((uintptr_t)d->c % 16 == 0) && (d->lda % 4 == 0) && (d->ldb % 4 == 0) && (d->ldc % 4 == 0) &&
+                   (p.strideA % 4 == 0) && (p.strideB % 4 == 0) && (p.strideC % 4 == 0) && (p.innerA % 4 == 0) &&
+                   (p.innerB % 4 == 0) && (p.innerC % 4 == 0) &&
+                   (((unsigned long long)m + 256) * d->lda + k + 256 < (1ull << 30)) &&
+                   ((rowsB + 256) * d->ldb + colsB + 1024 < (1ull << 30));
   hipStream_t s = as_stream(stream);
+  if (tb) {
+    if (vec) return launch<2, 2, 1, 1, true, 1, true>(s, p);
+    TFCC_REQUIRE((unsigned long long)m * d->ldc < (1ull << 32) && (unsigned long long)m * d->lda < (1ull << 32) &&
+                 rowsB * d->ldb < (1ull << 32), "sgemm: operand larger than 2^32 elements");
+    return launch<2, 2, 1, 1, false, 1, true>(s, p);
+  }
   // 128x128 tiles once there are enough of them to fill the 256 CUs twice over, else 64x64
   const unsigned long long big = (unsigned long long)((m + 127) / 128) * ((n + 127) / 128) * batch;
   if (vec) {
@@ -355,7 +423,7 @@ extern "C" int tfcc_rocm_sgemm_fused(void* stream, const float* a, uint64_t stri
     if (small <= 640 && k >= 256) return launch<2, 2, 1, 1, true, 2>(s, p);
     return launch<2, 2, 1, 1, true>(s, p);
   }
-  TFCC_REQUIRE((unsigned long long)m * n < (1ull << 32) && (unsigned long long)m * k < (1ull << 32) &&
-               (unsigned long long)k * n < (1ull << 32), "sgemm: operand larger than 2^32 elements");
+  TFCC_REQUIRE((unsigned long long)m * d->ldc < (1ull << 32) && (unsigned long long)m * d->lda < (1ull << 32) &&
+               rowsB * d->ldb < (1ull << 32), "sgemm: operand larger than 2^32 elements");
   return launch<2, 2, 1, 1, false>(s, p);
 }

@@ -641,6 +641,87 @@ Variable<float> matmul_fused(const Tensor<float>& a, const Tensor<float>& b, con
   if (dynamic_cast<ROCMDevice*>(Device::getThreadDefault()) == nullptr) throw NotImplementedError();
   return rocm_sgemm(a, b, bias, residual, static_cast<int>(activation));
 }
+namespace {
+struct PermutedView {
+  unsigned dims[4];
+  uint64_t strides[4];
+};
+// dims and element strides of transpose(t, perm) seen on t's dense storage
+PermutedView permuted_view(const Shape& shape, const std::vector<size_t>& perm) {
+  if (shape.size() != 4 || (!perm.empty() && perm.size() != 4)) throw NotImplementedError("matmul_permuted: rank 4 only");
+  uint64_t dense[4];
+  uint64_t acc = 1;
+  for (int i = 3; i >= 0; --i) {
+    dense[i] = acc;
+    acc *= shape[i];
+  }
+  bool seen[4] = {false, false, false, false};
+  PermutedView v;
+  for (size_t i = 0; i < 4; ++i) {
+    const size_t src = perm.empty() ? i : perm[i];
+    if (src >= 4 || seen[src]) throw InvalidArgumentError("invalid perm");
+    seen[src] = true;
+    v.dims[i] = shape[src];
+    v.strides[i] = dense[src];
+  }
+  return v;
+}
+}  // namespace
+
+Variable<float> matmul_permuted(const Tensor<float>& a, const std::vector<size_t>& permA, const Tensor<float>& b,
+                                const std::vector<size_t>& permB, const std::vector<size_t>& permC) {
+  if (dynamic_cast<ROCMDevice*>(Device::getThreadDefault()) == nullptr) throw NotImplementedError();
+  const PermutedView va = permuted_view(a.shape(), permA), vb = permuted_view(b.shape(), permB);
+  if (va.dims[0] != vb.dims[0] || va.dims[1] != vb.dims[1] || va.dims[3] != vb.dims[2]) throw InvalidArgumentError("shape invalid");
+  if (a.size() == 0 || b.size() == 0) throw NotImplementedError("matmul_permuted: empty operand");
+  const unsigned m = va.dims[2], k = va.dims[3], n = vb.dims[3];
+  // the result tensor: dims of [B0, B1, m, n] permuted by permC, dense
+  const unsigned logical[4] = {va.dims[0], va.dims[1], m, n};
+  std::vector<unsigned> outDims(4);
+  uint64_t cStride[4] = {0, 0, 0, 0};
+  {
+    bool seen[4] = {false, false, false, false};
+    for (size_t p = 0; p < 4; ++p) {
+      const size_t src = permC.empty() ? p : permC[p];
+      if ((!permC.empty() && permC.size() != 4) || src >= 4 || seen[src]) throw InvalidArgumentError("invalid perm");
+      seen[src] = true;
+      outDims[p] = logical[src];
+    }
+    uint64_t acc = 1;
+    for (int p = 3; p >= 0; --p) {
+      cStride[permC.empty() ? p : permC[p]] = acc;
+      acc *= outDims[p];
+    }
+  }
+  if (va.strides[3] != 1 && k != 1) throw NotImplementedError("matmul_permuted: k is not contiguous in a");
+  if (cStride[3] != 1 && n != 1) throw NotImplementedError("matmul_permuted: n is not contiguous in the result");
+  tfcc_rocm_sgemm_desc d{};
+  if (vb.strides[3] == 1 || n == 1) {
+    d.trans_b = 0;
+    d.ldb = static_cast<unsigned>(vb.strides[2]);
+  } else if (vb.strides[2] == 1 || k == 1) {
+    d.trans_b = 1;
+    d.ldb = static_cast<unsigned>(vb.strides[3]);
+  } else {
+    throw NotImplementedError("matmul_permuted: neither k nor n is contiguous in b");
+  }
+  d.lda = static_cast<unsigned>(va.strides[2]);
+  d.ldc = static_cast<unsigned>(cStride[2]);
+  // a dimension of extent 1 may carry any stride: give it the smallest valid one
+  if (m == 1) { d.lda = std::max(d.lda, k); d.ldc = std::max(d.ldc, n); }
+  if (d.lda < k) d.lda = k;
+  if (d.ldc < n) d.ldc = n;
+  if (d.ldb < (d.trans_b ? k : n)) d.ldb = d.trans_b ? k : n;
+  Variable<float> result{Shape(outDims)};
+  d.a = a.data(); d.b = b.data(); d.c = result.data();
+  d.m = m; d.n = n; d.k = k;
+  d.batch_outer = logical[0]; d.batch_inner = logical[1];
+  d.stride_a = va.strides[0]; d.inner_stride_a = va.strides[1];
+  d.stride_b = vb.strides[0]; d.inner_stride_b = vb.strides[1];
+  d.stride_c = cStride[0]; d.inner_stride_c = cStride[1];
+  check(tfcc_rocm_sgemm_general(current_stream(), &d));
+  return result;
+}
 }  // namespace blas
 namespace math {
 Variable<float> softmax_div(const Tensor<float>& a, size_t axis, float divisor) {

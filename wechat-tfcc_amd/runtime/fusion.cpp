@@ -5,6 +5,7 @@
 //   MatmulWithBias -> Gelu                 one GEMM with the activation in its tile store
 //   MatmulWithBias -> Add(other tensor)    one GEMM that also adds the other tensor (residual)
 //   Div(tensor, value) -> Softmax          one softmax pass that divides first
+//   Transpose -> Matmul -> Transpose       a batched product that walks the permuted tensors in place
 //   Identity of a variable nobody else reads: the buffer is handed over instead of copied
 //
 // A producer is absorbed only when its output is a float VARIABLE symbol with exactly one consumer
@@ -93,6 +94,27 @@ std::vector<FusionPlan> plan_fusions(const proto::Graph& g, SymbolManager& sm) {
                is_value(sm.getSymbolInfo(g.nodes[i].inputs[1]).stype)) {
       plan[j] = {FusionPlan::DIV_SOFTMAX, i, 0};
       plan[i] = {FusionPlan::ABSORBED, j, 0};
+    } else if (is_op(n, "math.Matmul", 2) && float_variable(sm, n.outputs[0]) && all_float_tensors(n)) {
+      FusionPlan f;
+      f.kind = FusionPlan::MATMUL_PERMUTED;
+      size_t t = 0;
+      if (sole_producer(n.inputs[0], j, t) && is_op(g.nodes[t], "base.Transpose", 1) && float_tensor(sm, g.nodes[t].inputs[0]))
+        f.transposeA = t;
+      if (n.inputs[1] != n.inputs[0] && sole_producer(n.inputs[1], j, t) && is_op(g.nodes[t], "base.Transpose", 1) &&
+          float_tensor(sm, g.nodes[t].inputs[0]))
+        f.transposeB = t;
+      const std::string& out = n.outputs[0];
+      if (!kept.count(out) && consumers[out].size() == 1 && consumers[out][0] > j) {
+        const size_t c = consumers[out][0];
+        if (plan[c].kind == FusionPlan::NONE && is_op(g.nodes[c], "base.Transpose", 1) &&
+            float_variable(sm, g.nodes[c].outputs[0]))
+          f.transposeC = c;
+      }
+      if (f.transposeA != FusionPlan::kNoNode || f.transposeB != FusionPlan::kNoNode || f.transposeC != FusionPlan::kNoNode) {
+        plan[j] = f;
+        for (size_t t2 : {f.transposeA, f.transposeB, f.transposeC})
+          if (t2 != FusionPlan::kNoNode) plan[t2] = {FusionPlan::ABSORBED, j, 0};
+      }
     } else if (is_op(n, "base.Identity", 1) && float_variable(sm, n.outputs[0]) && float_variable(sm, n.inputs[0]) &&
                producer.count(n.inputs[0]) && producer[n.inputs[0]] < j && consumers[n.inputs[0]].size() == 1 &&
                !kept.count(n.inputs[0])) {
@@ -102,9 +124,48 @@ std::vector<FusionPlan> plan_fusions(const proto::Graph& g, SymbolManager& sm) {
   return plan;
 }
 
+namespace {
+std::vector<size_t> transpose_perm(const proto::Node& n) {
+  std::vector<size_t> perm;
+  wire::Reader r(n.operation);
+  uint32_t field, type;
+  while (r.next(field, type)) {
+    if (field == 1) r.repeatedVarint(type, perm);
+    else r.skip(type);
+  }
+  return perm;
+}
+}  // namespace
+
 void emit_fused(const proto::Graph& g, const FusionPlan& f, size_t j, Graph& graph) {
   SymbolManager& sm = graph.getSymbolManager();
   const proto::Node& n = g.nodes[j];
+  if (f.kind == FusionPlan::MATMUL_PERMUTED) {
+    const bool ta = f.transposeA != FusionPlan::kNoNode, tb = f.transposeB != FusionPlan::kNoNode,
+               tc = f.transposeC != FusionPlan::kNoNode;
+    const Tensor<float>* a = sm.getTensor(ta ? g.nodes[f.transposeA].inputs[0] : n.inputs[0], float());
+    const Tensor<float>* b = sm.getTensor(tb ? g.nodes[f.transposeB].inputs[0] : n.inputs[1], float());
+    Variable<float>* result = sm.getVariable(tc ? g.nodes[f.transposeC].outputs[0] : n.outputs[0], float());
+    const std::vector<size_t> pa = ta ? transpose_perm(g.nodes[f.transposeA]) : std::vector<size_t>();
+    const std::vector<size_t> pb = tb ? transpose_perm(g.nodes[f.transposeB]) : std::vector<size_t>();
+    const std::vector<size_t> pc = tc ? transpose_perm(g.nodes[f.transposeC]) : std::vector<size_t>();
+    graph.addStep([a, b, result, pa, pb, pc, ta, tb, tc] {
+      try {
+        *result = rocm::blas::matmul_permuted(*a, pa, *b, pb, pc);
+        return;
+      } catch (NotImplementedError&) {
+        // a layout the strided kernel does not take: run the nodes as written
+      }
+      Variable<float> xa, xb;
+      if (ta) xa = base::transpose(*a, pa);
+      if (tb) xb = base::transpose(*b, pb);
+      Variable<float> c = blas::matmul(ta ? static_cast<const Tensor<float>&>(xa) : *a,
+                                       tb ? static_cast<const Tensor<float>&>(xb) : *b);
+      if (tc) *result = base::transpose(c, pc);
+      else *result = std::move(c);
+    });
+    return;
+  }
   Variable<float>* out = sm.getVariable(n.outputs[0], float());
   if (f.kind == FusionPlan::MOVE_IDENTITY) {
     Variable<float>* in = sm.getVariable(n.inputs[0], float());
