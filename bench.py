@@ -202,6 +202,29 @@ def bench_other(torch, pkg, dev, steps, warmup, c3):
         out["c5_int8_gemv_m%d_4096x11008" % m] = {"ms": round(ms, 5), "gbs": round(gbs, 1),
                                                    "frac_hbm": round(gbs / PEAK_HBM_GBS, 4),
                                                    "gops": round(2.0 * m * n * k / ms / 1e6, 1)}
+    # the same decode shapes on weights packed once (column slabs in matrix-core operand order)
+    packs = [pkg.gemv_pack(x) for x in bs]
+    for m in (1, 4, 8):
+        am = t(rng.integers(0, 256, (m, k), dtype=np.uint8))
+        rsm = pkg.reduce_sum(am, True)
+        acc = torch.empty((m, n), dtype=torch.int32, device=dev)
+        f32 = torch.empty((m, n), dtype=torch.float32, device=dev)
+        idx = [0]
+
+        def step():
+            i = idx[0] % sets
+            idx[0] += 1
+            st = lib.tfcc_rocm_gemv_u8s8s32_packed(stream, am.data_ptr(), packs[i].data_ptr(), rsm.data_ptr(),
+                                                   css[i].data_ptr(), -128, 0, m, n, k, acc.data_ptr(), 0.02,
+                                                   scale_b.data_ptr(), f32.data_ptr())
+            if st != 0:
+                pkg.check(st)
+        ms = time_launches(torch, step, max(steps, 50), warmup)
+        nbytes = k * n + m * k + 4 * n + 4 * m * n
+        gbs = nbytes / ms / 1e6
+        out["c5_int8_gemv_packed_m%d_4096x11008" % m] = {"ms": round(ms, 5), "gbs": round(gbs, 1),
+                                                          "frac_hbm": round(gbs / PEAK_HBM_GBS, 4)}
+    del packs
 
     # C4: one BERT-base encoder layer through the model runtime (fp32, batch 8, seq 128); the entrance
     # graph alone is timed with events on the runtime's stream, tensors resident in HBM

@@ -184,6 +184,19 @@ int tfcc_rocm_gemv_u8s8s32(void* stream, const uint8_t* a, const int8_t* b,
                            int32_t offset_b, unsigned m, unsigned n, unsigned k, int32_t* acc_out,
                            float scale_a, const float* scale_b, float* f32_out);
 
+/* The same product on a B that was packed once (weights): column slabs of 16, each K x 16 bytes
+ * contiguous and already in matrix-core operand order, so that a decode step streams B at the rate
+ * of a plain contiguous read.  The reference re-packs its B operand on every call
+ * (tfcc/mkl/gemm/tfcc_mklinputpackermanager.h:34-47) and keeps constants per device
+ * (tfcc/core/framework/tfcc_constant.cpp:69-76); packing once per constant is the GPU counterpart.
+ * tfcc_rocm_gemv_packed_size gives the byte size of the packed buffer (device memory, 16-byte aligned). */
+size_t tfcc_rocm_gemv_packed_size(unsigned n, unsigned k);
+int tfcc_rocm_gemv_pack_b(void* stream, const int8_t* b, unsigned n, unsigned k, void* packed);
+int tfcc_rocm_gemv_u8s8s32_packed(void* stream, const uint8_t* a, const void* packed_b,
+                                  const int32_t* rowsum_a, const int32_t* colsum_b, int32_t offset_a,
+                                  int32_t offset_b, unsigned m, unsigned n, unsigned k, int32_t* acc_out,
+                                  float scale_a, const float* scale_b, float* f32_out);
+
 /*
  * Row sums (out [batch][row]) and column sums (out [batch][col]) in int32.
  * Replaces _mkl_reduce_sum_row / _mkl_reduce_sum_column,

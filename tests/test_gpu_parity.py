@@ -183,6 +183,28 @@ def test_gemv_against_oracle(pkg, T, m, n, k):
     assert np.array_equal(T.n(got), O.qgemm(a, b, -128, 0, rs, cs))
 
 
+@pytest.mark.parametrize("m", [1, 5, 8])
+@pytest.mark.parametrize("n,k", [(11008, 4096), (16, 16), (100, 80), (260, 4000), (4096, 8320)])
+def test_gemv_on_packed_weights(pkg, T, m, n, k):
+    print("gemv packed", m, n, k, flush=True)
+    rng = np.random.default_rng(m * 7 + n + k)
+    a = rng.integers(0, 256, (m, k), dtype=np.uint8)
+    b = rng.integers(-128, 128, (k, n), dtype=np.int8)
+    rs, cs = O.reduce_sum(a, True), O.reduce_sum(b, False)
+    scale_b = rng.uniform(0.001, 0.01, n).astype(np.float32)
+    scale_a = float(np.float32(0.02))
+    packed = pkg.gemv_pack(T.t(b))
+    for oa, ob in ((-128, 0), (-57, 93)):
+        want = O.qgemm(a, b, oa, ob, rs, cs)
+        out, acc = pkg.gemv_dequant_packed(T.t(a), packed, n, T.t(rs), T.t(cs), oa, ob, scale_a, T.t(scale_b))
+        assert np.array_equal(T.n(acc), want), (oa, ob)
+        assert np.array_equal(T.n(out), O.dequant_per_channel(want, scale_a, scale_b))
+    # column sums as given by the caller, as the reference uses them
+    wrong = (cs + 3).astype(np.int32)
+    _, acc = pkg.gemv_dequant_packed(T.t(a), packed, n, T.t(rs), T.t(wrong), -57, 93, 1.0, None)
+    assert np.array_equal(T.n(acc), O.qgemm(a, b, -57, 93, rs, wrong))
+
+
 def test_gemv_full_size_hash(pkg, T):
     h = json.load(open(os.path.join(GOLDEN, "qgemm_ref_hashes.json")))["c5_m8"]
     a, b = gen_inputs(h["seed"], h["shape_a"], h["shape_b"])

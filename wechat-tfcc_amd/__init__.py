@@ -75,6 +75,9 @@ SYMBOLS = {
     "tfcc_rocm_sgemm_strided_batched": (_I, [_VP, _VP, _U64, _VP, _U64, _VP, _VP, _U64, _U, _U, _U, _U]),
     "tfcc_rocm_gemm_u8s8s32": (_I, [_VP, C.POINTER(QGemmDesc), _VP]),
     "tfcc_rocm_gemm_u8s8s32_requant_u8": (_I, [_VP, C.POINTER(QGemmDesc), _VP, _VP, _D, _D, _D, _I64, _VP, _VP]),
+    "tfcc_rocm_gemv_packed_size": (C.c_size_t, [_U, _U]),
+    "tfcc_rocm_gemv_pack_b": (_I, [_VP, _VP, _U, _U, _VP]),
+    "tfcc_rocm_gemv_u8s8s32_packed": (_I, [_VP, _VP, _VP, _VP, _VP, C.c_int32, C.c_int32, _U, _U, _U, _VP, _F, _VP, _VP]),
     "tfcc_rocm_gemv_u8s8s32": (_I, [_VP, _VP, _VP, _VP, _VP, C.c_int32, C.c_int32, _U, _U, _U, _VP, _F, _VP, _VP]),
     "tfcc_rocm_reduce_sum_rows": (_I, [_VP, _VP, _I, _U, _U, _U, _VP]),
     "tfcc_rocm_reduce_sum_cols": (_I, [_VP, _VP, _I, _U, _U, _U, _VP]),
@@ -319,6 +322,28 @@ def gemv_dequant(a, b, reduce_a, reduce_b, offset_a, offset_b, scale_a, scale_b,
     out = torch.empty((m, n), dtype=torch.float32, device=a.device) if scale_b is not None else None
     check(lib().tfcc_rocm_gemv_u8s8s32(_stream(), _ptr(a), _ptr(b), _ptr(reduce_a), _ptr(reduce_b), offset_a,
                                         offset_b, m, n, k, _ptr(acc), float(scale_a), _ptr(scale_b), _ptr(out)))
+    return out, acc
+
+
+def gemv_pack(b):
+    """Packs an int8 [K, N] weight matrix once for gemv_dequant_packed; returns the packed buffer."""
+    import torch
+    b = b.contiguous()
+    k, n = b.shape
+    packed = torch.empty(lib().tfcc_rocm_gemv_packed_size(n, k), dtype=torch.uint8, device=b.device)
+    check(lib().tfcc_rocm_gemv_pack_b(_stream(), _ptr(b), n, k, _ptr(packed)))
+    return packed
+
+
+def gemv_dequant_packed(a, packed, n, reduce_a, reduce_b, offset_a, offset_b, scale_a, scale_b, want_acc=True):
+    """gemv_dequant on weights packed by gemv_pack (n: the column count of the original matrix)."""
+    import torch
+    a = a.contiguous()
+    m, k = a.shape
+    acc = torch.empty((m, n), dtype=torch.int32, device=a.device) if want_acc else None
+    out = torch.empty((m, n), dtype=torch.float32, device=a.device) if scale_b is not None else None
+    check(lib().tfcc_rocm_gemv_u8s8s32_packed(_stream(), _ptr(a), _ptr(packed), _ptr(reduce_a), _ptr(reduce_b), offset_a,
+                                               offset_b, m, n, k, _ptr(acc), float(scale_a), _ptr(scale_b), _ptr(out)))
     return out, acc
 
 

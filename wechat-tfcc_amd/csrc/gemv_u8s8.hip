@@ -159,6 +159,104 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(const GemvParams p) {
   }
 }
 
+
+// ---- pre-packed B (weights that are multiplied many times) --------------------------------------------
+// Layout: [N/16 column slabs][K/64 steps][64 lanes][16 bytes], where lane (kg = lane / 16, j = lane % 16)
+// of step t holds B[64 t + 16 kg + 0..15][16 slab + j]: exactly the B operand of one
+// v_mfma_i32_16x16x64_i8, so a wavefront fetches an operand with one contiguous 1 KiB load and no
+// byte shuffling, and a workgroup streams one contiguous slab (K x 16 bytes).  Rows past K and columns
+// past N are stored as zeros.
+constexpr int kPackWaves = 4;
+constexpr int kPackThreads = kPackWaves * 64;
+constexpr int kPackInFlight = 16;  // operand loads in flight per wavefront
+
+__global__ __launch_bounds__(256) void gemv_pack_kernel(const signed char* b, unsigned N, unsigned K, unsigned steps,
+                                                        size_t chunks, unsigned char* packed) {
+  // one 16-byte chunk per thread (gathered from 16 rows of B: this runs once per weight matrix)
+  const size_t c = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (c >= chunks) return;
+  const unsigned lane = (unsigned)(c & 63);
+  const size_t st = c >> 6;
+  const unsigned t = (unsigned)(st % steps), slab = (unsigned)(st / steps);
+  const unsigned col = slab * 16 + (lane & 15), k0 = t * 64 + (lane >> 4) * 16;
+  unsigned w[4] = {0, 0, 0, 0};
+  if (col < N) {
+#pragma unroll
+    for (int q = 0; q < 16; ++q) {
+      const unsigned k = k0 + q;
+      const unsigned v = k < K ? (unsigned char)b[(size_t)k * N + col] : 0u;
+      w[q >> 2] |= v << (8 * (q & 3));
+    }
+  }
+  *reinterpret_cast<v4i*>(packed + c * 16) = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
+}
+
+__global__ __launch_bounds__(kPackThreads) void gemv_packed_kernel(const GemvParams p, const unsigned char* packed,
+                                                                  unsigned steps) {
+  __shared__ int red[kPackWaves][kPartRows][16];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const unsigned slab = blockIdx.x;
+  const unsigned M = p.M, N = p.N, K = p.K;
+  const int j = lane & 15, kg = lane >> 4;
+  const unsigned char* src = packed + (size_t)slab * steps * 1024 + lane * 16;
+  const __amdgpu_buffer_rsrc_t rsrcA =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(p.A), 0, (int)(M * K), 0x00020000);
+  const v4i ones = {0x01010101, 0x01010101, 0x01010101, 0x01010101};
+  v4i acc = {0, 0, 0, 0};
+  // what the store needs from memory is fetched first, so that its latency hides behind the B stream
+  const unsigned er = tid >> 4, ec = tid & 15, egn = slab * 16 + ec;
+  const bool eActive = tid < (int)(M * 16) && egn < N;
+  int eRowsum = 0, eColsum = 0;
+  float eScale = 0.f;
+  if (eActive) {
+    eRowsum = p.rowsumA[er];
+    eColsum = p.colsumB[egn];
+    if (p.f32Out) eScale = p.scaleB[egn];
+  }
+  // the wavefronts deal the steps among themselves, kPackInFlight at a time
+  for (unsigned t0 = wave * kPackInFlight; t0 < steps; t0 += kPackWaves * kPackInFlight) {
+    v4i bv[kPackInFlight], av[kPackInFlight];
+#pragma unroll
+    for (int u = 0; u < kPackInFlight; ++u) {
+      const unsigned t = t0 + u;
+      bv[u] = v4i{0, 0, 0, 0};
+      av[u] = v4i{0, 0, 0, 0};
+      if (t < steps) {
+        bv[u] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(src + (size_t)t * 1024));  // streamed once
+        if ((unsigned)j < M)
+          av[u] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrcA, (unsigned)j * K + t * 64 + kg * 16, 0, 0)) ^
+                  (int)0x80808080;
+        else if (j == kRows - 1)
+          av[u] = ones;
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < kPackInFlight; ++u) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(av[u], bv[u], acc, 0, 0, 0);
+  }
+  // lane (j, kg) holds rows 4 kg + r of column j
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int row = 4 * kg + r;
+    if (row < kMaxM) red[wave][row][j] = acc[r];
+    else if (row == kRows - 1) red[wave][kMaxM][j] = acc[r];
+  }
+  __syncthreads();
+  int oA = p.offsetA, oB = p.offsetB;
+  const unsigned offA = (unsigned)oA, offB = (unsigned)oB;
+  const unsigned global = offA * offB * K;
+  if (eActive) {
+    unsigned sum = 0, cs = 0;
+#pragma unroll
+    for (int w = 0; w < kPackWaves; ++w) {
+      sum += (unsigned)red[w][er][ec];
+      cs += (unsigned)red[w][kMaxM][ec];
+    }
+    const unsigned v = sum + 128u * cs + global + (unsigned)eRowsum * offB + (unsigned)eColsum * offA;
+    if (p.accOut) p.accOut[(size_t)er * N + egn] = (int)v;
+    if (p.f32Out) p.f32Out[(size_t)er * N + egn] = (float)((double)(int)v * ((double)p.scaleA * (double)eScale));
+  }
+}
+
 }  // namespace
 
 // Whether the skinny kernel can take this shape (else the caller uses the general kernel).
@@ -227,4 +325,41 @@ extern "C" int tfcc_rocm_gemv_u8s8s32(void* stream, const uint8_t* a, const int8
     return check_launch("per-channel dequantize");
   }
   return TFCC_ROCM_OK;
+}
+
+extern "C" size_t tfcc_rocm_gemv_packed_size(unsigned n, unsigned k) {
+  return (size_t)((n + 15) / 16) * ((k + 63) / 64) * 1024;
+}
+
+extern "C" int tfcc_rocm_gemv_pack_b(void* stream, const int8_t* b, unsigned n, unsigned k, void* packed) {
+  TFCC_REQUIRE(b && packed, "pack: null argument");
+  TFCC_REQUIRE(n > 0 && k > 0, "pack: empty operand");
+  TFCC_REQUIRE((uintptr_t)packed % 16 == 0, "pack: the packed buffer must be 16-byte aligned");
+  const unsigned steps = (k + 63) / 64;
+  const size_t chunks = tfcc_rocm_gemv_packed_size(n, k) / 16;
+  TFCC_REQUIRE((chunks + 255) / 256 < (1ull << 31), "pack: operand too large");
+  hipLaunchKernelGGL(gemv_pack_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, as_stream(stream),
+                     reinterpret_cast<const signed char*>(b), n, k, steps, chunks, static_cast<unsigned char*>(packed));
+  return check_launch("pack");
+}
+
+extern "C" int tfcc_rocm_gemv_u8s8s32_packed(void* stream, const uint8_t* a, const void* packed_b,
+                                             const int32_t* rowsum_a, const int32_t* colsum_b, int32_t offset_a,
+                                             int32_t offset_b, unsigned m, unsigned n, unsigned k, int32_t* acc_out,
+                                             float scale_a, const float* scale_b, float* f32_out) {
+  TFCC_REQUIRE(a && packed_b && rowsum_a && colsum_b, "skinny quantized matmul: null operand");
+  TFCC_REQUIRE(m > 0 && n > 0 && k > 0, "skinny quantized matmul: empty operand");
+  TFCC_REQUIRE(m <= (unsigned)kMaxM, "skinny quantized matmul on packed weights: at most %d rows", kMaxM);
+  TFCC_REQUIRE(k % 16 == 0 && (uintptr_t)a % 16 == 0 && (uintptr_t)packed_b % 16 == 0,
+               "skinny quantized matmul on packed weights: k and the operands must be multiples of / aligned to 16");
+  TFCC_REQUIRE((unsigned long long)m * k < (1ull << 31), "skinny quantized matmul: operand too large");
+  TFCC_REQUIRE(acc_out || f32_out, "skinny quantized matmul: no output");
+  TFCC_REQUIRE(!f32_out || scale_b, "skinny quantized matmul: dequantize needs scale_b");
+  GemvParams p{};
+  p.A = a; p.rowsumA = rowsum_a; p.colsumB = colsum_b; p.accOut = acc_out; p.f32Out = f32_out;
+  p.scaleA = scale_a; p.scaleB = scale_b; p.offsetA = offset_a; p.offsetB = offset_b;
+  p.M = m; p.N = n; p.K = k;
+  hipLaunchKernelGGL(gemv_packed_kernel, dim3((n + 15) / 16), dim3(kPackThreads), 0, as_stream(stream), p,
+                     static_cast<const unsigned char*>(packed_b), (k + 63) / 64);
+  return check_launch("skinny quantized matmul (packed)");
 }
