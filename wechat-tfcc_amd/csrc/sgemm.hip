@@ -317,7 +317,10 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_kernel(const Sg
       if (vecOK) {
         if constexpr (NI == 4) *reinterpret_cast<v4f*>(C + off) = v4f{v[0], v[1], v[2], v[3]};
         else if constexpr (NI == 2) *reinterpret_cast<float2*>(C + off) = make_float2(v[0], v[1]);
-        else C[off] = v[0];
+        else {
+#pragma unroll
+          for (int j = 0; j < NI; ++j) C[off + j] = v[j];
+        }
       } else {
 #pragma unroll
         for (int j = 0; j < NI; ++j)
