@@ -126,6 +126,14 @@ typedef struct tfcc_rocm_sgemm_desc {
 } tfcc_rocm_sgemm_desc;
 int tfcc_rocm_sgemm_general(void* stream, const tfcc_rocm_sgemm_desc* desc);
 
+/* Up to four products a * b[g] (+ bias[g]) -> c[g] that share a dense [m, k] operand a and have equal
+ * shapes ([k, n] each, dense), in one launch: e.g. the query / key / value projections of an attention
+ * block, which the reference issues as three matmul calls on the same input
+ * (tfcc_runtime/operations/math/matmulwithbias.cpp:29-40 per node).  b, bias (may be NULL) and c are
+ * host arrays of `groups` device pointers.  Every product is computed exactly as by a launch of its own. */
+int tfcc_rocm_sgemm_grouped(void* stream, const float* a, const float* const* b, const float* const* bias,
+                            float* const* c, unsigned groups, unsigned m, unsigned n, unsigned k);
+
 /* ---------------------------------------------------------------------------------------------
  * Quantized uint8 x int8 -> int32 matmul.
  * Replaces _mkl_create_offset_matrix + _MKLQuantizationMatmulAVX256::quantizedMatmulColMajor,

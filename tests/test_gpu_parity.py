@@ -395,6 +395,19 @@ def test_sgemm_general_multiplies_permuted_views_in_place(pkg, T, b, s, h, d):
     assert np.array_equal(dense, T.n(scores))
 
 
+@pytest.mark.parametrize("m,n,k,groups", [(1024, 768, 768, 3), (100, 52, 36, 4), (64, 64, 1028, 2), (7, 4, 4, 1)])
+def test_sgemm_grouped_equals_separate_launches(pkg, T, m, n, k, groups):
+    rng = np.random.default_rng(m + n + k + groups)
+    a = rng.normal(0, 1, (m, k)).astype(np.float32)
+    bs = [rng.normal(0, 1, (k, n)).astype(np.float32) for _ in range(groups)]
+    biases = [rng.uniform(-1, 1, n).astype(np.float32) for _ in range(groups)]
+    outs = pkg.sgemm_grouped(T.t(a), [T.t(b) for b in bs], [T.t(b) for b in biases])
+    for b, bias, out in zip(bs, biases, outs):
+        single = T.n(pkg.blas_matmul(T.t(a), T.t(b), T.t(bias)))
+        assert np.array_equal(T.n(out), single)
+        assert rel_fro(T.n(out), a.astype(np.float64) @ b.astype(np.float64) + bias) <= FP32_TOL
+
+
 def test_matmul_validation_and_empty(pkg, T):
     """Error behaviour of tfcc::blas::matmul (tfcc/core/operations/tfcc_blas.cpp:26-54)."""
     z = lambda *s: T.t(np.zeros(s, np.float32))

@@ -100,6 +100,7 @@ SYMBOLS = {
     "tfcc_rocm_graph_destroy": (_I, [_VP]),
     "tfcc_rocm_sgemm_fused": (_I, [_VP, _VP, _U64, _VP, _U64, _VP, _VP, _U64, _VP, _U64, _U, _U, _U, _U, _I]),
     "tfcc_rocm_sgemm_general": (_I, [_VP, _VP]),
+    "tfcc_rocm_sgemm_grouped": (_I, [_VP, _VP, C.POINTER(_VP), C.POINTER(_VP), C.POINTER(_VP), _U, _U, _U, _U]),
     "tfcc_rocm_softmax_div_f32": (_I, [_VP, _VP, _U64, _U, _F, _VP]),
     "tfcc_rocm_transform2_f32": (_I, [_VP, _VP, _U64, _F, _F, _VP]),
     "tfcc_rocm_binary_f32": (_I, [_VP, _I, _VP, _VP, _U64, _U64, _VP]),
@@ -207,6 +208,20 @@ def sgemm_general(a, b, c, m, n, k, lda, ldb, ldc, trans_b=False, batch_outer=1,
     d.activation = activation
     check(lib().tfcc_rocm_sgemm_general(_stream(), C.byref(d)))
     return c
+
+
+def sgemm_grouped(a, bs, biases):
+    """[a @ b + bias for b, bias in zip(bs, biases)] in one launch (a: [m, k]; every b: [k, n])."""
+    import torch
+    a = a.contiguous()
+    m, k = a.shape
+    n = bs[0].shape[1]
+    groups = len(bs)
+    outs = [torch.empty((m, n), dtype=torch.float32, device=a.device) for _ in bs]
+    arr = lambda ts: (_VP * groups)(*[_ptr(t) for t in ts])
+    check(lib().tfcc_rocm_sgemm_grouped(_stream(), _ptr(a), arr(bs), arr(biases) if biases is not None else None,
+                                        arr(outs), groups, m, n, k))
+    return outs
 
 
 def reduce_sum(a, row):

@@ -33,6 +33,11 @@ struct SgemmParams {
   unsigned batchInner;    // batch entry bi = (bi / batchInner, bi % batchInner); 1 for a flat batch
   unsigned lda, ldb, ldc; // row strides of A, of B (of B^T when transposed) and of C, in elements
   int act;                // 0 none, 1 erf-form GELU applied last
+  // grouped form (groups > 0): batch entry g multiplies the shared A by groupB[g] into groupC[g]
+  unsigned groups;
+  const float* groupB[4];
+  const float* groupBias[4];
+  float* groupC[4];
   unsigned M, N, K, batch;
   unsigned tilesM, tilesN, tilesTotal, chunk;
 };
@@ -91,6 +96,13 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_kernel(const Sg
   const unsigned bo = bi / p.batchInner, bn = bi - bo * p.batchInner;
   const float* __restrict__ A = p.A + (size_t)bo * p.strideA + (size_t)bn * p.innerA;
   const float* __restrict__ B = p.B + (size_t)bo * p.strideB + (size_t)bn * p.innerB;
+  const float* biasPtr = p.bias;
+  float* Cbase = p.C + (size_t)bo * p.strideC + (size_t)bn * p.innerC;
+  if (p.groups) {  // selects, not indexing: the argument block stays in scalar registers
+    B = bi == 0 ? p.groupB[0] : bi == 1 ? p.groupB[1] : bi == 2 ? p.groupB[2] : p.groupB[3];
+    biasPtr = bi == 0 ? p.groupBias[0] : bi == 1 ? p.groupBias[1] : bi == 2 ? p.groupBias[2] : p.groupBias[3];
+    Cbase = bi == 0 ? p.groupC[0] : bi == 1 ? p.groupC[1] : bi == 2 ? p.groupC[2] : p.groupC[3];
+  }
   const unsigned lda = p.lda, ldb = p.ldb, ldc = p.ldc;
 
   v16f acc[MI][NI];
@@ -284,13 +296,13 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_kernel(const Sg
 
   // ---- epilogue: + bias, store.  Lane (i, g) owns columns NI*i .. NI*i+NI-1 of the wavefront's
   // column range and rows 8*(r/4) + 4*g + r%4 of each 32-row block.
-  float* __restrict__ C = p.C + (size_t)bo * p.strideC + (size_t)bn * p.innerC;
+  float* __restrict__ C = Cbase;
   const float* __restrict__ R = p.residual ? p.residual + (size_t)bi * p.strideR : nullptr;  // dense, flat batch
   const int act = p.act;
   const unsigned gcol = n0 + wn * WN + NI * lrow;
   float bv[NI];
 #pragma unroll
-  for (int j = 0; j < NI; ++j) bv[j] = (p.bias && gcol + j < N) ? p.bias[gcol + j] : 0.f;
+  for (int j = 0; j < NI; ++j) bv[j] = (biasPtr && gcol + j < N) ? biasPtr[gcol + j] : 0.f;
   const bool vecOK = VEC && (gcol + NI <= N);
 #pragma unroll
   for (int i = 0; i < MI; ++i) {
@@ -352,6 +364,37 @@ int launch(hipStream_t stream, SgemmParams p) {
   return check_launch("sgemm");
 }
 
+// Picks the tile configuration from the shape of one product and the number of batch entries that
+// count towards filling the chip (`fillBatch`), and launches.
+int dispatch(hipStream_t s, const SgemmParams& p, bool vec, bool tb, unsigned fillBatch, unsigned lda, unsigned ldb,
+             unsigned ldc) {
+  const unsigned m = p.M, n = p.N, k = p.K;
+  const unsigned long long rowsB = tb ? n : k;
+  if (tb) {
+    if (vec) return launch<2, 2, 1, 1, true, 1, true>(s, p);
+    TFCC_REQUIRE((unsigned long long)m * ldc < (1ull << 32) && (unsigned long long)m * lda < (1ull << 32) &&
+                 rowsB * ldb < (1ull << 32), "sgemm: operand larger than 2^32 elements");
+    return launch<2, 2, 1, 1, false, 1, true>(s, p);
+  }
+  // 128x128 tiles once there are enough of them to fill the 256 CUs twice over, else 64x64
+  const unsigned long long big = (unsigned long long)((m + 127) / 128) * ((n + 127) / 128) * fillBatch;
+  if (vec) {
+    if (big >= 512) return launch<4, 1, 1, 4, true>(s, p);
+    // few 64x64 tiles and a long K: several K groups per workgroup keep the CUs that have a tile busy
+    const unsigned long long small = (unsigned long long)((m + 63) / 64) * ((n + 63) / 64) * fillBatch;
+    // 32x96 tiles when they cover the 256 CUs in fewer tile-area rounds than 64x64 tiles would
+    const unsigned long long flat = (unsigned long long)((m + 31) / 32) * ((n + 95) / 96) * fillBatch;
+    const bool preferFlat = ((flat + 255) / 256) * (32 * 96) < ((small + 255) / 256) * (64 * 64);
+    if (preferFlat && flat <= 320 && k >= 512) return launch<1, 3, 1, 1, true, 4>(s, p);
+    if (small <= 320 && k >= 512) return launch<2, 2, 1, 1, true, 4>(s, p);
+    if (small <= 640 && k >= 256) return launch<2, 2, 1, 1, true, 2>(s, p);
+    return launch<2, 2, 1, 1, true>(s, p);
+  }
+  TFCC_REQUIRE((unsigned long long)m * ldc < (1ull << 32) && (unsigned long long)m * lda < (1ull << 32) &&
+               rowsB * ldb < (1ull << 32), "sgemm: operand larger than 2^32 elements");
+  return launch<2, 2, 1, 1, false>(s, p);
+}
+
 }  // namespace
 }  // namespace tfcc_rocm
 
@@ -406,27 +449,32 @@ extern "C" int tfcc_rocm_sgemm_general(void* stream, const tfcc_rocm_sgemm_desc*
                    (((unsigned long long)m + 256) * d->lda + k + 256 < (1ull << 30)) &&
                    ((rowsB + 256) * d->ldb + colsB + 1024 < (1ull << 30));
   hipStream_t s = as_stream(stream);
-  if (tb) {
-    if (vec) return launch<2, 2, 1, 1, true, 1, true>(s, p);
-    TFCC_REQUIRE((unsigned long long)m * d->ldc < (1ull << 32) && (unsigned long long)m * d->lda < (1ull << 32) &&
-                 rowsB * d->ldb < (1ull << 32), "sgemm: operand larger than 2^32 elements");
-    return launch<2, 2, 1, 1, false, 1, true>(s, p);
+  return dispatch(s, p, vec, tb, batch, d->lda, d->ldb, d->ldc);
+}
+
+extern "C" int tfcc_rocm_sgemm_grouped(void* stream, const float* a, const float* const* b, const float* const* bias,
+                                       float* const* c, unsigned groups, unsigned m, unsigned n, unsigned k) {
+  TFCC_REQUIRE(a && b && c, "grouped sgemm: null operand");
+  TFCC_REQUIRE(groups >= 1 && groups <= 4, "grouped sgemm: 1 to 4 products per launch, got %u", groups);
+  TFCC_REQUIRE(m > 0 && n > 0 && k > 0, "grouped sgemm: empty operand");
+  SgemmParams p{};
+  p.A = a; p.M = m; p.N = n; p.K = k; p.batch = groups; p.batchInner = 1;
+  p.lda = k; p.ldb = n; p.ldc = n;
+  p.groups = groups;
+  bool aligned = (uintptr_t)a % 16 == 0;
+  for (unsigned g = 0; g < 4; ++g) {
+    const unsigned src = g < groups ? g : 0;
+    TFCC_REQUIRE(b[src] && c[src], "grouped sgemm: null operand");
+    p.groupB[g] = b[src];
+    p.groupBias[g] = bias ? bias[src] : nullptr;
+    p.groupC[g] = c[src];
+    aligned = aligned && (uintptr_t)b[src] % 16 == 0 && (uintptr_t)c[src] % 16 == 0;
   }
-  // 128x128 tiles once there are enough of them to fill the 256 CUs twice over, else 64x64
-  const unsigned long long big = (unsigned long long)((m + 127) / 128) * ((n + 127) / 128) * batch;
-  if (vec) {
-    if (big >= 512) return launch<4, 1, 1, 4, true>(s, p);
-    // few 64x64 tiles and a long K: several K groups per workgroup keep the CUs that have a tile busy
-    const unsigned long long small = (unsigned long long)((m + 63) / 64) * ((n + 63) / 64) * batch;
-    // 32x96 tiles when they cover the 256 CUs in fewer tile-area rounds than 64x64 tiles would
-    const unsigned long long flat = (unsigned long long)((m + 31) / 32) * ((n + 95) / 96) * batch;
-    const bool preferFlat = ((flat + 255) / 256) * (32 * 96) < ((small + 255) / 256) * (64 * 64);
-    if (preferFlat && flat <= 320 && k >= 512) return launch<1, 3, 1, 1, true, 4>(s, p);
-    if (small <= 320 && k >= 512) return launch<2, 2, 1, 1, true, 4>(s, p);
-    if (small <= 640 && k >= 256) return launch<2, 2, 1, 1, true, 2>(s, p);
-    return launch<2, 2, 1, 1, true>(s, p);
-  }
-  TFCC_REQUIRE((unsigned long long)m * d->ldc < (1ull << 32) && (unsigned long long)m * d->lda < (1ull << 32) &&
-               rowsB * d->ldb < (1ull << 32), "sgemm: operand larger than 2^32 elements");
-  return launch<2, 2, 1, 1, false>(s, p);
+  p.B = p.groupB[0];
+  p.C = p.groupC[0];
+  const bool vec = aligned && (k % 4 == 0) && (n % 4 == 0) && (((unsigned long long)m + 256) * k + k + 256 < (1ull << 30)) &&
+                   (((unsigned long long)k + 256) * n + n + 1024 < (1ull << 30));
+  // the tile configuration is the one a single product of this shape gets, so that every product
+  // of the group is summed in exactly the order of a launch of its own
+  return dispatch(as_stream(stream), p, vec, false, 1, k, n, n);
 }

@@ -326,10 +326,15 @@ Variable<float> rocm_sgemm(const Tensor<float>& a, const Tensor<float>& b, const
   s[s.size() - 1] = n;
   Variable<float> result{Shape(std::move(s))};
   if (residual && !(residual->shape() == result.shape())) throw InvalidArgumentError("residual and result don't match");
-  const unsigned batch = result.size() / (m * n);
+  unsigned rows = m, batch = result.size() / (m * n);
+  if (rb == 2 && ra > 2) {
+    // one matrix b for the whole batch of a: the batch is just more rows of one product
+    rows = m * batch;
+    batch = 1;
+  }
   check(tfcc_rocm_sgemm_fused(current_stream(), a.data(), strideA, b.data(), strideB, bias ? bias->data() : nullptr,
-                              residual ? residual->data() : nullptr, static_cast<uint64_t>(m) * n, result.data(),
-                              static_cast<uint64_t>(m) * n, m, n, k, batch, activation));
+                              residual ? residual->data() : nullptr, static_cast<uint64_t>(rows) * n, result.data(),
+                              static_cast<uint64_t>(rows) * n, rows, n, k, batch, activation));
   return result;
 }
 
@@ -721,6 +726,34 @@ Variable<float> matmul_permuted(const Tensor<float>& a, const std::vector<size_t
   d.stride_c = cStride[0]; d.inner_stride_c = cStride[1];
   check(tfcc_rocm_sgemm_general(current_stream(), &d));
   return result;
+}
+std::vector<Variable<float>> matmul_grouped(const Tensor<float>& a, const std::vector<const Tensor<float>*>& b,
+                                            const std::vector<const Tensor<float>*>& bias) {
+  if (dynamic_cast<ROCMDevice*>(Device::getThreadDefault()) == nullptr) throw NotImplementedError();
+  const size_t groups = b.size();
+  if (groups < 1 || groups > 4 || bias.size() != groups) throw NotImplementedError("matmul_grouped: 1 to 4 products");
+  const size_t ra = a.shape().size();
+  if (ra < 2 || a.size() == 0) throw NotImplementedError("matmul_grouped: operand a");
+  const unsigned k = a.shape(ra - 1), m = a.size() / k, n = b[0]->shape().size() == 2 ? b[0]->shape(1) : 0;
+  for (size_t g = 0; g < groups; ++g) {
+    if (b[g]->shape().size() != 2 || b[g]->shape(0) != k || b[g]->shape(1) != n || n == 0 || bias[g] == nullptr ||
+        bias[g]->shape().size() != 1 || bias[g]->size() != n)
+      throw NotImplementedError("matmul_grouped: the weight matrices need one common [k, n] shape and [n] biases");
+  }
+  std::vector<unsigned> shape = a.shape().toVector();
+  shape.back() = n;
+  std::vector<Variable<float>> results;
+  const float* bp[4];
+  const float* biasp[4];
+  float* cp[4];
+  for (size_t g = 0; g < groups; ++g) {
+    results.emplace_back(Shape(shape));
+    bp[g] = b[g]->data();
+    biasp[g] = bias[g]->data();
+    cp[g] = results.back().data();
+  }
+  check(tfcc_rocm_sgemm_grouped(current_stream(), a.data(), bp, biasp, cp, static_cast<unsigned>(groups), m, n, k));
+  return results;
 }
 }  // namespace blas
 namespace math {

@@ -95,6 +95,11 @@ Variable<float> matmul_fused(const Tensor<float>& a, const Tensor<float>& b, con
 // anything else raises NotImplementedError.  Results equal the step-by-step form bit for bit.
 Variable<float> matmul_permuted(const Tensor<float>& a, const std::vector<size_t>& permA, const Tensor<float>& b,
                                 const std::vector<size_t>& permB, const std::vector<size_t>& permC);
+// { a * b[g] + bias[g] } for up to four weight matrices of one shape ([k, n], rank 2) in a single launch;
+// a: [..., k] of any rank >= 2 (its leading dimensions are the rows).  Each result equals
+// tfcc::blas::matmul(a, b[g], bias[g]) bit for bit.  Raises NotImplementedError for anything else.
+std::vector<Variable<float>> matmul_grouped(const Tensor<float>& a, const std::vector<const Tensor<float>*>& b,
+                                            const std::vector<const Tensor<float>*>& bias);
 }  // namespace blas
 namespace math {
 // softmax(a / divisor, axis)

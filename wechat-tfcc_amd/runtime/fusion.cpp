@@ -6,6 +6,7 @@
 //   MatmulWithBias -> Add(other tensor)    one GEMM that also adds the other tensor (residual)
 //   Div(tensor, value) -> Softmax          one softmax pass that divides first
 //   Transpose -> Matmul -> Transpose       a batched product that walks the permuted tensors in place
+//   2-4 x MatmulWithBias on one input with constant weights of one shape (query / key / value): one launch
 //   Identity of a variable nobody else reads: the buffer is handed over instead of copied
 //
 // A producer is absorbed only when its output is a float VARIABLE symbol with exactly one consumer
@@ -121,6 +122,38 @@ std::vector<FusionPlan> plan_fusions(const proto::Graph& g, SymbolManager& sm) {
       plan[j] = {FusionPlan::MOVE_IDENTITY, j, 0};
     }
   }
+  // MatmulWithBias nodes left as they are that share their input and have constant weights: groups of up to 4
+  std::unordered_map<std::string, std::vector<size_t>> byInput;
+  std::vector<std::string> order;
+  for (size_t j = 0; j < g.nodes.size(); ++j) {
+    const proto::Node& n = g.nodes[j];
+    if (plan[j].kind != FusionPlan::NONE || !is_op(n, "math.MatmulWithBias", 3) || !all_float_tensors(n) ||
+        !float_variable(sm, n.outputs[0]))
+      continue;
+    if (sm.getSymbolInfo(n.inputs[1]).stype != SymbolType::CONSTANT_TENSOR ||
+        sm.getSymbolInfo(n.inputs[2]).stype != SymbolType::CONSTANT_TENSOR)
+      continue;
+    // the shared input must exist before the first member runs: a graph input or produced earlier
+    auto p = producer.find(n.inputs[0]);
+    if (p != producer.end() && p->second >= j) continue;
+    if (!byInput.count(n.inputs[0])) order.push_back(n.inputs[0]);
+    byInput[n.inputs[0]].push_back(j);
+  }
+  for (const std::string& name : order) {
+    std::vector<size_t>& members = byInput[name];
+    // the input's producer must precede the first member (members are in node order)
+    auto p = producer.find(name);
+    if (p != producer.end() && p->second > members.front()) continue;
+    for (size_t at = 0; at + 1 < members.size(); at += 4) {
+      const size_t count = std::min<size_t>(4, members.size() - at);
+      if (count < 2) break;
+      FusionPlan f;
+      f.kind = FusionPlan::MATMUL_GROUPED;
+      f.group.assign(members.begin() + at, members.begin() + at + count);
+      for (size_t q = 1; q < count; ++q) plan[f.group[q]] = {FusionPlan::ABSORBED, f.group[0], 0};
+      plan[f.group[0]] = f;
+    }
+  }
   return plan;
 }
 
@@ -140,6 +173,27 @@ std::vector<size_t> transpose_perm(const proto::Node& n) {
 void emit_fused(const proto::Graph& g, const FusionPlan& f, size_t j, Graph& graph) {
   SymbolManager& sm = graph.getSymbolManager();
   const proto::Node& n = g.nodes[j];
+  if (f.kind == FusionPlan::MATMUL_GROUPED) {
+    const Tensor<float>* a = sm.getTensor(n.inputs[0], float());
+    std::vector<const Tensor<float>*> bs, biases;
+    std::vector<Variable<float>*> outs;
+    for (size_t member : f.group) {
+      bs.push_back(sm.getTensor(g.nodes[member].inputs[1], float()));
+      biases.push_back(sm.getTensor(g.nodes[member].inputs[2], float()));
+      outs.push_back(sm.getVariable(g.nodes[member].outputs[0], float()));
+    }
+    graph.addStep([a, bs, biases, outs] {
+      try {
+        std::vector<Variable<float>> results = rocm::blas::matmul_grouped(*a, bs, biases);
+        for (size_t q = 0; q < outs.size(); ++q) *outs[q] = std::move(results[q]);
+        return;
+      } catch (NotImplementedError&) {
+        // weights of different shapes, or a layout the grouped launch does not take: one launch each
+      }
+      for (size_t q = 0; q < outs.size(); ++q) *outs[q] = blas::matmul(*a, *bs[q], *biases[q]);
+    });
+    return;
+  }
   if (f.kind == FusionPlan::MATMUL_PERMUTED) {
     const bool ta = f.transposeA != FusionPlan::kNoNode, tb = f.transposeB != FusionPlan::kNoNode,
                tc = f.transposeC != FusionPlan::kNoNode;
