@@ -8,8 +8,10 @@
 #include <cstdio>
 #include <cstdlib>
 #include <functional>
+#include <algorithm>
 #include <random>
 #include <string>
+#include <thread>
 
 #include "tfcc_rocm_device.h"
 
@@ -416,6 +418,66 @@ static void test_layer_ops() {
   CHECK(std::fabs(mean) < 1e-5f);
 }
 
+// Two threads, each with a session (= stream) of its own on the shared device, running the same mix of
+// operations at the same time: fp32 matmul, quantize with its min/max reduction, quantized matmul.  Every
+// result is checked on the thread that produced it (tfcc/core/framework/tfcc_session.h:29,60-62: device
+// and session are per-thread defaults).
+static void thread_body(unsigned seed, int rounds, int* failures) {
+  try {
+    tfcc::initialize_rocm();
+    std::mt19937 rng(seed);
+    std::uniform_real_distribution<float> dist(-3.f, 3.f);
+    for (int round = 0; round < rounds; ++round) {
+      const unsigned m = 17 + (rng() % 90), k = 8 + (rng() % 200), n = 5 + (rng() % 120);
+      std::vector<float> ha(size_t(m) * k), hb(size_t(k) * n);
+      for (auto& v : ha) v = dist(rng);
+      for (auto& v : hb) v = dist(rng);
+      tfcc::Variable<float> a = tfcc::data::set(ha, {m, k}), b = tfcc::data::set(hb, {k, n});
+      std::vector<float> got = tfcc::data::get(tfcc::blas::matmul(a, b));
+      for (unsigned i = 0; i < m; i += 7)
+        for (unsigned j = 0; j < n; j += 5) {
+          double s = 0;
+          for (unsigned p = 0; p < k; ++p) s += double(ha[size_t(i) * k + p]) * double(hb[size_t(p) * n + j]);
+          if (!is_similar(got[size_t(i) * n + j], float(s))) ++*failures;
+        }
+      // quantize finds this tensor's own range even while the other thread reduces another tensor
+      tfcc::Variable<uint8_t> qa;
+      tfcc::Variable<float> mn, mx;
+      std::tie(qa, mn, mx) = tfcc::quantization::quantize<uint8_t>(a);
+      float wantMin = ha[0], wantMax = ha[0];
+      for (float v : ha) { wantMin = std::min(wantMin, v); wantMax = std::max(wantMax, v); }
+      if (tfcc::data::get(mn)[0] != wantMin || tfcc::data::get(mx)[0] != wantMax) ++*failures;
+      tfcc::Variable<int8_t> qb;
+      tfcc::Variable<float> mnB, mxB, mnC, mxC;
+      std::tie(qb, mnB, mxB) = tfcc::quantization::quantize<int8_t>(b);
+      tfcc::Variable<int32_t> ra = tfcc::rocm::quantization::reduce_sum(qa, true), rb = tfcc::rocm::quantization::reduce_sum(qb, false);
+      tfcc::Variable<int32_t> qc;
+      std::tie(qc, mnC, mxC) = tfcc::rocm::quantization::matmul(qa, ra, mn, mx, qb, rb, mnB, mxB);
+      std::vector<float> approx = tfcc::data::get(tfcc::quantization::dequantize(qc, mnC, mxC));
+      // 8-bit operands: a loose bound is enough to catch results that belong to the other thread
+      double err = 0, ref = 0;
+      for (unsigned i = 0; i < m; i += 7)
+        for (unsigned j = 0; j < n; j += 5) {
+          err += std::fabs(approx[size_t(i) * n + j] - got[size_t(i) * n + j]);
+          ref += std::fabs(got[size_t(i) * n + j]);
+        }
+      if (!(err <= 0.1 * ref + 1.0)) ++*failures;
+    }
+  } catch (const std::exception& e) {
+    std::printf("  thread exception: %s\n", e.what());
+    ++*failures;
+  }
+}
+
+static void test_two_sessions_on_two_threads() {
+  int f1 = 0, f2 = 0;
+  std::thread t1(thread_body, 11u, 12, &f1), t2(thread_body, 23u, 12, &f2);
+  t1.join();
+  t2.join();
+  CHECK(f1 == 0);
+  CHECK(f2 == 0);
+}
+
 int main(int argc, char** argv) {
   const std::string mode = argc > 1 ? argv[1] : "cpu";
   std::unique_ptr<tfcc::HostDevice> hostDevice;
@@ -442,6 +504,7 @@ int main(int argc, char** argv) {
     run("quantization.rocm_matmul_round_trips", test_quantized_matmul_round_trips);
     run("quantization.rocm_matmul_exact", test_quantized_matmul_exact);
     run("layer.elementwise", test_layer_ops);
+    run("threads.two_sessions", test_two_sessions_on_two_threads);
   } else {
     run("blas.matmul_validation", [] {
       // on the host device only the checks run; a valid shape reaches the (absent) backend

@@ -377,11 +377,14 @@ int launch(hipStream_t stream, QGemmParams p) {
   constexpr size_t lds = 2 * (size_t)(BM + BN) * BK;
   static_assert(lds >= (size_t)(BM + BN) * 4, "epilogue terms must fit in the slab buffers");
   auto kern = qgemm_kernel<BM, BN, BK, ALIGNED, REQUANT>;
-  static bool attrSet = false;  // one flag per instantiation
-  if (!attrSet) {
+  static bool attrSet[16] = {};  // per device: the attribute belongs to the function on one device
+  int dev = 0;
+  TFCC_HIP_CHECK(hipGetDevice(&dev));
+  TFCC_REQUIRE(dev >= 0 && dev < 16, "device index %d", dev);
+  if (!attrSet[dev]) {
     TFCC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    attrSet = true;
+    attrSet[dev] = true;
   }
   hipLaunchKernelGGL(kern, dim3(p.chunk * 8), dim3(kThreads), lds, stream, p);
   return check_launch("quantized matmul");

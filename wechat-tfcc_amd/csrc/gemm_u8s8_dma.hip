@@ -394,11 +394,14 @@ int launch(hipStream_t stream, QGemmParams p) {
   constexpr size_t lds = ring > epi ? ring : epi;
   static_assert(lds <= 160 * 1024, "LDS budget");
   auto kern = qgemm_dma_kernel<BM, BN, WGM, WGN, STAGES, REQUANT>;
-  static bool attrSet = false;
-  if (!attrSet) {
+  static bool attrSet[16] = {};  // per device: the attribute belongs to the function on one device
+  int dev = 0;
+  TFCC_HIP_CHECK(hipGetDevice(&dev));
+  TFCC_REQUIRE(dev >= 0 && dev < 16, "device index %d", dev);
+  if (!attrSet[dev]) {
     TFCC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    attrSet = true;
+    attrSet[dev] = true;
   }
   hipLaunchKernelGGL(kern, dim3(p.chunk * 8), dim3(kThreads), lds, stream, p);
   return check_launch("quantized matmul (dma)");

@@ -215,12 +215,15 @@ __device__ __forceinline__ float dec(unsigned u) {
   return __uint_as_float((u & 0x80000000u) ? (u & 0x7fffffffu) : ~u);
 }
 
-__global__ void minmax_init_kernel(unsigned* scratch) {
-  scratch[0] = 0xffffffffu;  // min
-  scratch[1] = 0u;           // max
+// The running minimum / maximum live, order-encoded as unsigned words, in the caller's own result words
+// until the finish kernel decodes them in place: no scratch memory that calls on other streams could share.
+__global__ void minmax_init_kernel(unsigned* mnWord, unsigned* mxWord) {
+  *mnWord = 0xffffffffu;
+  *mxWord = 0u;
 }
 
-__global__ __launch_bounds__(256) void minmax_kernel(const float* in, size_t total, unsigned* scratch) {
+__global__ __launch_bounds__(256) void minmax_kernel(const float* in, size_t total, unsigned* mnWord,
+                                                     unsigned* mxWord) {
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   const size_t step = (size_t)gridDim.x * blockDim.x;
   float mn = 3.402823466e+38f, mx = -3.402823466e+38f;
@@ -235,14 +238,14 @@ __global__ __launch_bounds__(256) void minmax_kernel(const float* in, size_t tot
     mx = fmaxf(mx, __shfl_down(mx, off, 64));
   }
   if ((threadIdx.x & 63) == 0) {
-    atomicMin(&scratch[0], enc(mn));
-    atomicMax(&scratch[1], enc(mx));
+    atomicMin(mnWord, enc(mn));
+    atomicMax(mxWord, enc(mx));
   }
 }
 
-__global__ void minmax_finish_kernel(const unsigned* scratch, float* mn, float* mx) {
-  *mn = dec(scratch[0]);
-  *mx = dec(scratch[1]);
+__global__ void minmax_finish_kernel(float* mn, float* mx) {
+  *mn = dec(*reinterpret_cast<const unsigned*>(mn));
+  *mx = dec(*reinterpret_cast<const unsigned*>(mx));
 }
 
 unsigned grid_for(size_t total, unsigned perThread = 1) {
@@ -287,9 +290,6 @@ int reduce_cols(hipStream_t s, const void* a, unsigned batch, unsigned row, unsi
                        static_cast<const T*>(a), row, col, rowsPerSlab, out);
   return check_launch("reduce_sum cols");
 }
-
-// scratch for quantize_minmax: two words per device, allocated once
-unsigned* g_minmax[16] = {};
 
 }  // namespace
 }  // namespace tfcc_rocm
@@ -366,14 +366,12 @@ int tfcc_rocm_quantize_minmax(void* stream, const float* in, uint64_t total, voi
   TFCC_REQUIRE(in && out && min_v && max_v, "quantize: null argument");
   TFCC_REQUIRE(total > 0, "quantize: empty tensor");
   TFCC_REQUIRE(valid_type(out_type), "quantize: bad type code");
-  int dev = 0;
-  TFCC_HIP_CHECK(hipGetDevice(&dev));
-  TFCC_REQUIRE(dev >= 0 && dev < 16, "quantize: device index %d", dev);
-  if (!g_minmax[dev]) TFCC_HIP_CHECK(hipMalloc(reinterpret_cast<void**>(&g_minmax[dev]), 2 * sizeof(unsigned)));
   hipStream_t s = as_stream(stream);
-  hipLaunchKernelGGL(minmax_init_kernel, dim3(1), dim3(1), 0, s, g_minmax[dev]);
-  hipLaunchKernelGGL(minmax_kernel, dim3(grid_for(total, 4)), dim3(256), 0, s, in, (size_t)total, g_minmax[dev]);
-  hipLaunchKernelGGL(minmax_finish_kernel, dim3(1), dim3(1), 0, s, g_minmax[dev], min_v, max_v);
+  unsigned* mnWord = reinterpret_cast<unsigned*>(min_v);
+  unsigned* mxWord = reinterpret_cast<unsigned*>(max_v);
+  hipLaunchKernelGGL(minmax_init_kernel, dim3(1), dim3(1), 0, s, mnWord, mxWord);
+  hipLaunchKernelGGL(minmax_kernel, dim3(grid_for(total, 4)), dim3(256), 0, s, in, (size_t)total, mnWord, mxWord);
+  hipLaunchKernelGGL(minmax_finish_kernel, dim3(1), dim3(1), 0, s, min_v, max_v);
   hipLaunchKernelGGL(quantize_kernel, dim3(grid_for(total)), dim3(256), 0, s, in, (size_t)total, min_v, max_v, out,
                      out_type, 1);
   return check_launch("quantize");

@@ -354,11 +354,14 @@ int launch(hipStream_t stream, SgemmParams p) {
   constexpr size_t lds = KSPLIT * 2 * (size_t)(BM + BN) * BK * sizeof(float);
   static_assert(lds <= 160 * 1024 && (size_t)(KSPLIT - 1) * BM * BN * sizeof(float) <= lds, "LDS budget");
   auto kern = sgemm_kernel<WGM, WGN, MI, NI, VEC, KSPLIT, TRANSB>;
-  static bool attrSet = false;
-  if (!attrSet) {
+  static bool attrSet[16] = {};  // per device: the attribute belongs to the function on one device
+  int dev = 0;
+  TFCC_HIP_CHECK(hipGetDevice(&dev));
+  TFCC_REQUIRE(dev >= 0 && dev < 16, "device index %d", dev);
+  if (!attrSet[dev]) {
     TFCC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    attrSet = true;
+    attrSet[dev] = true;
   }
   hipLaunchKernelGGL(kern, dim3(p.chunk * 8), dim3(WGM * WGN * 64 * KSPLIT), lds, stream, p);
   return check_launch("sgemm");
