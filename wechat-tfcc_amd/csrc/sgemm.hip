@@ -113,6 +113,32 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_kernel(const Sg
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
+  // The residual values this lane adds in the store are fetched now, in the small-tile configurations where
+  // the launch is short and a load issued at the end would be waited for in full.
+  float bv[NI];  // bias of this lane's columns, fetched before the main loop for the same reason
+  {
+    const unsigned col0 = n0 + wn * WN + NI * (lane & 31);
+#pragma unroll
+    for (int j = 0; j < NI; ++j) bv[j] = (biasPtr && col0 + j < N) ? biasPtr[col0 + j] : 0.f;
+  }
+  constexpr bool EARLY_RESIDUAL = MI * NI * 16 <= 32;
+  float rv[EARLY_RESIDUAL ? MI : 1][EARLY_RESIDUAL ? NI : 1][16];
+  if constexpr (EARLY_RESIDUAL) {
+    if (p.residual && grp == 0) {
+      const float* Rp = p.residual + (size_t)bi * p.strideR;
+      const unsigned col0 = n0 + wn * WN + NI * (lane & 31);
+#pragma unroll
+      for (int i = 0; i < MI; ++i)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const unsigned grow = m0 + wm * WM + i * 32 + 8 * (r / 4) + 4 * (lane >> 5) + (r & 3);
+#pragma unroll
+          for (int j = 0; j < NI; ++j)
+            rv[i][j][r] = (grow < M && col0 + j < N) ? Rp[(size_t)grow * N + col0 + j] : 0.f;
+        }
+    }
+  }
+
   v4f aReg[A_ITEMS];
   v4f bReg[B_ITEMS][TRANSB ? 1 : 4];
 
@@ -300,9 +326,6 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_kernel(const Sg
   const float* __restrict__ R = p.residual ? p.residual + (size_t)bi * p.strideR : nullptr;  // dense, flat batch
   const int act = p.act;
   const unsigned gcol = n0 + wn * WN + NI * lrow;
-  float bv[NI];
-#pragma unroll
-  for (int j = 0; j < NI; ++j) bv[j] = (biasPtr && gcol + j < N) ? biasPtr[gcol + j] : 0.f;
   const bool vecOK = VEC && (gcol + NI <= N);
 #pragma unroll
   for (int i = 0; i < MI; ++i) {
@@ -315,10 +338,15 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_kernel(const Sg
       for (int j = 0; j < NI; ++j) v[j] = acc[i][j][r] + bv[j];
       const size_t off = (size_t)grow * ldc + gcol;
       if (R) {
-        const size_t roff = (size_t)grow * N + gcol;
+        if constexpr (EARLY_RESIDUAL) {
 #pragma unroll
-        for (int j = 0; j < NI; ++j)
-          if (gcol + j < N) v[j] += R[roff + j];
+          for (int j = 0; j < NI; ++j) v[j] += rv[i][j][r];
+        } else {
+          const size_t roff = (size_t)grow * N + gcol;
+#pragma unroll
+          for (int j = 0; j < NI; ++j)
+            if (gcol + j < N) v[j] += R[roff + j];
+        }
       }
       if (act == 1) {
         // same expression as the stand-alone GELU kernel, so that fusing changes no bit
