@@ -130,6 +130,17 @@ __global__ __launch_bounds__(WGM * WGN * 64, 2) void qgemm_dma_kernel(const QGem
     }
   }
 
+  // The caller's row / column sums this thread turns into offset terms after the main loop are fetched now:
+  // at the end their latency would be waited for in full (one tile per CU, nothing to overlap it with).
+  static_assert(BM <= kThreads && BN <= kThreads, "one row sum and one column sum per thread");
+  unsigned rsPre = 0, csPre = 0;
+  {
+    const int* rsA = p.rowsumA + (size_t)bi * p.strideRA;
+    const int* csB = p.colsumB + (size_t)bi * p.strideRB;
+    if (tid < BM && m0 + tid < M) rsPre = (unsigned)rsA[m0 + tid];
+    if (tid < BN && n0 + tid < N) csPre = (unsigned)csB[n0 + tid];
+  }
+
   // ---- per-thread copy descriptors: which 16 bytes of the slab this lane moves in each copy.
   // LDS slot s (16 bytes) of the A image holds row s/8, physical chunk s%8 = logical chunk ^ swzA(row).
   unsigned aOff[A_COPIES], bOff[B_COPIES];  // byte offsets into A / B for slab 0
@@ -297,19 +308,9 @@ __global__ __launch_bounds__(WGM * WGN * 64, 2) void qgemm_dma_kernel(const QGem
     }
   }
   __syncthreads();
-  const int* rsA = p.rowsumA + (size_t)bi * p.strideRA;
-  const int* csB = p.colsumB + (size_t)bi * p.strideRB;
   const unsigned global = (unsigned)offA * (unsigned)offB * K;
-  for (int i = tid; i < BN; i += kThreads) {
-    unsigned gn = n0 + i;
-    unsigned cs = gn < N ? (unsigned)csB[gn] : 0u;
-    colTerm[i] = (int)(128u * (unsigned)colTerm[i] + cs * (unsigned)offA);
-  }
-  for (int i = tid; i < BM; i += kThreads) {
-    unsigned gm = m0 + i;
-    unsigned rs = gm < M ? (unsigned)rsA[gm] : 0u;
-    rowTerm[i] = (int)(global + rs * (unsigned)offB);
-  }
+  if (tid < BN) colTerm[tid] = (int)(128u * (unsigned)colTerm[tid] + csPre * (unsigned)offA);
+  if (tid < BM) rowTerm[tid] = (int)(global + rsPre * (unsigned)offB);
   __syncthreads();
 
   RequantScalars rq;
