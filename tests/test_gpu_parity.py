@@ -432,6 +432,14 @@ def test_elementwise_against_oracle(pkg, T):
     x = rng.normal(0, 1, (1024, 768)).astype(np.float32)
     g, b = rng.normal(1, 0.1, 768).astype(np.float32), rng.normal(0, 0.1, 768).astype(np.float32)
     assert np.allclose(T.n(pkg.layer_norm(T.t(x), T.t(g), T.t(b), 1e-12)), O.layer_norm(x, g, b, 1e-12), rtol=1e-5, atol=1e-5)
+    for rows, cols in ((3, 1), (5, 255), (4, 1024), (2, 1025), (3, 3000)):  # register-resident rows and long rows
+        xr = rng.normal(0.5, 2, (rows, cols)).astype(np.float32)
+        gr, br = rng.normal(1, 0.1, cols).astype(np.float32), rng.normal(0, 0.1, cols).astype(np.float32)
+        assert np.allclose(T.n(pkg.layer_norm(T.t(xr), T.t(gr), T.t(br), 1e-5)), O.layer_norm(xr, gr, br, 1e-5),
+                           rtol=1e-5, atol=1e-5)
+    for op, ref in (("sub", np.subtract), ("mul", np.multiply), ("div", np.divide)):
+        assert np.array_equal(T.n(pkg.binary(op, T.t(x), T.t(g))), ref(x, g))
+    assert np.array_equal(T.n(pkg.transform2(T.t(x), 3.0, 0.5)), x / np.float32(3.0) + np.float32(0.5))
     assert np.allclose(T.n(pkg.gelu_accurate(T.t(x))), O.gelu_accurate(x), rtol=1e-6, atol=1e-7)
     assert np.array_equal(T.n(pkg.transform(T.t(x), 0.125, 0.0)), x * np.float32(0.125))
     assert np.array_equal(T.n(pkg.add(T.t(x), T.t(g))), x + g)

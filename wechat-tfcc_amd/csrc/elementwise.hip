@@ -108,6 +108,43 @@ __global__ __launch_bounds__(256) void layer_norm_kernel(const float* in, const 
   for (unsigned i = threadIdx.x; i < cols; i += 256) o[i] = (a[i] - mean) * (inv * gamma[i]) + beta[i];
 }
 
+// rows of at most 256 * PER columns: the row, gamma and beta are read once and stay in registers (same sums
+// in the same order as the kernel above)
+template <int PER>
+__global__ __launch_bounds__(256) void layer_norm_reg_kernel(const float* in, const float* gamma, const float* beta,
+                                                             float eps, unsigned cols, float* out) {
+  __shared__ float sh[4];
+  const float* a = in + (size_t)blockIdx.x * cols;
+  float* o = out + (size_t)blockIdx.x * cols;
+  float x[PER], gm[PER], bt[PER];
+#pragma unroll
+  for (int q = 0; q < PER; ++q) {
+    const unsigned i = threadIdx.x + 256 * q;
+    x[q] = i < cols ? a[i] : 0.f;
+    gm[q] = i < cols ? gamma[i] : 0.f;
+    bt[q] = i < cols ? beta[i] : 0.f;
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int q = 0; q < PER; ++q)
+    if (threadIdx.x + 256 * q < cols) s += x[q];
+  const float mean = block_reduce<false>(s, sh) / (float)cols;
+  float v = 0.f;
+#pragma unroll
+  for (int q = 0; q < PER; ++q)
+    if (threadIdx.x + 256 * q < cols) {
+      float t = x[q] - mean;
+      v += t * t;
+    }
+  const float var = block_reduce<false>(v, sh) / (float)cols;
+  const float inv = 1.0f / sqrtf(var + eps);
+#pragma unroll
+  for (int q = 0; q < PER; ++q) {
+    const unsigned i = threadIdx.x + 256 * q;
+    if (i < cols) o[i] = (x[q] - mean) * (inv * gm[q]) + bt[q];
+  }
+}
+
 __global__ __launch_bounds__(256) void gelu_kernel(const float* in, size_t total, float* out) {
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   const size_t step = (size_t)gridDim.x * blockDim.x;
@@ -219,8 +256,12 @@ int tfcc_rocm_layer_norm_f32(void* stream, const float* in, const float* gamma, 
   TFCC_REQUIRE(in && gamma && beta && out, "layer_norm: null argument");
   TFCC_REQUIRE(rows > 0 && cols > 0, "layer_norm: empty tensor");
   TFCC_REQUIRE(rows < (1ull << 31), "layer_norm: too many rows");
-  hipLaunchKernelGGL(layer_norm_kernel, dim3((unsigned)rows), dim3(256), 0, as_stream(stream), in, gamma, beta,
-                     epsilon, cols, out);
+  if (cols <= 256 * 4)
+    hipLaunchKernelGGL(layer_norm_reg_kernel<4>, dim3((unsigned)rows), dim3(256), 0, as_stream(stream), in, gamma, beta,
+                       epsilon, cols, out);
+  else
+    hipLaunchKernelGGL(layer_norm_kernel, dim3((unsigned)rows), dim3(256), 0, as_stream(stream), in, gamma, beta,
+                       epsilon, cols, out);
   return check_launch("layer_norm");
 }
 
