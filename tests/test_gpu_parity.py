@@ -20,25 +20,8 @@ def wrap32(x):
     return (np.asarray(x, np.int64) & 0xFFFFFFFF).astype(np.uint32).view(np.int32)
 
 
-@pytest.fixture(scope="module")
-def T(dev):
-    import torch
+from conftest import rel_fro  # noqa: E402
 
-    class Helper:
-        def t(self, x):
-            return torch.from_numpy(np.ascontiguousarray(x)).to(dev)
-
-        def f1(self, v):
-            return torch.tensor([v], dtype=torch.float32, device=dev)
-
-        def n(self, x):
-            torch.cuda.synchronize()
-            return x.cpu().numpy()
-    return Helper()
-
-
-def rel_fro(got, want64):
-    return np.linalg.norm(got.astype(np.float64) - want64) / max(np.linalg.norm(want64), 1e-300)
 
 
 # ---- quantized matmul ----------------------------------------------------------------------------
