@@ -184,6 +184,31 @@ def bench_other(torch, pkg, dev, steps, warmup, c3):
     sgemm_case("c2_fp32_qk_16x12x128x64x128", (16, 12, 128, 64), (16, 12, 64, 128), False)
     sgemm_case("c2_fp32_pv_16x12x128x128x64", (16, 12, 128, 128), (16, 12, 128, 64), False)
     sgemm_case("c4_fp32_ffn_up_1024x768x3072_bias", (8, 128, 768), (768, 3072), True)
+
+    # C2 as one launch: softmax(q k^T / 8) v on [batch, seq, heads, size] tensors, 16 x 12 heads of 128 x 64
+    def attention_case(name, B, H, S, D, sets=4):
+        bufs = []
+        for _ in range(sets):
+            q, k, v = (torch.randn((B, S, H, D), device=dev, dtype=torch.float32) for _ in range(3))
+            o = torch.empty((B, S, H, D), device=dev, dtype=torch.float32)
+            bufs.append((pkg.attention_desc(q, k, v, o, S, S, D, (H * D,) * 4, batch_outer=B, batch_inner=H,
+                                            strides=(S * H * D,) * 4, inner_strides=(D,) * 4, divisor=8.0), (q, k, v, o)))
+        idx = [0]
+
+        def step():
+            desc = bufs[idx[0] % sets][0]
+            idx[0] += 1
+            st = lib.tfcc_rocm_attention_f32(stream, desc)
+            if st != 0:
+                pkg.check(st)
+        ms = time_launches(torch, step, steps, warmup, pkg, stream)
+        flop = 4.0 * B * H * S * S * D
+        nbytes = 4.0 * 4 * B * S * H * D
+        out[name] = {"ms": round(ms, 5), "tflops": round(flop / ms / 1e9, 3),
+                     "frac_fp32_mfma": round(flop / ms / 1e9 / PEAK_FP32_TFLOPS, 4), "gbs": round(nbytes / ms / 1e6, 1),
+                     "frac_hbm": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
+
+    attention_case("c2_fp32_attention_one_launch_16x12x128x64", 16, 12, 128, 64)
     sgemm_case("fp32_4096x4096x4096", (4096, 4096), (4096, 4096), False, sets=1)
 
     # C3 with the int32 accumulators also written (67 MB more traffic)

@@ -244,6 +244,31 @@ int tfcc_rocm_softmax_f32(void* stream, const float* in, uint64_t rows, unsigned
  * `a / s` (tfcc/core/operations/tfcc_operator.cpp:78-95) followed by softmax, in one pass */
 int tfcc_rocm_softmax_div_f32(void* stream, const float* in, uint64_t rows, unsigned cols, float divisor,
                               float* out);
+/* out = softmax(q k^T [/ divisor]) v for every entry of an outer x inner batch grid, in one launch:
+ * q is [s, d], k and v are [t, d], out is [s, d], each with a row stride and two batch strides of its
+ * own (in elements), so that the per-head matrices of [batch, seq, heads, size] tensors are used where
+ * they lie.  It stands for the node sequence Transpose x3 -> Matmul -> Div -> Softmax -> Matmul ->
+ * Transpose that the reference's runtime runs one operation at a time
+ * (tfcc_runtime/operations/math/matmul.cpp:27-41, softmax.cpp, base/transpose.cpp) and returns what
+ * tfcc_rocm_sgemm_general (trans_b) + tfcc_rocm_softmax_div_f32 + tfcc_rocm_sgemm_general return, bit
+ * for bit.  Limits: t <= 128, d <= 64 and a multiple of 4, input strides multiples of 4, inputs 16-byte
+ * aligned; tfcc_rocm_attention_f32_supported() tells (1 / 0) whether a descriptor is within them.
+ * out must not overlap the inputs. */
+typedef struct tfcc_rocm_attention_desc {
+  const float* q;
+  const float* k;
+  const float* v;
+  float* out;
+  unsigned s, t, d;
+  unsigned ldq, ldk, ldv, ldo;
+  unsigned batch_outer, batch_inner;
+  uint64_t stride_q, stride_k, stride_v, stride_out;                         /* between outer entries */
+  uint64_t inner_stride_q, inner_stride_k, inner_stride_v, inner_stride_out; /* between inner entries */
+  float divisor;
+  int has_divisor; /* 0: plain softmax(q k^T) */
+} tfcc_rocm_attention_desc;
+int tfcc_rocm_attention_f32_supported(const tfcc_rocm_attention_desc* desc);
+int tfcc_rocm_attention_f32(void* stream, const tfcc_rocm_attention_desc* desc);
 /* _mkl_layer_normalize, tfcc/mkl/interfaces/tfcc_mklnormalizationinterface.cpp:29-62 */
 int tfcc_rocm_layer_norm_f32(void* stream, const float* in, const float* gamma, const float* beta,
                              float epsilon, uint64_t rows, unsigned cols, float* out);

@@ -1,0 +1,114 @@
+"""softmax(q k^T / divisor) v in one launch against (a) the three separate kernels, bit for bit, and
+(b) a float64 restatement of the node sequence of tfcc_runtime/operations/math/matmul.cpp:27-41,
+softmax.cpp and tfcc/core/operations/tfcc_operator.cpp:78-95 within 1e-5 relative Frobenius error."""
+import numpy as np
+import pytest
+
+from conftest import rel_fro
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture
+def gpu(T):
+    return T
+
+
+def reference64(q, k, v, divisor):
+    s = np.einsum("bhsd,bhtd->bhst", q.astype(np.float64), k.astype(np.float64))
+    if divisor is not None:
+        s = s / divisor
+    s = s - s.max(axis=-1, keepdims=True)
+    e = np.exp(s)
+    p = e / e.sum(axis=-1, keepdims=True)
+    return np.einsum("bhst,bhtd->bhsd", p, v.astype(np.float64))
+
+
+def separate_kernels(pkg, torch, q, k, v, B, H, S, T, D, divisor, layout):
+    """The same result from two products and one softmax, each in a launch of its own."""
+    dev = q.device
+    scores = torch.empty((B, H, S, T), dtype=torch.float32, device=dev)
+    if layout == "bshd":
+        sq, iq, ldq = (S * H * D, H * D), D, H * D
+        sk, ldk = T * H * D, H * D
+    else:
+        sq, iq, ldq = (H * S * D,), S * D, D
+        sk, ldk = H * T * D, D
+    ik = D if layout == "bshd" else T * D
+    pkg.sgemm_general(q, k, scores, S, T, D, ldq, ldk, T, trans_b=True, batch_outer=B, batch_inner=H,
+                      strides=(sq[0], sk, H * S * T), inner_strides=(iq, ik, S * T))
+    probs = torch.empty_like(scores)
+    if divisor is None:
+        pkg.check(pkg.lib().tfcc_rocm_softmax_f32(pkg._stream(), scores.data_ptr(), B * H * S, T, probs.data_ptr()))
+    else:
+        pkg.check(pkg.lib().tfcc_rocm_softmax_div_f32(pkg._stream(), scores.data_ptr(), B * H * S, T, divisor,
+                                                      probs.data_ptr()))
+    out = torch.empty((B, S, H, D) if layout == "bshd" else (B, H, S, D), dtype=torch.float32, device=dev)
+    if layout == "bshd":
+        so, io, ldo = S * H * D, D, H * D
+    else:
+        so, io, ldo = H * S * D, S * D, D
+    pkg.sgemm_general(probs, v, out, S, D, T, T, ldk, ldo, batch_outer=B, batch_inner=H,
+                      strides=(H * S * T, sk, so), inner_strides=(S * T, ik, io))
+    return out
+
+
+CASES = [
+    # B, H, S, T, D, divisor, layout
+    (2, 12, 128, 128, 64, 8.0, "bshd"),     # the encoder layer's attention core
+    (1, 3, 100, 77, 36, 6.0, "bshd"),       # ragged everywhere, head width not a multiple of 8
+    (2, 2, 200, 128, 64, None, "bhsd"),     # several row blocks, no divisor, dense per-head matrices
+    (1, 1, 1, 1, 4, 2.0, "bhsd"),           # the smallest
+    (3, 5, 64, 5, 4, 0.5, "bshd"),
+    (1, 4, 65, 64, 32, 5.656854, "bhsd"),   # one row past a block; only the first column half is live
+    (1, 2, 31, 97, 60, 7.75, "bshd"),
+]
+
+
+@pytest.mark.parametrize("B,H,S,Tk,D,divisor,layout", CASES)
+def test_attention_equals_separate_kernels(pkg, gpu, B, H, S, Tk, D, divisor, layout):
+    import torch
+    rng = np.random.default_rng(B * 1000 + S * 7 + Tk * 3 + D)
+    if layout == "bshd":
+        shape_q, shape_kv = (B, S, H, D), (B, Tk, H, D)
+        to_bhxd = lambda x: x.transpose(0, 2, 1, 3)
+    else:
+        shape_q, shape_kv = (B, H, S, D), (B, H, Tk, D)
+        to_bhxd = lambda x: x
+    q = rng.standard_normal(shape_q).astype(np.float32)
+    k = rng.standard_normal(shape_kv).astype(np.float32)
+    v = rng.standard_normal(shape_kv).astype(np.float32)
+    tq, tk, tv = gpu.t(q), gpu.t(k), gpu.t(v)
+    out = torch.full(shape_q, float("nan"), dtype=torch.float32, device=tq.device)
+    if layout == "bshd":
+        ld = (H * D,) * 4
+        strides = (S * H * D, Tk * H * D, Tk * H * D, S * H * D)
+        inner = (D, D, D, D)
+    else:
+        ld = (D,) * 4
+        strides = (H * S * D, H * Tk * D, H * Tk * D, H * S * D)
+        inner = (S * D, Tk * D, Tk * D, S * D)
+    desc = pkg.attention_desc(tq, tk, tv, out, S, Tk, D, ld, batch_outer=B, batch_inner=H, strides=strides,
+                              inner_strides=inner, divisor=divisor)
+    assert pkg.attention_supported(desc)
+    pkg.attention(desc)
+    got = gpu.n(out)
+    assert np.isfinite(got).all()
+    want = gpu.n(separate_kernels(pkg, torch, tq, tk, tv, B, H, S, Tk, D, divisor, layout))
+    assert np.array_equal(got, want), "fused and separate kernels differ by %g" % np.abs(got - want).max()
+    ref = reference64(to_bhxd(q), to_bhxd(k), to_bhxd(v), divisor)
+    assert rel_fro(to_bhxd(got), ref) <= 1e-5
+
+
+def test_attention_limits_are_reported(pkg, gpu):
+    import torch
+    x = torch.zeros(256 * 256, dtype=torch.float32, device=gpu.t(np.zeros(1, np.float32)).device)
+    ok = pkg.attention_desc(x, x, x, x, 16, 128, 64, (64,) * 4)
+    assert pkg.attention_supported(ok)
+    for s, t, d, ld in [(16, 129, 64, 64), (16, 16, 68, 68), (16, 16, 6, 8), (16, 16, 8, 10)]:
+        bad = pkg.attention_desc(x, x, x, x, s, t, d, (ld,) * 4)
+        assert not pkg.attention_supported(bad)
+        with pytest.raises(pkg.TfccRocmError):
+            pkg.attention(bad)
+    with pytest.raises(pkg.TfccRocmError):
+        pkg.attention(pkg.attention_desc(x, x, x, x, 0, 16, 8, (8,) * 4))

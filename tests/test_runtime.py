@@ -232,7 +232,8 @@ def test_replay_reproduces_step_by_step_results(mf, rt, dev):
 @pytest.mark.gpu
 def test_fused_graph_is_bit_identical_to_the_graph_as_written(mf, rt, dev):
     rng = np.random.default_rng(7)
-    for batch, seq, hidden, heads, ffn in ((2, 16, 64, 4, 128), (3, 7, 96, 3, 200), (4, 128, 256, 4, 1024)):
+    for batch, seq, hidden, heads, ffn in ((2, 16, 64, 4, 128), (3, 7, 96, 3, 200), (4, 128, 256, 4, 1024),
+                                           (1, 160, 64, 2, 128), (2, 9, 60, 4, 64)):
         w = mf.bert_layer_weights(rng, hidden, ffn)
         g = mf.bert_encoder_layer(w, batch, seq, heads)
         blob = mf.write_model([g], g.name)
@@ -243,9 +244,10 @@ def test_fused_graph_is_bit_identical_to_the_graph_as_written(mf, rt, dev):
         rt.set_fusion(True)
         fused = rt.Model(blob)
         got = fused.run({"hidden_states": x})["layer_output"]
-        # matmul+gelu, 2 x matmul+add and div+softmax each save one step, the four transposes around the
-        # two batched products are folded into them, query / key / value projections share one launch
-        assert plain.step_count() - fused.step_count() == 10
+        # matmul+gelu and 2 x matmul+add each save one step, query / key / value projections share one launch,
+        # the four transposes, the two batched products, the division and the softmax between them are one
+        # step (one launch up to 128 keys and head size 64, three launches in the last two cases)
+        assert plain.step_count() - fused.step_count() == 12
         assert np.array_equal(got, want)
         fused.set_replay(True)
         for _ in range(3):
@@ -265,6 +267,29 @@ def test_fused_graph_is_bit_identical_to_the_graph_as_written(mf, rt, dev):
         outs.append(rt.Model(mf.write_model([g], "g")).run({"a": av})[y])
     rt.set_fusion(True)
     assert np.array_equal(outs[0], outs[1])
+    # softmax(q k^T) v without a division, from per-head tensors; then with keys given as [.., size, keys],
+    # a layout the one-launch form does not take
+    for keys_transposed in (True, False):
+        g = mf.GraphBuilder("g")
+        q = g.input("q", mf.FLOAT, [2, 3, 20, 8])
+        k = g.input("k", mf.FLOAT, [2, 3, 24, 8] if keys_transposed else [2, 3, 8, 24])
+        v = g.input("v", mf.FLOAT, [2, 3, 24, 8])
+        y = g.matmul(g.softmax(g.matmul(q, g.transpose(k, [0, 1, 3, 2]) if keys_transposed else k), 3), v)
+        g.output(y)
+        feeds = {"q": rng.normal(size=(2, 3, 20, 8)).astype(np.float32),
+                 "k": rng.normal(size=(2, 3, 24, 8) if keys_transposed else (2, 3, 8, 24)).astype(np.float32),
+                 "v": rng.normal(size=(2, 3, 24, 8)).astype(np.float32)}
+        outs = []
+        for enable in (False, True):
+            rt.set_fusion(enable)
+            outs.append(rt.Model(mf.write_model([g], "g")).run(feeds)[y])
+        rt.set_fusion(True)
+        kt = feeds["k"].transpose(0, 1, 3, 2) if keys_transposed else feeds["k"]
+        sc = np.matmul(feeds["q"].astype(np.float64), kt.astype(np.float64))
+        e = np.exp(sc - sc.max(axis=-1, keepdims=True))
+        want = np.matmul(e / e.sum(axis=-1, keepdims=True), feeds["v"].astype(np.float64))
+        assert np.array_equal(outs[0], outs[1])
+        assert rel_frobenius(outs[1], want) <= 1e-5
     # transposes around a batched product in layouts the strided kernel takes (k or n contiguous) and does
     # not take (A with k strided: falls back to the nodes as written)
     for perm_a, perm_b, perm_c in (([0, 2, 1, 3], [0, 2, 3, 1], None), ([0, 1, 3, 2], None, [0, 2, 1, 3]),

@@ -54,6 +54,20 @@ class SgemmDesc(C.Structure):
     ]
 
 
+class AttentionDesc(C.Structure):
+    """tfcc_rocm_attention_desc"""
+    _fields_ = [
+        ("q", C.c_void_p), ("k", C.c_void_p), ("v", C.c_void_p), ("out", C.c_void_p),
+        ("s", C.c_uint), ("t", C.c_uint), ("d", C.c_uint),
+        ("ldq", C.c_uint), ("ldk", C.c_uint), ("ldv", C.c_uint), ("ldo", C.c_uint),
+        ("batch_outer", C.c_uint), ("batch_inner", C.c_uint),
+        ("stride_q", C.c_uint64), ("stride_k", C.c_uint64), ("stride_v", C.c_uint64), ("stride_out", C.c_uint64),
+        ("inner_stride_q", C.c_uint64), ("inner_stride_k", C.c_uint64), ("inner_stride_v", C.c_uint64),
+        ("inner_stride_out", C.c_uint64),
+        ("divisor", C.c_float), ("has_divisor", C.c_int),
+    ]
+
+
 # name -> (restype, argtypes): every symbol include/tfcc_rocm.h declares
 _VP, _U64, _U, _I, _F, _D, _I64 = C.c_void_p, C.c_uint64, C.c_uint, C.c_int, C.c_float, C.c_double, C.c_int64
 SYMBOLS = {
@@ -102,6 +116,8 @@ SYMBOLS = {
     "tfcc_rocm_sgemm_general": (_I, [_VP, _VP]),
     "tfcc_rocm_sgemm_grouped": (_I, [_VP, _VP, C.POINTER(_VP), C.POINTER(_VP), C.POINTER(_VP), _U, _U, _U, _U]),
     "tfcc_rocm_softmax_div_f32": (_I, [_VP, _VP, _U64, _U, _F, _VP]),
+    "tfcc_rocm_attention_f32_supported": (_I, [C.POINTER(AttentionDesc)]),
+    "tfcc_rocm_attention_f32": (_I, [_VP, C.POINTER(AttentionDesc)]),
     "tfcc_rocm_transform2_f32": (_I, [_VP, _VP, _U64, _F, _F, _VP]),
     "tfcc_rocm_binary_f32": (_I, [_VP, _I, _VP, _VP, _U64, _U64, _VP]),
     "tfcc_rocm_transpose_f32": (_I, [_VP, _VP, C.POINTER(C.c_uint), C.POINTER(C.c_uint), _I, _VP]),
@@ -208,6 +224,30 @@ def sgemm_general(a, b, c, m, n, k, lda, ldb, ldc, trans_b=False, batch_outer=1,
     d.activation = activation
     check(lib().tfcc_rocm_sgemm_general(_stream(), C.byref(d)))
     return c
+
+
+def attention_desc(q, k, v, out, s, t, d, ld, batch_outer=1, batch_inner=1, strides=(0, 0, 0, 0),
+                   inner_strides=(0, 0, 0, 0), divisor=None):
+    """A tfcc_rocm_attention_desc over torch tensors used as raw buffers; ld = (ldq, ldk, ldv, ldo)."""
+    a = AttentionDesc()
+    a.q, a.k, a.v, a.out = _ptr(q), _ptr(k), _ptr(v), _ptr(out)
+    a.s, a.t, a.d = s, t, d
+    a.ldq, a.ldk, a.ldv, a.ldo = ld
+    a.batch_outer, a.batch_inner = batch_outer, batch_inner
+    a.stride_q, a.stride_k, a.stride_v, a.stride_out = strides
+    a.inner_stride_q, a.inner_stride_k, a.inner_stride_v, a.inner_stride_out = inner_strides
+    a.divisor = 1.0 if divisor is None else divisor
+    a.has_divisor = 0 if divisor is None else 1
+    return a
+
+
+def attention_supported(desc):
+    return bool(lib().tfcc_rocm_attention_f32_supported(C.byref(desc)))
+
+
+def attention(desc):
+    """tfcc_rocm_attention_f32: out = softmax(q k^T [/ divisor]) v per batch entry."""
+    check(lib().tfcc_rocm_attention_f32(_stream(), C.byref(desc)))
 
 
 def sgemm_grouped(a, bs, biases):

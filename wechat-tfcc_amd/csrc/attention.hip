@@ -1,0 +1,317 @@
+// softmax(Q K^T [/ divisor]) V per batch entry in one launch, for key sequences that fit in LDS.
+//
+// Stands where the reference's runtime runs the attention core of an encoder layer as separate
+// operations on tensors in HBM: Matmul (tfcc_runtime/operations/math/matmul.cpp:27-41), Div by a
+// value, Softmax (tfcc_runtime/operations/math/softmax.cpp), Matmul again, with base::transpose
+// (tfcc/core/operations/tfcc_base.cpp:124-134) before and after.  Here the score matrix of a block of
+// 64 query rows never leaves the CU.
+//
+// Every number is computed by the same instruction sequence as in the three separate kernels
+// (fp32 32x32x2 matrix ops over ascending k into one accumulator; the softmax of one row by one
+// wavefront holding columns l and l + 64), and is rounded to fp32 between the steps, so the result
+// equals theirs bit for bit.
+#include <float.h>
+
+#include "common.hpp"
+
+namespace tfcc_rocm {
+namespace {
+
+typedef float v4f __attribute__((ext_vector_type(4)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+constexpr int kRows = 64;        // query rows per workgroup
+constexpr int kThreads = 512;    // eight wavefronts
+constexpr int kMaxT = 128;       // key rows
+constexpr int kMaxD = 64;        // head width
+constexpr int kPitchQK = kMaxD + 4;   // floats; 128-bit row reads of 32 consecutive rows hit all banks once
+constexpr int kPitchV = kMaxD + 8;    // 32-bit reads of rows r and r + 4 land 32 banks apart
+constexpr int kPitchS = kMaxT + 4;
+constexpr int kLdsFloats = kRows * kPitchQK + kMaxT * kPitchQK + kMaxT * kPitchV + kRows * kPitchS;
+
+struct AttentionParams {
+  const float* Q;
+  const float* K;
+  const float* V;
+  float* O;
+  unsigned S, T, D;
+  unsigned ldq, ldk, ldv, ldo;
+  unsigned long long outerQ, outerK, outerV, outerO;
+  unsigned long long innerQ, innerK, innerV, innerO;
+  unsigned batchInner, blocksS, total, chunk;
+  float divisor;
+  int divide;
+};
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+__global__ __launch_bounds__(kThreads) void attention_kernel(const AttentionParams p) {
+  extern __shared__ __align__(16) float lds[];
+  float* Qs = lds;                        // [64][kPitchQK]
+  float* Ks = Qs + kRows * kPitchQK;      // [128][kPitchQK]
+  float* Vs = Ks + kMaxT * kPitchQK;      // [128][kPitchV]
+  float* Sc = Vs + kMaxT * kPitchV;       // [64][kPitchS]  scores, then probabilities
+
+  // consecutive workgroup ids land on different XCDs: the blocks of one head stay on one XCD
+  const unsigned wg = blockIdx.x;
+  const unsigned L = (wg & 7u) * p.chunk + (wg >> 3);
+  if ((wg >> 3) >= p.chunk || L >= p.total) return;
+  const unsigned bi = L / p.blocksS, blk = L - bi * p.blocksS;
+  const unsigned bo = bi / p.batchInner, bn = bi - bo * p.batchInner;
+  const unsigned s0 = blk * kRows;
+  const unsigned S = p.S, T = p.T, D = p.D;
+  const float* __restrict__ Q = p.Q + (size_t)bo * p.outerQ + (size_t)bn * p.innerQ;
+  const float* __restrict__ K = p.K + (size_t)bo * p.outerK + (size_t)bn * p.innerK;
+  const float* __restrict__ V = p.V + (size_t)bo * p.outerV + (size_t)bn * p.innerV;
+  float* __restrict__ O = p.O + (size_t)bo * p.outerO + (size_t)bn * p.innerO;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lrow = lane & 31, g = lane >> 5;
+  const unsigned Dp = (D + 7u) & ~7u;   // k extent of the score product
+  const unsigned Tp = (T + 7u) & ~7u;   // k extent of the second product
+
+  // ---- all three operands to LDS; everything past the operands' extents that a matrix op will read
+  // is zero: a buffer load whose offset lies past the end of its operand returns zero
+  {
+    constexpr int CH = kMaxD / 4;  // 16-byte chunks per row
+    constexpr int Q_ITEMS = kRows * CH / kThreads, KV_ITEMS = kMaxT * CH / kThreads;
+    constexpr unsigned kPastEnd = 0xfffffff0u;
+    const __amdgpu_buffer_rsrc_t rq = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(Q), 0, (int)(((S - 1) * p.ldq + D) * 4u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(K), 0, (int)(((T - 1) * p.ldk + D) * 4u), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(V), 0, (int)(((T - 1) * p.ldv + D) * 4u), 0x00020000);
+    v4f q[Q_ITEMS], k[KV_ITEMS], v[KV_ITEMS];
+#pragma unroll
+    for (int it = 0; it < Q_ITEMS; ++it) {
+      const unsigned w = tid + it * kThreads, row = s0 + w / CH, ch = w % CH;
+      const unsigned off = (row < S && ch * 4 < D) ? (row * p.ldq + ch * 4) * 4u : kPastEnd;
+      q[it] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rq, off, 0, 0));
+    }
+#pragma unroll
+    for (int it = 0; it < KV_ITEMS; ++it) {
+      const unsigned w = tid + it * kThreads, row = w / CH, ch = w % CH;
+      const bool in = row < T && ch * 4 < D;
+      k[it] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rk, in ? (row * p.ldk + ch * 4) * 4u : kPastEnd, 0, 0));
+      v[it] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rv, in ? (row * p.ldv + ch * 4) * 4u : kPastEnd, 0, 0));
+    }
+#pragma unroll
+    for (int it = 0; it < Q_ITEMS; ++it) {
+      const int w = tid + it * kThreads, row = w / CH, ch = w % CH;
+      *reinterpret_cast<v4f*>(Qs + row * kPitchQK + ch * 4) = q[it];
+    }
+#pragma unroll
+    for (int it = 0; it < KV_ITEMS; ++it) {
+      const int w = tid + it * kThreads, row = w / CH, ch = w % CH;
+      *reinterpret_cast<v4f*>(Ks + row * kPitchQK + ch * 4) = k[it];
+      *reinterpret_cast<v4f*>(Vs + row * kPitchV + ch * 4) = v[it];
+    }
+  }
+  __syncthreads();
+
+  // ---- scores: wavefront (wm, wn) of a 2 x 4 grid owns the 32 x 32 block at rows 32*wm, columns 32*wn
+  // of the 64 x 128 block.  All operands are fetched from LDS first, so that their latency is paid once.
+  // A divisor that is a power of two divides exactly like a multiplication by its reciprocal.
+  {
+    const int wm = wave >> 2, wn = wave & 3;
+    if ((unsigned)(32 * wn) < T) {
+      constexpr int KB = kMaxD / 8;
+      v16f acc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+      const float* qa = Qs + (32 * wm + lrow) * kPitchQK + 4 * g;
+      const float* ka = Ks + (32 * wn + lrow) * kPitchQK + 4 * g;
+      v4f af[KB], bf[KB];
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb) {
+        af[kb] = v4f{0.f, 0.f, 0.f, 0.f};
+        bf[kb] = v4f{0.f, 0.f, 0.f, 0.f};
+        if ((unsigned)kb * 8 < Dp) {
+          af[kb] = *reinterpret_cast<const v4f*>(qa + kb * 8);
+          bf[kb] = *reinterpret_cast<const v4f*>(ka + kb * 8);
+        }
+      }
+#pragma unroll
+      for (int kb = 0; kb < KB; ++kb) {
+        if ((unsigned)kb * 8 < Dp) {
+#pragma unroll
+          for (int s = 0; s < 4; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[kb][s], bf[kb][s], acc, 0, 0, 0);
+        }
+      }
+      float* sc = Sc + (32 * wm + 4 * g) * kPitchS + 32 * wn + lrow;
+      const float divisor = p.divisor;
+      const unsigned bits = __builtin_bit_cast(unsigned, divisor), expo = (bits >> 23) & 0xffu;
+      if (!p.divide) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sc[(8 * (r / 4) + (r & 3)) * kPitchS] = acc[r];
+      } else if ((bits & 0x007fffffu) == 0 && expo >= 2 && expo <= 252) {
+        const float inverse = 1.0f / divisor;  // exact: also a power of two
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sc[(8 * (r / 4) + (r & 3)) * kPitchS] = acc[r] * inverse;
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sc[(8 * (r / 4) + (r & 3)) * kPitchS] = acc[r] / divisor;
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- softmax of each row by one wavefront, eight rows in flight; columns T .. Tp-1 become the zeros
+  // the next product reads
+  {
+    const unsigned rows = min((unsigned)kRows, S - s0);
+    constexpr int R = 8, W = kThreads / 64;
+    for (unsigned base = wave; base < rows; base += W * R) {
+      float v[R][2], mx[R], sum[R];
+#pragma unroll
+      for (int u = 0; u < R; ++u) {
+        const unsigned row = min(base + W * u, (unsigned)kRows - 1);  // a row past the block's end is computed and dropped
+        const float* sc = Sc + row * kPitchS;
+        mx[u] = -FLT_MAX;
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+          const unsigned i = lane + 64 * q;
+          v[u][q] = i < T ? sc[i] : -FLT_MAX;
+          mx[u] = fmaxf(mx[u], v[u][q]);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < R; ++u) mx[u] = wave_max(mx[u]);
+#pragma unroll
+      for (int u = 0; u < R; ++u) {
+        sum[u] = 0.f;
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+          const unsigned i = lane + 64 * q;
+          v[u][q] = i < T ? expf(v[u][q] - mx[u]) : 0.f;
+          sum[u] += v[u][q];
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < R; ++u) sum[u] = wave_sum(sum[u]);
+#pragma unroll
+      for (int u = 0; u < R; ++u) {
+        const unsigned row = base + W * u;
+        if (row < rows) {
+          float* sc = Sc + row * kPitchS;
+#pragma unroll
+          for (int q = 0; q < 2; ++q) {
+            const unsigned i = lane + 64 * q;
+            sc[i] = i < T ? v[u][q] / sum[u] : 0.f;
+          }
+        }
+      }
+    }
+  }
+  __syncthreads();
+
+  // ---- probabilities x V: the first four wavefronts, (wm, wn) owning rows 32*wm.. and columns 32*wn.. of the
+  // 64 x D result (one accumulator per element over all of T, as in a product of its own)
+  const int wm = wave >> 1, wn = wave & 1;
+  if (wave < 4 && (unsigned)(32 * wn) < D) {
+    constexpr int KB = kMaxT / 8;
+    v16f acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+    const float* pa = Sc + (32 * wm + lrow) * kPitchS + 4 * g;
+    const float* vb = Vs + (4 * g) * kPitchV + 32 * wn + lrow;
+    v4f af[KB], bf[KB];
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) {
+      af[kb] = v4f{0.f, 0.f, 0.f, 0.f};
+      bf[kb] = v4f{0.f, 0.f, 0.f, 0.f};
+      if ((unsigned)kb * 8 < Tp) {
+        af[kb] = *reinterpret_cast<const v4f*>(pa + kb * 8);
+#pragma unroll
+        for (int s = 0; s < 4; ++s) bf[kb][s] = vb[(kb * 8 + s) * kPitchV];
+      }
+    }
+#pragma unroll
+    for (int kb = 0; kb < KB; ++kb) {
+      if ((unsigned)kb * 8 < Tp) {
+#pragma unroll
+        for (int s = 0; s < 4; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[kb][s], bf[kb][s], acc, 0, 0, 0);
+      }
+    }
+    const unsigned col = 32 * wn + lrow;
+    if (col < D) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const unsigned row = s0 + 32 * wm + 8 * (r / 4) + 4 * g + (r & 3);
+        if (row < S) O[(size_t)row * p.ldo + col] = acc[r];
+      }
+    }
+  }
+}
+
+const char* unsupported(const tfcc_rocm_attention_desc* d) {
+  if (d->t > (unsigned)kMaxT) return "more than 128 key rows";
+  if (d->d > (unsigned)kMaxD) return "head width above 64";
+  if (d->d % 4 != 0) return "head width not a multiple of 4";
+  if (d->ldq % 4 || d->ldk % 4 || d->ldv % 4) return "row stride not a multiple of 4 elements";
+  if (d->stride_q % 4 || d->stride_k % 4 || d->stride_v % 4 || d->inner_stride_q % 4 || d->inner_stride_k % 4 ||
+      d->inner_stride_v % 4)
+    return "batch stride not a multiple of 4 elements";
+  if ((uintptr_t)d->q % 16 || (uintptr_t)d->k % 16 || (uintptr_t)d->v % 16) return "operand not 16-byte aligned";
+  const unsigned long long rows = d->s > d->t ? d->s : d->t, ld = d->ldq > d->ldk ? (d->ldq > d->ldv ? d->ldq : d->ldv)
+                                                                                  : (d->ldk > d->ldv ? d->ldk : d->ldv);
+  if (rows * ld + d->d >= (1ull << 28)) return "one batch entry spans 2^28 elements or more";
+  return nullptr;
+}
+
+}  // namespace
+}  // namespace tfcc_rocm
+
+using namespace tfcc_rocm;
+
+extern "C" int tfcc_rocm_attention_f32_supported(const tfcc_rocm_attention_desc* d) {
+  return d != nullptr && unsupported(d) == nullptr ? 1 : 0;
+}
+
+extern "C" int tfcc_rocm_attention_f32(void* stream, const tfcc_rocm_attention_desc* d) {
+  TFCC_REQUIRE(d != nullptr, "attention: null descriptor");
+  TFCC_REQUIRE(d->q && d->k && d->v && d->out, "attention: null operand");
+  TFCC_REQUIRE(d->s > 0 && d->t > 0 && d->d > 0 && d->batch_outer > 0 && d->batch_inner > 0, "attention: empty operand");
+  TFCC_REQUIRE(d->ldq >= d->d && d->ldk >= d->d && d->ldv >= d->d && d->ldo >= d->d,
+               "attention: row stride shorter than a row");
+  const char* why = unsupported(d);
+  TFCC_REQUIRE(why == nullptr, "attention: %s (use the separate products and softmax)", why);
+  AttentionParams p{};
+  p.Q = d->q; p.K = d->k; p.V = d->v; p.O = d->out;
+  p.S = d->s; p.T = d->t; p.D = d->d;
+  p.ldq = d->ldq; p.ldk = d->ldk; p.ldv = d->ldv; p.ldo = d->ldo;
+  p.outerQ = d->stride_q; p.outerK = d->stride_k; p.outerV = d->stride_v; p.outerO = d->stride_out;
+  p.innerQ = d->inner_stride_q; p.innerK = d->inner_stride_k; p.innerV = d->inner_stride_v; p.innerO = d->inner_stride_out;
+  p.batchInner = d->batch_inner;
+  p.blocksS = (d->s + kRows - 1) / kRows;
+  const unsigned long long total = (unsigned long long)p.blocksS * d->batch_outer * d->batch_inner;
+  TFCC_REQUIRE(total < (1ull << 31) - 8, "attention: too many blocks");
+  p.total = (unsigned)total;
+  p.chunk = (p.total + 7) / 8;
+  p.divisor = d->divisor;
+  p.divide = d->has_divisor ? 1 : 0;
+  constexpr size_t ldsBytes = (size_t)kLdsFloats * sizeof(float);
+  static_assert(ldsBytes <= 160 * 1024, "LDS budget");
+  static bool attrSet[16] = {};
+  int dev = 0;
+  TFCC_HIP_CHECK(hipGetDevice(&dev));
+  TFCC_REQUIRE(dev >= 0 && dev < 16, "device index %d", dev);
+  if (!attrSet[dev]) {
+    TFCC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes));
+    attrSet[dev] = true;
+  }
+  hipLaunchKernelGGL(attention_kernel, dim3(p.chunk * 8), dim3(kThreads), ldsBytes, as_stream(stream), p);
+  return check_launch("attention");
+}

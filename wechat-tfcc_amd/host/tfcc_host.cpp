@@ -727,6 +727,60 @@ Variable<float> matmul_permuted(const Tensor<float>& a, const std::vector<size_t
   check(tfcc_rocm_sgemm_general(current_stream(), &d));
   return result;
 }
+Variable<float> attention_permuted(const Tensor<float>& q, const std::vector<size_t>& permQ, const Tensor<float>& k,
+                                   const std::vector<size_t>& permK, const Tensor<float>& v,
+                                   const std::vector<size_t>& permV, const std::vector<size_t>& permOut,
+                                   const float* divisor) {
+  if (dynamic_cast<ROCMDevice*>(Device::getThreadDefault()) == nullptr) throw NotImplementedError();
+  if (q.size() == 0 || k.size() == 0 || v.size() == 0) throw NotImplementedError("attention_permuted: empty operand");
+  const PermutedView vq = permuted_view(q.shape(), permQ), vk = permuted_view(k.shape(), permK),
+                     vv = permuted_view(v.shape(), permV);
+  // [b0, b1, s, d] x [b0, b1, d, t] -> [b0, b1, s, t];  x [b0, b1, t, d2] -> [b0, b1, s, d2]
+  const unsigned s = vq.dims[2], d = vq.dims[3], t = vk.dims[3];
+  for (int i = 0; i < 2; ++i)
+    if (vq.dims[i] != vk.dims[i] || vq.dims[i] != vv.dims[i]) throw InvalidArgumentError("shape invalid");
+  if (vk.dims[2] != d || vv.dims[2] != t) throw InvalidArgumentError("shape invalid");
+  if (vv.dims[3] != d) throw NotImplementedError("attention_permuted: value size differs from key size");
+  const unsigned logical[4] = {vq.dims[0], vq.dims[1], s, d};
+  std::vector<unsigned> outDims(4);
+  uint64_t oStride[4] = {0, 0, 0, 0};
+  {
+    bool seen[4] = {false, false, false, false};
+    for (size_t p = 0; p < 4; ++p) {
+      const size_t src = permOut.empty() ? p : permOut[p];
+      if ((!permOut.empty() && permOut.size() != 4) || src >= 4 || seen[src]) throw InvalidArgumentError("invalid perm");
+      seen[src] = true;
+      outDims[p] = logical[src];
+    }
+    uint64_t acc = 1;
+    for (int p = 3; p >= 0; --p) {
+      oStride[permOut.empty() ? p : permOut[p]] = acc;
+      acc *= outDims[p];
+    }
+  }
+  // size must be the contiguous dimension everywhere: q rows, k rows (k is taken as K, not K^T), v rows, result rows
+  if ((vq.strides[3] != 1 || vk.strides[2] != 1 || vv.strides[3] != 1 || oStride[3] != 1) && d != 1)
+    throw NotImplementedError("attention_permuted: head size is not the contiguous dimension");
+  tfcc_rocm_attention_desc a{};
+  a.s = s; a.t = t; a.d = d;
+  a.ldq = static_cast<unsigned>(std::max<uint64_t>(vq.strides[2], d));
+  a.ldk = static_cast<unsigned>(std::max<uint64_t>(vk.strides[3], d));
+  a.ldv = static_cast<unsigned>(std::max<uint64_t>(vv.strides[2], d));
+  a.ldo = static_cast<unsigned>(std::max<uint64_t>(oStride[2], d));
+  a.batch_outer = logical[0]; a.batch_inner = logical[1];
+  a.stride_q = vq.strides[0]; a.inner_stride_q = vq.strides[1];
+  a.stride_k = vk.strides[0]; a.inner_stride_k = vk.strides[1];
+  a.stride_v = vv.strides[0]; a.inner_stride_v = vv.strides[1];
+  a.stride_out = oStride[0]; a.inner_stride_out = oStride[1];
+  a.divisor = divisor ? *divisor : 1.f;
+  a.has_divisor = divisor ? 1 : 0;
+  a.q = q.data(); a.k = k.data(); a.v = v.data();
+  if (!tfcc_rocm_attention_f32_supported(&a)) throw NotImplementedError("attention_permuted: outside the kernel's limits");
+  Variable<float> result{Shape(outDims)};
+  a.out = result.data();
+  check(tfcc_rocm_attention_f32(current_stream(), &a));
+  return result;
+}
 std::vector<Variable<float>> matmul_grouped(const Tensor<float>& a, const std::vector<const Tensor<float>*>& b,
                                             const std::vector<const Tensor<float>*>& bias) {
   if (dynamic_cast<ROCMDevice*>(Device::getThreadDefault()) == nullptr) throw NotImplementedError();

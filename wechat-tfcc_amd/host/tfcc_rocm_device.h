@@ -100,6 +100,16 @@ Variable<float> matmul_permuted(const Tensor<float>& a, const std::vector<size_t
 // tfcc::blas::matmul(a, b[g], bias[g]) bit for bit.  Raises NotImplementedError for anything else.
 std::vector<Variable<float>> matmul_grouped(const Tensor<float>& a, const std::vector<const Tensor<float>*>& b,
                                             const std::vector<const Tensor<float>*>& bias);
+// transpose(matmul(softmax(matmul(transpose(q, permQ), transpose(k, permK)) [/ *divisor], last axis),
+// transpose(v, permV)), permOut) for rank-4 tensors in one launch (an empty perm is the identity;
+// divisor may be null).  transpose(k, permK) is the [.., size, keys] operand the first product takes.
+// The result equals the step-by-step form bit for bit.  Raises NotImplementedError when the layout or
+// the sizes are outside what the kernel takes (more than 128 keys, head size above 64, a head size or
+// strides that are not multiples of 4, size not the contiguous dimension of q, k, v and the result).
+Variable<float> attention_permuted(const Tensor<float>& q, const std::vector<size_t>& permQ, const Tensor<float>& k,
+                                   const std::vector<size_t>& permK, const Tensor<float>& v,
+                                   const std::vector<size_t>& permV, const std::vector<size_t>& permOut,
+                                   const float* divisor);
 }  // namespace blas
 namespace math {
 // softmax(a / divisor, axis)

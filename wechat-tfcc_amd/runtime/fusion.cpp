@@ -6,6 +6,7 @@
 //   MatmulWithBias -> Add(other tensor)    one GEMM that also adds the other tensor (residual)
 //   Div(tensor, value) -> Softmax          one softmax pass that divides first
 //   Transpose -> Matmul -> Transpose       a batched product that walks the permuted tensors in place
+//   Matmul -> [Div] -> Softmax -> Matmul   (each Matmul with its Transposes) the attention core in one launch
 //   2-4 x MatmulWithBias on one input with constant weights of one shape (query / key / value): one launch
 //   Identity of a variable nobody else reads: the buffer is handed over instead of copied
 //
@@ -37,6 +38,14 @@ bool float_variable(SymbolManager& sm, const std::string& name) {
   if (!sm.has(name)) return false;
   const SymbolInfo& info = sm.getSymbolInfo(name);
   return info.dtype == FLOAT && info.stype == SymbolType::VARIABLE;
+}
+
+FusionPlan simple_plan(FusionPlan::Kind kind, size_t partner, unsigned side = 0) {
+  FusionPlan f;
+  f.kind = kind;
+  f.partner = partner;
+  f.side = side;
+  return f;
 }
 
 }  // namespace
@@ -78,14 +87,14 @@ std::vector<FusionPlan> plan_fusions(const proto::Graph& g, SymbolManager& sm) {
     size_t i = 0;
     if (is_op(n, "math.Gelu", 1) && float_variable(sm, n.outputs[0]) && sole_producer(n.inputs[0], j, i) &&
         is_op(g.nodes[i], "math.MatmulWithBias", 3) && all_float_tensors(g.nodes[i])) {
-      plan[j] = {FusionPlan::MATMUL_GELU, i, 0};
-      plan[i] = {FusionPlan::ABSORBED, j, 0};
+      plan[j] = simple_plan(FusionPlan::MATMUL_GELU, i, 0);
+      plan[i] = simple_plan(FusionPlan::ABSORBED, j);
     } else if (is_op(n, "math.Add", 2) && float_variable(sm, n.outputs[0]) && all_float_tensors(n)) {
       for (unsigned side = 0; side < 2; ++side) {
         if (sole_producer(n.inputs[side], j, i) && is_op(g.nodes[i], "math.MatmulWithBias", 3) &&
             all_float_tensors(g.nodes[i]) && n.inputs[0] != n.inputs[1]) {
-          plan[j] = {FusionPlan::MATMUL_ADD, i, side};
-          plan[i] = {FusionPlan::ABSORBED, j, 0};
+          plan[j] = simple_plan(FusionPlan::MATMUL_ADD, i, side);
+          plan[i] = simple_plan(FusionPlan::ABSORBED, j);
           break;
         }
       }
@@ -93,8 +102,8 @@ std::vector<FusionPlan> plan_fusions(const proto::Graph& g, SymbolManager& sm) {
                is_op(g.nodes[i], "math.Div", 2) && float_tensor(sm, g.nodes[i].inputs[0]) &&
                sm.has(g.nodes[i].inputs[1]) && sm.getSymbolInfo(g.nodes[i].inputs[1]).dtype == FLOAT &&
                is_value(sm.getSymbolInfo(g.nodes[i].inputs[1]).stype)) {
-      plan[j] = {FusionPlan::DIV_SOFTMAX, i, 0};
-      plan[i] = {FusionPlan::ABSORBED, j, 0};
+      plan[j] = simple_plan(FusionPlan::DIV_SOFTMAX, i, 0);
+      plan[i] = simple_plan(FusionPlan::ABSORBED, j);
     } else if (is_op(n, "math.Matmul", 2) && float_variable(sm, n.outputs[0]) && all_float_tensors(n)) {
       FusionPlan f;
       f.kind = FusionPlan::MATMUL_PERMUTED;
@@ -114,13 +123,62 @@ std::vector<FusionPlan> plan_fusions(const proto::Graph& g, SymbolManager& sm) {
       if (f.transposeA != FusionPlan::kNoNode || f.transposeB != FusionPlan::kNoNode || f.transposeC != FusionPlan::kNoNode) {
         plan[j] = f;
         for (size_t t2 : {f.transposeA, f.transposeB, f.transposeC})
-          if (t2 != FusionPlan::kNoNode) plan[t2] = {FusionPlan::ABSORBED, j, 0};
+          if (t2 != FusionPlan::kNoNode) plan[t2] = simple_plan(FusionPlan::ABSORBED, j);
       }
     } else if (is_op(n, "base.Identity", 1) && float_variable(sm, n.outputs[0]) && float_variable(sm, n.inputs[0]) &&
                producer.count(n.inputs[0]) && producer[n.inputs[0]] < j && consumers[n.inputs[0]].size() == 1 &&
                !kept.count(n.inputs[0])) {
-      plan[j] = {FusionPlan::MOVE_IDENTITY, j, 0};
+      plan[j] = simple_plan(FusionPlan::MOVE_IDENTITY, j, 0);
     }
+  }
+  // softmax(Q K^T [/ value]) V: two products (with whatever Transposes they folded) around a Softmax
+  for (size_t j = 0; j < g.nodes.size(); ++j) {
+    const proto::Node& n = g.nodes[j];
+    if (!is_op(n, "math.Matmul", 2) || !sm.has(n.outputs[0]) || !float_variable(sm, n.outputs[0]) || !all_float_tensors(n))
+      continue;
+    if (plan[j].kind != FusionPlan::NONE && plan[j].kind != FusionPlan::MATMUL_PERMUTED) continue;
+    if (plan[j].kind == FusionPlan::MATMUL_PERMUTED && plan[j].transposeA != FusionPlan::kNoNode) continue;
+    // a value produced by node `from` for one reader, droppable from the graph
+    auto private_value = [&](const std::string& name, size_t reader, size_t& from) {
+      auto p = producer.find(name);
+      if (p == producer.end() || p->second >= reader || kept.count(name)) return false;
+      if (consumers[name].size() != 1 || !float_variable(sm, name)) return false;
+      from = p->second;
+      return true;
+    };
+    size_t soft = 0, first = 0;
+    if (!private_value(n.inputs[0], j, soft) || n.inputs[0] == n.inputs[1]) continue;
+    const proto::Node& softNode = g.nodes[soft];
+    if (!is_op(softNode, "math.Softmax", 1)) continue;
+    if (plan[soft].kind != FusionPlan::NONE && plan[soft].kind != FusionPlan::DIV_SOFTMAX) continue;
+    const size_t div = plan[soft].kind == FusionPlan::DIV_SOFTMAX ? plan[soft].partner : FusionPlan::kNoNode;
+    const std::string& scoresName = div != FusionPlan::kNoNode ? g.nodes[div].inputs[0] : softNode.inputs[0];
+    if (!private_value(scoresName, div != FusionPlan::kNoNode ? div : soft, first)) continue;
+    const proto::Node& firstNode = g.nodes[first];
+    if (!is_op(firstNode, "math.Matmul", 2) || !all_float_tensors(firstNode)) continue;
+    if (plan[first].kind != FusionPlan::NONE && plan[first].kind != FusionPlan::MATMUL_PERMUTED) continue;
+    if (plan[first].kind == FusionPlan::MATMUL_PERMUTED && plan[first].transposeC != FusionPlan::kNoNode) continue;
+    FusionPlan f;
+    f.kind = FusionPlan::ATTENTION;
+    f.scoresNode = first;
+    f.softmaxNode = soft;
+    f.divNode = div;
+    if (plan[first].kind == FusionPlan::MATMUL_PERMUTED) {
+      f.transposeA = plan[first].transposeA;
+      f.transposeB = plan[first].transposeB;
+    }
+    if (plan[j].kind == FusionPlan::MATMUL_PERMUTED) {
+      f.transposeV = plan[j].transposeB;
+      f.transposeC = plan[j].transposeC;
+    }
+    // every input of the fused step must exist before the first absorbed node ran in the plain order; it runs
+    // at the position of the second product (or of its folded Transpose), which is later
+    plan[j] = f;
+    plan[first] = simple_plan(FusionPlan::ABSORBED, j);
+    plan[soft] = simple_plan(FusionPlan::ABSORBED, j);
+    if (div != FusionPlan::kNoNode) plan[div] = simple_plan(FusionPlan::ABSORBED, j);
+    for (size_t t2 : {f.transposeA, f.transposeB, f.transposeV, f.transposeC})
+      if (t2 != FusionPlan::kNoNode) plan[t2] = simple_plan(FusionPlan::ABSORBED, j);
   }
   // MatmulWithBias nodes left as they are that share their input and have constant weights: groups of up to 4
   std::unordered_map<std::string, std::vector<size_t>> byInput;
@@ -150,7 +208,7 @@ std::vector<FusionPlan> plan_fusions(const proto::Graph& g, SymbolManager& sm) {
       FusionPlan f;
       f.kind = FusionPlan::MATMUL_GROUPED;
       f.group.assign(members.begin() + at, members.begin() + at + count);
-      for (size_t q = 1; q < count; ++q) plan[f.group[q]] = {FusionPlan::ABSORBED, f.group[0], 0};
+      for (size_t q = 1; q < count; ++q) plan[f.group[q]] = simple_plan(FusionPlan::ABSORBED, f.group[0]);
       plan[f.group[0]] = f;
     }
   }
@@ -168,11 +226,78 @@ std::vector<size_t> transpose_perm(const proto::Node& n) {
   }
   return perm;
 }
+size_t softmax_axis(const proto::Node& n) {
+  size_t axis = 0;
+  wire::Reader r(n.operation);
+  uint32_t field, type;
+  while (r.next(field, type)) {
+    if (field == 1 && type == 0) axis = static_cast<size_t>(r.varint());
+    else r.skip(type);
+  }
+  return axis;
+}
+
+// transpose(matmul(transpose(a, pa), transpose(b, pb)), pc); an empty perm stands for no Transpose node
+Variable<float> permuted_product(const Tensor<float>& a, const std::vector<size_t>& pa, const Tensor<float>& b,
+                                 const std::vector<size_t>& pb, const std::vector<size_t>& pc) {
+  if (!pa.empty() || !pb.empty() || !pc.empty()) {
+    try {
+      return rocm::blas::matmul_permuted(a, pa, b, pb, pc);
+    } catch (NotImplementedError&) {
+      // a layout the strided kernel does not take: run the nodes as written
+    }
+  }
+  Variable<float> xa, xb;
+  if (!pa.empty()) xa = base::transpose(a, pa);
+  if (!pb.empty()) xb = base::transpose(b, pb);
+  Variable<float> c = blas::matmul(pa.empty() ? a : static_cast<const Tensor<float>&>(xa),
+                                   pb.empty() ? b : static_cast<const Tensor<float>&>(xb));
+  if (!pc.empty()) return base::transpose(c, pc);
+  return c;
+}
+
+// softmax(a [/ *divisor], axis)
+Variable<float> divided_softmax(const Tensor<float>& a, const float* divisor, size_t axis) {
+  if (divisor == nullptr) return math::softmax(a, axis);
+  if (axis + 1 == a.shape().size()) return rocm::math::softmax_div(a, axis, *divisor);
+  Variable<float> t = a / *divisor;
+  return math::softmax(t, axis);
+}
 }  // namespace
 
 void emit_fused(const proto::Graph& g, const FusionPlan& f, size_t j, Graph& graph) {
   SymbolManager& sm = graph.getSymbolManager();
   const proto::Node& n = g.nodes[j];
+  if (f.kind == FusionPlan::ATTENTION) {
+    const proto::Node& first = g.nodes[f.scoresNode];
+    auto perm_of = [&](size_t node) { return node != FusionPlan::kNoNode ? transpose_perm(g.nodes[node]) : std::vector<size_t>(); };
+    auto source = [&](size_t transposeNode, const std::string& name) {
+      return sm.getTensor(transposeNode != FusionPlan::kNoNode ? g.nodes[transposeNode].inputs[0] : name, float());
+    };
+    const Tensor<float>* q = source(f.transposeA, first.inputs[0]);
+    const Tensor<float>* k = source(f.transposeB, first.inputs[1]);
+    const Tensor<float>* v = source(f.transposeV, n.inputs[1]);
+    const std::vector<size_t> pq = perm_of(f.transposeA), pk = perm_of(f.transposeB), pv = perm_of(f.transposeV),
+                              po = perm_of(f.transposeC);
+    const float* divisor = f.divNode != FusionPlan::kNoNode ? sm.getValue(g.nodes[f.divNode].inputs[1], float()) : nullptr;
+    const size_t axis = softmax_axis(g.nodes[f.softmaxNode]);
+    Variable<float>* result =
+        sm.getVariable(f.transposeC != FusionPlan::kNoNode ? g.nodes[f.transposeC].outputs[0] : n.outputs[0], float());
+    graph.addStep([q, k, v, pq, pk, pv, po, divisor, axis, result] {
+      if (axis == 3 && q->shape().size() == 4 && k->shape().size() == 4 && v->shape().size() == 4) {
+        try {
+          *result = rocm::blas::attention_permuted(*q, pq, *k, pk, *v, pv, po, divisor);
+          return;
+        } catch (NotImplementedError&) {
+          // longer sequences, wider heads or another layout: the three steps one after the other
+        }
+      }
+      Variable<float> scores = permuted_product(*q, pq, *k, pk, {});
+      Variable<float> probabilities = divided_softmax(scores, divisor, axis);
+      *result = permuted_product(probabilities, {}, *v, pv, po);
+    });
+    return;
+  }
   if (f.kind == FusionPlan::MATMUL_GROUPED) {
     const Tensor<float>* a = sm.getTensor(n.inputs[0], float());
     std::vector<const Tensor<float>*> bs, biases;
@@ -203,21 +328,7 @@ void emit_fused(const proto::Graph& g, const FusionPlan& f, size_t j, Graph& gra
     const std::vector<size_t> pa = ta ? transpose_perm(g.nodes[f.transposeA]) : std::vector<size_t>();
     const std::vector<size_t> pb = tb ? transpose_perm(g.nodes[f.transposeB]) : std::vector<size_t>();
     const std::vector<size_t> pc = tc ? transpose_perm(g.nodes[f.transposeC]) : std::vector<size_t>();
-    graph.addStep([a, b, result, pa, pb, pc, ta, tb, tc] {
-      try {
-        *result = rocm::blas::matmul_permuted(*a, pa, *b, pb, pc);
-        return;
-      } catch (NotImplementedError&) {
-        // a layout the strided kernel does not take: run the nodes as written
-      }
-      Variable<float> xa, xb;
-      if (ta) xa = base::transpose(*a, pa);
-      if (tb) xb = base::transpose(*b, pb);
-      Variable<float> c = blas::matmul(ta ? static_cast<const Tensor<float>&>(xa) : *a,
-                                       tb ? static_cast<const Tensor<float>&>(xb) : *b);
-      if (tc) *result = base::transpose(c, pc);
-      else *result = std::move(c);
-    });
+    graph.addStep([a, b, result, pa, pb, pc] { *result = permuted_product(*a, pa, *b, pb, pc); });
     return;
   }
   Variable<float>* out = sm.getVariable(n.outputs[0], float());
@@ -230,21 +341,8 @@ void emit_fused(const proto::Graph& g, const FusionPlan& f, size_t j, Graph& gra
   if (f.kind == FusionPlan::DIV_SOFTMAX) {
     const Tensor<float>* a = sm.getTensor(p.inputs[0], float());
     const float* divisor = sm.getValue(p.inputs[1], float());
-    size_t axis = 0;
-    wire::Reader r(n.operation);
-    uint32_t field, type;
-    while (r.next(field, type)) {
-      if (field == 1 && type == 0) axis = static_cast<size_t>(r.varint());
-      else r.skip(type);
-    }
-    graph.addStep([a, divisor, axis, out] {
-      if (axis + 1 == a->shape().size()) {
-        *out = rocm::math::softmax_div(*a, axis, *divisor);
-      } else {
-        Variable<float> t = *a / *divisor;
-        *out = math::softmax(t, axis);
-      }
-    });
+    const size_t axis = softmax_axis(n);
+    graph.addStep([a, divisor, axis, out] { *out = divided_softmax(*a, divisor, axis); });
     return;
   }
   const Tensor<float>* a = sm.getTensor(p.inputs[0], float());

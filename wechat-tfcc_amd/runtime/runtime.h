@@ -269,13 +269,17 @@ const std::vector<std::unique_ptr<Operation>>& operations_for(const std::string&
 // later node runs it as part of a fused step (ABSORBED, partner = that node), or run it fused with
 // the producer `partner` of one of its inputs (side: which input of an Add the product is).
 struct FusionPlan {
-  enum Kind { NONE, ABSORBED, MATMUL_GELU, MATMUL_ADD, DIV_SOFTMAX, MOVE_IDENTITY, MATMUL_PERMUTED, MATMUL_GROUPED } kind = NONE;
+  enum Kind { NONE, ABSORBED, MATMUL_GELU, MATMUL_ADD, DIV_SOFTMAX, MOVE_IDENTITY, MATMUL_PERMUTED, MATMUL_GROUPED, ATTENTION } kind = NONE;
   size_t partner = 0;
   unsigned side = 0;
   // MATMUL_PERMUTED: the Transpose nodes folded into a Matmul (producer of input 0 / of input 1 /
   // consumer of the output), kNoNode where there is none
   static constexpr size_t kNoNode = ~static_cast<size_t>(0);
   size_t transposeA = kNoNode, transposeB = kNoNode, transposeC = kNoNode;
+  // ATTENTION (on the second Matmul): the first Matmul, the Softmax between them, the Div folded into the
+  // Softmax and the Transpose of the second Matmul's other operand; transposeA / transposeB are those of
+  // the first Matmul, transposeC that of the second
+  size_t scoresNode = kNoNode, softmaxNode = kNoNode, divNode = kNoNode, transposeV = kNoNode;
   // MATMUL_GROUPED: the MatmulWithBias nodes (this one first) that share their first input and run as one launch
   std::vector<size_t> group;
 };
