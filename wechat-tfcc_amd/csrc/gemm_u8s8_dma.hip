@@ -26,6 +26,7 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "lds_dma.hpp"
 #include "qgemm_dma.hpp"
 
 namespace tfcc_rocm {
@@ -38,34 +39,6 @@ namespace {
 
 constexpr int BK = 128;      // bytes of k per slab: a row piece of A is one full 128-byte memory line
 constexpr int KS = BK / 32;  // 32-deep matrix-op steps per slab
-
-// One asynchronous 16-byte-per-lane copy HBM -> LDS.  The LDS address of lane i is ldsBase + 16*i
-// (ldsBase wave-uniform, goes through M0); voffset is the lane's byte offset into the buffer.
-// Inline asm on purpose: the outstanding-copy count is managed by hand (s_waitcnt vmcnt) so that
-// several slabs stay in flight across iterations.
-__device__ __forceinline__ v4i make_rsrc(const void* base, unsigned bytes) {
-  const unsigned long long a = reinterpret_cast<unsigned long long>(base);
-  v4i r;
-  r[0] = __builtin_amdgcn_readfirstlane((int)(unsigned)a);
-  r[1] = __builtin_amdgcn_readfirstlane((int)((unsigned)(a >> 32) & 0xffffu));
-  r[2] = __builtin_amdgcn_readfirstlane((int)bytes);
-  r[3] = 0x00020000;
-  return r;
-}
-
-__device__ __forceinline__ void dma16(v4i rsrc, unsigned ldsBase, unsigned voffset) {
-  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
-               :
-               : "s"(ldsBase), "v"(voffset), "s"(rsrc)
-               : "memory", "m0");
-}
-
-template <int N>
-__device__ __forceinline__ void wait_vmcnt() {
-  // s_waitcnt simm16: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt_hi[15:14]; leave the others at max
-  static_assert(N >= 0 && N < 64, "vmcnt range");
-  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | 0x0f70);
-}
 
 // 16 consecutive rows of one logical chunk fall into 16 different 16-byte slots of the 256-byte bank stripe
 __device__ __forceinline__ int swzA(int row) { return (row >> 1) & 7; }

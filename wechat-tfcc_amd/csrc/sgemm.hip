@@ -14,33 +14,16 @@
 // index, and tile columns are stored interleaved (LDS row j*32+i holds tile column NI*i+j of the
 // wavefront's column range) so that a lane owns NI consecutive output columns.
 #include "common.hpp"
+#include "sgemm_params.hpp"
 
 namespace tfcc_rocm {
+
+using sgemm_detail::SgemmParams;
 
 typedef float v4f __attribute__((ext_vector_type(4)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 
 namespace {
-
-struct SgemmParams {
-  const float* A;
-  const float* B;
-  const float* bias;
-  const float* residual;  // optional, laid out like C (batch stride strideR): added after the bias
-  float* C;
-  unsigned long long strideA, strideB, strideC, strideR;  // between outer batch entries (elements)
-  unsigned long long innerA, innerB, innerC;              // between inner batch entries
-  unsigned batchInner;    // batch entry bi = (bi / batchInner, bi % batchInner); 1 for a flat batch
-  unsigned lda, ldb, ldc; // row strides of A, of B (of B^T when transposed) and of C, in elements
-  int act;                // 0 none, 1 erf-form GELU applied last
-  // grouped form (groups > 0): batch entry g multiplies the shared A by groupB[g] into groupC[g]
-  unsigned groups;
-  const float* groupB[4];
-  const float* groupBias[4];
-  float* groupC[4];
-  unsigned M, N, K, batch;
-  unsigned tilesM, tilesN, tilesTotal, chunk;
-};
 
 constexpr int BK = 32;
 constexpr int CH = BK / 4;  // 16-byte chunks per LDS row
@@ -373,12 +356,7 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_kernel(const Sg
 template <int WGM, int WGN, int MI, int NI, bool VEC, int KSPLIT = 1, bool TRANSB = false>
 int launch(hipStream_t stream, SgemmParams p) {
   constexpr int BM = WGM * MI * 32, BN = WGN * NI * 32;
-  p.tilesM = (p.M + BM - 1) / BM;
-  p.tilesN = (p.N + BN - 1) / BN;
-  unsigned long long total = (unsigned long long)p.tilesM * p.tilesN * p.batch;
-  if (total > 0x7fffffffull) return set_error(TFCC_ROCM_INVALID_ARGUMENT, "sgemm: too many tiles");
-  p.tilesTotal = (unsigned)total;
-  p.chunk = (p.tilesTotal + 7) / 8;
+  if (!sgemm_detail::set_tiles(p, BM, BN)) return set_error(TFCC_ROCM_INVALID_ARGUMENT, "sgemm: too many tiles");
   constexpr size_t lds = KSPLIT * 2 * (size_t)(BM + BN) * BK * sizeof(float);
   static_assert(lds <= 160 * 1024 && (size_t)(KSPLIT - 1) * BM * BN * sizeof(float) <= lds, "LDS budget");
   auto kern = sgemm_kernel<WGM, WGN, MI, NI, VEC, KSPLIT, TRANSB>;
@@ -416,10 +394,13 @@ int dispatch(hipStream_t s, const SgemmParams& p, bool vec, bool tb, unsigned fi
     // 32x96 tiles when they cover the 256 CUs in fewer tile-area rounds than 64x64 tiles would
     const unsigned long long flat = (unsigned long long)((m + 31) / 32) * ((n + 95) / 96) * fillBatch;
     const bool preferFlat = ((flat + 255) / 256) * (32 * 96) < ((small + 255) / 256) * (64 * 64);
-    if (preferFlat && flat <= 320 && k >= 512) return launch<1, 3, 1, 1, true, 4>(s, p);
-    if (small <= 320 && k >= 512) return launch<2, 2, 1, 1, true, 4>(s, p);
-    if (small <= 640 && k >= 256) return launch<2, 2, 1, 1, true, 2>(s, p);
-    return launch<2, 2, 1, 1, true>(s, p);
+    // whole slabs of K: the same tile configurations with the slabs copied straight into LDS (same results)
+    const bool dma = k % 32 == 0;
+    if (preferFlat && flat <= 320 && k >= 512)
+      return dma ? sgemm_detail::sgemm_dma_launch(s, p, 1, 4) : launch<1, 3, 1, 1, true, 4>(s, p);
+    if (small <= 320 && k >= 512) return dma ? sgemm_detail::sgemm_dma_launch(s, p, 0, 4) : launch<2, 2, 1, 1, true, 4>(s, p);
+    if (small <= 640 && k >= 256) return dma ? sgemm_detail::sgemm_dma_launch(s, p, 0, 2) : launch<2, 2, 1, 1, true, 2>(s, p);
+    return dma ? sgemm_detail::sgemm_dma_launch(s, p, 0, 1) : launch<2, 2, 1, 1, true>(s, p);
   }
   TFCC_REQUIRE((unsigned long long)m * ldc < (1ull << 32) && (unsigned long long)m * lda < (1ull << 32) &&
                rowsB * ldb < (1ull << 32), "sgemm: operand larger than 2^32 elements");

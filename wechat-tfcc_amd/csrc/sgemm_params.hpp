@@ -1,0 +1,47 @@
+// Argument block shared by the fp32 GEMM kernels (register-staged in sgemm.hip, direct-to-LDS in
+// sgemm_dma.hip) and the entry points that pick between them.
+#pragma once
+
+#include "common.hpp"
+
+namespace tfcc_rocm {
+namespace sgemm_detail {
+
+struct SgemmParams {
+  const float* A;
+  const float* B;
+  const float* bias;
+  const float* residual;  // optional, laid out like C (batch stride strideR): added after the bias
+  float* C;
+  unsigned long long strideA, strideB, strideC, strideR;  // between outer batch entries (elements)
+  unsigned long long innerA, innerB, innerC;              // between inner batch entries
+  unsigned batchInner;    // batch entry bi = (bi / batchInner, bi % batchInner); 1 for a flat batch
+  unsigned lda, ldb, ldc; // row strides of A, of B (of B^T when transposed) and of C, in elements
+  int act;                // 0 none, 1 erf-form GELU applied last
+  // grouped form (groups > 0): batch entry g multiplies the shared A by groupB[g] into groupC[g]
+  unsigned groups;
+  const float* groupB[4];
+  const float* groupBias[4];
+  float* groupC[4];
+  unsigned M, N, K, batch;
+  unsigned tilesM, tilesN, tilesTotal, chunk;
+};
+
+// Fills in the tile counts for BM x BN tiles; false when there are too many tiles for one grid.
+inline bool set_tiles(SgemmParams& p, unsigned bm, unsigned bn) {
+  p.tilesM = (p.M + bm - 1) / bm;
+  p.tilesN = (p.N + bn - 1) / bn;
+  const unsigned long long total = (unsigned long long)p.tilesM * p.tilesN * p.batch;
+  if (total > 0x7fffffffull) return false;
+  p.tilesTotal = (unsigned)total;
+  p.chunk = (p.tilesTotal + 7) / 8;
+  return true;
+}
+
+// The direct-to-LDS kernels (sgemm_dma.hip).  `config`: 0 = 64x64 tiles, 1 = 32x96 tiles; ksplit 1, 2 or 4.
+// Requires 16-byte aligned operands and strides, K a multiple of 32 and B not transposed.
+bool sgemm_dma_available(int config, int ksplit);
+int sgemm_dma_launch(hipStream_t stream, SgemmParams p, int config, int ksplit);
+
+}  // namespace sgemm_detail
+}  // namespace tfcc_rocm
