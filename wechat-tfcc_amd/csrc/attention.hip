@@ -4,7 +4,8 @@
 // operations on tensors in HBM: Matmul (tfcc_runtime/operations/math/matmul.cpp:27-41), Div by a
 // value, Softmax (tfcc_runtime/operations/math/softmax.cpp), Matmul again, with base::transpose
 // (tfcc/core/operations/tfcc_base.cpp:124-134) before and after.  Here the score matrix of a block of
-// 64 query rows never leaves the CU.
+// 64 query rows never leaves the CU: Q is held in registers, K in LDS, the scores and probabilities in
+// LDS, V in registers until the scores are done and then in K's place (70.7 KB, two workgroups per CU).
 //
 // Every number is computed by the same instruction sequence as in the three separate kernels
 // (fp32 32x32x2 matrix ops over ascending k into one accumulator; the softmax of one row by one
@@ -24,10 +25,11 @@ constexpr int kRows = 64;        // query rows per workgroup
 constexpr int kThreads = 512;    // eight wavefronts
 constexpr int kMaxT = 128;       // key rows
 constexpr int kMaxD = 64;        // head width
-constexpr int kPitchQK = kMaxD + 4;   // floats; 128-bit row reads of 32 consecutive rows hit all banks once
+constexpr int kPitchK = kMaxD + 4;    // floats; 128-bit row reads of 32 consecutive rows hit all banks once
 constexpr int kPitchV = kMaxD + 8;    // 32-bit reads of rows r and r + 4 land 32 banks apart
 constexpr int kPitchS = kMaxT + 4;
-constexpr int kLdsFloats = kRows * kPitchQK + kMaxT * kPitchQK + kMaxT * kPitchV + kRows * kPitchS;
+// K and, once the scores are done, V share one region; Q stays in registers.  70.7 KB: two workgroups per CU.
+constexpr int kLdsFloats = kMaxT * kPitchV + kRows * kPitchS;
 
 struct AttentionParams {
   const float* Q;
@@ -54,12 +56,10 @@ __device__ __forceinline__ float wave_max(float v) {
   return v;
 }
 
-__global__ __launch_bounds__(kThreads) void attention_kernel(const AttentionParams p) {
+__global__ __launch_bounds__(kThreads, 4) void attention_kernel(const AttentionParams p) {
   extern __shared__ __align__(16) float lds[];
-  float* Qs = lds;                        // [64][kPitchQK]
-  float* Ks = Qs + kRows * kPitchQK;      // [128][kPitchQK]
-  float* Vs = Ks + kMaxT * kPitchQK;      // [128][kPitchV]
-  float* Sc = Vs + kMaxT * kPitchV;       // [64][kPitchS]  scores, then probabilities
+  float* KVs = lds;                       // K as [128][kPitchK], later V as [128][kPitchV]
+  float* Sc = KVs + kMaxT * kPitchV;      // [64][kPitchS]  scores, then probabilities
 
   // consecutive workgroup ids land on different XCDs: the blocks of one head stay on one XCD
   const unsigned wg = blockIdx.x;
@@ -80,92 +80,104 @@ __global__ __launch_bounds__(kThreads) void attention_kernel(const AttentionPara
   const unsigned Dp = (D + 7u) & ~7u;   // k extent of the score product
   const unsigned Tp = (T + 7u) & ~7u;   // k extent of the second product
 
-  // ---- all three operands to LDS; everything past the operands' extents that a matrix op will read
-  // is zero: a buffer load whose offset lies past the end of its operand returns zero
+  // ---- loads.  K goes to LDS; Q goes through the region the scores will later occupy into the registers
+  // the score product takes it from; V waits in registers until K is no longer needed.  A buffer load whose
+  // offset lies past the end of its operand returns zero: that is how everything past the operands' extents
+  // that a matrix op will read becomes zero.
+  const int wmS = wave >> 2, wnS = wave & 3;  // scores: 2 x 4 wavefronts, one 32 x 32 block each
+  constexpr int CH = kMaxD / 4;               // 16-byte chunks per row
+  constexpr int KV_ITEMS = kMaxT * CH / kThreads, Q_ITEMS = kRows * CH / kThreads, KBQ = kMaxD / 8;
+  constexpr unsigned kPastEnd = 0xfffffff0u;
+  v4f qf[KBQ], vreg[KV_ITEMS];
   {
-    constexpr int CH = kMaxD / 4;  // 16-byte chunks per row
-    constexpr int Q_ITEMS = kRows * CH / kThreads, KV_ITEMS = kMaxT * CH / kThreads;
-    constexpr unsigned kPastEnd = 0xfffffff0u;
     const __amdgpu_buffer_rsrc_t rq = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<float*>(Q), 0, (int)(((S - 1) * p.ldq + D) * 4u), 0x00020000);
     const __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<float*>(K), 0, (int)(((T - 1) * p.ldk + D) * 4u), 0x00020000);
     const __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc(
         const_cast<float*>(V), 0, (int)(((T - 1) * p.ldv + D) * 4u), 0x00020000);
-    v4f q[Q_ITEMS], k[KV_ITEMS], v[KV_ITEMS];
+    v4f qreg[Q_ITEMS], kreg[KV_ITEMS];
 #pragma unroll
     for (int it = 0; it < Q_ITEMS; ++it) {
       const unsigned w = tid + it * kThreads, row = s0 + w / CH, ch = w % CH;
-      const unsigned off = (row < S && ch * 4 < D) ? (row * p.ldq + ch * 4) * 4u : kPastEnd;
-      q[it] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rq, off, 0, 0));
+      qreg[it] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(
+                                             rq, (row < S && ch * 4 < D) ? (row * p.ldq + ch * 4) * 4u : kPastEnd, 0, 0));
     }
 #pragma unroll
     for (int it = 0; it < KV_ITEMS; ++it) {
       const unsigned w = tid + it * kThreads, row = w / CH, ch = w % CH;
       const bool in = row < T && ch * 4 < D;
-      k[it] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rk, in ? (row * p.ldk + ch * 4) * 4u : kPastEnd, 0, 0));
-      v[it] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rv, in ? (row * p.ldv + ch * 4) * 4u : kPastEnd, 0, 0));
-    }
-#pragma unroll
-    for (int it = 0; it < Q_ITEMS; ++it) {
-      const int w = tid + it * kThreads, row = w / CH, ch = w % CH;
-      *reinterpret_cast<v4f*>(Qs + row * kPitchQK + ch * 4) = q[it];
+      kreg[it] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rk, in ? (row * p.ldk + ch * 4) * 4u : kPastEnd, 0, 0));
+      vreg[it] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rv, in ? (row * p.ldv + ch * 4) * 4u : kPastEnd, 0, 0));
     }
 #pragma unroll
     for (int it = 0; it < KV_ITEMS; ++it) {
       const int w = tid + it * kThreads, row = w / CH, ch = w % CH;
-      *reinterpret_cast<v4f*>(Ks + row * kPitchQK + ch * 4) = k[it];
-      *reinterpret_cast<v4f*>(Vs + row * kPitchV + ch * 4) = v[it];
+      *reinterpret_cast<v4f*>(KVs + row * kPitchK + ch * 4) = kreg[it];
+    }
+#pragma unroll
+    for (int it = 0; it < Q_ITEMS; ++it) {
+      const int w = tid + it * kThreads, row = w / CH, ch = w % CH;
+      *reinterpret_cast<v4f*>(Sc + row * kPitchK + ch * 4) = qreg[it];
+    }
+  }
+  __syncthreads();
+  {
+    const float* qa = Sc + (32 * wmS + lrow) * kPitchK + 4 * g;
+#pragma unroll
+    for (int kb = 0; kb < KBQ; ++kb) {
+      qf[kb] = v4f{0.f, 0.f, 0.f, 0.f};
+      if ((unsigned)kb * 8 < Dp) qf[kb] = *reinterpret_cast<const v4f*>(qa + kb * 8);
+    }
+  }
+
+  // ---- scores.  All K operands are fetched from LDS before the first matrix op, so that their latency
+  // is paid once.  A divisor that is a power of two divides exactly like a multiplication by its reciprocal.
+  const bool liveS = (unsigned)(32 * wnS) < T;  // wave-uniform: this wavefront's 32 columns exist
+  v4f bf[KBQ];
+  {
+    const float* ka = KVs + (32 * wnS + lrow) * kPitchK + 4 * g;
+#pragma unroll
+    for (int kb = 0; kb < KBQ; ++kb) {
+      bf[kb] = v4f{0.f, 0.f, 0.f, 0.f};
+      if (liveS && (unsigned)kb * 8 < Dp) bf[kb] = *reinterpret_cast<const v4f*>(ka + kb * 8);
+    }
+  }
+  __syncthreads();  // every wavefront has taken its Q operands out of the region the scores go to
+  if (liveS) {
+    v16f acc;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+#pragma unroll
+    for (int kb = 0; kb < KBQ; ++kb) {
+      if ((unsigned)kb * 8 < Dp) {
+#pragma unroll
+        for (int s = 0; s < 4; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[kb][s], bf[kb][s], acc, 0, 0, 0);
+      }
+    }
+    float* sc = Sc + (32 * wmS + 4 * g) * kPitchS + 32 * wnS + lrow;
+    const float divisor = p.divisor;
+    const unsigned bits = __builtin_bit_cast(unsigned, divisor), expo = (bits >> 23) & 0xffu;
+    if (!p.divide) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sc[(8 * (r / 4) + (r & 3)) * kPitchS] = acc[r];
+    } else if ((bits & 0x007fffffu) == 0 && expo >= 2 && expo <= 252) {
+      const float inverse = 1.0f / divisor;  // exact: also a power of two
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sc[(8 * (r / 4) + (r & 3)) * kPitchS] = acc[r] * inverse;
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sc[(8 * (r / 4) + (r & 3)) * kPitchS] = acc[r] / divisor;
     }
   }
   __syncthreads();
 
-  // ---- scores: wavefront (wm, wn) of a 2 x 4 grid owns the 32 x 32 block at rows 32*wm, columns 32*wn
-  // of the 64 x 128 block.  All operands are fetched from LDS first, so that their latency is paid once.
-  // A divisor that is a power of two divides exactly like a multiplication by its reciprocal.
-  {
-    const int wm = wave >> 2, wn = wave & 3;
-    if ((unsigned)(32 * wn) < T) {
-      constexpr int KB = kMaxD / 8;
-      v16f acc;
+  // ---- K is done with: V takes its place
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-      const float* qa = Qs + (32 * wm + lrow) * kPitchQK + 4 * g;
-      const float* ka = Ks + (32 * wn + lrow) * kPitchQK + 4 * g;
-      v4f af[KB], bf[KB];
-#pragma unroll
-      for (int kb = 0; kb < KB; ++kb) {
-        af[kb] = v4f{0.f, 0.f, 0.f, 0.f};
-        bf[kb] = v4f{0.f, 0.f, 0.f, 0.f};
-        if ((unsigned)kb * 8 < Dp) {
-          af[kb] = *reinterpret_cast<const v4f*>(qa + kb * 8);
-          bf[kb] = *reinterpret_cast<const v4f*>(ka + kb * 8);
-        }
-      }
-#pragma unroll
-      for (int kb = 0; kb < KB; ++kb) {
-        if ((unsigned)kb * 8 < Dp) {
-#pragma unroll
-          for (int s = 0; s < 4; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[kb][s], bf[kb][s], acc, 0, 0, 0);
-        }
-      }
-      float* sc = Sc + (32 * wm + 4 * g) * kPitchS + 32 * wn + lrow;
-      const float divisor = p.divisor;
-      const unsigned bits = __builtin_bit_cast(unsigned, divisor), expo = (bits >> 23) & 0xffu;
-      if (!p.divide) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) sc[(8 * (r / 4) + (r & 3)) * kPitchS] = acc[r];
-      } else if ((bits & 0x007fffffu) == 0 && expo >= 2 && expo <= 252) {
-        const float inverse = 1.0f / divisor;  // exact: also a power of two
-#pragma unroll
-        for (int r = 0; r < 16; ++r) sc[(8 * (r / 4) + (r & 3)) * kPitchS] = acc[r] * inverse;
-      } else {
-#pragma unroll
-        for (int r = 0; r < 16; ++r) sc[(8 * (r / 4) + (r & 3)) * kPitchS] = acc[r] / divisor;
-      }
-    }
+  for (int it = 0; it < KV_ITEMS; ++it) {
+    const int w = tid + it * kThreads, row = w / CH, ch = w % CH;
+    *reinterpret_cast<v4f*>(KVs + row * kPitchV + ch * 4) = vreg[it];
   }
-  __syncthreads();
 
   // ---- softmax of each row by one wavefront, eight rows in flight; columns T .. Tp-1 become the zeros
   // the next product reads
@@ -217,31 +229,36 @@ __global__ __launch_bounds__(kThreads) void attention_kernel(const AttentionPara
   __syncthreads();
 
   // ---- probabilities x V: the first four wavefronts, (wm, wn) owning rows 32*wm.. and columns 32*wn.. of the
-  // 64 x D result (one accumulator per element over all of T, as in a product of its own)
+  // 64 x D result (one accumulator per element over all of T, as in a product of its own); operands are
+  // fetched from LDS for eight steps at a time
   const int wm = wave >> 1, wn = wave & 1;
   if (wave < 4 && (unsigned)(32 * wn) < D) {
-    constexpr int KB = kMaxT / 8;
+    constexpr int KB = kMaxT / 8, HALF = KB / 2;
     v16f acc;
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[r] = 0.f;
     const float* pa = Sc + (32 * wm + lrow) * kPitchS + 4 * g;
-    const float* vb = Vs + (4 * g) * kPitchV + 32 * wn + lrow;
-    v4f af[KB], bf[KB];
+    const float* vb = KVs + (4 * g) * kPitchV + 32 * wn + lrow;
 #pragma unroll
-    for (int kb = 0; kb < KB; ++kb) {
-      af[kb] = v4f{0.f, 0.f, 0.f, 0.f};
-      bf[kb] = v4f{0.f, 0.f, 0.f, 0.f};
-      if ((unsigned)kb * 8 < Tp) {
-        af[kb] = *reinterpret_cast<const v4f*>(pa + kb * 8);
+    for (int h = 0; h < 2; ++h) {
+      v4f af[HALF], bf[HALF];
 #pragma unroll
-        for (int s = 0; s < 4; ++s) bf[kb][s] = vb[(kb * 8 + s) * kPitchV];
+      for (int q = 0; q < HALF; ++q) {
+        const int kb = h * HALF + q;
+        af[q] = v4f{0.f, 0.f, 0.f, 0.f};
+        bf[q] = v4f{0.f, 0.f, 0.f, 0.f};
+        if ((unsigned)kb * 8 < Tp) {
+          af[q] = *reinterpret_cast<const v4f*>(pa + kb * 8);
+#pragma unroll
+          for (int s = 0; s < 4; ++s) bf[q][s] = vb[(kb * 8 + s) * kPitchV];
+        }
       }
-    }
 #pragma unroll
-    for (int kb = 0; kb < KB; ++kb) {
-      if ((unsigned)kb * 8 < Tp) {
+      for (int q = 0; q < HALF; ++q) {
+        if ((unsigned)(h * HALF + q) * 8 < Tp) {
 #pragma unroll
-        for (int s = 0; s < 4; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[kb][s], bf[kb][s], acc, 0, 0, 0);
+          for (int s = 0; s < 4; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[q][s], bf[q][s], acc, 0, 0, 0);
+        }
       }
     }
     const unsigned col = 32 * wn + lrow;
@@ -302,7 +319,7 @@ extern "C" int tfcc_rocm_attention_f32(void* stream, const tfcc_rocm_attention_d
   p.divisor = d->divisor;
   p.divide = d->has_divisor ? 1 : 0;
   constexpr size_t ldsBytes = (size_t)kLdsFloats * sizeof(float);
-  static_assert(ldsBytes <= 160 * 1024, "LDS budget");
+  static_assert(ldsBytes <= 80 * 1024, "two workgroups per CU");
   static bool attrSet[16] = {};
   int dev = 0;
   TFCC_HIP_CHECK(hipGetDevice(&dev));
