@@ -22,6 +22,10 @@ FP32_TOL = 1e-5
     (2048, 4096, 64), (2048, 3968, 64),
     # alignment: k or n not a multiple of 4 takes the scalar-load kernel
     (130, 258, 515), (129, 255, 512),
+    # K a multiple of 32: the kernels that copy slabs straight into LDS.  One slab, two (= the ring depth), three;
+    # every tile shape (32x32, 32x64, 32x96, 64x64) with 1, 2 and 4 K groups; ragged M and N edges
+    (64, 64, 32), (64, 64, 64), (33, 36, 96), (96, 96, 256), (512, 512, 512), (128, 3072, 768), (100, 3000, 288),
+    (1000, 760, 736), (1024, 3072, 128), (1021, 3068, 160), (640, 1280, 256), (2048, 2048, 32),
 ])
 def test_sgemm_around_configuration_thresholds(pkg, T, m, n, k):
     print("sgemm", m, n, k, flush=True)
@@ -32,6 +36,8 @@ def test_sgemm_around_configuration_thresholds(pkg, T, m, n, k):
     want = a.astype(np.float64) @ b.astype(np.float64) + bias
     got = T.n(pkg.blas_matmul(T.t(a), T.t(b), T.t(bias)))
     assert got.shape == want.shape and rel_fro(got, want) <= FP32_TOL
+    # every element, not only the norm: a tile edge that went wrong shows up as a few far-off values
+    assert np.abs(got - want).max() <= 1e-4 * max(1.0, np.abs(want).max())
 
 
 @pytest.mark.parametrize("m,n,k", [

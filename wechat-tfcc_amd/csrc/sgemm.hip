@@ -394,13 +394,32 @@ int dispatch(hipStream_t s, const SgemmParams& p, bool vec, bool tb, unsigned fi
     // 32x96 tiles when they cover the 256 CUs in fewer tile-area rounds than 64x64 tiles would
     const unsigned long long flat = (unsigned long long)((m + 31) / 32) * ((n + 95) / 96) * fillBatch;
     const bool preferFlat = ((flat + 255) / 256) * (32 * 96) < ((small + 255) / 256) * (64 * 64);
-    // whole slabs of K: the same tile configurations with the slabs copied straight into LDS (same results)
-    const bool dma = k % 32 == 0;
-    if (preferFlat && flat <= 320 && k >= 512)
-      return dma ? sgemm_detail::sgemm_dma_launch(s, p, 1, 4) : launch<1, 3, 1, 1, true, 4>(s, p);
-    if (small <= 320 && k >= 512) return dma ? sgemm_detail::sgemm_dma_launch(s, p, 0, 4) : launch<2, 2, 1, 1, true, 4>(s, p);
-    if (small <= 640 && k >= 256) return dma ? sgemm_detail::sgemm_dma_launch(s, p, 0, 2) : launch<2, 2, 1, 1, true, 2>(s, p);
-    return dma ? sgemm_detail::sgemm_dma_launch(s, p, 0, 1) : launch<2, 2, 1, 1, true>(s, p);
+    if (k % 32 == 0) {
+      // Whole slabs of K: the kernels that copy the slabs straight into LDS.  Tile: the one that covers the
+      // 256 CUs in the fewest tile-area rounds, the larger one on a tie (less operand traffic).  K groups:
+      // as few as give every CU eight wavefronts, each group keeping at least four slabs.
+      static const struct { int config; unsigned bm, bn, waves; } kTiles[] = {
+          {0, 64, 64, 4}, {1, 32, 96, 3}, {2, 32, 64, 2}, {3, 32, 32, 1}};
+      int best = 0;
+      unsigned long long bestCost = ~0ull, bestTiles = 0;
+      for (int c = 0; c < 4; ++c) {
+        const unsigned long long tiles =
+            (unsigned long long)((m + kTiles[c].bm - 1) / kTiles[c].bm) * ((n + kTiles[c].bn - 1) / kTiles[c].bn) * fillBatch;
+        const unsigned long long cost = ((tiles + 255) / 256) * (kTiles[c].bm * kTiles[c].bn);
+        if (cost < bestCost) {  // the table is ordered by falling tile area
+          best = c;
+          bestCost = cost;
+          bestTiles = tiles;
+        }
+      }
+      int ksplit = 1;
+      while (ksplit < 4 && bestTiles * kTiles[best].waves * ksplit < 256ull * 8 && k >= 128u * (ksplit * 2)) ksplit *= 2;
+      return sgemm_detail::sgemm_dma_launch(s, p, kTiles[best].config, ksplit);
+    }
+    if (preferFlat && flat <= 320 && k >= 512) return launch<1, 3, 1, 1, true, 4>(s, p);
+    if (small <= 320 && k >= 512) return launch<2, 2, 1, 1, true, 4>(s, p);
+    if (small <= 640 && k >= 256) return launch<2, 2, 1, 1, true, 2>(s, p);
+    return launch<2, 2, 1, 1, true>(s, p);
   }
   TFCC_REQUIRE((unsigned long long)m * ldc < (1ull << 32) && (unsigned long long)m * lda < (1ull << 32) &&
                rowsB * ldb < (1ull << 32), "sgemm: operand larger than 2^32 elements");
