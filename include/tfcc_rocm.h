@@ -157,6 +157,9 @@ typedef struct tfcc_rocm_qgemm_desc {
    * may be NULL) receive the int32 result's range (tfcc/core/utils/tfcc_quantizationutils.h:30-43). */
   const float *min_a, *max_a, *min_b, *max_b;
   float *min_c, *max_c;
+  /* Optional: b as packed once by tfcc_rocm_gemv_pack_b (weights).  A product of at most 8 rows
+   * (batch == 1) then streams the packed copy; every other shape reads b. */
+  const void* packed_b;
 } tfcc_rocm_qgemm_desc;
 
 /* int32 result only */

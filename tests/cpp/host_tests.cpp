@@ -9,6 +9,7 @@
 #include <cstdlib>
 #include <functional>
 #include <algorithm>
+#include <array>
 #include <random>
 #include <string>
 #include <thread>
@@ -381,6 +382,40 @@ static void test_quantized_matmul_exact() {
     CHECK(tfcc::data::get(fused) == tfcc::data::get(separate));
     CHECK(tfcc::data::get(acc) == got);
   }
+  // weights prepared once (column sums + packed copy): the same int32 result as the plain call, for decode
+  // shapes (the packed copy is streamed) and for more rows than that (the weights themselves are read)
+  for (unsigned m : {1u, 5u, 8u, 9u, 40u}) {
+    const unsigned k = 512, n = 2064;
+    std::vector<uint8_t> ha(size_t(m) * k);
+    std::vector<int8_t> hb(size_t(k) * n);
+    for (auto& v : ha) v = uint8_t(rng() & 255);
+    for (auto& v : hb) v = int8_t(int(rng() % 255) - 128);
+    tfcc::Variable<uint8_t> a = tfcc::data::set(ha, {m, k});
+    tfcc::Variable<int8_t> b = tfcc::data::set(hb, {k, n});
+    tfcc::Variable<float> tAmin = tfcc::data::set(std::vector<float>{-1.5f}, {1}), tAmax = tfcc::data::set(std::vector<float>{2.25f}, {1});
+    tfcc::Variable<float> tBmin = tfcc::data::set(std::vector<float>{-0.75f}, {1}), tBmax = tfcc::data::set(std::vector<float>{0.5f}, {1});
+    tfcc::Variable<int32_t> ra = tfcc::rocm::quantization::reduce_sum(a, true), rb = tfcc::rocm::quantization::reduce_sum(b, false);
+    tfcc::rocm::quantization::PreparedWeights w(b);
+    CHECK(tfcc::data::get(w.reduceSum()) == tfcc::data::get(rb));
+    tfcc::Variable<int32_t> plain, prepared;
+    tfcc::Variable<float> minC, maxC, minP, maxP;
+    std::tie(plain, minC, maxC) = tfcc::rocm::quantization::matmul(a, ra, tAmin, tAmax, b, rb, tBmin, tBmax);
+    std::tie(prepared, minP, maxP) = tfcc::rocm::quantization::matmul(a, ra, tAmin, tAmax, w, tBmin, tBmax);
+    CHECK(tfcc::data::get(prepared) == tfcc::data::get(plain));
+    CHECK(tfcc::data::get(minP) == tfcc::data::get(minC) && tfcc::data::get(maxP) == tfcc::data::get(maxC));
+    if (m == 5) {  // and against the definition
+      const long long oa = offset_of(-1.5f, 2.25f), ob = offset_of(-0.75f, 0.5f) + 128;
+      std::vector<int32_t> got = tfcc::data::get(prepared);
+      bool ok = true;
+      for (unsigned i = 0; i < m && ok; ++i)
+        for (unsigned j = 0; j < n; j += 7) {
+          long long sum = 0;
+          for (unsigned q = 0; q < k; ++q) sum += (ha[size_t(i) * k + q] + oa) * (hb[size_t(q) * n + j] + ob);
+          if (got[size_t(i) * n + j] != static_cast<int32_t>(static_cast<uint32_t>(sum))) { ok = false; break; }
+        }
+      CHECK(ok);
+    }
+  }
   // error texts of tfcc/mkl/operations/tfcc_mklquantization.cpp:75-118
   tfcc::Variable<uint8_t> a({4, 8});
   tfcc::Variable<int8_t> b({8, 3}), bBad({7, 3});
@@ -469,6 +504,35 @@ static void thread_body(unsigned seed, int rounds, int* failures) {
   }
 }
 
+static void test_attention_permuted() {
+  // softmax(q k^T / c) v on [batch, seq, heads, size] tensors in one launch against the operations one
+  // at a time (tfcc_runtime runs Transpose, Matmul, Div, Softmax, Matmul, Transpose): the same bits
+  std::mt19937 rng(5);
+  std::normal_distribution<float> dist(0.f, 1.f);
+  const std::vector<size_t> toHeads = {0, 2, 1, 3}, toHeadsT = {0, 2, 3, 1};
+  for (auto dims : {std::array<unsigned, 5>{2, 20, 3, 8, 24}, std::array<unsigned, 5>{1, 70, 2, 64, 128}, std::array<unsigned, 5>{2, 5, 2, 12, 7}}) {
+    const unsigned batch = dims[0], seq = dims[1], heads = dims[2], size = dims[3], keys = dims[4];
+    std::vector<float> hq(size_t(batch) * seq * heads * size), hk(size_t(batch) * keys * heads * size), hv(hk.size());
+    for (auto& x : hq) x = dist(rng);
+    for (auto& x : hk) x = dist(rng);
+    for (auto& x : hv) x = dist(rng);
+    tfcc::Variable<float> q = tfcc::data::set(hq, {batch, seq, heads, size});
+    tfcc::Variable<float> k = tfcc::data::set(hk, {batch, keys, heads, size});
+    tfcc::Variable<float> v = tfcc::data::set(hv, {batch, keys, heads, size});
+    const float divisor = 3.0f;
+    tfcc::Variable<float> scores = tfcc::blas::matmul(tfcc::base::transpose(q, toHeads), tfcc::base::transpose(k, toHeadsT));
+    tfcc::Variable<float> scaled = scores / divisor;
+    tfcc::Variable<float> context = tfcc::blas::matmul(tfcc::math::softmax(scaled, 3), tfcc::base::transpose(v, toHeads));
+    std::vector<float> want = tfcc::data::get(tfcc::base::transpose(context, toHeads));
+    tfcc::Variable<float> fused = tfcc::rocm::blas::attention_permuted(q, toHeads, k, toHeadsT, v, toHeads, toHeads, &divisor);
+    CHECK((fused.shape() == tfcc::Shape({batch, seq, heads, size})));
+    CHECK(tfcc::data::get(fused) == want);
+  }
+  // more keys than the kernel holds in LDS: the caller is told to run the steps separately
+  tfcc::Variable<float> q({1, 4, 1, 8}), k({1, 200, 1, 8}), v({1, 200, 1, 8});
+  CHECK_THROWS(tfcc::rocm::blas::attention_permuted(q, toHeads, k, toHeadsT, v, toHeads, toHeads, nullptr), tfcc::NotImplementedError);
+}
+
 static void test_two_sessions_on_two_threads() {
   int f1 = 0, f2 = 0;
   std::thread t1(thread_body, 11u, 12, &f1), t2(thread_body, 23u, 12, &f2);
@@ -504,6 +568,7 @@ int main(int argc, char** argv) {
     run("quantization.rocm_matmul_round_trips", test_quantized_matmul_round_trips);
     run("quantization.rocm_matmul_exact", test_quantized_matmul_exact);
     run("layer.elementwise", test_layer_ops);
+    run("layer.attention_permuted", test_attention_permuted);
     run("threads.two_sessions", test_two_sessions_on_two_threads);
   } else {
     run("blas.matmul_validation", [] {

@@ -36,6 +36,7 @@ class QGemmDesc(C.Structure):
         ("offset_a", C.c_int32), ("offset_b", C.c_int32),
         ("min_a", C.c_void_p), ("max_a", C.c_void_p), ("min_b", C.c_void_p), ("max_b", C.c_void_p),
         ("min_c", C.c_void_p), ("max_c", C.c_void_p),
+        ("packed_b", C.c_void_p),
     ]
 
 

@@ -436,7 +436,14 @@ extern "C" int tfcc_rocm_gemm_u8s8s32(void* stream, const tfcc_rocm_qgemm_desc* 
   if (int e = fill_params(desc, p)) return e;
   TFCC_REQUIRE(c != nullptr, "quantized matmul: null result");
   p.C = c;
-  // decode shapes: a few rows against a large B are bandwidth bound and take the skinny kernel
+  // decode shapes: a few rows against a large B are bandwidth bound and take the skinny kernel, on the
+  // packed copy of B when the caller has one
+  if (desc->packed_b && p.batch == 1 && gemv_packed_supported(p.A, desc->packed_b, p.M, p.K)) {
+    const float* ranges[4] = {p.minA, p.maxA, p.minB, p.maxB};
+    float* rangeOut[2] = {p.minC, p.maxC};
+    return gemv_packed_launch(as_stream(stream), p.A, desc->packed_b, p.rowsumA, p.colsumB, p.offsetA, p.offsetB,
+                              ranges, rangeOut, p.M, p.N, p.K, c, 0.f, nullptr, nullptr);
+  }
   if (p.batch == 1 && p.M <= 8 && (unsigned long long)p.N * p.K >= (1u << 20) && gemv_supported(p.A, p.B, p.M, p.N, p.K)) {
     const float* ranges[4] = {p.minA, p.maxA, p.minB, p.maxB};
     float* rangeOut[2] = {p.minC, p.maxC};

@@ -13,4 +13,11 @@ int gemv_launch(hipStream_t stream, const unsigned char* a, const signed char* b
                 float* const rangeOut[2], unsigned m, unsigned n, unsigned k, int* accOut,
                 float scaleA, const float* scaleB, float* f32Out);
 
+// The same on weights packed by tfcc_rocm_gemv_pack_b.
+bool gemv_packed_supported(const void* a, const void* packed, unsigned m, unsigned k);
+int gemv_packed_launch(hipStream_t stream, const unsigned char* a, const void* packed, const int* rowsumA,
+                       const int* colsumB, int offsetA, int offsetB, const float* const ranges[4],
+                       float* const rangeOut[2], unsigned m, unsigned n, unsigned k, int* accOut, float scaleA,
+                       const float* scaleB, float* f32Out);
+
 }  // namespace tfcc_rocm

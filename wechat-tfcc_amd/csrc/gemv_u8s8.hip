@@ -213,6 +213,8 @@ __global__ __launch_bounds__(kPackThreads) void gemv_packed_kernel(const GemvPar
     eColsum = p.colsumB[egn];
     if (p.f32Out) eScale = p.scaleB[egn];
   }
+  float mnA = 0.f, mxA = 0.f, mnB = 0.f, mxB = 0.f;  // ranges in device memory override the immediate offsets
+  if (p.minA) { mnA = *p.minA; mxA = *p.maxA; mnB = *p.minB; mxB = *p.maxB; }
   // the wavefronts deal the steps among themselves, kPackInFlight at a time
   for (unsigned t0 = wave * kPackInFlight; t0 < steps; t0 += kPackWaves * kPackInFlight) {
     v4i bv[kPackInFlight], av[kPackInFlight];
@@ -242,6 +244,15 @@ __global__ __launch_bounds__(kPackThreads) void gemv_packed_kernel(const GemvPar
   }
   __syncthreads();
   int oA = p.offsetA, oB = p.offsetB;
+  if (p.minA) {
+    qmatmul_offsets(mnA, mxA, mnB, mxB, &oA, &oB);
+    if (blockIdx.x == 0 && tid == 0) {
+      float mnC, mxC;
+      qmatmul_range(mnA, mxA, mnB, mxB, &mnC, &mxC);
+      if (p.minC) *p.minC = mnC;
+      if (p.maxC) *p.maxC = mxC;
+    }
+  }
   const unsigned offA = (unsigned)oA, offB = (unsigned)oB;
   const unsigned global = offA * offB * K;
   if (eActive) {
@@ -343,6 +354,30 @@ extern "C" int tfcc_rocm_gemv_pack_b(void* stream, const int8_t* b, unsigned n, 
   return check_launch("pack");
 }
 
+namespace tfcc_rocm {
+bool gemv_packed_supported(const void* a, const void* packed, unsigned m, unsigned k) {
+  return m >= 1 && m <= (unsigned)kMaxM && k % 16 == 0 && (uintptr_t)a % 16 == 0 && (uintptr_t)packed % 16 == 0 &&
+         (unsigned long long)m * k < (1ull << 31);
+}
+
+int gemv_packed_launch(hipStream_t stream, const unsigned char* a, const void* packed, const int* rowsumA,
+                       const int* colsumB, int offsetA, int offsetB, const float* const ranges[4],
+                       float* const rangeOut[2], unsigned m, unsigned n, unsigned k, int* accOut, float scaleA,
+                       const float* scaleB, float* f32Out) {
+  GemvParams p{};
+  if (ranges && ranges[0]) {
+    p.minA = ranges[0]; p.maxA = ranges[1]; p.minB = ranges[2]; p.maxB = ranges[3];
+    if (rangeOut) { p.minC = rangeOut[0]; p.maxC = rangeOut[1]; }
+  }
+  p.A = a; p.rowsumA = rowsumA; p.colsumB = colsumB; p.accOut = accOut; p.f32Out = f32Out;
+  p.scaleA = scaleA; p.scaleB = scaleB; p.offsetA = offsetA; p.offsetB = offsetB;
+  p.M = m; p.N = n; p.K = k;
+  hipLaunchKernelGGL(gemv_packed_kernel, dim3((n + 15) / 16), dim3(kPackThreads), 0, stream, p,
+                     static_cast<const unsigned char*>(packed), (k + 63) / 64);
+  return check_launch("skinny quantized matmul (packed)");
+}
+}  // namespace tfcc_rocm
+
 extern "C" int tfcc_rocm_gemv_u8s8s32_packed(void* stream, const uint8_t* a, const void* packed_b,
                                              const int32_t* rowsum_a, const int32_t* colsum_b, int32_t offset_a,
                                              int32_t offset_b, unsigned m, unsigned n, unsigned k, int32_t* acc_out,
@@ -355,11 +390,6 @@ extern "C" int tfcc_rocm_gemv_u8s8s32_packed(void* stream, const uint8_t* a, con
   TFCC_REQUIRE((unsigned long long)m * k < (1ull << 31), "skinny quantized matmul: operand too large");
   TFCC_REQUIRE(acc_out || f32_out, "skinny quantized matmul: no output");
   TFCC_REQUIRE(!f32_out || scale_b, "skinny quantized matmul: dequantize needs scale_b");
-  GemvParams p{};
-  p.A = a; p.rowsumA = rowsum_a; p.colsumB = colsum_b; p.accOut = acc_out; p.f32Out = f32_out;
-  p.scaleA = scale_a; p.scaleB = scale_b; p.offsetA = offset_a; p.offsetB = offset_b;
-  p.M = m; p.N = n; p.K = k;
-  hipLaunchKernelGGL(gemv_packed_kernel, dim3((n + 15) / 16), dim3(kPackThreads), 0, as_stream(stream), p,
-                     static_cast<const unsigned char*>(packed_b), (k + 63) / 64);
-  return check_launch("skinny quantized matmul (packed)");
+  return gemv_packed_launch(as_stream(stream), a, packed_b, rowsum_a, colsum_b, offset_a, offset_b, nullptr, nullptr, m, n,
+                            k, acc_out, scale_a, scale_b, f32_out);
 }

@@ -901,6 +901,27 @@ std::tuple<Variable<int32_t>, Variable<float>, Variable<float>> matmul(
   return std::make_tuple(std::move(result), std::move(minResult), std::move(maxResult));
 }
 
+PreparedWeights::PreparedWeights(const Tensor<int8_t>& b)
+    : _b(&b), _reduceSum(reduce_sum(b, false)), _packed() {
+  if (b.shape().size() != 2 || b.size() == 0) throw InvalidArgumentError("invalid weight tensor b");
+  const unsigned k = b.shape(0), n = b.shape(1);
+  _packed = Variable<uint8_t>({static_cast<unsigned>(tfcc_rocm_gemv_packed_size(n, k))});
+  check(tfcc_rocm_gemv_pack_b(current_stream(), b.data(), n, k, _packed.data()));
+}
+
+std::tuple<Variable<int32_t>, Variable<float>, Variable<float>> matmul(
+    const Tensor<uint8_t>& a, const Tensor<int32_t>& reduceSumA, const Tensor<float>& minA,
+    const Tensor<float>& maxA, const PreparedWeights& w, const Tensor<float>& minB, const Tensor<float>& maxB) {
+  QPlan p = plan(a, reduceSumA, minA, maxA, w.weights(), w.reduceSum(), minB, maxB);
+  Variable<int32_t> result{Shape(p.shape)};
+  Variable<float> minResult({1}), maxResult({1});
+  p.desc.min_c = minResult.data();
+  p.desc.max_c = maxResult.data();
+  p.desc.packed_b = w.packed();
+  check(tfcc_rocm_gemm_u8s8s32(current_stream(), &p.desc, result.data()));
+  return std::make_tuple(std::move(result), std::move(minResult), std::move(maxResult));
+}
+
 std::tuple<Variable<uint8_t>, Variable<float>, Variable<float>> matmul_requantize(
     const Tensor<uint8_t>& a, const Tensor<int32_t>& reduceSumA, const Tensor<float>& minA,
     const Tensor<float>& maxA, const Tensor<int8_t>& b, const Tensor<int32_t>& reduceSumB,

@@ -137,6 +137,31 @@ std::tuple<Variable<uint8_t>, Variable<float>, Variable<float>> matmul_requantiz
 template <class T>
 Variable<int32_t> reduce_sum(const Tensor<T>& a, bool row);
 
+// What a constant weight matrix of a quantized matmul needs besides itself, computed once: its column
+// sums (the reference recomputes reduce_sum(b) per call, tfcc/test/quantization.cpp:112-118) and a copy
+// in the layout the skinny kernel streams at full rate (the reference re-packs b inside every call,
+// tfcc/mkl/gemm/tfcc_mklinputpackermanager.h:34-47).  Build it next to the Constant it belongs to; it
+// refers to `b`, which must outlive it, and belongs to the device that was current when it was built.
+class PreparedWeights {
+  const Tensor<int8_t>* _b;
+  Variable<int32_t> _reduceSum;
+  Variable<uint8_t> _packed;
+
+ public:
+  explicit PreparedWeights(const Tensor<int8_t>& b);  // b: [k, n]
+  PreparedWeights(PreparedWeights&&) = default;
+  PreparedWeights& operator=(PreparedWeights&&) = default;
+  const Tensor<int8_t>& weights() const { return *_b; }
+  const Tensor<int32_t>& reduceSum() const { return _reduceSum; }  // reduce_sum(b, false)
+  const void* packed() const { return _packed.data(); }
+};
+
+// matmul(a, reduceSumA, minA, maxA, w.weights(), w.reduceSum(), minB, maxB): the same checks and the
+// same result; products of at most 8 rows stream the packed copy.
+std::tuple<Variable<int32_t>, Variable<float>, Variable<float>> matmul(
+    const Tensor<uint8_t>& a, const Tensor<int32_t>& reduceSumA, const Tensor<float>& minA,
+    const Tensor<float>& maxA, const PreparedWeights& w, const Tensor<float>& minB, const Tensor<float>& maxB);
+
 }  // namespace quantization
 }  // namespace rocm
 }  // namespace tfcc
