@@ -376,6 +376,16 @@ def main():
     traffic_file = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(traffic_file):
         result["roofline"]["traffic"] = json.load(open(traffic_file)).get("qgemm_c3_bytes_per_launch")
+    # What the matrix cores sustain with nothing else in the way: register-resident instruction loops of the
+    # headline's op count (2 x 4 wavefronts per CU, 1024 instructions each), with operands that stay the same
+    # and with operands that change from one instruction to the next like the rows of real matrices.
+    probe_out = torch.empty(512 * 256, dtype=torch.int32, device=dev)
+    stream0 = torch.cuda.current_stream().cuda_stream
+    for label, changing in (("matrix_cores_alone_constant_operands", 0), ("matrix_cores_alone_changing_operands", 1)):
+        def probe():
+            pkg.check(pkg.lib().tfcc_rocm_probe_mfma(stream0, 0, changing, 512, 256, probe_out.data_ptr()))
+        ms = time_launches(torch, probe, args.steps, args.warmup)
+        result["roofline"][label] = round(512 * 4 * 4 * 256 * 65536.0 / ms / 1e9, 2)
     if not args.no_other:
         # on a stream of its own (not the default stream) so that short kernels can be timed as graph replays
         side = torch.cuda.Stream()

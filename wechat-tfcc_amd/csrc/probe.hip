@@ -1,0 +1,100 @@
+// Register-resident matrix-core loops: what the matrix cores of this part sustain when nothing else
+// limits them (no LDS, no memory), with operands that stay the same from one instruction to the next
+// and with operands that change every instruction, as the rows and columns of real matrices do.
+// A measuring aid for the benchmark (it says how far a GEMM kernel is from what the hardware delivers
+// at the clocks its power limit allows); nothing in the library calls it.
+#include "common.hpp"
+
+namespace tfcc_rocm {
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+typedef float v16f __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ unsigned hash32(unsigned x) {
+  x ^= x >> 16; x *= 0x7feb352du; x ^= x >> 15; x *= 0x846ca68bu; x ^= x >> 16;
+  return x;
+}
+
+// Four accumulators per wavefront (independent instructions back to back), four operand pairs.
+template <bool CHANGING>
+__global__ __launch_bounds__(256) void probe_i8_kernel(unsigned iters, int* out) {
+  const unsigned id = blockIdx.x * 256 + threadIdx.x;
+  v4i a[4], b[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const unsigned s = CHANGING ? id * 8 + q : 0x01020304u;  // the same bytes in every lane and register, or noise
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      a[q][e] = (int)(CHANGING ? hash32(s * 4 + e) : s);
+      b[q][e] = (int)(CHANGING ? hash32(s * 4 + e + 0x9e3779b9u) : s);
+    }
+  }
+  v16i c[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) c[j][r] = 0;
+  for (unsigned i = 0; i < iters; i += 4) {  // iters is a multiple of 4
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) c[j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[j], b[(j + q) & 3], c[j], 0, 0, 0);
+  }
+  int s = 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s += c[j][r];
+  out[id] = s;
+}
+
+template <bool CHANGING>
+__global__ __launch_bounds__(256) void probe_f32_kernel(unsigned iters, int* out) {
+  const unsigned id = blockIdx.x * 256 + threadIdx.x;
+  float a[4], b[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    a[q] = CHANGING ? (float)(hash32(id * 8 + q) & 0xffff) / 65536.f - 0.5f : 0.5f;
+    b[q] = CHANGING ? (float)(hash32(id * 8 + q + 4) & 0xffff) / 65536.f - 0.5f : 0.25f;
+  }
+  v16f c[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) c[j][r] = 0.f;
+  for (unsigned i = 0; i < iters; i += 4) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) c[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[j], b[(j + q) & 3], c[j], 0, 0, 0);
+  }
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) s += c[j][r];
+  out[id] = (int)s;
+}
+
+}  // namespace
+}  // namespace tfcc_rocm
+
+using namespace tfcc_rocm;
+
+extern "C" int tfcc_rocm_probe_mfma(void* stream, int kind, int changing_operands, unsigned blocks, unsigned iters,
+                                    int32_t* out) {
+  TFCC_REQUIRE(out != nullptr, "probe: null output (blocks * 256 words)");
+  TFCC_REQUIRE(blocks > 0 && blocks <= 65536 && iters > 0 && iters % 4 == 0, "probe: blocks 1..65536, iters a positive multiple of 4");
+  TFCC_REQUIRE(kind == 0 || kind == 1, "probe: kind 0 (int8 32x32x32) or 1 (fp32 32x32x2)");
+  hipStream_t s = as_stream(stream);
+  if (kind == 0) {
+    if (changing_operands) hipLaunchKernelGGL(probe_i8_kernel<true>, dim3(blocks), dim3(256), 0, s, iters, out);
+    else hipLaunchKernelGGL(probe_i8_kernel<false>, dim3(blocks), dim3(256), 0, s, iters, out);
+  } else {
+    if (changing_operands) hipLaunchKernelGGL(probe_f32_kernel<true>, dim3(blocks), dim3(256), 0, s, iters, out);
+    else hipLaunchKernelGGL(probe_f32_kernel<false>, dim3(blocks), dim3(256), 0, s, iters, out);
+  }
+  return check_launch("probe");
+}
