@@ -245,6 +245,28 @@ def bench_other(torch, pkg, dev, steps, warmup, c3):
         out["c5_int8_gemv_m%d_4096x11008" % m] = {"ms": round(ms, 5), "gbs": round(gbs, 1),
                                                    "frac_hbm": round(gbs / PEAK_HBM_GBS, 4),
                                                    "gops": round(2.0 * m * n * k / ms / 1e6, 1)}
+    # what bounds those launches on this part: a launch that only reads the same 45 MB (same rotation of
+    # buffers), and a launch of workgroups that do nothing
+    probe_word = torch.zeros(16, dtype=torch.int32, device=dev)
+    for blocks in (512, 1024, 2048):
+        idx = [0]
+
+        def step():
+            i = idx[0] % sets
+            idx[0] += 1
+            st = lib.tfcc_rocm_probe_read(stream, bs[i].data_ptr(), k * n, blocks, probe_word.data_ptr())
+            if st != 0:
+                pkg.check(st)
+        ms = time_launches(torch, step, max(steps, 50), warmup, pkg, stream)
+        out["probe_read_only_45mb_%d_workgroups" % blocks] = {"ms": round(ms, 5), "gbs": round(k * n / ms / 1e6, 1),
+                                                               "frac_hbm": round(k * n / ms / 1e6 / PEAK_HBM_GBS, 4)}
+
+    def step():
+        st = lib.tfcc_rocm_probe_launch(stream, probe_word.data_ptr())
+        if st != 0:
+            pkg.check(st)
+    out["probe_empty_launch"] = {"ms": round(time_launches(torch, step, max(steps, 50), warmup, pkg, stream), 5)}
+
     # the same decode shapes on weights packed once (column slabs in matrix-core operand order)
     packs = [pkg.gemv_pack(x) for x in bs]
     for m in (1, 4, 8):

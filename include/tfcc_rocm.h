@@ -246,6 +246,11 @@ int tfcc_rocm_quantize_minmax(void* stream, const float* in, uint64_t total, voi
  * out receives blocks * 256 words that only keep the loop alive. */
 int tfcc_rocm_probe_mfma(void* stream, int kind, int changing_operands, unsigned blocks, unsigned iters,
                          int32_t* out);
+/* More measuring aids: a launch that only reads `bytes` from src once (blocks workgroups of 512 threads,
+ * contiguous shares, 16-byte loads) - the time a read-bound kernel of that size cannot beat - and a
+ * launch of 256 workgroups that do nothing - the time from dispatch to completion that every kernel pays. */
+int tfcc_rocm_probe_read(void* stream, const void* src, uint64_t bytes, unsigned blocks, int32_t* out);
+int tfcc_rocm_probe_launch(void* stream, int32_t* out);
 
 /* ---------------------------------------------------------------------------------------------
  * The element-wise neighbours of matmul inside one transformer encoder layer (fp32).

@@ -167,7 +167,7 @@ def test_gemv_against_oracle(pkg, T, m, n, k):
 
 
 @pytest.mark.parametrize("m", [1, 5, 8])
-@pytest.mark.parametrize("n,k", [(11008, 4096), (16, 16), (100, 80), (260, 4000), (4096, 8320)])
+@pytest.mark.parametrize("n,k", [(11008, 4096), (16, 16), (100, 80), (260, 4000), (4096, 8320), (64, 12352)])
 def test_gemv_on_packed_weights(pkg, T, m, n, k):
     print("gemv packed", m, n, k, flush=True)
     rng = np.random.default_rng(m * 7 + n + k)

@@ -62,7 +62,8 @@ __device__ __forceinline__ void transpose4x4(const unsigned r[4], unsigned c[4])
 __global__ __launch_bounds__(kThreads) void gemv_kernel(const GemvParams p) {
   __shared__ int red[kWaves][kPartRows][kCols];
 
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: the step loop's bounds stay scalar
   // consecutive workgroup ids go to different XCDs: give each XCD a run of adjacent column groups
   const unsigned cg = (blockIdx.x & 7u) * p.groupsPerXcd + (blockIdx.x >> 3);
   if ((blockIdx.x >> 3) >= p.groupsPerXcd || cg >= p.colGroups) return;
@@ -166,7 +167,9 @@ __global__ __launch_bounds__(kThreads) void gemv_kernel(const GemvParams p) {
 // v_mfma_i32_16x16x64_i8, so a wavefront fetches an operand with one contiguous 1 KiB load and no
 // byte shuffling, and a workgroup streams one contiguous slab (K x 16 bytes).  Rows past K and columns
 // past N are stored as zeros.
-constexpr int kPackWaves = 4;
+constexpr int kPackWaves = 4;   // wavefronts that share the K steps of one 16-column slab (one slab per workgroup:
+                                // two slabs sharing one staged copy of A measured slower, 12.4 against 10.0 us)
+constexpr int kStageLoads = 8;  // 16-byte loads per thread in flight while A is staged
 constexpr int kPackThreads = kPackWaves * 64;
 constexpr int kPackInFlight = 16;  // operand loads in flight per wavefront
 
@@ -191,10 +194,18 @@ __global__ __launch_bounds__(256) void gemv_pack_kernel(const signed char* b, un
   *reinterpret_cast<v4i*>(packed + c * 16) = v4i{(int)w[0], (int)w[1], (int)w[2], (int)w[3]};
 }
 
+// STAGE_A: the rows of A (at most 8 x K bytes, the same for every workgroup) are copied to LDS once with
+// full-width loads, already xor 0x80, and the operands are read from there.  Fetching them from memory
+// per step costs as many load instructions as the B stream itself, mostly empty (M * 4 of 64 lanes):
+// 12.7 us against 8.8 us without them for 4096 x 11008.  Without STAGE_A (A too large for LDS) the
+// operands are fetched per step.
+template <bool STAGE_A>
 __global__ __launch_bounds__(kPackThreads) void gemv_packed_kernel(const GemvParams p, const unsigned char* packed,
                                                                   unsigned steps) {
   __shared__ int red[kPackWaves][kPartRows][16];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  extern __shared__ __align__(16) unsigned char aLds[];  // [M][steps * 64 + 16]: the pad spreads the rows over the banks
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: the step loop's bounds stay scalar
   const unsigned slab = blockIdx.x;
   const unsigned M = p.M, N = p.N, K = p.K;
   const int j = lane & 15, kg = lane >> 4;
@@ -215,21 +226,56 @@ __global__ __launch_bounds__(kPackThreads) void gemv_packed_kernel(const GemvPar
   }
   float mnA = 0.f, mxA = 0.f, mnB = 0.f, mxB = 0.f;  // ranges in device memory override the immediate offsets
   if (p.minA) { mnA = *p.minA; mxA = *p.maxA; mnB = *p.minB; mxB = *p.maxB; }
-  // the wavefronts deal the steps among themselves, kPackInFlight at a time
-  for (unsigned t0 = wave * kPackInFlight; t0 < steps; t0 += kPackWaves * kPackInFlight) {
-    v4i bv[kPackInFlight], av[kPackInFlight];
+
+  // the wavefronts deal the steps among themselves, kPackInFlight at a time; the first batch of B is
+  // requested before A is staged
+  v4i bv[kPackInFlight];
+  auto loadB = [&](unsigned t0) {
 #pragma unroll
     for (int u = 0; u < kPackInFlight; ++u) {
       const unsigned t = t0 + u;
       bv[u] = v4i{0, 0, 0, 0};
+      if (t < steps) bv[u] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(src + (size_t)t * 1024));  // streamed once
+    }
+  };
+  loadB(wave * kPackInFlight);
+  const unsigned pitch = steps * 64 + 16;
+  if constexpr (STAGE_A) {
+    const unsigned chunksPerRow = steps * 4, total = M * chunksPerRow;
+    for (unsigned c0 = 0; c0 < total; c0 += kPackThreads * kStageLoads) {
+      v4i v[kStageLoads];
+#pragma unroll
+      for (int u = 0; u < kStageLoads; ++u) {
+        const unsigned c = c0 + u * kPackThreads + tid, row = c / chunksPerRow, ch = c - row * chunksPerRow;
+        // past the end of a row (K not a multiple of 64) and past the last row: zeros from the bounds check
+        const unsigned off = (c < total && ch * 16 < K) ? row * K + ch * 16 : 0xfffffff0u;
+        v[u] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrcA, off, 0, 0));
+      }
+#pragma unroll
+      for (int u = 0; u < kStageLoads; ++u) {
+        const unsigned c = c0 + u * kPackThreads + tid, row = c / chunksPerRow, ch = c - row * chunksPerRow;
+        if (c < total) *reinterpret_cast<v4i*>(aLds + row * pitch + ch * 16) = v[u] ^ (int)0x80808080;
+      }
+    }
+    __syncthreads();
+  }
+  for (unsigned t0 = wave * kPackInFlight; t0 < steps; t0 += kPackWaves * kPackInFlight) {
+    if (t0 != (unsigned)wave * kPackInFlight) loadB(t0);
+    v4i av[kPackInFlight];
+#pragma unroll
+    for (int u = 0; u < kPackInFlight; ++u) {
+      const unsigned t = t0 + u;
       av[u] = v4i{0, 0, 0, 0};
       if (t < steps) {
-        bv[u] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(src + (size_t)t * 1024));  // streamed once
-        if ((unsigned)j < M)
-          av[u] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrcA, (unsigned)j * K + t * 64 + kg * 16, 0, 0)) ^
-                  (int)0x80808080;
-        else if (j == kRows - 1)
+        if ((unsigned)j < M) {
+          if constexpr (STAGE_A)
+            av[u] = *reinterpret_cast<const v4i*>(aLds + (unsigned)j * pitch + t * 64 + kg * 16);
+          else
+            av[u] = __builtin_bit_cast(v4i, __builtin_amdgcn_raw_buffer_load_b128(rsrcA, (unsigned)j * K + t * 64 + kg * 16, 0, 0)) ^
+                    (int)0x80808080;
+        } else if (j == kRows - 1) {
           av[u] = ones;
+        }
       }
     }
 #pragma unroll
@@ -372,8 +418,27 @@ int gemv_packed_launch(hipStream_t stream, const unsigned char* a, const void* p
   p.A = a; p.rowsumA = rowsumA; p.colsumB = colsumB; p.accOut = accOut; p.f32Out = f32Out;
   p.scaleA = scaleA; p.scaleB = scaleB; p.offsetA = offsetA; p.offsetB = offsetB;
   p.M = m; p.N = n; p.K = k;
-  hipLaunchKernelGGL(gemv_packed_kernel, dim3((n + 15) / 16), dim3(kPackThreads), 0, stream, p,
-                     static_cast<const unsigned char*>(packed), (k + 63) / 64);
+  const unsigned steps = (k + 63) / 64;
+  const size_t aBytes = (size_t)m * (steps * 64 + 16);
+  if (aBytes <= 96 * 1024) {
+    auto kern = gemv_packed_kernel<true>;
+    if (aBytes > 48 * 1024) {
+      static bool attrSet[16] = {};  // per device
+      int dev = 0;
+      TFCC_HIP_CHECK(hipGetDevice(&dev));
+      TFCC_REQUIRE(dev >= 0 && dev < 16, "device index %d", dev);
+      if (!attrSet[dev]) {
+        TFCC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           96 * 1024));
+        attrSet[dev] = true;
+      }
+    }
+    hipLaunchKernelGGL(kern, dim3((n + 15) / 16), dim3(kPackThreads), aBytes, stream, p,
+                       static_cast<const unsigned char*>(packed), steps);
+  } else {
+    hipLaunchKernelGGL(gemv_packed_kernel<false>, dim3((n + 15) / 16), dim3(kPackThreads), 0, stream, p,
+                       static_cast<const unsigned char*>(packed), steps);
+  }
   return check_launch("skinny quantized matmul (packed)");
 }
 }  // namespace tfcc_rocm

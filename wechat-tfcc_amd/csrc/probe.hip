@@ -78,10 +78,48 @@ __global__ __launch_bounds__(256) void probe_f32_kernel(unsigned iters, int* out
   out[id] = (int)s;
 }
 
+// Streams `bytes` once: workgroup w reads a contiguous share with 16-byte loads, 16 of them in flight
+// per lane.  Nothing is written (one word, never in practice): the time of a launch is what a kernel
+// bound by reading that many bytes cannot beat on this part.
+__global__ __launch_bounds__(512) void probe_read_kernel(const unsigned char* src, unsigned long long bytes, int* out) {
+  const unsigned long long per = ((bytes / gridDim.x) + 15) / 16 * 16;
+  const unsigned long long lo = blockIdx.x * per, hi = lo + per < bytes ? lo + per : bytes;
+  v4i acc = {0, 0, 0, 0};
+  unsigned long long i = lo + threadIdx.x * 16ull;
+  for (; i + 15ull * 512 * 16 + 16 <= hi; i += 16ull * 512 * 16) {
+    v4i v[16];
+#pragma unroll
+    for (int u = 0; u < 16; ++u) v[u] = __builtin_nontemporal_load(reinterpret_cast<const v4i*>(src + i + u * (512ull * 16)));
+#pragma unroll
+    for (int u = 0; u < 16; ++u) acc += v[u];
+  }
+  for (; i + 16 <= hi; i += 512ull * 16) acc += __builtin_nontemporal_load(reinterpret_cast<const v4i*>(src + i));
+  const int s = acc[0] + acc[1] + acc[2] + acc[3];
+  if (s == 0x12345678) out[0] = s;
+}
+
+__global__ void probe_empty_kernel(int* out) {
+  if (out == nullptr && threadIdx.x == 1024) __builtin_trap();  // never: keeps the kernel from being dropped
+}
+
 }  // namespace
 }  // namespace tfcc_rocm
 
 using namespace tfcc_rocm;
+
+extern "C" int tfcc_rocm_probe_read(void* stream, const void* src, uint64_t bytes, unsigned blocks, int32_t* out) {
+  TFCC_REQUIRE(src && out, "probe: null argument");
+  TFCC_REQUIRE(bytes >= 16 && (uintptr_t)src % 16 == 0 && blocks > 0 && blocks <= 65536, "probe: 16-byte aligned source, 1..65536 blocks");
+  hipLaunchKernelGGL(probe_read_kernel, dim3(blocks), dim3(512), 0, as_stream(stream),
+                     static_cast<const unsigned char*>(src), (unsigned long long)bytes, out);
+  return check_launch("probe");
+}
+
+extern "C" int tfcc_rocm_probe_launch(void* stream, int32_t* out) {
+  TFCC_REQUIRE(out != nullptr, "probe: null argument");
+  hipLaunchKernelGGL(probe_empty_kernel, dim3(256), dim3(256), 0, as_stream(stream), out);
+  return check_launch("probe");
+}
 
 extern "C" int tfcc_rocm_probe_mfma(void* stream, int kind, int changing_operands, unsigned blocks, unsigned iters,
                                     int32_t* out) {
