@@ -414,7 +414,11 @@ int dispatch(hipStream_t s, const SgemmParams& p, bool vec, bool tb, unsigned fi
       }
       int ksplit = 1;
       while (ksplit < 4 && bestTiles * kTiles[best].waves * ksplit < 256ull * 8 && k >= 128u * (ksplit * 2)) ksplit *= 2;
-      return sgemm_detail::sgemm_dma_launch(s, p, kTiles[best].config, ksplit);
+      // Several products in one launch (p.batch counts them; fillBatch = 1 chose the configuration of a single
+      // one so that each is summed exactly as on its own): when they fill the chip without the K groups, one
+      // group per tile plays all of them.
+      const bool serial = ksplit > 1 && bestTiles * (p.batch / fillBatch) * kTiles[best].waves >= 256ull * 8;
+      return sgemm_detail::sgemm_dma_launch(s, p, kTiles[best].config, ksplit, serial);
     }
     if (preferFlat && flat <= 320 && k >= 512) return launch<1, 3, 1, 1, true, 4>(s, p);
     if (small <= 320 && k >= 512) return launch<2, 2, 1, 1, true, 4>(s, p);

@@ -38,8 +38,13 @@ __device__ __forceinline__ int row_swizzle(int row) { return (row >> 1) & 7; }
 
 // WGM x WGN wavefronts, one 32x32 block each; KSPLIT groups of them on the same tile, group q walking
 // the slabs q, q + KSPLIT, ... through a ring of its own.
-template <int WGM, int WGN, int KSPLIT, int STAGES>
+// VSPLIT > 1 (with KSPLIT == 1): one group does the work of VSPLIT groups one slab after the other, with an
+// accumulator per would-be group (slab s goes to accumulator s % VSPLIT) and the same final additions in
+// group order - bit for bit the result of KSPLIT = VSPLIT, for launches that fill the chip without
+// splitting K across wavefronts (several products in one launch).
+template <int WGM, int WGN, int KSPLIT, int STAGES, int VSPLIT = 1>
 __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_dma_kernel(const SgemmParams p) {
+  static_assert(VSPLIT == 1 || KSPLIT == 1, "accumulators per would-be group only without real groups");
   constexpr int GW = WGM * WGN;
   constexpr int BM = WGM * 32, BN = WGN * 32;
   constexpr int A_BYTES = BM * BK * 4, B_BYTES = BK * BN * 4, STAGE_BYTES = A_BYTES + B_BYTES;
@@ -141,9 +146,11 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_dma_kernel(cons
     }
   };
 
-  v16f acc;
+  v16f accs[VSPLIT];
 #pragma unroll
-  for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+  for (int v = 0; v < VSPLIT; ++v)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) accs[v][r] = 0.f;
 
   // ---- operand addresses inside a stage: A row wm*32 + lrow, logical chunk 2*kb + g; B column
   // wn*32 + lrow, k rows 8*kb + 4*g + s
@@ -156,7 +163,7 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_dma_kernel(cons
 #pragma unroll
     for (int s = 0; s < 4; ++s) b[s] = *reinterpret_cast<const float*>(st + bBase + (8 * kb + s) * (BN * 4));
   };
-  auto mma = [&](const v4f& a, const v4f& b) {
+  auto mma = [&](v16f& acc, const v4f& a, const v4f& b) {
 #pragma unroll
     for (int s = 0; s < 4; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc, 0, 0, 0);
   };
@@ -172,23 +179,32 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_dma_kernel(cons
   __syncthreads();
   v4f fa[2], fb[2];
   readOps(0, 0, fa[0], fb[0]);
-  for (unsigned kt = 0; kt < KT; ++kt) {
-    const unsigned cur = kt % STAGES, nxt = (kt + 1) % STAGES;
+  for (unsigned ko = 0; ko < (KT + VSPLIT - 1) / VSPLIT; ++ko) {
 #pragma unroll
-    for (int kb = 0; kb < KS - 1; ++kb) {
-      readOps(cur, kb + 1, fa[(kb + 1) & 1], fb[(kb + 1) & 1]);
-      mma(fa[kb & 1], fb[kb & 1]);
+    for (int v = 0; v < VSPLIT; ++v) {  // a slab past the end of K is all zeros
+      const unsigned kt = ko * VSPLIT + v;
+      const unsigned cur = kt % STAGES, nxt = (kt + 1) % STAGES;
+#pragma unroll
+      for (int kb = 0; kb < KS - 1; ++kb) {
+        readOps(cur, kb + 1, fa[(kb + 1) & 1], fb[(kb + 1) & 1]);
+        mma(accs[v], fa[kb & 1], fb[kb & 1]);
+      }
+      wait_vmcnt<COPIES*(STAGES - 2)>();
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the reads of slab kt have returned
+      __syncthreads();
+      readOps(nxt, 0, fa[0], fb[0]);
+      issueSlab(kt + STAGES);
+      mma(accs[v], fa[(KS - 1) & 1], fb[(KS - 1) & 1]);
     }
-    wait_vmcnt<COPIES*(STAGES - 2)>();
-    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the reads of slab kt have returned
-    __syncthreads();
-    readOps(nxt, 0, fa[0], fb[0]);
-    issueSlab(kt + STAGES);
-    mma(fa[(KS - 1) & 1], fb[(KS - 1) & 1]);
   }
   wait_vmcnt<0>();
   __syncthreads();
 
+  v16f acc = accs[0];
+#pragma unroll
+  for (int v = 1; v < VSPLIT; ++v)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[r] += accs[v][r];
   if constexpr (KSPLIT > 1) {
     // partial tiles of groups 1 .. KSPLIT-1 go through LDS (the rings are idle now) and are added by
     // group 0 in group order
@@ -222,7 +238,7 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_dma_kernel(cons
   }
 }
 
-template <int WGM, int WGN, int KSPLIT, int STAGES>
+template <int WGM, int WGN, int KSPLIT, int STAGES, int VSPLIT = 1>
 int launch(hipStream_t stream, SgemmParams p) {
   constexpr int GW = WGM * WGN, BM = WGM * 32, BN = WGN * 32;
   constexpr int STAGE_BYTES = (BM + BN) * BK * 4, UNITS = STAGE_BYTES / 1024;
@@ -230,7 +246,7 @@ int launch(hipStream_t stream, SgemmParams p) {
   constexpr size_t lds = (size_t)KSPLIT * (STAGES * STAGE_BYTES + (COPIES * GW != UNITS ? 1024 : 0));
   static_assert(lds <= 160 * 1024 && (size_t)(KSPLIT - 1) * BM * BN * sizeof(float) <= lds, "LDS budget");
   if (!sgemm_detail::set_tiles(p, BM, BN)) return set_error(TFCC_ROCM_INVALID_ARGUMENT, "sgemm: too many tiles");
-  auto kern = sgemm_dma_kernel<WGM, WGN, KSPLIT, STAGES>;
+  auto kern = sgemm_dma_kernel<WGM, WGN, KSPLIT, STAGES, VSPLIT>;
   static bool attrSet[16] = {};  // per device: the attribute belongs to the function on one device
   int dev = 0;
   TFCC_HIP_CHECK(hipGetDevice(&dev));
@@ -254,12 +270,14 @@ bool sgemm_dma_available(int config, int ksplit) {
 
 // Two stages everywhere: more workgroups per CU beat a deeper ring (measured 42.3 against 43.9 us with
 // three stages, 1024 x 3072 x 768 in 64x64 tiles).
-int sgemm_dma_launch(hipStream_t stream, SgemmParams p, int config, int ksplit) {
-#define TFCC_DMA_CASE(C, WGM, WGN)                                    \
-  if (config == C) {                                                  \
-    if (ksplit == 1) return launch<WGM, WGN, 1, 2>(stream, p);        \
-    if (ksplit == 2) return launch<WGM, WGN, 2, 2>(stream, p);        \
-    if (ksplit == 4) return launch<WGM, WGN, 4, 2>(stream, p);        \
+int sgemm_dma_launch(hipStream_t stream, SgemmParams p, int config, int ksplit, bool serialGroups) {
+#define TFCC_DMA_CASE(C, WGM, WGN)                                                  \
+  if (config == C) {                                                                \
+    if (ksplit == 1) return launch<WGM, WGN, 1, 2>(stream, p);                      \
+    if (ksplit == 2 && serialGroups) return launch<WGM, WGN, 1, 2, 2>(stream, p);   \
+    if (ksplit == 4 && serialGroups) return launch<WGM, WGN, 1, 2, 4>(stream, p);   \
+    if (ksplit == 2) return launch<WGM, WGN, 2, 2>(stream, p);                      \
+    if (ksplit == 4) return launch<WGM, WGN, 4, 2>(stream, p);                      \
   }
   TFCC_DMA_CASE(0, 2, 2)  // 64 x 64
   TFCC_DMA_CASE(1, 1, 3)  // 32 x 96

@@ -42,7 +42,9 @@ inline bool set_tiles(SgemmParams& p, unsigned bm, unsigned bn) {
 // ksplit 1, 2 or 4 groups of wavefronts on one tile.
 // Requires 16-byte aligned operands and strides, K a multiple of 32 and B not transposed.
 bool sgemm_dma_available(int config, int ksplit);
-int sgemm_dma_launch(hipStream_t stream, SgemmParams p, int config, int ksplit);
+// serialGroups: one group of wavefronts per tile does the work of the `ksplit` groups one slab after the other
+// (same additions, same result) - for launches that fill the chip anyway.
+int sgemm_dma_launch(hipStream_t stream, SgemmParams p, int config, int ksplit, bool serialGroups);
 
 }  // namespace sgemm_detail
 }  // namespace tfcc_rocm
