@@ -210,6 +210,16 @@ def bench_other(torch, pkg, dev, steps, warmup, c3):
 
     attention_case("c2_fp32_attention_one_launch_16x12x128x64", 16, 12, 128, 64)
     sgemm_case("fp32_4096x4096x4096", (4096, 4096), (4096, 4096), False, sets=1)
+    # what the fp32 matrix cores sustain alone (register-resident loop of the 4096^3 instruction count)
+    probe_out = torch.empty(1024 * 256, dtype=torch.int32, device=dev)
+    for label, changing in (("changing", 1),):
+        def step():
+            st = lib.tfcc_rocm_probe_mfma(stream, 1, changing, 1024, 2048, probe_out.data_ptr())
+            if st != 0:
+                pkg.check(st)
+        ms = time_launches(torch, step, max(10, steps // 10), max(3, warmup // 10), pkg, stream)
+        out["probe_fp32_matrix_cores_alone_%s_operands" % label] = {
+            "ms": round(ms, 5), "tflops": round(1024 * 4 * 4 * 2048 * 4096.0 / ms / 1e9, 2)}
 
     # C3 with the int32 accumulators also written (67 MB more traffic)
     a, b, ta, tb, rs, cs, ranges, out_range = c3
