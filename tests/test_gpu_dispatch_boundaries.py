@@ -43,6 +43,8 @@ def test_sgemm_around_configuration_thresholds(pkg, T, m, n, k):
 @pytest.mark.parametrize("m,n,k", [
     # direct-to-LDS kernel: 256x256 tiles from 192 tiles on, 128x128 below; K not a multiple of the 128-byte slab
     (256 * 12, 256 * 16, 144), (256 * 12 - 1, 256 * 16, 144), (256 * 11, 256 * 16, 272), (512, 384, 4000),
+    # 64x128 tiles below 128 tiles of 128x128 (1024 x 768 has 48), 128x128 from there on; ragged edges
+    (1024, 768, 3072), (1000, 752, 272), (64, 128, 128), (2048, 1024, 256), (2048 - 128, 1024, 256),
     # K or N not a multiple of 16: the register-staged kernel
     (300, 272, 1000), (300, 260, 1024),
     # skinny kernel from N * K = 2^20 on (M <= 8), general kernel below

@@ -396,6 +396,11 @@ int qgemm_dma_launch(hipStream_t stream, const QGemmParams& p, bool requant) {
   if (big >= 192) {
     return requant ? launch<256, 256, 2, 4, 2, true>(stream, p) : launch<256, 256, 2, 4, 2, false>(stream, p);
   }
+  // fewer than half a chip of 128x128 tiles: 64x128 tiles (four wavefronts side by side) put twice as many CUs to work
+  const unsigned long long mid = (unsigned long long)((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batch;
+  if (mid < 128) {
+    return requant ? launch<64, 128, 1, 4, 2, true>(stream, p) : launch<64, 128, 1, 4, 2, false>(stream, p);
+  }
   return requant ? launch<128, 128, 2, 2, 2, true>(stream, p) : launch<128, 128, 2, 2, 2, false>(stream, p);
 }
 
