@@ -388,7 +388,7 @@ int dispatch(hipStream_t s, const SgemmParams& p, bool vec, bool tb, unsigned fi
   // 128x128 tiles once there are enough of them to fill the 256 CUs twice over, else 64x64
   const unsigned long long big = (unsigned long long)((m + 127) / 128) * ((n + 127) / 128) * fillBatch;
   if (vec) {
-    if (big >= 512) return launch<4, 1, 1, 4, true>(s, p);
+    if (big >= 512) return k % 32 == 0 ? sgemm_detail::sgemm_dma_launch(s, p, 4, 1, false) : launch<4, 1, 1, 4, true>(s, p);
     // few 64x64 tiles and a long K: several K groups per workgroup keep the CUs that have a tile busy
     const unsigned long long small = (unsigned long long)((m + 63) / 64) * ((n + 63) / 64) * fillBatch;
     // 32x96 tiles when they cover the 256 CUs in fewer tile-area rounds than 64x64 tiles would

@@ -36,17 +36,19 @@ constexpr unsigned kPastEnd = 0xfffffff0u;  // a byte offset past the end of any
 
 __device__ __forceinline__ int row_swizzle(int row) { return (row >> 1) & 7; }
 
-// WGM x WGN wavefronts, one 32x32 block each; KSPLIT groups of them on the same tile, group q walking
-// the slabs q, q + KSPLIT, ... through a ring of its own.
+// WGM x WGN wavefronts, each owning a 32 x (32 * NI) block (a lane owns NI consecutive columns); KSPLIT
+// groups of them on the same tile, group q walking the slabs q, q + KSPLIT, ... through a ring of its own.
 // VSPLIT > 1 (with KSPLIT == 1): one group does the work of VSPLIT groups one slab after the other, with an
 // accumulator per would-be group (slab s goes to accumulator s % VSPLIT) and the same final additions in
 // group order - bit for bit the result of KSPLIT = VSPLIT, for launches that fill the chip without
 // splitting K across wavefronts (several products in one launch).
-template <int WGM, int WGN, int KSPLIT, int STAGES, int VSPLIT = 1>
+template <int WGM, int WGN, int NI, int KSPLIT, int STAGES, int VSPLIT = 1>
 __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_dma_kernel(const SgemmParams p) {
   static_assert(VSPLIT == 1 || KSPLIT == 1, "accumulators per would-be group only without real groups");
+  static_assert(NI == 1 || NI == 4, "a lane reads its B operands as one or four consecutive words");
   constexpr int GW = WGM * WGN;
-  constexpr int BM = WGM * 32, BN = WGN * 32;
+  constexpr int WN = 32 * NI;
+  constexpr int BM = WGM * 32, BN = WGN * WN;
   constexpr int A_BYTES = BM * BK * 4, B_BYTES = BK * BN * 4, STAGE_BYTES = A_BYTES + B_BYTES;
   constexpr int A_UNITS = A_BYTES / 1024, UNITS = STAGE_BYTES / 1024;  // 1 KB copies per slab
   constexpr int COPIES = (UNITS + GW - 1) / GW;                        // per wavefront per slab
@@ -101,15 +103,20 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_dma_kernel(cons
   const int lrow = lane & 31, g = lane >> 5;
 
   // values needed only in the tile store are fetched now: at the end their latency would be waited for in full
-  const unsigned gcol = n0 + wn * 32 + lrow;
-  const float bv = (biasPtr && gcol < N) ? biasPtr[gcol] : 0.f;
-  float rv[16];
-  if (p.residual && grp == 0) {
-    const float* Rp = p.residual + (size_t)bi * p.strideR;
+  const unsigned gcol = n0 + wn * WN + NI * lrow;  // first of this lane's NI columns
+  float bv[NI];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const unsigned grow = m0 + wm * 32 + 8 * (r / 4) + 4 * g + (r & 3);
-      rv[r] = (grow < M && gcol < N) ? Rp[(size_t)grow * N + gcol] : 0.f;
+  for (int j = 0; j < NI; ++j) bv[j] = (biasPtr && gcol + j < N) ? biasPtr[gcol + j] : 0.f;
+  constexpr bool EARLY_RESIDUAL = NI == 1;  // short launches on small tiles; a large tile fetches it in the store
+  float rv[EARLY_RESIDUAL ? 16 : 1];
+  if constexpr (EARLY_RESIDUAL) {
+    if (p.residual && grp == 0) {
+      const float* Rp = p.residual + (size_t)bi * p.strideR;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const unsigned grow = m0 + wm * 32 + 8 * (r / 4) + 4 * g + (r & 3);
+        rv[r] = (grow < M && gcol < N) ? Rp[(size_t)grow * N + gcol] : 0.f;
+      }
     }
   }
 
@@ -146,26 +153,39 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_dma_kernel(cons
     }
   };
 
-  v16f accs[VSPLIT];
+  v16f accs[VSPLIT][NI];
 #pragma unroll
   for (int v = 0; v < VSPLIT; ++v)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) accs[v][r] = 0.f;
+    for (int j = 0; j < NI; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) accs[v][j][r] = 0.f;
 
-  // ---- operand addresses inside a stage: A row wm*32 + lrow, logical chunk 2*kb + g; B column
-  // wn*32 + lrow, k rows 8*kb + 4*g + s
+  // ---- operand addresses inside a stage: A row wm*32 + lrow, logical chunk 2*kb + g; B columns
+  // wn*WN + NI*lrow .. + NI-1, k rows 8*kb + 4*g + s
+  struct BOps { float v[4][NI]; };  // [s][j]
   const int arow = wm * 32 + lrow;
   const int aBase = arow * (BK * 4), aSwz = row_swizzle(arow);
-  const int bBase = A_BYTES + (4 * g) * (BN * 4) + (wn * 32 + lrow) * 4;
-  auto readOps = [&](unsigned stage, int kb, v4f& a, v4f& b) {
+  const int bBase = A_BYTES + (4 * g) * (BN * 4) + (wn * WN + NI * lrow) * 4;
+  auto readOps = [&](unsigned stage, int kb, v4f& a, BOps& b) {
     const unsigned char* st = gsm + stage * STAGE_BYTES;
     a = *reinterpret_cast<const v4f*>(st + aBase + (((2 * kb + g) ^ aSwz) << 4));
 #pragma unroll
-    for (int s = 0; s < 4; ++s) b[s] = *reinterpret_cast<const float*>(st + bBase + (8 * kb + s) * (BN * 4));
-  };
-  auto mma = [&](v16f& acc, const v4f& a, const v4f& b) {
+    for (int s = 0; s < 4; ++s) {
+      if constexpr (NI == 4) {
+        const v4f w = *reinterpret_cast<const v4f*>(st + bBase + (8 * kb + s) * (BN * 4));
 #pragma unroll
-    for (int s = 0; s < 4; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc, 0, 0, 0);
+        for (int j = 0; j < 4; ++j) b.v[s][j] = w[j];
+      } else {
+        b.v[s][0] = *reinterpret_cast<const float*>(st + bBase + (8 * kb + s) * (BN * 4));
+      }
+    }
+  };
+  auto mma = [&](v16f (&acc)[NI], const v4f& a, const BOps& b) {
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+#pragma unroll
+      for (int j = 0; j < NI; ++j) acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b.v[s][j], acc[j], 0, 0, 0);
   };
 
   // ---- software pipeline.  Before the barrier of slab kt: this wavefront's copies of slab kt+1 have
@@ -177,7 +197,8 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_dma_kernel(cons
   for (int s = 0; s < STAGES; ++s) issueSlab(s);
   wait_vmcnt<COPIES*(STAGES - 1)>();
   __syncthreads();
-  v4f fa[2], fb[2];
+  v4f fa[2];
+  BOps fb[2];
   readOps(0, 0, fa[0], fb[0]);
   for (unsigned ko = 0; ko < (KT + VSPLIT - 1) / VSPLIT; ++ko) {
 #pragma unroll
@@ -200,53 +221,84 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_dma_kernel(cons
   wait_vmcnt<0>();
   __syncthreads();
 
-  v16f acc = accs[0];
+  v16f acc[NI];
 #pragma unroll
-  for (int v = 1; v < VSPLIT; ++v)
+  for (int j = 0; j < NI; ++j) {
+    acc[j] = accs[0][j];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[r] += accs[v][r];
+    for (int v = 1; v < VSPLIT; ++v)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[j][r] += accs[v][j][r];
+  }
   if constexpr (KSPLIT > 1) {
     // partial tiles of groups 1 .. KSPLIT-1 go through LDS (the rings are idle now) and are added by
     // group 0 in group order
     float* red = reinterpret_cast<float*>(smem);
     if (grp > 0) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) red[((((grp - 1) * GW + wave) * 16 + r) * 64) + lane] = acc[r];
+      for (int j = 0; j < NI; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) red[(((((grp - 1) * GW + wave) * NI + j) * 16 + r) * 64) + lane] = acc[j][r];
     }
     __syncthreads();
     if (grp > 0) return;
 #pragma unroll
     for (int q = 1; q < KSPLIT; ++q)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) acc[r] += red[((((q - 1) * GW + wave) * 16 + r) * 64) + lane];
+      for (int j = 0; j < NI; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[j][r] += red[(((((q - 1) * GW + wave) * NI + j) * 16 + r) * 64) + lane];
   }
 
-  // ---- tile store: + bias, + residual, GELU.  Lane (lrow, g) owns column lrow of the wavefront's block
-  // and rows 8*(r/4) + 4*g + r%4.
+  // ---- tile store: + bias, + residual, GELU.  Lane (lrow, g) owns columns NI*lrow .. of the wavefront's
+  // block and rows 8*(r/4) + 4*g + r%4.
   if (gcol >= N) return;
-  const bool hasResidual = p.residual != nullptr;
+  const float* R = p.residual ? p.residual + (size_t)bi * p.strideR : nullptr;  // dense, flat batch
   const int act = p.act;
+  const bool whole = gcol + NI <= N;
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const unsigned grow = m0 + wm * 32 + 8 * (r / 4) + 4 * g + (r & 3);
     if (grow >= M) continue;
-    float v = acc[r] + bv;
-    if (hasResidual) v += rv[r];
+    float v[NI];
+#pragma unroll
+    for (int j = 0; j < NI; ++j) v[j] = acc[j][r] + bv[j];
+    if (R) {
+      if constexpr (EARLY_RESIDUAL) {
+        v[0] += rv[r];
+      } else {
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+          if (gcol + j < N) v[j] += R[(size_t)grow * N + gcol + j];
+      }
+    }
     // same expression as the stand-alone GELU kernel, so that fusing changes no bit
-    if (act == 1) v = (float)(0.5 * (double)v * (double)(1.0f + erff(v / 1.4142135623730951f)));
-    Cbase[(size_t)grow * ldc + gcol] = v;
+    if (act == 1) {
+#pragma unroll
+      for (int j = 0; j < NI; ++j) v[j] = (float)(0.5 * (double)v[j] * (double)(1.0f + erff(v[j] / 1.4142135623730951f)));
+    }
+    float* dst = Cbase + (size_t)grow * ldc + gcol;
+    if constexpr (NI == 4) {
+      if (whole) {
+        *reinterpret_cast<v4f*>(dst) = v4f{v[0], v[1], v[2], v[3]};
+        continue;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < NI; ++j)
+      if (gcol + j < N) dst[j] = v[j];
   }
 }
 
-template <int WGM, int WGN, int KSPLIT, int STAGES, int VSPLIT = 1>
+template <int WGM, int WGN, int NI, int KSPLIT, int STAGES, int VSPLIT = 1>
 int launch(hipStream_t stream, SgemmParams p) {
-  constexpr int GW = WGM * WGN, BM = WGM * 32, BN = WGN * 32;
+  constexpr int GW = WGM * WGN, BM = WGM * 32, BN = WGN * 32 * NI;
   constexpr int STAGE_BYTES = (BM + BN) * BK * 4, UNITS = STAGE_BYTES / 1024;
   constexpr int COPIES = (UNITS + GW - 1) / GW;
   constexpr size_t lds = (size_t)KSPLIT * (STAGES * STAGE_BYTES + (COPIES * GW != UNITS ? 1024 : 0));
   static_assert(lds <= 160 * 1024 && (size_t)(KSPLIT - 1) * BM * BN * sizeof(float) <= lds, "LDS budget");
   if (!sgemm_detail::set_tiles(p, BM, BN)) return set_error(TFCC_ROCM_INVALID_ARGUMENT, "sgemm: too many tiles");
-  auto kern = sgemm_dma_kernel<WGM, WGN, KSPLIT, STAGES, VSPLIT>;
+  auto kern = sgemm_dma_kernel<WGM, WGN, NI, KSPLIT, STAGES, VSPLIT>;
   static bool attrSet[16] = {};  // per device: the attribute belongs to the function on one device
   int dev = 0;
   TFCC_HIP_CHECK(hipGetDevice(&dev));
@@ -265,7 +317,7 @@ int launch(hipStream_t stream, SgemmParams p) {
 namespace sgemm_detail {
 
 bool sgemm_dma_available(int config, int ksplit) {
-  return config >= 0 && config <= 3 && (ksplit == 1 || ksplit == 2 || ksplit == 4);
+  return (config >= 0 && config <= 3 && (ksplit == 1 || ksplit == 2 || ksplit == 4)) || (config == 4 && ksplit == 1);
 }
 
 // Two stages everywhere: more workgroups per CU beat a deeper ring (measured 42.3 against 43.9 us with
@@ -273,17 +325,18 @@ bool sgemm_dma_available(int config, int ksplit) {
 int sgemm_dma_launch(hipStream_t stream, SgemmParams p, int config, int ksplit, bool serialGroups) {
 #define TFCC_DMA_CASE(C, WGM, WGN)                                                  \
   if (config == C) {                                                                \
-    if (ksplit == 1) return launch<WGM, WGN, 1, 2>(stream, p);                      \
-    if (ksplit == 2 && serialGroups) return launch<WGM, WGN, 1, 2, 2>(stream, p);   \
-    if (ksplit == 4 && serialGroups) return launch<WGM, WGN, 1, 2, 4>(stream, p);   \
-    if (ksplit == 2) return launch<WGM, WGN, 2, 2>(stream, p);                      \
-    if (ksplit == 4) return launch<WGM, WGN, 4, 2>(stream, p);                      \
+    if (ksplit == 1) return launch<WGM, WGN, 1, 1, 2>(stream, p);                      \
+    if (ksplit == 2 && serialGroups) return launch<WGM, WGN, 1, 1, 2, 2>(stream, p);   \
+    if (ksplit == 4 && serialGroups) return launch<WGM, WGN, 1, 1, 2, 4>(stream, p);   \
+    if (ksplit == 2) return launch<WGM, WGN, 1, 2, 2>(stream, p);                      \
+    if (ksplit == 4) return launch<WGM, WGN, 1, 4, 2>(stream, p);                      \
   }
   TFCC_DMA_CASE(0, 2, 2)  // 64 x 64
   TFCC_DMA_CASE(1, 1, 3)  // 32 x 96
   TFCC_DMA_CASE(2, 1, 2)  // 32 x 64
   TFCC_DMA_CASE(3, 1, 1)  // 32 x 32
 #undef TFCC_DMA_CASE
+  if (config == 4 && ksplit == 1) return launch<4, 1, 4, 1, 2>(stream, p);  // 128 x 128: four wavefronts of 32 x 128
   return set_error(TFCC_ROCM_INVALID_ARGUMENT, "sgemm: no direct-to-LDS kernel for this configuration");
 }
 
