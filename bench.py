@@ -185,6 +185,39 @@ def bench_other(torch, pkg, dev, steps, warmup, c3):
     sgemm_case("c2_fp32_pv_16x12x128x128x64", (16, 12, 128, 128), (16, 12, 128, 64), False)
     sgemm_case("c4_fp32_ffn_up_1024x768x3072_bias", (8, 128, 768), (768, 3072), True)
 
+    # C2, second case: a [1, 12, 64, 64] weight broadcast over the batch of a [16, 12, 128, 64] input
+    def broadcast_case(name, shape_a, shape_b, sets=4):
+        p = pkg.matmul_plan(shape_a, shape_b)
+        g = p["grid"]
+        bufs = []
+        for _ in range(sets):
+            a = torch.randn(shape_a, device=dev, dtype=torch.float32)
+            b = torch.randn(shape_b, device=dev, dtype=torch.float32)
+            c = torch.empty(p["shape"], device=dev, dtype=torch.float32)
+            d = pkg.SgemmDesc()
+            d.a, d.b, d.c = a.data_ptr(), b.data_ptr(), c.data_ptr()
+            d.m, d.n, d.k, d.lda, d.ldb, d.ldc = p["m"], p["n"], p["k"], p["k"], p["n"], p["n"]
+            d.batch_outer, d.batch_inner = g["outer"], g["inner"]
+            d.stride_a, d.stride_b, d.stride_c = g["strides"]
+            d.inner_stride_a, d.inner_stride_b, d.inner_stride_c = g["inner_strides"]
+            bufs.append((d, (a, b, c)))
+        idx = [0]
+
+        def step():
+            d = bufs[idx[0] % sets][0]
+            idx[0] += 1
+            st = lib.tfcc_rocm_sgemm_general(stream, C.byref(d))
+            if st != 0:
+                pkg.check(st)
+        ms = time_launches(torch, step, steps, warmup, pkg, stream)
+        flop = 2.0 * p["m"] * p["n"] * p["k"] * p["batch"]
+        nbytes = 4.0 * (int(np.prod(shape_a)) + int(np.prod(shape_b)) + int(np.prod(p["shape"])))
+        out[name] = {"ms": round(ms, 5), "tflops": round(flop / ms / 1e9, 3),
+                     "frac_fp32_mfma": round(flop / ms / 1e9 / PEAK_FP32_TFLOPS, 4), "gbs": round(nbytes / ms / 1e6, 1),
+                     "frac_hbm": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
+
+    broadcast_case("c2_fp32_broadcast_16x12x128x64_by_1x12x64x64", (16, 12, 128, 64), (1, 12, 64, 64))
+
     # C2 as one launch: softmax(q k^T / 8) v on [batch, seq, heads, size] tensors, 16 x 12 heads of 128 x 64
     def attention_case(name, B, H, S, D, sets=4):
         bufs = []

@@ -108,7 +108,7 @@ int tfcc_rocm_sgemm_fused(void* stream, const float* a, uint64_t stride_a, const
  * (trans_b), a result written in [batch, seq, heads, size] order - where the reference materialises
  * each permutation first with base::transpose (tfcc/core/operations/tfcc_base.cpp:124-134) because
  * its matmul has no stride or transpose arguments (tfcc/core/operations/tfcc_blas.cpp:26-58).
- * All strides are in elements.  A residual requires ldc == n and batch_inner == 1. */
+ * All strides are in elements.  A residual requires a dense result (ldc == n, batch entries back to back). */
 typedef struct tfcc_rocm_sgemm_desc {
   const float* a;        /* [m, k], row stride lda */
   const float* b;        /* [k, n], row stride ldb; with trans_b: [n, k], row stride ldb */

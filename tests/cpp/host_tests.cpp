@@ -192,11 +192,11 @@ static void test_matmul_validation() {
   // tfcc/core/operations/tfcc_blas.cpp:26-54: thrown before any device work
   using tfcc::InvalidArgumentError;
   tfcc::Variable<float> v3({3}), m34({3, 4}), m45({4, 5}), m56({5, 6}), b234({2, 3, 4}), b5647({5, 6, 4, 7}),
-      b145({1, 4, 5}), bias4({4}), bias15({1, 5});
+      b345({3, 4, 5}), bias4({4}), bias15({1, 5});
   CHECK_THROWS_MSG(tfcc::blas::matmul(v3, m34), InvalidArgumentError, "matmul require tensors with two or more dimensions");
   CHECK_THROWS_MSG(tfcc::blas::matmul(b234, b5647), InvalidArgumentError, "shape invalid");
   CHECK_THROWS_MSG(tfcc::blas::matmul(m34, m56), InvalidArgumentError, "shape invalid");
-  CHECK_THROWS_MSG(tfcc::blas::matmul(b234, b145), InvalidArgumentError, "shape invalid");  // no size-1 broadcast
+  CHECK_THROWS_MSG(tfcc::blas::matmul(b234, b345), InvalidArgumentError, "shape invalid");  // unequal leading dimensions
   CHECK_THROWS_MSG(tfcc::blas::matmul(m34, m45, bias4), InvalidArgumentError, "shape invalid");
   CHECK_THROWS_MSG(tfcc::blas::matmul(m34, m45, bias15), InvalidArgumentError, "shape invalid");
   tfcc::Variable<float> e({2, 0, 4}), f({2, 4, 5});
@@ -286,6 +286,33 @@ static void test_blas() {
     matmul_case(rng, {m, k}, {b1, k, n});
     matmul_case(rng, {b1, b2, m, k}, {b1, b2, k, n});
   }
+}
+
+static void test_matmul_broadcast() {
+  // a leading dimension of 1 on one side is broadcast (beyond tfcc/core/operations/tfcc_blas.cpp:36-42)
+  std::mt19937 rng(3);
+  std::uniform_real_distribution<float> dist(-1.f, 1.f);
+  const unsigned batch = 3, heads = 2, m = 5, k = 8, n = 4;
+  std::vector<float> ha(batch * heads * m * k), hb(heads * k * n);
+  for (auto& v : ha) v = dist(rng);
+  for (auto& v : hb) v = dist(rng);
+  tfcc::Variable<float> a = tfcc::data::set(ha, {batch, heads, m, k});
+  tfcc::Variable<float> b = tfcc::data::set(hb, {1, heads, k, n});
+  tfcc::Variable<float> c = tfcc::blas::matmul(a, b);
+  CHECK((c.shape() == tfcc::Shape({batch, heads, m, n})));
+  std::vector<float> got = tfcc::data::get(c);
+  bool ok = true;
+  for (unsigned x = 0; x < batch; ++x)
+    for (unsigned h = 0; h < heads; ++h)
+      for (unsigned i = 0; i < m; ++i)
+        for (unsigned j = 0; j < n; ++j) {
+          double s = 0;
+          for (unsigned p = 0; p < k; ++p) s += double(ha[((x * heads + h) * m + i) * k + p]) * double(hb[(h * k + p) * n + j]);
+          ok = ok && is_similar(got[((x * heads + h) * m + i) * n + j], float(s));
+        }
+  CHECK(ok);
+  tfcc::Variable<float> bad({2, heads, k, n});
+  CHECK_THROWS_MSG(tfcc::blas::matmul(a, bad), tfcc::InvalidArgumentError, "shape invalid");
 }
 
 static void test_dequantize_requantize_known_answers() {
@@ -564,6 +591,7 @@ int main(int argc, char** argv) {
     run("blas.matmul_validation", test_matmul_validation);
     run("data.set_get_copy", test_data);
     run("blas.matmul", test_blas);
+    run("blas.matmul_broadcast", test_matmul_broadcast);
     run("quantization.known_answers", test_dequantize_requantize_known_answers);
     run("quantization.rocm_matmul_round_trips", test_quantized_matmul_round_trips);
     run("quantization.rocm_matmul_exact", test_quantized_matmul_exact);

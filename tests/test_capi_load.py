@@ -42,7 +42,7 @@ def test_bad_arguments_are_rejected_without_a_device(pkg):
 def test_matmul_plan_rules(pkg):
     # tfcc/core/operations/tfcc_blas.cpp:26-42 and tfcc/mkl/interfaces/tfcc_mklblasinterface.cpp:127-145
     import oracle_lib as O
-    cases = [((3,), (3, 4), None), ((2, 3, 4), (5, 6, 4, 7), None), ((3, 4), (5, 6), None), ((2, 3, 4), (1, 4, 5), None),
+    cases = [((3,), (3, 4), None), ((2, 3, 4), (5, 6, 4, 7), None), ((3, 4), (5, 6), None), ((2, 3, 4), (3, 4, 5), None),
              ((3, 4), (4, 5), (4,)), ((6, 3, 4), (4, 5), None), ((3, 4), (6, 4, 5), (5,)), ((2, 3, 5, 7), (2, 3, 7, 4), None)]
     for sa, sb, sbias in cases:
         st, want = O.matmul_plan(sa, sb, sbias)
@@ -53,3 +53,16 @@ def test_matmul_plan_rules(pkg):
             got = pkg.matmul_plan(sa, sb, sbias)
             assert (got["m"], got["n"], got["k"], got["batch"], got["shape"]) == (want["m"], want["n"], want["k"], want["batch"], want["shape"])
             assert (got["stride_a"], got["stride_b"], got["stride_c"]) == (want["strideA"], want["strideB"], want["strideC"])
+    # beyond the reference (which raises "shape invalid" for unequal leading dimensions): extent 1 is broadcast
+    assert O.matmul_plan((16, 12, 128, 64), (1, 12, 64, 64))[0] == 2
+    got = pkg.matmul_plan((16, 12, 128, 64), (1, 12, 64, 64))
+    assert got["shape"] == (16, 12, 128, 64) and got["batch"] == 192
+    assert got["grid"] == dict(outer=16, inner=12, strides=(12 * 128 * 64, 0, 12 * 128 * 64), inner_strides=(128 * 64, 64 * 64, 128 * 64))
+    got = pkg.matmul_plan((2, 3, 1, 7, 8), (2, 3, 4, 8, 6))  # adjacent dimensions with compatible strides merge
+    assert got["shape"] == (2, 3, 4, 7, 6)
+    assert got["grid"] == dict(outer=6, inner=4, strides=(56, 4 * 48, 4 * 42), inner_strides=(0, 48, 42))
+    assert pkg.matmul_plan((5, 1, 3, 4), (1, 1, 4, 2))["grid"] == dict(outer=5, inner=1, strides=(12, 0, 6), inner_strides=(0, 0, 0))
+    with pytest.raises(NotImplementedError):
+        pkg.matmul_plan((4, 1, 5, 7, 8), (1, 3, 5, 8, 6))
+    with pytest.raises(pkg.InvalidArgumentError):
+        pkg.matmul_plan((2, 3, 4), (3, 4, 5))

@@ -304,6 +304,30 @@ def test_sgemm_config_c1(pkg, T):
     assert rel_fro(T.n(pkg.blas_matmul(T.t(a), T.t(b))), want2) <= FP32_TOL
 
 
+@pytest.mark.parametrize("shape_a,shape_b", [
+    ((16, 12, 128, 64), (1, 12, 64, 64)),   # one weight per head, shared by the batch
+    ((1, 12, 128, 64), (16, 12, 64, 64)), ((2, 3, 1, 7, 8), (2, 3, 4, 8, 6)), ((5, 1, 3, 4), (1, 1, 4, 2)),
+    ((3, 1, 33, 20), (1, 4, 20, 17)),
+])
+def test_matmul_broadcast_of_leading_dimensions(pkg, T, shape_a, shape_b):
+    """Leading dimensions of extent 1 stand for every index of the other operand's (the reference raises for
+    unequal leading dimensions, tfcc/core/operations/tfcc_blas.cpp:36-42).  Checked against the oracle's
+    two-dimensional product, one batch entry at a time."""
+    rng = np.random.default_rng(sum(shape_a) * 3 + sum(shape_b))
+    a = rng.normal(0, 1, shape_a).astype(np.float32)
+    b = rng.normal(0, 1, shape_b).astype(np.float32)
+    bias = rng.uniform(-1, 1, shape_b[-1]).astype(np.float32)
+    lead = tuple(max(x, y) for x, y in zip(shape_a[:-2], shape_b[:-2]))
+    ab = np.broadcast_to(a, lead + shape_a[-2:]).reshape((-1,) + shape_a[-2:])
+    bb = np.broadcast_to(b, lead + shape_b[-2:]).reshape((-1,) + shape_b[-2:])
+    want = np.stack([O.sgemm(np.ascontiguousarray(x), np.ascontiguousarray(y), bias, want64=True)[1] for x, y in zip(ab, bb)])
+    want = want.reshape(lead + (shape_a[-2], shape_b[-1]))
+    got = T.n(pkg.blas_matmul(T.t(a), T.t(b), T.t(bias)))
+    assert got.shape == want.shape and rel_fro(got, want) <= FP32_TOL
+    got = T.n(pkg.blas_matmul(T.t(a), T.t(b)))
+    assert rel_fro(got, want - bias) <= FP32_TOL
+
+
 def test_sgemm_exact_cases(pkg, T):
     rng = np.random.default_rng(20)
     a = rng.uniform(-1, 1, (137, 253)).astype(np.float32)
@@ -396,7 +420,7 @@ def test_matmul_validation_and_empty(pkg, T):
     z = lambda *s: T.t(np.zeros(s, np.float32))
     with pytest.raises(pkg.InvalidArgumentError, match="two or more dimensions"):
         pkg.blas_matmul(z(3), z(3, 4))
-    for sa, sb in (((2, 3, 4), (5, 6, 4, 7)), ((3, 4), (5, 6)), ((2, 3, 4), (1, 4, 5))):
+    for sa, sb in (((2, 3, 4), (5, 6, 4, 7)), ((3, 4), (5, 6)), ((2, 3, 4), (3, 4, 5))):
         with pytest.raises(pkg.InvalidArgumentError, match="shape invalid"):
             pkg.blas_matmul(z(*sa), z(*sb))
     with pytest.raises(pkg.InvalidArgumentError, match="shape invalid"):

@@ -180,10 +180,37 @@ def matmul_plan(shape_a, shape_b, shape_bias=None):
         raise InvalidArgumentError("shape invalid")
     if shape_bias is not None and (len(shape_bias) != 1 or shape_bias[0] != shape_b[-1]):
         raise InvalidArgumentError("shape invalid")
-    if ra == rb and tuple(shape_a[:-2]) != tuple(shape_b[:-2]):
-        raise InvalidArgumentError("shape invalid")
     m, n, k = shape_a[-2], shape_b[-1], shape_a[-1]
     lead = tuple(shape_a[:-2]) if ra > rb else tuple(shape_b[:-2])
+    grid = None
+    if ra == rb and tuple(shape_a[:-2]) != tuple(shape_b[:-2]):
+        # beyond the reference (which raises here): a leading dimension of 1 on one side is broadcast
+        lead = []
+        for ea, eb in zip(shape_a[:-2], shape_b[:-2]):
+            if ea != eb and ea != 1 and eb != 1:
+                raise InvalidArgumentError("shape invalid")
+            lead.append(eb if ea == 1 else ea)
+        lead = tuple(lead)
+        dims, sa, sb, sc = [], [], [], []
+        da, db, dc = m * k, k * n, m * n
+        for ea, eb, e in reversed(list(zip(shape_a[:-2], shape_b[:-2], lead))):
+            if e > 1:
+                dims.insert(0, e); sa.insert(0, 0 if ea == 1 else da); sb.insert(0, 0 if eb == 1 else db); sc.insert(0, dc)
+            da, db, dc = da * ea, db * eb, dc * e
+        i = 0
+        while i + 1 < len(dims):
+            if all(s[i] == s[i + 1] * dims[i + 1] for s in (sa, sb, sc)):
+                dims[i + 1] *= dims[i]
+                for lst in (dims, sa, sb, sc):
+                    del lst[i]
+                i = max(i - 1, 0)
+            else:
+                i += 1
+        if len(dims) > 2:
+            raise NotImplementedError("matmul: broadcast over more than two groups of batch dimensions")
+        while len(dims) < 2:
+            dims.append(1); sa.append(0); sb.append(0); sc.append(0)
+        grid = dict(outer=dims[0], inner=dims[1], strides=(sa[0], sb[0], sc[0]), inner_strides=(sa[1], sb[1], sc[1]))
     batch = 1
     for d in lead:
         batch *= d
@@ -194,7 +221,7 @@ def matmul_plan(shape_a, shape_b, shape_bias=None):
         if rb == 2:
             stride_b = 0
     return dict(m=m, n=n, k=k, batch=batch, shape=lead + (m, n), stride_a=stride_a, stride_b=stride_b,
-                stride_c=m * n)
+                stride_c=m * n, grid=grid)
 
 
 def blas_matmul(a, b, bias=None):
@@ -209,6 +236,10 @@ def blas_matmul(a, b, bias=None):
         return out  # uninitialised, as the reference returns it
     a, b = a.contiguous(), b.contiguous()
     bias = None if bias is None else bias.contiguous()
+    if p["grid"] is not None:
+        g = p["grid"]
+        return sgemm_general(a, b, out, p["m"], p["n"], p["k"], p["k"], p["n"], p["n"], batch_outer=g["outer"],
+                             batch_inner=g["inner"], strides=g["strides"], inner_strides=g["inner_strides"], bias=bias)
     check(lib().tfcc_rocm_sgemm_strided_batched(_stream(), _ptr(a), p["stride_a"], _ptr(b), p["stride_b"],
                                                  _ptr(bias), _ptr(out), p["stride_c"], p["m"], p["n"], p["k"],
                                                  p["batch"]))

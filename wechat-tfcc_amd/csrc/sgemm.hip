@@ -465,7 +465,9 @@ extern "C" int tfcc_rocm_sgemm_general(void* stream, const tfcc_rocm_sgemm_desc*
   TFCC_REQUIRE(d->lda >= k && d->ldc >= n && d->ldb >= (d->trans_b ? k : n), "sgemm: row stride shorter than a row");
   const unsigned long long batch64 = (unsigned long long)d->batch_outer * d->batch_inner;
   TFCC_REQUIRE(batch64 < (1ull << 31), "sgemm: too many batch entries");
-  TFCC_REQUIRE(!d->residual || (d->ldc == n && d->batch_inner == 1), "sgemm: a residual needs a dense result");
+  TFCC_REQUIRE(!d->residual || (d->ldc == n && (d->batch_inner == 1 || (d->inner_stride_c == (uint64_t)m * n &&
+                                                                          d->stride_c == (uint64_t)d->batch_inner * m * n))),
+               "sgemm: a residual needs a dense result");
   SgemmParams p{};
   p.A = d->a; p.B = d->b; p.bias = d->bias; p.C = d->c; p.residual = d->residual; p.strideR = d->stride_residual;
   p.act = d->activation;

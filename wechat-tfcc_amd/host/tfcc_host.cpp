@@ -321,11 +321,55 @@ Variable<float> rocm_sgemm(const Tensor<float>& a, const Tensor<float>& b, const
     if (ra == 2) strideA = 0;
     if (rb == 2) strideB = 0;
   }
-  std::vector<unsigned> s = ra > rb ? a.shape().toVector() : b.shape().toVector();
-  s[s.size() - 2] = m;
-  s[s.size() - 1] = n;
-  Variable<float> result{Shape(std::move(s))};
+  std::vector<unsigned> s = tfcc::blas::detail::check<float>(a, b, bias);
+  Variable<float> result{Shape(s)};
   if (residual && !(residual->shape() == result.shape())) throw InvalidArgumentError("residual and result don't match");
+  bool broadcast = false;
+  if (ra == rb)
+    for (size_t i = 0; i + 2 < ra; ++i) broadcast = broadcast || a.shape(i) != b.shape(i);
+  if (broadcast) {
+    // leading dimensions of extent 1 on one side: per-dimension strides (0 where broadcast), adjacent
+    // dimensions merged where the strides allow, at most two left for the kernel's outer x inner batch grid
+    std::vector<unsigned> dims;
+    std::vector<uint64_t> sa, sb, sc;
+    uint64_t da = static_cast<uint64_t>(m) * k, db = static_cast<uint64_t>(k) * n, dc = static_cast<uint64_t>(m) * n;
+    for (size_t i = ra - 2; i-- > 0;) {  // innermost leading dimension first
+      const unsigned ea = a.shape(i), eb = b.shape(i), e = s[i];
+      if (e > 1) {
+        dims.insert(dims.begin(), e);
+        sa.insert(sa.begin(), ea == 1 ? 0 : da);
+        sb.insert(sb.begin(), eb == 1 ? 0 : db);
+        sc.insert(sc.begin(), dc);
+      }
+      da *= ea; db *= eb; dc *= e;
+    }
+    for (size_t i = 0; i + 1 < dims.size();) {
+      if (sa[i] == sa[i + 1] * dims[i + 1] && sb[i] == sb[i + 1] * dims[i + 1] && sc[i] == sc[i + 1] * dims[i + 1]) {
+        dims[i + 1] *= dims[i];
+        dims.erase(dims.begin() + i); sa.erase(sa.begin() + i); sb.erase(sb.begin() + i); sc.erase(sc.begin() + i);
+        if (i > 0) --i;
+      } else {
+        ++i;
+      }
+    }
+    if (dims.size() > 2) throw NotImplementedError("matmul: broadcast over more than two groups of batch dimensions");
+    tfcc_rocm_sgemm_desc d{};
+    d.a = a.data(); d.b = b.data(); d.c = result.data();
+    d.bias = bias ? bias->data() : nullptr;
+    d.residual = residual ? residual->data() : nullptr;
+    d.stride_residual = static_cast<uint64_t>(m) * n;
+    d.m = m; d.n = n; d.k = k; d.lda = k; d.ldb = n; d.ldc = n;
+    d.activation = activation;
+    d.batch_outer = 1; d.batch_inner = 1;
+    if (dims.size() == 2) {
+      d.batch_outer = dims[0]; d.stride_a = sa[0]; d.stride_b = sb[0]; d.stride_c = sc[0];
+      d.batch_inner = dims[1]; d.inner_stride_a = sa[1]; d.inner_stride_b = sb[1]; d.inner_stride_c = sc[1];
+    } else if (dims.size() == 1) {
+      d.batch_outer = dims[0]; d.stride_a = sa[0]; d.stride_b = sb[0]; d.stride_c = sc[0];
+    }
+    check(tfcc_rocm_sgemm_general(current_stream(), &d));
+    return result;
+  }
   unsigned rows = m, batch = result.size() / (m * n);
   if (rb == 2 && ra > 2) {
     // one matrix b for the whole batch of a: the batch is just more rows of one product

@@ -193,11 +193,15 @@ std::vector<unsigned> check(const Tensor<T>& a, const Tensor<T>& b, const Tensor
   if (ra != rb && ra != 2 && rb != 2) throw InvalidArgumentError("shape invalid");
   if (a.shape(ra - 1) != b.shape(rb - 2)) throw InvalidArgumentError("shape invalid");
   if (bias && (bias->shape().size() != 1 || bias->size() != b.shape(rb - 1))) throw InvalidArgumentError("shape invalid");
-  if (ra == rb) {
-    for (size_t i = 0; i + 2 < ra; ++i)
-      if (a.shape(i) != b.shape(i)) throw InvalidArgumentError("shape invalid");
-  }
   std::vector<unsigned> s = ra > rb ? a.shape().toVector() : b.shape().toVector();
+  if (ra == rb) {
+    // The reference wants equal leading dimensions (tfcc/core/operations/tfcc_blas.cpp:36-42).  Accepted on
+    // top of that: a leading dimension of 1 on one side stands for every index of the other side's.
+    for (size_t i = 0; i + 2 < ra; ++i) {
+      if (a.shape(i) != b.shape(i) && a.shape(i) != 1 && b.shape(i) != 1) throw InvalidArgumentError("shape invalid");
+      s[i] = a.shape(i) == 1 ? b.shape(i) : a.shape(i);
+    }
+  }
   s[s.size() - 2] = a.shape(ra - 2);
   s[s.size() - 1] = b.shape(rb - 1);
   return s;
