@@ -218,6 +218,37 @@ def bench_other(torch, pkg, dev, steps, warmup, c3):
 
     broadcast_case("c2_fp32_broadcast_16x12x128x64_by_1x12x64x64", (16, 12, 128, 64), (1, 12, 64, 64))
 
+    # C2, first product with K used as stored: scores = Q K^T from K [16, 12, 128, 64] (B given transposed)
+    def qkt_case(name, B, H, S, D, sets=4):
+        bufs = []
+        for _ in range(sets):
+            q = torch.randn((B, H, S, D), device=dev, dtype=torch.float32)
+            k = torch.randn((B, H, S, D), device=dev, dtype=torch.float32)
+            c = torch.empty((B, H, S, S), device=dev, dtype=torch.float32)
+            d = pkg.SgemmDesc()
+            d.a, d.b, d.c = q.data_ptr(), k.data_ptr(), c.data_ptr()
+            d.m, d.n, d.k, d.lda, d.ldb, d.ldc = S, S, D, D, D, S
+            d.trans_b = 1
+            d.batch_outer, d.batch_inner = B * H, 1
+            d.stride_a, d.stride_b, d.stride_c = S * D, S * D, S * S
+            bufs.append((d, (q, k, c)))
+        idx = [0]
+
+        def step():
+            d = bufs[idx[0] % sets][0]
+            idx[0] += 1
+            st = lib.tfcc_rocm_sgemm_general(stream, C.byref(d))
+            if st != 0:
+                pkg.check(st)
+        ms = time_launches(torch, step, steps, warmup, pkg, stream)
+        flop = 2.0 * B * H * S * S * D
+        nbytes = 4.0 * (2 * B * H * S * D + B * H * S * S)
+        out[name] = {"ms": round(ms, 5), "tflops": round(flop / ms / 1e9, 3),
+                     "frac_fp32_mfma": round(flop / ms / 1e9 / PEAK_FP32_TFLOPS, 4), "gbs": round(nbytes / ms / 1e6, 1),
+                     "frac_hbm": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4)}
+
+    qkt_case("c2_fp32_qkt_k_as_stored_16x12x128x64", 16, 12, 128, 64)
+
     # C2 as one launch: softmax(q k^T / 8) v on [batch, seq, heads, size] tensors, 16 x 12 heads of 128 x 64
     def attention_case(name, B, H, S, D, sets=4):
         bufs = []
