@@ -289,6 +289,16 @@ int tfcc_rocm_attention_f32(void* stream, const tfcc_rocm_attention_desc* desc);
 /* _mkl_layer_normalize, tfcc/mkl/interfaces/tfcc_mklnormalizationinterface.cpp:29-62 */
 int tfcc_rocm_layer_norm_f32(void* stream, const float* in, const float* gamma, const float* beta,
                              float epsilon, uint64_t rows, unsigned cols, float* out);
+/* Element-wise functions of one tensor with the expressions of the reference's float kernels
+ * (tfcc/mkl/kernel/tfcc_mklactivationkernel.hpp:48-110,222-228,284-291): sigmoid 1/(1+exp(0-x)), tanh, relu,
+ * softplus log(exp(x)+1), log, rsqrt 1/sqrt(x), erf, abs, sign; and neg 0-x, reciprocal 1/x, sqrt 1/rsqrt(x) as
+ * tfcc_runtime/operations/math/neg.cpp:30, reciprocal.cpp:31, sqrt.cpp:31 compose them. */
+enum {
+  TFCC_ROCM_UNARY_SIGMOID = 0, TFCC_ROCM_UNARY_TANH = 1, TFCC_ROCM_UNARY_RELU = 2, TFCC_ROCM_UNARY_SOFTPLUS = 3,
+  TFCC_ROCM_UNARY_LOG = 4, TFCC_ROCM_UNARY_RSQRT = 5, TFCC_ROCM_UNARY_ERF = 6, TFCC_ROCM_UNARY_ABS = 7,
+  TFCC_ROCM_UNARY_SIGN = 8, TFCC_ROCM_UNARY_NEG = 9, TFCC_ROCM_UNARY_RECIPROCAL = 10, TFCC_ROCM_UNARY_SQRT = 11
+};
+int tfcc_rocm_unary_f32(void* stream, int op, const float* in, uint64_t total, float* out);
 /* _MKLActivationKernel::geluAccurate, tfcc/mkl/kernel/tfcc_mklactivationkernel.hpp:213-220 */
 int tfcc_rocm_gelu_accurate_f32(void* stream, const float* in, uint64_t total, float* out);
 /* out = a * alpha + beta: TransformationInterface::transform, tfcc/core/operations/tfcc_operator.cpp:78-95 */

@@ -431,6 +431,27 @@ def test_matmul_validation_and_empty(pkg, T):
 
 # ---- element-wise neighbours --------------------------------------------------------------------------
 
+def test_unary_functions_against_numpy_float64(pkg, T):
+    """tfcc_rocm_unary_f32 against the expressions of tfcc/mkl/kernel/tfcc_mklactivationkernel.hpp:48-110,222-228,
+    284-291 evaluated in float64; sizes on both sides of the grid-stride loop's first pass."""
+    import math
+    rng = np.random.default_rng(12)
+    ref = {"sigmoid": lambda x: 1 / (1 + np.exp(-x)), "tanh": np.tanh, "relu": lambda x: np.maximum(x, 0),
+           "softplus": lambda x: np.log(np.exp(x) + 1), "log": np.log, "rsqrt": lambda x: 1 / np.sqrt(x),
+           "erf": np.vectorize(math.erf), "abs": np.abs, "sign": np.sign, "neg": lambda x: -x,
+           "reciprocal": lambda x: 1 / x, "sqrt": np.sqrt}
+    assert set(ref) == set(pkg.UNARY)
+    for total in (1, 255, 70001):
+        x = rng.normal(0, 3, total).astype(np.float32)
+        pos = rng.uniform(1e-4, 100, total).astype(np.float32)
+        for name, f in ref.items():
+            src = pos if name in ("log", "rsqrt", "sqrt") else x
+            got = T.n(pkg.unary(name, T.t(src)))
+            assert np.allclose(got, f(src.astype(np.float64)), rtol=2e-6, atol=1e-7), (name, total)
+    with pytest.raises(pkg.TfccRocmError):
+        pkg.check(pkg.lib().tfcc_rocm_unary_f32(None, 99, 16, 1, 16))
+
+
 def test_elementwise_against_oracle(pkg, T):
     rng = np.random.default_rng(50)
     for shape in ((8, 12, 128, 128), (7, 33), (5, 1000)):

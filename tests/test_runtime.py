@@ -7,6 +7,8 @@ import os
 import re
 import zipfile
 
+import math
+
 import numpy as np
 import pytest
 
@@ -314,6 +316,61 @@ def test_fused_graph_is_bit_identical_to_the_graph_as_written(mf, rt, dev):
         want = want.transpose(perm_c) if perm_c else want
         assert outs[0].shape == want.shape and np.array_equal(outs[0], outs[1])
         assert rel_frobenius(outs[1], want) <= 1e-5
+
+
+UNARY_NUMPY = {
+    # expressions of tfcc/mkl/kernel/tfcc_mklactivationkernel.hpp:48-110,222-228,284-291 and of
+    # tfcc_runtime/operations/math/neg.cpp:30, reciprocal.cpp:31, sqrt.cpp:31, evaluated in float64
+    "Sigmoid": lambda x: 1 / (1 + np.exp(-x)), "Tanh": np.tanh, "Relu": lambda x: np.maximum(x, 0),
+    "Softplus": lambda x: np.log(np.exp(x) + 1), "Log": np.log, "Rsqrt": lambda x: 1 / np.sqrt(x),
+    "Erf": np.vectorize(math.erf), "Abs": np.abs, "Sign": np.sign, "Neg": lambda x: -x,
+    "Reciprocal": lambda x: 1 / x, "Sqrt": np.sqrt,
+}
+
+
+def test_value_forms_of_unary_nodes_on_host(mf, rt):
+    g = mf.GraphBuilder("g")
+    a = g.value_input("a", mf.FLOAT)
+    for op in ("Neg", "Reciprocal", "Rsqrt", "Sqrt"):
+        out = g._symbol("r_" + op, mf.FLOAT, mf.VALUE)
+        g.node("math." + op, [a], [out])
+        g.output(out)
+    res = rt.Model(mf.write_model([g], "g"), host=True).run({"a": np.array([6.25], np.float32)})
+    want = [np.float32(-6.25), np.float32(1) / np.float32(6.25), np.float32(1) / np.float32(2.5), np.float32(2.5)]
+    assert [res["r_" + op][0] for op in ("Neg", "Reciprocal", "Rsqrt", "Sqrt")] == want
+    # a function without a value form is not taken: the node is unknown to the runtime
+    g = mf.GraphBuilder("g")
+    a = g.value_input("a", mf.FLOAT)
+    out = g._symbol("r", mf.FLOAT, mf.VALUE)
+    g.node("math.Tanh", [a], [out])
+    g.output(out)
+    with pytest.raises(rt.RuntimeError_):
+        rt.Model(mf.write_model([g], "g"), host=True).run({"a": np.array([1.0], np.float32)})
+
+
+@pytest.mark.gpu
+def test_unary_nodes_against_numpy_float64(mf, rt, dev):
+    rng = np.random.default_rng(11)
+    g = mf.GraphBuilder("g")
+    x = g.input("x", mf.FLOAT, [3, 5, 7])
+    pos = g.input("pos", mf.FLOAT, [3, 5, 7])
+    outs = {}
+    for op in UNARY_NUMPY:
+        outs[op] = g.unary("math." + op, pos if op in ("Log", "Rsqrt", "Sqrt") else x)
+        g.output(outs[op])
+    xv = rng.normal(0, 2, (3, 5, 7)).astype(np.float32)
+    xv[0, 0, :2] = (0.0, -0.0)
+    pv = rng.uniform(1e-3, 50, (3, 5, 7)).astype(np.float32)
+    res = rt.Model(mf.write_model([g], "g")).run({"x": xv, "pos": pv})
+    for op, f in UNARY_NUMPY.items():
+        src = pv if op in ("Log", "Rsqrt", "Sqrt") else xv
+        with np.errstate(divide="ignore"):
+            want = f(src.astype(np.float64))  # 1 / (+-0) = +-inf on both sides
+        assert res[outs[op]].shape == want.shape
+        assert np.allclose(res[outs[op]], want, rtol=2e-6, atol=1e-7), op
+    # exact where the function is exact in float
+    assert np.array_equal(res[outs["Relu"]], np.maximum(xv, 0)) and np.array_equal(res[outs["Abs"]], np.abs(xv))
+    assert np.array_equal(res[outs["Neg"]], 0 - xv) and np.array_equal(res[outs["Sign"]], np.sign(xv))
 
 
 @pytest.mark.gpu

@@ -116,6 +116,7 @@ SYMBOLS = {
     "tfcc_rocm_sgemm_fused": (_I, [_VP, _VP, _U64, _VP, _U64, _VP, _VP, _U64, _VP, _U64, _U, _U, _U, _U, _I]),
     "tfcc_rocm_sgemm_general": (_I, [_VP, _VP]),
     "tfcc_rocm_sgemm_grouped": (_I, [_VP, _VP, C.POINTER(_VP), C.POINTER(_VP), C.POINTER(_VP), _U, _U, _U, _U]),
+    "tfcc_rocm_unary_f32": (_I, [_VP, _I, _VP, _U64, _VP]),
     "tfcc_rocm_probe_mfma": (_I, [_VP, _I, _I, _U, _U, _VP]),
     "tfcc_rocm_probe_read": (_I, [_VP, _VP, _U64, _U, _VP]),
     "tfcc_rocm_probe_launch": (_I, [_VP, _VP]),
@@ -502,6 +503,19 @@ def layer_norm(a, gamma, beta, eps):
     out = torch.empty_like(a)
     check(lib().tfcc_rocm_layer_norm_f32(_stream(), _ptr(a), _ptr(gamma.contiguous()), _ptr(beta.contiguous()),
                                           eps, a.numel() // a.shape[-1], a.shape[-1], _ptr(out)))
+    return out
+
+
+UNARY = {"sigmoid": 0, "tanh": 1, "relu": 2, "softplus": 3, "log": 4, "rsqrt": 5, "erf": 6, "abs": 7, "sign": 8,
+         "neg": 9, "reciprocal": 10, "sqrt": 11}
+
+
+def unary(name, a):
+    """tfcc_rocm_unary_f32: one of UNARY applied element-wise."""
+    import torch
+    a = a.contiguous()
+    out = torch.empty_like(a)
+    check(lib().tfcc_rocm_unary_f32(_stream(), UNARY[name], _ptr(a), a.numel(), _ptr(out)))
     return out
 
 

@@ -222,6 +222,31 @@ unsigned grid_for(size_t total) {
   return (unsigned)blocks;
 }
 
+// Element-wise functions of one tensor, each with the expression of the reference's float kernel
+// (tfcc/mkl/kernel/tfcc_mklactivationkernel.hpp:48-110,222-228,284-291; neg, reciprocal and sqrt as
+// tfcc_runtime/operations/math/neg.cpp:30, reciprocal.cpp:31 and sqrt.cpp:31 compose them).
+template <int OP>
+__device__ __forceinline__ float unary_value(float v) {
+  if (OP == TFCC_ROCM_UNARY_SIGMOID) return 1.f / (1.f + expf(0.f - v));
+  if (OP == TFCC_ROCM_UNARY_TANH) return tanhf(v);
+  if (OP == TFCC_ROCM_UNARY_RELU) return fmaxf(v, 0.f);
+  if (OP == TFCC_ROCM_UNARY_SOFTPLUS) return logf(expf(v) + 1.f);
+  if (OP == TFCC_ROCM_UNARY_LOG) return logf(v);
+  if (OP == TFCC_ROCM_UNARY_RSQRT) return 1.f / sqrtf(v);
+  if (OP == TFCC_ROCM_UNARY_ERF) return erff(v);
+  if (OP == TFCC_ROCM_UNARY_ABS) return fabsf(v);
+  if (OP == TFCC_ROCM_UNARY_SIGN) return v < 0.f ? -1.f : (v > 0.f ? 1.f : 0.f);
+  if (OP == TFCC_ROCM_UNARY_NEG) return 0.f - v;
+  if (OP == TFCC_ROCM_UNARY_RECIPROCAL) return 1.f / v;
+  return 1.f / (1.f / sqrtf(v));  // TFCC_ROCM_UNARY_SQRT: 1 / rsqrt(v), rounded twice like the composition
+}
+
+template <int OP>
+__global__ __launch_bounds__(256) void unary_kernel(const float* in, size_t total, float* out) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += stride) out[i] = unary_value<OP>(in[i]);
+}
+
 }  // namespace
 }  // namespace tfcc_rocm
 
@@ -346,6 +371,32 @@ int tfcc_rocm_transpose_f32(void* stream, const float* in, const unsigned* shape
   }
   hipLaunchKernelGGL(transpose_kernel, dim3(grid_for(total)), dim3(256), 0, as_stream(stream), in, total, p, out);
   return check_launch("transpose");
+}
+
+int tfcc_rocm_unary_f32(void* stream, int op, const float* in, uint64_t total, float* out) {
+  TFCC_REQUIRE(in && out, "unary: null argument");
+  TFCC_REQUIRE(total > 0, "unary: empty tensor");
+  hipStream_t s = as_stream(stream);
+  const unsigned grid = grid_for(total);
+#define TFCC_UNARY_CASE(OP) \
+  case OP: hipLaunchKernelGGL(unary_kernel<OP>, dim3(grid), dim3(256), 0, s, in, (size_t)total, out); break;
+  switch (op) {
+    TFCC_UNARY_CASE(TFCC_ROCM_UNARY_SIGMOID)
+    TFCC_UNARY_CASE(TFCC_ROCM_UNARY_TANH)
+    TFCC_UNARY_CASE(TFCC_ROCM_UNARY_RELU)
+    TFCC_UNARY_CASE(TFCC_ROCM_UNARY_SOFTPLUS)
+    TFCC_UNARY_CASE(TFCC_ROCM_UNARY_LOG)
+    TFCC_UNARY_CASE(TFCC_ROCM_UNARY_RSQRT)
+    TFCC_UNARY_CASE(TFCC_ROCM_UNARY_ERF)
+    TFCC_UNARY_CASE(TFCC_ROCM_UNARY_ABS)
+    TFCC_UNARY_CASE(TFCC_ROCM_UNARY_SIGN)
+    TFCC_UNARY_CASE(TFCC_ROCM_UNARY_NEG)
+    TFCC_UNARY_CASE(TFCC_ROCM_UNARY_RECIPROCAL)
+    TFCC_UNARY_CASE(TFCC_ROCM_UNARY_SQRT)
+    default: return set_error(TFCC_ROCM_INVALID_ARGUMENT, "unary: unknown function %d", op);
+  }
+#undef TFCC_UNARY_CASE
+  return check_launch("unary");
 }
 
 }  // extern "C"

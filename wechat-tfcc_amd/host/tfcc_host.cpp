@@ -466,6 +466,11 @@ class ROCMActivationInterface : public ActivationInterface<float> {
     check(tfcc_rocm_gelu_accurate_f32(current_stream(), a.data(), a.size(), r.data()));
     return r;
   }
+  Variable<float> unary(const Tensor<float>& a, int function) override {
+    Variable<float> r(a.shape());
+    check(tfcc_rocm_unary_f32(current_stream(), function, a.data(), a.size(), r.data()));
+    return r;
+  }
 };
 
 class ROCMNormalizationInterface : public NormalizationInterface<float> {

@@ -81,7 +81,12 @@ class ActivationInterface {
   virtual ~ActivationInterface() {}
   virtual Variable<T> softmax(const Tensor<T>&, size_t) { throw NotImplementedError(); }
   virtual Variable<T> geluAccurate(const Tensor<T>&) { throw NotImplementedError(); }
+  // one of the UnaryFunction values below applied to every element
+  virtual Variable<T> unary(const Tensor<T>&, int) { throw NotImplementedError(); }
 };
+
+// element-wise functions of one tensor (the numbering of the kernel library's TFCC_ROCM_UNARY_* values)
+enum class UnaryFunction { SIGMOID = 0, TANH, RELU, SOFTPLUS, LOG, RSQRT, ERF, ABS, SIGN, NEG, RECIPROCAL, SQRT };
 
 template <class T>
 class NormalizationInterface {
@@ -297,6 +302,26 @@ Variable<T> gelu_accurate(const Tensor<T>& a) {
   if (a.size() == 0) throw InvalidArgumentError("invalid tensor");
   return Operation<T>::getCurrentInterface().getActivationInterface().geluAccurate(a);
 }
+// tfcc::math::sigmoid, tanh, relu, softplus, log, rsqrt, erf, abs, sign (tfcc/core/operations/tfcc_math.h); neg,
+// reciprocal and sqrt stand for 0 - a, 1 / a and 1 / rsqrt(a) as the reference's runtime writes them
+template <class T>
+Variable<T> unary(const Tensor<T>& a, UnaryFunction f) {
+  if (a.size() == 0) throw InvalidArgumentError("invalid tensor");
+  return Operation<T>::getCurrentInterface().getActivationInterface().unary(a, static_cast<int>(f));
+}
+#define TFCC_UNARY_FUNCTION(NAME, VALUE) \
+  template <class T>                     \
+  Variable<T> NAME(const Tensor<T>& a) { return unary(a, UnaryFunction::VALUE); }
+TFCC_UNARY_FUNCTION(sigmoid, SIGMOID)
+TFCC_UNARY_FUNCTION(tanh, TANH)
+TFCC_UNARY_FUNCTION(relu, RELU)
+TFCC_UNARY_FUNCTION(softplus, SOFTPLUS)
+TFCC_UNARY_FUNCTION(log, LOG)
+TFCC_UNARY_FUNCTION(rsqrt, RSQRT)
+TFCC_UNARY_FUNCTION(erf, ERF)
+TFCC_UNARY_FUNCTION(abs, ABS)
+TFCC_UNARY_FUNCTION(sign, SIGN)
+#undef TFCC_UNARY_FUNCTION
 // a + b with b's shape equal to the trailing dimensions of a's (or the same shape)
 template <class T>
 Variable<T> add(const Tensor<T>& a, const Tensor<T>& b) {

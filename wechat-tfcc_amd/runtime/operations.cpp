@@ -6,10 +6,13 @@
 //   math.Matmul, math.MatmulWithBias    operations/math/matmul.cpp:52-81, matmulwithbias.cpp:52-88
 //   math.Add / Sub / Mul / Div          operations/math/add.cpp:80-126 (tensor and value operand forms)
 //   math.Gelu, math.Softmax             operations/math/gelu.cpp, softmax.cpp
+//   math.Abs / Erf / Log / Neg / Reciprocal / Relu / Rsqrt / Sigmoid / Sign / Softplus / Sqrt / Tanh
+//                                       operations/math/<name>.cpp
 //   nn.LayerNormalization               operations/nn/layernormalization.cpp:52-88
 //   base.Transpose, base.Reshape, base.Identity, base.CreateVector
 //                                       operations/base/transpose.cpp, reshape.cpp:27-59,74-104,
 //                                       identity.cpp, createvector.cpp:63-121
+#include <cmath>
 #include <map>
 
 #include "runtime.h"
@@ -127,6 +130,60 @@ class Arithmetic : public TypedOperation<T> {
       return false;
     }
     return true;
+  }
+};
+
+// ---- element-wise functions of one symbol ---------------------------------------------------------------
+// tensor -> tensor and value -> value forms, as tfcc_runtime/operations/math/{abs,erf,log,neg,reciprocal,relu,
+// rsqrt,sigmoid,sign,softplus,sqrt,tanh}.cpp register them (the value forms exist there for neg, reciprocal,
+// rsqrt and sqrt: neg.cpp:41, reciprocal.cpp:42, rsqrt.cpp:41, sqrt.cpp:41)
+template <UnaryFunction F, class T>
+class Unary : public TypedOperation<T> {
+  static const char* message() {
+    switch (F) {
+      case UnaryFunction::SIGMOID: return "math.Sigmoid";
+      case UnaryFunction::TANH: return "math.Tanh";
+      case UnaryFunction::RELU: return "math.Relu";
+      case UnaryFunction::SOFTPLUS: return "math.Softplus";
+      case UnaryFunction::LOG: return "math.Log";
+      case UnaryFunction::RSQRT: return "math.Rsqrt";
+      case UnaryFunction::ERF: return "math.Erf";
+      case UnaryFunction::ABS: return "math.Abs";
+      case UnaryFunction::SIGN: return "math.Sign";
+      case UnaryFunction::NEG: return "math.Neg";
+      case UnaryFunction::RECIPROCAL: return "math.Reciprocal";
+      default: return "math.Sqrt";
+    }
+  }
+  static constexpr bool kValueForm = F == UnaryFunction::NEG || F == UnaryFunction::RECIPROCAL ||
+                                     F == UnaryFunction::RSQRT || F == UnaryFunction::SQRT;
+  static T value(T a) {
+    if (F == UnaryFunction::NEG) return static_cast<T>(0) - a;
+    if (F == UnaryFunction::RECIPROCAL) return static_cast<T>(1) / a;
+    if (F == UnaryFunction::RSQRT) return static_cast<T>(1) / static_cast<T>(std::sqrt(a));
+    return static_cast<T>(std::sqrt(a));
+  }
+
+ public:
+  Unary() : TypedOperation<T>(message()) {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 1 || node.outputs.size() != 1) return false;
+    if (!same_dtype(graph, node.outputs, this->DTYPE) || !same_dtype(graph, node.inputs, this->DTYPE)) return false;
+    auto& sm = graph.getSymbolManager();
+    const SymbolType si = stype_of(graph, node.inputs[0]), so = stype_of(graph, node.outputs[0]);
+    if (is_tensor(si) && is_tensor(so)) {
+      const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+      Variable<T>* out = sm.getVariable(node.outputs[0], T());
+      graph.addStep([a, out] { *out = math::unary(*a, F); });
+      return true;
+    }
+    if (kValueForm && is_value(si) && is_value(so)) {
+      const T* a = sm.getValue(node.inputs[0], T());
+      T* out = sm.getValue(node.outputs[0], T());
+      graph.addStep([a, out] { *out = value(*a); });
+      return true;
+    }
+    return false;
   }
 };
 
@@ -386,6 +443,18 @@ class Collector {
     add(new Arithmetic<Arith::MUL, T>());
     add(new Arithmetic<Arith::DIV, T>());
     add(new Gelu<T>());
+    add(new Unary<UnaryFunction::SIGMOID, T>());
+    add(new Unary<UnaryFunction::TANH, T>());
+    add(new Unary<UnaryFunction::RELU, T>());
+    add(new Unary<UnaryFunction::SOFTPLUS, T>());
+    add(new Unary<UnaryFunction::LOG, T>());
+    add(new Unary<UnaryFunction::RSQRT, T>());
+    add(new Unary<UnaryFunction::ERF, T>());
+    add(new Unary<UnaryFunction::ABS, T>());
+    add(new Unary<UnaryFunction::SIGN, T>());
+    add(new Unary<UnaryFunction::NEG, T>());
+    add(new Unary<UnaryFunction::RECIPROCAL, T>());
+    add(new Unary<UnaryFunction::SQRT, T>());
     add(new Softmax<T>());
     add(new LayerNormalization<T>());
     add(new Transpose<T>());
