@@ -150,11 +150,14 @@ __global__ __launch_bounds__(WGM * WGN * 64, 2) void qgemm_dma_kernel(const QGem
     for (int j = 0; j < NI; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
-  int colsum[NI][4];  // four independent partial sums per block: a single chain would stall on the dot latency
+  // Column sums: wavefront row wm owns the blocks j = wm + WGM * t.  Four independent partial sums per block:
+  // a single chain would stall on the dot latency.
+  constexpr int NT = NI / WGM;
+  int colsum[NT][4];
 #pragma unroll
-  for (int j = 0; j < NI; ++j)
+  for (int t = 0; t < NT; ++t)
 #pragma unroll
-    for (int q = 0; q < 4; ++q) colsum[j][q] = 0;
+    for (int q = 0; q < 4; ++q) colsum[t][q] = 0;
 
   // ---- operand addresses inside a stage
   const int l32 = lane & 31, g = lane >> 5;
@@ -209,12 +212,12 @@ __global__ __launch_bounds__(WGM * WGN * 64, 2) void qgemm_dma_kernel(const QGem
     const unsigned char* as = smem + stage * STAGE_BYTES;
     const unsigned char* bs = as + A_BYTES;
 #pragma unroll
-    for (int j = 0; j < NI; ++j) {
-      if (j % WGM == wm) {
-        asm volatile("" ::: "memory");  // keep this a wave-uniform branch, not a select over both blocks
+    for (int t = 0; t < NT; ++t) {
+      v4i own = ub[WGM * t];  // the block of this wavefront row: selects on a wave-uniform condition, no branches
 #pragma unroll
-        for (int q = 0; q < 4; ++q) colsum[j][q] = __builtin_amdgcn_sdot4(ub[j][q], 0x01010101, colsum[j][q], false);
-      }
+      for (int w = 1; w < WGM; ++w) own = wm == w ? ub[WGM * t + w] : own;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) colsum[t][q] = __builtin_amdgcn_sdot4(own[q], 0x01010101, colsum[t][q], false);
     }
     v4i ax = {0, 0, 0, 0};
 #pragma unroll
@@ -273,12 +276,11 @@ __global__ __launch_bounds__(WGM * WGN * 64, 2) void qgemm_dma_kernel(const QGem
   // lanes l and l+32 hold the two k halves of the same column; the transposing read hands lane
   // (colHalf, s16) column 16*colHalf + s16 of the 32-column block
 #pragma unroll
-  for (int j = 0; j < NI; ++j) {
-    if (j % WGM == wm) {
-      int s = colsum[j][0] + colsum[j][1] + colsum[j][2] + colsum[j][3];
-      s += __shfl_xor(s, 32, 64);
-      if (g == 0) colTerm[wn * WN + 32 * j + 16 * colHalf + s16] = s;
-    }
+  for (int t = 0; t < NT; ++t) {
+    const int j = wm + WGM * t;
+    int s = colsum[t][0] + colsum[t][1] + colsum[t][2] + colsum[t][3];
+    s += __shfl_xor(s, 32, 64);
+    if (g == 0) colTerm[wn * WN + 32 * j + 16 * colHalf + s16] = s;
   }
   __syncthreads();
   const unsigned global = (unsigned)offA * (unsigned)offB * K;
