@@ -333,6 +333,21 @@ __global__ __launch_bounds__(WGM * WGN * 64, 2) void qgemm_dma_kernel(const QGem
           }
         }
       }
+      if constexpr (FLAVOUR != 0) {
+        // The rows of block row i (32 per wavefront row) are staged: write them out now, so that the stores are
+        // in flight while the next block row is requantized.  16 lanes write one 256-byte row segment.
+        __syncthreads();
+        constexpr int CHUNKS = BN / 16, PHASE_ROWS = WGM * 32;
+        for (int idx = tid; idx < PHASE_ROWS * CHUNKS; idx += kThreads) {
+          const int pr = idx / CHUNKS, ch = idx % CHUNKS;
+          const int row = (pr >> 5) * WM + 32 * i + (pr & 31);
+          const unsigned grow = m0 + row, gcol = n0 + ch * 16;
+          if (grow >= M || gcol >= N) continue;
+          const unsigned* src = reinterpret_cast<const unsigned*>(stageQ + row * QPITCH + ch * 16);
+          v4i v = {(int)src[0], (int)src[1], (int)src[2], (int)src[3]};
+          *reinterpret_cast<v4i*>(Q + (size_t)grow * N + gcol) = v;
+        }
+      }
     }
   };
   if constexpr (!REQUANT) {
@@ -342,17 +357,6 @@ __global__ __launch_bounds__(WGM * WGN * 64, 2) void qgemm_dma_kernel(const QGem
     else if (rq.fast32OK) storeTile(std::integral_constant<int, 4>{});
     else if (rq.fastOK) storeTile(std::integral_constant<int, 1>{});
     else storeTile(std::integral_constant<int, 2>{});
-    __syncthreads();
-    // staged tile -> HBM: 16 lanes write one 256-byte row segment
-    constexpr int CHUNKS = BN / 16;
-    for (int idx = tid; idx < BM * CHUNKS; idx += kThreads) {
-      const int row = idx / CHUNKS, ch = idx % CHUNKS;
-      const unsigned grow = m0 + row, gcol = n0 + ch * 16;
-      if (grow >= M || gcol >= N) continue;
-      const unsigned* src = reinterpret_cast<const unsigned*>(stageQ + row * QPITCH + ch * 16);
-      v4i v = {(int)src[0], (int)src[1], (int)src[2], (int)src[3]};
-      *reinterpret_cast<v4i*>(Q + (size_t)grow * N + gcol) = v;
-    }
   }
 }
 
