@@ -43,7 +43,8 @@ constexpr int KS = BK / 32;  // 32-deep matrix-op steps per slab
 // 16 consecutive rows of one logical chunk fall into 16 different 16-byte slots of the 256-byte bank stripe
 __device__ __forceinline__ int swzA(int row) { return (row >> 1) & 7; }
 
-template <int BM, int BN, int WGM, int WGN, int STAGES, bool REQUANT>
+// WRITE_C: the int32 result is stored (always without REQUANT; with it only when the caller wants both).
+template <int BM, int BN, int WGM, int WGN, int STAGES, bool REQUANT, bool WRITE_C>
 __global__ __launch_bounds__(WGM * WGN * 64, 2) void qgemm_dma_kernel(const QGemmParams p) {
   constexpr int kThreads = WGM * WGN * 64;
   constexpr int WM = BM / WGM, WN = BN / WGN;
@@ -299,7 +300,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 2) void qgemm_dma_kernel(const QGem
     }
   }
 
-  int* C = p.C ? p.C + (size_t)bi * p.strideC : nullptr;
+  int* C = WRITE_C ? p.C + (size_t)bi * p.strideC : nullptr;
   unsigned char* Q = REQUANT ? p.Q + (size_t)bi * p.strideC : nullptr;
 
   auto storeTile = [&](auto flavour) {
@@ -318,8 +319,10 @@ __global__ __launch_bounds__(WGM * WGN * 64, 2) void qgemm_dma_kernel(const QGem
           int v[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) v[e] = (int)((unsigned)acc[i][j][4 * rq4 + e] + (unsigned)rt + (unsigned)ct[e]);
-          if (C && grow < M && n0 + tcol < N)  // N % 16 == 0: the four columns are in or out together
-            *reinterpret_cast<v4i*>(C + (size_t)grow * N + n0 + tcol) = v4i{v[0], v[1], v[2], v[3]};
+          if constexpr (WRITE_C) {
+            if (grow < M && n0 + tcol < N)  // N % 16 == 0: the four columns are in or out together
+              *reinterpret_cast<v4i*>(C + (size_t)grow * N + n0 + tcol) = v4i{v[0], v[1], v[2], v[3]};
+          }
           if constexpr (FLAVOUR != 0) {
             unsigned q[4];
 #pragma unroll
@@ -360,7 +363,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 2) void qgemm_dma_kernel(const QGem
   }
 }
 
-template <int BM, int BN, int WGM, int WGN, int STAGES, bool REQUANT>
+template <int BM, int BN, int WGM, int WGN, int STAGES, bool REQUANT, bool WRITE_C>
 int launch(hipStream_t stream, QGemmParams p) {
   constexpr int kThreads = WGM * WGN * 64;
   p.tilesM = (p.M + BM - 1) / BM;
@@ -373,7 +376,7 @@ int launch(hipStream_t stream, QGemmParams p) {
   constexpr size_t epi = (size_t)(BM + BN) * 4 + (size_t)BM * (BN + 4);
   constexpr size_t lds = ring > epi ? ring : epi;
   static_assert(lds <= 160 * 1024, "LDS budget");
-  auto kern = qgemm_dma_kernel<BM, BN, WGM, WGN, STAGES, REQUANT>;
+  auto kern = qgemm_dma_kernel<BM, BN, WGM, WGN, STAGES, REQUANT, WRITE_C>;
   static bool attrSet[16] = {};  // per device: the attribute belongs to the function on one device
   int dev = 0;
   TFCC_HIP_CHECK(hipGetDevice(&dev));
@@ -397,17 +400,21 @@ bool qgemm_dma_supported(const QGemmParams& p, bool requant) {
          ((unsigned long long)p.M + 512) * p.K < (1ull << 32) && ((unsigned long long)p.K + 1024) * p.N + 1024 < (1ull << 32);
 }
 
+namespace {
+template <int BM, int BN, int WGM, int WGN, int STAGES>
+int launch_for_outputs(hipStream_t stream, const QGemmParams& p, bool requant) {
+  if (!requant) return launch<BM, BN, WGM, WGN, STAGES, false, true>(stream, p);
+  return p.C ? launch<BM, BN, WGM, WGN, STAGES, true, true>(stream, p) : launch<BM, BN, WGM, WGN, STAGES, true, false>(stream, p);
+}
+}  // namespace
+
 int qgemm_dma_launch(hipStream_t stream, const QGemmParams& p, bool requant) {
   const unsigned long long big = (unsigned long long)((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batch;
-  if (big >= 192) {
-    return requant ? launch<256, 256, 2, 4, 2, true>(stream, p) : launch<256, 256, 2, 4, 2, false>(stream, p);
-  }
+  if (big >= 192) return launch_for_outputs<256, 256, 2, 4, 2>(stream, p, requant);
   // fewer than half a chip of 128x128 tiles: 64x128 tiles (four wavefronts side by side) put twice as many CUs to work
   const unsigned long long mid = (unsigned long long)((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batch;
-  if (mid < 128) {
-    return requant ? launch<64, 128, 1, 4, 2, true>(stream, p) : launch<64, 128, 1, 4, 2, false>(stream, p);
-  }
-  return requant ? launch<128, 128, 2, 2, 2, true>(stream, p) : launch<128, 128, 2, 2, 2, false>(stream, p);
+  if (mid < 128) return launch_for_outputs<64, 128, 1, 4, 2>(stream, p, requant);
+  return launch_for_outputs<128, 128, 2, 2, 2>(stream, p, requant);
 }
 
 }  // namespace tfcc_rocm
