@@ -309,7 +309,10 @@ __global__ __launch_bounds__(WGM * WGN * 64, 2) void qgemm_dma_kernel(const QGem
     for (int i = 0; i < MI; ++i) {
       const int trow = wm * WM + 32 * i + l32;
       const unsigned grow = m0 + trow;
-      const int rt = rowTerm[trow];
+      // without an int32 result to store, the 2^31 that turns the accumulator into its offset from INT32_MIN is
+      // folded into the row term
+      constexpr unsigned kBias = (REQUANT && !WRITE_C) ? 0x80000000u : 0u;
+      const int rt = (int)((unsigned)rowTerm[trow] + kBias);
 #pragma unroll
       for (int j = 0; j < NI; ++j) {
 #pragma unroll
@@ -327,9 +330,10 @@ __global__ __launch_bounds__(WGM * WGN * 64, 2) void qgemm_dma_kernel(const QGem
             unsigned q[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
-              if constexpr (FLAVOUR == 1) q[e] = (unsigned)requantize_one_fast((double)((unsigned)v[e] ^ 0x80000000u), rq);
-              else if constexpr (FLAVOUR == 2) q[e] = (unsigned)requantize_one_exact((long long)v[e], rq);
-              else if constexpr (FLAVOUR == 4) q[e] = (unsigned)requantize_one_fast32((double)((unsigned)v[e] ^ 0x80000000u), rq);
+              const unsigned off = (unsigned)v[e] ^ (0x80000000u ^ kBias);  // v - INT32_MIN
+              if constexpr (FLAVOUR == 1) q[e] = (unsigned)requantize_one_fast((double)off, rq);
+              else if constexpr (FLAVOUR == 2) q[e] = (unsigned)requantize_one_exact((long long)(int)(off ^ 0x80000000u), rq);
+              else if constexpr (FLAVOUR == 4) q[e] = (unsigned)requantize_one_fast32((double)off, rq);
               else q[e] = (unsigned)rq.fillValue;
             }
             *reinterpret_cast<unsigned*>(stageQ + trow * QPITCH + tcol) = q[0] | (q[1] << 8) | (q[2] << 16) | (q[3] << 24);
