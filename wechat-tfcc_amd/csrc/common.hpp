@@ -115,6 +115,10 @@ struct RequantScalars {
   int fastOK;                // the double shortcut is exact for every input
   int fast32OK;              // ... and rint(y), rint(y) - (outOffset - outLowest) stay inside int32
   int offsetMinusLowest32;
+  // fast32OK, the output scale a power of two and outOffset - outLowest even: the scale is folded into the
+  // first step's constants and the offset into the rounding constant (see requantize_one_folded)
+  int foldedOK;
+  double inScaleFolded, inMinFolded, magicFolded;
 };
 
 // offMax = highest - lowest of the input type (its largest x - inLowest)
@@ -128,6 +132,18 @@ __host__ __device__ static inline void finish_requant_scalars(RequantScalars& s,
   const double dAbs = d < 0 ? -(double)d : (double)d;
   s.fast32OK = (s.fastOK && bound + dAbs < 2147483000.0) ? 1 : 0;
   s.offsetMinusLowest32 = s.fast32OK ? (int)d : 0;
+  // Multiplying by 2^e commutes with rounding (no overflow, no subnormals: real is 0 or at least 2^-60 in size
+  // for 32-bit inputs and scales of normal size), so fma(off, inScale * 2^e, inMin * 2^e) is the reference's
+  // real * outScale bit for bit.  An even d keeps the parity of the candidates of a tie, so adding
+  // 1.5 * 2^52 - d rounds exactly like rint(y) - d.
+  int e = 0;
+  const double mant = frexp(s.outScale, &e);  // outScale = mant * 2^e, mant = 0.5 for a positive power of two
+  const bool pow2 = mant == 0.5 && e > -200 && e < 200 && fabs(s.inScale) > 1e-60 && fabs(s.inScale) < 1e60 &&
+                    (s.inMin == 0.0 || (fabs(s.inMin) > 1e-60 && fabs(s.inMin) < 1e60));
+  s.foldedOK = (s.fast32OK && pow2 && (d & 1) == 0) ? 1 : 0;
+  s.inScaleFolded = s.inScale * s.outScale;
+  s.inMinFolded = s.inMin * s.outScale;
+  s.magicFolded = 6755399441055744.0 - (double)d;
 }
 
 // Valid when RequantScalars::fast32OK.  Adding 1.5 * 2^52 rounds y to the nearest integer (ties to
@@ -137,6 +153,14 @@ __device__ static inline int requantize_one_fast32(double off, const RequantScal
   const double y = fma(off, s.inScale, s.inMin) * s.outScale;
   const int r = (int)(unsigned)__double_as_longlong(y + 6755399441055744.0);
   const int q = r - s.offsetMinusLowest32;
+  const int lo = (int)s.outLowest, hi = (int)s.outHighest;
+  return q < lo ? lo : (q > hi ? hi : q);
+}
+
+// Valid when RequantScalars::foldedOK: two double operations instead of four, the same value.
+__device__ static inline int requantize_one_folded(double off, const RequantScalars& s) {
+  const double y = fma(off, s.inScaleFolded, s.inMinFolded);
+  const int q = (int)(unsigned)__double_as_longlong(y + s.magicFolded);
   const int lo = (int)s.outLowest, hi = (int)s.outHighest;
   return q < lo ? lo : (q > hi ? hi : q);
 }

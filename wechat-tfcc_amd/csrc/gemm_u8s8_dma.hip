@@ -304,7 +304,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 2) void qgemm_dma_kernel(const QGem
   unsigned char* Q = REQUANT ? p.Q + (size_t)bi * p.strideC : nullptr;
 
   auto storeTile = [&](auto flavour) {
-    constexpr int FLAVOUR = decltype(flavour)::value;  // 0 int32 only, 1 double shortcut, 2 exact int64, 3 fill, 4 int32 shortcut
+    constexpr int FLAVOUR = decltype(flavour)::value;  // 0 int32 only, 1 double shortcut, 2 exact int64, 3 fill, 4 int32 shortcut, 5 folded
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
       const int trow = wm * WM + 32 * i + l32;
@@ -334,6 +334,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 2) void qgemm_dma_kernel(const QGem
               if constexpr (FLAVOUR == 1) q[e] = (unsigned)requantize_one_fast((double)off, rq);
               else if constexpr (FLAVOUR == 2) q[e] = (unsigned)requantize_one_exact((long long)(int)(off ^ 0x80000000u), rq);
               else if constexpr (FLAVOUR == 4) q[e] = (unsigned)requantize_one_fast32((double)off, rq);
+              else if constexpr (FLAVOUR == 5) q[e] = (unsigned)requantize_one_folded((double)off, rq);
               else q[e] = (unsigned)rq.fillValue;
             }
             *reinterpret_cast<unsigned*>(stageQ + trow * QPITCH + tcol) = q[0] | (q[1] << 8) | (q[2] << 16) | (q[3] << 24);
@@ -361,6 +362,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 2) void qgemm_dma_kernel(const QGem
     storeTile(std::integral_constant<int, 0>{});
   } else {
     if (rq.mode) storeTile(std::integral_constant<int, 3>{});
+    else if (rq.foldedOK) storeTile(std::integral_constant<int, 5>{});
     else if (rq.fast32OK) storeTile(std::integral_constant<int, 4>{});
     else if (rq.fastOK) storeTile(std::integral_constant<int, 1>{});
     else storeTile(std::integral_constant<int, 2>{});
