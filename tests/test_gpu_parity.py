@@ -275,6 +275,32 @@ def test_dequantize_and_quantize_against_oracle(pkg, T):
     assert np.array_equal(T.n(got), np.full(100, -128, np.int8))
 
 
+@pytest.mark.parametrize("total", [4096, 65540, 9_000_004])
+def test_streaming_quantization_kernels_at_size(pkg, T, total):
+    """The four-loads-in-flight kernels over sizes of one pass, a partial pass and several passes of the capped
+    grid: requantize int32 -> uint8 (both the general and the folded arithmetic), dequantize int32, quantize with
+    a given range and with the range found by the two-step reduction that parks its partial results in the
+    output buffer."""
+    import torch
+    rng = np.random.default_rng(total)
+    acc = rng.integers(-2 ** 26, 2 ** 26, total).astype(np.int32)
+    acc[:8] = (-2 ** 31, 2 ** 31 - 1, 0, -1, 1, 131072, -131072, 393216)
+    mn_c, mx_c = O.qmatmul_range(-128.0, 127.0, -128.0, 127.0)
+    for mn_o, mx_o in ((-128.0 * 2 ** 18, 127.0 * 2 ** 18), (-3.1e7, 2.9e7)):  # power-of-two scale / general
+        got = pkg.requantize(T.t(acc), T.f1(mn_c), T.f1(mx_c), T.f1(mn_o), T.f1(mx_o), torch.uint8)
+        assert np.array_equal(T.n(got), O.requantize_s32_u8(acc, mn_c, mx_c, mn_o, mx_o))
+    assert np.array_equal(T.n(pkg.dequantize(T.t(acc), T.f1(-3.25), T.f1(7.5))), O.dequantize(acc, -3.25, 7.5))
+    x = rng.normal(0, 2, total).astype(np.float32)
+    x[total // 3] = 11.5     # the extremes away from the ends
+    x[total // 2] = -13.25
+    for dtype, tdt in ((np.uint8, torch.uint8), (np.int8, torch.int8)):
+        got = pkg.quantize(T.t(x), tdt, T.f1(-6.0), T.f1(6.5))
+        assert np.array_equal(T.n(got), O.quantize(x, -6.0, 6.5, dtype))
+        got, mn_t, mx_t = pkg.quantize(T.t(x), tdt)
+        assert (float(T.n(mn_t)[0]), float(T.n(mx_t)[0])) == (-13.25, 11.5)
+        assert np.array_equal(T.n(got), O.quantize(x, -13.25, 11.5, dtype))
+
+
 def test_quantized_matmul_round_trip(pkg, T):
     """tfcc/test/quantization.cpp:105-189: quantize -> reduce_sum -> matmul -> dequantize gives 5, 11, 17."""
     import torch

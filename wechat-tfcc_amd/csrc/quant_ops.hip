@@ -131,35 +131,88 @@ __global__ __launch_bounds__(256) void requantize_kernel(const void* in, int inT
   }
 }
 
-// int32 -> uint8, the matmul epilogue's type pair, four elements per thread
+// 16-byte loads of data that is read once
+typedef int nt_v4i __attribute__((ext_vector_type(4)));
+typedef float nt_v4f __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ int4 load_streamed(const int4* p) {
+  const nt_v4i v = __builtin_nontemporal_load(reinterpret_cast<const nt_v4i*>(p));
+  return make_int4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ float4 load_streamed(const float4* p) {
+  const nt_v4f v = __builtin_nontemporal_load(reinterpret_cast<const nt_v4f*>(p));
+  return make_float4(v[0], v[1], v[2], v[3]);
+}
+
+// int32 -> uint8, the matmul epilogue's type pair.  Four elements per 16-byte load, four loads in flight per
+// thread, few enough threads that the scalar set-up (a few hundred double operations) is not what the launch
+// spends its time on.
+template <int FLAVOUR>  // 1 double shortcut, 2 exact int64, 3 fill, 4 int32 shortcut, 5 folded
+__device__ __forceinline__ unsigned requantize_four(const int4& v, const RequantScalars& s) {
+  const int x[4] = {v.x, v.y, v.z, v.w};
+  unsigned q[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const double off = (double)((unsigned)x[e] ^ 0x80000000u);
+    if (FLAVOUR == 5) q[e] = (unsigned)requantize_one_folded(off, s);
+    else if (FLAVOUR == 4) q[e] = (unsigned)requantize_one_fast32(off, s);
+    else if (FLAVOUR == 1) q[e] = (unsigned)requantize_one_fast(off, s);
+    else if (FLAVOUR == 2) q[e] = (unsigned)requantize_one_exact(x[e], s);
+    else q[e] = (unsigned)s.fillValue;
+  }
+  return (q[0] | (q[1] << 8)) | ((q[2] | (q[3] << 8)) << 16);
+}
+
+template <int FLAVOUR>
+__device__ __forceinline__ void requantize_s32_u8_loop(const int4* in, unsigned* out, size_t total4, const RequantScalars& s) {
+  const size_t step = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total4; i += 4 * step) {
+    int4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (i + u * step < total4) v[u] = load_streamed(in + i + u * step);
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (i + u * step < total4) out[i + u * step] = requantize_four<FLAVOUR>(v[u], s);
+  }
+}
+
 __global__ __launch_bounds__(256) void requantize_s32_u8_vec_kernel(const int4* in, unsigned* out, size_t total4,
                                                                     const float* minIn, const float* maxIn,
                                                                     const float* minOut, const float* maxOut) {
   const RequantScalars s = make_requant_scalars(TFCC_ROCM_S32, TFCC_ROCM_U8, *minIn, *maxIn, *minOut, *maxOut);
-  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (s.mode) requantize_s32_u8_loop<3>(in, out, total4, s);
+  else if (s.foldedOK) requantize_s32_u8_loop<5>(in, out, total4, s);
+  else if (s.fast32OK) requantize_s32_u8_loop<4>(in, out, total4, s);
+  else if (s.fastOK) requantize_s32_u8_loop<1>(in, out, total4, s);
+  else requantize_s32_u8_loop<2>(in, out, total4, s);
+}
+
+// int32 -> float, four elements per thread and load (the accumulators of a quantized matmul)
+__global__ __launch_bounds__(256) void dequantize_s32_vec_kernel(const int4* in, size_t total4, const float* minV,
+                                                                 const float* maxV, float4* out) {
+  const float mn = *minV, mx = *maxV;
+  double scale = 0, minRounded = 0;
+  const bool constant = mn >= mx;  // tfcc_mklquantizationinterface.cpp:321-324
+  if (!constant) dequantized_scale_info(32, mn, mx, &scale, &minRounded);
   const size_t step = (size_t)gridDim.x * blockDim.x;
-  for (; i < total4; i += step) {
-    int4 v = in[i];
-    unsigned q0, q1, q2, q3;
-    if (s.mode) {
-      q0 = q1 = q2 = q3 = (unsigned)s.fillValue;
-    } else if (s.fast32OK) {
-      q0 = (unsigned)requantize_one_fast32((double)((unsigned)v.x ^ 0x80000000u), s);
-      q1 = (unsigned)requantize_one_fast32((double)((unsigned)v.y ^ 0x80000000u), s);
-      q2 = (unsigned)requantize_one_fast32((double)((unsigned)v.z ^ 0x80000000u), s);
-      q3 = (unsigned)requantize_one_fast32((double)((unsigned)v.w ^ 0x80000000u), s);
-    } else if (s.fastOK) {
-      q0 = (unsigned)requantize_one_fast((double)((unsigned)v.x ^ 0x80000000u), s);
-      q1 = (unsigned)requantize_one_fast((double)((unsigned)v.y ^ 0x80000000u), s);
-      q2 = (unsigned)requantize_one_fast((double)((unsigned)v.z ^ 0x80000000u), s);
-      q3 = (unsigned)requantize_one_fast((double)((unsigned)v.w ^ 0x80000000u), s);
-    } else {
-      q0 = (unsigned)requantize_one_exact(v.x, s);
-      q1 = (unsigned)requantize_one_exact(v.y, s);
-      q2 = (unsigned)requantize_one_exact(v.z, s);
-      q3 = (unsigned)requantize_one_exact(v.w, s);
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total4; i += 4 * step) {
+    int4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (i + u * step < total4) v[u] = load_streamed(in + i + u * step);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (i + u * step >= total4) continue;
+      float4 r = make_float4(mn, mn, mn, mn);
+      if (!constant) {
+        // (double)x - (double)INT32_MIN, exact in double
+        r.x = (float)fma((double)((unsigned)v[u].x ^ 0x80000000u), scale, minRounded);
+        r.y = (float)fma((double)((unsigned)v[u].y ^ 0x80000000u), scale, minRounded);
+        r.z = (float)fma((double)((unsigned)v[u].z ^ 0x80000000u), scale, minRounded);
+        r.w = (float)fma((double)((unsigned)v[u].w ^ 0x80000000u), scale, minRounded);
+      }
+      out[i + u * step] = r;
     }
-    out[i] = q0 | (q1 << 8) | (q2 << 16) | (q3 << 24);
   }
 }
 
@@ -206,6 +259,43 @@ __global__ __launch_bounds__(256) void quantize_kernel(const float* in, size_t t
   }
 }
 
+// float -> uint8 / int8, four elements per thread and load, four loads in flight
+__global__ __launch_bounds__(256) void quantize_8bit_vec_kernel(const float4* in, size_t total4, const float* minV,
+                                                                const float* maxV, unsigned* out, int outType,
+                                                                int fromData) {
+  const float mn = *minV, mx = *maxV;
+  const IntRange r = int_range(outType);
+  const bool fillLowest = fromData ? (mn == mx) : (mn >= mx);
+  double scale = 0;
+  long long offset = 0;
+  if (!fillLowest) quantized_scale_info(r.bits, mn, mx, &scale, &offset);
+  const size_t step = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total4; i += 4 * step) {
+    float4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (i + u * step < total4) v[u] = load_streamed(in + i + u * step);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (i + u * step >= total4) continue;
+      const float x[4] = {v[u].x, v[u].y, v[u].z, v[u].w};
+      unsigned word = 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        long long q = r.lowest;
+        if (!fillLowest) {
+          q = to_int64_x86(rint((double)x[e] * scale));
+          q = (long long)((unsigned long long)q - (unsigned long long)offset + (unsigned long long)r.lowest);
+          q = q < r.lowest ? r.lowest : q;
+          q = q > r.highest ? r.highest : q;
+        }
+        word |= ((unsigned)q & 0xffu) << (8 * e);
+      }
+      out[i + u * step] = word;
+    }
+  }
+}
+
 // min / max of a float tensor.  Monotone uint encoding so that unsigned atomics order floats.
 __device__ __forceinline__ unsigned enc(float f) {
   unsigned u = __float_as_uint(f);
@@ -243,6 +333,71 @@ __global__ __launch_bounds__(256) void minmax_kernel(const float* in, size_t tot
   }
 }
 
+// The same reduction without atomics for tensors large enough to matter: every workgroup leaves its minimum
+// and maximum in the (not yet written) output buffer of the quantize call, one more workgroup reduces those.
+// 65536 atomics on two words took 380 us for 16.7 M floats; this takes the time of reading them once.
+__global__ __launch_bounds__(256) void minmax_partial_kernel(const float* in, size_t total, float* partials) {
+  __shared__ float shMn[4], shMx[4];
+  const size_t total4 = total / 4, step = (size_t)gridDim.x * blockDim.x;
+  const float4* in4 = reinterpret_cast<const float4*>(in);
+  float mn = 3.402823466e+38f, mx = -3.402823466e+38f;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < total4; i += 4 * step) {
+    float4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (i + u * step < total4) v[u] = load_streamed(in4 + i + u * step);
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (i + u * step >= total4) continue;
+      mn = fminf(fminf(mn, fminf(v[u].x, v[u].y)), fminf(v[u].z, v[u].w));
+      mx = fmaxf(fmaxf(mx, fmaxf(v[u].x, v[u].y)), fmaxf(v[u].z, v[u].w));
+    }
+  }
+  if (blockIdx.x == 0 && threadIdx.x < total - total4 * 4) {  // the last 1..3 elements
+    const float v = in[total4 * 4 + threadIdx.x];
+    mn = fminf(mn, v);
+    mx = fmaxf(mx, v);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    mn = fminf(mn, __shfl_down(mn, off, 64));
+    mx = fmaxf(mx, __shfl_down(mx, off, 64));
+  }
+  if ((threadIdx.x & 63) == 0) {
+    shMn[threadIdx.x >> 6] = mn;
+    shMx[threadIdx.x >> 6] = mx;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    partials[2 * blockIdx.x] = fminf(fminf(shMn[0], shMn[1]), fminf(shMn[2], shMn[3]));
+    partials[2 * blockIdx.x + 1] = fmaxf(fmaxf(shMx[0], shMx[1]), fmaxf(shMx[2], shMx[3]));
+  }
+}
+
+__global__ __launch_bounds__(256) void minmax_final_kernel(const float* partials, unsigned blocks, float* mnOut,
+                                                           float* mxOut) {
+  __shared__ float shMn[4], shMx[4];
+  float mn = 3.402823466e+38f, mx = -3.402823466e+38f;
+  for (unsigned i = threadIdx.x; i < blocks; i += 256) {
+    mn = fminf(mn, partials[2 * i]);
+    mx = fmaxf(mx, partials[2 * i + 1]);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    mn = fminf(mn, __shfl_down(mn, off, 64));
+    mx = fmaxf(mx, __shfl_down(mx, off, 64));
+  }
+  if ((threadIdx.x & 63) == 0) {
+    shMn[threadIdx.x >> 6] = mn;
+    shMx[threadIdx.x >> 6] = mx;
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    *mnOut = fminf(fminf(shMn[0], shMn[1]), fminf(shMn[2], shMn[3]));
+    *mxOut = fmaxf(fmaxf(shMx[0], shMx[1]), fmaxf(shMx[2], shMx[3]));
+  }
+}
+
 __global__ void minmax_finish_kernel(float* mn, float* mx) {
   *mn = dec(*reinterpret_cast<const unsigned*>(mn));
   *mx = dec(*reinterpret_cast<const unsigned*>(mx));
@@ -255,7 +410,28 @@ unsigned grid_for(size_t total, unsigned perThread = 1) {
   return (unsigned)blocks;
 }
 
+// the vector kernels: four 16-byte loads per thread per pass, at most 8 workgroups per CU
+unsigned stream_grid(size_t total4) {
+  size_t blocks = (total4 + 1023) / 1024;
+  if (blocks > 256u * 8u) blocks = 256u * 8u;
+  if (blocks < 1) blocks = 1;
+  return (unsigned)blocks;
+}
+
 bool valid_type(int t) { return t >= TFCC_ROCM_S8 && t <= TFCC_ROCM_U32; }
+
+void launch_quantize(hipStream_t s, const float* in, uint64_t total, const float* minV, const float* maxV, void* out,
+                     int outType, int fromData) {
+  if ((outType == TFCC_ROCM_U8 || outType == TFCC_ROCM_S8) && total % 4 == 0 && (uintptr_t)in % 16 == 0 &&
+      (uintptr_t)out % 4 == 0) {
+    hipLaunchKernelGGL(quantize_8bit_vec_kernel, dim3(stream_grid(total / 4)), dim3(256), 0, s,
+                       reinterpret_cast<const float4*>(in), (size_t)(total / 4), minV, maxV, static_cast<unsigned*>(out),
+                       outType, fromData);
+  } else {
+    hipLaunchKernelGGL(quantize_kernel, dim3(grid_for(total)), dim3(256), 0, s, in, (size_t)total, minV, maxV, out,
+                       outType, fromData);
+  }
+}
 
 template <class T>
 int reduce_rows(hipStream_t s, const void* a, unsigned batch, unsigned row, unsigned col, int* out) {
@@ -331,7 +507,7 @@ int tfcc_rocm_requantize(void* stream, const void* in, int in_type, void* out, i
   hipStream_t s = as_stream(stream);
   if (in_type == TFCC_ROCM_S32 && out_type == TFCC_ROCM_U8 && total % 4 == 0 && (uintptr_t)in % 16 == 0 &&
       (uintptr_t)out % 4 == 0) {
-    hipLaunchKernelGGL(requantize_s32_u8_vec_kernel, dim3(grid_for(total / 4)), dim3(256), 0, s,
+    hipLaunchKernelGGL(requantize_s32_u8_vec_kernel, dim3(stream_grid(total / 4)), dim3(256), 0, s,
                        static_cast<const int4*>(in), static_cast<unsigned*>(out), (size_t)(total / 4), min_in,
                        max_in, min_out, max_out);
   } else {
@@ -346,8 +522,13 @@ int tfcc_rocm_dequantize(void* stream, const void* in, int in_type, uint64_t tot
   TFCC_REQUIRE(in && out && min_v && max_v, "dequantize: null argument");
   TFCC_REQUIRE(total > 0, "dequantize: empty tensor");
   TFCC_REQUIRE(valid_type(in_type), "dequantize: bad type code");
-  hipLaunchKernelGGL(dequantize_kernel, dim3(grid_for(total)), dim3(256), 0, as_stream(stream), in, in_type,
-                     (size_t)total, min_v, max_v, out);
+  if (in_type == TFCC_ROCM_S32 && total % 4 == 0 && (uintptr_t)in % 16 == 0 && (uintptr_t)out % 16 == 0) {
+    hipLaunchKernelGGL(dequantize_s32_vec_kernel, dim3(stream_grid(total / 4)), dim3(256), 0, as_stream(stream),
+                       static_cast<const int4*>(in), (size_t)(total / 4), min_v, max_v, reinterpret_cast<float4*>(out));
+  } else {
+    hipLaunchKernelGGL(dequantize_kernel, dim3(grid_for(total)), dim3(256), 0, as_stream(stream), in, in_type,
+                       (size_t)total, min_v, max_v, out);
+  }
   return check_launch("dequantize");
 }
 
@@ -356,8 +537,7 @@ int tfcc_rocm_quantize(void* stream, const float* in, uint64_t total, const floa
   TFCC_REQUIRE(in && out && min_v && max_v, "quantize: null argument");
   TFCC_REQUIRE(total > 0, "quantize: empty tensor");
   TFCC_REQUIRE(valid_type(out_type), "quantize: bad type code");
-  hipLaunchKernelGGL(quantize_kernel, dim3(grid_for(total)), dim3(256), 0, as_stream(stream), in, (size_t)total,
-                     min_v, max_v, out, out_type, 0);
+  launch_quantize(as_stream(stream), in, total, min_v, max_v, out, out_type, 0);
   return check_launch("quantize");
 }
 
@@ -369,11 +549,20 @@ int tfcc_rocm_quantize_minmax(void* stream, const float* in, uint64_t total, voi
   hipStream_t s = as_stream(stream);
   unsigned* mnWord = reinterpret_cast<unsigned*>(min_v);
   unsigned* mxWord = reinterpret_cast<unsigned*>(max_v);
-  hipLaunchKernelGGL(minmax_init_kernel, dim3(1), dim3(1), 0, s, mnWord, mxWord);
-  hipLaunchKernelGGL(minmax_kernel, dim3(grid_for(total, 4)), dim3(256), 0, s, in, (size_t)total, mnWord, mxWord);
-  hipLaunchKernelGGL(minmax_finish_kernel, dim3(1), dim3(1), 0, s, min_v, max_v);
-  hipLaunchKernelGGL(quantize_kernel, dim3(grid_for(total)), dim3(256), 0, s, in, (size_t)total, min_v, max_v, out,
-                     out_type, 1);
+  const IntRange range = int_range(out_type);
+  const size_t outBytes = (size_t)total * (range.bits / 8);
+  const unsigned blocks = stream_grid(total / 4);
+  if ((uintptr_t)in % 16 == 0 && (uintptr_t)out % 4 == 0 && outBytes >= (size_t)blocks * 8 && total >= 4096) {
+    // partial results rest in the output buffer until the quantize pass overwrites it
+    float* partials = static_cast<float*>(out);
+    hipLaunchKernelGGL(minmax_partial_kernel, dim3(blocks), dim3(256), 0, s, in, (size_t)total, partials);
+    hipLaunchKernelGGL(minmax_final_kernel, dim3(1), dim3(256), 0, s, partials, blocks, min_v, max_v);
+  } else {
+    hipLaunchKernelGGL(minmax_init_kernel, dim3(1), dim3(1), 0, s, mnWord, mxWord);
+    hipLaunchKernelGGL(minmax_kernel, dim3(grid_for(total, 4)), dim3(256), 0, s, in, (size_t)total, mnWord, mxWord);
+    hipLaunchKernelGGL(minmax_finish_kernel, dim3(1), dim3(1), 0, s, min_v, max_v);
+  }
+  launch_quantize(s, in, total, min_v, max_v, out, out_type, 1);
   return check_launch("quantize");
 }
 
