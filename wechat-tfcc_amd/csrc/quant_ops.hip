@@ -49,17 +49,27 @@ __global__ __launch_bounds__(256) void reduce_rows_kernel(const T* a, unsigned r
   constexpr unsigned PER = 16 / sizeof(T);
   if (col % PER == 0 && ((uintptr_t)a % 16 == 0)) {
     const uint4* v = reinterpret_cast<const uint4*>(p);
-    for (unsigned i = lane; i < col / PER; i += 64) {
-      uint4 q = v[i];
-      unsigned w[4] = {q.x, q.y, q.z, q.w};
+    const unsigned chunks = col / PER;
+    // eight loads in flight per lane; bytes are summed four at a time by the dot-product instructions
+    for (unsigned i0 = lane; i0 < chunks; i0 += 64 * 8) {
+      uint4 q[8];
 #pragma unroll
-      for (int d = 0; d < 4; ++d) {
-        if (sizeof(T) == 1) {
+      for (int u = 0; u < 8; ++u) {
+        q[u] = make_uint4(0, 0, 0, 0);
+        if (i0 + 64 * u < chunks) q[u] = v[i0 + 64 * u];
+      }
 #pragma unroll
-          for (int b = 0; b < 4; ++b) s += (unsigned)(int)(T)(w[d] >> (8 * b));
-        } else {
+      for (int u = 0; u < 8; ++u) {
+        const unsigned w[4] = {q[u].x, q[u].y, q[u].z, q[u].w};
 #pragma unroll
-          for (int b = 0; b < 2; ++b) s += (unsigned)(int)(T)(w[d] >> (16 * b));
+        for (int d = 0; d < 4; ++d) {
+          if (sizeof(T) == 1) {
+            if (T(-1) < T(0)) s = (unsigned)__builtin_amdgcn_sdot4((int)w[d], 0x01010101, (int)s, false);
+            else s = __builtin_amdgcn_udot4(w[d], 0x01010101u, s, false);
+          } else {
+#pragma unroll
+            for (int b = 0; b < 2; ++b) s += (unsigned)(int)(T)(w[d] >> (16 * b));
+          }
         }
       }
     }
