@@ -160,6 +160,11 @@ typedef struct tfcc_rocm_qgemm_desc {
   /* Optional: b as packed once by tfcc_rocm_gemv_pack_b (weights).  A product of at most 8 rows
    * (batch == 1) then streams the packed copy; every other shape reads b. */
   const void* packed_b;
+  /* Optional promise: colsum_b holds the true column sums of b (it came from tfcc_rocm_reduce_sum_cols
+   * on this b).  The kernel needs the true sums on top of colsum_b as given (it feeds a - 128 to the
+   * signed matrix cores) and otherwise accumulates them itself; with the promise it skips that.  The
+   * result is the same whenever the promise holds. */
+  int colsum_b_is_exact;
 } tfcc_rocm_qgemm_desc;
 
 /* int32 result only */

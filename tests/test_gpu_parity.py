@@ -45,6 +45,9 @@ def test_qgemm_golden_vectors(pkg, T, seed, shape_a, shape_b):
                                                      T.f1(mn_o), T.f1(mx_o), want_acc=True)
     assert np.array_equal(T.n(c2), z[p + "c"])
     assert np.array_equal(T.n(q), z[p + "q"])
+    q_promised, _, _, _ = pkg.quantization_matmul_requantize(T.t(a), T.t(rs), r[0], r[1], T.t(b), T.t(cs), r[2], r[3],
+                                                              T.f1(mn_o), T.f1(mx_o), colsum_exact=True)
+    assert np.array_equal(T.n(q_promised), T.n(q))  # cs holds the true column sums: the promise changes nothing
     q_only, none, _, _ = pkg.quantization_matmul_requantize(T.t(a), T.t(rs), r[0], r[1], T.t(b), T.t(cs), r[2],
                                                             r[3], T.f1(mn_o), T.f1(mx_o), want_acc=False)
     assert none is None and np.array_equal(T.n(q_only), z[p + "q"])
@@ -102,6 +105,12 @@ def test_qgemm_full_size_hash(pkg, T, name):
     q2, _, _, _ = pkg.quantization_matmul_requantize(T.t(a), T.t(rs), r[0], r[1], T.t(b), T.t(cs), r[2], r[3],
                                                      T.f1(mn_o), T.f1(mx_o), want_acc=False)
     assert hashlib.sha256(T.n(q2).tobytes()).hexdigest() == h["sha256_q"]
+    # with the promise that the column sums passed in are the true ones (they are) the kernel skips its own
+    for want_acc in (False, True):
+        q3, c3, _, _ = pkg.quantization_matmul_requantize(T.t(a), T.t(rs), r[0], r[1], T.t(b), T.t(cs), r[2], r[3],
+                                                          T.f1(mn_o), T.f1(mx_o), want_acc=want_acc, colsum_exact=True)
+        assert hashlib.sha256(T.n(q3).tobytes()).hexdigest() == h["sha256_q"]
+        assert c3 is None or hashlib.sha256(T.n(c3).tobytes()).hexdigest() == h["sha256_c"]
     # sums computed on the device equal the oracle's
     assert np.array_equal(T.n(pkg.reduce_sum(T.t(a), True)), rs)
     assert np.array_equal(T.n(pkg.reduce_sum(T.t(b), False)), cs)

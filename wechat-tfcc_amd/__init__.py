@@ -36,7 +36,7 @@ class QGemmDesc(C.Structure):
         ("offset_a", C.c_int32), ("offset_b", C.c_int32),
         ("min_a", C.c_void_p), ("max_a", C.c_void_p), ("min_b", C.c_void_p), ("max_b", C.c_void_p),
         ("min_c", C.c_void_p), ("max_c", C.c_void_p),
-        ("packed_b", C.c_void_p),
+        ("packed_b", C.c_void_p), ("colsum_b_is_exact", C.c_int),
     ]
 
 
@@ -385,8 +385,9 @@ def quantization_matmul_offsets(a, reduce_a, b, reduce_b, offset_a, offset_b):
 
 
 def quantization_matmul_requantize(a, reduce_a, min_a, max_a, b, reduce_b, min_b, max_b, min_out, max_out,
-                                   want_acc=False):
-    """matmul followed by requantize<uint8_t> in one kernel.  Returns (uint8 Q, int32 C or None, minC, maxC)."""
+                                   want_acc=False, colsum_exact=False):
+    """matmul followed by requantize<uint8_t> in one kernel.  Returns (uint8 Q, int32 C or None, minC, maxC).
+    colsum_exact: the caller's promise that reduce_b holds the true column sums of b."""
     import torch
     a, b, reduce_a, reduce_b = a.contiguous(), b.contiguous(), reduce_a.contiguous(), reduce_b.contiguous()
     for t, nm in ((min_a, "minA"), (max_a, "maxA"), (min_b, "minB"), (max_b, "maxB"), (min_out, "minOutput"),
@@ -399,6 +400,7 @@ def quantization_matmul_requantize(a, reduce_a, min_a, max_a, b, reduce_b, min_b
     max_c = torch.empty(1, dtype=torch.float32, device=a.device)
     d.min_a, d.max_a, d.min_b, d.max_b = _ptr(min_a), _ptr(max_a), _ptr(min_b), _ptr(max_b)
     d.min_c, d.max_c = _ptr(min_c), _ptr(max_c)
+    d.colsum_b_is_exact = 1 if colsum_exact else 0
     check(lib().tfcc_rocm_gemm_u8s8s32_requant_u8(_stream(), C.byref(d), _ptr(c), _ptr(q), 0.0, 0.0, 0.0, 0,
                                                    _ptr(min_out), _ptr(max_out)))
     return q, c, min_c, max_c

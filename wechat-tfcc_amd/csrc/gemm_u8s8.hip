@@ -422,6 +422,7 @@ int fill_params(const tfcc_rocm_qgemm_desc* d, QGemmParams& p) {
   p.strideRB = d->stride_colsum_b; p.strideC = d->stride_c;
   p.M = d->m; p.N = d->n; p.K = d->k; p.batch = d->batch;
   p.offsetA = d->offset_a; p.offsetB = d->offset_b;
+  p.colsumExact = d->colsum_b_is_exact ? 1 : 0;
   if (allRange) { p.minA = d->min_a; p.maxA = d->max_a; p.minB = d->min_b; p.maxB = d->max_b; p.minC = d->min_c; p.maxC = d->max_c; }
   return TFCC_ROCM_OK;
 }

@@ -44,7 +44,9 @@ constexpr int KS = BK / 32;  // 32-deep matrix-op steps per slab
 __device__ __forceinline__ int swzA(int row) { return (row >> 1) & 7; }
 
 // WRITE_C: the int32 result is stored (always without REQUANT; with it only when the caller wants both).
-template <int BM, int BN, int WGM, int WGN, int STAGES, bool REQUANT, bool WRITE_C>
+// OWN_COLSUM: the true column sums of B are accumulated here (the caller's colsum_b is used as given, whatever
+// it holds, like the reference does); without it the caller has promised that colsum_b holds them.
+template <int BM, int BN, int WGM, int WGN, int STAGES, bool REQUANT, bool WRITE_C, bool OWN_COLSUM>
 __global__ __launch_bounds__(WGM * WGN * 64, 2) void qgemm_dma_kernel(const QGemmParams p) {
   constexpr int kThreads = WGM * WGN * 64;
   constexpr int WM = BM / WGM, WN = BN / WGN;
@@ -213,7 +215,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 2) void qgemm_dma_kernel(const QGem
     const unsigned char* as = smem + stage * STAGE_BYTES;
     const unsigned char* bs = as + A_BYTES;
 #pragma unroll
-    for (int t = 0; t < NT; ++t) {
+    for (int t = 0; t < (OWN_COLSUM ? NT : 0); ++t) {
       v4i own = ub[WGM * t];  // the block of this wavefront row: selects on a wave-uniform condition, no branches
 #pragma unroll
       for (int w = 1; w < WGM; ++w) own = wm == w ? ub[WGM * t + w] : own;
@@ -277,7 +279,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 2) void qgemm_dma_kernel(const QGem
   // lanes l and l+32 hold the two k halves of the same column; the transposing read hands lane
   // (colHalf, s16) column 16*colHalf + s16 of the 32-column block
 #pragma unroll
-  for (int t = 0; t < NT; ++t) {
+  for (int t = 0; t < (OWN_COLSUM ? NT : 0); ++t) {
     const int j = wm + WGM * t;
     int s = colsum[t][0] + colsum[t][1] + colsum[t][2] + colsum[t][3];
     s += __shfl_xor(s, 32, 64);
@@ -285,7 +287,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 2) void qgemm_dma_kernel(const QGem
   }
   __syncthreads();
   const unsigned global = (unsigned)offA * (unsigned)offB * K;
-  if (tid < BN) colTerm[tid] = (int)(128u * (unsigned)colTerm[tid] + csPre * (unsigned)offA);
+  if (tid < BN) colTerm[tid] = (int)(128u * (OWN_COLSUM ? (unsigned)colTerm[tid] : csPre) + csPre * (unsigned)offA);
   if (tid < BM) rowTerm[tid] = (int)(global + rsPre * (unsigned)offB);
   __syncthreads();
 
@@ -369,7 +371,7 @@ __global__ __launch_bounds__(WGM * WGN * 64, 2) void qgemm_dma_kernel(const QGem
   }
 }
 
-template <int BM, int BN, int WGM, int WGN, int STAGES, bool REQUANT, bool WRITE_C>
+template <int BM, int BN, int WGM, int WGN, int STAGES, bool REQUANT, bool WRITE_C, bool OWN_COLSUM>
 int launch(hipStream_t stream, QGemmParams p) {
   constexpr int kThreads = WGM * WGN * 64;
   p.tilesM = (p.M + BM - 1) / BM;
@@ -382,7 +384,7 @@ int launch(hipStream_t stream, QGemmParams p) {
   constexpr size_t epi = (size_t)(BM + BN) * 4 + (size_t)BM * (BN + 4);
   constexpr size_t lds = ring > epi ? ring : epi;
   static_assert(lds <= 160 * 1024, "LDS budget");
-  auto kern = qgemm_dma_kernel<BM, BN, WGM, WGN, STAGES, REQUANT, WRITE_C>;
+  auto kern = qgemm_dma_kernel<BM, BN, WGM, WGN, STAGES, REQUANT, WRITE_C, OWN_COLSUM>;
   static bool attrSet[16] = {};  // per device: the attribute belongs to the function on one device
   int dev = 0;
   TFCC_HIP_CHECK(hipGetDevice(&dev));
@@ -407,10 +409,16 @@ bool qgemm_dma_supported(const QGemmParams& p, bool requant) {
 }
 
 namespace {
+template <int BM, int BN, int WGM, int WGN, int STAGES, bool OWN_COLSUM>
+int launch_for_outputs2(hipStream_t stream, const QGemmParams& p, bool requant) {
+  if (!requant) return launch<BM, BN, WGM, WGN, STAGES, false, true, OWN_COLSUM>(stream, p);
+  return p.C ? launch<BM, BN, WGM, WGN, STAGES, true, true, OWN_COLSUM>(stream, p)
+             : launch<BM, BN, WGM, WGN, STAGES, true, false, OWN_COLSUM>(stream, p);
+}
 template <int BM, int BN, int WGM, int WGN, int STAGES>
 int launch_for_outputs(hipStream_t stream, const QGemmParams& p, bool requant) {
-  if (!requant) return launch<BM, BN, WGM, WGN, STAGES, false, true>(stream, p);
-  return p.C ? launch<BM, BN, WGM, WGN, STAGES, true, true>(stream, p) : launch<BM, BN, WGM, WGN, STAGES, true, false>(stream, p);
+  return p.colsumExact ? launch_for_outputs2<BM, BN, WGM, WGN, STAGES, false>(stream, p, requant)
+                       : launch_for_outputs2<BM, BN, WGM, WGN, STAGES, true>(stream, p, requant);
 }
 }  // namespace
 

@@ -21,6 +21,7 @@ struct QGemmParams {
   double inScale, inMin, outScale;
   long long outOffset;
   const float *minOut, *maxOut;
+  int colsumExact;    // colsumB holds the true column sums of B: no need to accumulate them
   // tile bookkeeping filled by the launcher
   unsigned tilesM, tilesN, tilesTotal, chunk;
 };

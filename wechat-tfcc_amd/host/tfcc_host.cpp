@@ -967,6 +967,7 @@ std::tuple<Variable<int32_t>, Variable<float>, Variable<float>> matmul(
   p.desc.min_c = minResult.data();
   p.desc.max_c = maxResult.data();
   p.desc.packed_b = w.packed();
+  p.desc.colsum_b_is_exact = 1;  // w.reduceSum() was computed from w.weights()
   check(tfcc_rocm_gemm_u8s8s32(current_stream(), &p.desc, result.data()));
   return std::make_tuple(std::move(result), std::move(minResult), std::move(maxResult));
 }

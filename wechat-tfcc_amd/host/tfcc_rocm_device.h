@@ -157,7 +157,8 @@ class PreparedWeights {
 };
 
 // matmul(a, reduceSumA, minA, maxA, w.weights(), w.reduceSum(), minB, maxB): the same checks and the
-// same result; products of at most 8 rows stream the packed copy.
+// same result; products of at most 8 rows stream the packed copy, large ones skip the accumulation of the
+// true column sums (they are what w.reduceSum() holds).
 std::tuple<Variable<int32_t>, Variable<float>, Variable<float>> matmul(
     const Tensor<uint8_t>& a, const Tensor<int32_t>& reduceSumA, const Tensor<float>& minA,
     const Tensor<float>& maxA, const PreparedWeights& w, const Tensor<float>& minB, const Tensor<float>& maxB);
