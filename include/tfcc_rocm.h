@@ -325,6 +325,35 @@ int tfcc_rocm_binary_f32(void* stream, int op, const float* a, const float* b, u
 int tfcc_rocm_transpose_f32(void* stream, const float* in, const unsigned* shape,
                             const unsigned* perm, int rank, float* out);
 
+/* ---- recurrent cells: the element-wise step after the two matrix products of a time step -------------------
+ * All tensors row-major and dense; one launch each.
+ *
+ * CellInterface::processLSTMCell (tfcc/core/interfaces/tfcc_cellinterface.h:33-47; arithmetic of
+ * _MKLCellKernel::processLSTMCell, tfcc/mkl/kernel/tfcc_mklcellkernel.hpp:51-87): state_c [batch, units],
+ * input_value and state_h_value [batch, 4 * units] in gate order i, c, f, o, bias [4 * units];
+ * cs = tanh(xc) * sigmoid(xi) + state_c * sigmoid(xf + forget), h = tanh(cs) * sigmoid(xo).
+ * h and cs are [batch, units]; cs may be state_c itself. */
+int tfcc_rocm_lstm_cell_f32(void* stream, unsigned batch, unsigned units, const float* state_c,
+                            const float* input_value, const float* state_h_value, const float* bias, float forget,
+                            float* h, float* cs);
+/* CellInterface::processGRUCellGates (tfcc_cellinterface.h:49-59; tfcc_mklcellkernel.hpp:89-133):
+ * result [batch, input_size + units] = concat(inputs, sigmoid(value[:, :units] + bias[:units]) * state);
+ * value [batch, 2 * units], bias [2 * units]. */
+int tfcc_rocm_gru_cell_gates_f32(void* stream, unsigned batch, unsigned units, unsigned input_size,
+                                 const float* state, const float* inputs, const float* value, const float* bias,
+                                 float* result);
+/* CellInterface::processGRUCellCandidate (tfcc_cellinterface.h:61-70; tfcc_mklcellkernel.hpp:135-158):
+ * u = sigmoid(value[:, units:] + bias[units:]), c = tanh(c_value + c_bias), result = u * state + (1 - u) * c. */
+int tfcc_rocm_gru_cell_candidate_f32(void* stream, unsigned batch, unsigned units, const float* state,
+                                     const float* value, const float* bias, const float* c_value,
+                                     const float* c_bias, float* result);
+/* CellInterface::processPyTorchGRUCell (tfcc_cellinterface.h:72-86; tfcc_mklcellkernel.hpp:160-189):
+ * input_value and state_value [batch, 3 * units] (r, z, n), gate_bias [2 * units];
+ * n = tanh(ni + r * nh), result = n + z * (state - n). */
+int tfcc_rocm_pytorch_gru_cell_f32(void* stream, unsigned batch, unsigned units, const float* state,
+                                   const float* input_value, const float* state_value, const float* gate_bias,
+                                   const float* candidate_i_bias, const float* candidate_h_bias, float* result);
+
 #ifdef __cplusplus
 }
 #endif

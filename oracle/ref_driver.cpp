@@ -1,4 +1,4 @@
-// C entry points over the REFERENCE's own quantized-matmul and quantization kernels.
+// C entry points over the REFERENCE's own quantized-matmul, quantization and recurrent-cell kernels.
 // TEST INFRASTRUCTURE ONLY.  This file contains no arithmetic of the hot path: the matmul
 // micro-kernel, the AVX2 requantize / quantize / dequantize kernels, the scalar kernels and the
 // range helpers are the reference's, compiled from where they lie in the reference tree
@@ -16,6 +16,7 @@
 #include "kernel/tfcc_mklquantizationkernel.avx256.h"
 #include "kernel/tfcc_mklquantizationkernel.hpp"
 #include "kernel/tfcc_mklquantizationmatmul.avx256.h"
+#include "kernel/tfcc_mklcellkernel.hpp"
 #include "utils/tfcc_quantizationutils.h"
 
 namespace {
@@ -144,5 +145,25 @@ REF_DEQUANTIZE(ref_dequantize_s32, int32_t)
   }
 REF_QUANTIZE(ref_quantize_u8, uint8_t)
 REF_QUANTIZE(ref_quantize_s8, int8_t)
+
+// The scalar recurrent-cell kernels of the reference (tfcc/mkl/kernel/tfcc_mklcellkernel.hpp), as compiled.
+void ref_lstm_cell(unsigned batch, unsigned units, const float* stateC, const float* inputValue,
+                   const float* stateHValue, const float* bias, float forget, float* h, float* cs) {
+  tfcc::_MKLCellKernel<float>::processLSTMCell(batch, units, stateC, inputValue, stateHValue, bias, forget, h, cs);
+}
+void ref_gru_cell_gates(unsigned batch, unsigned units, unsigned inputSize, const float* state, const float* inputs,
+                        const float* value, const float* bias, float* result) {
+  tfcc::_MKLCellKernel<float>::processGRUCellGates(batch, units, inputSize, state, inputs, value, bias, result);
+}
+void ref_gru_cell_candidate(unsigned batch, unsigned units, const float* state, const float* value, const float* bias,
+                            const float* cValue, const float* cBias, float* result) {
+  tfcc::_MKLCellKernel<float>::processGRUCellCandidate(batch, units, state, value, bias, cValue, cBias, result);
+}
+void ref_pytorch_gru_cell(unsigned batch, unsigned units, const float* state, const float* inputValue,
+                          const float* stateValue, const float* gateBias, const float* candidateIBias,
+                          const float* candidateHBias, float* result) {
+  tfcc::_MKLCellKernel<float>::processPyTorchGRUCell(batch, units, state, inputValue, stateValue, gateBias,
+                                                     candidateIBias, candidateHBias, result);
+}
 
 }  // extern "C"

@@ -355,3 +355,88 @@ void oracle_gelu_accurate(const float* a, uint64_t total, float* out) {
     out[i] = (float)(0.5 * (double)v * (double)(1 + erff(v / 1.4142135623730951f)));
   }
 }
+
+/* ---- recurrent cells ------------------------------------------------------------------------- */
+
+static float oracle_sigmoid(float v) { return 1.f / (1.f + expf(0.f - v)); }
+
+void oracle_lstm_cell(unsigned batch, unsigned units, const float* stateC, const float* inputValue,
+                      const float* stateHValue, const float* bias, float forget, float* h, float* cs) {
+  for (unsigned b = 0; b < batch; ++b) {
+    const float* x = inputValue + (size_t)b * 4 * units;
+    const float* s = stateHValue + (size_t)b * 4 * units;
+    for (unsigned i = 0; i < units; ++i) {
+      float xi = x[i] + s[i] + bias[i];
+      float xc = x[i + units] + s[i + units] + bias[i + units];
+      float xf = x[i + 2 * units] + s[i + 2 * units] + bias[i + 2 * units];
+      float xo = x[i + 3 * units] + s[i + 3 * units] + bias[i + 3 * units];
+      xi = oracle_sigmoid(xi);
+      xc = tanhf(xc);
+      xf = oracle_sigmoid(xf + forget);
+      xo = oracle_sigmoid(xo);
+      float c = xc * xi + stateC[(size_t)b * units + i] * xf;
+      h[(size_t)b * units + i] = tanhf(c) * xo;
+      cs[(size_t)b * units + i] = c;
+    }
+  }
+}
+
+void oracle_gru_cell_gates(unsigned batch, unsigned units, unsigned inputSize, const float* state,
+                           const float* inputs, const float* value, const float* bias, float* result) {
+  for (unsigned b = 0; b < batch; ++b) {
+    float* r = result + (size_t)b * (inputSize + units);
+    memcpy(r, inputs + (size_t)b * inputSize, inputSize * sizeof(float));
+    for (unsigned i = 0; i < units; ++i)
+      r[inputSize + i] = oracle_sigmoid(value[(size_t)b * 2 * units + i] + bias[i]) * state[(size_t)b * units + i];
+  }
+}
+
+void oracle_gru_cell_candidate(unsigned batch, unsigned units, const float* state, const float* value,
+                               const float* bias, const float* cValue, const float* cBias, float* result) {
+  for (unsigned b = 0; b < batch; ++b)
+    for (unsigned i = 0; i < units; ++i) {
+      float u = oracle_sigmoid(value[(size_t)b * 2 * units + units + i] + bias[units + i]);
+      float c = tanhf(cValue[(size_t)b * units + i] + cBias[i]);
+      result[(size_t)b * units + i] = u * state[(size_t)b * units + i] + (1.f - u) * c;
+    }
+}
+
+void oracle_pytorch_gru_cell(unsigned batch, unsigned units, const float* state, const float* inputValue,
+                             const float* stateValue, const float* gateBias, const float* candidateIBias,
+                             const float* candidateHBias, float* result) {
+  for (unsigned b = 0; b < batch; ++b) {
+    const float* x = inputValue + (size_t)b * 3 * units;
+    const float* s = stateValue + (size_t)b * 3 * units;
+    for (unsigned i = 0; i < units; ++i) {
+      float r = oracle_sigmoid(x[i] + s[i] + gateBias[i]);
+      float z = oracle_sigmoid(x[i + units] + s[i + units] + gateBias[i + units]);
+      float ni = x[i + 2 * units] + candidateIBias[i];
+      float nh = s[i + 2 * units] + candidateHBias[i];
+      float n = tanhf(ni + r * nh);
+      result[(size_t)b * units + i] = n + z * (state[(size_t)b * units + i] - n);
+    }
+  }
+}
+
+void oracle_lstm_sequence(int backward, unsigned seq, unsigned batch, unsigned length, unsigned hidden,
+                          const float* a, const float* inputKernel, const float* stateKernel, const float* bias,
+                          const float* ih, const float* ic, float* out, float* h, float* c) {
+  const size_t state = (size_t)batch * hidden;
+  float* xv = (float*)malloc(state * 4 * sizeof(float));
+  float* hv = (float*)malloc(state * 4 * sizeof(float));
+  float* hprev = (float*)malloc(state * sizeof(float));
+  memcpy(hprev, ih, state * sizeof(float));
+  memcpy(c, ic, state * sizeof(float));
+  for (unsigned step = 0; step < seq; ++step) {
+    const unsigned t = backward ? seq - 1 - step : step;
+    oracle_sgemm_strided_batched(a + (size_t)t * batch * length, 0, inputKernel, 0, NULL, xv, NULL, 0, batch, 4 * hidden,
+                                 length, 1);
+    oracle_sgemm_strided_batched(hprev, 0, stateKernel, 0, NULL, hv, NULL, 0, batch, 4 * hidden, hidden, 1);
+    oracle_lstm_cell(batch, hidden, c, xv, hv, bias, 0.f, h, c);
+    memcpy(out + (size_t)step * state, h, state * sizeof(float));
+    memcpy(hprev, h, state * sizeof(float));
+  }
+  free(xv);
+  free(hv);
+  free(hprev);
+}

@@ -25,6 +25,13 @@
  *       mathematics (fp64 accumulation; identity / one-hot / all-ones /
  *       power-of-two cases; brute force) under the stated tolerance
  *       (relative Frobenius error <= 1e-5).
+ *   oracle_lstm_cell, oracle_gru_cell_*, oracle_pytorch_gru_cell
+ *       pinned by the reference's own scalar cell kernels (oracle/_ref, built from the reference
+ *       header) and by the formulas of the reference's test generators
+ *       (tfcc/test/python/testcase/rnn/lstmcell.py:31-44, pytorchgrucell.py) evaluated in float64.
+ *   oracle_lstm_sequence
+ *       pinned by the recurrence of tfcc/test/python/testcase/rnn/lstmforward.py:33-44,62-69 and
+ *       lstmbackward.py evaluated in float64, under the fp32 tolerance of the matrix products.
  */
 #ifndef TFCC_ORACLE_H_
 #define TFCC_ORACLE_H_
@@ -175,6 +182,33 @@ void oracle_layer_norm(const float* a, const float* gamma, const float* beta, fl
                        uint64_t rows, unsigned cols, float* out);
 /* 0.5*v*(1+erf(v/sqrt 2)): tfcc/mkl/kernel/tfcc_mklactivationkernel.hpp:213-220 */
 void oracle_gelu_accurate(const float* a, uint64_t total, float* out);
+
+/* ---- recurrent cells and the LSTM sequence that calls matmul once per time step -- */
+
+/* tfcc/mkl/kernel/tfcc_mklcellkernel.hpp:51-87 (gate order i, c, f, o; sigmoid :45-48) */
+void oracle_lstm_cell(unsigned batch, unsigned units, const float* stateC, const float* inputValue,
+                      const float* stateHValue, const float* bias, float forget, float* h, float* cs);
+/* tfcc/mkl/kernel/tfcc_mklcellkernel.hpp:89-133 */
+void oracle_gru_cell_gates(unsigned batch, unsigned units, unsigned inputSize, const float* state,
+                           const float* inputs, const float* value, const float* bias, float* result);
+/* tfcc/mkl/kernel/tfcc_mklcellkernel.hpp:135-158 */
+void oracle_gru_cell_candidate(unsigned batch, unsigned units, const float* state, const float* value,
+                               const float* bias, const float* cValue, const float* cBias, float* result);
+/* tfcc/mkl/kernel/tfcc_mklcellkernel.hpp:160-189 */
+void oracle_pytorch_gru_cell(unsigned batch, unsigned units, const float* state, const float* inputValue,
+                             const float* stateValue, const float* gateBias, const float* candidateIBias,
+                             const float* candidateHBias, float* result);
+/*
+ * tfcc::rnn::lstm_forward / lstm_backward, tfcc/core/operations/tfcc_rnn.cpp:29-81, 83-135:
+ * a [seq, batch, length], inputKernel [length, 4 hidden], stateKernel [hidden, 4 hidden], bias [4 hidden],
+ * ih / ic [batch, hidden]; per step matmul(x_t, inputKernel), matmul(h, stateKernel), LSTM cell with forget 0.
+ * backward != 0 walks the steps from the last to the first; outputs are stored in the order they are produced
+ * (:127-133 concatenates them in that order).  out [seq, batch, hidden], h and c [batch, hidden].
+ * The two products accumulate in double (the reference's sgemm is oneDNN's; see oracle_sgemm_strided_batched).
+ */
+void oracle_lstm_sequence(int backward, unsigned seq, unsigned batch, unsigned length, unsigned hidden,
+                          const float* a, const float* inputKernel, const float* stateKernel, const float* bias,
+                          const float* ih, const float* ic, float* out, float* h, float* c);
 
 #ifdef __cplusplus
 }

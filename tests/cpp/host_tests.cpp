@@ -480,6 +480,114 @@ static void test_layer_ops() {
   CHECK(std::fabs(mean) < 1e-5f);
 }
 
+// tfcc/test/rnn.cpp:126-175 with the generators of tfcc/test/python/testcase/rnn/lstmforward.py and
+// lstmbackward.py (seeded here): sequences of 1-7 steps, batch 1-4, 32-63 units and inputs; expectations
+// from the same recurrence in double.
+static void test_lstm_sequences() {
+  std::mt19937 rng(2024);
+  std::uniform_real_distribution<float> dist(-1.f, 1.f);
+  auto sig = [](double v) { return 1.0 / (1.0 + std::exp(-v)); };
+  for (int round = 0; round < 6; ++round) {
+    const bool backward = round % 2 == 1;
+    const unsigned seq = 1 + rng() % 7, batch = 1 + rng() % 4, hidden = 32 + rng() % 32, length = 32 + rng() % 32;
+    std::vector<float> ha(size_t(seq) * batch * length), wi(size_t(length) * 4 * hidden), wh(size_t(hidden) * 4 * hidden),
+        hb(4 * hidden), hih(size_t(batch) * hidden), hic(size_t(batch) * hidden);
+    for (auto* v : {&ha, &wi, &wh, &hb, &hih, &hic})
+      for (auto& x : *v) x = dist(rng);
+    std::vector<double> h(hih.begin(), hih.end()), c(hic.begin(), hic.end()), want;
+    for (unsigned step = 0; step < seq; ++step) {
+      const unsigned t = backward ? seq - 1 - step : step;
+      std::vector<double> nh(h.size()), nc(c.size());
+      for (unsigned b = 0; b < batch; ++b)
+        for (unsigned u = 0; u < hidden; ++u) {
+          double g[4];
+          for (unsigned q = 0; q < 4; ++q) {
+            double acc = hb[q * hidden + u];
+            for (unsigned p = 0; p < length; ++p)
+              acc += double(ha[(size_t(t) * batch + b) * length + p]) * wi[size_t(p) * 4 * hidden + q * hidden + u];
+            for (unsigned p = 0; p < hidden; ++p) acc += h[size_t(b) * hidden + p] * wh[size_t(p) * 4 * hidden + q * hidden + u];
+            g[q] = acc;
+          }
+          nc[size_t(b) * hidden + u] = std::tanh(g[1]) * sig(g[0]) + c[size_t(b) * hidden + u] * sig(g[2]);
+          nh[size_t(b) * hidden + u] = std::tanh(nc[size_t(b) * hidden + u]) * sig(g[3]);
+        }
+      h = nh;
+      c = nc;
+      want.insert(want.end(), h.begin(), h.end());
+    }
+    tfcc::Variable<float> a = tfcc::data::set(ha, {seq, batch, length}), ik = tfcc::data::set(wi, {length, 4 * hidden}),
+                          sk = tfcc::data::set(wh, {hidden, 4 * hidden}), bias = tfcc::data::set(hb, {4 * hidden}),
+                          ih = tfcc::data::set(hih, {batch, hidden}), ic = tfcc::data::set(hic, {batch, hidden});
+    tfcc::Variable<float> result, rh, rc;
+    std::tie(result, rh, rc) = backward ? tfcc::rnn::lstm_backward(a, ik, sk, bias, ih, ic)
+                                        : tfcc::rnn::lstm_forward(a, ik, sk, bias, ih, ic);
+    CHECK(result.shape() == tfcc::Shape({seq, batch, hidden}) && rh.shape() == ih.shape() && rc.shape() == ic.shape());
+    std::vector<float> got = tfcc::data::get(result), gh = tfcc::data::get(rh), gc = tfcc::data::get(rc);
+    bool ok = got.size() == want.size();
+    for (size_t i = 0; ok && i < got.size(); ++i) ok = is_similar(got[i], float(want[i]));
+    for (size_t i = 0; ok && i < gh.size(); ++i) ok = is_similar(gh[i], float(h[i])) && is_similar(gc[i], float(c[i]));
+    CHECK(ok);
+    // the checks of tfcc/core/operations/tfcc_rnn.cpp:33-53
+    tfcc::Variable<float> badBias({4 * hidden + 1}), badState({hidden + 1, 4 * hidden}), flat({seq * batch, length});
+    CHECK_THROWS_MSG(tfcc::rnn::lstm_forward(flat, ik, sk, bias, ih, ic), tfcc::InvalidArgumentError, "invalid input");
+    CHECK_THROWS_MSG(tfcc::rnn::lstm_forward(a, ik, sk, badBias, ih, ic), tfcc::InvalidArgumentError, "invalid bias");
+    CHECK_THROWS_MSG(tfcc::rnn::lstm_backward(a, ik, badState, bias, ih, ic), tfcc::InvalidArgumentError, "invalid state kernel");
+    if (length != hidden)
+      CHECK_THROWS_MSG(tfcc::rnn::lstm_forward(a, sk, sk, bias, ih, ic), tfcc::InvalidArgumentError, "invalid input kernel");
+    CHECK_THROWS_MSG(tfcc::rnn::lstm_forward(a, ik, sk, bias, ih, bias), tfcc::InvalidArgumentError, "invalid ih or ic");
+  }
+}
+
+// The four cells of tfcc/test/rnn.cpp:36-124 at the level of CellInterface: results against the formulas of the
+// interface's own documentation (tfcc/core/interfaces/tfcc_cellinterface.h:33-86) in double.
+static void test_cells() {
+  std::mt19937 rng(77);
+  std::uniform_real_distribution<float> dist(-2.f, 2.f);
+  auto sig = [](double v) { return 1.0 / (1.0 + std::exp(-v)); };
+  const unsigned batch = 3, units = 70, inputSize = 19;
+  auto make = [&](std::vector<unsigned> shape, std::vector<float>& host) {
+    size_t n = 1;
+    for (unsigned d : shape) n *= d;
+    host.resize(n);
+    for (auto& v : host) v = dist(rng);
+    return tfcc::data::set(host, tfcc::Shape(shape));
+  };
+  std::vector<float> hs, hx4, hh4, hb4, hx3, hh3, hb2, hv2, hin, hcv, hcb, hbi, hbh;
+  tfcc::Variable<float> state = make({batch, units}, hs), x4 = make({batch, 4 * units}, hx4), h4 = make({batch, 4 * units}, hh4),
+                        b4 = make({4 * units}, hb4), x3 = make({batch, 3 * units}, hx3), h3 = make({batch, 3 * units}, hh3),
+                        b2 = make({2 * units}, hb2), v2 = make({batch, 2 * units}, hv2), in = make({batch, inputSize}, hin),
+                        cv = make({batch, units}, hcv), cb = make({units}, hcb), bi = make({units}, hbi), bh = make({units}, hbh);
+  tfcc::CellInterface<float>& cell = tfcc::Operation<float>::getCurrentInterface().getCellInterface();
+  tfcc::Variable<float> h, cs;
+  std::tie(h, cs) = cell.processLSTMCell(state, x4, h4, b4, 1.0f);
+  std::vector<float> gh = tfcc::data::get(h), gcs = tfcc::data::get(cs), gates = tfcc::data::get(cell.processGRUCellGates(state, in, v2, b2)),
+                     cand = tfcc::data::get(cell.processGRUCellCandidate(state, v2, b2, cv, cb)),
+                     pt = tfcc::data::get(cell.processPyTorchGRUCell(state, x3, h3, b2, bi, bh));
+  bool ok = true;
+  for (unsigned b = 0; b < batch; ++b)
+    for (unsigned u = 0; u < units; ++u) {
+      auto pre4 = [&](unsigned q) { return double(hx4[b * 4 * units + q * units + u]) + hh4[b * 4 * units + q * units + u] + hb4[q * units + u]; };
+      const double c = std::tanh(pre4(1)) * sig(pre4(0)) + hs[b * units + u] * sig(pre4(2) + 1.0);
+      ok = ok && is_similar(gcs[b * units + u], float(c)) && is_similar(gh[b * units + u], float(std::tanh(c) * sig(pre4(3))));
+      const double r = sig(double(hv2[b * 2 * units + u]) + hb2[u]), z = sig(double(hv2[b * 2 * units + units + u]) + hb2[units + u]);
+      ok = ok && is_similar(gates[b * (inputSize + units) + inputSize + u], float(r * hs[b * units + u]));
+      ok = ok && is_similar(cand[b * units + u], float(z * hs[b * units + u] + (1 - z) * std::tanh(double(hcv[b * units + u]) + hcb[u])));
+      const double pr = sig(double(hx3[b * 3 * units + u]) + hh3[b * 3 * units + u] + hb2[u]);
+      const double pz = sig(double(hx3[b * 3 * units + units + u]) + hh3[b * 3 * units + units + u] + hb2[units + u]);
+      const double n = std::tanh(double(hx3[b * 3 * units + 2 * units + u]) + hbi[u] + pr * (double(hh3[b * 3 * units + 2 * units + u]) + hbh[u]));
+      ok = ok && is_similar(pt[b * units + u], float(n + pz * (hs[b * units + u] - n)));
+    }
+  for (unsigned b = 0; b < batch; ++b)
+    for (unsigned j = 0; j < inputSize; ++j) ok = ok && gates[b * (inputSize + units) + j] == hin[b * inputSize + j];
+  CHECK(ok);
+  CHECK_THROWS_MSG(cell.processLSTMCell(state, x3, h4, b4, 0.f), tfcc::InvalidArgumentError, "invalid inputValue");
+  CHECK_THROWS_MSG(cell.processLSTMCell(state, x4, h3, b4, 0.f), tfcc::InvalidArgumentError, "invalid stateHValue");
+  CHECK_THROWS_MSG(cell.processLSTMCell(b4, x4, h4, b4, 0.f), tfcc::InvalidArgumentError, "invalid stateC");
+  CHECK_THROWS_MSG(cell.processGRUCellGates(state, in, x4, b2), tfcc::InvalidArgumentError, "invalid value");
+  CHECK_THROWS_MSG(cell.processGRUCellCandidate(state, v2, b2, cv, b2), tfcc::InvalidArgumentError, "invalid cBias");
+  CHECK_THROWS_MSG(cell.processPyTorchGRUCell(state, x3, h3, b2, bi, b2), tfcc::InvalidArgumentError, "invalid candidateHBias");
+}
+
 // Two threads, each with a session (= stream) of its own on the shared device, running the same mix of
 // operations at the same time: fp32 matmul, quantize with its min/max reduction, quantized matmul.  Every
 // result is checked on the thread that produced it (tfcc/core/framework/tfcc_session.h:29,60-62: device
@@ -597,6 +705,8 @@ int main(int argc, char** argv) {
     run("quantization.rocm_matmul_exact", test_quantized_matmul_exact);
     run("layer.elementwise", test_layer_ops);
     run("layer.attention_permuted", test_attention_permuted);
+    run("rnn.cells", test_cells);
+    run("rnn.lstm_forward_backward", test_lstm_sequences);
     run("threads.two_sessions", test_two_sessions_on_two_threads);
   } else {
     run("blas.matmul_validation", [] {

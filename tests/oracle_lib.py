@@ -23,6 +23,22 @@ _f64p = np.ctypeslib.ndpointer(np.float64, flags="C")
 _u32p = np.ctypeslib.ndpointer(np.uint32, flags="C")
 
 
+def _bind_cells(lib, prefix):
+    """The four recurrent-cell entry points, which the oracle and the reference build share."""
+    f = getattr(lib, prefix + "lstm_cell")
+    f.restype = None
+    f.argtypes = [C.c_uint, C.c_uint, _f32p, _f32p, _f32p, _f32p, C.c_float, _f32p, _f32p]
+    f = getattr(lib, prefix + "gru_cell_gates")
+    f.restype = None
+    f.argtypes = [C.c_uint, C.c_uint, C.c_uint, _f32p, _f32p, _f32p, _f32p, _f32p]
+    f = getattr(lib, prefix + "gru_cell_candidate")
+    f.restype = None
+    f.argtypes = [C.c_uint, C.c_uint, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p]
+    f = getattr(lib, prefix + "pytorch_gru_cell")
+    f.restype = None
+    f.argtypes = [C.c_uint, C.c_uint, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p, _f32p]
+
+
 def build_oracle():
     """Compile the oracle with the Makefile beside it (a few seconds)."""
     subprocess.check_call(["make", "-s", "-C", ORACLE_DIR], stdout=subprocess.DEVNULL)
@@ -80,6 +96,9 @@ def _load_oracle():
     lib.oracle_layer_norm.argtypes = [_f32p, _f32p, _f32p, C.c_float, C.c_uint64, C.c_uint, _f32p]
     lib.oracle_gelu_accurate.restype = None
     lib.oracle_gelu_accurate.argtypes = [_f32p, C.c_uint64, _f32p]
+    _bind_cells(lib, "oracle_")
+    lib.oracle_lstm_sequence.restype = None
+    lib.oracle_lstm_sequence.argtypes = [C.c_int] + [C.c_uint] * 4 + [_f32p] * 9
     return lib
 
 
@@ -131,6 +150,7 @@ def ref():
             f = getattr(lib, "ref_quantize_" + name)
             f.restype = None
             f.argtypes = [_f32p, C.c_uint64, C.c_float, C.c_float, C.c_int, p]
+        _bind_cells(lib, "ref_")
         _ref = lib
     return _ref
 
@@ -308,3 +328,50 @@ def gelu_accurate(a):
     out = np.empty_like(a)
     oracle().oracle_gelu_accurate(a, a.size, out)
     return out
+
+
+def _f32(*arrays):
+    return [np.ascontiguousarray(a, np.float32) for a in arrays]
+
+
+def lstm_cell(state_c, input_value, state_h_value, bias, forget, lib=None, prefix="oracle_"):
+    state_c, input_value, state_h_value, bias = _f32(state_c, input_value, state_h_value, bias)
+    h, cs = np.empty_like(state_c), np.empty_like(state_c)
+    getattr(lib or oracle(), prefix + "lstm_cell")(state_c.shape[0], state_c.shape[1], state_c, input_value,
+                                                  state_h_value, bias, forget, h, cs)
+    return h, cs
+
+
+def gru_cell_gates(state, inputs, value, bias, lib=None, prefix="oracle_"):
+    state, inputs, value, bias = _f32(state, inputs, value, bias)
+    out = np.empty((state.shape[0], inputs.shape[1] + state.shape[1]), np.float32)
+    getattr(lib or oracle(), prefix + "gru_cell_gates")(state.shape[0], state.shape[1], inputs.shape[1], state,
+                                                       inputs, value, bias, out)
+    return out
+
+
+def gru_cell_candidate(state, value, bias, c_value, c_bias, lib=None, prefix="oracle_"):
+    state, value, bias, c_value, c_bias = _f32(state, value, bias, c_value, c_bias)
+    out = np.empty_like(state)
+    getattr(lib or oracle(), prefix + "gru_cell_candidate")(state.shape[0], state.shape[1], state, value, bias,
+                                                           c_value, c_bias, out)
+    return out
+
+
+def pytorch_gru_cell(state, input_value, state_value, gate_bias, ci_bias, ch_bias, lib=None, prefix="oracle_"):
+    arrays = _f32(state, input_value, state_value, gate_bias, ci_bias, ch_bias)
+    out = np.empty_like(arrays[0])
+    getattr(lib or oracle(), prefix + "pytorch_gru_cell")(arrays[0].shape[0], arrays[0].shape[1], *arrays, out)
+    return out
+
+
+def lstm_sequence(a, input_kernel, state_kernel, bias, ih, ic, backward=False):
+    """tfcc::rnn::lstm_forward / lstm_backward: (outputs [seq, batch, hidden], h, c)."""
+    a, input_kernel, state_kernel, bias, ih, ic = _f32(a, input_kernel, state_kernel, bias, ih, ic)
+    seq, batch, length = a.shape
+    hidden = ih.shape[1]
+    out = np.empty((seq, batch, hidden), np.float32)
+    h, c = np.empty_like(ih), np.empty_like(ih)
+    oracle().oracle_lstm_sequence(int(backward), seq, batch, length, hidden, a, input_kernel, state_kernel, bias,
+                                  ih, ic, out, h, c)
+    return out, h, c

@@ -487,6 +487,57 @@ def test_unary_functions_against_numpy_float64(pkg, T):
         pkg.check(pkg.lib().tfcc_rocm_unary_f32(None, 99, 16, 1, 16))
 
 
+@pytest.mark.parametrize("batch,units,input_size", [(1, 1, 1), (3, 67, 5), (4, 256, 64), (2, 511, 130), (64, 1024, 8)])
+def test_recurrent_cells_against_oracle(pkg, T, batch, units, input_size):
+    """The four cells of CellInterface against the scalar restatement of tfcc/mkl/kernel/tfcc_mklcellkernel.hpp:
+    same expressions, device expf / tanhf instead of libm's (a few ulp)."""
+    rng = np.random.default_rng(batch * 1000 + units)
+    u = lambda *s: rng.uniform(-1, 1, s).astype(np.float32)  # noqa: E731
+    state, c = u(batch, units), u(batch, units)
+    x4, h4, b4 = u(batch, 4 * units) * 3, u(batch, 4 * units) * 3, u(4 * units)
+    x3, h3, b2 = u(batch, 3 * units) * 3, u(batch, 3 * units) * 3, u(2 * units)
+    v2, inputs, cv, cb, bi, bh = u(batch, 2 * units) * 3, u(batch, input_size), u(batch, units) * 3, u(units), u(units), u(units)
+    tol = dict(rtol=2e-6, atol=2e-7)
+    for forget in (0.0, 1.0):
+        h, cs = pkg.lstm_cell(T.t(c), T.t(x4), T.t(h4), T.t(b4), forget)
+        wh, wc = O.lstm_cell(c, x4, h4, b4, forget)
+        assert np.allclose(T.n(h), wh, **tol) and np.allclose(T.n(cs), wc, **tol)
+    got = T.n(pkg.gru_cell_gates(T.t(state), T.t(inputs), T.t(v2), T.t(b2)))
+    assert np.array_equal(got[:, :input_size], inputs)
+    assert np.allclose(got, O.gru_cell_gates(state, inputs, v2, b2), **tol)
+    assert np.allclose(T.n(pkg.gru_cell_candidate(T.t(state), T.t(v2), T.t(b2), T.t(cv), T.t(cb))),
+                       O.gru_cell_candidate(state, v2, b2, cv, cb), **tol)
+    assert np.allclose(T.n(pkg.pytorch_gru_cell(T.t(state), T.t(x3), T.t(h3), T.t(b2), T.t(bi), T.t(bh))),
+                       O.pytorch_gru_cell(state, x3, h3, b2, bi, bh), **tol)
+    with pytest.raises(pkg.InvalidArgumentError, match="invalid inputValue"):
+        pkg.lstm_cell(T.t(c), T.t(x3), T.t(h4), T.t(b4), 0.0)
+    with pytest.raises(pkg.InvalidArgumentError, match="invalid cBias"):
+        pkg.gru_cell_candidate(T.t(state), T.t(v2), T.t(b2), T.t(cv), T.t(b2))
+
+
+def test_lstm_cell_in_place_state_and_sequence(pkg, T):
+    """The cell may write cs over stateC (each thread reads its element before writing it): a short sequence
+    driven through the C ABI the way tfcc::rnn::lstm_forward (tfcc/core/operations/tfcc_rnn.cpp:29-81) is,
+    against the oracle's sequence."""
+    import torch
+    rng = np.random.default_rng(8)
+    seq, batch, length, hidden = 6, 3, 48, 40
+    u = lambda *s: rng.uniform(-1, 1, s).astype(np.float32)  # noqa: E731
+    a, wi, wh, bias, ih, ic = u(seq, batch, length), u(length, 4 * hidden), u(hidden, 4 * hidden), u(4 * hidden), \
+        u(batch, hidden), u(batch, hidden)
+    want_out, want_h, want_c = O.lstm_sequence(a, wi, wh, bias, ih, ic)
+    xw = pkg.blas_matmul(T.t(a.reshape(seq * batch, length)), T.t(wi))
+    out = torch.empty((seq, batch, hidden), dtype=torch.float32, device=xw.device)
+    c, h, dwh, dbias = T.t(ic.copy()), T.t(ih), T.t(wh), T.t(bias)
+    for t in range(seq):
+        hv = pkg.blas_matmul(h, dwh)
+        pkg.check(pkg.lib().tfcc_rocm_lstm_cell_f32(None, batch, hidden, c.data_ptr(), xw[t * batch:].data_ptr(),
+                                                    hv.data_ptr(), dbias.data_ptr(), 0.0, out[t].data_ptr(), c.data_ptr()))
+        h = out[t]
+    for got, want in ((T.n(out), want_out), (T.n(h), want_h), (T.n(c), want_c)):
+        assert np.linalg.norm(got - want) <= 1e-5 * np.linalg.norm(want)
+
+
 def test_elementwise_against_oracle(pkg, T):
     rng = np.random.default_rng(50)
     for shape in ((8, 12, 128, 128), (7, 33), (5, 1000)):

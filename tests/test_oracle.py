@@ -384,3 +384,103 @@ def test_elementwise_against_numpy_double():
     ln = (xd - xd.mean(-1, keepdims=True)) / np.sqrt(xd.var(-1, keepdims=True) + 1e-12) * g + b
     assert np.allclose(O.layer_norm(x, g, b, 1e-12), ln, rtol=1e-4, atol=1e-5)
     assert np.allclose(O.gelu_accurate(x), 0.5 * xd * (1 + erf(xd / np.sqrt(2))), rtol=1e-5, atol=1e-6)
+
+
+# ---- recurrent cells -------------------------------------------------------------------------------
+
+def _sig(v):
+    return 1 / (1 + np.exp(-v))
+
+
+def cell_inputs(seed, batch, units, input_size):
+    rng = np.random.default_rng(seed)
+    u = lambda *s: rng.uniform(-1, 1, s).astype(np.float32)  # noqa: E731
+    return dict(state=u(batch, units), c=u(batch, units), x4=u(batch, 4 * units) * 3, h4=u(batch, 4 * units) * 3,
+                b4=u(4 * units), x3=u(batch, 3 * units) * 3, h3=u(batch, 3 * units) * 3, b2=u(2 * units),
+                v2=u(batch, 2 * units) * 3, inputs=u(batch, input_size), cv=u(batch, units) * 3, cb=u(units),
+                bi=u(units), bh=u(units))
+
+
+CELL_SHAPES = [(1, 1, 1), (3, 67, 5), (4, 256, 64), (2, 511, 130)]
+
+
+@pytest.mark.parametrize("batch,units,input_size", CELL_SHAPES)
+def test_cells_against_the_generator_formulas_in_double(batch, units, input_size):
+    """The closed forms of tfcc/test/python/testcase/rnn/lstmcell.py:31-44, grucell.py and pytorchgrucell.py,
+    evaluated in float64 on the pre-activations: a swapped gate, a dropped forget bias or a wrong bias segment
+    changes the result by far more than the tolerance."""
+    d = cell_inputs(batch * 1000 + units, batch, units, input_size)
+    D = {k: v.astype(np.float64) for k, v in d.items()}
+    for forget in (0.0, 1.0):
+        i, ci, f, o = np.split(D["x4"] + D["h4"] + D["b4"], 4, axis=1)
+        cs = np.tanh(ci) * _sig(i) + D["c"] * _sig(f + forget)
+        want_h = np.tanh(cs) * _sig(o)
+        h, c = O.lstm_cell(d["c"], d["x4"], d["h4"], d["b4"], forget)
+        assert np.allclose(h, want_h, rtol=1e-5, atol=1e-6) and np.allclose(c, cs, rtol=1e-5, atol=1e-6)
+    r = _sig(D["v2"][:, :units] + D["b2"][:units])
+    want = np.concatenate([D["inputs"], r * D["state"]], axis=1)
+    assert np.allclose(O.gru_cell_gates(d["state"], d["inputs"], d["v2"], d["b2"]), want, rtol=1e-5, atol=1e-6)
+    u = _sig(D["v2"][:, units:] + D["b2"][units:])
+    want = u * D["state"] + (1 - u) * np.tanh(D["cv"] + D["cb"])
+    assert np.allclose(O.gru_cell_candidate(d["state"], d["v2"], d["b2"], d["cv"], d["cb"]), want,
+                       rtol=1e-5, atol=1e-6)
+    g = _sig(D["x3"][:, :2 * units] + D["h3"][:, :2 * units] + D["b2"])
+    n = np.tanh(D["x3"][:, 2 * units:] + D["bi"] + g[:, :units] * (D["h3"][:, 2 * units:] + D["bh"]))
+    want = n + g[:, units:] * (D["state"] - n)
+    assert np.allclose(O.pytorch_gru_cell(d["state"], d["x3"], d["h3"], d["b2"], d["bi"], d["bh"]), want,
+                       rtol=1e-5, atol=1e-6)
+
+
+@needs_ref
+@pytest.mark.parametrize("batch,units,input_size", CELL_SHAPES)
+def test_cells_against_the_reference_kernels(batch, units, input_size):
+    """The reference's scalar cell kernels as compiled (oracle/_ref).  The two builds share libm, so the only
+    freedom left is contraction of a * b + c * d by the compiler: a few ulp."""
+    d = cell_inputs(batch * 7 + units, batch, units, input_size)
+    R = O.ref()
+    for forget in (0.0, 1.0):
+        got = O.lstm_cell(d["c"], d["x4"], d["h4"], d["b4"], forget)
+        want = O.lstm_cell(d["c"], d["x4"], d["h4"], d["b4"], forget, lib=R, prefix="ref_")
+        assert np.allclose(got[0], want[0], rtol=1e-6, atol=1e-7) and np.allclose(got[1], want[1], rtol=1e-6, atol=1e-7)
+    assert np.allclose(O.gru_cell_gates(d["state"], d["inputs"], d["v2"], d["b2"]),
+                       O.gru_cell_gates(d["state"], d["inputs"], d["v2"], d["b2"], lib=R, prefix="ref_"),
+                       rtol=1e-6, atol=1e-7)
+    assert np.allclose(O.gru_cell_candidate(d["state"], d["v2"], d["b2"], d["cv"], d["cb"]),
+                       O.gru_cell_candidate(d["state"], d["v2"], d["b2"], d["cv"], d["cb"], lib=R, prefix="ref_"),
+                       rtol=1e-6, atol=1e-7)
+    assert np.allclose(O.pytorch_gru_cell(d["state"], d["x3"], d["h3"], d["b2"], d["bi"], d["bh"]),
+                       O.pytorch_gru_cell(d["state"], d["x3"], d["h3"], d["b2"], d["bi"], d["bh"], lib=R, prefix="ref_"),
+                       rtol=1e-6, atol=1e-7)
+
+
+def lstm_sequence_double(a, wi, wh, bias, ih, ic, backward):
+    """tfcc/test/python/testcase/rnn/lstmforward.py:33-44,62-69 (lstmbackward.py:62-69 walks inputs[-i - 1]),
+    in float64."""
+    a, wi, wh, bias, h, c = (np.asarray(t, np.float64) for t in (a, wi, wh, bias, ih, ic))
+    outs = []
+    for step in range(a.shape[0]):
+        x = a[-step - 1] if backward else a[step]
+        i, ci, f, o = np.split(x @ wi + h @ wh + bias, 4, axis=1)
+        c = np.tanh(ci) * _sig(i) + c * _sig(f)
+        h = np.tanh(c) * _sig(o)
+        outs.append(h)
+    return np.stack(outs), h, c
+
+
+@pytest.mark.parametrize("backward", [False, True])
+@pytest.mark.parametrize("seq,batch,length,hidden", [(1, 1, 32, 32), (7, 4, 63, 50), (5, 3, 40, 33)])
+def test_lstm_sequence_against_the_generator_recurrence(seq, batch, length, hidden, backward):
+    rng = np.random.default_rng(seq * 100 + hidden)
+    u = lambda *s: rng.uniform(-1, 1, s).astype(np.float32)  # noqa: E731
+    a, wi, wh, bias, ih, ic = u(seq, batch, length), u(length, 4 * hidden), u(hidden, 4 * hidden), u(4 * hidden), \
+        u(batch, hidden), u(batch, hidden)
+    got = O.lstm_sequence(a, wi, wh, bias, ih, ic, backward)
+    want = lstm_sequence_double(a, wi, wh, bias, ih, ic, backward)
+    for g, w in zip(got, want):
+        assert np.linalg.norm(g - w) <= 1e-5 * np.linalg.norm(w)
+    # the last output row block is the final h; forward and backward differ unless the sequence is a palindrome
+    assert np.array_equal(got[0][-1], got[1])
+    if seq > 1:
+        other = O.lstm_sequence(a, wi, wh, bias, ih, ic, not backward)
+        assert not np.allclose(other[0], got[0])
+        assert np.array_equal(O.lstm_sequence(a[::-1], wi, wh, bias, ih, ic, not backward)[0], got[0])

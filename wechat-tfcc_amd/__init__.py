@@ -126,6 +126,10 @@ SYMBOLS = {
     "tfcc_rocm_transform2_f32": (_I, [_VP, _VP, _U64, _F, _F, _VP]),
     "tfcc_rocm_binary_f32": (_I, [_VP, _I, _VP, _VP, _U64, _U64, _VP]),
     "tfcc_rocm_transpose_f32": (_I, [_VP, _VP, C.POINTER(C.c_uint), C.POINTER(C.c_uint), _I, _VP]),
+    "tfcc_rocm_lstm_cell_f32": (_I, [_VP, _U, _U, _VP, _VP, _VP, _VP, _F, _VP, _VP]),
+    "tfcc_rocm_gru_cell_gates_f32": (_I, [_VP, _U, _U, _U, _VP, _VP, _VP, _VP, _VP]),
+    "tfcc_rocm_gru_cell_candidate_f32": (_I, [_VP, _U, _U, _VP, _VP, _VP, _VP, _VP, _VP]),
+    "tfcc_rocm_pytorch_gru_cell_f32": (_I, [_VP, _U, _U, _VP, _VP, _VP, _VP, _VP, _VP, _VP]),
 }
 
 _lib = None
@@ -518,6 +522,87 @@ def unary(name, a):
     a = a.contiguous()
     out = torch.empty_like(a)
     check(lib().tfcc_rocm_unary_f32(_stream(), UNARY[name], _ptr(a), a.numel(), _ptr(out)))
+    return out
+
+
+def lstm_cell(state_c, input_value, state_h_value, bias, forget):
+    """CellInterface::processLSTMCell (tfcc/mkl/interfaces/tfcc_mklcellinterface.cpp:33-63): (h, cs)."""
+    import torch
+    if state_c.dim() != 2:
+        raise InvalidArgumentError("invalid stateC")
+    batch, units = state_c.shape
+    if tuple(input_value.shape) != (batch, units * 4):
+        raise InvalidArgumentError("invalid inputValue")
+    if tuple(state_h_value.shape) != (batch, units * 4):
+        raise InvalidArgumentError("invalid stateHValue")
+    if tuple(bias.shape) != (units * 4,):
+        raise InvalidArgumentError("invalid bias")
+    state_c, input_value, state_h_value, bias = (t.contiguous() for t in (state_c, input_value, state_h_value, bias))
+    h, cs = torch.empty_like(state_c), torch.empty_like(state_c)
+    check(lib().tfcc_rocm_lstm_cell_f32(_stream(), batch, units, _ptr(state_c), _ptr(input_value),
+                                        _ptr(state_h_value), _ptr(bias), float(forget), _ptr(h), _ptr(cs)))
+    return h, cs
+
+
+def gru_cell_gates(state, inputs, value, bias):
+    """CellInterface::processGRUCellGates (tfcc/mkl/interfaces/tfcc_mklcellinterface.cpp:65-92)."""
+    import torch
+    if state.dim() != 2:
+        raise InvalidArgumentError("invalid state")
+    batch, units = state.shape
+    if inputs.dim() != 2 or inputs.shape[0] != batch:
+        raise InvalidArgumentError("invalid inputs")
+    if tuple(value.shape) != (batch, units * 2):
+        raise InvalidArgumentError("invalid value")
+    if tuple(bias.shape) != (units * 2,):
+        raise InvalidArgumentError("invalid bias")
+    state, inputs, value, bias = (t.contiguous() for t in (state, inputs, value, bias))
+    out = torch.empty((batch, inputs.shape[1] + units), dtype=state.dtype, device=state.device)
+    check(lib().tfcc_rocm_gru_cell_gates_f32(_stream(), batch, units, inputs.shape[1], _ptr(state), _ptr(inputs),
+                                             _ptr(value), _ptr(bias), _ptr(out)))
+    return out
+
+
+def gru_cell_candidate(state, value, bias, c_value, c_bias):
+    """CellInterface::processGRUCellCandidate (tfcc/mkl/interfaces/tfcc_mklcellinterface.cpp:94-125)."""
+    import torch
+    if state.dim() != 2:
+        raise InvalidArgumentError("invalid state")
+    batch, units = state.shape
+    if tuple(value.shape) != (batch, units * 2):
+        raise InvalidArgumentError("invalid value")
+    if tuple(bias.shape) != (units * 2,):
+        raise InvalidArgumentError("invalid bias")
+    if tuple(c_value.shape) != (batch, units):
+        raise InvalidArgumentError("invalid cValue")
+    if tuple(c_bias.shape) != (units,):
+        raise InvalidArgumentError("invalid cBias")
+    state, value, bias, c_value, c_bias = (t.contiguous() for t in (state, value, bias, c_value, c_bias))
+    out = torch.empty_like(state)
+    check(lib().tfcc_rocm_gru_cell_candidate_f32(_stream(), batch, units, _ptr(state), _ptr(value), _ptr(bias),
+                                                 _ptr(c_value), _ptr(c_bias), _ptr(out)))
+    return out
+
+
+def pytorch_gru_cell(state, input_value, state_value, gate_bias, candidate_i_bias, candidate_h_bias):
+    """CellInterface::processPyTorchGRUCell (tfcc/mkl/interfaces/tfcc_mklcellinterface.cpp:127-165)."""
+    import torch
+    if state.dim() != 2:
+        raise InvalidArgumentError("invalid state")
+    batch, units = state.shape
+    if tuple(input_value.shape) != (batch, units * 3):
+        raise InvalidArgumentError("invalid inputValue")
+    if tuple(state_value.shape) != (batch, units * 3):
+        raise InvalidArgumentError("invalid stateValue")
+    if tuple(gate_bias.shape) != (units * 2,):
+        raise InvalidArgumentError("invalid gateBias")
+    if tuple(candidate_i_bias.shape) != (units,):
+        raise InvalidArgumentError("invalid candidateIBias")
+    if tuple(candidate_h_bias.shape) != (units,):
+        raise InvalidArgumentError("invalid candidateHBias")
+    ts = [t.contiguous() for t in (state, input_value, state_value, gate_bias, candidate_i_bias, candidate_h_bias)]
+    out = torch.empty_like(ts[0])
+    check(lib().tfcc_rocm_pytorch_gru_cell_f32(_stream(), batch, units, *[_ptr(t) for t in ts], _ptr(out)))
     return out
 
 

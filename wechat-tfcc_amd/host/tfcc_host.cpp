@@ -473,6 +473,89 @@ class ROCMActivationInterface : public ActivationInterface<float> {
   }
 };
 
+// Checks and error texts of tfcc/mkl/interfaces/tfcc_mklcellinterface.cpp:33-165.
+class ROCMCellInterface : public CellInterface<float> {
+  static void check_lstm(const Tensor<float>& stateC, const Tensor<float>& inputValue, const Tensor<float>& stateHValue,
+                         const Tensor<float>& bias) {
+    if (stateC.shape().size() != 2) throw InvalidArgumentError("invalid stateC");
+    const unsigned batch = stateC.shape(0), units = stateC.shape(1);
+    if (inputValue.shape().size() != 2 || inputValue.shape(0) != batch || inputValue.shape(1) != units * 4)
+      throw InvalidArgumentError("invalid inputValue");
+    if (stateHValue.shape().size() != 2 || stateHValue.shape(0) != batch || stateHValue.shape(1) != units * 4)
+      throw InvalidArgumentError("invalid stateHValue");
+    if (bias.shape().size() != 1 || bias.shape(0) != units * 4) throw InvalidArgumentError("invalid bias");
+  }
+
+ public:
+  std::tuple<Variable<float>, Variable<float>> processLSTMCell(const Tensor<float>& stateC,
+                                                               const Tensor<float>& inputValue,
+                                                               const Tensor<float>& stateHValue,
+                                                               const Tensor<float>& bias, float forget) override {
+    check_lstm(stateC, inputValue, stateHValue, bias);
+    Variable<float> h(stateC.shape()), cs(stateC.shape());
+    check(tfcc_rocm_lstm_cell_f32(current_stream(), stateC.shape(0), stateC.shape(1), stateC.data(), inputValue.data(),
+                                  stateHValue.data(), bias.data(), forget, h.data(), cs.data()));
+    return std::make_tuple(std::move(h), std::move(cs));
+  }
+  void processLSTMCellInto(const Tensor<float>& stateC, const Tensor<float>& inputValue,
+                           const Tensor<float>& stateHValue, const Tensor<float>& bias, float forget, float* h,
+                           float* cs) override {
+    check_lstm(stateC, inputValue, stateHValue, bias);
+    check(tfcc_rocm_lstm_cell_f32(current_stream(), stateC.shape(0), stateC.shape(1), stateC.data(), inputValue.data(),
+                                  stateHValue.data(), bias.data(), forget, h, cs));
+  }
+  Variable<float> processGRUCellGates(const Tensor<float>& state, const Tensor<float>& inputs,
+                                      const Tensor<float>& value, const Tensor<float>& bias) override {
+    if (state.shape().size() != 2) throw InvalidArgumentError("invalid state");
+    const unsigned batch = state.shape(0), units = state.shape(1);
+    if (inputs.shape().size() != 2 || inputs.shape(0) != batch) throw InvalidArgumentError("invalid inputs");
+    if (value.shape().size() != 2 || value.shape(0) != batch || value.shape(1) != units * 2)
+      throw InvalidArgumentError("invalid value");
+    if (bias.shape().size() != 1 || bias.shape(0) != units * 2) throw InvalidArgumentError("invalid bias");
+    Variable<float> r({batch, inputs.shape(1) + units});
+    check(tfcc_rocm_gru_cell_gates_f32(current_stream(), batch, units, inputs.shape(1), state.data(), inputs.data(),
+                                       value.data(), bias.data(), r.data()));
+    return r;
+  }
+  Variable<float> processGRUCellCandidate(const Tensor<float>& state, const Tensor<float>& value,
+                                          const Tensor<float>& bias, const Tensor<float>& cValue,
+                                          const Tensor<float>& cBias) override {
+    if (state.shape().size() != 2) throw InvalidArgumentError("invalid state");
+    const unsigned batch = state.shape(0), units = state.shape(1);
+    if (value.shape().size() != 2 || value.shape(0) != batch || value.shape(1) != units * 2)
+      throw InvalidArgumentError("invalid value");
+    if (bias.shape().size() != 1 || bias.shape(0) != units * 2) throw InvalidArgumentError("invalid bias");
+    if (cValue.shape().size() != 2 || cValue.shape(0) != batch || cValue.shape(1) != units)
+      throw InvalidArgumentError("invalid cValue");
+    if (cBias.shape().size() != 1 || cBias.shape(0) != units) throw InvalidArgumentError("invalid cBias");
+    Variable<float> r(state.shape());
+    check(tfcc_rocm_gru_cell_candidate_f32(current_stream(), batch, units, state.data(), value.data(), bias.data(),
+                                           cValue.data(), cBias.data(), r.data()));
+    return r;
+  }
+  Variable<float> processPyTorchGRUCell(const Tensor<float>& state, const Tensor<float>& inputValue,
+                                        const Tensor<float>& stateValue, const Tensor<float>& gateBias,
+                                        const Tensor<float>& candidateIBias,
+                                        const Tensor<float>& candidateHBias) override {
+    if (state.shape().size() != 2) throw InvalidArgumentError("invalid state");
+    const unsigned batch = state.shape(0), units = state.shape(1);
+    if (inputValue.shape().size() != 2 || inputValue.shape(0) != batch || inputValue.shape(1) != units * 3)
+      throw InvalidArgumentError("invalid inputValue");
+    if (stateValue.shape().size() != 2 || stateValue.shape(0) != batch || stateValue.shape(1) != units * 3)
+      throw InvalidArgumentError("invalid stateValue");
+    if (gateBias.shape().size() != 1 || gateBias.shape(0) != units * 2) throw InvalidArgumentError("invalid gateBias");
+    if (candidateIBias.shape().size() != 1 || candidateIBias.shape(0) != units)
+      throw InvalidArgumentError("invalid candidateIBias");
+    if (candidateHBias.shape().size() != 1 || candidateHBias.shape(0) != units)
+      throw InvalidArgumentError("invalid candidateHBias");
+    Variable<float> r(state.shape());
+    check(tfcc_rocm_pytorch_gru_cell_f32(current_stream(), batch, units, state.data(), inputValue.data(),
+                                         stateValue.data(), gateBias.data(), candidateIBias.data(),
+                                         candidateHBias.data(), r.data()));
+    return r;
+  }
+};
+
 class ROCMNormalizationInterface : public NormalizationInterface<float> {
  public:
   Variable<float> layerNormalize(const Tensor<float>& a, const Tensor<float>& gamma, const Tensor<float>& beta,
@@ -605,6 +688,7 @@ ROCMDevice::ROCMDevice(unsigned index, std::unique_ptr<Allocator> allocator)
   _interfaces->f32.setNormalizationInterface(std::unique_ptr<NormalizationInterface<float>>(new ROCMNormalizationInterface()));
   _interfaces->f32.setBasicInterface(std::unique_ptr<BasicInterface<float>>(new ROCMBasicInterface()));
   _interfaces->f32.setArithmeticInterface(std::unique_ptr<ArithmeticInterface<float>>(new ROCMArithmeticInterface()));
+  _interfaces->f32.setCellInterface(std::unique_ptr<CellInterface<float>>(new ROCMCellInterface()));
   _interfaces->f32.setTransformationInterface(std::unique_ptr<TransformationInterface<float>>(new ROCMTransformationInterface()));
 }
 

@@ -122,6 +122,33 @@ class TransformationInterface {
   virtual Variable<T> transform2(const Tensor<T>&, T, T) { throw NotImplementedError(); }  // a / alpha + beta
 };
 
+// tfcc/core/interfaces/tfcc_cellinterface.h:23-88.  processLSTMCellInto is an addition for callers that own
+// the memory of a whole sequence: the same step written into h and cs ([batch, units] each; cs may be
+// stateC's own memory), so that a sequence needs neither a copy nor a concat per step.
+template <class T>
+class CellInterface {
+ public:
+  virtual ~CellInterface() {}
+  virtual std::tuple<Variable<T>, Variable<T>> processLSTMCell(const Tensor<T>&, const Tensor<T>&, const Tensor<T>&,
+                                                               const Tensor<T>&, T) {
+    throw NotImplementedError();
+  }
+  virtual void processLSTMCellInto(const Tensor<T>&, const Tensor<T>&, const Tensor<T>&, const Tensor<T>&, T, T*, T*) {
+    throw NotImplementedError();
+  }
+  virtual Variable<T> processGRUCellGates(const Tensor<T>&, const Tensor<T>&, const Tensor<T>&, const Tensor<T>&) {
+    throw NotImplementedError();
+  }
+  virtual Variable<T> processGRUCellCandidate(const Tensor<T>&, const Tensor<T>&, const Tensor<T>&, const Tensor<T>&,
+                                              const Tensor<T>&) {
+    throw NotImplementedError();
+  }
+  virtual Variable<T> processPyTorchGRUCell(const Tensor<T>&, const Tensor<T>&, const Tensor<T>&, const Tensor<T>&,
+                                            const Tensor<T>&, const Tensor<T>&) {
+    throw NotImplementedError();
+  }
+};
+
 template <class T>
 class Interface {
 #define TFCC_SUB_INTERFACE(NAME)                                                     \
@@ -139,6 +166,7 @@ class Interface {
   TFCC_SUB_INTERFACE(Basic)
   TFCC_SUB_INTERFACE(Arithmetic)
   TFCC_SUB_INTERFACE(Transformation)
+  TFCC_SUB_INTERFACE(Cell)
 #undef TFCC_SUB_INTERFACE
 };
 
@@ -360,6 +388,68 @@ Variable<T> layer_normalization(const Tensor<T>& a, const Tensor<T>& gamma, cons
 }
 
 }  // namespace nn
+
+namespace rnn {
+
+namespace detail {
+// tfcc::rnn::lstm_forward / lstm_backward (tfcc/core/operations/tfcc_rnn.cpp:29-81, 83-135): the same checks,
+// gate layout, forget bias 0 and output order (outputs in the order the steps are taken).  The products of the
+// inputs with inputKernel do not depend on the recurrence, so all steps share one matmul of [seq * batch, length];
+// each step then costs one matmul with stateKernel and one cell launch that writes h straight into its row block
+// of the result.
+template <class T>
+std::tuple<Variable<T>, Variable<T>, Variable<T>> lstm_sequence(bool backward, const Tensor<T>& a,
+                                                                const Tensor<T>& inputKernel,
+                                                                const Tensor<T>& stateKernel, const Tensor<T>& bias,
+                                                                const Tensor<T>& ih, const Tensor<T>& ic) {
+  if (a.shape().size() != 3) throw InvalidArgumentError("invalid input");
+  const unsigned seq = a.shape(0), batch = a.shape(1), length = a.shape(2);
+  if (ih.shape() != ic.shape() || ih.shape().size() != 2 || ih.shape(0) != batch)
+    throw InvalidArgumentError("invalid ih or ic");
+  const unsigned hidden = ih.shape(1);
+  if (inputKernel.shape().size() != 2 || inputKernel.shape(0) != length || inputKernel.shape(1) != hidden * 4)
+    throw InvalidArgumentError("invalid input kernel");
+  if (stateKernel.shape().size() != 2 || stateKernel.shape(0) != hidden || stateKernel.shape(1) != hidden * 4)
+    throw InvalidArgumentError("invalid state kernel");
+  if (bias.shape().size() != 1 || bias.shape(0) != 4 * hidden) throw InvalidArgumentError("invalid bias");
+  if (a.size() == 0 || hidden == 0) throw InvalidArgumentError("invalid input");
+
+  Interface<T>& interface = Operation<T>::getCurrentInterface();
+  View<T> flat(a, Shape({seq * batch, length}));
+  Variable<T> inputValues = interface.getBlasInterface().matmul(flat, inputKernel);  // [seq * batch, 4 hidden]
+  Variable<T> result({seq, batch, hidden});
+  Variable<T> c = interface.getDataInterface().copy(ic);
+  const size_t state = static_cast<size_t>(batch) * hidden;
+  View<T> h(ih);
+  for (unsigned step = 0; step < seq; ++step) {
+    const unsigned t = backward ? seq - 1 - step : step;
+    View<T> x(inputValues, inputValues.shape(), t * batch, (t + 1) * batch);
+    Variable<T> stateValues = interface.getBlasInterface().matmul(h, stateKernel);
+    interface.getCellInterface().processLSTMCellInto(c, x, stateValues, bias, static_cast<T>(0),
+                                                     result.data() + step * state, c.data());
+    h = View<T>(result, result.shape(), step, step + 1);
+    h.reshape(Shape({batch, hidden}));
+  }
+  Variable<T> lastH = interface.getDataInterface().copy(h);
+  return std::make_tuple(std::move(result), std::move(lastH), std::move(c));
+}
+}  // namespace detail
+
+template <class T>
+std::tuple<Variable<T>, Variable<T>, Variable<T>> lstm_forward(const Tensor<T>& a, const Tensor<T>& inputKernel,
+                                                               const Tensor<T>& stateKernel, const Tensor<T>& bias,
+                                                               const Tensor<T>& ih, const Tensor<T>& ic) {
+  return detail::lstm_sequence(false, a, inputKernel, stateKernel, bias, ih, ic);
+}
+
+template <class T>
+std::tuple<Variable<T>, Variable<T>, Variable<T>> lstm_backward(const Tensor<T>& a, const Tensor<T>& inputKernel,
+                                                                const Tensor<T>& stateKernel, const Tensor<T>& bias,
+                                                                const Tensor<T>& ih, const Tensor<T>& ic) {
+  return detail::lstm_sequence(true, a, inputKernel, stateKernel, bias, ih, ic);
+}
+
+}  // namespace rnn
 
 namespace base {
 
