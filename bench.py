@@ -275,6 +275,10 @@ def bench_other(torch, pkg, dev, steps, warmup, c3):
 
     attention_case("c2_fp32_attention_one_launch_16x12x128x64", 16, 12, 128, 64)
     sgemm_case("fp32_4096x4096x4096", (4096, 4096), (4096, 4096), False, sets=1)
+    # up to eight rows of A in fp32 (C5's shape and a square weight): one streaming pass over B
+    sgemm_case("fp32_few_rows_m1_4096x11008", (1, 4096), (4096, 11008), False, sets=2)
+    sgemm_case("fp32_few_rows_m8_4096x11008", (8, 4096), (4096, 11008), False, sets=2)
+    sgemm_case("fp32_few_rows_m8_4096x4096", (8, 4096), (4096, 4096), False, sets=4)
     # what the fp32 matrix cores sustain alone (register-resident loop of the 4096^3 instruction count)
     probe_out = torch.empty(1024 * 256, dtype=torch.int32, device=dev)
     for label, changing in (("changing", 1),):

@@ -274,7 +274,9 @@ int tfcc_rocm_softmax_div_f32(void* stream, const float* in, uint64_t rows, unsi
  * (tfcc_runtime/operations/math/matmul.cpp:27-41, softmax.cpp, base/transpose.cpp) and returns what
  * tfcc_rocm_sgemm_general (trans_b) + tfcc_rocm_softmax_div_f32 + tfcc_rocm_sgemm_general return, bit
  * for bit.  Limits: t <= 128, d <= 64 and a multiple of 4, input strides multiples of 4, inputs 16-byte
- * aligned; tfcc_rocm_attention_f32_supported() tells (1 / 0) whether a descriptor is within them.
+ * aligned, and not a single head (batch_outer * batch_inner == 1) of s <= 8 rows, whose separate product
+ * runs on the streaming kernel for short A and sums in another order;
+ * tfcc_rocm_attention_f32_supported() tells (1 / 0) whether a descriptor is within them.
  * out must not overlap the inputs. */
 typedef struct tfcc_rocm_attention_desc {
   const float* q;

@@ -58,7 +58,8 @@ CASES = [
     (2, 12, 128, 128, 64, 8.0, "bshd"),     # the encoder layer's attention core
     (1, 3, 100, 77, 36, 6.0, "bshd"),       # ragged everywhere, head width not a multiple of 8
     (2, 2, 200, 128, 64, None, "bhsd"),     # several row blocks, no divisor, dense per-head matrices
-    (1, 1, 1, 1, 4, 2.0, "bhsd"),           # the smallest
+    (1, 2, 1, 1, 4, 2.0, "bhsd"),           # the smallest: one query, one key, two heads
+    (1, 1, 9, 3, 8, 2.0, "bhsd"),           # a single head of more than eight rows
     (3, 5, 64, 5, 4, 0.5, "bshd"),
     (1, 4, 65, 64, 32, 5.656854, "bhsd"),   # one row past a block; only the first column half is live
     (1, 2, 31, 97, 60, 7.75, "bshd"),
@@ -112,3 +113,9 @@ def test_attention_limits_are_reported(pkg, gpu):
             pkg.attention(bad)
     with pytest.raises(pkg.TfccRocmError):
         pkg.attention(pkg.attention_desc(x, x, x, x, 0, 16, 8, (8,) * 4))
+    # a lone head of at most eight query rows: the separate product takes the streaming kernel, whose sums are
+    # ordered differently, so the fused kernel declines rather than differ in the last bit
+    assert not pkg.attention_supported(pkg.attention_desc(x, x, x, x, 8, 16, 8, (8,) * 4))
+    assert pkg.attention_supported(pkg.attention_desc(x, x, x, x, 9, 16, 8, (8,) * 4))
+    assert pkg.attention_supported(pkg.attention_desc(x, x, x, x, 8, 16, 8, (8,) * 4, batch_outer=2,
+                                                      strides=(1024,) * 4))

@@ -41,6 +41,54 @@ def test_sgemm_around_configuration_thresholds(pkg, T, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [
+    # up to eight rows of A: the streaming kernel.  32 columns per wavefront below N = 8192, 64 from there on;
+    # K below, at and past one 64-row chunk per wavefront (16 * 64 = 1024), ragged chunk tails, ragged N edges
+    (1, 1, 1), (1, 64, 64), (2, 65, 63), (3, 31, 1000), (4, 4096, 1024), (5, 100, 1025), (8, 3072, 768),
+    (8, 33, 2049), (7, 8192, 96), (8, 8200, 130), (1, 11008, 512), (6, 8191, 70),
+    # nine rows: back on the tiled kernels
+    (9, 3072, 768),
+])
+def test_sgemm_with_few_rows(pkg, T, m, n, k):
+    import torch
+    print("sgemv", m, n, k, flush=True)
+    rng = np.random.default_rng(m * 3 + n * 5 + k)
+    a = rng.normal(0, 1, (m, k)).astype(np.float32)
+    b = rng.normal(0, 1, (k, n)).astype(np.float32)
+    bias = rng.uniform(-1, 1, n).astype(np.float32)
+    res = rng.normal(0, 1, (m, n)).astype(np.float32)
+    want = a.astype(np.float64) @ b.astype(np.float64)
+    ta, tb, tbias, tres = T.t(a), T.t(b), T.t(bias), T.t(res)
+    plain = T.n(pkg.blas_matmul(ta, tb))
+    assert rel_fro(plain, want) <= FP32_TOL
+    assert np.abs(plain - want).max() <= 1e-4 * max(1.0, np.abs(want).max())
+    with_bias = T.n(pkg.blas_matmul(ta, tb, tbias))
+    assert np.array_equal(with_bias, plain + bias)  # the bias is added to the finished sum
+    # bias + residual + GELU in the same launch: the same bits as the separate kernels give
+    out = torch.empty((m, n), dtype=torch.float32, device=ta.device)
+    pkg.check(pkg.lib().tfcc_rocm_sgemm_fused(None, ta.data_ptr(), 0, tb.data_ptr(), 0, tbias.data_ptr(),
+                                              tres.data_ptr(), 0, out.data_ptr(), 0, m, n, k, 1, 1))
+    separate = T.n(pkg.gelu_accurate(pkg.add(pkg.blas_matmul(ta, tb, tbias), tres)))
+    assert np.array_equal(T.n(out), separate)
+    # three products that share A in one launch: each as on its own
+    bs = [tb, T.t(b[:, ::-1].copy()), T.t((b * 0.5).astype(np.float32))]
+    grouped = pkg.sgemm_grouped(ta, bs, [tbias, tbias, tbias])
+    for g, bb in zip(grouped, bs):
+        assert np.array_equal(T.n(g), T.n(pkg.blas_matmul(ta, bb, tbias)))
+    # a strided A and C (rows further apart than their length) through the general entry point
+    lda, ldc = k + 3, n + 5
+    a_wide = np.zeros((m, lda), np.float32)
+    a_wide[:, :k] = a
+    c_wide = torch.full((m, ldc), 7.0, dtype=torch.float32, device=ta.device)
+    pkg.sgemm_general(T.t(a_wide), tb, c_wide, m, n, k, lda, n, ldc)
+    got = T.n(c_wide)
+    assert np.all(got[:, n:] == 7.0)
+    if m <= 8:
+        assert np.array_equal(got[:, :n], plain)  # the streaming kernel does not care about alignment
+    else:
+        assert rel_fro(got[:, :n], want) <= FP32_TOL  # unaligned rows: another tiled kernel, another order of sums
+
+
+@pytest.mark.parametrize("m,n,k", [
     # direct-to-LDS kernel: 256x256 tiles from 192 tiles on, 128x128 below; K not a multiple of the 128-byte slab
     (256 * 12, 256 * 16, 144), (256 * 12 - 1, 256 * 16, 144), (256 * 11, 256 * 16, 272), (512, 384, 4000),
     # 64x128 tiles below 128 tiles of 128x128 (1024 x 768 has 48), 128x128 from there on; ragged edges

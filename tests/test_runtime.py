@@ -373,6 +373,52 @@ def test_unary_nodes_against_numpy_float64(mf, rt, dev):
     assert np.array_equal(res[outs["Neg"]], 0 - xv) and np.array_equal(res[outs["Sign"]], np.sign(xv))
 
 
+def bidirectional_lstm_graph(mf, rng, seq, batch, length, hidden, hidden_field=None):
+    u = lambda *s: rng.uniform(-1, 1, s).astype(np.float32)  # noqa: E731
+    w = dict(ik=u(2, length, 4 * hidden), sk=u(2, hidden, 4 * hidden), bias=u(2, 4 * hidden), ih=u(2, batch, hidden),
+             ic=u(2, batch, hidden))
+    g = mf.GraphBuilder("g")
+    x = g.input("x", mf.FLOAT, [seq, batch, length])
+    ins = [x] + [g.constant(k, w[k]) for k in ("ik", "sk", "bias", "ih", "ic")]
+    outs = [g.variable(n) for n in ("fo", "bo", "fh", "bh", "fc", "bc")]
+    g.node("rnn.BidirectionalLSTM", ins, outs, mf.f_varint(1, hidden if hidden_field is None else hidden_field))
+    for o in outs:
+        g.output(o)
+    return g, w, outs
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("seq,batch,length,hidden", [(5, 2, 24, 16), (1, 1, 32, 32), (9, 4, 50, 61)])
+def test_bidirectional_lstm_node_against_oracle(mf, rt, dev, seq, batch, length, hidden):
+    """tfcc_runtime/operations/rnn/bidirectionallstm.cpp:27-66: direction 0 of every weight runs lstm_forward,
+    direction 1 lstm_backward, over the same input."""
+    rng = np.random.default_rng(seq * 10 + hidden)
+    g, w, outs = bidirectional_lstm_graph(mf, rng, seq, batch, length, hidden)
+    xv = rng.uniform(-1, 1, (seq, batch, length)).astype(np.float32)
+    res = rt.Model(mf.write_model([g], "g")).run({"x": xv})
+    for d, backward in ((0, False), (1, True)):
+        want = O.lstm_sequence(xv, w["ik"][d], w["sk"][d], w["bias"][d], w["ih"][d], w["ic"][d], backward)
+        for got, wnt in zip((res[outs[0 + d]], res[outs[2 + d]], res[outs[4 + d]]), want):
+            assert got.shape == wnt.shape
+            assert rel_frobenius(got, wnt) <= 1e-5
+
+
+def test_bidirectional_lstm_node_accept_rules(mf, rt):
+    """hidden_size 0 and wrong input / output counts are refused when the graph is built
+    (tfcc_runtime/operations/rnn/bidirectionallstm.cpp:81-98): nobody takes the node."""
+    rng = np.random.default_rng(1)
+    g, _, _ = bidirectional_lstm_graph(mf, rng, 2, 1, 8, 8, hidden_field=0)
+    with pytest.raises(rt.RuntimeError_, match="(?i)unknow"):
+        rt.Model(mf.write_model([g], "g")).run({"x": np.zeros((2, 1, 8), np.float32)})
+    g = mf.GraphBuilder("g")
+    x = g.input("x", mf.FLOAT, [2, 1, 8])
+    out = g.variable("o")
+    g.node("rnn.BidirectionalLSTM", [x], [out], mf.f_varint(1, 8))
+    g.output(out)
+    with pytest.raises(rt.RuntimeError_, match="(?i)unknow"):
+        rt.Model(mf.write_model([g], "g")).run({"x": np.zeros((2, 1, 8), np.float32)})
+
+
 @pytest.mark.gpu
 def test_matmul_nodes_of_other_dtypes_fail_at_run_time(mf, rt, dev):
     """accepted when the graph is built, NotImplementedError when run - as on the reference's

@@ -274,6 +274,8 @@ __global__ __launch_bounds__(kThreads, 4) void attention_kernel(const AttentionP
 
 const char* unsupported(const tfcc_rocm_attention_desc* d) {
   if (d->t > (unsigned)kMaxT) return "more than 128 key rows";
+  // a lone product of at most eight rows runs on the streaming kernel (sgemv.hip), whose sums are ordered differently
+  if (d->s <= 8 && (unsigned long long)d->batch_outer * d->batch_inner == 1) return "a single head of at most eight query rows";
   if (d->d > (unsigned)kMaxD) return "head width above 64";
   if (d->d % 4 != 0) return "head width not a multiple of 4";
   if (d->ldq % 4 || d->ldk % 4 || d->ldv % 4) return "row stride not a multiple of 4 elements";

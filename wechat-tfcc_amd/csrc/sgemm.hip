@@ -385,6 +385,10 @@ int dispatch(hipStream_t s, const SgemmParams& p, bool vec, bool tb, unsigned fi
                  rowsB * ldb < (1ull << 32), "sgemm: operand larger than 2^32 elements");
     return launch<2, 2, 1, 1, false, 1, true>(s, p);
   }
+  // One product (or a few that share A) of at most eight rows: a single pass over B decides the time, and the
+  // streaming kernel makes it without tiles.  A true batch keeps the tiled kernels, whose sums the fused attention
+  // kernel reproduces bit for bit.
+  if (fillBatch == 1 && sgemm_detail::sgemv_supported(p)) return sgemm_detail::sgemv_launch(s, p);
   // 128x128 tiles once there are enough of them to fill the 256 CUs twice over, else 64x64
   const unsigned long long big = (unsigned long long)((m + 127) / 128) * ((n + 127) / 128) * fillBatch;
   if (vec) {

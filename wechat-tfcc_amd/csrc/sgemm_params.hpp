@@ -46,5 +46,9 @@ bool sgemm_dma_available(int config, int ksplit);
 // (same additions, same result) - for launches that fill the chip anyway.
 int sgemm_dma_launch(hipStream_t stream, SgemmParams p, int config, int ksplit, bool serialGroups);
 
+// The streaming kernel for up to eight rows of A (sgemv.hip): any K, N, strides and alignment; B not transposed.
+bool sgemv_supported(const SgemmParams& p);
+int sgemv_launch(hipStream_t stream, const SgemmParams& p);
+
 }  // namespace sgemm_detail
 }  // namespace tfcc_rocm

@@ -1,0 +1,142 @@
+// fp32 matmul for up to eight rows of A (one decode step, one recurrent step): the product is bound by the single
+// pass over B, so it runs on the vector ALUs with B streamed straight from memory and no tile staging.
+//
+// A workgroup of sixteen wavefronts owns 64 (or 32) columns.  Wavefront w walks rows [w * per, (w + 1) * per) of B
+// in chunks of 64, one column per lane (a row of B is read as 256 contiguous bytes per wavefront, or two rows as
+// 128 bytes each), eight rows in flight per lane, and keeps one accumulator per row of A.  The values of A are the
+// same for every lane of a group: they go through a piece of LDS private to the wavefront.  The partial sums of
+// an element are then added in a fixed order (wavefronts ascending, lane groups ascending) through LDS, so a
+// result does not depend on timing.  Bias, residual and the erf-form GELU follow with the expressions of the tiled
+// kernels' epilogue (sgemm.hip), which are those of tfcc::blas::matmul(a, b, bias) on the reference's CPU device
+// (tfcc/mkl/interfaces/tfcc_mklblasinterface.cpp:127-190) followed by its element-wise kernels.
+#include "sgemm_params.hpp"
+
+namespace tfcc_rocm {
+namespace {
+
+using sgemm_detail::SgemmParams;
+
+constexpr int kWaves = 16;  // wavefronts of a workgroup, each with its own range of K
+constexpr int kRows = 8;    // rows of B a lane has in flight
+constexpr int kChunk = 64;  // rows of K whose values of A a wavefront holds in LDS at a time
+
+// COLS columns per wavefront (64 or 32): the 64 / COLS groups of COLS lanes take consecutive pieces of each
+// 64-row chunk, so a narrow B still spreads over many workgroups while every load covers whole 128-byte lines.
+template <int MR, int COLS>
+__global__ __launch_bounds__(kWaves * 64) void sgemv_kernel(SgemmParams p) {
+  constexpr int SUBS = 64 / COLS;       // lane groups of a wavefront
+  constexpr int PIECE = kChunk / SUBS;  // rows of a chunk per lane group
+  static_assert(PIECE % kRows == 0, "whole batches of rows per lane group");
+  // [wave][row of A][64]: first each wavefront's current 64 values of every row of A, at the end its partial sums
+  __shared__ __attribute__((aligned(16))) float smem[kWaves][MR][64];
+  const unsigned lane = threadIdx.x & 63;
+  const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const unsigned sub = lane / COLS, lcol = lane % COLS;
+  const unsigned bi = blockIdx.y;
+  const unsigned M = p.M, N = p.N, K = p.K;
+  const unsigned bo = bi / p.batchInner, bn = bi - bo * p.batchInner;
+  const float* __restrict__ A = p.A + (size_t)bo * p.strideA + (size_t)bn * p.innerA;
+  const float* __restrict__ B = p.B + (size_t)bo * p.strideB + (size_t)bn * p.innerB;
+  const float* biasPtr = p.bias;
+  float* Cbase = p.C + (size_t)bo * p.strideC + (size_t)bn * p.innerC;
+  if (p.groups) {
+    B = bi == 0 ? p.groupB[0] : bi == 1 ? p.groupB[1] : bi == 2 ? p.groupB[2] : p.groupB[3];
+    biasPtr = bi == 0 ? p.groupBias[0] : bi == 1 ? p.groupBias[1] : bi == 2 ? p.groupBias[2] : p.groupBias[3];
+    Cbase = bi == 0 ? p.groupC[0] : bi == 1 ? p.groupC[1] : bi == 2 ? p.groupC[2] : p.groupC[3];
+  }
+  const unsigned lda = p.lda, ldb = p.ldb, ldc = p.ldc;
+  const unsigned col = blockIdx.x * COLS + lcol;
+  const unsigned colRead = col < N ? col : N - 1;  // lanes past the edge read a valid column and drop the sum
+
+  // rows of A beyond M repeat the last one; their sums are never stored
+  const float* __restrict__ arow[MR];
+#pragma unroll
+  for (int m = 0; m < MR; ++m) arow[m] = A + (size_t)((unsigned)m < M ? m : M - 1) * lda;
+
+  const unsigned per = ((K + kWaves * kChunk - 1) / (kWaves * kChunk)) * kChunk;
+  const unsigned k0 = min(K, wave * per), k1 = min(K, k0 + per);
+  float acc[MR];
+#pragma unroll
+  for (int m = 0; m < MR; ++m) acc[m] = 0.f;
+
+  // Lane l fetches value l of every row of A for the chunk; each lane group then reads its piece back, four
+  // values per instruction.  The piece of LDS is this wavefront's own: no barrier is involved.
+  float (*mine)[64] = smem[wave];
+  for (unsigned k = k0; k < k1; k += kChunk) {
+    const unsigned rows = min((unsigned)kChunk, k1 - k);
+#pragma unroll
+    for (int m = 0; m < MR; ++m) mine[m][lane] = lane < rows ? arow[m][k + lane] : 0.f;
+    const float* __restrict__ bp = B + (size_t)(k + sub * PIECE) * ldb + colRead;
+    if (rows == (unsigned)kChunk) {
+#pragma unroll
+      for (int r = 0; r < PIECE; r += kRows) {
+        float b[kRows];
+#pragma unroll
+        for (int u = 0; u < kRows; ++u) b[u] = bp[(size_t)(r + u) * ldb];
+#pragma unroll
+        for (int m = 0; m < MR; ++m) {
+#pragma unroll
+          for (int q = 0; q < kRows; q += 4) {
+            const float4 a4 = *reinterpret_cast<const float4*>(&mine[m][sub * PIECE + r + q]);
+            acc[m] = fmaf(a4.x, b[q], acc[m]);
+            acc[m] = fmaf(a4.y, b[q + 1], acc[m]);
+            acc[m] = fmaf(a4.z, b[q + 2], acc[m]);
+            acc[m] = fmaf(a4.w, b[q + 3], acc[m]);
+          }
+        }
+      }
+    } else {
+      for (unsigned r = 0; r < (unsigned)PIECE && sub * PIECE + r < rows; ++r) {
+        const float b = bp[(size_t)r * ldb];
+#pragma unroll
+        for (int m = 0; m < MR; ++m) acc[m] = fmaf(mine[m][sub * PIECE + r], b, acc[m]);
+      }
+    }
+  }
+
+#pragma unroll
+  for (int m = 0; m < MR; ++m) smem[wave][m][lane] = acc[m];
+  __syncthreads();
+  // row m of the result: wavefront m adds the partial sums in wavefront order, lane groups in order within each
+  if (wave < (unsigned)MR && wave < M && lane < (unsigned)COLS && col < N) {
+    float v = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w)
+#pragma unroll
+      for (int g = 0; g < SUBS; ++g) v += smem[w][wave][g * COLS + lane];
+    if (biasPtr) v += biasPtr[col];
+    if (p.residual) v += p.residual[(size_t)bi * p.strideR + (size_t)wave * N + col];
+    if (p.act == 1) v = (float)(0.5 * (double)v * (double)(1.0f + erff(v / 1.4142135623730951f)));
+    Cbase[(size_t)wave * ldc + col] = v;
+  }
+}
+
+template <int MR, int COLS>
+int launch_rows(hipStream_t stream, const SgemmParams& p) {
+  hipLaunchKernelGGL((sgemv_kernel<MR, COLS>), dim3((p.N + COLS - 1) / COLS, p.batch), dim3(kWaves * 64), 0, stream, p);
+  return check_launch("sgemv");
+}
+
+template <int COLS>
+int launch_width(hipStream_t stream, const SgemmParams& p) {
+  if (p.M == 1) return launch_rows<1, COLS>(stream, p);
+  if (p.M == 2) return launch_rows<2, COLS>(stream, p);
+  if (p.M <= 4) return launch_rows<4, COLS>(stream, p);
+  return launch_rows<8, COLS>(stream, p);
+}
+
+}  // namespace
+
+namespace sgemm_detail {
+
+bool sgemv_supported(const SgemmParams& p) { return p.M >= 1 && p.M <= 8 && p.batch <= 65535u && p.N < (1u << 30); }
+
+// 64 columns per wavefront read B in the longest runs (5.7 TB/s at N = 11008); below 128 such column blocks too
+// few CUs take part, and 32 columns per wavefront with twice the workgroups are faster (17 against 23 us at
+// 4096 x 4096).  The choice depends on N alone, so that a product is summed the same way alone and in a group.
+int sgemv_launch(hipStream_t stream, const SgemmParams& p) {
+  return p.N >= 8192 ? launch_width<64>(stream, p) : launch_width<32>(stream, p);
+}
+
+}  // namespace sgemm_detail
+}  // namespace tfcc_rocm

@@ -9,9 +9,11 @@
 //   math.Abs / Erf / Log / Neg / Reciprocal / Relu / Rsqrt / Sigmoid / Sign / Softplus / Sqrt / Tanh
 //                                       operations/math/<name>.cpp
 //   nn.LayerNormalization               operations/nn/layernormalization.cpp:52-88
+//   rnn.BidirectionalLSTM               operations/rnn/bidirectionallstm.cpp:27-128
 //   base.Transpose, base.Reshape, base.Identity, base.CreateVector
 //                                       operations/base/transpose.cpp, reshape.cpp:27-59,74-104,
 //                                       identity.cpp, createvector.cpp:63-121
+#include <array>
 #include <cmath>
 #include <map>
 
@@ -429,6 +431,56 @@ class CreateVector : public TypedOperation<T> {
   }
 };
 
+// ---- rnn.BidirectionalLSTM ---------------------------------------------------------------------------------
+// tfcc_runtime/operations/rnn/bidirectionallstm.cpp:27-128: six inputs (a [seq, batch, length]; input kernel
+// [2, length, 4 hidden], state kernel [2, hidden, 4 hidden], bias [2, 4 hidden], initial h and c [2, batch, hidden],
+// index 0 the forward direction) and six outputs (forward / backward outputs, h, c); hidden_size 0 is refused.
+template <class T>
+class BidirectionalLSTM : public TypedOperation<T> {
+  static View<T> direction(const Tensor<T>& t, unsigned d) {
+    View<T> v(t, t.shape(), d, d + 1);
+    std::vector<unsigned> dims = t.shape().toVector();
+    dims.erase(dims.begin());
+    v.reshape(Shape(std::move(dims)));
+    return v;
+  }
+
+ public:
+  BidirectionalLSTM() : TypedOperation<T>("rnn.BidirectionalLSTM") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 6 || node.outputs.size() != 6) return false;
+    auto& sm = graph.getSymbolManager();
+    if (sm.getSymbolInfo(node.outputs[0]).dtype != this->DTYPE) return false;
+    uint64_t hiddenSize = 0;
+    wire::Reader r(node.operation);
+    uint32_t f, t;
+    while (r.next(f, t)) {
+      if (f == 1 && t == 0) hiddenSize = r.varint();
+      else r.skip(t);
+    }
+    if (hiddenSize == 0) return false;
+    const Tensor<T>* in[6];
+    Variable<T>* out[6];
+    for (int i = 0; i < 6; ++i) {
+      in[i] = sm.getTensor(node.inputs[i], T());
+      out[i] = sm.getVariable(node.outputs[i], T());
+    }
+    std::array<const Tensor<T>*, 6> i6{in[0], in[1], in[2], in[3], in[4], in[5]};
+    std::array<Variable<T>*, 6> o6{out[0], out[1], out[2], out[3], out[4], out[5]};
+    graph.addStep([i6, o6] {
+      for (unsigned d = 0; d < 2; ++d) {
+        for (int i = 1; i < 6; ++i)
+          if (i6[i]->shape().size() < 2 || i6[i]->shape(0) != 2) throw InvalidArgumentError("invalid shape");
+        View<T> ik = direction(*i6[1], d), sk = direction(*i6[2], d), bias = direction(*i6[3], d),
+                ih = direction(*i6[4], d), ic = direction(*i6[5], d);
+        std::tie(*o6[0 + d], *o6[2 + d], *o6[4 + d]) =
+            d == 0 ? rnn::lstm_forward(*i6[0], ik, sk, bias, ih, ic) : rnn::lstm_backward(*i6[0], ik, sk, bias, ih, ic);
+      }
+    });
+    return true;
+  }
+};
+
 class Collector {
   std::map<std::string, std::vector<std::unique_ptr<Operation>>> _operations;
 
@@ -462,6 +514,7 @@ class Collector {
     add(new Reshape<T, int64_t>());
     add(new Identity<T>());
     add(new CreateVector<T>());
+    add(new BidirectionalLSTM<T>());
   }
 
  public:
