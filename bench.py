@@ -478,7 +478,7 @@ def main():
                    "m": size, "n": size, "k": size},
         "roofline": {"bound": "mfma", "achieved": round(kernel_tops, 2), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                      "frac": round(kernel_tops / PEAK_INT8_TOPS, 4), "traffic": None,
-                     "kernel": "qgemm_dma_kernel<256,256,2,4,2,true,false>", "kernel_ms": round(kernel_ms, 5),
+                     "kernel": "qgemm_dma_kernel<256,256,2,4,2,true,false,true>", "kernel_ms": round(kernel_ms, 5),
                      "algorithmic_ops_per_launch": ops},
     }
     traffic_file = os.path.join(ROOT, "profiles", "traffic.json")
