@@ -14,6 +14,7 @@
 #include <string>
 #include <thread>
 
+#include "tfcc_layers.h"
 #include "tfcc_rocm_device.h"
 
 static int g_failures = 0;
@@ -588,6 +589,116 @@ static void test_cells() {
   CHECK_THROWS_MSG(cell.processPyTorchGRUCell(state, x3, h3, b2, bi, b2), tfcc::InvalidArgumentError, "invalid candidateHBias");
 }
 
+// Scopes, the npz loader, constants and configures on any device (tfcc/test/scope.cpp, framework.cpp).
+static void test_scopes_and_constants() {
+  CHECK(tfcc::Scope::getCurrentScope().getFullName() == "");
+  {
+    auto a = tfcc::Scope::scope("layer");
+    auto b = tfcc::Scope::scope("dense");
+    CHECK(tfcc::Scope::getCurrentScope().getFullName() == "layer/dense/");
+    CHECK(&tfcc::Scope::getRootScope().getChild("layer").getChild("dense") == &tfcc::Scope::getCurrentScope());
+    {
+      tfcc::ScopeGuard moved = tfcc::Scope::scope("0");
+      tfcc::ScopeGuard target(std::move(moved));  // only the target pops
+      CHECK(tfcc::Scope::getCurrentScope().getFullName() == "layer/dense/0/");
+      CHECK(tfcc::Configure<unsigned>::getConfigure("units") > 0);
+      CHECK(tfcc::Configure<unsigned>::getConfigure("absent", 5u) == 5u);
+      CHECK_THROWS(tfcc::Configure<unsigned>::getConfigure("absent"), tfcc::RuntimeError);
+      tfcc::Constant<float>& k = tfcc::Constant<float>::getConstant("dense/kernel");
+      CHECK(k.shape().size() == 2 && k.available() && k.data() != nullptr);
+      tfcc::Constant<float>& t = tfcc::Constant<float>::getConstant("dense/bias");
+      std::vector<float> bias = tfcc::data::get(t);
+      CHECK(bias.size() == k.shape(1));
+      // an integer view of a float array converts element by element (tfcc/core/utils/tfcc_commutils.cpp:411-436)
+      std::vector<int32_t> asInt = tfcc::data::get(tfcc::Constant<int32_t>::getConstant("dense/bias"));
+      bool same = asInt.size() == bias.size();
+      for (size_t i = 0; same && i < bias.size(); ++i) same = asInt[i] == static_cast<int32_t>(bias[i]);
+      CHECK(same);
+    }
+    CHECK(tfcc::Scope::getCurrentScope().getFullName() == "layer/dense/");
+    CHECK(tfcc::Configure<uint64_t>::getConfigure("__count__") >= 1);
+  }
+  CHECK(tfcc::Scope::getCurrentScope().getFullName() == "");
+  CHECK(tfcc::DataLoader::getGlobalDefault()->hasData("rnn/lstmcell/0/inputs"));
+  CHECK(!tfcc::DataLoader::getGlobalDefault()->hasData("rnn/lstmcell/0/nothing"));
+  CHECK(tfcc::DataLoader::getGlobalDefault()->getAllNames().size() > 10);
+}
+
+// is_similar over whole tensors, as tfcc::is_similar (tfcc/core/utils/tfcc_debugutils.cpp) is used by the
+// reference's tests
+static bool all_similar(const tfcc::Tensor<float>& a, const tfcc::Tensor<float>& b) {
+  if (a.shape() != b.shape()) return false;
+  std::vector<float> x = tfcc::data::get(a), y = tfcc::data::get(b);
+  for (size_t i = 0; i < x.size(); ++i)
+    if (!is_similar(x[i], y[i])) return false;
+  return true;
+}
+
+// tfcc/test/rnn.cpp:81-104, data named as tfcc/test/python/createtestdata.py names it
+// ("rnn/lstmcell/<i>/..."), generated by the Python side of this test with the formulas of
+// tfcc/test/python/testcase/rnn/lstmcell.py:31-44.
+static void test_lstmcell_from_constants() {
+  auto scope1 = tfcc::Scope::scope("rnn");
+  auto scope2 = tfcc::Scope::scope("lstmcell");
+  size_t count = tfcc::Configure<uint64_t>::getConfigure("__count__");
+  CHECK(count > 0);
+  for (size_t i = 0; i < count; ++i) {
+    auto scope3 = tfcc::Scope::scope(std::to_string(i));
+    unsigned units = tfcc::Configure<unsigned>::getConfigure("units");
+    tfcc::rnn::LSTMCell<float> cell(units);
+    tfcc::Constant<float>& inputs = tfcc::Constant<float>::getConstant("inputs");
+    tfcc::rnn::LSTMCell<float>::State state;
+    state.h = tfcc::data::copy(tfcc::Constant<float>::getConstant("h"));
+    state.cs = tfcc::data::copy(tfcc::Constant<float>::getConstant("cs"));
+    tfcc::Constant<float>& expect = tfcc::Constant<float>::getConstant("expect");
+    tfcc::Constant<float>& expectCs = tfcc::Constant<float>::getConstant("ecs");
+    tfcc::Variable<float> result;
+    tfcc::rnn::LSTMCell<float>::State nextState;
+    std::tie(result, nextState) = cell(inputs, state, 0, {});
+    CHECK(all_similar(result, expect));
+    CHECK(all_similar(nextState.h, expect));
+    CHECK(all_similar(nextState.cs, expectCs));
+    CHECK_THROWS(cell(inputs, state, 0, {1u, 2u, 3u, 4u, 5u, 6u, 7u}), tfcc::InvalidArgumentError);
+    // the same constant asked for again is the same object; under another scope it is looked up anew
+    CHECK(&tfcc::Constant<float>::getConstant("inputs") == &inputs);
+    auto other = tfcc::Scope::scope("nowhere");
+    const std::string missing = "Name: [rnn/lstmcell/" + std::to_string(i) + "/nowhere/inputs] not found in data loader";
+    CHECK_THROWS_MSG(tfcc::Constant<float>::getConstant("inputs"), tfcc::RuntimeError, missing.c_str());
+  }
+}
+
+// tfcc::layer::Dense (tfcc/core/layers/tfcc_denselayer.cpp:47-87) in the style of the reference's layer tests:
+// inputs of rank 2 and 3, with and without bias, custom constant names, and its checks.
+static void test_dense_from_constants() {
+  auto scope1 = tfcc::Scope::scope("layer");
+  auto scope2 = tfcc::Scope::scope("dense");
+  size_t count = tfcc::Configure<uint64_t>::getConfigure("__count__");
+  CHECK(count > 0);
+  for (size_t i = 0; i < count; ++i) {
+    auto scope3 = tfcc::Scope::scope(std::to_string(i));
+    unsigned units = tfcc::Configure<unsigned>::getConfigure("units");
+    tfcc::Constant<float>& inputs = tfcc::Constant<float>::getConstant("inputs");
+    CHECK(all_similar(tfcc::layer::dense(inputs, units, true), tfcc::Constant<float>::getConstant("expect")));
+    CHECK(all_similar(tfcc::layer::dense(inputs, 0u, false), tfcc::Constant<float>::getConstant("expect_nobias")));
+    CHECK(all_similar(tfcc::layer::dense(inputs, units, true, "other", "w", "b"), tfcc::Constant<float>::getConstant("expect_other")));
+    // with a bias the layer is one launch; it returns what matmul followed by the broadcast add returns
+    tfcc::layer::Dense<float> layer(units, true);
+    tfcc::Variable<float> fused = layer(inputs);
+    auto inner = tfcc::Scope::scope("dense");
+    tfcc::Variable<float> separate = tfcc::blas::matmul(inputs, tfcc::Constant<float>::getConstant("kernel")) +
+                                     tfcc::Constant<float>::getConstant("bias");
+    CHECK(tfcc::data::get(fused) == tfcc::data::get(separate));
+  }
+  auto scope3 = tfcc::Scope::scope("0");
+  tfcc::Constant<float>& inputs = tfcc::Constant<float>::getConstant("inputs");
+  CHECK_THROWS_MSG(tfcc::layer::dense(inputs, 7777u, true), tfcc::InvalidDataError, "kernel and units don't match");
+  CHECK_THROWS_MSG(tfcc::layer::dense(inputs, 0u, true, "dense", "bias", "bias"), tfcc::InvalidDataError, "invalid kernel");
+  CHECK_THROWS_MSG(tfcc::layer::dense(inputs, 0u, true, "dense", "kernel", "kernel"), tfcc::InvalidDataError, "invalid bias");
+  tfcc::Variable<float> flat({inputs.size()}), wrong({3, inputs.shape(inputs.shape().size() - 1) + 1});
+  CHECK_THROWS_MSG(tfcc::layer::dense(flat, 0u, true), tfcc::InvalidArgumentError, "invalid inputs");
+  CHECK_THROWS_MSG(tfcc::layer::dense(wrong, 0u, true), tfcc::InvalidArgumentError, "inputs and kernel don't match");
+}
+
 // Two threads, each with a session (= stream) of its own on the shared device, running the same mix of
 // operations at the same time: fp32 matmul, quantize with its min/max reduction, quantized matmul.  Every
 // result is checked on the thread that produced it (tfcc/core/framework/tfcc_session.h:29,60-62: device
@@ -707,6 +818,14 @@ int main(int argc, char** argv) {
     run("layer.attention_permuted", test_attention_permuted);
     run("rnn.cells", test_cells);
     run("rnn.lstm_forward_backward", test_lstm_sequences);
+    if (argc > 2) {  // an .npz of named test data, written by the Python side
+      tfcc::NPZDataLoader loader{std::string(argv[2])};
+      tfcc::DataLoader::setGlobalDefault(&loader);
+      run("framework.scopes_and_constants", test_scopes_and_constants);
+      run("rnn.lstmcell", test_lstmcell_from_constants);
+      run("layer.dense", test_dense_from_constants);
+      tfcc::DataLoader::setGlobalDefault(nullptr);
+    }
     run("threads.two_sessions", test_two_sessions_on_two_threads);
   } else {
     run("blas.matmul_validation", [] {
@@ -715,6 +834,12 @@ int main(int argc, char** argv) {
       tfcc::Variable<float> a({3, 4}), b({4, 5});
       CHECK_THROWS(tfcc::blas::matmul(a, b), tfcc::NotImplementedError);
     });
+    if (argc > 2) {
+      tfcc::NPZDataLoader loader{std::string(argv[2])};
+      tfcc::DataLoader::setGlobalDefault(&loader);
+      run("framework.scopes_and_constants", test_scopes_and_constants);
+      tfcc::DataLoader::setGlobalDefault(nullptr);
+    }
   }
   if (mode != "gpu") {
     tfcc::Session::setThreadDefault(nullptr);

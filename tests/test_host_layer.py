@@ -4,26 +4,68 @@ the GPU part runs the reference's data / blas / quantization cases on the ROCm d
 import os
 import subprocess
 
+import numpy as np
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 DRIVER = os.path.join(ROOT, "wechat-tfcc_amd", "host", "build", "host_tests")
 
 
-def _run(mode):
+def _sig(v):
+    return 1 / (1 + np.exp(-v))
+
+
+def write_named_test_data(path, seed=5):
+    """An .npz named the way tfcc/test/python/createtestdata.py names the reference's test data
+    ("<package>/<case>/<i>/<key>", "<package>/<case>/__count__"), holding LSTM-cell cases made with the formulas of
+    tfcc/test/python/testcase/rnn/lstmcell.py:31-44 (forget bias 1) and dense-layer cases (matmul + bias), with the
+    expectations formed in float64."""
+    rng = np.random.default_rng(seed)
+    u = lambda *s: rng.uniform(-1.0, 1.0, s).astype(np.float32)  # noqa: E731
+    data = {}
+    cases = [(1, 64, 64), (4, 300, 100), (3, 130, 511)]
+    data["rnn/lstmcell/__count__"] = np.asarray([len(cases)], np.int32)
+    for i, (batch, units, input_size) in enumerate(cases):
+        inputs, kernel, bias, h, cs = u(batch, input_size), u(input_size + units, units * 4), u(units * 4), \
+            u(batch, units), u(batch, units)
+        xh = np.concatenate((inputs, h), axis=1).astype(np.float64) @ kernel.astype(np.float64) + bias
+        gi, ci, f, o = np.split(xh, 4, axis=1)
+        next_cs = np.tanh(ci) * _sig(gi) + cs * _sig(f + 1)
+        expect = np.tanh(next_cs) * _sig(o)
+        prefix = "rnn/lstmcell/%d/" % i
+        data.update({prefix + "units": np.asarray([units], np.int32), prefix + "inputs": inputs, prefix + "h": h,
+                     prefix + "cs": cs, prefix + "lstm_cell/kernel": kernel, prefix + "lstm_cell/bias": bias,
+                     prefix + "ecs": next_cs.astype(np.float32), prefix + "expect": expect.astype(np.float32)})
+    cases = [((5, 70), 33), ((2, 3, 768), 3072), ((1, 512), 2048), ((2, 2, 9, 40), 17)]
+    data["layer/dense/__count__"] = np.asarray([len(cases)], np.int32)
+    for i, (shape, units) in enumerate(cases):
+        inputs, kernel, bias, w, b = u(*shape), u(shape[-1], units), u(units), u(shape[-1], units), u(units)
+        prefix = "layer/dense/%d/" % i
+        x64 = inputs.astype(np.float64)
+        data.update({prefix + "units": np.asarray([units], np.int32), prefix + "inputs": inputs,
+                     prefix + "dense/kernel": kernel, prefix + "dense/bias": bias, prefix + "other/w": w,
+                     prefix + "other/b": b, prefix + "expect": (x64 @ kernel + bias).astype(np.float32),
+                     prefix + "expect_nobias": (x64 @ kernel).astype(np.float32),
+                     prefix + "expect_other": (x64 @ w + b).astype(np.float32)})
+    np.savez(path, **data)
+
+
+def _run(mode, data=None):
     if not os.path.exists(DRIVER):
         subprocess.check_call(["make", "-C", os.path.join(ROOT, "wechat-tfcc_amd", "csrc")])
         subprocess.check_call(["make", "-C", os.path.join(ROOT, "wechat-tfcc_amd", "host")])
-    res = subprocess.run([DRIVER, mode], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
+    res = subprocess.run([DRIVER, mode] + ([data] if data else []), stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=300)
     print(res.stdout)
     assert res.returncode == 0, res.stdout[-4000:]
     assert "0 failures" in res.stdout
 
 
-def test_host_layer_framework_cpu():
-    _run("cpu")
+def test_host_layer_framework_cpu(tmp_path):
+    write_named_test_data(str(tmp_path / "named.npz"))
+    _run("cpu", str(tmp_path / "named.npz"))
 
 
 @pytest.mark.gpu
-def test_host_layer_gpu():
-    _run("gpu")
+def test_host_layer_gpu(tmp_path):
+    write_named_test_data(str(tmp_path / "named.npz"))
+    _run("gpu", str(tmp_path / "named.npz"))

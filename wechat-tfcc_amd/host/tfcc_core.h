@@ -25,6 +25,7 @@
 #include <mutex>
 #include <set>
 #include <string>
+#include <tuple>
 #include <vector>
 
 namespace tfcc {
@@ -187,6 +188,10 @@ class Device {
   unsigned _deviceID;
   std::unique_ptr<Allocator> _allocator;
   std::unique_ptr<InterfaceSet> _interfaces;
+  // Constants of this device, keyed by (scope, name, element type): tfcc/core/framework/tfcc_constantmanager.cpp:35-49.
+  // Declared after the allocator so that they are released before it.
+  std::mutex _constantMutex;
+  std::map<std::tuple<const void*, std::string, int>, std::shared_ptr<void>> _constants;
 
  public:
   Device(DeviceType type, unsigned index, std::unique_ptr<Allocator> allocator);
@@ -204,6 +209,11 @@ class Device {
 
   template <class T>
   Interface<T>& getInterface(T = T());
+
+  // The constant registered under (scope, name, typeKey), created with `make` on first use.
+  std::shared_ptr<void> getConstantSlot(const void* scope, const std::string& name, int typeKey,
+                                        const std::function<std::shared_ptr<void>()>& make);
+  void removeConstants(const void* scope);
 
   unsigned getDeviceID() const { return _deviceID; }  // type << 24 | index
   DeviceType getDeviceType() const { return static_cast<DeviceType>(_deviceID >> 24); }

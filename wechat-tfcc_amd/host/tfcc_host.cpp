@@ -5,6 +5,7 @@
 #include <cstring>
 
 #include "tfcc_rocm.h"
+#include "tfcc_layers.h"
 #include "tfcc_rocm_device.h"
 
 namespace tfcc {
@@ -23,6 +24,78 @@ Device::Device(DeviceType type, unsigned index, std::unique_ptr<Allocator> alloc
 Device::~Device() {
   if (_threadDevice == this) _threadDevice = nullptr;
 }
+
+std::shared_ptr<void> Device::getConstantSlot(const void* scope, const std::string& name, int typeKey,
+                                              const std::function<std::shared_ptr<void>()>& make) {
+  std::lock_guard<std::mutex> lck(_constantMutex);
+  std::shared_ptr<void>& slot = _constants[std::make_tuple(scope, name, typeKey)];
+  if (!slot) slot = make();
+  return slot;
+}
+
+void Device::removeConstants(const void* scope) {
+  std::lock_guard<std::mutex> lck(_constantMutex);
+  for (auto it = _constants.begin(); it != _constants.end();)
+    it = std::get<0>(it->first) == scope ? _constants.erase(it) : std::next(it);
+}
+
+// ---- scopes and data loaders (tfcc/core/framework/tfcc_scope.cpp, tfcc/core/dataloaders/) ---------------------
+Scope Scope::_root(nullptr, "");
+thread_local Scope* Scope::_currentScope = &Scope::_root;
+
+ScopeGuard::~ScopeGuard() {
+  if (_valid) Scope::popScope();
+}
+
+Scope& Scope::getChild(const std::string& name) {
+  std::lock_guard<std::mutex> lck(_mtx);
+  auto it = _children.find(name);
+  if (it != _children.end()) return *it->second;
+  Scope* p = new Scope(this, name);
+  _children[name] = std::unique_ptr<Scope>(p);
+  return *p;
+}
+
+std::string Scope::getFullName() const { return _parent == nullptr ? "" : _parent->getFullName() + _name + "/"; }
+
+void Scope::pushScope(const std::string& name) { _currentScope = &_currentScope->getChild(name); }
+void Scope::popScope() { _currentScope = _currentScope->_parent ? _currentScope->_parent : &_root; }
+ScopeGuard Scope::scope(const std::string& name) {
+  pushScope(name);
+  return ScopeGuard();
+}
+
+DataLoader* DataLoader::_defaultDataLoader = nullptr;
+DataLoader* DataLoader::getGlobalDefault() { return _defaultDataLoader; }
+void DataLoader::setGlobalDefault(DataLoader* loader) { _defaultDataLoader = loader; }
+
+void NPZDataLoader::fill(const std::map<std::string, std::string>& members) {
+  for (const auto& kv : members) {
+    if (kv.first.size() < 4 || kv.first.substr(kv.first.size() - 4) != ".npy") continue;
+    try {  // members that are not arrays are skipped (tfcc/core/dataloaders/tfcc_npzdataloader.cpp:27-42)
+      runtime::NpyArray a = runtime::parse_npy(kv.second);
+      _dataMap[kv.first.substr(0, kv.first.size() - 4)] = std::make_tuple(Shape(a.shape), a.type, std::move(a.body));
+    } catch (const std::exception&) {
+    }
+  }
+}
+
+NPZDataLoader::NPZDataLoader(const std::string& path) { fill(runtime::unzip_from_path(path)); }
+NPZDataLoader::NPZDataLoader(const char* data, size_t dataLen) { fill(runtime::unzip(std::string(data, dataLen))); }
+
+const std::tuple<Shape, std::string, std::string>& NPZDataLoader::loadData(const std::string& name) const {
+  auto it = _dataMap.find(name);
+  if (it == _dataMap.end()) throw RuntimeError("Name: [" + name + "] not found in data loader");
+  return it->second;
+}
+
+std::vector<std::tuple<std::string, std::string>> NPZDataLoader::getAllNames() const {
+  std::vector<std::tuple<std::string, std::string>> result;
+  for (const auto& kv : _dataMap) result.emplace_back(kv.first, std::get<1>(kv.second));
+  return result;
+}
+
+bool NPZDataLoader::hasData(const std::string& name) const { return _dataMap.count(name) != 0; }
 
 void Session::preRelease() {
   for (auto& cb : _releaseCallbacks) cb(this);
