@@ -437,7 +437,10 @@ def test_sgemm_general_multiplies_permuted_views_in_place(pkg, T, b, s, h, d):
     assert np.array_equal(dense, T.n(scores))
 
 
-@pytest.mark.parametrize("m,n,k,groups", [(1024, 768, 768, 3), (100, 52, 36, 4), (64, 64, 1028, 2), (7, 4, 4, 1)])
+@pytest.mark.parametrize("m,n,k,groups", [
+    (1024, 768, 768, 3), (100, 52, 36, 4), (64, 64, 1028, 2), (7, 4, 4, 1),
+    # 128 x 96 tiles shared by the products (four and two K groups' worth of sums per tile), ragged edges
+    (1000, 760, 768, 3), (2048, 768, 768, 2), (2040, 764, 512, 2)])
 def test_sgemm_grouped_equals_separate_launches(pkg, T, m, n, k, groups):
     rng = np.random.default_rng(m + n + k + groups)
     a = rng.normal(0, 1, (m, k)).astype(np.float32)

@@ -422,6 +422,13 @@ int dispatch(hipStream_t s, const SgemmParams& p, bool vec, bool tb, unsigned fi
       // one so that each is summed exactly as on its own): when they fill the chip without the K groups, one
       // group per tile plays all of them.
       const bool serial = ksplit > 1 && bestTiles * (p.batch / fillBatch) * kTiles[best].waves >= 256ull * 8;
+      // ... and when 128 x 96 tiles over all of them still occupy most of the CUs in one round, twelve wavefronts
+      // share each copy of B among four times the rows (44.1 against 46.8 us for three 1024 x 768 x 768 products);
+      // the sums are those of the 32 x 96 tiles.
+      if (serial && kTiles[best].config == 1) {
+        const unsigned long long wide = (unsigned long long)((m + 127) / 128) * ((n + 95) / 96) * p.batch;
+        if (wide <= 256 && wide >= 160) return sgemm_detail::sgemm_dma_launch(s, p, 5, ksplit, true);
+      }
       return sgemm_detail::sgemm_dma_launch(s, p, kTiles[best].config, ksplit, serial);
     }
     if (preferFlat && flat <= 320 && k >= 512) return launch<1, 3, 1, 1, true, 4>(s, p);

@@ -39,7 +39,7 @@ inline bool set_tiles(SgemmParams& p, unsigned bm, unsigned bn) {
 }
 
 // The direct-to-LDS kernels (sgemm_dma.hip).  `config`: 0 = 64x64 tiles, 1 = 32x96, 2 = 32x64, 3 = 32x32, 4 = 128x128
-// (ksplit 1 only); ksplit 1, 2 or 4 groups of wavefronts on one tile.
+// (ksplit 1 only), 5 = 128x96 (serial groups only); ksplit 1, 2 or 4 groups of wavefronts on one tile.
 // Requires 16-byte aligned operands and strides, K a multiple of 32 and B not transposed.
 bool sgemm_dma_available(int config, int ksplit);
 // serialGroups: one group of wavefronts per tile does the work of the `ksplit` groups one slab after the other
