@@ -322,6 +322,11 @@ int tfcc_rocm_transform2_f32(void* stream, const float* in, uint64_t total, floa
  * ArithmeticInterface::add/sub/mul/div, tfcc/core/interfaces/tfcc_arithmeticinterface.h:34-79 */
 int tfcc_rocm_binary_f32(void* stream, int op, const float* a, const float* b, uint64_t total,
                          uint64_t period, float* out);
+/* out = a op b with numpy-style broadcasting: dims[rank] is the result's shape, stride_a / stride_b the element strides
+ * of each operand per result dimension (0 where the operand's extent is 1).  rank <= 6; callers merge adjacent
+ * dimensions of the same kind first, as tfcc::math::add does (tfcc/core/operations/tfcc_math.cpp:38-104). */
+int tfcc_rocm_binary_broadcast_f32(void* stream, int op, const float* a, const float* b, int rank,
+                                   const unsigned* dims, const uint64_t* stride_a, const uint64_t* stride_b, float* out);
 /* rank <= 6 permutation: BasicInterface::transpose, tfcc/core/operations/tfcc_base.cpp:124-134.
  * shape / perm are HOST arrays of length rank. */
 int tfcc_rocm_transpose_f32(void* stream, const float* in, const unsigned* shape,

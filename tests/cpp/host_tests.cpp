@@ -699,6 +699,50 @@ static void test_dense_from_constants() {
   CHECK_THROWS_MSG(tfcc::layer::dense(wrong, 0u, true), tfcc::InvalidArgumentError, "inputs and kernel don't match");
 }
 
+// tfcc::math::add / sub / mul / div with the broadcasting of tfcc/core/operations/tfcc_math.cpp:38-104
+// (tfcc/test/math.cpp's broadcast cases): attention mask, both sides broadcast, either operand the larger.
+static void test_broadcast_arithmetic() {
+  std::mt19937 rng(21);
+  std::uniform_real_distribution<float> dist(0.5f, 2.f);
+  struct Case { std::vector<unsigned> sa, sb; };
+  for (const Case& c : {Case{{2, 4, 8, 8}, {2, 1, 1, 8}}, Case{{3, 1, 5}, {1, 4, 1}}, Case{{33}, {7, 33}}, Case{{5, 6}, {1}},
+                        Case{{2, 3, 4, 5, 6, 7}, {2, 1, 4, 1, 6, 1}}}) {
+    size_t na = 1, nb = 1;
+    for (unsigned d : c.sa) na *= d;
+    for (unsigned d : c.sb) nb *= d;
+    std::vector<float> ha(na), hb(nb);
+    for (auto& v : ha) v = dist(rng);
+    for (auto& v : hb) v = dist(rng);
+    tfcc::Variable<float> a = tfcc::data::set(ha, tfcc::Shape(c.sa)), b = tfcc::data::set(hb, tfcc::Shape(c.sb));
+    const size_t rank = std::max(c.sa.size(), c.sb.size());
+    std::vector<unsigned> da(rank, 1), db(rank, 1), dr(rank);
+    std::copy(c.sa.begin(), c.sa.end(), da.begin() + (rank - c.sa.size()));
+    std::copy(c.sb.begin(), c.sb.end(), db.begin() + (rank - c.sb.size()));
+    size_t total = 1;
+    for (size_t d = 0; d < rank; ++d) total *= dr[d] = std::max(da[d], db[d]);
+    tfcc::Variable<float> sum = a + b, dif = a - b, pro = a * b, quo = a / b;
+    CHECK(sum.shape() == tfcc::Shape(dr) && quo.shape() == tfcc::Shape(dr));
+    std::vector<float> gs = tfcc::data::get(sum), gd = tfcc::data::get(dif), gp = tfcc::data::get(pro), gq = tfcc::data::get(quo);
+    bool ok = gs.size() == total;
+    for (size_t i = 0; ok && i < total; ++i) {
+      size_t rem = i, ia = 0, ib = 0, sa = 1, sb = 1;
+      for (size_t d = rank; d-- > 0;) {
+        const size_t coord = rem % dr[d];
+        rem /= dr[d];
+        ia += (da[d] == 1 ? 0 : coord) * sa;
+        ib += (db[d] == 1 ? 0 : coord) * sb;
+        sa *= da[d];
+        sb *= db[d];
+      }
+      ok = gs[i] == ha[ia] + hb[ib] && gd[i] == ha[ia] - hb[ib] && gp[i] == ha[ia] * hb[ib] && gq[i] == ha[ia] / hb[ib];
+    }
+    CHECK(ok);
+  }
+  tfcc::Variable<float> a({2, 3}), b({2, 2}), e({0, 3}), one({1, 3});
+  CHECK_THROWS_MSG(a + b, tfcc::InvalidArgumentError, "broadcast failed");
+  CHECK((e + one).shape() == tfcc::Shape({0, 3}));
+}
+
 // Two threads, each with a session (= stream) of its own on the shared device, running the same mix of
 // operations at the same time: fp32 matmul, quantize with its min/max reduction, quantized matmul.  Every
 // result is checked on the thread that produced it (tfcc/core/framework/tfcc_session.h:29,60-62: device
@@ -815,6 +859,7 @@ int main(int argc, char** argv) {
     run("quantization.rocm_matmul_round_trips", test_quantized_matmul_round_trips);
     run("quantization.rocm_matmul_exact", test_quantized_matmul_exact);
     run("layer.elementwise", test_layer_ops);
+    run("math.broadcast_arithmetic", test_broadcast_arithmetic);
     run("layer.attention_permuted", test_attention_permuted);
     run("rnn.cells", test_cells);
     run("rnn.lstm_forward_backward", test_lstm_sequences);

@@ -4,6 +4,7 @@ import ctypes as C
 import os
 import re
 
+import numpy as np
 import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -66,3 +67,31 @@ def test_matmul_plan_rules(pkg):
         pkg.matmul_plan((4, 1, 5, 7, 8), (1, 3, 5, 8, 6))
     with pytest.raises(pkg.InvalidArgumentError):
         pkg.matmul_plan((2, 3, 4), (3, 4, 5))
+
+
+def test_broadcast_shape_rule(pkg):
+    """The shape rule of tfcc/core/operations/tfcc_math.cpp:38-86 against numpy's, and its merged forms: equal rank,
+    each dimension equal or 1 on one side, neighbouring dimensions never of the same kind, products preserved."""
+    rng = np.random.default_rng(0)
+    for _ in range(300):
+        rank = int(rng.integers(1, 6))
+        full = [int(rng.integers(1, 5)) for _ in range(rank)]
+        s1 = [d if rng.random() < 0.6 else 1 for d in full][int(rng.integers(0, rank)):]
+        s2 = [d if rng.random() < 0.6 else 1 for d in full][int(rng.integers(0, rank)):]
+        shape, c1, c2 = pkg.broadcast_shapes(s1, s2)
+        assert shape == tuple(np.broadcast_shapes(tuple(s1), tuple(s2)))
+        assert len(c1) == len(c2) >= 1
+        assert int(np.prod(c1)) == int(np.prod(s1)) and int(np.prod(c2)) == int(np.prod(s2))
+        kinds = [0 if x == y else (1 if x == 1 else 2) for x, y in zip(c1, c2)]
+        assert all(x == y or x == 1 or y == 1 for x, y in zip(c1, c2))
+        assert all(k1 != k2 for k1, k2 in zip(kinds, kinds[1:]))
+        # the merged shapes broadcast to the same values as the originals
+        a = rng.normal(size=s1)
+        b = rng.normal(size=s2)
+        assert np.array_equal((a.reshape(c1) + b.reshape(c2)).reshape(shape), a + b)
+    assert pkg.broadcast_shapes((16, 12, 128, 128), (16, 1, 1, 128)) == ((16, 12, 128, 128), (16, 1536, 128), (16, 1, 128))
+    assert pkg.broadcast_shapes((7, 33), (33,)) == ((7, 33), (7, 33), (1, 33))
+    assert pkg.broadcast_shapes((1,), (1,)) == ((1,), (1,), (1,))
+    for bad in (((2, 3), (2, 2)), ((), (3,))):
+        with pytest.raises(pkg.InvalidArgumentError):
+            pkg.broadcast_shapes(*bad)

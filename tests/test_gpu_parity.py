@@ -541,6 +541,38 @@ def test_lstm_cell_in_place_state_and_sequence(pkg, T):
         assert np.linalg.norm(got - want) <= 1e-5 * np.linalg.norm(want)
 
 
+BROADCAST_PAIRS = [
+    ((2, 4, 8, 8), (2, 1, 1, 8)),        # attention scores + mask
+    ((3, 1, 5), (1, 4, 1)),              # both sides broadcast
+    ((5, 6), (1,)), ((1,), (5, 6)),      # a one-element tensor on either side
+    ((7, 33), (33,)), ((33,), (7, 33)),  # bias forms, either order
+    ((2, 3, 4, 5, 6, 7), (2, 1, 4, 1, 6, 1)),  # six groups
+    ((4, 1, 6), (4, 5, 6)), ((1, 1, 9), (8, 1, 1)), ((16, 12, 128, 128), (16, 1, 1, 128)),
+]
+
+
+@pytest.mark.parametrize("sa,sb", BROADCAST_PAIRS)
+def test_broadcast_arithmetic_equals_numpy(pkg, T, sa, sb):
+    """tfcc::math::add / sub / mul / div with the broadcasting of tfcc/core/operations/tfcc_math.cpp:38-104: one
+    rounding per element, so the results are numpy's bit for bit."""
+    rng = np.random.default_rng(len(sa) * 100 + len(sb))
+    a = rng.normal(0, 2, sa).astype(np.float32)
+    b = rng.uniform(0.5, 3, sb).astype(np.float32) * rng.choice([-1, 1], sb).astype(np.float32)
+    for op, ref in (("add", np.add), ("sub", np.subtract), ("mul", np.multiply), ("div", np.divide)):
+        got = T.n(pkg.math_binary(op, T.t(a), T.t(b)))
+        want = ref(a, b)
+        assert got.shape == want.shape and np.array_equal(got, want), op
+
+
+def test_broadcast_arithmetic_rejects_what_the_reference_rejects(pkg, T):
+    a = T.t(np.zeros((2, 3), np.float32))
+    with pytest.raises(pkg.InvalidArgumentError, match="broadcast failed"):
+        pkg.math_binary("add", a, T.t(np.zeros((2, 2), np.float32)))
+    with pytest.raises(pkg.InvalidArgumentError, match="broadcast failed"):
+        pkg.math_binary("mul", a, T.t(np.zeros((4, 1, 3, 3), np.float32)))
+    assert tuple(pkg.math_binary("add", T.t(np.zeros((0, 3), np.float32)), T.t(np.zeros((1, 3), np.float32))).shape) == (0, 3)
+
+
 def test_elementwise_against_oracle(pkg, T):
     rng = np.random.default_rng(50)
     for shape in ((8, 12, 128, 128), (7, 33), (5, 1000)):

@@ -373,6 +373,27 @@ def test_unary_nodes_against_numpy_float64(mf, rt, dev):
     assert np.array_equal(res[outs["Neg"]], 0 - xv) and np.array_equal(res[outs["Sign"]], np.sign(xv))
 
 
+@pytest.mark.gpu
+def test_arithmetic_nodes_broadcast_like_numpy(mf, rt, dev):
+    """math.Add / Sub / Mul / Div on tensors broadcast as tfcc::math does (tfcc/core/operations/tfcc_math.cpp:38-104):
+    scores [B, H, S, S] with a mask [B, 1, 1, S], and a column against a row."""
+    rng = np.random.default_rng(3)
+    g = mf.GraphBuilder("g")
+    scores = g.input("scores", mf.FLOAT, [2, 3, 5, 5])
+    mask = g.input("mask", mf.FLOAT, [2, 1, 1, 5])
+    col = g.input("col", mf.FLOAT, [4, 1])
+    row = g.input("row", mf.FLOAT, [1, 6])
+    outs = {"add": g.binary("Add", scores, mask), "sub": g.binary("Sub", mask, scores), "mul": g.binary("Mul", col, row),
+            "div": g.binary("Div", row, col)}
+    for o in outs.values():
+        g.output(o)
+    sv, mv = rng.normal(0, 1, (2, 3, 5, 5)).astype(np.float32), rng.normal(0, 1, (2, 1, 1, 5)).astype(np.float32)
+    cv, rv = rng.uniform(1, 2, (4, 1)).astype(np.float32), rng.uniform(1, 2, (1, 6)).astype(np.float32)
+    res = rt.Model(mf.write_model([g], "g")).run({"scores": sv, "mask": mv, "col": cv, "row": rv})
+    assert np.array_equal(res[outs["add"]], sv + mv) and np.array_equal(res[outs["sub"]], mv - sv)
+    assert np.array_equal(res[outs["mul"]], cv * rv) and np.array_equal(res[outs["div"]], rv / cv)
+
+
 def bidirectional_lstm_graph(mf, rng, seq, batch, length, hidden, hidden_field=None):
     u = lambda *s: rng.uniform(-1, 1, s).astype(np.float32)  # noqa: E731
     w = dict(ik=u(2, length, 4 * hidden), sk=u(2, hidden, 4 * hidden), bias=u(2, 4 * hidden), ih=u(2, batch, hidden),

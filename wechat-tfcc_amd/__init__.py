@@ -126,6 +126,8 @@ SYMBOLS = {
     "tfcc_rocm_transform2_f32": (_I, [_VP, _VP, _U64, _F, _F, _VP]),
     "tfcc_rocm_binary_f32": (_I, [_VP, _I, _VP, _VP, _U64, _U64, _VP]),
     "tfcc_rocm_transpose_f32": (_I, [_VP, _VP, C.POINTER(C.c_uint), C.POINTER(C.c_uint), _I, _VP]),
+    "tfcc_rocm_binary_broadcast_f32": (_I, [_VP, _I, _VP, _VP, _I, C.POINTER(C.c_uint), C.POINTER(_U64),
+                                           C.POINTER(_U64), _VP]),
     "tfcc_rocm_lstm_cell_f32": (_I, [_VP, _U, _U, _VP, _VP, _VP, _VP, _F, _VP, _VP]),
     "tfcc_rocm_gru_cell_gates_f32": (_I, [_VP, _U, _U, _U, _VP, _VP, _VP, _VP, _VP]),
     "tfcc_rocm_gru_cell_candidate_f32": (_I, [_VP, _U, _U, _VP, _VP, _VP, _VP, _VP, _VP]),
@@ -649,6 +651,62 @@ def binary(op, a, b):
     a, b = a.contiguous(), b.contiguous()
     out = torch.empty_like(a)
     check(lib().tfcc_rocm_binary_f32(_stream(), BINARY_OPS[op], _ptr(a), _ptr(b), a.numel(), b.numel(), _ptr(out)))
+    return out
+
+
+def broadcast_shapes(s1, s2):
+    """_get_broadcast_shape of tfcc/core/operations/tfcc_math.cpp:38-86: (result shape, collapsed s1, collapsed s2).
+    Right-aligned; extents must be equal or 1; runs of dimensions of the same kind are merged."""
+    s1, s2 = list(s1), list(s2)
+    if not s1 or not s2:
+        raise InvalidArgumentError("invalid tensor shape")
+    result = list(s1 if len(s1) > len(s2) else s2)
+    for i in range(min(len(s1), len(s2))):
+        l1, l2 = s1[-1 - i], s2[-1 - i]
+        if l1 != l2 and l1 != 1 and l2 != 1:
+            raise InvalidArgumentError("broadcast failed")
+        result[-1 - i] = l2 if l1 == 1 else l1  # the reference takes max(): 0 against 1 would give 1 and read past the empty operand
+    kind = lambda l1, l2: 0 if l1 == l2 else (1 if l1 == 1 else 2)  # noqa: E731
+    n1, n2 = [], []
+    len1, len2 = s1[-1], s2[-1]
+    cur = kind(len1, len2)
+    for i in range(1, max(len(s1), len(s2))):
+        l1 = s1[-1 - i] if i < len(s1) else 1
+        l2 = s2[-1 - i] if i < len(s2) else 1
+        if kind(l1, l2) != cur:
+            n1.insert(0, len1)
+            n2.insert(0, len2)
+            cur, len1, len2 = kind(l1, l2), l1, l2
+        else:
+            len1 *= l1
+            len2 *= l2
+    if len1 != 1 or len2 != 1 or not n1:
+        n1.insert(0, len1)
+        n2.insert(0, len2)
+    return tuple(result), tuple(n1), tuple(n2)
+
+
+def math_binary(op, a, b):
+    """tfcc::math::add / sub / mul / div (op in BINARY_OPS) with the reference's broadcasting."""
+    import torch
+    shape, ca, cb = broadcast_shapes(a.shape, b.shape)
+    out = torch.empty(shape, dtype=torch.float32, device=a.device)
+    if out.numel() == 0:
+        return out
+    if len(ca) > 6:
+        raise NotImplementedError("more than six groups of broadcast dimensions")
+    a, b = a.contiguous(), b.contiguous()
+    dims = [max(x, y) for x, y in zip(ca, cb)]
+
+    def strides(c):
+        st, acc = [0] * len(c), 1
+        for d in range(len(c) - 1, -1, -1):
+            st[d] = 0 if c[d] == 1 and dims[d] != 1 else acc
+            acc *= c[d]
+        return st
+    n = len(dims)
+    check(lib().tfcc_rocm_binary_broadcast_f32(_stream(), BINARY_OPS[op], _ptr(a), _ptr(b), n, (C.c_uint * n)(*dims),
+                                               (_U64 * n)(*strides(ca)), (_U64 * n)(*strides(cb)), _ptr(out)))
     return out
 
 

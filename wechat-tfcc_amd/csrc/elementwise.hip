@@ -180,6 +180,32 @@ __global__ __launch_bounds__(256) void binary_kernel(const float* a, const float
   }
 }
 
+// The general numpy-style broadcast: every dimension has the output's extent on one side or both, the other side's
+// stride is 0 there.
+struct BroadcastParams {
+  unsigned dims[6];
+  unsigned long long strideA[6], strideB[6];
+  int rank;
+};
+
+template <int OP>
+__global__ __launch_bounds__(256) void binary_broadcast_kernel(const float* a, const float* b, size_t total,
+                                                               BroadcastParams p, float* out) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t step = (size_t)gridDim.x * blockDim.x;
+  for (; i < total; i += step) {
+    size_t rem = i, ia = 0, ib = 0;
+    for (int d = p.rank - 1; d >= 0; --d) {
+      const size_t c = rem % p.dims[d];
+      rem /= p.dims[d];
+      ia += c * p.strideA[d];
+      ib += c * p.strideB[d];
+    }
+    const float x = a[ia], y = b[ib];
+    out[i] = OP == 0 ? x + y : OP == 1 ? x - y : OP == 2 ? x * y : x / y;
+  }
+}
+
 struct TransposeParams {
   unsigned outShape[6];
   unsigned long long inStride[6];  // input stride of each OUTPUT dim
@@ -327,6 +353,32 @@ int tfcc_rocm_binary_f32(void* stream, int op, const float* a, const float* b, u
     default: hipLaunchKernelGGL(binary_kernel<3>, grid, block, 0, s, a, b, (size_t)total, (size_t)period, out); break;
   }
   return check_launch("binary");
+}
+
+int tfcc_rocm_binary_broadcast_f32(void* stream, int op, const float* a, const float* b, int rank,
+                                   const unsigned* dims, const uint64_t* stride_a, const uint64_t* stride_b, float* out) {
+  TFCC_REQUIRE(a && b && out && dims && stride_a && stride_b, "binary_broadcast: null argument");
+  TFCC_REQUIRE(op >= 0 && op <= 3, "binary_broadcast: unknown operation %d", op);
+  TFCC_REQUIRE(rank >= 1 && rank <= 6, "binary_broadcast: rank %d (1..6)", rank);
+  BroadcastParams p{};
+  p.rank = rank;
+  size_t total = 1;
+  for (int d = 0; d < rank; ++d) {
+    TFCC_REQUIRE(dims[d] > 0, "binary_broadcast: empty tensor");
+    p.dims[d] = dims[d];
+    p.strideA[d] = stride_a[d];
+    p.strideB[d] = stride_b[d];
+    total *= dims[d];
+  }
+  const dim3 grid(grid_for(total)), block(256);
+  hipStream_t s = as_stream(stream);
+  switch (op) {
+    case 0: hipLaunchKernelGGL(binary_broadcast_kernel<0>, grid, block, 0, s, a, b, total, p, out); break;
+    case 1: hipLaunchKernelGGL(binary_broadcast_kernel<1>, grid, block, 0, s, a, b, total, p, out); break;
+    case 2: hipLaunchKernelGGL(binary_broadcast_kernel<2>, grid, block, 0, s, a, b, total, p, out); break;
+    default: hipLaunchKernelGGL(binary_broadcast_kernel<3>, grid, block, 0, s, a, b, total, p, out); break;
+  }
+  return check_launch("binary_broadcast");
 }
 
 int tfcc_rocm_add_f32(void* stream, const float* a, const float* b, uint64_t total, uint64_t period, float* out) {

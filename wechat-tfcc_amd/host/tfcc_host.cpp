@@ -657,24 +657,38 @@ class ROCMBasicInterface : public BasicInterface<float> {
   }
 };
 
+// a and b arrive with equal rank, every dimension equal or 1 on one side (tfcc::math merges the rest away).
 class ROCMArithmeticInterface : public ArithmeticInterface<float> {
-  // b equals the trailing dimensions of a once leading 1s are dropped (bias / residual forms)
-  static bool trailing(const Tensor<float>& a, const Tensor<float>& b) {
-    const size_t ra = a.shape().size();
-    size_t skip = 0;
-    while (skip + 1 < b.shape().size() && b.shape(skip) == 1) ++skip;
-    const size_t rb = b.shape().size() - skip;
-    bool ok = rb <= ra && a.size() > 0 && b.size() > 0;
-    for (size_t i = 0; ok && i < rb; ++i) ok = a.shape(ra - rb + i) == b.shape(skip + i);
-    return ok;
-  }
   static Variable<float> run(int op, const Tensor<float>& a, const Tensor<float>& b) {
-    if (!trailing(a, b)) {
-      if ((op == 0 || op == 2) && trailing(b, a)) return run(op, b, a);  // commutative: swap
-      throw NotImplementedError("element-wise operation: only a trailing-dimension broadcast of one operand");
+    const size_t rank = a.shape().size();
+    if (rank == 0 || rank != b.shape().size()) throw InvalidArgumentError("invalid tensor shape");
+    std::vector<unsigned> dims(rank);
+    for (size_t d = 0; d < rank; ++d) {
+      if (a.shape(d) != b.shape(d) && a.shape(d) != 1 && b.shape(d) != 1) throw InvalidArgumentError("broadcast failed");
+      dims[d] = std::max(a.shape(d), b.shape(d));
     }
-    Variable<float> r(a.shape());
-    check(tfcc_rocm_binary_f32(current_stream(), op, a.data(), b.data(), a.size(), b.size(), r.data()));
+    Variable<float> r{Shape(dims)};
+    if (r.size() == 0) return r;
+    // b repeats along the leading dimensions of a only: the one-pass kernel with a period
+    bool periodic = a.size() == r.size();
+    for (size_t d = 0, seenFull = 0; periodic && d < rank; ++d) {
+      if (b.shape(d) == dims[d] && dims[d] != 1) seenFull = 1;
+      else if (seenFull && dims[d] != 1) periodic = false;  // b broadcasts again after one of its own dimensions
+    }
+    if (periodic) {
+      check(tfcc_rocm_binary_f32(current_stream(), op, a.data(), b.data(), a.size(), b.size(), r.data()));
+      return r;
+    }
+    if (rank > 6) throw NotImplementedError("element-wise operation: more than six groups of broadcast dimensions");
+    uint64_t sa[6], sb[6], accA = 1, accB = 1;
+    for (size_t d = rank; d-- > 0;) {
+      sa[d] = a.shape(d) == 1 && dims[d] != 1 ? 0 : accA;
+      sb[d] = b.shape(d) == 1 && dims[d] != 1 ? 0 : accB;
+      accA *= a.shape(d);
+      accB *= b.shape(d);
+    }
+    check(tfcc_rocm_binary_broadcast_f32(current_stream(), op, a.data(), b.data(), static_cast<int>(rank), dims.data(), sa,
+                                         sb, r.data()));
     return r;
   }
 

@@ -19,6 +19,7 @@
 //   base::transpose         tfcc_base.cpp:124-134
 #pragma once
 
+#include <algorithm>
 #include <tuple>
 
 #include "tfcc_core.h"
@@ -350,22 +351,71 @@ TFCC_UNARY_FUNCTION(erf, ERF)
 TFCC_UNARY_FUNCTION(abs, ABS)
 TFCC_UNARY_FUNCTION(sign, SIGN)
 #undef TFCC_UNARY_FUNCTION
-// a + b with b's shape equal to the trailing dimensions of a's (or the same shape)
+namespace detail {
+// _get_broadcast_shape of tfcc/core/operations/tfcc_math.cpp:38-86: numpy-style right-aligned broadcasting (extents
+// equal or 1); runs of dimensions of the same kind (equal / first broadcast / second broadcast) are merged, so the
+// interface sees two shapes of equal rank.  Returns (result shape, merged shape of s1, merged shape of s2).
+inline std::tuple<Shape, Shape, Shape> broadcast_shapes(const Shape& s1, const Shape& s2) {
+  if (s1.size() == 0 || s2.size() == 0) throw InvalidArgumentError("invalid tensor shape");
+  std::vector<unsigned> resultS = s1.size() > s2.size() ? s1.toVector() : s2.toVector(), newS1, newS2;
+  for (size_t i = 0; i < s1.size() && i < s2.size(); ++i) {
+    const unsigned l1 = s1[s1.size() - 1 - i], l2 = s2[s2.size() - 1 - i];
+    if (l1 != l2 && l1 != 1 && l2 != 1) throw InvalidArgumentError("broadcast failed");
+    // the reference takes max(l1, l2): an empty dimension against 1 would come out as 1 and the empty operand be read
+    resultS[resultS.size() - 1 - i] = l1 == 1 ? l2 : l1;
+  }
+  auto kind = [](unsigned l1, unsigned l2) { return l1 == l2 ? 0 : l1 == 1 ? 1 : 2; };
+  const size_t maxLen = std::max(s1.size(), s2.size());
+  unsigned len1 = s1[s1.size() - 1], len2 = s2[s2.size() - 1];
+  int type = kind(len1, len2);
+  for (size_t i = 1; i < maxLen; ++i) {
+    const unsigned l1 = i < s1.size() ? s1[s1.size() - 1 - i] : 1, l2 = i < s2.size() ? s2[s2.size() - 1 - i] : 1;
+    if (kind(l1, l2) != type) {
+      newS1.insert(newS1.begin(), len1);
+      newS2.insert(newS2.begin(), len2);
+      type = kind(l1, l2);
+      len1 = l1;
+      len2 = l2;
+    } else {
+      len1 *= l1;
+      len2 *= l2;
+    }
+  }
+  if (len1 != 1 || len2 != 1 || newS1.empty()) {
+    newS1.insert(newS1.begin(), len1);
+    newS2.insert(newS2.begin(), len2);
+  }
+  return std::make_tuple(Shape(std::move(resultS)), Shape(std::move(newS1)), Shape(std::move(newS2)));
+}
+
+template <class T, class F>
+Variable<T> broadcast_binary(const Tensor<T>& a, const Tensor<T>& b, F call) {
+  Shape resultS, newAS, newBS;
+  std::tie(resultS, newAS, newBS) = broadcast_shapes(a.shape(), b.shape());
+  if (resultS.area() == 0) return Variable<T>(resultS);
+  View<T> aView(a, newAS), bView(b, newBS);
+  Variable<T> result = call(Operation<T>::getCurrentInterface().getArithmeticInterface(), aView, bView);
+  result.reshape(std::move(resultS));
+  return result;
+}
+}  // namespace detail
+
+// tfcc::math::add / sub / mul / div (tfcc/core/operations/tfcc_math.cpp:88-150)
 template <class T>
 Variable<T> add(const Tensor<T>& a, const Tensor<T>& b) {
-  return Operation<T>::getCurrentInterface().getArithmeticInterface().add(a, b);
+  return detail::broadcast_binary(a, b, [](ArithmeticInterface<T>& i, const Tensor<T>& x, const Tensor<T>& y) { return i.add(x, y); });
 }
 template <class T>
 Variable<T> sub(const Tensor<T>& a, const Tensor<T>& b) {
-  return Operation<T>::getCurrentInterface().getArithmeticInterface().sub(a, b);
+  return detail::broadcast_binary(a, b, [](ArithmeticInterface<T>& i, const Tensor<T>& x, const Tensor<T>& y) { return i.sub(x, y); });
 }
 template <class T>
 Variable<T> mul(const Tensor<T>& a, const Tensor<T>& b) {
-  return Operation<T>::getCurrentInterface().getArithmeticInterface().mul(a, b);
+  return detail::broadcast_binary(a, b, [](ArithmeticInterface<T>& i, const Tensor<T>& x, const Tensor<T>& y) { return i.mul(x, y); });
 }
 template <class T>
 Variable<T> div(const Tensor<T>& a, const Tensor<T>& b) {
-  return Operation<T>::getCurrentInterface().getArithmeticInterface().div(a, b);
+  return detail::broadcast_binary(a, b, [](ArithmeticInterface<T>& i, const Tensor<T>& x, const Tensor<T>& y) { return i.div(x, y); });
 }
 template <class T>
 Variable<T> transform(const Tensor<T>& a, T alpha, T beta) {
