@@ -272,8 +272,8 @@ int tfcc_rocm_softmax_div_f32(void* stream, const float* in, uint64_t rows, unsi
  * they lie.  It stands for the node sequence Transpose x3 -> Matmul -> Div -> Softmax -> Matmul ->
  * Transpose that the reference's runtime runs one operation at a time
  * (tfcc_runtime/operations/math/matmul.cpp:27-41, softmax.cpp, base/transpose.cpp) and returns what
- * tfcc_rocm_sgemm_general (trans_b) + tfcc_rocm_softmax_div_f32 + tfcc_rocm_sgemm_general return, bit
- * for bit.  Limits: t <= 128, d <= 64 and a multiple of 4, input strides multiples of 4, inputs 16-byte
+ * tfcc_rocm_sgemm_general (trans_b) + tfcc_rocm_softmax_div_f32 (or division, mask addition and softmax one after
+ * the other) + tfcc_rocm_sgemm_general return, bit for bit.  Limits: t <= 128, d <= 64 and a multiple of 4, input strides multiples of 4, inputs 16-byte
  * aligned, and not a single head (batch_outer * batch_inner == 1) of s <= 8 rows, whose separate product
  * runs on the streaming kernel for short A and sums in another order;
  * tfcc_rocm_attention_f32_supported() tells (1 / 0) whether a descriptor is within them.
@@ -290,6 +290,11 @@ typedef struct tfcc_rocm_attention_desc {
   uint64_t inner_stride_q, inner_stride_k, inner_stride_v, inner_stride_out; /* between inner entries */
   float divisor;
   int has_divisor; /* 0: plain softmax(q k^T) */
+  /* optional (NULL: none): t values per batch entry added to every row of the divided scores before the softmax, as
+   * the Add of an attention mask [batch, 1, 1, t] between Div and Softmax does; batch strides in elements (0 where
+   * the mask is shared) */
+  const float* mask;
+  uint64_t stride_mask, inner_stride_mask;
 } tfcc_rocm_attention_desc;
 int tfcc_rocm_attention_f32_supported(const tfcc_rocm_attention_desc* desc);
 int tfcc_rocm_attention_f32(void* stream, const tfcc_rocm_attention_desc* desc);

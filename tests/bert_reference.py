@@ -6,7 +6,7 @@ import numpy as np
 import oracle_lib as O
 
 
-def encoder_layer(x, w, heads, epsilon=1e-12):
+def encoder_layer(x, w, heads, epsilon=1e-12, mask=None):
     batch, seq, hidden = x.shape
     size = hidden // heads
     x2 = x.reshape(batch * seq, hidden)
@@ -18,6 +18,8 @@ def encoder_layer(x, w, heads, epsilon=1e-12):
     kt = np.ascontiguousarray(project("wk", "bk").transpose(0, 2, 3, 1))
     v = np.ascontiguousarray(project("wv", "bv").transpose(0, 2, 1, 3))
     scores = O.sgemm(q, kt) / np.float32(np.sqrt(size))
+    if mask is not None:  # [batch, 1, 1, seq], added to every head's and every query's scores
+        scores = scores.astype(np.float32) + mask.astype(np.float32)
     probs = O.softmax(scores.astype(np.float32))
     context = np.ascontiguousarray(O.sgemm(probs, v).transpose(0, 2, 1, 3)).reshape(batch * seq, hidden)
     attention = O.layer_norm(O.sgemm(context, w["wo"], w["bo"]) + x2, w["ln1_gamma"], w["ln1_beta"], epsilon)

@@ -24,7 +24,7 @@ def reference64(q, k, v, divisor):
     return np.einsum("bhst,bhtd->bhsd", p, v.astype(np.float64))
 
 
-def separate_kernels(pkg, torch, q, k, v, B, H, S, T, D, divisor, layout):
+def separate_kernels(pkg, torch, q, k, v, B, H, S, T, D, divisor, layout, mask=None):
     """The same result from two products and one softmax, each in a launch of its own."""
     dev = q.device
     scores = torch.empty((B, H, S, T), dtype=torch.float32, device=dev)
@@ -38,7 +38,13 @@ def separate_kernels(pkg, torch, q, k, v, B, H, S, T, D, divisor, layout):
     pkg.sgemm_general(q, k, scores, S, T, D, ldq, ldk, T, trans_b=True, batch_outer=B, batch_inner=H,
                       strides=(sq[0], sk, H * S * T), inner_strides=(iq, ik, S * T))
     probs = torch.empty_like(scores)
-    if divisor is None:
+    if mask is not None:
+        # Div, Add and Softmax as the nodes of a graph run them: one kernel each
+        if divisor is not None:
+            scores = pkg.transform2(scores, divisor, 0.0)
+        scores = pkg.math_binary("add", scores, mask)
+        pkg.check(pkg.lib().tfcc_rocm_softmax_f32(pkg._stream(), scores.data_ptr(), B * H * S, T, probs.data_ptr()))
+    elif divisor is None:
         pkg.check(pkg.lib().tfcc_rocm_softmax_f32(pkg._stream(), scores.data_ptr(), B * H * S, T, probs.data_ptr()))
     else:
         pkg.check(pkg.lib().tfcc_rocm_softmax_div_f32(pkg._stream(), scores.data_ptr(), B * H * S, T, divisor,
@@ -99,6 +105,40 @@ def test_attention_equals_separate_kernels(pkg, gpu, B, H, S, Tk, D, divisor, la
     assert np.array_equal(got, want), "fused and separate kernels differ by %g" % np.abs(got - want).max()
     ref = reference64(to_bhxd(q), to_bhxd(k), to_bhxd(v), divisor)
     assert rel_fro(to_bhxd(got), ref) <= 1e-5
+
+
+@pytest.mark.parametrize("B,H,S,Tk,D,divisor,per_head", [
+    (2, 12, 128, 128, 64, 8.0, False),   # the encoder layer's attention core with a [B, 1, 1, T] mask
+    (3, 2, 70, 100, 36, 6.0, False), (2, 3, 33, 65, 16, None, False), (2, 4, 40, 24, 32, 5.0, True),
+    (1, 2, 5, 7, 8, 3.0, False),
+])
+def test_attention_with_mask_equals_separate_kernels(pkg, gpu, B, H, S, Tk, D, divisor, per_head):
+    """A mask [B, 1, 1, T] (or [B, H, 1, T]) added between the division and the softmax, as BERT graphs do:
+    large negative entries for padded keys, whose probabilities must come out as exact zeros."""
+    import torch
+    rng = np.random.default_rng(B * 100 + S + Tk)
+    q = rng.standard_normal((B, S, H, D)).astype(np.float32)
+    k = rng.standard_normal((B, Tk, H, D)).astype(np.float32)
+    v = rng.standard_normal((B, Tk, H, D)).astype(np.float32)
+    mask = np.where(rng.random((B, H if per_head else 1, 1, Tk)) < 0.3, -10000.0, 0.0).astype(np.float32)
+    mask[..., 0] = 0.0  # at least one live key per row
+    mask += rng.normal(0, 0.1, mask.shape).astype(np.float32)
+    tq, tk, tv, tm = gpu.t(q), gpu.t(k), gpu.t(v), gpu.t(mask)
+    out = torch.full((B, S, H, D), float("nan"), dtype=torch.float32, device=tq.device)
+    desc = pkg.attention_desc(tq, tk, tv, out, S, Tk, D, (H * D,) * 4, batch_outer=B, batch_inner=H,
+                              strides=(S * H * D, Tk * H * D, Tk * H * D, S * H * D), inner_strides=(D,) * 4,
+                              divisor=divisor, mask=tm,
+                              mask_strides=((H if per_head else 1) * Tk, Tk if per_head else 0))
+    assert pkg.attention_supported(desc)
+    pkg.attention(desc)
+    got = gpu.n(out)
+    want = gpu.n(separate_kernels(pkg, torch, tq, tk, tv, B, H, S, Tk, D, divisor, "bshd", mask=tm))
+    assert np.isfinite(got).all() and np.array_equal(got, want)
+    s64 = np.einsum("bshd,bthd->bhst", q.astype(np.float64), k.astype(np.float64))
+    s64 = (s64 / divisor if divisor is not None else s64) + mask
+    e = np.exp(s64 - s64.max(-1, keepdims=True))
+    ref = np.einsum("bhst,bthd->bshd", e / e.sum(-1, keepdims=True), v.astype(np.float64))
+    assert rel_fro(got, ref) <= 1e-5
 
 
 def test_attention_limits_are_reported(pkg, gpu):

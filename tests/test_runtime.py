@@ -254,6 +254,28 @@ def test_fused_graph_is_bit_identical_to_the_graph_as_written(mf, rt, dev):
         fused.set_replay(True)
         for _ in range(3):
             assert np.array_equal(fused.run({"hidden_states": x})["layer_output"], want)
+    # the same layer with an attention mask added between the division and the softmax (one more node in the
+    # one-launch step; with 160 keys the fallback runs division, addition and softmax one after the other)
+    for batch, seq, hidden, heads, ffn in ((2, 16, 64, 4, 128), (3, 40, 96, 3, 200), (1, 160, 64, 2, 128)):
+        w = mf.bert_layer_weights(rng, hidden, ffn)
+        g = mf.bert_encoder_layer(w, batch, seq, heads, with_mask=True)
+        blob = mf.write_model([g], g.name)
+        feeds = {"hidden_states": rng.normal(size=(batch, seq, hidden)).astype(np.float32),
+                 "attention_mask": np.where(rng.random((batch, 1, 1, seq)) < 0.3, -10000.0, 0.0).astype(np.float32)}
+        feeds["attention_mask"][..., 0] = 0.0
+        rt.set_fusion(False)
+        plain = rt.Model(blob)
+        want = plain.run(feeds)["layer_output"]
+        rt.set_fusion(True)
+        fused = rt.Model(blob)
+        assert plain.step_count() - fused.step_count() == 13
+        assert np.array_equal(fused.run(feeds)["layer_output"], want)
+        # the mask matters: without the masked keys the output differs
+        other = dict(feeds, attention_mask=np.zeros_like(feeds["attention_mask"]))
+        assert not np.array_equal(fused.run(other)["layer_output"], want)
+        # against float64: the encoder layer of the reference model with the mask added to the scores
+        ref = bert_reference.encoder_layer(feeds["hidden_states"], w, heads, mask=feeds["attention_mask"])
+        assert rel_frobenius(want, ref) <= 1e-5
     # an Add whose other operand does not have the product's shape runs unfused, same result
     g = mf.GraphBuilder("g")
     a = g.input("a", mf.FLOAT, [5, 8])

@@ -66,6 +66,7 @@ class AttentionDesc(C.Structure):
         ("inner_stride_q", C.c_uint64), ("inner_stride_k", C.c_uint64), ("inner_stride_v", C.c_uint64),
         ("inner_stride_out", C.c_uint64),
         ("divisor", C.c_float), ("has_divisor", C.c_int),
+        ("mask", C.c_void_p), ("stride_mask", C.c_uint64), ("inner_stride_mask", C.c_uint64),
     ]
 
 
@@ -269,7 +270,7 @@ def sgemm_general(a, b, c, m, n, k, lda, ldb, ldc, trans_b=False, batch_outer=1,
 
 
 def attention_desc(q, k, v, out, s, t, d, ld, batch_outer=1, batch_inner=1, strides=(0, 0, 0, 0),
-                   inner_strides=(0, 0, 0, 0), divisor=None):
+                   inner_strides=(0, 0, 0, 0), divisor=None, mask=None, mask_strides=(0, 0)):
     """A tfcc_rocm_attention_desc over torch tensors used as raw buffers; ld = (ldq, ldk, ldv, ldo)."""
     a = AttentionDesc()
     a.q, a.k, a.v, a.out = _ptr(q), _ptr(k), _ptr(v), _ptr(out)
@@ -280,6 +281,8 @@ def attention_desc(q, k, v, out, s, t, d, ld, batch_outer=1, batch_inner=1, stri
     a.inner_stride_q, a.inner_stride_k, a.inner_stride_v, a.inner_stride_out = inner_strides
     a.divisor = 1.0 if divisor is None else divisor
     a.has_divisor = 0 if divisor is None else 1
+    a.mask = None if mask is None else _ptr(mask)
+    a.stride_mask, a.inner_stride_mask = mask_strides
     return a
 
 

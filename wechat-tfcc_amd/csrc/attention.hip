@@ -43,6 +43,8 @@ struct AttentionParams {
   unsigned batchInner, blocksS, total, chunk;
   float divisor;
   int divide;
+  const float* mask;  // optional: one value per key column, added to the (divided) scores of every query row
+  unsigned long long outerM, innerM;
 };
 
 __device__ __forceinline__ float wave_sum(float v) {
@@ -76,6 +78,15 @@ __global__ __launch_bounds__(kThreads, 4) void attention_kernel(const AttentionP
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  // this lane's two mask values, fetched now: the softmax phase that adds them is far away
+  const bool masked = p.mask != nullptr;
+  float mk[2] = {0.f, 0.f};
+  if (masked) {
+    const float* __restrict__ mrow = p.mask + (size_t)bo * p.outerM + (size_t)bn * p.innerM;
+#pragma unroll
+    for (int q = 0; q < 2; ++q)
+      if ((unsigned)lane + 64u * q < T) mk[q] = mrow[lane + 64 * q];
+  }
   const int lrow = lane & 31, g = lane >> 5;
   const unsigned Dp = (D + 7u) & ~7u;   // k extent of the score product
   const unsigned Tp = (T + 7u) & ~7u;   // k extent of the second product
@@ -194,7 +205,7 @@ __global__ __launch_bounds__(kThreads, 4) void attention_kernel(const AttentionP
 #pragma unroll
         for (int q = 0; q < 2; ++q) {
           const unsigned i = lane + 64 * q;
-          v[u][q] = i < T ? sc[i] : -FLT_MAX;
+          v[u][q] = i < T ? (masked ? sc[i] + mk[q] : sc[i]) : -FLT_MAX;
           mx[u] = fmaxf(mx[u], v[u][q]);
         }
       }
@@ -320,6 +331,9 @@ extern "C" int tfcc_rocm_attention_f32(void* stream, const tfcc_rocm_attention_d
   p.chunk = (p.total + 7) / 8;
   p.divisor = d->divisor;
   p.divide = d->has_divisor ? 1 : 0;
+  p.mask = d->mask;
+  p.outerM = d->stride_mask;
+  p.innerM = d->inner_stride_mask;
   constexpr size_t ldsBytes = (size_t)kLdsFloats * sizeof(float);
   static_assert(ldsBytes <= 80 * 1024, "two workgroups per CU");
   static bool attrSet[16] = {};

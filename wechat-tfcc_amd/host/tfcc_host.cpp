@@ -950,7 +950,7 @@ Variable<float> matmul_permuted(const Tensor<float>& a, const std::vector<size_t
 Variable<float> attention_permuted(const Tensor<float>& q, const std::vector<size_t>& permQ, const Tensor<float>& k,
                                    const std::vector<size_t>& permK, const Tensor<float>& v,
                                    const std::vector<size_t>& permV, const std::vector<size_t>& permOut,
-                                   const float* divisor) {
+                                   const float* divisor, const Tensor<float>* mask) {
   if (dynamic_cast<ROCMDevice*>(Device::getThreadDefault()) == nullptr) throw NotImplementedError();
   if (q.size() == 0 || k.size() == 0 || v.size() == 0) throw NotImplementedError("attention_permuted: empty operand");
   const PermutedView vq = permuted_view(q.shape(), permQ), vk = permuted_view(k.shape(), permK),
@@ -995,6 +995,14 @@ Variable<float> attention_permuted(const Tensor<float>& q, const std::vector<siz
   a.divisor = divisor ? *divisor : 1.f;
   a.has_divisor = divisor ? 1 : 0;
   a.q = q.data(); a.k = k.data(); a.v = v.data();
+  if (mask != nullptr) {
+    const Shape& ms = mask->shape();
+    if (ms.size() != 4 || ms[3] != t || ms[2] != 1 || (ms[0] != 1 && ms[0] != logical[0]) || (ms[1] != 1 && ms[1] != logical[1]))
+      throw NotImplementedError("attention_permuted: the mask is not [b0 or 1, b1 or 1, 1, keys]");
+    a.mask = mask->data();
+    a.stride_mask = ms[0] == 1 ? 0 : static_cast<uint64_t>(ms[1]) * t;
+    a.inner_stride_mask = ms[1] == 1 ? 0 : t;
+  }
   if (!tfcc_rocm_attention_f32_supported(&a)) throw NotImplementedError("attention_permuted: outside the kernel's limits");
   Variable<float> result{Shape(outDims)};
   a.out = result.data();

@@ -106,10 +106,12 @@ std::vector<Variable<float>> matmul_grouped(const Tensor<float>& a, const std::v
 // The result equals the step-by-step form bit for bit.  Raises NotImplementedError when the layout or
 // the sizes are outside what the kernel takes (more than 128 keys, head size above 64, a head size or
 // strides that are not multiples of 4, size not the contiguous dimension of q, k, v and the result).
+// mask (optional): added to the divided scores before the softmax; a rank-4 tensor [b0 or 1, b1 or 1, 1, keys]
+// against scores [b0, b1, queries, keys], anything else raises NotImplementedError.
 Variable<float> attention_permuted(const Tensor<float>& q, const std::vector<size_t>& permQ, const Tensor<float>& k,
                                    const std::vector<size_t>& permK, const Tensor<float>& v,
                                    const std::vector<size_t>& permV, const std::vector<size_t>& permOut,
-                                   const float* divisor);
+                                   const float* divisor, const Tensor<float>* mask = nullptr);
 }  // namespace blas
 namespace math {
 // softmax(a / divisor, axis)

@@ -290,8 +290,9 @@ def bert_layer_weights(rng, hidden=768, ffn=3072, std=0.02):
     return w
 
 
-def bert_encoder_layer(weights, batch, seq, heads, epsilon=1e-12, graph_name="encoder"):
-    """One encoder layer: input `hidden_states` [batch, seq, hidden] -> output `layer_output`."""
+def bert_encoder_layer(weights, batch, seq, heads, epsilon=1e-12, graph_name="encoder", with_mask=False):
+    """One encoder layer: input `hidden_states` [batch, seq, hidden] -> output `layer_output`.  with_mask: a second
+    input `attention_mask` [batch, 1, 1, seq] is added to the divided scores before the softmax."""
     hidden = weights["wq"].shape[0]
     size = hidden // heads
     g = GraphBuilder(graph_name)
@@ -306,6 +307,8 @@ def bert_encoder_layer(weights, batch, seq, heads, epsilon=1e-12, graph_name="en
     kt = heads_of(g.matmul(x, c["wk"], c["bk"]), [0, 2, 3, 1])       # [b, h, d, s]
     v = heads_of(g.matmul(x, c["wv"], c["bv"]), [0, 2, 1, 3])
     scores = g.binary("Div", g.matmul(q, kt), scale)
+    if with_mask:
+        scores = g.binary("Add", scores, g.input("attention_mask", FLOAT, [batch, 1, 1, seq]))
     probs = g.softmax(scores, 3)
     context = g.reshape(g.transpose(g.matmul(probs, v), [0, 2, 1, 3]), [0, 0, hidden])
     attention = g.layer_norm(g.binary("Add", g.matmul(context, c["wo"], c["bo"]), x), c["ln1_gamma"], c["ln1_beta"],

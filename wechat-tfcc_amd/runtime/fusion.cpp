@@ -151,9 +151,40 @@ std::vector<FusionPlan> plan_fusions(const proto::Graph& g, SymbolManager& sm) {
     const proto::Node& softNode = g.nodes[soft];
     if (!is_op(softNode, "math.Softmax", 1)) continue;
     if (plan[soft].kind != FusionPlan::NONE && plan[soft].kind != FusionPlan::DIV_SOFTMAX) continue;
-    const size_t div = plan[soft].kind == FusionPlan::DIV_SOFTMAX ? plan[soft].partner : FusionPlan::kNoNode;
-    const std::string& scoresName = div != FusionPlan::kNoNode ? g.nodes[div].inputs[0] : softNode.inputs[0];
-    if (!private_value(scoresName, div != FusionPlan::kNoNode ? div : soft, first)) continue;
+    size_t div = plan[soft].kind == FusionPlan::DIV_SOFTMAX ? plan[soft].partner : FusionPlan::kNoNode;
+    // Softmax(Add(scores [/ value], mask)): the Add of an attention mask, either operand order
+    size_t maskNode = FusionPlan::kNoNode, reader = div != FusionPlan::kNoNode ? div : soft;
+    unsigned maskSide = 0;
+    std::string scoresName = div != FusionPlan::kNoNode ? g.nodes[div].inputs[0] : softNode.inputs[0];
+    size_t add = 0;
+    if (div == FusionPlan::kNoNode && private_value(scoresName, soft, add) && is_op(g.nodes[add], "math.Add", 2) &&
+        plan[add].kind == FusionPlan::NONE && all_float_tensors(g.nodes[add]) &&
+        g.nodes[add].inputs[0] != g.nodes[add].inputs[1]) {
+      for (unsigned side = 0; side < 2 && maskNode == FusionPlan::kNoNode; ++side) {
+        const std::string& chain = g.nodes[add].inputs[side];
+        size_t from = 0;
+        if (!private_value(chain, add, from) || plan[from].kind == FusionPlan::ABSORBED) continue;
+        const proto::Node& fromNode = g.nodes[from];
+        const bool valueDiv = is_op(fromNode, "math.Div", 2) && plan[from].kind == FusionPlan::NONE &&
+                              float_tensor(sm, fromNode.inputs[0]) && sm.has(fromNode.inputs[1]) &&
+                              sm.getSymbolInfo(fromNode.inputs[1]).dtype == FLOAT &&
+                              is_value(sm.getSymbolInfo(fromNode.inputs[1]).stype);
+        if (valueDiv) {
+          maskNode = add;
+          maskSide = 1 - side;
+          div = from;
+          scoresName = fromNode.inputs[0];
+          reader = from;
+        } else if (is_op(fromNode, "math.Matmul", 2)) {
+          maskNode = add;
+          maskSide = 1 - side;
+          scoresName = chain;
+          reader = add;
+        }
+      }
+      if (maskNode == FusionPlan::kNoNode) continue;
+    }
+    if (!private_value(scoresName, reader, first)) continue;
     const proto::Node& firstNode = g.nodes[first];
     if (!is_op(firstNode, "math.Matmul", 2) || !all_float_tensors(firstNode)) continue;
     if (plan[first].kind != FusionPlan::NONE && plan[first].kind != FusionPlan::MATMUL_PERMUTED) continue;
@@ -163,6 +194,8 @@ std::vector<FusionPlan> plan_fusions(const proto::Graph& g, SymbolManager& sm) {
     f.scoresNode = first;
     f.softmaxNode = soft;
     f.divNode = div;
+    f.maskNode = maskNode;
+    f.maskSide = maskSide;
     if (plan[first].kind == FusionPlan::MATMUL_PERMUTED) {
       f.transposeA = plan[first].transposeA;
       f.transposeB = plan[first].transposeB;
@@ -177,6 +210,7 @@ std::vector<FusionPlan> plan_fusions(const proto::Graph& g, SymbolManager& sm) {
     plan[first] = simple_plan(FusionPlan::ABSORBED, j);
     plan[soft] = simple_plan(FusionPlan::ABSORBED, j);
     if (div != FusionPlan::kNoNode) plan[div] = simple_plan(FusionPlan::ABSORBED, j);
+    if (maskNode != FusionPlan::kNoNode) plan[maskNode] = simple_plan(FusionPlan::ABSORBED, j);
     for (size_t t2 : {f.transposeA, f.transposeB, f.transposeV, f.transposeC})
       if (t2 != FusionPlan::kNoNode) plan[t2] = simple_plan(FusionPlan::ABSORBED, j);
   }
@@ -281,19 +315,29 @@ void emit_fused(const proto::Graph& g, const FusionPlan& f, size_t j, Graph& gra
                               po = perm_of(f.transposeC);
     const float* divisor = f.divNode != FusionPlan::kNoNode ? sm.getValue(g.nodes[f.divNode].inputs[1], float()) : nullptr;
     const size_t axis = softmax_axis(g.nodes[f.softmaxNode]);
+    const Tensor<float>* mask =
+        f.maskNode != FusionPlan::kNoNode ? sm.getTensor(g.nodes[f.maskNode].inputs[f.maskSide], float()) : nullptr;
+    const bool maskFirst = f.maskSide == 0;
     Variable<float>* result =
         sm.getVariable(f.transposeC != FusionPlan::kNoNode ? g.nodes[f.transposeC].outputs[0] : n.outputs[0], float());
-    graph.addStep([q, k, v, pq, pk, pv, po, divisor, axis, result] {
+    graph.addStep([q, k, v, pq, pk, pv, po, divisor, axis, mask, maskFirst, result] {
       if (axis == 3 && q->shape().size() == 4 && k->shape().size() == 4 && v->shape().size() == 4) {
         try {
-          *result = rocm::blas::attention_permuted(*q, pq, *k, pk, *v, pv, po, divisor);
+          *result = rocm::blas::attention_permuted(*q, pq, *k, pk, *v, pv, po, divisor, mask);
           return;
         } catch (NotImplementedError&) {
-          // longer sequences, wider heads or another layout: the three steps one after the other
+          // longer sequences, wider heads, another layout or mask shape: the steps one after the other
         }
       }
       Variable<float> scores = permuted_product(*q, pq, *k, pk, {});
-      Variable<float> probabilities = divided_softmax(scores, divisor, axis);
+      Variable<float> probabilities;
+      if (mask == nullptr) {
+        probabilities = divided_softmax(scores, divisor, axis);
+      } else {
+        if (divisor != nullptr) scores = scores / *divisor;
+        Variable<float> masked = maskFirst ? *mask + scores : scores + *mask;
+        probabilities = math::softmax(masked, axis);
+      }
       *result = permuted_product(probabilities, {}, *v, pv, po);
     });
     return;

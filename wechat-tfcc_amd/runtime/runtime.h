@@ -280,6 +280,9 @@ struct FusionPlan {
   // Softmax and the Transpose of the second Matmul's other operand; transposeA / transposeB are those of
   // the first Matmul, transposeC that of the second
   size_t scoresNode = kNoNode, softmaxNode = kNoNode, divNode = kNoNode, transposeV = kNoNode;
+  // ... and the Add of a mask between the (divided) scores and the Softmax; maskSide: which input of it the mask is
+  size_t maskNode = kNoNode;
+  unsigned maskSide = 0;
   // MATMUL_GROUPED: the MatmulWithBias nodes (this one first) that share their first input and run as one launch
   std::vector<size_t> group;
 };
