@@ -89,6 +89,28 @@ def test_sgemm_with_few_rows(pkg, T, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [
+    # few tiles and a long K (four and two K groups in the kernels for B as stored), many tiles (one group),
+    # K not a multiple of 32 (the register-staged kernels' own rule), ragged edges, nine rows
+    (128, 96, 1024), (96, 96, 2048), (640, 640, 512), (512, 512, 512), (1024, 768, 768), (2048, 4096, 64),
+    (100, 52, 36), (300, 260, 1000), (64 * 20, 64 * 16, 508), (9, 3072, 768), (33, 36, 96),
+])
+def test_sgemm_with_b_given_transposed_equals_transpose_then_multiply(pkg, T, m, n, k):
+    """B handed over as [n, k] (trans_b) is summed with the K groups the kernels for [k, n] would use: the same bits
+    as transposing B first, whatever the shape."""
+    import torch
+    print("sgemm trans_b", m, n, k, flush=True)
+    rng = np.random.default_rng(m + n * 3 + k * 7)
+    a = rng.normal(0, 1, (m, k)).astype(np.float32)
+    bt = rng.normal(0, 1, (n, k)).astype(np.float32)
+    ta, tbt = T.t(a), T.t(bt)
+    c = torch.empty((m, n), dtype=torch.float32, device=ta.device)
+    pkg.sgemm_general(ta, tbt, c, m, n, k, k, k, n, trans_b=True)
+    plain = T.n(pkg.blas_matmul(ta, T.t(np.ascontiguousarray(bt.T))))
+    assert np.array_equal(T.n(c), plain)
+    assert rel_fro(plain, a.astype(np.float64) @ bt.T.astype(np.float64)) <= FP32_TOL
+
+
+@pytest.mark.parametrize("m,n,k", [
     # direct-to-LDS kernel: 256x256 tiles from 192 tiles on, 128x128 below; K not a multiple of the 128-byte slab
     (256 * 12, 256 * 16, 144), (256 * 12 - 1, 256 * 16, 144), (256 * 11, 256 * 16, 272), (512, 384, 4000),
     # 64x128 tiles below 128 tiles of 128x128 (1024 x 768 has 48), 128x128 from there on; ragged edges

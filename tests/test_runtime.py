@@ -340,6 +340,48 @@ def test_fused_graph_is_bit_identical_to_the_graph_as_written(mf, rt, dev):
         assert rel_frobenius(outs[1], want) <= 1e-5
 
 
+@pytest.mark.gpu
+def test_gemm_lowering_patterns_fused_and_plain_agree(mf, rt, dev):
+    """What the converter makes of an ONNX Gemm (tfcc_code_generator/frontend/onnx/converter/math/gemm.py:22-92):
+    Transpose nodes in front of Matmul / MatmulWithBias.  A transposed constant weight is transposed once and kept;
+    a transposed activation is multiplied as it lies; a transposed first operand falls back to the nodes as written.
+    Every form gives the bits of the plain graph."""
+    rng = np.random.default_rng(17)
+    cases = [
+        # m, k, n, bias, transA, transB, B constant
+        (64, 768, 96, True, False, True, True),      # Linear layer: x W^T + b, four K groups
+        (640, 512, 640, True, False, True, True),
+        (64, 768, 96, True, False, True, False),     # the same with W an input: multiplied as stored
+        (100, 36, 52, False, False, True, False), (300, 1000, 260, True, False, True, False),
+        (5, 64, 48, True, False, True, False),       # at most eight rows: the separate steps
+        (48, 40, 56, True, True, False, True), (33, 96, 36, False, True, True, False),
+    ]
+    for m, k, n, with_bias, trans_a, trans_b, const_b in cases:
+        g = mf.GraphBuilder("g")
+        av = rng.normal(size=(k, m) if trans_a else (m, k)).astype(np.float32)
+        bv = rng.normal(size=(n, k) if trans_b else (k, n)).astype(np.float32)
+        biasv = rng.normal(size=n).astype(np.float32)
+        a = g.input("a", mf.FLOAT, list(av.shape))
+        b = g.constant("w", bv) if const_b else g.input("b", mf.FLOAT, list(bv.shape))
+        left = g.transpose(a, [1, 0]) if trans_a else a
+        right = g.transpose(b, [1, 0]) if trans_b else b
+        y = g.matmul(left, right, g.constant("bias", biasv) if with_bias else None)
+        g.output(y)
+        feeds = {"a": av} if const_b else {"a": av, "b": bv}
+        blob = mf.write_model([g], "g")
+        rt.set_fusion(False)
+        plain = rt.Model(blob)
+        want = plain.run(feeds)[y]
+        rt.set_fusion(True)
+        fused = rt.Model(blob)
+        assert plain.step_count() - fused.step_count() == int(trans_a) + int(trans_b)
+        for _ in range(3):  # the second and third run use the kept copy of a transposed constant
+            assert np.array_equal(fused.run(feeds)[y], want), (m, k, n, trans_a, trans_b, const_b)
+        ref = (av.T if trans_a else av).astype(np.float64) @ (bv.T if trans_b else bv).astype(np.float64)
+        assert rel_frobenius(want, ref + (biasv if with_bias else 0)) <= 1e-5
+    rt.set_fusion(True)
+
+
 UNARY_NUMPY = {
     # expressions of tfcc/mkl/kernel/tfcc_mklactivationkernel.hpp:48-110,222-228,284-291 and of
     # tfcc_runtime/operations/math/neg.cpp:30, reciprocal.cpp:31, sqrt.cpp:31, evaluated in float64

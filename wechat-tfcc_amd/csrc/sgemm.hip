@@ -373,6 +373,52 @@ int launch(hipStream_t stream, SgemmParams p) {
   return check_launch("sgemm");
 }
 
+// The tile table of the kernels that copy K slabs straight into LDS, ordered by falling tile area.
+const struct { int config; unsigned bm, bn, waves; } kTiles[] = {{0, 64, 64, 4}, {1, 32, 96, 3}, {2, 32, 64, 2}, {3, 32, 32, 1}};
+
+// Tile and number of K groups for m x n x k with K a multiple of 32: the tile that covers the 256 CUs in the fewest
+// tile-area rounds, the larger one on a tie (less operand traffic); as few K groups as give every CU eight
+// wavefronts, each group keeping at least four slabs.
+void choose_dma_tiles(unsigned m, unsigned n, unsigned k, unsigned fillBatch, int& best, unsigned long long& bestTiles,
+                      int& ksplit) {
+  best = 0;
+  unsigned long long bestCost = ~0ull;
+  bestTiles = 0;
+  for (int c = 0; c < 4; ++c) {
+    const unsigned long long tiles =
+        (unsigned long long)((m + kTiles[c].bm - 1) / kTiles[c].bm) * ((n + kTiles[c].bn - 1) / kTiles[c].bn) * fillBatch;
+    const unsigned long long cost = ((tiles + 255) / 256) * (kTiles[c].bm * kTiles[c].bn);
+    if (cost < bestCost) {
+      best = c;
+      bestCost = cost;
+      bestTiles = tiles;
+    }
+  }
+  ksplit = 1;
+  while (ksplit < 4 && bestTiles * kTiles[best].waves * ksplit < 256ull * 8 && k >= 128u * (ksplit * 2)) ksplit *= 2;
+}
+
+// The number of K groups the kernels for B as stored [k, n] would sum this product with (the sums of an element
+// are defined by it, not by the tile shape): B given transposed must use the same, so that transposing B first
+// and multiplying give the same bits as multiplying the transposed view.
+int k_groups_of_plain_product(unsigned m, unsigned n, unsigned k, unsigned fillBatch) {
+  const unsigned long long big = (unsigned long long)((m + 127) / 128) * ((n + 127) / 128) * fillBatch;
+  if (big >= 512) return 1;
+  if (k % 32 == 0) {
+    int best, ksplit;
+    unsigned long long tiles;
+    choose_dma_tiles(m, n, k, fillBatch, best, tiles, ksplit);
+    return ksplit;
+  }
+  const unsigned long long small = (unsigned long long)((m + 63) / 64) * ((n + 63) / 64) * fillBatch;
+  const unsigned long long flat = (unsigned long long)((m + 31) / 32) * ((n + 95) / 96) * fillBatch;
+  const bool preferFlat = ((flat + 255) / 256) * (32 * 96) < ((small + 255) / 256) * (64 * 64);
+  if (preferFlat && flat <= 320 && k >= 512) return 4;
+  if (small <= 320 && k >= 512) return 4;
+  if (small <= 640 && k >= 256) return 2;
+  return 1;
+}
+
 // Picks the tile configuration from the shape of one product and the number of batch entries that
 // count towards filling the chip (`fillBatch`), and launches.
 int dispatch(hipStream_t s, const SgemmParams& p, bool vec, bool tb, unsigned fillBatch, unsigned lda, unsigned ldb,
@@ -380,7 +426,12 @@ int dispatch(hipStream_t s, const SgemmParams& p, bool vec, bool tb, unsigned fi
   const unsigned m = p.M, n = p.N, k = p.K;
   const unsigned long long rowsB = tb ? n : k;
   if (tb) {
-    if (vec) return launch<2, 2, 1, 1, true, 1, true>(s, p);
+    if (vec) {
+      const int groups = k_groups_of_plain_product(m, n, k, fillBatch);
+      if (groups == 4) return launch<2, 2, 1, 1, true, 4, true>(s, p);
+      if (groups == 2) return launch<2, 2, 1, 1, true, 2, true>(s, p);
+      return launch<2, 2, 1, 1, true, 1, true>(s, p);
+    }
     TFCC_REQUIRE((unsigned long long)m * ldc < (1ull << 32) && (unsigned long long)m * lda < (1ull << 32) &&
                  rowsB * ldb < (1ull << 32), "sgemm: operand larger than 2^32 elements");
     return launch<2, 2, 1, 1, false, 1, true>(s, p);
@@ -399,25 +450,10 @@ int dispatch(hipStream_t s, const SgemmParams& p, bool vec, bool tb, unsigned fi
     const unsigned long long flat = (unsigned long long)((m + 31) / 32) * ((n + 95) / 96) * fillBatch;
     const bool preferFlat = ((flat + 255) / 256) * (32 * 96) < ((small + 255) / 256) * (64 * 64);
     if (k % 32 == 0) {
-      // Whole slabs of K: the kernels that copy the slabs straight into LDS.  Tile: the one that covers the
-      // 256 CUs in the fewest tile-area rounds, the larger one on a tie (less operand traffic).  K groups:
-      // as few as give every CU eight wavefronts, each group keeping at least four slabs.
-      static const struct { int config; unsigned bm, bn, waves; } kTiles[] = {
-          {0, 64, 64, 4}, {1, 32, 96, 3}, {2, 32, 64, 2}, {3, 32, 32, 1}};
-      int best = 0;
-      unsigned long long bestCost = ~0ull, bestTiles = 0;
-      for (int c = 0; c < 4; ++c) {
-        const unsigned long long tiles =
-            (unsigned long long)((m + kTiles[c].bm - 1) / kTiles[c].bm) * ((n + kTiles[c].bn - 1) / kTiles[c].bn) * fillBatch;
-        const unsigned long long cost = ((tiles + 255) / 256) * (kTiles[c].bm * kTiles[c].bn);
-        if (cost < bestCost) {  // the table is ordered by falling tile area
-          best = c;
-          bestCost = cost;
-          bestTiles = tiles;
-        }
-      }
-      int ksplit = 1;
-      while (ksplit < 4 && bestTiles * kTiles[best].waves * ksplit < 256ull * 8 && k >= 128u * (ksplit * 2)) ksplit *= 2;
+      // whole slabs of K: the kernels that copy the slabs straight into LDS
+      int best, ksplit;
+      unsigned long long bestTiles;
+      choose_dma_tiles(m, n, k, fillBatch, best, bestTiles, ksplit);
       // Several products in one launch (p.batch counts them; fillBatch = 1 chose the configuration of a single
       // one so that each is summed exactly as on its own): when they fill the chip without the K groups, one
       // group per tile plays all of them.

@@ -872,21 +872,26 @@ struct PermutedView {
   uint64_t strides[4];
 };
 // dims and element strides of transpose(t, perm) seen on t's dense storage
+// Tensors of rank 2 and 3 count as rank 4 with leading dimensions of 1.
 PermutedView permuted_view(const Shape& shape, const std::vector<size_t>& perm) {
-  if (shape.size() != 4 || (!perm.empty() && perm.size() != 4)) throw NotImplementedError("matmul_permuted: rank 4 only");
+  const size_t rank = shape.size();
+  if (rank < 2 || rank > 4 || (!perm.empty() && perm.size() != rank)) throw NotImplementedError("matmul_permuted: rank 2 to 4");
+  const size_t pad = 4 - rank;
+  unsigned full[4] = {1, 1, 1, 1};
+  for (size_t i = 0; i < rank; ++i) full[pad + i] = shape[i];
   uint64_t dense[4];
   uint64_t acc = 1;
   for (int i = 3; i >= 0; --i) {
     dense[i] = acc;
-    acc *= shape[i];
+    acc *= full[i];
   }
   bool seen[4] = {false, false, false, false};
   PermutedView v;
   for (size_t i = 0; i < 4; ++i) {
-    const size_t src = perm.empty() ? i : perm[i];
+    const size_t src = (perm.empty() || i < pad) ? i : pad + perm[i - pad];
     if (src >= 4 || seen[src]) throw InvalidArgumentError("invalid perm");
     seen[src] = true;
-    v.dims[i] = shape[src];
+    v.dims[i] = full[src];
     v.strides[i] = dense[src];
   }
   return v;
@@ -894,30 +899,39 @@ PermutedView permuted_view(const Shape& shape, const std::vector<size_t>& perm) 
 }  // namespace
 
 Variable<float> matmul_permuted(const Tensor<float>& a, const std::vector<size_t>& permA, const Tensor<float>& b,
-                                const std::vector<size_t>& permB, const std::vector<size_t>& permC) {
+                                const std::vector<size_t>& permB, const std::vector<size_t>& permC,
+                                const Tensor<float>* bias) {
   if (dynamic_cast<ROCMDevice*>(Device::getThreadDefault()) == nullptr) throw NotImplementedError();
+  if (a.shape().size() != b.shape().size()) throw NotImplementedError("matmul_permuted: operands of different rank");
+  const size_t rank = a.shape().size();
+  if (!permC.empty() && permC.size() != rank) throw InvalidArgumentError("invalid perm");
   const PermutedView va = permuted_view(a.shape(), permA), vb = permuted_view(b.shape(), permB);
   if (va.dims[0] != vb.dims[0] || va.dims[1] != vb.dims[1] || va.dims[3] != vb.dims[2]) throw InvalidArgumentError("shape invalid");
   if (a.size() == 0 || b.size() == 0) throw NotImplementedError("matmul_permuted: empty operand");
   const unsigned m = va.dims[2], k = va.dims[3], n = vb.dims[3];
   // the result tensor: dims of [B0, B1, m, n] permuted by permC, dense
+  if (bias != nullptr && (bias->shape().size() != 1 || bias->size() != n)) throw InvalidArgumentError("shape invalid");
   const unsigned logical[4] = {va.dims[0], va.dims[1], m, n};
-  std::vector<unsigned> outDims(4);
+  const size_t pad = 4 - rank;
+  std::vector<unsigned> outDims4(4);
   uint64_t cStride[4] = {0, 0, 0, 0};
   {
     bool seen[4] = {false, false, false, false};
+    size_t srcOf[4];
     for (size_t p = 0; p < 4; ++p) {
-      const size_t src = permC.empty() ? p : permC[p];
-      if ((!permC.empty() && permC.size() != 4) || src >= 4 || seen[src]) throw InvalidArgumentError("invalid perm");
+      const size_t src = (permC.empty() || p < pad) ? p : pad + permC[p - pad];
+      if (src >= 4 || seen[src]) throw InvalidArgumentError("invalid perm");
       seen[src] = true;
-      outDims[p] = logical[src];
+      srcOf[p] = src;
+      outDims4[p] = logical[src];
     }
     uint64_t acc = 1;
     for (int p = 3; p >= 0; --p) {
-      cStride[permC.empty() ? p : permC[p]] = acc;
-      acc *= outDims[p];
+      cStride[srcOf[p]] = acc;
+      acc *= outDims4[p];
     }
   }
+  const std::vector<unsigned> outDims(outDims4.begin() + pad, outDims4.end());
   if (va.strides[3] != 1 && k != 1) throw NotImplementedError("matmul_permuted: k is not contiguous in a");
   if (cStride[3] != 1 && n != 1) throw NotImplementedError("matmul_permuted: n is not contiguous in the result");
   tfcc_rocm_sgemm_desc d{};
@@ -937,8 +951,13 @@ Variable<float> matmul_permuted(const Tensor<float>& a, const std::vector<size_t
   if (d.lda < k) d.lda = k;
   if (d.ldc < n) d.ldc = n;
   if (d.ldb < (d.trans_b ? k : n)) d.ldb = d.trans_b ? k : n;
+  // a lone product of at most eight rows with B as stored runs on the streaming kernel, whose sums are ordered
+  // differently from the tiled kernel a transposed B needs: leave that case to the separate steps
+  if (d.trans_b && m <= 8 && static_cast<uint64_t>(logical[0]) * logical[1] == 1)
+    throw NotImplementedError("matmul_permuted: a single product of at most eight rows with a transposed b");
   Variable<float> result{Shape(outDims)};
   d.a = a.data(); d.b = b.data(); d.c = result.data();
+  d.bias = bias ? bias->data() : nullptr;
   d.m = m; d.n = n; d.k = k;
   d.batch_outer = logical[0]; d.batch_inner = logical[1];
   d.stride_a = va.strides[0]; d.inner_stride_a = va.strides[1];

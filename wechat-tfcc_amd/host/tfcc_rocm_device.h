@@ -88,13 +88,14 @@ enum class Activation { NONE = 0, GELU = 1 };
 // Checks and shape rules of tfcc::blas::matmul.
 Variable<float> matmul_fused(const Tensor<float>& a, const Tensor<float>& b, const Tensor<float>* bias,
                              const Tensor<float>* residual, Activation activation);
-// transpose(matmul(transpose(a, permA), transpose(b, permB)), permC) for rank-4 tensors without
-// materialising any of the three permutations (an empty perm is the identity): the kernel walks the
+// transpose(matmul(transpose(a, permA), transpose(b, permB)) [+ bias], permC) for tensors of one rank from 2 to 4
+// without materialising any of the three permutations (an empty perm is the identity): the kernel walks the
 // operands through their strides.  Needs the k dimension of the permuted a, the k or the n dimension
 // of the permuted b and the n dimension of the result to be the contiguous one of their tensors;
 // anything else raises NotImplementedError.  Results equal the step-by-step form bit for bit.
 Variable<float> matmul_permuted(const Tensor<float>& a, const std::vector<size_t>& permA, const Tensor<float>& b,
-                                const std::vector<size_t>& permB, const std::vector<size_t>& permC);
+                                const std::vector<size_t>& permB, const std::vector<size_t>& permC,
+                                const Tensor<float>* bias = nullptr);
 // { a * b[g] + bias[g] } for up to four weight matrices of one shape ([k, n], rank 2) in a single launch;
 // a: [..., k] of any rank >= 2 (its leading dimensions are the rows).  Each result equals
 // tfcc::blas::matmul(a, b[g], bias[g]) bit for bit.  Raises NotImplementedError for anything else.

@@ -125,6 +125,22 @@ std::vector<FusionPlan> plan_fusions(const proto::Graph& g, SymbolManager& sm) {
         for (size_t t2 : {f.transposeA, f.transposeB, f.transposeC})
           if (t2 != FusionPlan::kNoNode) plan[t2] = simple_plan(FusionPlan::ABSORBED, j);
       }
+    } else if (is_op(n, "math.MatmulWithBias", 3) && float_variable(sm, n.outputs[0]) && all_float_tensors(n)) {
+      // what the converter makes of an ONNX Gemm with transA / transB (tfcc_code_generator/frontend/onnx/converter/
+      // math/gemm.py:37-68): Transpose nodes in front of the product's operands
+      FusionPlan f;
+      f.kind = FusionPlan::MATMUL_PERMUTED;
+      size_t t = 0;
+      if (sole_producer(n.inputs[0], j, t) && is_op(g.nodes[t], "base.Transpose", 1) && float_tensor(sm, g.nodes[t].inputs[0]))
+        f.transposeA = t;
+      if (n.inputs[1] != n.inputs[0] && sole_producer(n.inputs[1], j, t) && is_op(g.nodes[t], "base.Transpose", 1) &&
+          float_tensor(sm, g.nodes[t].inputs[0]))
+        f.transposeB = t;
+      if (f.transposeA != FusionPlan::kNoNode || f.transposeB != FusionPlan::kNoNode) {
+        plan[j] = f;
+        for (size_t t2 : {f.transposeA, f.transposeB})
+          if (t2 != FusionPlan::kNoNode) plan[t2] = simple_plan(FusionPlan::ABSORBED, j);
+      }
     } else if (is_op(n, "base.Identity", 1) && float_variable(sm, n.outputs[0]) && float_variable(sm, n.inputs[0]) &&
                producer.count(n.inputs[0]) && producer[n.inputs[0]] < j && consumers[n.inputs[0]].size() == 1 &&
                !kept.count(n.inputs[0])) {
@@ -273,10 +289,11 @@ size_t softmax_axis(const proto::Node& n) {
 
 // transpose(matmul(transpose(a, pa), transpose(b, pb)), pc); an empty perm stands for no Transpose node
 Variable<float> permuted_product(const Tensor<float>& a, const std::vector<size_t>& pa, const Tensor<float>& b,
-                                 const std::vector<size_t>& pb, const std::vector<size_t>& pc) {
+                                 const std::vector<size_t>& pb, const std::vector<size_t>& pc,
+                                 const Tensor<float>* bias = nullptr) {
   if (!pa.empty() || !pb.empty() || !pc.empty()) {
     try {
-      return rocm::blas::matmul_permuted(a, pa, b, pb, pc);
+      return rocm::blas::matmul_permuted(a, pa, b, pb, pc, bias);
     } catch (NotImplementedError&) {
       // a layout the strided kernel does not take: run the nodes as written
     }
@@ -284,8 +301,9 @@ Variable<float> permuted_product(const Tensor<float>& a, const std::vector<size_
   Variable<float> xa, xb;
   if (!pa.empty()) xa = base::transpose(a, pa);
   if (!pb.empty()) xb = base::transpose(b, pb);
-  Variable<float> c = blas::matmul(pa.empty() ? a : static_cast<const Tensor<float>&>(xa),
-                                   pb.empty() ? b : static_cast<const Tensor<float>&>(xb));
+  const Tensor<float>& ra = pa.empty() ? a : static_cast<const Tensor<float>&>(xa);
+  const Tensor<float>& rb = pb.empty() ? b : static_cast<const Tensor<float>&>(xb);
+  Variable<float> c = bias ? blas::matmul(ra, rb, *bias) : blas::matmul(ra, rb);
   if (!pc.empty()) return base::transpose(c, pc);
   return c;
 }
@@ -372,7 +390,22 @@ void emit_fused(const proto::Graph& g, const FusionPlan& f, size_t j, Graph& gra
     const std::vector<size_t> pa = ta ? transpose_perm(g.nodes[f.transposeA]) : std::vector<size_t>();
     const std::vector<size_t> pb = tb ? transpose_perm(g.nodes[f.transposeB]) : std::vector<size_t>();
     const std::vector<size_t> pc = tc ? transpose_perm(g.nodes[f.transposeC]) : std::vector<size_t>();
-    graph.addStep([a, b, result, pa, pb, pc] { *result = permuted_product(*a, pa, *b, pb, pc); });
+    const Tensor<float>* bias = n.inputs.size() == 3 ? sm.getTensor(n.inputs[2], float()) : nullptr;
+    // A constant weight given transposed (a Linear layer exported as Gemm with transB): transposed once, at the
+    // first run, and multiplied as stored from then on - the plain graph transposes it in every run.
+    if (tb && sm.getSymbolInfo(g.nodes[f.transposeB].inputs[0]).stype == SymbolType::CONSTANT_TENSOR) {
+      auto cached = std::make_shared<Variable<float>>();
+      auto filled = std::make_shared<bool>(false);
+      graph.addStep([a, b, result, pa, pb, pc, bias, cached, filled] {
+        if (!*filled) {
+          *cached = base::transpose(*b, pb);
+          *filled = true;
+        }
+        *result = permuted_product(*a, pa, *cached, {}, pc, bias);
+      });
+      return;
+    }
+    graph.addStep([a, b, result, pa, pb, pc, bias] { *result = permuted_product(*a, pa, *b, pb, pc, bias); });
     return;
   }
   Variable<float>* out = sm.getVariable(n.outputs[0], float());
