@@ -275,6 +275,22 @@ def bench_other(torch, pkg, dev, steps, warmup, c3):
 
     attention_case("c2_fp32_attention_one_launch_16x12x128x64", 16, 12, 128, 64)
     sgemm_case("fp32_4096x4096x4096", (4096, 4096), (4096, 4096), False, sets=1)
+    # one LSTM time step (tfcc::rnn::lstm_forward's inner loop): state product and cell in one launch
+    for batch, hidden in ((1, 512), (4, 512), (8, 1024)):
+        wh = torch.randn(hidden, 4 * hidden, device=dev) * 0.05
+        inter = pkg.transpose(wh.reshape(hidden, 4, hidden), (0, 2, 1)).reshape(hidden, 4 * hidden)
+        xw, bias_l = torch.randn(batch, 4 * hidden, device=dev), torch.randn(4 * hidden, device=dev)
+        h0, c0 = torch.zeros(batch, hidden, device=dev), torch.zeros(batch, hidden, device=dev)
+        h1 = torch.empty_like(h0)
+
+        def step():
+            st = lib.tfcc_rocm_lstm_step_f32(stream, batch, hidden, h0.data_ptr(), inter.data_ptr(), xw.data_ptr(),
+                                             bias_l.data_ptr(), 0.0, c0.data_ptr(), h1.data_ptr(), c0.data_ptr())
+            if st != 0:
+                pkg.check(st)
+        ms = time_launches(torch, step, max(steps, 50), warmup, pkg, stream)
+        out["lstm_step_one_launch_batch%d_hidden%d" % (batch, hidden)] = {
+            "ms": round(ms, 5), "gbs": round(16.0 * hidden * hidden / ms / 1e6, 1)}
     # up to eight rows of A in fp32 (C5's shape and a square weight): one streaming pass over B
     sgemm_case("fp32_few_rows_m1_4096x11008", (1, 4096), (4096, 11008), False, sets=2)
     sgemm_case("fp32_few_rows_m8_4096x11008", (8, 4096), (4096, 11008), False, sets=2)

@@ -348,6 +348,14 @@ int tfcc_rocm_transpose_f32(void* stream, const float* in, const unsigned* shape
 int tfcc_rocm_lstm_cell_f32(void* stream, unsigned batch, unsigned units, const float* state_c,
                             const float* input_value, const float* state_h_value, const float* bias, float forget,
                             float* h, float* cs);
+/* One step of tfcc::rnn::lstm_forward / lstm_backward (tfcc/core/operations/tfcc_rnn.cpp:62-71) in one launch:
+ * matmul(h_prev, state kernel) and the LSTM cell above on its sums.  batch <= 8.  The state kernel is passed with its
+ * gates interleaved: element [k, 4 * u + g] = state_kernel[k, g * units + u], i.e. the [units, 4, units] view of the
+ * reference's [units, 4 * units] kernel transposed with perm (0, 2, 1) (tfcc_rocm_transpose_f32 does it once per
+ * sequence).  input_value and bias keep the reference's layout.  h must not be h_prev; cs may be state_c. */
+int tfcc_rocm_lstm_step_f32(void* stream, unsigned batch, unsigned units, const float* h_prev,
+                            const float* state_kernel_interleaved, const float* input_value, const float* bias,
+                            float forget, const float* state_c, float* h, float* cs);
 /* CellInterface::processGRUCellGates (tfcc_cellinterface.h:49-59; tfcc_mklcellkernel.hpp:89-133):
  * result [batch, input_size + units] = concat(inputs, sigmoid(value[:, :units] + bias[:units]) * state);
  * value [batch, 2 * units], bias [2 * units]. */

@@ -573,6 +573,43 @@ def test_broadcast_arithmetic_rejects_what_the_reference_rejects(pkg, T):
     assert tuple(pkg.math_binary("add", T.t(np.zeros((0, 3), np.float32)), T.t(np.zeros((1, 3), np.float32))).shape) == (0, 3)
 
 
+@pytest.mark.parametrize("seq,batch,length,hidden", [(6, 3, 48, 40), (3, 1, 32, 513), (4, 8, 64, 128), (2, 5, 16, 7)])
+def test_lstm_step_in_one_launch(pkg, T, seq, batch, length, hidden):
+    """tfcc_rocm_lstm_step_f32 (state product and cell in one launch, state kernel with interleaved gates) driven as
+    tfcc::rnn::lstm_forward drives its steps, against the oracle's sequence and against product + cell launches."""
+    import torch
+    rng = np.random.default_rng(hidden)
+    u = lambda *s: rng.uniform(-1, 1, s).astype(np.float32)  # noqa: E731
+    a, wi, wh, bias, ih, ic = u(seq, batch, length), u(length, 4 * hidden), u(hidden, 4 * hidden), u(4 * hidden), \
+        u(batch, hidden), u(batch, hidden)
+    want_out, want_h, want_c = O.lstm_sequence(a, wi, wh, bias, ih, ic)
+    xw = pkg.blas_matmul(T.t(a.reshape(seq * batch, length)), T.t(wi))
+    inter = pkg.transpose(T.t(wh.reshape(hidden, 4, hidden)), (0, 2, 1)).reshape(hidden, 4 * hidden)
+    assert np.array_equal(T.n(inter)[:, 4 * 3 + 2], wh[:, 2 * hidden + 3]) if hidden > 3 else True
+    out = torch.empty((seq, batch, hidden), dtype=torch.float32, device=xw.device)
+    c, h, dbias = T.t(ic.copy()), T.t(ih), T.t(bias)
+    for t in range(seq):
+        pkg.check(pkg.lib().tfcc_rocm_lstm_step_f32(None, batch, hidden, h.data_ptr(), inter.data_ptr(),
+                                                    xw[t * batch:].data_ptr(), dbias.data_ptr(), 0.0, c.data_ptr(),
+                                                    out[t].data_ptr(), c.data_ptr()))
+        h = out[t]
+    for got, want in ((T.n(out), want_out), (T.n(h), want_h), (T.n(c), want_c)):
+        assert np.linalg.norm(got - want) <= 1e-5 * np.linalg.norm(want)
+    # one step against the separate launches on the same operands: the same expressions on sums that differ only in
+    # the order of their partial sums
+    tih, tic = T.t(ih), T.t(ic)
+    hv = pkg.blas_matmul(tih, T.t(wh))
+    h2, c2 = pkg.lstm_cell(tic, xw[:batch].contiguous(), hv, dbias, 0.0)
+    h1 = torch.empty_like(h2)
+    c1 = torch.empty_like(c2)
+    pkg.check(pkg.lib().tfcc_rocm_lstm_step_f32(None, batch, hidden, tih.data_ptr(), inter.data_ptr(), xw.data_ptr(),
+                                                dbias.data_ptr(), 0.0, tic.data_ptr(), h1.data_ptr(), c1.data_ptr()))
+    assert np.allclose(T.n(h1), T.n(h2), rtol=1e-4, atol=1e-5) and np.allclose(T.n(c1), T.n(c2), rtol=1e-4, atol=1e-5)
+    with pytest.raises(pkg.TfccRocmError):
+        pkg.check(pkg.lib().tfcc_rocm_lstm_step_f32(None, 9, hidden, h.data_ptr(), inter.data_ptr(), xw.data_ptr(),
+                                                    dbias.data_ptr(), 0.0, c.data_ptr(), out.data_ptr(), c.data_ptr()))
+
+
 def test_elementwise_against_oracle(pkg, T):
     rng = np.random.default_rng(50)
     for shape in ((8, 12, 128, 128), (7, 33), (5, 1000)):

@@ -130,6 +130,7 @@ SYMBOLS = {
     "tfcc_rocm_binary_broadcast_f32": (_I, [_VP, _I, _VP, _VP, _I, C.POINTER(C.c_uint), C.POINTER(_U64),
                                            C.POINTER(_U64), _VP]),
     "tfcc_rocm_lstm_cell_f32": (_I, [_VP, _U, _U, _VP, _VP, _VP, _VP, _F, _VP, _VP]),
+    "tfcc_rocm_lstm_step_f32": (_I, [_VP, _U, _U, _VP, _VP, _VP, _VP, _F, _VP, _VP, _VP]),
     "tfcc_rocm_gru_cell_gates_f32": (_I, [_VP, _U, _U, _U, _VP, _VP, _VP, _VP, _VP]),
     "tfcc_rocm_gru_cell_candidate_f32": (_I, [_VP, _U, _U, _VP, _VP, _VP, _VP, _VP, _VP]),
     "tfcc_rocm_pytorch_gru_cell_f32": (_I, [_VP, _U, _U, _VP, _VP, _VP, _VP, _VP, _VP, _VP]),

@@ -22,30 +22,20 @@ constexpr int kChunk = 64;  // rows of K whose values of A a wavefront holds in 
 
 // COLS columns per wavefront (64 or 32): the 64 / COLS groups of COLS lanes take consecutive pieces of each
 // 64-row chunk, so a narrow B still spreads over many workgroups while every load covers whole 128-byte lines.
+//
+// The streaming part shared by the kernels below: the partial sums of rows 0 .. MR-1 of A times columns
+// colBase .. colBase + COLS - 1 of B, left in smem[wave][row][lane] for all sixteen wavefronts (barrier included).
 template <int MR, int COLS>
-__global__ __launch_bounds__(kWaves * 64) void sgemv_kernel(SgemmParams p) {
+__device__ __forceinline__ void stream_partial_sums(const float* __restrict__ A, unsigned lda, unsigned M,
+                                                    const float* __restrict__ B, unsigned ldb, unsigned N, unsigned K,
+                                                    unsigned colBase, float (*smem)[MR][64]) {
   constexpr int SUBS = 64 / COLS;       // lane groups of a wavefront
   constexpr int PIECE = kChunk / SUBS;  // rows of a chunk per lane group
   static_assert(PIECE % kRows == 0, "whole batches of rows per lane group");
-  // [wave][row of A][64]: first each wavefront's current 64 values of every row of A, at the end its partial sums
-  __shared__ __attribute__((aligned(16))) float smem[kWaves][MR][64];
   const unsigned lane = threadIdx.x & 63;
   const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const unsigned sub = lane / COLS, lcol = lane % COLS;
-  const unsigned bi = blockIdx.y;
-  const unsigned M = p.M, N = p.N, K = p.K;
-  const unsigned bo = bi / p.batchInner, bn = bi - bo * p.batchInner;
-  const float* __restrict__ A = p.A + (size_t)bo * p.strideA + (size_t)bn * p.innerA;
-  const float* __restrict__ B = p.B + (size_t)bo * p.strideB + (size_t)bn * p.innerB;
-  const float* biasPtr = p.bias;
-  float* Cbase = p.C + (size_t)bo * p.strideC + (size_t)bn * p.innerC;
-  if (p.groups) {
-    B = bi == 0 ? p.groupB[0] : bi == 1 ? p.groupB[1] : bi == 2 ? p.groupB[2] : p.groupB[3];
-    biasPtr = bi == 0 ? p.groupBias[0] : bi == 1 ? p.groupBias[1] : bi == 2 ? p.groupBias[2] : p.groupBias[3];
-    Cbase = bi == 0 ? p.groupC[0] : bi == 1 ? p.groupC[1] : bi == 2 ? p.groupC[2] : p.groupC[3];
-  }
-  const unsigned lda = p.lda, ldb = p.ldb, ldc = p.ldc;
-  const unsigned col = blockIdx.x * COLS + lcol;
+  const unsigned col = colBase + lcol;
   const unsigned colRead = col < N ? col : N - 1;  // lanes past the edge read a valid column and drop the sum
 
   // rows of A beyond M repeat the last one; their sums are never stored
@@ -97,17 +87,97 @@ __global__ __launch_bounds__(kWaves * 64) void sgemv_kernel(SgemmParams p) {
 #pragma unroll
   for (int m = 0; m < MR; ++m) smem[wave][m][lane] = acc[m];
   __syncthreads();
-  // row m of the result: wavefront m adds the partial sums in wavefront order, lane groups in order within each
+}
+
+// element (row, column c of the workgroup's COLS): wavefronts in order, lane groups in order within each
+template <int MR, int COLS>
+__device__ __forceinline__ float summed(float (*smem)[MR][64], unsigned row, unsigned c) {
+  float v = 0.f;
+#pragma unroll
+  for (int w = 0; w < kWaves; ++w)
+#pragma unroll
+    for (int g = 0; g < 64 / COLS; ++g) v += smem[w][row][g * COLS + c];
+  return v;
+}
+
+template <int MR, int COLS>
+__global__ __launch_bounds__(kWaves * 64) void sgemv_kernel(SgemmParams p) {
+  // [wave][row of A][64]: first each wavefront's current 64 values of every row of A, at the end its partial sums
+  __shared__ __attribute__((aligned(16))) float smem[kWaves][MR][64];
+  const unsigned lane = threadIdx.x & 63;
+  const unsigned wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const unsigned bi = blockIdx.y;
+  const unsigned M = p.M, N = p.N;
+  const unsigned bo = bi / p.batchInner, bn = bi - bo * p.batchInner;
+  const float* __restrict__ A = p.A + (size_t)bo * p.strideA + (size_t)bn * p.innerA;
+  const float* __restrict__ B = p.B + (size_t)bo * p.strideB + (size_t)bn * p.innerB;
+  const float* biasPtr = p.bias;
+  float* Cbase = p.C + (size_t)bo * p.strideC + (size_t)bn * p.innerC;
+  if (p.groups) {
+    B = bi == 0 ? p.groupB[0] : bi == 1 ? p.groupB[1] : bi == 2 ? p.groupB[2] : p.groupB[3];
+    biasPtr = bi == 0 ? p.groupBias[0] : bi == 1 ? p.groupBias[1] : bi == 2 ? p.groupBias[2] : p.groupBias[3];
+    Cbase = bi == 0 ? p.groupC[0] : bi == 1 ? p.groupC[1] : bi == 2 ? p.groupC[2] : p.groupC[3];
+  }
+  stream_partial_sums<MR, COLS>(A, p.lda, M, B, p.ldb, N, p.K, blockIdx.x * COLS, smem);
+  // row m of the result is finished by wavefront m
+  const unsigned col = blockIdx.x * COLS + lane;
   if (wave < (unsigned)MR && wave < M && lane < (unsigned)COLS && col < N) {
-    float v = 0.f;
-#pragma unroll
-    for (int w = 0; w < kWaves; ++w)
-#pragma unroll
-      for (int g = 0; g < SUBS; ++g) v += smem[w][wave][g * COLS + lane];
+    float v = summed<MR, COLS>(smem, wave, lane);
     if (biasPtr) v += biasPtr[col];
     if (p.residual) v += p.residual[(size_t)bi * p.strideR + (size_t)wave * N + col];
     if (p.act == 1) v = (float)(0.5 * (double)v * (double)(1.0f + erff(v / 1.4142135623730951f)));
-    Cbase[(size_t)wave * ldc + col] = v;
+    Cbase[(size_t)wave * p.ldc + col] = v;
+  }
+}
+
+// One LSTM time step in one launch: the product of the previous h with the state kernel, streamed as above, and
+// the cell (tfcc/mkl/kernel/tfcc_mklcellkernel.hpp:51-87, the expressions of lstm_cell_kernel in cell.hip) on the
+// finished sums.  The state kernel is given with its gates interleaved - column 4 u + g holds gate g (i, c, f, o)
+// of unit u - so that the 32 columns of a workgroup are the four gates of 8 units and still contiguous.
+struct LstmStepParams {
+  const float* hPrev;        // [batch, units]
+  const float* kernel;       // [units, units * 4], gates interleaved
+  const float* inputValue;   // [batch, 4 * units], gate-major as the reference lays it out
+  const float* bias;         // [4 * units], gate-major
+  const float* stateC;       // [batch, units]
+  float* h;                  // [batch, units]; not hPrev
+  float* cs;                 // [batch, units]; may be stateC
+  unsigned batch, units;
+  float forget;
+};
+
+__device__ __forceinline__ float sigmoid_value(float v) { return 1.f / (1.f + expf(0.f - v)); }
+
+template <int MR>
+__global__ __launch_bounds__(kWaves * 64) void lstm_step_kernel(LstmStepParams p) {
+  constexpr int COLS = 32, UNITS = COLS / 4;
+  __shared__ __attribute__((aligned(16))) float smem[kWaves][MR][64];
+  const unsigned units = p.units;
+  // Thread (row m, column c of the workgroup's 32 = unit j, gate g) finishes one gate: it fetches what that needs
+  // besides the sum now, not after the barrier.  The four gates of a (row, unit) pair sit in neighbouring lanes.
+  const unsigned tid = threadIdx.x, m = tid / COLS, c = tid % COLS, j = c / 4, g = c % 4, u = blockIdx.x * UNITS + j;
+  const bool finisher = m < (unsigned)MR;                  // whole wavefronts (or the lower half of one)
+  const bool valid = finisher && m < p.batch && u < units;
+  const size_t idx = (size_t)m * units + u;
+  float xin = 0.f, bv = 0.f, cPrev = 0.f;
+  if (valid) {
+    xin = p.inputValue[(size_t)m * 4 * units + (size_t)g * units + u];
+    bv = p.bias[(size_t)g * units + u];
+    if (g == 0) cPrev = p.stateC[idx];
+  }
+  stream_partial_sums<MR, COLS>(p.hPrev, units, p.batch, p.kernel, 4 * units, 4 * units, units, blockIdx.x * COLS, smem);
+  if (finisher) {
+    float pre = xin + summed<MR, COLS>(smem, m, c) + bv;
+    if (g == 2) pre += p.forget;
+    const float act = g == 1 ? tanhf(pre) : sigmoid_value(pre);
+    const int base = (int)(threadIdx.x & 63u) & ~3;
+    const float xi = __shfl(act, base, 64), xc = __shfl(act, base + 1, 64), xf = __shfl(act, base + 2, 64),
+                xo = __shfl(act, base + 3, 64);
+    if (valid && g == 0) {
+      const float cs = __fadd_rn(__fmul_rn(xc, xi), __fmul_rn(cPrev, xf));
+      p.h[idx] = tanhf(cs) * xo;
+      p.cs[idx] = cs;
+    }
   }
 }
 
@@ -140,3 +210,22 @@ int sgemv_launch(hipStream_t stream, const SgemmParams& p) {
 
 }  // namespace sgemm_detail
 }  // namespace tfcc_rocm
+
+using namespace tfcc_rocm;
+
+extern "C" int tfcc_rocm_lstm_step_f32(void* stream, unsigned batch, unsigned units, const float* h_prev,
+                                       const float* state_kernel_interleaved, const float* input_value,
+                                       const float* bias, float forget, const float* state_c, float* h, float* cs) {
+  TFCC_REQUIRE(h_prev && state_kernel_interleaved && input_value && bias && state_c && h && cs, "lstm_step: null argument");
+  TFCC_REQUIRE(batch >= 1 && batch <= 8, "lstm_step: 1 to 8 rows per step, got %u", batch);
+  TFCC_REQUIRE(units >= 1 && units < (1u << 28), "lstm_step: %u units", units);
+  TFCC_REQUIRE(h != h_prev, "lstm_step: h must not be the previous h (other workgroups still read it)");
+  LstmStepParams p{h_prev, state_kernel_interleaved, input_value, bias, state_c, h, cs, batch, units, forget};
+  const dim3 grid((units + 7) / 8), block(kWaves * 64);
+  hipStream_t s = as_stream(stream);
+  if (batch == 1) hipLaunchKernelGGL(lstm_step_kernel<1>, grid, block, 0, s, p);
+  else if (batch == 2) hipLaunchKernelGGL(lstm_step_kernel<2>, grid, block, 0, s, p);
+  else if (batch <= 4) hipLaunchKernelGGL(lstm_step_kernel<4>, grid, block, 0, s, p);
+  else hipLaunchKernelGGL(lstm_step_kernel<8>, grid, block, 0, s, p);
+  return check_launch("lstm_step");
+}

@@ -577,6 +577,32 @@ class ROCMCellInterface : public CellInterface<float> {
     check(tfcc_rocm_lstm_cell_f32(current_stream(), stateC.shape(0), stateC.shape(1), stateC.data(), inputValue.data(),
                                   stateHValue.data(), bias.data(), forget, h, cs));
   }
+  // [units, 4 units] -> gates interleaved, [units, units, 4]: column 4 u + g is gate g of unit u
+  Variable<float> prepareLSTMStateKernel(const Tensor<float>& stateKernel, unsigned batch) override {
+    if (batch < 1 || batch > 8) throw NotImplementedError("one-launch LSTM step: 1 to 8 rows");
+    if (stateKernel.shape().size() != 2 || stateKernel.shape(1) != stateKernel.shape(0) * 4 || stateKernel.size() == 0)
+      throw InvalidArgumentError("invalid state kernel");
+    const unsigned units = stateKernel.shape(0);
+    Variable<float> r({units, units * 4});
+    const unsigned shape[3] = {units, 4, units}, perm[3] = {0, 2, 1};
+    check(tfcc_rocm_transpose_f32(current_stream(), stateKernel.data(), shape, perm, 3, r.data()));
+    return r;
+  }
+  void processLSTMStepInto(const Tensor<float>& stateC, const Tensor<float>& inputValue, const Tensor<float>& h,
+                           const Tensor<float>& preparedStateKernel, const Tensor<float>& bias, float forget, float* hOut,
+                           float* csOut) override {
+    if (stateC.shape().size() != 2) throw InvalidArgumentError("invalid stateC");
+    const unsigned batch = stateC.shape(0), units = stateC.shape(1);
+    if (inputValue.shape().size() != 2 || inputValue.shape(0) != batch || inputValue.shape(1) != units * 4)
+      throw InvalidArgumentError("invalid inputValue");
+    if (h.shape() != stateC.shape()) throw InvalidArgumentError("invalid h");
+    if (preparedStateKernel.shape().size() != 2 || preparedStateKernel.shape(0) != units ||
+        preparedStateKernel.shape(1) != units * 4)
+      throw InvalidArgumentError("invalid state kernel");
+    if (bias.shape().size() != 1 || bias.shape(0) != units * 4) throw InvalidArgumentError("invalid bias");
+    check(tfcc_rocm_lstm_step_f32(current_stream(), batch, units, h.data(), preparedStateKernel.data(), inputValue.data(),
+                                  bias.data(), forget, stateC.data(), hOut, csOut));
+  }
   Variable<float> processGRUCellGates(const Tensor<float>& state, const Tensor<float>& inputs,
                                       const Tensor<float>& value, const Tensor<float>& bias) override {
     if (state.shape().size() != 2) throw InvalidArgumentError("invalid state");

@@ -137,6 +137,15 @@ class CellInterface {
   virtual void processLSTMCellInto(const Tensor<T>&, const Tensor<T>&, const Tensor<T>&, const Tensor<T>&, T, T*, T*) {
     throw NotImplementedError();
   }
+  // A whole time step in one launch, for devices that have one: the state kernel in the layout that launch wants
+  // (made once per sequence), then per step matmul(h, stateKernel) and the cell together.  NotImplementedError
+  // (the default, or for shapes the device does not take) sends the caller to the two calls above.
+  virtual Variable<T> prepareLSTMStateKernel(const Tensor<T>&, unsigned /*batch*/) { throw NotImplementedError(); }
+  virtual void processLSTMStepInto(const Tensor<T>& /*stateC*/, const Tensor<T>& /*inputValue*/, const Tensor<T>& /*h*/,
+                                   const Tensor<T>& /*preparedStateKernel*/, const Tensor<T>& /*bias*/, T /*forget*/,
+                                   T* /*hOut*/, T* /*csOut*/) {
+    throw NotImplementedError();
+  }
   virtual Variable<T> processGRUCellGates(const Tensor<T>&, const Tensor<T>&, const Tensor<T>&, const Tensor<T>&) {
     throw NotImplementedError();
   }
@@ -445,8 +454,8 @@ namespace detail {
 // tfcc::rnn::lstm_forward / lstm_backward (tfcc/core/operations/tfcc_rnn.cpp:29-81, 83-135): the same checks,
 // gate layout, forget bias 0 and output order (outputs in the order the steps are taken).  The products of the
 // inputs with inputKernel do not depend on the recurrence, so all steps share one matmul of [seq * batch, length];
-// each step then costs one matmul with stateKernel and one cell launch that writes h straight into its row block
-// of the result.
+// each step then costs one launch (the product with stateKernel and the cell together, where the device offers
+// that) or two (matmul, then a cell launch), and writes h straight into its row block of the result.
 template <class T>
 std::tuple<Variable<T>, Variable<T>, Variable<T>> lstm_sequence(bool backward, const Tensor<T>& a,
                                                                 const Tensor<T>& inputKernel,
@@ -471,12 +480,24 @@ std::tuple<Variable<T>, Variable<T>, Variable<T>> lstm_sequence(bool backward, c
   Variable<T> c = interface.getDataInterface().copy(ic);
   const size_t state = static_cast<size_t>(batch) * hidden;
   View<T> h(ih);
+  Variable<T> prepared;  // the state kernel as the one-launch step wants it, where the device has such a step
+  bool oneLaunch = false;
+  try {
+    prepared = interface.getCellInterface().prepareLSTMStateKernel(stateKernel, batch);
+    oneLaunch = true;
+  } catch (const NotImplementedError&) {
+  }
   for (unsigned step = 0; step < seq; ++step) {
     const unsigned t = backward ? seq - 1 - step : step;
     View<T> x(inputValues, inputValues.shape(), t * batch, (t + 1) * batch);
-    Variable<T> stateValues = interface.getBlasInterface().matmul(h, stateKernel);
-    interface.getCellInterface().processLSTMCellInto(c, x, stateValues, bias, static_cast<T>(0),
-                                                     result.data() + step * state, c.data());
+    if (oneLaunch) {
+      interface.getCellInterface().processLSTMStepInto(c, x, h, prepared, bias, static_cast<T>(0),
+                                                       result.data() + step * state, c.data());
+    } else {
+      Variable<T> stateValues = interface.getBlasInterface().matmul(h, stateKernel);
+      interface.getCellInterface().processLSTMCellInto(c, x, stateValues, bias, static_cast<T>(0),
+                                                       result.data() + step * state, c.data());
+    }
     h = View<T>(result, result.shape(), step, step + 1);
     h.reshape(Shape({batch, hidden}));
   }
