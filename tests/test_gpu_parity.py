@@ -207,12 +207,21 @@ def test_gemv_full_size_hash(pkg, T):
 
 # ---- sums, quantize, requantize, dequantize ----------------------------------------------------------
 
-@pytest.mark.parametrize("shape", [(1, 1), (17, 29), (3, 64, 256), (2, 100, 1000), (4096, 512), (5, 7, 16)])
+@pytest.mark.parametrize("shape", [
+    (1, 1), (17, 29), (3, 64, 256), (2, 100, 1000), (4096, 512), (5, 7, 16),
+    # 16-byte column groups: the wide column-sum kernel; row counts on both sides of its 16-row rounds and 64-row slabs,
+    # column counts that leave part of the last 1024-column block empty, extreme values (all -128 / 127 / 255)
+    (64, 16), (65, 1040), (2, 130, 2064), (4096, 4096), (1000, 11008), (3, 63, 32), (127, 48)])
 def test_reduce_sum(pkg, T, shape):
     rng = np.random.default_rng(sum(shape))
-    for x in (rng.integers(0, 256, shape, dtype=np.uint8), rng.integers(-128, 128, shape, dtype=np.int8)):
+    cases = [rng.integers(0, 256, shape, dtype=np.uint8), rng.integers(-128, 128, shape, dtype=np.int8)]
+    if shape[-2] >= 64 and shape[-2] * shape[-1] <= 1 << 21:
+        cases += [np.full(shape, 255, np.uint8), np.full(shape, -128, np.int8), np.full(shape, 127, np.int8)]
+    for x in cases:
         assert np.array_equal(T.n(pkg.reduce_sum(T.t(x), True)), O.reduce_sum(x, True))
-        assert np.array_equal(T.n(pkg.reduce_sum(T.t(x), False)), O.reduce_sum(x, False))
+        got = T.n(pkg.reduce_sum(T.t(x), False))
+        assert np.array_equal(got, O.reduce_sum(x, False))
+        assert np.array_equal(got, x.astype(np.int64).sum(axis=-2))  # the closed form, independent of the oracle
 
 
 def test_requantize_known_answer_and_fma_cases(pkg, T):

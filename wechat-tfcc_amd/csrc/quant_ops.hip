@@ -119,6 +119,87 @@ __global__ __launch_bounds__(256) void reduce_cols_vec_kernel(const T* a, unsign
   for (int e = 0; e < 4; ++e) atomicAdd(o + e, s[e]);
 }
 
+// 16-byte loads of data that is read once
+typedef int nt_v4i __attribute__((ext_vector_type(4)));
+typedef float nt_v4f __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ int4 load_streamed(const int4* p) {
+  const nt_v4i v = __builtin_nontemporal_load(reinterpret_cast<const nt_v4i*>(p));
+  return make_int4(v[0], v[1], v[2], v[3]);
+}
+__device__ __forceinline__ float4 load_streamed(const float4* p) {
+  const nt_v4f v = __builtin_nontemporal_load(reinterpret_cast<const nt_v4f*>(p));
+  return make_float4(v[0], v[1], v[2], v[3]);
+}
+
+// Column sums of a 1-byte type with col % 16 == 0 and 16-byte aligned rows.  A workgroup owns 1024 columns
+// (64 threads x 16 bytes: whole 1 KB row segments) and a slab of rows, dealt to four row lanes.  A thread takes its
+// rows four at a time, transposes each 4 x 4 byte block in registers so that a word holds one column's four rows,
+// and adds those with one dot-product instruction; the four row lanes meet in LDS and the slab's sums go to the
+// (zeroed) result with integer atomics, whose order does not matter.
+__device__ __forceinline__ void transpose_bytes_4x4(const unsigned r[4], unsigned c[4]) {
+  const unsigned t0 = __builtin_amdgcn_perm(r[1], r[0], 0x05010400u), t1 = __builtin_amdgcn_perm(r[1], r[0], 0x07030602u);
+  const unsigned t2 = __builtin_amdgcn_perm(r[3], r[2], 0x05010400u), t3 = __builtin_amdgcn_perm(r[3], r[2], 0x07030602u);
+  c[0] = __builtin_amdgcn_perm(t2, t0, 0x05040100u);
+  c[1] = __builtin_amdgcn_perm(t2, t0, 0x07060302u);
+  c[2] = __builtin_amdgcn_perm(t3, t1, 0x05040100u);
+  c[3] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
+}
+
+template <class T>
+__global__ __launch_bounds__(256) void reduce_cols_wide_kernel(const T* a, unsigned row, unsigned col,
+                                                               unsigned rowsPerSlab, int* out) {
+  constexpr bool kSigned = T(-1) < T(0);
+  __shared__ int part[4][64][17];
+  const unsigned b = blockIdx.z, cg = threadIdx.x & 63u, rl = threadIdx.x >> 6;
+  const unsigned c16 = blockIdx.x * 64 + cg;
+  const unsigned r0 = blockIdx.y * rowsPerSlab, r1 = min(r0 + rowsPerSlab, row);
+  int s[16];
+#pragma unroll
+  for (int e = 0; e < 16; ++e) s[e] = 0;
+  if (c16 * 16 < col) {
+    const size_t pitch = col / 16;
+    const int4* p = reinterpret_cast<const int4*>(a + (size_t)b * row * col) + c16;
+    unsigned r = r0 + rl;
+#pragma unroll 2
+    for (; r + 12 < r1; r += 16) {
+      const int4 v0 = load_streamed(p + (size_t)r * pitch), v1 = load_streamed(p + (size_t)(r + 4) * pitch),
+                 v2 = load_streamed(p + (size_t)(r + 8) * pitch), v3 = load_streamed(p + (size_t)(r + 12) * pitch);
+      const unsigned w[4][4] = {{(unsigned)v0.x, (unsigned)v1.x, (unsigned)v2.x, (unsigned)v3.x},
+                                {(unsigned)v0.y, (unsigned)v1.y, (unsigned)v2.y, (unsigned)v3.y},
+                                {(unsigned)v0.z, (unsigned)v1.z, (unsigned)v2.z, (unsigned)v3.z},
+                                {(unsigned)v0.w, (unsigned)v1.w, (unsigned)v2.w, (unsigned)v3.w}};
+#pragma unroll
+      for (int d = 0; d < 4; ++d) {
+        unsigned c[4];
+        transpose_bytes_4x4(w[d], c);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          s[4 * d + e] = kSigned ? __builtin_amdgcn_sdot4((int)c[e], 0x01010101, s[4 * d + e], false)
+                                 : (int)__builtin_amdgcn_udot4(c[e], 0x01010101u, (unsigned)s[4 * d + e], false);
+      }
+    }
+    for (; r < r1; r += 4) {
+      const int4 v = load_streamed(p + (size_t)r * pitch);
+      const unsigned w[4] = {(unsigned)v.x, (unsigned)v.y, (unsigned)v.z, (unsigned)v.w};
+#pragma unroll
+      for (int d = 0; d < 4; ++d)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) s[4 * d + e] += (int)(T)(w[d] >> (8 * e));
+    }
+  }
+#pragma unroll
+  for (int e = 0; e < 16; ++e) part[rl][cg][e] = s[e];
+  __syncthreads();
+  // 1024 sums per workgroup, four per thread
+  unsigned* o = reinterpret_cast<unsigned*>(out) + (size_t)b * col;
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const unsigned idx = threadIdx.x + 256u * q, g = idx >> 4, e = idx & 15u;
+    const unsigned column = (blockIdx.x * 64 + g) * 16 + e;
+    if (column < col) atomicAdd(o + column, (unsigned)(part[0][g][e] + part[1][g][e] + part[2][g][e] + part[3][g][e]));
+  }
+}
+
 __global__ void zero_kernel(int* p, size_t n) {
   size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = 0;
@@ -141,17 +222,6 @@ __global__ __launch_bounds__(256) void requantize_kernel(const void* in, int inT
   }
 }
 
-// 16-byte loads of data that is read once
-typedef int nt_v4i __attribute__((ext_vector_type(4)));
-typedef float nt_v4f __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ int4 load_streamed(const int4* p) {
-  const nt_v4i v = __builtin_nontemporal_load(reinterpret_cast<const nt_v4i*>(p));
-  return make_int4(v[0], v[1], v[2], v[3]);
-}
-__device__ __forceinline__ float4 load_streamed(const float4* p) {
-  const nt_v4f v = __builtin_nontemporal_load(reinterpret_cast<const nt_v4f*>(p));
-  return make_float4(v[0], v[1], v[2], v[3]);
-}
 
 // int32 -> uint8, the matmul epilogue's type pair.  Four elements per 16-byte load, four loads in flight per
 // thread, few enough threads that the scalar set-up (a few hundred double operations) is not what the launch
@@ -458,6 +528,24 @@ int reduce_cols(hipStream_t s, const void* a, unsigned batch, unsigned row, unsi
   size_t n = (size_t)batch * col;
   hipLaunchKernelGGL(zero_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, out, n);
   if (int e = check_launch("reduce_sum cols (zero)")) return e;
+  if (batch > 65535) return set_error(TFCC_ROCM_INVALID_ARGUMENT, "reduce_sum: batch too large");
+  if constexpr (sizeof(T) == 1) {
+    if (col % 16 == 0 && (uintptr_t)a % 16 == 0 && row >= 64) {
+      // slabs of at least 64 rows (sixteen 16-byte loads per thread), about a thousand workgroups where the
+      // matrix is large enough
+      const unsigned wideBlocks = (col / 16 + 63) / 64;
+      unsigned wideSlabs = (1024 + wideBlocks * batch - 1) / (wideBlocks * batch);
+      if (wideSlabs > row / 64) wideSlabs = row / 64;
+      if (wideSlabs < 1) wideSlabs = 1;
+      if (wideSlabs > 65535) wideSlabs = 65535;
+      unsigned perSlab = (row + wideSlabs - 1) / wideSlabs;
+      perSlab = (perSlab + 15) / 16 * 16;  // whole rounds of the four row lanes' four rows
+      wideSlabs = (row + perSlab - 1) / perSlab;
+      hipLaunchKernelGGL(reduce_cols_wide_kernel<T>, dim3(wideBlocks, wideSlabs, batch), dim3(256), 0, s,
+                         static_cast<const T*>(a), row, col, perSlab, out);
+      return check_launch("reduce_sum cols");
+    }
+  }
   const bool vec = sizeof(T) == 1 && col % 4 == 0 && (uintptr_t)a % 4 == 0;
   const unsigned colBlocks = vec ? (col / 4 + 255) / 256 : (col + 255) / 256;
   // enough row slabs for ~2048 workgroups
@@ -465,7 +553,6 @@ int reduce_cols(hipStream_t s, const void* a, unsigned batch, unsigned row, unsi
   if (slabs > (row + 31) / 32) slabs = (row + 31) / 32;
   if (slabs < 1) slabs = 1;
   if (slabs > 65535) slabs = 65535;
-  if (batch > 65535) return set_error(TFCC_ROCM_INVALID_ARGUMENT, "reduce_sum: batch too large");
   const unsigned rowsPerSlab = (row + slabs - 1) / slabs;
   slabs = (row + rowsPerSlab - 1) / rowsPerSlab;
   if (vec)
