@@ -321,6 +321,21 @@ def bench_other(torch, pkg, dev, steps, warmup, c3):
     out["c3_int8_4096_requant_colsum_declared_exact"] = {"ms": round(ms, 5), "tops": round(tops, 2),
                                                         "frac_int8_mfma": round(tops / PEAK_INT8_TOPS, 4)}
 
+    # C3 the way the reference's callers run it (tfcc/test/quantization.cpp:112-118): row sums of A and column
+    # sums of B are recomputed for every product, then the product itself (here with the fused requantize)
+    gemm_step = make_c3_step(torch, pkg, ta, tb, rs, cs, ranges, out_range, want_acc=False)
+
+    def call_sequence():
+        for st in (lib.tfcc_rocm_reduce_sum_rows(stream, ta.data_ptr(), pkg.U8, 1, 4096, 4096, rs.data_ptr()),
+                   lib.tfcc_rocm_reduce_sum_cols(stream, tb.data_ptr(), pkg.S8, 1, 4096, 4096, cs.data_ptr())):
+            if st != 0:
+                pkg.check(st)
+        gemm_step()
+    ms = time_launches(torch, call_sequence, steps, warmup)
+    tops = 2.0 * 4096 ** 3 / ms / 1e9
+    out["c3_int8_4096_with_row_and_column_sums_per_call"] = {"ms": round(ms, 5), "tops": round(tops, 2),
+                                                            "frac_int8_mfma": round(tops / PEAK_INT8_TOPS, 4)}
+
     # C5: skinny decode shapes, B streamed once; rotate B buffers larger than the last-level cache
     n, k = 11008, 4096
     sets = 8
