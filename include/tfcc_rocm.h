@@ -38,6 +38,11 @@ enum {
   TFCC_ROCM_U16 = 3,
   TFCC_ROCM_S32 = 4,
   TFCC_ROCM_U32 = 5,
+  /* index types of gather and the remaining types of cast */
+  TFCC_ROCM_S64 = 6,
+  TFCC_ROCM_U64 = 7,
+  TFCC_ROCM_F32 = 8,
+  TFCC_ROCM_F64 = 9,
 };
 
 const char* tfcc_rocm_last_error_string(void);
@@ -373,6 +378,20 @@ int tfcc_rocm_gru_cell_candidate_f32(void* stream, unsigned batch, unsigned unit
 int tfcc_rocm_pytorch_gru_cell_f32(void* stream, unsigned batch, unsigned units, const float* state,
                                    const float* input_value, const float* state_value, const float* gate_bias,
                                    const float* candidate_i_bias, const float* candidate_h_bias, float* result);
+
+/* ---- data movement between the products: one pass each ------------------------------------------------------------
+ * rows x width bytes from src (rows src_pitch bytes apart) to dst (rows dst_pitch bytes apart).  BasicInterface::slice
+ * (tfcc/mkl/interfaces/tfcc_mklbasicinterface.cpp:488-515: a [s1, s2, s3] tensor, rows = s1, src = a + start * s3,
+ * width = length * s3) and concat (tfcc/core/operations/tfcc_base.cpp:86-106: one copy per value into its column
+ * range of the result) are one call each per operand. */
+int tfcc_rocm_copy2d(void* stream, const void* src, uint64_t src_pitch, void* dst, uint64_t dst_pitch, uint64_t rows,
+                     uint64_t width);
+/* GatherInterface::gather (tfcc/mkl/interfaces/tfcc_mklgatherinterface.cpp:28-66): out row i = params row indices[i]
+ * (chunk_bytes each), a row of zeros where the index is outside [0, batch).  index_type: TFCC_ROCM_S32 / U32 / S64 / U64. */
+int tfcc_rocm_gather_rows(void* stream, const void* params, unsigned batch, uint64_t chunk_bytes, const void* indices,
+                          int index_type, uint64_t length, void* out);
+/* tfcc::data::cast: out[i] = static_cast<out type>(in[i]) for any pair of the ten element types above. */
+int tfcc_rocm_cast(void* stream, const void* in, int in_type, void* out, int out_type, uint64_t total);
 
 #ifdef __cplusplus
 }

@@ -550,6 +550,41 @@ def test_lstm_cell_in_place_state_and_sequence(pkg, T):
         assert np.linalg.norm(got - want) <= 1e-5 * np.linalg.norm(want)
 
 
+def test_gather_slice_concat_cast_equal_numpy(pkg, T):
+    """Row gather (out-of-range indices give zeros, tfcc/mkl/interfaces/tfcc_mklgatherinterface.cpp:35-39), slice and
+    concat along every axis (byte, 4-byte and 16-byte copy paths), casts between element types: numpy bit for bit."""
+    import torch
+    rng = np.random.default_rng(13)
+    table = rng.normal(size=(50, 768)).astype(np.float32)
+    for idx_type in (np.int32, np.int64):
+        idx = rng.integers(-3, 55, (4, 9)).astype(idx_type)
+        want = np.where(((idx >= 0) & (idx < 50))[..., None], table[np.clip(idx, 0, 49)], 0).astype(np.float32)
+        assert np.array_equal(T.n(pkg.gather(T.t(table), T.t(idx))), want)
+    small = rng.integers(-100, 100, (7, 3), dtype=np.int8)          # 3-byte rows: the byte path
+    assert np.array_equal(T.n(pkg.gather(T.t(small), T.t(np.array([6, 0, 7, 2], np.int32)))),
+                          np.concatenate([small[[6, 0]], np.zeros((1, 3), np.int8), small[[2]]]))
+    odd = rng.normal(size=(5, 3, 6)).astype(np.float32)             # 72-byte rows: the 4-byte path
+    assert np.array_equal(T.n(pkg.gather(T.t(odd), T.t(np.array([[4], [1]], np.int64)))), odd[[[4], [1]]])
+    x = rng.normal(size=(3, 10, 8, 4)).astype(np.float32)
+    for axis, start, end in ((0, 1, 3), (1, 0, 10), (1, 3, 4), (2, 5, 99), (3, 1, 3)):
+        assert np.array_equal(T.n(pkg.slice_axis(T.t(x), axis, start, end)), np.take(x, range(start, min(end, x.shape[axis])), axis))
+    for bad, text in (((4, 0, 1), "invalid axis"), ((1, 3, 3), "start large than end"), ((1, 10, 12), "invalid start")):
+        with pytest.raises(pkg.InvalidArgumentError, match=text):
+            pkg.slice_axis(T.t(x), *bad)
+    for axis in range(4):
+        parts = [rng.normal(size=[d if i != axis else n for i, d in enumerate(x.shape)]).astype(np.float32) for n in (1, 5, 2)]
+        assert np.array_equal(T.n(pkg.concat([T.t(p) for p in parts], axis)), np.concatenate(parts, axis))
+    bytes_ = [rng.integers(0, 255, (3, n), dtype=np.uint8) for n in (5, 2, 9)]
+    assert np.array_equal(T.n(pkg.concat([T.t(b) for b in bytes_], 1)), np.concatenate(bytes_, 1))
+    with pytest.raises(pkg.InvalidArgumentError, match="invalid shape"):
+        pkg.concat([T.t(x), T.t(x[:, :, :7])], 1)
+    ints = rng.integers(-1000, 1000, (33, 7)).astype(np.int32)
+    floats = (rng.normal(size=(33, 7)) * 50).astype(np.float32)
+    for src, dtype, np_dtype in ((ints, torch.float32, np.float32), (floats, torch.int32, np.int32), (ints, torch.int64, np.int64),
+                                 (floats, torch.float64, np.float64), (ints, torch.int8, np.int8), (floats, torch.int64, np.int64)):
+        assert np.array_equal(T.n(pkg.cast(T.t(src), dtype)), src.astype(np_dtype))
+
+
 BROADCAST_PAIRS = [
     ((2, 4, 8, 8), (2, 1, 1, 8)),        # attention scores + mask
     ((3, 1, 5), (1, 4, 1)),              # both sides broadcast

@@ -67,6 +67,73 @@ def test_reshape_identity_on_host(mf, rt):
                                     mf.f_bytes(4, b"\0" * 8)))
 
 
+def test_shape_nodes_on_host(mf, rt):
+    """base.Squeeze / Unsqueeze / Flatten give Views of the input under the shapes of
+    tfcc_runtime/operations/base/squeeze.cpp:27-52, unsqueeze.cpp:27-52, flatten.cpp:27-50; base.GetDimension a value
+    of whatever type the graph asks for, base.GetShape a uint32 vector (consumed here by a Reshape)."""
+    rng = np.random.default_rng(4)
+    a = rng.normal(size=(2, 1, 3, 1)).astype(np.float32)
+
+    def run(build):
+        g = mf.GraphBuilder("g")
+        x = g.input("x", mf.FLOAT, [2, 1, 3, 1])
+        outs = build(g, x)
+        for o in outs:
+            g.output(o)
+        m = rt.Model(mf.write_model([g], "g"), host=True)
+        res = m.run({"x": a})
+        m.close()
+        return [res[o] for o in outs]
+
+    def shaped(op, payload):
+        def build(g, x):
+            v = g.view("v")
+            g.node(op, [x], [v], payload)
+            y = g.variable("y")
+            g.node("base.Identity", [v], [y])
+            return [y]
+        return build
+    for op, payload, want in (("base.Squeeze", mf.f_packed(1, [1, 3]), (2, 3)), ("base.Squeeze", mf.f_packed(1, [3]), (2, 1, 3)),
+                              ("base.Squeeze", b"", (2, 1, 3, 1)), ("base.Unsqueeze", mf.f_packed(1, [0, 3]), (1, 2, 1, 1, 3, 1)),
+                              ("base.Unsqueeze", mf.f_packed(1, [5, 4]), (2, 1, 3, 1, 1, 1)),
+                              ("base.Flatten", mf.f_varint(1, 2), (2, 3)), ("base.Flatten", b"", (1, 6)),
+                              ("base.Flatten", mf.f_varint(1, 3), (6, 1))):
+        out, = run(shaped(op, payload))
+        assert out.shape == want and np.array_equal(out.ravel(), a.ravel()), (op, want)
+    for op, payload, text in (("base.Squeeze", mf.f_packed(1, [0]), "Squeeze: invalid axes"),
+                              ("base.Squeeze", mf.f_packed(1, [1, 7]), "Squeeze: invalid axes"),
+                              ("base.Unsqueeze", mf.f_packed(1, [9]), "Unsqueeze: invalid axes"),
+                              ("base.Flatten", mf.f_varint(1, 4), "Flatten: axis error")):
+        with pytest.raises(rt.RuntimeError_, match=text):
+            run(shaped(op, payload))
+
+    def dimensions(g, x):
+        outs = []
+        for dtype, axis in ((mf.INT64, 0), (mf.UINT32, 2), (mf.FLOAT, 2), (mf.INT32, 3)):
+            v = g._symbol("d_%d_%d" % (dtype, axis), dtype, mf.VALUE)
+            g.node("base.GetDimension", [x], [v], mf.f_varint(1, axis))
+            outs.append(v)
+        return outs
+    got = run(dimensions)
+    assert [float(v[0]) for v in got] == [2.0, 3.0, 3.0, 1.0]
+    assert [v.dtype for v in got] == [np.int64, np.uint32, np.float32, np.int32]
+    with pytest.raises(rt.RuntimeError_, match="GetDimension: axis error"):
+        run(lambda g, x: [g.node("base.GetDimension", [x], [g._symbol("bad", mf.INT64, mf.VALUE)], mf.f_varint(1, 4)) or "bad"])
+
+    def shape_round_trip(g, x):
+        flat = g.view("flat")
+        g.node("base.Flatten", [x], [flat], mf.f_varint(1, 1))
+        shape = g.vector("shape", mf.UINT32)
+        g.node("base.GetShape", [x], [shape])
+        back = g.view("back")
+        g.node("base.Reshape", [flat, shape], [back])
+        y = g.variable("y")
+        g.node("base.Identity", [back], [y])
+        return [y]
+    out, = run(shape_round_trip)
+    assert out.shape == (2, 1, 3, 1) and np.array_equal(out, a)
+
+
 @pytest.mark.parametrize("compress", [False, True])
 def test_constants_from_npz(mf, rt, compress):
     """element conversion, Fortran order, 0-d arrays, stored and deflated members"""

@@ -16,7 +16,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libtfcc_rocm.so")
 CSRC_DIR = os.path.join(_HERE, "csrc")
 
-S8, U8, S16, U16, S32, U32 = range(6)
+S8, U8, S16, U16, S32, U32, S64, U64, F32, F64 = range(10)
 
 
 class TfccRocmError(RuntimeError):
@@ -130,6 +130,9 @@ SYMBOLS = {
     "tfcc_rocm_binary_broadcast_f32": (_I, [_VP, _I, _VP, _VP, _I, C.POINTER(C.c_uint), C.POINTER(_U64),
                                            C.POINTER(_U64), _VP]),
     "tfcc_rocm_lstm_cell_f32": (_I, [_VP, _U, _U, _VP, _VP, _VP, _VP, _F, _VP, _VP]),
+    "tfcc_rocm_copy2d": (_I, [_VP, _VP, _U64, _VP, _U64, _U64, _U64]),
+    "tfcc_rocm_gather_rows": (_I, [_VP, _VP, _U, _U64, _VP, _I, _U64, _VP]),
+    "tfcc_rocm_cast": (_I, [_VP, _VP, _I, _VP, _I, _U64]),
     "tfcc_rocm_lstm_step_f32": (_I, [_VP, _U, _U, _VP, _VP, _VP, _VP, _F, _VP, _VP, _VP]),
     "tfcc_rocm_gru_cell_gates_f32": (_I, [_VP, _U, _U, _U, _VP, _VP, _VP, _VP, _VP]),
     "tfcc_rocm_gru_cell_candidate_f32": (_I, [_VP, _U, _U, _VP, _VP, _VP, _VP, _VP, _VP]),
@@ -174,7 +177,8 @@ def _ptr(t):
 
 def _type_code(dtype):
     import torch
-    return {torch.int8: S8, torch.uint8: U8, torch.int16: S16, torch.int32: S32}[dtype]
+    return {torch.int8: S8, torch.uint8: U8, torch.int16: S16, torch.int32: S32, torch.int64: S64, torch.float32: F32,
+            torch.float64: F64}[dtype]
 
 
 def matmul_plan(shape_a, shape_b, shape_bias=None):
@@ -655,6 +659,90 @@ def binary(op, a, b):
     a, b = a.contiguous(), b.contiguous()
     out = torch.empty_like(a)
     check(lib().tfcc_rocm_binary_f32(_stream(), BINARY_OPS[op], _ptr(a), _ptr(b), a.numel(), b.numel(), _ptr(out)))
+    return out
+
+
+def gather(params, indices):
+    """tfcc::nn::gather (tfcc/core/operations/tfcc_nn.cpp:345-385): rows of params by index, zeros for an index
+    outside [0, rows)."""
+    import torch
+    if params.numel() == 0:
+        raise InvalidArgumentError("invalid tensor")
+    params, indices = params.contiguous(), indices.contiguous()
+    out = torch.empty(tuple(indices.shape) + tuple(params.shape[1:]), dtype=params.dtype, device=params.device)
+    if indices.numel() == 0:
+        return out
+    chunk = params.numel() // params.shape[0] * params.element_size()
+    check(lib().tfcc_rocm_gather_rows(_stream(), _ptr(params), params.shape[0], chunk, _ptr(indices),
+                                      _type_code(indices.dtype), indices.numel(), _ptr(out)))
+    return out
+
+
+def cast(a, dtype):
+    """tfcc::data::cast: element-wise static_cast."""
+    import torch
+    a = a.contiguous()
+    out = torch.empty(a.shape, dtype=dtype, device=a.device)
+    if a.numel():
+        check(lib().tfcc_rocm_cast(_stream(), _ptr(a), _type_code(a.dtype), _ptr(out), _type_code(dtype), a.numel()))
+    return out
+
+
+def _split_at(shape, axis):
+    s1 = 1
+    for d in shape[:axis]:
+        s1 *= d
+    s3 = 1
+    for d in shape[axis + 1:]:
+        s3 *= d
+    return s1, shape[axis], s3
+
+
+def slice_axis(a, axis, start, end):
+    """tfcc::base::slice (tfcc/core/operations/tfcc_base.cpp:28-41; end is clipped to the dimension as
+    tfcc/mkl/interfaces/tfcc_mklbasicinterface.cpp:490 clips it)."""
+    import torch
+    if axis >= a.dim():
+        raise InvalidArgumentError("invalid axis")
+    if start >= end:
+        raise InvalidArgumentError("start large than end")
+    if start >= a.shape[axis]:
+        raise InvalidArgumentError("invalid start")
+    a = a.contiguous()
+    end = min(end, a.shape[axis])
+    s1, s2, s3 = _split_at(tuple(a.shape), axis)
+    shape = list(a.shape)
+    shape[axis] = end - start
+    out = torch.empty(shape, dtype=a.dtype, device=a.device)
+    e = a.element_size()
+    if out.numel():
+        check(lib().tfcc_rocm_copy2d(_stream(), a.data_ptr() + start * s3 * e, s2 * s3 * e, _ptr(out),
+                                     (end - start) * s3 * e, s1, (end - start) * s3 * e))
+    return out
+
+
+def concat(values, axis):
+    """tfcc::base::concat (tfcc/core/operations/tfcc_base.cpp:86-106)."""
+    import torch
+    if len(values) == 0:
+        raise InvalidArgumentError("values.size could not be zero")
+    for v in values:
+        if axis >= v.dim():
+            raise InvalidArgumentError("invalid axis")
+        if v.dim() != values[0].dim() or any(i != axis and v.shape[i] != values[0].shape[i] for i in range(v.dim())):
+            raise InvalidArgumentError("invalid shape")
+    values = [v.contiguous() for v in values]
+    shape = list(values[0].shape)
+    shape[axis] = sum(v.shape[axis] for v in values)
+    out = torch.empty(shape, dtype=values[0].dtype, device=values[0].device)
+    s1, total, s3 = _split_at(tuple(shape), axis)
+    e = out.element_size()
+    offset = 0
+    for v in values:
+        width = v.shape[axis] * s3 * e
+        if width and s1:
+            check(lib().tfcc_rocm_copy2d(_stream(), _ptr(v), width, out.data_ptr() + offset, total * s3 * e, s1, width))
+        offset += width
     return out
 
 

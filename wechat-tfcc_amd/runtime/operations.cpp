@@ -10,9 +10,12 @@
 //                                       operations/math/<name>.cpp
 //   nn.LayerNormalization               operations/nn/layernormalization.cpp:52-88
 //   rnn.BidirectionalLSTM               operations/rnn/bidirectionallstm.cpp:27-128
+//   base.Squeeze / Unsqueeze / Flatten  operations/base/squeeze.cpp, unsqueeze.cpp, flatten.cpp (Views of the input)
+//   base.GetShape, base.GetDimension    operations/base/getshape.cpp, getdimension.cpp
 //   base.Transpose, base.Reshape, base.Identity, base.CreateVector
 //                                       operations/base/transpose.cpp, reshape.cpp:27-59,74-104,
 //                                       identity.cpp, createvector.cpp:63-121
+#include <algorithm>
 #include <array>
 #include <cmath>
 #include <map>
@@ -321,6 +324,119 @@ class Reshape : public TypedOperation<T> {
   }
 };
 
+// ---- base.Squeeze / base.Unsqueeze / base.Flatten: the output is a View of the input under another shape ---------
+// tfcc_runtime/operations/base/squeeze.cpp:27-52,78-113, unsqueeze.cpp:27-52,78-113, flatten.cpp:27-90
+enum class Reshaping { SQUEEZE, UNSQUEEZE, FLATTEN };
+
+template <Reshaping KIND, class T>
+class ShapeView : public TypedOperation<T> {
+  static const char* message() {
+    return KIND == Reshaping::SQUEEZE ? "base.Squeeze" : KIND == Reshaping::UNSQUEEZE ? "base.Unsqueeze" : "base.Flatten";
+  }
+
+ public:
+  ShapeView() : TypedOperation<T>(message()) {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 1 || node.outputs.size() != 1) return false;
+    if (!same_dtype(graph, node.outputs, this->DTYPE) || !same_dtype(graph, node.inputs, this->DTYPE)) return false;
+    std::vector<size_t> axes;  // Flatten: its one axis
+    wire::Reader r(node.operation);
+    uint32_t f, t;
+    while (r.next(f, t)) {
+      if (f == 1 && KIND == Reshaping::FLATTEN && t == 0) axes.assign(1, static_cast<size_t>(r.varint()));
+      else if (f == 1 && KIND != Reshaping::FLATTEN) r.repeatedVarint(t, axes);
+      else r.skip(t);
+    }
+    if (KIND == Reshaping::FLATTEN && axes.empty()) axes.assign(1, 0);  // proto3: a zero field is not written
+    std::sort(axes.begin(), axes.end());
+    auto& sm = graph.getSymbolManager();
+    const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+    View<T>* out = sm.getView(node.outputs[0], T());
+    graph.addStep([a, out, axes] {
+      std::vector<unsigned> shape;
+      const size_t rank = a->shape().size();
+      if (KIND == Reshaping::FLATTEN) {
+        if (axes[0] >= rank) throw RuntimeError("Flatten: axis error");
+        unsigned s1 = 1, s2 = 1;
+        for (size_t i = 0; i < rank; ++i) (i < axes[0] ? s1 : s2) *= a->shape(i);
+        shape = {s1, s2};
+      } else if (axes.empty()) {
+        shape = a->shape().toVector();
+      } else if (KIND == Reshaping::SQUEEZE) {
+        size_t pos = 0;
+        for (size_t i = 0; i < rank; ++i) {
+          if (pos < axes.size() && i == axes[pos]) {
+            if (a->shape(i) != 1) throw RuntimeError("Squeeze: invalid axes");
+            ++pos;
+          } else {
+            shape.push_back(a->shape(i));
+          }
+        }
+        if (pos != axes.size()) throw RuntimeError("Squeeze: invalid axes");
+      } else {
+        shape.resize(rank + axes.size());
+        size_t pos0 = 0, pos1 = 0;
+        for (size_t i = 0; i < shape.size(); ++i) {
+          if (pos1 < axes.size() && i == axes[pos1]) {
+            shape[i] = 1;
+            ++pos1;
+          } else {
+            if (pos0 >= rank) throw RuntimeError("Unsqueeze: invalid axes");
+            shape[i] = a->shape(pos0++);
+          }
+        }
+      }
+      *out = View<T>(*a, Shape(std::move(shape)));
+    });
+    return true;
+  }
+};
+
+// ---- base.GetShape (a uint32 vector) / base.GetDimension (a value of any type) -----------------------------------
+// tfcc_runtime/operations/base/getshape.cpp:27-78, getdimension.cpp:27-76
+template <class T>
+class GetShape : public TypedOperation<T> {
+ public:
+  GetShape() : TypedOperation<T>("base.GetShape") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 1 || node.outputs.size() != 1) return false;
+    auto& sm = graph.getSymbolManager();
+    if (sm.getSymbolInfo(node.outputs[0]).dtype != DataTypeOf<uint32_t>::value ||
+        sm.getSymbolInfo(node.inputs[0]).dtype != this->DTYPE)
+      return false;
+    const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+    std::vector<uint32_t>* out = sm.getVector(node.outputs[0], uint32_t());
+    graph.addStep([a, out] { *out = a->shape().toVector(); });
+    return true;
+  }
+};
+
+template <class SRC, class DST>
+class GetDimension : public TypedOperation<SRC> {
+ public:
+  GetDimension() : TypedOperation<SRC>("base.GetDimension") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 1 || node.outputs.size() != 1) return false;
+    auto& sm = graph.getSymbolManager();
+    if (sm.getSymbolInfo(node.outputs[0]).dtype != DataTypeOf<DST>::value || sm.getSymbolInfo(node.inputs[0]).dtype != this->DTYPE)
+      return false;
+    size_t axis = 0;
+    wire::Reader r(node.operation);
+    uint32_t f, t;
+    while (r.next(f, t)) {
+      if (f == 1 && t == 0) axis = static_cast<size_t>(r.varint());
+      else r.skip(t);
+    }
+    const Tensor<SRC>* a = sm.getTensor(node.inputs[0], SRC());
+    DST* out = sm.getValue(node.outputs[0], DST());
+    graph.addStep([a, out, axis] {
+      if (axis >= a->shape().size()) throw RuntimeError("GetDimension: axis error");
+      *out = static_cast<DST>(a->shape(axis));
+    });
+    return true;
+  }
+};
+
 // ---- base.Identity -----------------------------------------------------------------------------------------------
 template <class T>
 class Identity : public TypedOperation<T> {
@@ -511,10 +627,19 @@ class Collector {
     add(new LayerNormalization<T>());
     add(new Transpose<T>());
     add(new Reshape<T, int32_t>());
+    add(new Reshape<T, uint32_t>());
     add(new Reshape<T, int64_t>());
+    add(new Reshape<T, uint64_t>());
     add(new Identity<T>());
     add(new CreateVector<T>());
     add(new BidirectionalLSTM<T>());
+    add(new ShapeView<Reshaping::SQUEEZE, T>());
+    add(new ShapeView<Reshaping::UNSQUEEZE, T>());
+    add(new ShapeView<Reshaping::FLATTEN, T>());
+    add(new GetShape<T>());
+#define TFCC_RUNTIME_ADD_DIMENSION(DST, E) add(new GetDimension<T, DST>());
+    TFCC_RUNTIME_FOR_ALL_TYPES(TFCC_RUNTIME_ADD_DIMENSION)
+#undef TFCC_RUNTIME_ADD_DIMENSION
   }
 
  public:
