@@ -525,6 +525,95 @@ def test_arithmetic_nodes_broadcast_like_numpy(mf, rt, dev):
     assert np.array_equal(res[outs["mul"]], cv * rv) and np.array_equal(res[outs["div"]], rv / cv)
 
 
+@pytest.mark.gpu
+def test_embeddings_mask_and_answer_head_around_a_product(mf, rt, dev):
+    """The nodes a converted BERT puts around its encoder layers: nn.Gather for the embeddings (an index outside the
+    table gives a row of zeros), base.Unsqueeze / base.Cast and value arithmetic for the attention mask, a product
+    with the answer weights, base.SliceV1 + base.Squeeze for the two logits, base.Concat to join them again."""
+    rng = np.random.default_rng(23)
+    batch, seq, hidden, vocab = 3, 12, 32, 50
+    table = rng.normal(size=(vocab, hidden)).astype(np.float32)
+    positions = rng.normal(size=(seq, hidden)).astype(np.float32)
+    w_out = rng.normal(size=(hidden, 2)).astype(np.float32)
+    g = mf.GraphBuilder("g")
+    ids = g.input("ids", mf.INT64, [batch, seq])
+    keep = g.input("keep", mf.INT32, [batch, seq])
+    emb = g.variable("emb")
+    g.node("nn.Gather", [g.constant("table", table), ids], [emb])
+    x = g.binary("Add", emb, g.constant("positions", positions))                 # [B, S, H] + [S, H]
+    k4 = g.view("k4", mf.INT32)
+    g.node("base.Unsqueeze", [keep], [k4], mf.f_packed(1, [1, 2]))                # [B, 1, 1, S]
+    kf = g.variable("kf")
+    g.node("base.Cast", [k4], [kf], mf.f_varint(1, mf.FLOAT))
+    one = g.constant("one", np.array(1.0, np.float32), mf.CONSTANT_VALUE)
+    big = g.constant("big", np.array(-10000.0, np.float32), mf.CONSTANT_VALUE)
+    mask = g.binary("Mul", g.binary("Sub", one, kf), big)                          # (1 - keep) * -10000
+    logits = g.matmul(x, g.constant("w_out", w_out))                              # [B, S, 2]
+    parts = []
+    for pos in (0, 1):
+        start = g.constant("pos%d" % pos, np.array(pos, np.int64), mf.CONSTANT_VALUE)
+        piece = g.variable("piece")
+        g.node("base.SliceV1", [logits, start], [piece], mf.f_varint(1, 2) + mf.f_varint(2, 1))
+        sq = g.view("sq")
+        g.node("base.Squeeze", [piece], [sq], mf.f_packed(1, [2]))
+        flat = g.variable("logit%d" % pos)
+        g.node("base.Identity", [sq], [flat])
+        parts.append(flat)
+    joined = g.variable("joined")
+    g.node("base.Concat", parts, [joined], mf.f_varint(1, 1))
+    count = g._symbol("count", mf.INT64, mf.VALUE)
+    g.node("base.GetDimension", [joined], [count], mf.f_varint(1, 1))
+    as_float = g._symbol("count_f", mf.FLOAT, mf.VALUE)
+    g.node("base.Cast", [count], [as_float], mf.f_varint(1, mf.FLOAT))
+    for o in (x, mask, parts[0], parts[1], joined, count, as_float):
+        g.output(o)
+    idv = rng.integers(0, vocab, (batch, seq)).astype(np.int64)
+    idv[0, 0], idv[1, 3] = vocab, -1                                              # outside the table
+    keepv = (rng.random((batch, seq)) < 0.7).astype(np.int32)
+    res = rt.Model(mf.write_model([g], "g")).run({"ids": idv, "keep": keepv})
+    want_emb = np.where(((idv >= 0) & (idv < vocab))[..., None], table[np.clip(idv, 0, vocab - 1)], 0).astype(np.float32)
+    want_x = want_emb + positions
+    assert np.array_equal(res[x], want_x)
+    assert np.array_equal(res[mask], ((1 - keepv.astype(np.float32)) * np.float32(-10000.0)).reshape(batch, 1, 1, seq))
+    want_logits = want_x.astype(np.float64) @ w_out.astype(np.float64)
+    for pos in (0, 1):
+        assert res[parts[pos]].shape == (batch, seq) and rel_frobenius(res[parts[pos]], want_logits[..., pos]) <= 1e-5
+    assert res[joined].shape == (batch, 2 * seq)
+    assert np.array_equal(res[joined], np.concatenate([res[parts[0]], res[parts[1]]], axis=1))
+    assert int(res[count][0]) == 2 * seq and float(res[as_float][0]) == 2.0 * seq
+
+
+def test_data_movement_nodes_accept_rules(mf, rt):
+    """nn.Gather wants 32- or 64-bit integer indices, base.Cast a result symbol of the type its message names,
+    base.SliceV1 an integer position value: anything else is a node nobody takes
+    (tfcc_runtime/operations/nn/gather.cpp:60-70, base/cast.cpp:100-111, slicev1.cpp:66-75)."""
+    def refused(build):
+        g = mf.GraphBuilder("g")
+        x = g.input("x", mf.FLOAT, [4, 4])
+        out = build(g, x)
+        g.output(out)
+        with pytest.raises(rt.RuntimeError_, match="(?i)unknow"):
+            rt.Model(mf.write_model([g], "g"), host=True).run({"x": np.zeros((4, 4), np.float32)})
+
+    def gather_with_byte_indices(g, x):
+        out = g.variable("o")
+        g.node("nn.Gather", [x, g.constant("i", np.zeros(3, np.int8))], [out])
+        return out
+
+    def cast_to_another_type_than_declared(g, x):
+        out = g.variable("o", mf.INT32)
+        g.node("base.Cast", [x], [out], mf.f_varint(1, mf.INT64))
+        return out
+
+    def slice_at_a_float_position(g, x):
+        out = g.variable("o")
+        g.node("base.SliceV1", [x, g.constant("p", np.array(1.0, np.float32), mf.CONSTANT_VALUE)], [out],
+               mf.f_varint(1, 0) + mf.f_varint(2, 1))
+        return out
+    for build in (gather_with_byte_indices, cast_to_another_type_than_declared, slice_at_a_float_position):
+        refused(build)
+
+
 def bidirectional_lstm_graph(mf, rng, seq, batch, length, hidden, hidden_field=None):
     u = lambda *s: rng.uniform(-1, 1, s).astype(np.float32)  # noqa: E731
     w = dict(ik=u(2, length, 4 * hidden), sk=u(2, hidden, 4 * hidden), bias=u(2, 4 * hidden), ih=u(2, batch, hidden),

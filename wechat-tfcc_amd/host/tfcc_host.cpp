@@ -3,6 +3,7 @@
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
+#include <type_traits>
 
 #include "tfcc_rocm.h"
 #include "tfcc_layers.h"
@@ -374,6 +375,9 @@ class ROCMDataInterface : public DataInterface<T> {
     std::memcpy(&bits, &one, sizeof(T));
     check(tfcc_rocm_fill_async(current_stream(), a.data(), bits, sizeof(T), a.size()));
   }
+  void castFrom(const void* source, int sourceCode, Variable<T>& result) override {
+    check(tfcc_rocm_cast(current_stream(), source, sourceCode, result.data(), ElementCode<T>::value, result.size()));
+  }
   Variable<T> copy(const Tensor<T>& a) override {
     Variable<T> r(a.shape());
     check(tfcc_rocm_memcpy_d2d_async(current_stream(), r.data(), a.data(), static_cast<size_t>(a.size()) * sizeof(T)));
@@ -671,14 +675,65 @@ class ROCMNormalizationInterface : public NormalizationInterface<float> {
   }
 };
 
-class ROCMBasicInterface : public BasicInterface<float> {
+// slice, concat and gather move bytes and exist for every element type; transpose is the float kernel.
+template <class T>
+class ROCMBasicInterface : public BasicInterface<T> {
+  static void split_at(const Shape& shape, size_t axis, uint64_t& s1, uint64_t& s3) {
+    s1 = s3 = 1;
+    for (size_t i = 0; i < axis; ++i) s1 *= shape[i];
+    for (size_t i = axis + 1; i < shape.size(); ++i) s3 *= shape[i];
+  }
+
  public:
-  Variable<float> transpose(const Tensor<float>& a, const std::vector<size_t>& perm) override {
-    if (a.size() == 0) throw InvalidArgumentError("invalid tensor");
-    std::vector<unsigned> shape = a.shape().toVector(), p(perm.begin(), perm.end()), out(perm.size());
-    for (size_t i = 0; i < perm.size(); ++i) out[i] = shape[perm[i]];
-    Variable<float> r{Shape(std::move(out))};
-    check(tfcc_rocm_transpose_f32(current_stream(), a.data(), shape.data(), p.data(), static_cast<int>(p.size()), r.data()));
+  Variable<T> transpose(const Tensor<T>& a, const std::vector<size_t>& perm) override {
+    if constexpr (std::is_same<T, float>::value) {
+      if (a.size() == 0) throw InvalidArgumentError("invalid tensor");
+      std::vector<unsigned> shape = a.shape().toVector(), p(perm.begin(), perm.end()), out(perm.size());
+      for (size_t i = 0; i < perm.size(); ++i) out[i] = shape[perm[i]];
+      Variable<float> r{Shape(std::move(out))};
+      check(tfcc_rocm_transpose_f32(current_stream(), a.data(), shape.data(), p.data(), static_cast<int>(p.size()), r.data()));
+      return r;
+    } else {
+      throw NotImplementedError("transpose: float only");
+    }
+  }
+  Variable<T> slice(const Tensor<T>& a, size_t axis, unsigned start, unsigned end) override {
+    end = std::min(end, a.shape(axis));  // tfcc/mkl/interfaces/tfcc_mklbasicinterface.cpp:490
+    std::vector<unsigned> shape = a.shape().toVector();
+    shape[axis] = end - start;
+    Variable<T> r{Shape(shape)};
+    if (r.size() == 0) return r;
+    uint64_t s1, s3;
+    split_at(a.shape(), axis, s1, s3);
+    const uint64_t row = static_cast<uint64_t>(end - start) * s3 * sizeof(T);
+    check(tfcc_rocm_copy2d(current_stream(), a.data() + static_cast<size_t>(start) * s3, a.shape(axis) * s3 * sizeof(T),
+                           r.data(), row, s1, row));
+    return r;
+  }
+  Variable<T> concat(const std::vector<const Tensor<T>*>& values, size_t axis) override {
+    std::vector<unsigned> shape = values[0]->shape().toVector();
+    shape[axis] = 0;
+    for (const Tensor<T>* v : values) shape[axis] += v->shape(axis);
+    Variable<T> r{Shape(shape)};
+    if (r.size() == 0) return r;
+    uint64_t s1, s3;
+    split_at(r.shape(), axis, s1, s3);
+    const uint64_t pitch = static_cast<uint64_t>(shape[axis]) * s3 * sizeof(T);
+    size_t offset = 0;  // elements into a row of the result
+    for (const Tensor<T>* v : values) {
+      const uint64_t width = static_cast<uint64_t>(v->shape(axis)) * s3 * sizeof(T);
+      if (width != 0) check(tfcc_rocm_copy2d(current_stream(), v->data(), width, r.data() + offset, pitch, s1, width));
+      offset += static_cast<size_t>(v->shape(axis)) * s3;
+    }
+    return r;
+  }
+  Variable<T> gather(const Tensor<T>& params, const void* indices, int indexCode, const Shape& indexShape) override {
+    std::vector<unsigned> shape = indexShape.toVector();
+    for (size_t i = 1; i < params.shape().size(); ++i) shape.push_back(params.shape(i));
+    Variable<T> r{Shape(shape)};
+    const uint64_t chunk = static_cast<uint64_t>(params.size() / params.shape(0)) * sizeof(T);
+    check(tfcc_rocm_gather_rows(current_stream(), params.data(), params.shape(0), chunk, indices, indexCode, indexShape.area(),
+                                r.data()));
     return r;
   }
 };
@@ -744,6 +799,7 @@ class ROCMTransformationInterface : public TransformationInterface<float> {
 template <class T>
 void install_common(Interface<T>& i) {
   i.setDataInterface(std::unique_ptr<DataInterface<T>>(new ROCMDataInterface<T>()));
+  i.setBasicInterface(std::unique_ptr<BasicInterface<T>>(new ROCMBasicInterface<T>()));
 }
 template <class T>
 void install_quantization(Interface<T>& i) {
@@ -799,7 +855,6 @@ ROCMDevice::ROCMDevice(unsigned index, std::unique_ptr<Allocator> allocator)
   _interfaces->f32.setBlasInterface(std::unique_ptr<BlasInterface<float>>(new ROCMBlasInterface()));
   _interfaces->f32.setActivationInterface(std::unique_ptr<ActivationInterface<float>>(new ROCMActivationInterface()));
   _interfaces->f32.setNormalizationInterface(std::unique_ptr<NormalizationInterface<float>>(new ROCMNormalizationInterface()));
-  _interfaces->f32.setBasicInterface(std::unique_ptr<BasicInterface<float>>(new ROCMBasicInterface()));
   _interfaces->f32.setArithmeticInterface(std::unique_ptr<ArithmeticInterface<float>>(new ROCMArithmeticInterface()));
   _interfaces->f32.setCellInterface(std::unique_ptr<CellInterface<float>>(new ROCMCellInterface()));
   _interfaces->f32.setTransformationInterface(std::unique_ptr<TransformationInterface<float>>(new ROCMTransformationInterface()));

@@ -26,6 +26,14 @@
 
 namespace tfcc {
 
+// Element type codes shared by the type-generic calls below (the order of the C ABI's TFCC_ROCM_S8 .. F64).
+template <class T> struct ElementCode;
+#define TFCC_ELEMENT_CODE(T, V) template <> struct ElementCode<T> { static constexpr int value = V; };
+TFCC_ELEMENT_CODE(int8_t, 0) TFCC_ELEMENT_CODE(uint8_t, 1) TFCC_ELEMENT_CODE(int16_t, 2) TFCC_ELEMENT_CODE(uint16_t, 3)
+TFCC_ELEMENT_CODE(int32_t, 4) TFCC_ELEMENT_CODE(uint32_t, 5) TFCC_ELEMENT_CODE(int64_t, 6) TFCC_ELEMENT_CODE(uint64_t, 7)
+TFCC_ELEMENT_CODE(float, 8) TFCC_ELEMENT_CODE(double, 9)
+#undef TFCC_ELEMENT_CODE
+
 template <class T>
 class BlasInterface {
  public:
@@ -74,6 +82,8 @@ class DataInterface {
   virtual void zeros(Variable<T>&) { throw NotImplementedError(); }
   virtual void ones(Variable<T>&) { throw NotImplementedError(); }
   virtual Variable<T> copy(const Tensor<T>&) { throw NotImplementedError(); }
+  // static_cast of `total` elements of the type with code `sourceCode` (ElementCode) into a tensor of this type
+  virtual void castFrom(const void* /*source*/, int /*sourceCode*/, Variable<T>& /*result*/) { throw NotImplementedError(); }
 };
 
 template <class T>
@@ -103,6 +113,12 @@ class BasicInterface {
  public:
   virtual ~BasicInterface() {}
   virtual Variable<T> transpose(const Tensor<T>&, const std::vector<size_t>&) { throw NotImplementedError(); }
+  virtual Variable<T> slice(const Tensor<T>&, size_t, unsigned, unsigned) { throw NotImplementedError(); }
+  virtual Variable<T> concat(const std::vector<const Tensor<T>*>&, size_t) { throw NotImplementedError(); }
+  // rows of params by index (tfcc/core/interfaces/tfcc_gatherinterface.h): indices of the type with code indexCode
+  virtual Variable<T> gather(const Tensor<T>&, const void* /*indices*/, int /*indexCode*/, const Shape& /*indexShape*/) {
+    throw NotImplementedError();
+  }
 };
 
 template <class T>
@@ -446,6 +462,58 @@ Variable<T> layer_normalization(const Tensor<T>& a, const Tensor<T>& gamma, cons
                                                                                         beginNormAxis);
 }
 
+}  // namespace nn
+
+namespace data {
+// tfcc::data::cast<DST>(a): element-wise static_cast
+template <class DST, class SRC>
+Variable<DST> cast(const Tensor<SRC>& a) {
+  Variable<DST> result(a.shape());
+  if (a.size() == 0) return result;
+  Operation<DST>::getCurrentInterface().getDataInterface().castFrom(a.data(), ElementCode<SRC>::value, result);
+  return result;
+}
+}  // namespace data
+
+namespace base {
+// tfcc/core/operations/tfcc_base.cpp:28-41
+template <class T>
+Variable<T> slice(const Tensor<T>& a, size_t axis, unsigned start, unsigned end) {
+  if (axis >= a.shape().size()) throw InvalidArgumentError("invalid axis");
+  if (start >= end) throw InvalidArgumentError("start large than end");
+  if (start >= a.shape(axis)) throw InvalidArgumentError("invalid start");
+  return Operation<T>::getCurrentInterface().getBasicInterface().slice(a, axis, start, end);
+}
+// tfcc/core/operations/tfcc_base.cpp:86-121
+template <class T>
+Variable<T> concat(const std::vector<const Tensor<T>*>& values, size_t axis) {
+  if (values.size() == 0) throw InvalidArgumentError("values.size could not be zero");
+  for (const Tensor<T>* tensor : values) {
+    if (axis >= tensor->shape().size()) throw InvalidArgumentError("invalid axis");
+    if (tensor->shape().size() != values[0]->shape().size()) throw InvalidArgumentError("invalid shape");
+    for (size_t i = 0; i < tensor->shape().size(); ++i)
+      if (i != axis && tensor->shape(i) != values[0]->shape(i)) throw InvalidArgumentError("invalid shape");
+  }
+  return Operation<T>::getCurrentInterface().getBasicInterface().concat(values, axis);
+}
+template <class T>
+Variable<T> concat(std::initializer_list<const Tensor<T>*> values, size_t axis) {
+  return concat(std::vector<const Tensor<T>*>(values), axis);
+}
+}  // namespace base
+
+namespace nn {
+// tfcc::nn::gather (tfcc/core/operations/tfcc_nn.cpp:345-385) for int32 / uint32 / int64 / uint64 indices
+template <class T, class IDX>
+Variable<T> gather(const Tensor<T>& params, const Tensor<IDX>& indices) {
+  static_assert(ElementCode<IDX>::value >= 4 && ElementCode<IDX>::value <= 7, "indices of 32 or 64 bits");
+  if (params.size() == 0) throw InvalidArgumentError("invalid tensor");
+  std::vector<unsigned> shape = indices.shape().toVector();
+  for (size_t i = 1; i < params.shape().size(); ++i) shape.push_back(params.shape(i));
+  if (indices.size() == 0) return Variable<T>(Shape(std::move(shape)));
+  return Operation<T>::getCurrentInterface().getBasicInterface().gather(params, indices.data(), ElementCode<IDX>::value,
+                                                                      indices.shape());
+}
 }  // namespace nn
 
 namespace rnn {

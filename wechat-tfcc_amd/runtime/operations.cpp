@@ -12,6 +12,8 @@
 //   rnn.BidirectionalLSTM               operations/rnn/bidirectionallstm.cpp:27-128
 //   base.Squeeze / Unsqueeze / Flatten  operations/base/squeeze.cpp, unsqueeze.cpp, flatten.cpp (Views of the input)
 //   base.GetShape, base.GetDimension    operations/base/getshape.cpp, getdimension.cpp
+//   nn.Gather, base.Cast, base.SliceV1, base.Concat
+//                                       operations/nn/gather.cpp, base/cast.cpp, slicev1.cpp, concat.cpp
 //   base.Transpose, base.Reshape, base.Identity, base.CreateVector
 //                                       operations/base/transpose.cpp, reshape.cpp:27-59,74-104,
 //                                       identity.cpp, createvector.cpp:63-121
@@ -19,6 +21,7 @@
 #include <array>
 #include <cmath>
 #include <map>
+#include <type_traits>
 
 #include "runtime.h"
 
@@ -437,6 +440,124 @@ class GetDimension : public TypedOperation<SRC> {
   }
 };
 
+// ---- nn.Gather, base.Cast, base.SliceV1, base.Concat: data movement between the products -------------------------
+// tfcc_runtime/operations/nn/gather.cpp:27-92 (axis 0 only), base/cast.cpp:30-129 (tensor and value forms),
+// base/slicev1.cpp:27-92 (start from a value symbol, length from the message), base/concat.cpp:27-90
+template <class T, class IDX>
+class Gather : public TypedOperation<T> {
+ public:
+  Gather() : TypedOperation<T>("nn.Gather") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 2 || node.outputs.size() != 1) return false;
+    auto& sm = graph.getSymbolManager();
+    if (sm.getSymbolInfo(node.outputs[0]).dtype != this->DTYPE || sm.getSymbolInfo(node.inputs[0]).dtype != this->DTYPE)
+      return false;
+    if (sm.getSymbolInfo(node.inputs[1]).dtype != DataTypeOf<IDX>::value) return false;
+    uint64_t axis = 0;
+    wire::Reader r(node.operation);
+    uint32_t f, t;
+    while (r.next(f, t)) {
+      if (f == 1 && t == 0) axis = r.varint();
+      else r.skip(t);
+    }
+    const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+    const Tensor<IDX>* indices = sm.getTensor(node.inputs[1], IDX());
+    Variable<T>* out = sm.getVariable(node.outputs[0], T());
+    graph.addStep([a, indices, axis, out] {
+      if (axis != 0) throw RuntimeError("Gather: invalid axis");
+      *out = nn::gather(*a, *indices);
+    });
+    return true;
+  }
+};
+
+template <class SRC, class DST>
+class Cast : public TypedOperation<SRC> {
+ public:
+  Cast() : TypedOperation<SRC>("base.Cast") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 1 || node.outputs.size() != 1) return false;
+    auto& sm = graph.getSymbolManager();
+    const SymbolInfo& in = sm.getSymbolInfo(node.inputs[0]);
+    const SymbolInfo& outInfo = sm.getSymbolInfo(node.outputs[0]);
+    if (outInfo.dtype != DataTypeOf<DST>::value || in.dtype != this->DTYPE) return false;
+    uint64_t wanted = 0;
+    wire::Reader r(node.operation);
+    uint32_t f, t;
+    while (r.next(f, t)) {
+      if (f == 1 && t == 0) wanted = r.varint();
+      else r.skip(t);
+    }
+    if (wanted != static_cast<uint64_t>(DataTypeOf<DST>::value)) return false;
+    if (is_tensor(in.stype) && is_tensor(outInfo.stype)) {
+      const Tensor<SRC>* a = sm.getTensor(node.inputs[0], SRC());
+      Variable<DST>* out = sm.getVariable(node.outputs[0], DST());
+      graph.addStep([a, out] { *out = data::cast<DST>(*a); });
+    } else if (is_value(in.stype) && is_value(outInfo.stype)) {
+      const SRC* a = sm.getValue(node.inputs[0], SRC());
+      DST* out = sm.getValue(node.outputs[0], DST());
+      graph.addStep([a, out] { *out = static_cast<DST>(*a); });
+    } else {
+      return false;
+    }
+    return true;
+  }
+};
+
+template <class T, class POS>
+class SliceV1 : public TypedOperation<T> {
+ public:
+  SliceV1() : TypedOperation<T>("base.SliceV1") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (!std::is_integral<POS>::value) return false;  // the position is a value of one of the eight integer types
+    if (node.inputs.size() != 2 || node.outputs.size() != 1) return false;
+    auto& sm = graph.getSymbolManager();
+    if (sm.getSymbolInfo(node.outputs[0]).dtype != this->DTYPE || sm.getSymbolInfo(node.inputs[0]).dtype != this->DTYPE)
+      return false;
+    if (sm.getSymbolInfo(node.inputs[1]).dtype != DataTypeOf<POS>::value) return false;
+    uint64_t axis = 0, length = 0;
+    wire::Reader r(node.operation);
+    uint32_t f, t;
+    while (r.next(f, t)) {
+      if (f == 1 && t == 0) axis = r.varint();
+      else if (f == 2 && t == 0) length = r.varint();
+      else r.skip(t);
+    }
+    const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+    const POS* pos = sm.getValue(node.inputs[1], POS());
+    Variable<T>* out = sm.getVariable(node.outputs[0], T());
+    graph.addStep([a, pos, axis, length, out] {
+      if (*pos < POS(0)) throw RuntimeError("SliceV1: invalid pos");
+      const unsigned start = static_cast<unsigned>(*pos);
+      *out = base::slice(*a, static_cast<size_t>(axis), start, start + static_cast<unsigned>(length));
+    });
+    return true;
+  }
+};
+
+template <class T>
+class Concat : public TypedOperation<T> {
+ public:
+  Concat() : TypedOperation<T>("base.Concat") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.empty() || node.outputs.size() != 1) return false;
+    if (!same_dtype(graph, node.outputs, this->DTYPE) || !same_dtype(graph, node.inputs, this->DTYPE)) return false;
+    uint64_t axis = 0;
+    wire::Reader r(node.operation);
+    uint32_t f, t;
+    while (r.next(f, t)) {
+      if (f == 1 && t == 0) axis = r.varint();
+      else r.skip(t);
+    }
+    auto& sm = graph.getSymbolManager();
+    std::vector<const Tensor<T>*> values;
+    for (const std::string& name : node.inputs) values.push_back(sm.getTensor(name, T()));
+    Variable<T>* out = sm.getVariable(node.outputs[0], T());
+    graph.addStep([values, axis, out] { *out = base::concat(values, static_cast<size_t>(axis)); });
+    return true;
+  }
+};
+
 // ---- base.Identity -----------------------------------------------------------------------------------------------
 template <class T>
 class Identity : public TypedOperation<T> {
@@ -637,6 +758,16 @@ class Collector {
     add(new ShapeView<Reshaping::UNSQUEEZE, T>());
     add(new ShapeView<Reshaping::FLATTEN, T>());
     add(new GetShape<T>());
+    add(new Gather<T, int32_t>());
+    add(new Gather<T, uint32_t>());
+    add(new Gather<T, int64_t>());
+    add(new Gather<T, uint64_t>());
+    add(new Concat<T>());
+#define TFCC_RUNTIME_ADD_PAIR(OTHER, E) \
+  add(new Cast<T, OTHER>());            \
+  add(new SliceV1<T, OTHER>());
+    TFCC_RUNTIME_FOR_ALL_TYPES(TFCC_RUNTIME_ADD_PAIR)
+#undef TFCC_RUNTIME_ADD_PAIR
 #define TFCC_RUNTIME_ADD_DIMENSION(DST, E) add(new GetDimension<T, DST>());
     TFCC_RUNTIME_FOR_ALL_TYPES(TFCC_RUNTIME_ADD_DIMENSION)
 #undef TFCC_RUNTIME_ADD_DIMENSION
