@@ -667,6 +667,79 @@ static void test_lstmcell_from_constants() {
   }
 }
 
+// tfcc/test/rnn.cpp:36-54 and 106-124: the two GRU cells, data as tfcc/test/python/testcase/rnn/grucell.py and
+// pytorchgrucell.py make it ("rnn/grucell/<i>/...", "rnn/pytorch_grucell/<i>/...").
+static void test_grucells_from_constants() {
+  auto scope1 = tfcc::Scope::scope("rnn");
+  {
+    auto scope2 = tfcc::Scope::scope("grucell");
+    size_t count = tfcc::Configure<uint64_t>::getConfigure("__count__");
+    CHECK(count > 0);
+    for (size_t i = 0; i < count; ++i) {
+      auto scope3 = tfcc::Scope::scope(std::to_string(i));
+      unsigned units = tfcc::Configure<unsigned>::getConfigure("units");
+      tfcc::rnn::GRUCell<float> cell(units);
+      tfcc::Constant<float>& inputs = tfcc::Constant<float>::getConstant("inputs");
+      tfcc::Variable<float> state = tfcc::data::copy(tfcc::Constant<float>::getConstant("state"));
+      tfcc::Variable<float> result, nextState;
+      std::tie(result, nextState) = cell(inputs, state, 0, {});
+      CHECK(all_similar(result, tfcc::Constant<float>::getConstant("expect")));
+      CHECK(all_similar(nextState, tfcc::Constant<float>::getConstant("expect")));
+    }
+  }
+  {
+    auto scope2 = tfcc::Scope::scope("pytorch_grucell");
+    size_t count = tfcc::Configure<uint64_t>::getConfigure("__count__");
+    CHECK(count > 0);
+    for (size_t i = 0; i < count; ++i) {
+      auto scope3 = tfcc::Scope::scope(std::to_string(i));
+      unsigned units = tfcc::Configure<unsigned>::getConfigure("units");
+      tfcc::rnn::PyTorchGRUCell<float> cell(units);
+      tfcc::Constant<float>& inputs = tfcc::Constant<float>::getConstant("inputs");
+      tfcc::Variable<float> state = tfcc::data::copy(tfcc::Constant<float>::getConstant("state"));
+      tfcc::Variable<float> result, nextState;
+      std::tie(result, nextState) = cell(inputs, state, 0, {});
+      CHECK(all_similar(result, tfcc::Constant<float>::getConstant("expect")));
+      std::tie(result, nextState) = cell(inputs, state, 0, {});  // the joined kernels are kept
+      CHECK(all_similar(nextState, tfcc::Constant<float>::getConstant("expect")));
+    }
+  }
+}
+
+// tfcc::base::slice / concat, tfcc::nn::gather and tfcc::data::cast on other element types than float
+// (tfcc/test/base.cpp's slice and concat cases in kind): bytes moved, never converted.
+static void test_data_movement() {
+  std::vector<int32_t> hv(4 * 6);
+  for (size_t i = 0; i < hv.size(); ++i) hv[i] = static_cast<int32_t>(i * 7) - 40;
+  tfcc::Variable<int32_t> v = tfcc::data::set(hv, {4, 6});
+  std::vector<int32_t> s = tfcc::data::get(tfcc::base::slice(v, 1, 2, 5));
+  bool ok = s.size() == 12;
+  for (unsigned r = 0; ok && r < 4; ++r)
+    for (unsigned c = 0; c < 3; ++c) ok = ok && s[r * 3 + c] == hv[r * 6 + 2 + c];
+  CHECK(ok);
+  CHECK(tfcc::base::slice(v, 0, 3, 99).shape() == tfcc::Shape({1, 6}));
+  CHECK_THROWS_MSG(tfcc::base::slice(v, 2, 0, 1), tfcc::InvalidArgumentError, "invalid axis");
+  CHECK_THROWS_MSG(tfcc::base::slice(v, 1, 3, 3), tfcc::InvalidArgumentError, "start large than end");
+  CHECK_THROWS_MSG(tfcc::base::slice(v, 1, 6, 7), tfcc::InvalidArgumentError, "invalid start");
+  tfcc::Variable<int32_t> left = tfcc::base::slice(v, 1, 0, 2), right = tfcc::base::slice(v, 1, 2, 6);
+  CHECK(tfcc::data::get(tfcc::base::concat<int32_t>({&left, &right}, 1)) == hv);
+  tfcc::Variable<int32_t> top = tfcc::base::slice(v, 0, 0, 1), rest = tfcc::base::slice(v, 0, 1, 4);
+  CHECK(tfcc::data::get(tfcc::base::concat<int32_t>({&top, &rest}, 0)) == hv);
+  CHECK_THROWS_MSG(tfcc::base::concat<int32_t>({&left, &top}, 1), tfcc::InvalidArgumentError, "invalid shape");
+  tfcc::Variable<int64_t> idx = tfcc::data::set(std::vector<int64_t>{3, -1, 0, 4}, {2, 2});
+  std::vector<int32_t> g = tfcc::data::get(tfcc::nn::gather(v, idx));
+  ok = g.size() == 24;
+  for (unsigned c = 0; ok && c < 6; ++c) ok = g[c] == hv[18 + c] && g[6 + c] == 0 && g[12 + c] == hv[c] && g[18 + c] == 0;
+  CHECK(ok);
+  std::vector<float> f = tfcc::data::get(tfcc::data::cast<float>(v));
+  ok = true;
+  for (size_t i = 0; i < hv.size(); ++i) ok = ok && f[i] == static_cast<float>(hv[i]);
+  CHECK(ok);
+  tfcc::Variable<float> fv = tfcc::data::set(std::vector<float>{-2.5f, 0.f, 3.9f, 100.25f}, {4});
+  CHECK(tfcc::data::get(tfcc::data::cast<int8_t>(fv)) == (std::vector<int8_t>{-2, 0, 3, 100}));
+  CHECK(tfcc::data::get(tfcc::data::cast<uint64_t>(tfcc::data::cast<double>(fv)))[3] == 100u);
+}
+
 // tfcc::layer::Dense (tfcc/core/layers/tfcc_denselayer.cpp:47-87) in the style of the reference's layer tests:
 // inputs of rank 2 and 3, with and without bias, custom constant names, and its checks.
 static void test_dense_from_constants() {
@@ -861,6 +934,7 @@ int main(int argc, char** argv) {
     run("layer.elementwise", test_layer_ops);
     run("math.broadcast_arithmetic", test_broadcast_arithmetic);
     run("layer.attention_permuted", test_attention_permuted);
+    run("base.data_movement", test_data_movement);
     run("rnn.cells", test_cells);
     run("rnn.lstm_forward_backward", test_lstm_sequences);
     if (argc > 2) {  // an .npz of named test data, written by the Python side
@@ -869,6 +943,7 @@ int main(int argc, char** argv) {
       run("framework.scopes_and_constants", test_scopes_and_constants);
       run("rnn.lstmcell", test_lstmcell_from_constants);
       run("layer.dense", test_dense_from_constants);
+      run("rnn.grucells", test_grucells_from_constants);
       tfcc::DataLoader::setGlobalDefault(nullptr);
     }
     run("threads.two_sessions", test_two_sessions_on_two_threads);

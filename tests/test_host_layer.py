@@ -36,6 +36,33 @@ def write_named_test_data(path, seed=5):
         data.update({prefix + "units": np.asarray([units], np.int32), prefix + "inputs": inputs, prefix + "h": h,
                      prefix + "cs": cs, prefix + "lstm_cell/kernel": kernel, prefix + "lstm_cell/bias": bias,
                      prefix + "ecs": next_cs.astype(np.float32), prefix + "expect": expect.astype(np.float32)})
+    # tfcc/test/python/testcase/rnn/grucell.py:31-56 and pytorchgrucell.py:24-60
+    cases = [(1, 64, 64), (4, 130, 75), (9, 96, 200)]
+    data["rnn/grucell/__count__"] = np.asarray([len(cases)], np.int32)
+    data["rnn/pytorch_grucell/__count__"] = np.asarray([len(cases)], np.int32)
+    for i, (batch, units, input_size) in enumerate(cases):
+        inputs, state = u(batch, input_size), u(batch, units)
+        g_kernel, g_bias = u(input_size + units, units * 2), u(units * 2)
+        c_kernel, c_bias = u(input_size + units, units), u(units)
+        value = _sig(np.concatenate((inputs, state), axis=1).astype(np.float64) @ g_kernel + g_bias)
+        r, upd = np.split(value, 2, axis=1)
+        cand = np.tanh(np.concatenate((inputs, r * state), axis=1) @ c_kernel.astype(np.float64) + c_bias)
+        prefix = "rnn/grucell/%d/" % i
+        data.update({prefix + "units": np.asarray([units], np.int32), prefix + "inputs": inputs, prefix + "state": state,
+                     prefix + "gru_cell/gates/kernel": g_kernel, prefix + "gru_cell/gates/bias": g_bias,
+                     prefix + "gru_cell/candidate/kernel": c_kernel, prefix + "gru_cell/candidate/bias": c_bias,
+                     prefix + "expect": (upd * state + (1 - upd) * cand).astype(np.float32)})
+        ci_kernel, ci_bias, ch_kernel, ch_bias = u(input_size, units), u(units), u(units, units), u(units)
+        r, z = value[:, :units], value[:, units:]
+        ni = inputs.astype(np.float64) @ ci_kernel + ci_bias
+        nh = state.astype(np.float64) @ ch_kernel + ch_bias
+        n = np.tanh(ni + r * nh)
+        prefix = "rnn/pytorch_grucell/%d/" % i
+        data.update({prefix + "units": np.asarray([units], np.int32), prefix + "inputs": inputs, prefix + "state": state,
+                     prefix + "gru_cell/weight_gates": g_kernel, prefix + "gru_cell/bias_gates": g_bias,
+                     prefix + "gru_cell/weight_candidate_i": ci_kernel, prefix + "gru_cell/bias_candidate_i": ci_bias,
+                     prefix + "gru_cell/weight_candidate_h": ch_kernel, prefix + "gru_cell/bias_candidate_h": ch_bias,
+                     prefix + "expect": (n + z * (state - n)).astype(np.float32)})
     cases = [((5, 70), 33), ((2, 3, 768), 3072), ((1, 512), 2048), ((2, 2, 9, 40), 17)]
     data["layer/dense/__count__"] = np.asarray([len(cases)], np.int32)
     for i, (shape, units) in enumerate(cases):

@@ -6,6 +6,8 @@
 //   Configure<T>             tfcc/core/framework/tfcc_configure.h (scalars by name)
 //   layer::Dense, dense()    tfcc/core/layers/tfcc_denselayer.cpp:31-125
 //   rnn::LSTMCell            tfcc/core/rnn/tfcc_lstmcell.cpp:34-96
+//   rnn::GRUCell             tfcc/core/rnn/tfcc_grucell.cpp:46-105
+//   rnn::PyTorchGRUCell      tfcc/core/rnn/tfcc_pytorchgrucell.cpp:53-118
 // On the ROCm device Dense is one launch: the bias is added in the matmul's epilogue, which gives the bits of
 // matmul followed by the broadcast add the reference runs.
 #pragma once
@@ -297,6 +299,120 @@ class LSTMCell {
         blas::matmul(state.h, View<T>(*_kernel, _kernel->shape(), inputs.shape(1))), *_bias, static_cast<T>(1));
     Variable<T> output = data::copy(next.h);
     return std::make_pair(std::move(output), std::move(next));
+  }
+};
+
+// One step of a GRU in TensorFlow's layout (tfcc/core/rnn/tfcc_grucell.cpp:46-105): "<name>/gates/kernel"
+// [inputSize + units, 2 units] with "gates/bias", "<name>/candidate/kernel" [inputSize + units, units] with
+// "candidate/bias".  Sequence lengths are not implemented on this device.
+template <class T>
+class GRUCell {
+  bool _initialized = false;
+  unsigned _units;
+  std::string _name;
+  Constant<T>* _gatesKernel = nullptr;
+  Constant<T>* _gatesBias = nullptr;
+  Constant<T>* _candidateKernel = nullptr;
+  Constant<T>* _candidateBias = nullptr;
+
+ public:
+  using State = Variable<T>;
+
+  explicit GRUCell(unsigned units) : GRUCell(units, "gru_cell") {}
+  GRUCell(unsigned units, std::string name) : _units(units), _name(std::move(name)) {}
+
+  State zeroState(unsigned batch) {
+    State state({batch, _units});
+    data::zeros(state);
+    return state;
+  }
+
+  std::pair<Variable<T>, State> operator()(const Tensor<T>& input, const State& state, size_t step = 0,
+                                           const std::vector<unsigned>& lengths = {}) {
+    (void)step;
+    if (input.shape().size() != 2) throw InvalidArgumentError("invalid inputs");
+    if (input.shape(0) != state.shape(0)) throw InvalidArgumentError("state and inputs don't match");
+    if (lengths.size() != 0 && lengths.size() != input.shape(0)) throw InvalidArgumentError("invalid lengths");
+    if (lengths.size() != 0) throw NotImplementedError("GRUCell with sequence lengths");
+    auto scopeG = Scope::scope(_name);
+    if (!_initialized) {
+      {
+        auto scopeGates = Scope::scope("gates");
+        _gatesKernel = &Constant<T>::getConstant("kernel");
+        _gatesBias = &Constant<T>::getConstant("bias");
+      }
+      {
+        auto scopeCandidate = Scope::scope("candidate");
+        _candidateKernel = &Constant<T>::getConstant("kernel");
+        _candidateBias = &Constant<T>::getConstant("bias");
+      }
+      _initialized = true;
+    }
+    Variable<T> gi = base::concat<T>({&input, &state}, 1);
+    Variable<T> value = blas::matmul(gi, *_gatesKernel);
+    Interface<T>& interface = Operation<T>::getCurrentInterface();
+    Variable<T> ci = interface.getCellInterface().processGRUCellGates(state, input, value, *_gatesBias);
+    State h = interface.getCellInterface().processGRUCellCandidate(state, value, *_gatesBias,
+                                                                   blas::matmul(ci, *_candidateKernel), *_candidateBias);
+    Variable<T> output = data::copy(h);
+    return std::make_pair(std::move(output), std::move(h));
+  }
+};
+
+// One step of a GRU in PyTorch's formulation (tfcc/core/rnn/tfcc_pytorchgrucell.cpp:53-118): "weight_gates"
+// [inputSize + units, 2 units], "weight_candidate_i" [inputSize, units], "weight_candidate_h" [units, units] and the
+// three biases.  The reference joins them into an input kernel [inputSize, 3 units] and a state kernel
+// [units, 3 units] at first use and keeps those; so does this class (slice + concat on the device).
+template <class T>
+class PyTorchGRUCell {
+  bool _initialized = false;
+  unsigned _units;
+  std::string _name;
+  Constant<T>* _gatesBias = nullptr;
+  Constant<T>* _candidateIBias = nullptr;
+  Constant<T>* _candidateHBias = nullptr;
+  Variable<T> _inputKernel, _stateKernel;
+
+ public:
+  using State = Variable<T>;
+
+  explicit PyTorchGRUCell(unsigned units) : PyTorchGRUCell(units, "gru_cell") {}
+  PyTorchGRUCell(unsigned units, std::string name) : _units(units), _name(std::move(name)) {}
+
+  State zeroState(unsigned batch) {
+    State state({batch, _units});
+    data::zeros(state);
+    return state;
+  }
+
+  std::pair<Variable<T>, State> operator()(const Tensor<T>& input, const State& state, size_t step = 0,
+                                           const std::vector<unsigned>& lengths = {}) {
+    (void)step;
+    if (input.shape().size() != 2) throw InvalidArgumentError("invalid inputs");
+    if (input.shape(0) != state.shape(0)) throw InvalidArgumentError("state and inputs don't match");
+    if (lengths.size() != 0 && lengths.size() != input.shape(0)) throw InvalidArgumentError("invalid lengths");
+    if (lengths.size() != 0) throw NotImplementedError("PyTorchGRUCell with sequence lengths");
+    auto scopeG = Scope::scope(_name);
+    if (!_initialized) {
+      _gatesBias = &Constant<T>::getConstant("bias_gates");
+      _candidateIBias = &Constant<T>::getConstant("bias_candidate_i");
+      _candidateHBias = &Constant<T>::getConstant("bias_candidate_h");
+      Constant<T>& gatesKernel = Constant<T>::getConstant("weight_gates");
+      Constant<T>& candidateIKernel = Constant<T>::getConstant("weight_candidate_i");
+      Constant<T>& candidateHKernel = Constant<T>::getConstant("weight_candidate_h");
+      const unsigned inputSize = candidateIKernel.shape(0);
+      if (gatesKernel.shape().size() != 2 || gatesKernel.shape(0) <= inputSize) throw InvalidDataError("invalid kernel");
+      View<T> g1(gatesKernel, gatesKernel.shape(), 0, inputSize), g2(gatesKernel, gatesKernel.shape(), inputSize);
+      _inputKernel = base::concat<T>({&g1, &candidateIKernel}, 1);
+      _stateKernel = base::concat<T>({&g2, &candidateHKernel}, 1);
+      _initialized = true;
+    }
+    Variable<T> inputValue = blas::matmul(input, _inputKernel);
+    Variable<T> stateValue = blas::matmul(state, _stateKernel);
+    State hy = Operation<T>::getCurrentInterface().getCellInterface().processPyTorchGRUCell(
+        state, inputValue, stateValue, *_gatesBias, *_candidateIBias, *_candidateHBias);
+    Variable<T> output = data::copy(hy);
+    return std::make_pair(std::move(output), std::move(hy));
   }
 };
 
