@@ -134,6 +134,60 @@ def test_shape_nodes_on_host(mf, rt):
     assert out.shape == (2, 1, 3, 1) and np.array_equal(out, a)
 
 
+def test_symbol_kind_conversions_on_host(mf, rt):
+    """base.At / At1 pick an element of a vector, base.ToTensor / ToValue / ToVector move a symbol between the three
+    kinds (tfcc_runtime/operations/base/at.cpp, at1.cpp, totensor.cpp, tovalue.cpp, tovector.cpp): the way a converted
+    model computes a new shape from an input's shape."""
+    a = np.arange(24, dtype=np.float32).reshape(2, 1, 3, 4)
+    g = mf.GraphBuilder("g")
+    x = g.input("x", mf.FLOAT, [2, 1, 3, 4])
+    shape = g.vector("shape", mf.UINT32)
+    g.node("base.GetShape", [x], [shape])
+    third = g._symbol("third", mf.UINT32, mf.VALUE)
+    g.node("base.At1", [shape], [third], mf.f_varint(1, 2))
+    first = g._symbol("first", mf.UINT32, mf.VALUE)
+    g.node("base.At", [shape, g.constant("zero", np.array(0, np.int16), mf.CONSTANT_VALUE)], [first])
+    shape_tensor = g.variable("shape_tensor", mf.UINT32)
+    g.node("base.ToTensor", [shape], [shape_tensor])
+    back = g.vector("back", mf.UINT32)
+    g.node("base.ToVector", [shape_tensor], [back])
+    last = g._symbol("last", mf.UINT32, mf.VALUE)
+    g.node("base.At1", [back], [last], mf.f_varint(1, 3))
+    one_tensor = g.variable("one_tensor", mf.UINT32)
+    g.node("base.ToTensor", [third], [one_tensor])
+    again = g._symbol("again", mf.UINT32, mf.VALUE)
+    g.node("base.ToValue", [one_tensor], [again])
+    single = g.vector("single", mf.UINT32)
+    g.node("base.ToVector", [again], [single])
+    from_vector = g._symbol("from_vector", mf.UINT32, mf.VALUE)
+    g.node("base.ToValue", [single], [from_vector])
+    copy = g.variable("copy")
+    g.node("base.ToTensor", [x], [copy])
+    reshaped = g.view("reshaped")
+    g.node("base.Reshape", [copy, back], [reshaped])
+    y = g.variable("y")
+    g.node("base.Identity", [reshaped], [y])
+    for o in (third, first, shape_tensor, last, again, from_vector, y):
+        g.output(o)
+    m = rt.Model(mf.write_model([g], "g"), host=True)
+    res = m.run({"x": a})
+    assert [int(res[k][0]) for k in (third, first, last, again, from_vector)] == [3, 2, 4, 3, 3]
+    assert res[shape_tensor].tolist() == [2, 1, 3, 4] and res[shape_tensor].dtype == np.uint32
+    assert np.array_equal(res[y], a)
+    m.close()
+    for op, payload, inputs, text in (("base.At1", mf.f_varint(1, 4), ["shape"], "At1: invalid pos"),
+                                      ("base.ToValue", b"", ["shape"], "ToValue: invalid size of input")):
+        g2 = mf.GraphBuilder("g")
+        x2 = g2.input("x", mf.FLOAT, [2, 1, 3, 4])
+        sh = g2._symbol("shape", mf.UINT32, mf.VECTOR)
+        g2.node("base.GetShape", [x2], [sh])
+        out = g2._symbol("out", mf.UINT32, mf.VALUE)
+        g2.node(op, inputs, [out], payload)
+        g2.output(out)
+        with pytest.raises(rt.RuntimeError_, match=text):
+            rt.Model(mf.write_model([g2], "g"), host=True).run({"x": a})
+
+
 @pytest.mark.parametrize("compress", [False, True])
 def test_constants_from_npz(mf, rt, compress):
     """element conversion, Fortran order, 0-d arrays, stored and deflated members"""

@@ -12,6 +12,8 @@
 //   rnn.BidirectionalLSTM               operations/rnn/bidirectionallstm.cpp:27-128
 //   base.Squeeze / Unsqueeze / Flatten  operations/base/squeeze.cpp, unsqueeze.cpp, flatten.cpp (Views of the input)
 //   base.GetShape, base.GetDimension    operations/base/getshape.cpp, getdimension.cpp
+//   base.At / At1 / ToTensor / ToValue / ToVector
+//                                       operations/base/at.cpp, at1.cpp, totensor.cpp, tovalue.cpp, tovector.cpp
 //   nn.Gather, base.Cast, base.SliceV1, base.Concat
 //                                       operations/nn/gather.cpp, base/cast.cpp, slicev1.cpp, concat.cpp
 //   base.Transpose, base.Reshape, base.Identity, base.CreateVector
@@ -20,6 +22,7 @@
 #include <algorithm>
 #include <array>
 #include <cmath>
+#include <functional>
 #include <map>
 #include <type_traits>
 
@@ -558,6 +561,114 @@ class Concat : public TypedOperation<T> {
   }
 };
 
+// ---- base.At / At1 / ToTensor / ToValue / ToVector: between the three kinds of symbols ---------------------------
+// tfcc_runtime/operations/base/at.cpp:27-82, at1.cpp:27-75, totensor.cpp:27-116, tovalue.cpp:27-109,
+// tovector.cpp:27-110.  Reading a tensor into a value or a vector waits for the device.
+template <class T, class IDX>
+class At : public TypedOperation<T> {
+ public:
+  At() : TypedOperation<T>("base.At") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (!std::is_integral<IDX>::value) return false;
+    if (node.inputs.size() != 2 || node.outputs.size() != 1) return false;
+    auto& sm = graph.getSymbolManager();
+    if (sm.getSymbolInfo(node.outputs[0]).dtype != this->DTYPE || sm.getSymbolInfo(node.inputs[0]).dtype != this->DTYPE ||
+        sm.getSymbolInfo(node.inputs[1]).dtype != DataTypeOf<IDX>::value)
+      return false;
+    const std::vector<T>* a = sm.getVector(node.inputs[0], T());
+    const IDX* pos = sm.getValue(node.inputs[1], IDX());
+    T* out = sm.getValue(node.outputs[0], T());
+    graph.addStep([a, pos, out] {
+      if (*pos < IDX(0) || static_cast<size_t>(*pos) >= a->size()) throw RuntimeError("At: invalid pos");
+      *out = (*a)[static_cast<size_t>(*pos)];
+    });
+    return true;
+  }
+};
+
+template <class T>
+class At1 : public TypedOperation<T> {
+ public:
+  At1() : TypedOperation<T>("base.At1") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 1 || node.outputs.size() != 1) return false;
+    if (!same_dtype(graph, node.outputs, this->DTYPE) || !same_dtype(graph, node.inputs, this->DTYPE)) return false;
+    size_t idx = 0;
+    wire::Reader r(node.operation);
+    uint32_t f, t;
+    while (r.next(f, t)) {
+      if (f == 1 && t == 0) idx = static_cast<size_t>(r.varint());
+      else r.skip(t);
+    }
+    auto& sm = graph.getSymbolManager();
+    const std::vector<T>* a = sm.getVector(node.inputs[0], T());
+    T* out = sm.getValue(node.outputs[0], T());
+    graph.addStep([a, idx, out] {
+      if (idx >= a->size()) throw RuntimeError("At1: invalid pos");
+      *out = (*a)[idx];
+    });
+    return true;
+  }
+};
+
+enum class Target { TENSOR, VALUE, VECTOR };
+
+template <Target TO, class T>
+class Convert : public TypedOperation<T> {
+  static const char* message() {
+    return TO == Target::TENSOR ? "base.ToTensor" : TO == Target::VALUE ? "base.ToValue" : "base.ToVector";
+  }
+
+ public:
+  Convert() : TypedOperation<T>(message()) {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 1 || node.outputs.size() != 1) return false;
+    if (!same_dtype(graph, node.outputs, this->DTYPE) || !same_dtype(graph, node.inputs, this->DTYPE)) return false;
+    auto& sm = graph.getSymbolManager();
+    const SymbolType from = stype_of(graph, node.inputs[0]);
+    // the three sources, read into a host vector when the step runs
+    std::function<std::vector<T>()> read;
+    if (is_tensor(from)) {
+      const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+      if (TO == Target::TENSOR) {
+        Variable<T>* out = sm.getVariable(node.outputs[0], T());
+        graph.addStep([a, out] { *out = data::copy(*a); });
+        return true;
+      }
+      read = [a] { return data::get(*a); };
+    } else if (is_vector(from)) {
+      const std::vector<T>* a = sm.getVector(node.inputs[0], T());
+      read = [a] { return *a; };
+    } else if (is_value(from)) {
+      const T* a = sm.getValue(node.inputs[0], T());
+      read = [a] { return std::vector<T>(1, *a); };
+    } else {
+      return false;
+    }
+    if (TO == Target::TENSOR) {
+      Variable<T>* out = sm.getVariable(node.outputs[0], T());
+      graph.addStep([read, out] {
+        std::vector<T> v = read();
+        const unsigned n = static_cast<unsigned>(v.size());
+        *out = data::set(std::move(v), Shape({n}));
+      });
+    } else if (TO == Target::VALUE) {
+      T* out = sm.getValue(node.outputs[0], T());
+      const bool single = is_value(from);
+      graph.addStep([read, out, a = is_tensor(from) ? sm.getTensor(node.inputs[0], T()) : nullptr, single] {
+        if (a != nullptr && a->size() != 1) throw RuntimeError("ToValue: invalid size of input");
+        std::vector<T> v = read();
+        if (!single && v.size() != 1) throw RuntimeError("ToValue: invalid size of input");
+        *out = v[0];
+      });
+    } else {
+      std::vector<T>* out = sm.getVector(node.outputs[0], T());
+      graph.addStep([read, out] { *out = read(); });
+    }
+    return true;
+  }
+};
+
 // ---- base.Identity -----------------------------------------------------------------------------------------------
 template <class T>
 class Identity : public TypedOperation<T> {
@@ -763,9 +874,14 @@ class Collector {
     add(new Gather<T, int64_t>());
     add(new Gather<T, uint64_t>());
     add(new Concat<T>());
+    add(new At1<T>());
+    add(new Convert<Target::TENSOR, T>());
+    add(new Convert<Target::VALUE, T>());
+    add(new Convert<Target::VECTOR, T>());
 #define TFCC_RUNTIME_ADD_PAIR(OTHER, E) \
   add(new Cast<T, OTHER>());            \
-  add(new SliceV1<T, OTHER>());
+  add(new SliceV1<T, OTHER>());         \
+  add(new At<T, OTHER>());
     TFCC_RUNTIME_FOR_ALL_TYPES(TFCC_RUNTIME_ADD_PAIR)
 #undef TFCC_RUNTIME_ADD_PAIR
 #define TFCC_RUNTIME_ADD_DIMENSION(DST, E) add(new GetDimension<T, DST>());
