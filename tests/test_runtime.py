@@ -637,6 +637,49 @@ def test_embeddings_mask_and_answer_head_around_a_product(mf, rt, dev):
     assert int(res[count][0]) == 2 * seq and float(res[as_float][0]) == 2.0 * seq
 
 
+@pytest.mark.gpu
+def test_split_stack_slice_pad_nodes_equal_numpy(mf, rt, dev):
+    """base.Split (as many equal parts as outputs), base.Stack, base.SliceV2 (negative positions count from the end,
+    the end is clipped) and base.Pad: tfcc_runtime/operations/base/split.cpp, stack.cpp, slicev2.cpp, pad.cpp."""
+    rng = np.random.default_rng(31)
+    a = rng.normal(size=(2, 6, 4)).astype(np.float32)
+    g = mf.GraphBuilder("g")
+    x = g.input("x", mf.FLOAT, [2, 6, 4])
+    parts = [g.variable("part") for _ in range(3)]
+    g.node("base.Split", [x], parts, mf.f_varint(1, 1))
+    stacked = g.variable("stacked")
+    g.node("base.Stack", parts, [stacked])                      # axis 0: the field is not written
+    stacked2 = g.variable("stacked2")
+    g.node("base.Stack", parts, [stacked2], mf.f_varint(1, 3))
+    value = lambda name, v, dt=np.int64: g.constant(name, np.array(v, dt), mf.CONSTANT_VALUE)  # noqa: E731
+    tail = g.variable("tail")
+    g.node("base.SliceV2", [x, value("s1", -4), value("e1", -1)], [tail], mf.f_varint(1, 1))
+    clipped = g.variable("clipped")
+    g.node("base.SliceV2", [x, value("s2", 1, np.uint32), value("e2", 100, np.uint32)], [clipped], mf.f_varint(1, 2))
+    padded = g.variable("padded")
+    g.node("base.Pad", [x, value("h", 1, np.int32), value("t", 2, np.int32)], [padded], mf.f_varint(1, 2))
+    padded0 = g.variable("padded0")
+    g.node("base.Pad", [x, value("h0", 0), value("t0", 3)], [padded0])
+    for o in parts + [stacked, stacked2, tail, clipped, padded, padded0]:
+        g.output(o)
+    res = rt.Model(mf.write_model([g], "g")).run({"x": a})
+    want_parts = np.split(a, 3, axis=1)
+    for o, w in zip(parts, want_parts):
+        assert np.array_equal(res[o], w)
+    assert np.array_equal(res[stacked], np.stack(want_parts, 0)) and np.array_equal(res[stacked2], np.stack(want_parts, 3))
+    assert np.array_equal(res[tail], a[:, 2:5]) and np.array_equal(res[clipped], a[:, :, 1:])
+    assert np.array_equal(res[padded], np.pad(a, ((0, 0), (0, 0), (1, 2))))
+    assert np.array_equal(res[padded0], np.pad(a, ((0, 3), (0, 0), (0, 0))))
+    # five parts do not divide six rows
+    g = mf.GraphBuilder("g")
+    x = g.input("x", mf.FLOAT, [2, 6, 4])
+    outs = [g.variable("p") for _ in range(5)]
+    g.node("base.Split", [x], outs, mf.f_varint(1, 1))
+    g.output(outs[0])
+    with pytest.raises(rt.RuntimeError_, match="invalid num"):
+        rt.Model(mf.write_model([g], "g")).run({"x": a})
+
+
 def test_data_movement_nodes_accept_rules(mf, rt):
     """nn.Gather wants 32- or 64-bit integer indices, base.Cast a result symbol of the type its message names,
     base.SliceV1 an integer position value: anything else is a node nobody takes

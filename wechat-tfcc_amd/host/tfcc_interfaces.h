@@ -500,6 +500,57 @@ template <class T>
 Variable<T> concat(std::initializer_list<const Tensor<T>*> values, size_t axis) {
   return concat(std::vector<const Tensor<T>*>(values), axis);
 }
+// tfcc/core/operations/tfcc_base.cpp:43-59: num equal parts along axis
+template <class T>
+std::vector<Variable<T>> split(const Tensor<T>& a, size_t num, size_t axis) {
+  if (axis >= a.shape().size()) throw InvalidArgumentError("invalid axis");
+  if (num == 0 || a.shape(axis) % num != 0) throw InvalidArgumentError("invalid num");
+  const unsigned s = a.shape(axis) / static_cast<unsigned>(num);
+  std::vector<Variable<T>> values;
+  BasicInterface<T>& basic = Operation<T>::getCurrentInterface().getBasicInterface();
+  for (size_t i = 0; i < num; ++i)
+    values.emplace_back(basic.slice(a, axis, static_cast<unsigned>(i) * s, static_cast<unsigned>(i + 1) * s));
+  return values;
+}
+// tfcc/core/operations/tfcc_base.cpp:184-210: values of one shape joined along a new dimension at axis
+template <class T>
+Variable<T> stack(const std::vector<const Tensor<T>*>& values, size_t axis) {
+  if (values.size() == 0) throw InvalidArgumentError("values's size should be greater than zero");
+  if (axis > values[0]->shape().size()) throw InvalidArgumentError("invalid axis");
+  std::vector<unsigned> s = values[0]->shape().toVector();
+  s.insert(s.begin() + axis, 1);
+  std::vector<View<T>> views;
+  for (const Tensor<T>* tensor : values) {
+    if (tensor->shape() != values[0]->shape()) throw InvalidArgumentError("the shape of values are unequal");
+    views.emplace_back(*tensor, Shape(s));
+  }
+  std::vector<const Tensor<T>*> tensors;
+  for (View<T>& view : views) tensors.push_back(&view);
+  return concat(tensors, axis);
+}
+// tfcc/core/operations/tfcc_base.cpp:136-160: zeros in front of and behind a along axis
+template <class T>
+Variable<T> pad(const Tensor<T>& a, size_t axis, unsigned paddingHead, unsigned paddingEnd) {
+  if (axis >= a.shape().size()) throw InvalidArgumentError("invalid axis");
+  std::vector<unsigned> s = a.shape().toVector();
+  Variable<T> head, tail;
+  std::vector<const Tensor<T>*> parts;
+  DataInterface<T>& dataInterface = Operation<T>::getCurrentInterface().getDataInterface();
+  if (paddingHead > 0) {
+    s[axis] = paddingHead;
+    head = Variable<T>(Shape(s));
+    dataInterface.zeros(head);
+    parts.push_back(&head);
+  }
+  parts.push_back(&a);
+  if (paddingEnd > 0) {
+    s[axis] = paddingEnd;
+    tail = Variable<T>(Shape(s));
+    dataInterface.zeros(tail);
+    parts.push_back(&tail);
+  }
+  return concat(parts, axis);
+}
 }  // namespace base
 
 namespace nn {

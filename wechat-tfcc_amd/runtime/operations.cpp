@@ -14,6 +14,7 @@
 //   base.GetShape, base.GetDimension    operations/base/getshape.cpp, getdimension.cpp
 //   base.At / At1 / ToTensor / ToValue / ToVector
 //                                       operations/base/at.cpp, at1.cpp, totensor.cpp, tovalue.cpp, tovector.cpp
+//   base.Split / Stack / SliceV2 / Pad  operations/base/split.cpp, stack.cpp, slicev2.cpp, pad.cpp
 //   nn.Gather, base.Cast, base.SliceV1, base.Concat
 //                                       operations/nn/gather.cpp, base/cast.cpp, slicev1.cpp, concat.cpp
 //   base.Transpose, base.Reshape, base.Identity, base.CreateVector
@@ -561,6 +562,117 @@ class Concat : public TypedOperation<T> {
   }
 };
 
+// ---- base.Split / Stack / SliceV2 / Pad ------------------------------------------------------------------------------
+// tfcc_runtime/operations/base/split.cpp:27-87 (as many equal parts as the node has outputs), stack.cpp:27-87,
+// slicev2.cpp:27-121 (start and end from value symbols, negative ones count from the end), pad.cpp:27-91
+template <class T>
+class Split : public TypedOperation<T> {
+ public:
+  Split() : TypedOperation<T>("base.Split") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 1 || node.outputs.empty()) return false;
+    if (!same_dtype(graph, node.outputs, this->DTYPE) || !same_dtype(graph, node.inputs, this->DTYPE)) return false;
+    const uint64_t axis = first_varint(node);
+    auto& sm = graph.getSymbolManager();
+    const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+    std::vector<Variable<T>*> outs;
+    for (const std::string& name : node.outputs) outs.push_back(sm.getVariable(name, T()));
+    graph.addStep([a, axis, outs] {
+      std::vector<Variable<T>> parts = base::split(*a, outs.size(), static_cast<size_t>(axis));
+      for (size_t i = 0; i < outs.size(); ++i) *outs[i] = std::move(parts[i]);
+    });
+    return true;
+  }
+
+  static uint64_t first_varint(const proto::Node& node) {
+    uint64_t v = 0;
+    wire::Reader r(node.operation);
+    uint32_t f, t;
+    while (r.next(f, t)) {
+      if (f == 1 && t == 0) v = r.varint();
+      else r.skip(t);
+    }
+    return v;
+  }
+};
+
+template <class T>
+class Stack : public TypedOperation<T> {
+ public:
+  Stack() : TypedOperation<T>("base.Stack") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.empty() || node.outputs.size() != 1) return false;
+    if (!same_dtype(graph, node.outputs, this->DTYPE) || !same_dtype(graph, node.inputs, this->DTYPE)) return false;
+    const uint64_t axis = Split<T>::first_varint(node);
+    auto& sm = graph.getSymbolManager();
+    std::vector<const Tensor<T>*> values;
+    for (const std::string& name : node.inputs) values.push_back(sm.getTensor(name, T()));
+    Variable<T>* out = sm.getVariable(node.outputs[0], T());
+    graph.addStep([values, axis, out] { *out = base::stack(values, static_cast<size_t>(axis)); });
+    return true;
+  }
+};
+
+template <class T, class POS>
+class SliceV2 : public TypedOperation<T> {
+ public:
+  SliceV2() : TypedOperation<T>("base.SliceV2") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (!std::is_integral<POS>::value) return false;
+    if (node.inputs.size() != 3 || node.outputs.size() != 1) return false;
+    auto& sm = graph.getSymbolManager();
+    if (sm.getSymbolInfo(node.outputs[0]).dtype != this->DTYPE || sm.getSymbolInfo(node.inputs[0]).dtype != this->DTYPE)
+      return false;
+    if (sm.getSymbolInfo(node.inputs[1]).dtype != DataTypeOf<POS>::value ||
+        sm.getSymbolInfo(node.inputs[2]).dtype != DataTypeOf<POS>::value)
+      return false;
+    const uint64_t axis = Split<T>::first_varint(node);
+    const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+    const POS* start = sm.getValue(node.inputs[1], POS());
+    const POS* end = sm.getValue(node.inputs[2], POS());
+    Variable<T>* out = sm.getVariable(node.outputs[0], T());
+    graph.addStep([a, start, end, axis, out] {
+      if (axis >= a->shape().size()) throw RuntimeError("SliceV2: invalid axis");
+      long long s = static_cast<long long>(*start), e = static_cast<long long>(*end);
+      const long long extent = a->shape(static_cast<size_t>(axis));
+      if (std::is_signed<POS>::value && extent > 0) {
+        while (s < 0) s += extent;
+        while (e < 0) e += extent;
+      }
+      if (s < 0 || e < 0) throw RuntimeError("SliceV2: invalid position");
+      const unsigned limit = ~0u;
+      *out = base::slice(*a, static_cast<size_t>(axis), static_cast<unsigned>(std::min<long long>(s, limit)),
+                         static_cast<unsigned>(std::min<long long>(e, limit)));
+    });
+    return true;
+  }
+};
+
+template <class T, class IDX>
+class Pad : public TypedOperation<T> {
+ public:
+  Pad() : TypedOperation<T>("base.Pad") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (!std::is_integral<IDX>::value) return false;
+    if (node.inputs.size() != 3 || node.outputs.size() != 1) return false;
+    auto& sm = graph.getSymbolManager();
+    if (sm.getSymbolInfo(node.outputs[0]).dtype != this->DTYPE || sm.getSymbolInfo(node.inputs[0]).dtype != this->DTYPE)
+      return false;
+    if (sm.getSymbolInfo(node.inputs[1]).dtype != DataTypeOf<IDX>::value ||
+        sm.getSymbolInfo(node.inputs[2]).dtype != DataTypeOf<IDX>::value)
+      return false;
+    const uint64_t axis = Split<T>::first_varint(node);
+    const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+    const IDX* head = sm.getValue(node.inputs[1], IDX());
+    const IDX* tail = sm.getValue(node.inputs[2], IDX());
+    Variable<T>* out = sm.getVariable(node.outputs[0], T());
+    graph.addStep([a, head, tail, axis, out] {
+      *out = base::pad(*a, static_cast<size_t>(axis), static_cast<unsigned>(*head), static_cast<unsigned>(*tail));
+    });
+    return true;
+  }
+};
+
 // ---- base.At / At1 / ToTensor / ToValue / ToVector: between the three kinds of symbols ---------------------------
 // tfcc_runtime/operations/base/at.cpp:27-82, at1.cpp:27-75, totensor.cpp:27-116, tovalue.cpp:27-109,
 // tovector.cpp:27-110.  Reading a tensor into a value or a vector waits for the device.
@@ -875,13 +987,17 @@ class Collector {
     add(new Gather<T, uint64_t>());
     add(new Concat<T>());
     add(new At1<T>());
+    add(new Split<T>());
+    add(new Stack<T>());
     add(new Convert<Target::TENSOR, T>());
     add(new Convert<Target::VALUE, T>());
     add(new Convert<Target::VECTOR, T>());
 #define TFCC_RUNTIME_ADD_PAIR(OTHER, E) \
   add(new Cast<T, OTHER>());            \
   add(new SliceV1<T, OTHER>());         \
-  add(new At<T, OTHER>());
+  add(new At<T, OTHER>());              \
+  add(new SliceV2<T, OTHER>());         \
+  add(new Pad<T, OTHER>());
     TFCC_RUNTIME_FOR_ALL_TYPES(TFCC_RUNTIME_ADD_PAIR)
 #undef TFCC_RUNTIME_ADD_PAIR
 #define TFCC_RUNTIME_ADD_DIMENSION(DST, E) add(new GetDimension<T, DST>());
