@@ -328,10 +328,21 @@ int tfcc_rocm_add_f32(void* stream, const float* a, const float* b, uint64_t tot
 /* out = a / alpha + beta: TransformationInterface::transform2 (a / s in tfcc_operator.cpp:78-95) */
 int tfcc_rocm_transform2_f32(void* stream, const float* in, uint64_t total, float alpha, float beta,
                              float* out);
-/* op: 0 a + b, 1 a - b, 2 a * b, 3 a / b with the same trailing-dims broadcast of b as add:
- * ArithmeticInterface::add/sub/mul/div, tfcc/core/interfaces/tfcc_arithmeticinterface.h:34-79 */
+/* op: 0 a + b, 1 a - b, 2 a * b, 3 a / b, 4 pow(a, b), 5 max(a, b), 6 min(a, b) with the same trailing-dims
+ * broadcast of b as add: ArithmeticInterface::add/sub/mul/div, tfcc/core/interfaces/tfcc_arithmeticinterface.h:34-79;
+ * tfcc::math::pow / max / min */
 int tfcc_rocm_binary_f32(void* stream, int op, const float* a, const float* b, uint64_t total,
                          uint64_t period, float* out);
+/* Reductions over the trailing dimensions, rows x cols -> rows (ReduceInterface::reduceSum / reduceMean / reduceProd /
+ * reduceMax / reduceMin, tfcc/mkl/interfaces/tfcc_mklreduceinterface.cpp:107-230). */
+enum {
+  TFCC_ROCM_REDUCE_SUM = 0, TFCC_ROCM_REDUCE_MEAN = 1, TFCC_ROCM_REDUCE_PROD = 2, TFCC_ROCM_REDUCE_MAX = 3,
+  TFCC_ROCM_REDUCE_MIN = 4
+};
+int tfcc_rocm_reduce_f32(void* stream, int op, const float* in, uint64_t rows, unsigned cols, float* out);
+/* min(max(v, lo), hi) (tfcc::math::clip) and v > 0 ? v : v * alpha (tfcc::math::leaky_relu) */
+int tfcc_rocm_clip_f32(void* stream, const float* in, uint64_t total, float lo, float hi, float* out);
+int tfcc_rocm_leaky_relu_f32(void* stream, const float* in, uint64_t total, float alpha, float* out);
 /* out = a op b with numpy-style broadcasting: dims[rank] is the result's shape, stride_a / stride_b the element strides
  * of each operand per result dimension (0 where the operand's extent is 1).  rank <= 6; callers merge adjacent
  * dimensions of the same kind first, as tfcc::math::add does (tfcc/core/operations/tfcc_math.cpp:38-104). */

@@ -772,6 +772,61 @@ static void test_dense_from_constants() {
   CHECK_THROWS_MSG(tfcc::layer::dense(wrong, 0u, true), tfcc::InvalidArgumentError, "inputs and kernel don't match");
 }
 
+// tfcc::math::reduce_sum / mean / prod / max / min, min / max / pow of tensors and values, clip, leaky_relu
+// (tfcc/test/math.cpp's reduce and min / max cases): results against the same expressions in double on the host.
+static void test_reduce_minmax_pow() {
+  std::mt19937 rng(23);
+  std::uniform_real_distribution<float> dist(0.6f, 1.4f);
+  const unsigned d0 = 3, d1 = 5, d2 = 37;
+  std::vector<float> ha(d0 * d1 * d2), hb(d2);
+  for (size_t i = 0; i < ha.size(); ++i) ha[i] = (i % 3 == 1 ? -1.f : 1.f) * dist(rng);
+  for (auto& v : hb) v = dist(rng);
+  tfcc::Variable<float> a = tfcc::data::set(ha, {d0, d1, d2}), b = tfcc::data::set(hb, {d2});
+  for (size_t keep : {size_t(1), size_t(2)}) {
+    const size_t rows = keep == 1 ? d0 : d0 * d1, cols = ha.size() / rows;
+    tfcc::Variable<float> sum = tfcc::math::reduce_sum(a, keep), mean = tfcc::math::reduce_mean(a, keep),
+                          prod = tfcc::math::reduce_prod(a, keep), hi = tfcc::math::reduce_max(a, keep),
+                          lo = tfcc::math::reduce_min(a, keep);
+    CHECK(sum.shape() == (keep == 1 ? tfcc::Shape({d0, 1, 1}) : tfcc::Shape({d0, d1, 1})));
+    std::vector<float> gs = tfcc::data::get(sum), gm = tfcc::data::get(mean), gp = tfcc::data::get(prod),
+                       gh = tfcc::data::get(hi), gl = tfcc::data::get(lo);
+    bool ok = gs.size() == rows;
+    for (size_t r = 0; ok && r < rows; ++r) {
+      double s = 0, p = 1;
+      float mx = ha[r * cols], mn = ha[r * cols];
+      for (size_t c = 0; c < cols; ++c) {
+        const float v = ha[r * cols + c];
+        s += v;
+        p *= v;
+        mx = std::max(mx, v);
+        mn = std::min(mn, v);
+      }
+      ok = std::fabs(gs[r] - s) < 1e-4 && std::fabs(gm[r] - s / cols) < 1e-5 &&
+           std::fabs(gp[r] - p) <= 1e-4 * std::fabs(p) && gh[r] == mx && gl[r] == mn;
+    }
+    CHECK(ok);
+  }
+  CHECK_THROWS_MSG(tfcc::math::reduce_sum(a, 3), tfcc::InvalidArgumentError, "invalid keep dims");
+  std::vector<float> gmin = tfcc::data::get(tfcc::math::min(a, b)), gmax = tfcc::data::get(tfcc::math::max(b, a)),
+                     gminv = tfcc::data::get(tfcc::math::min(a, 0.25f)), gmaxv = tfcc::data::get(tfcc::math::max(0.25f, a)),
+                     gclip = tfcc::data::get(tfcc::math::clip(a, -0.75f, 1.f)),
+                     gleak = tfcc::data::get(tfcc::math::leaky_relu(a, 0.1f));
+  tfcc::Variable<float> mag = tfcc::math::abs(a);
+  std::vector<float> gpow = tfcc::data::get(tfcc::math::pow(mag, b)), gpowv = tfcc::data::get(tfcc::math::pow(mag, 2.5f)),
+                     gvpow = tfcc::data::get(tfcc::math::pow(1.5f, a));
+  bool ok = gmin.size() == ha.size() && gpow.size() == ha.size() && gvpow.size() == ha.size();
+  for (size_t i = 0; ok && i < ha.size(); ++i) {
+    const float x = ha[i], y = hb[i % d2];
+    ok = gmin[i] == std::min(x, y) && gmax[i] == std::max(x, y) && gminv[i] == std::min(x, 0.25f) &&
+         gmaxv[i] == std::max(x, 0.25f) && gclip[i] == std::min(std::max(x, -0.75f), 1.f) &&
+         gleak[i] == (x > 0.f ? x : x * 0.1f) &&
+         std::fabs(gpow[i] - std::pow(std::fabs((double)x), (double)y)) < 2e-6 * std::pow(std::fabs((double)x), (double)y) + 1e-7 &&
+         std::fabs(gpowv[i] - std::pow(std::fabs((double)x), 2.5)) < 2e-6 * std::pow(std::fabs((double)x), 2.5) + 1e-7 &&
+         std::fabs(gvpow[i] - std::pow(1.5, (double)x)) < 2e-6 * std::pow(1.5, (double)x) + 1e-7;
+  }
+  CHECK(ok);
+}
+
 // tfcc::math::add / sub / mul / div with the broadcasting of tfcc/core/operations/tfcc_math.cpp:38-104
 // (tfcc/test/math.cpp's broadcast cases): attention mask, both sides broadcast, either operand the larger.
 static void test_broadcast_arithmetic() {
@@ -933,6 +988,7 @@ int main(int argc, char** argv) {
     run("quantization.rocm_matmul_exact", test_quantized_matmul_exact);
     run("layer.elementwise", test_layer_ops);
     run("math.broadcast_arithmetic", test_broadcast_arithmetic);
+    run("math.reduce_minmax_pow", test_reduce_minmax_pow);
     run("layer.attention_permuted", test_attention_permuted);
     run("base.data_movement", test_data_movement);
     run("rnn.cells", test_cells);

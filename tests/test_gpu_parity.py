@@ -585,6 +585,39 @@ def test_gather_slice_concat_cast_equal_numpy(pkg, T):
         assert np.array_equal(T.n(pkg.cast(T.t(src), dtype)), src.astype(np_dtype))
 
 
+def test_reductions_pow_max_min_clip_leaky_relu(pkg, T):
+    """Reductions over the trailing dimensions (tfcc/mkl/interfaces/tfcc_mklreduceinterface.cpp:107-230) against numpy
+    float64 (sum, mean, product) and exactly (maximum, minimum); rows shorter and longer than a wavefront's and a
+    workgroup's share; pow / max / min of two tensors, clip and leaky relu of one."""
+    rng = np.random.default_rng(41)
+    for shape, keep in (((7, 33), 1), ((3, 5, 64), 1), ((2, 3, 4100), 2), ((5, 9000), 1), ((4, 1), 1), ((6, 2, 3), 0)):
+        x = rng.uniform(0.5, 1.5, shape).astype(np.float32) * rng.choice([-1.0, 1.0], shape).astype(np.float32)
+        axes = tuple(range(keep, len(shape)))
+        x64 = x.astype(np.float64)
+        for op, ref in (("sum", np.sum), ("mean", np.mean), ("max", np.max), ("min", np.min)):
+            got = T.n(pkg.reduce_trailing(op, T.t(x), keep))
+            want = ref(x64, axis=axes, keepdims=True)
+            assert got.shape == want.shape
+            if op in ("max", "min"):
+                assert np.array_equal(got, want.astype(np.float32))
+            else:
+                assert np.allclose(got, want, rtol=1e-5, atol=1e-4), (op, shape)
+        small = rng.uniform(0.9, 1.1, shape).astype(np.float32)
+        got = T.n(pkg.reduce_trailing("prod", T.t(small), keep))
+        assert np.allclose(got, np.prod(small.astype(np.float64), axis=axes, keepdims=True), rtol=1e-4)
+    with pytest.raises(pkg.InvalidArgumentError, match="invalid keep dims"):
+        pkg.reduce_trailing("sum", T.t(np.zeros((2, 3), np.float32)), 2)
+    a = rng.uniform(0.1, 3, (5, 7, 33)).astype(np.float32)
+    b = rng.uniform(-2, 2, (5, 7, 33)).astype(np.float32)
+    row = rng.uniform(-2, 2, 33).astype(np.float32)
+    assert np.allclose(T.n(pkg.binary("pow", T.t(a), T.t(b))), np.power(a.astype(np.float64), b), rtol=2e-6)
+    assert np.allclose(T.n(pkg.binary("pow", T.t(a), T.t(row))), np.power(a.astype(np.float64), row), rtol=2e-6)
+    assert np.array_equal(T.n(pkg.binary("max", T.t(b), T.t(row))), np.maximum(b, row))
+    assert np.array_equal(T.n(pkg.binary("min", T.t(b), T.t(a))), np.minimum(b, a))
+    assert np.array_equal(T.n(pkg.clip(T.t(b), -0.5, 1.25)), np.clip(b, np.float32(-0.5), np.float32(1.25)))
+    assert np.array_equal(T.n(pkg.leaky_relu(T.t(b), 0.1)), np.where(b > 0, b, b * np.float32(0.1)))
+
+
 BROADCAST_PAIRS = [
     ((2, 4, 8, 8), (2, 1, 1, 8)),        # attention scores + mask
     ((3, 1, 5), (1, 4, 1)),              # both sides broadcast

@@ -218,13 +218,14 @@ def test_value_arithmetic_and_vectors_on_host(mf, rt):
     a = g.value_input("a", mf.FLOAT)
     b = g.value_input("b", mf.FLOAT)
     results = {}
-    for op in ("Add", "Sub", "Mul", "Div"):
+    ops = ("Add", "Sub", "Mul", "Div", "Pow", "Max", "Min")
+    for op in ops:
         out = g._symbol("r_" + op, mf.FLOAT, mf.VALUE)
         g.node("math." + op, [a, b], [out])
         g.output(out)
     m = rt.Model(mf.write_model([g], "g"), host=True)
     res = m.run({"a": np.array([6.0], np.float32), "b": np.array([1.5], np.float32)})
-    assert [float(res["r_" + op][0]) for op in ("Add", "Sub", "Mul", "Div")] == [7.5, 4.5, 9.0, 4.0]
+    assert [float(res["r_" + op][0]) for op in ops] == [7.5, 4.5, 9.0, 4.0, np.float32(6.0 ** 1.5), 6.0, 1.5]
 
 
 def test_archive_and_graph_errors(mf, rt):
@@ -635,6 +636,57 @@ def test_embeddings_mask_and_answer_head_around_a_product(mf, rt, dev):
     assert res[joined].shape == (batch, 2 * seq)
     assert np.array_equal(res[joined], np.concatenate([res[parts[0]], res[parts[1]]], axis=1))
     assert int(res[count][0]) == 2 * seq and float(res[as_float][0]) == 2.0 * seq
+
+
+@pytest.mark.gpu
+def test_reduce_pow_max_min_clip_leaky_relu_nodes_equal_numpy(mf, rt, dev):
+    """math.ReduceSum / Mean / Prod / Max / Min over trailing, leading and scattered axes (the node moves them behind the
+    others first: tfcc_runtime/utils/reduceutils.h:25-50), math.Pow / Max / Min with tensor and value operands,
+    math.Clip with two values and math.LeakyRelu with alpha in the node."""
+    rng = np.random.default_rng(43)
+    a = (rng.uniform(0.6, 1.4, (3, 4, 5, 6)) * rng.choice([-1.0, 1.0], (3, 4, 5, 6))).astype(np.float32)
+    b = rng.uniform(0.5, 2.0, (5, 6)).astype(np.float32)
+    g = mf.GraphBuilder("g")
+    x = g.input("x", mf.FLOAT, [3, 4, 5, 6])
+    y = g.input("y", mf.FLOAT, [5, 6])
+    wants = {}
+    for name, ref in (("Sum", np.sum), ("Mean", np.mean), ("Prod", np.prod), ("Max", np.max), ("Min", np.min)):
+        for axes in ((3,), (2, 3), (0,), (1, 3), (3, 1), (0, 1, 2, 3)[:3]):
+            out = g.variable("r")
+            g.node("math.Reduce" + name, [x], [out], mf.f_packed(1, list(axes)))
+            g.output(out)
+            wants[out] = ref(a.astype(np.float64), axis=tuple(axes), keepdims=True)
+    value = lambda name, v: g.constant(name, np.array(v, np.float32), mf.CONSTANT_VALUE)  # noqa: E731
+    absx = g.unary("math.Abs", x)
+    for op, ref in (("Pow", np.power), ("Max", np.maximum), ("Min", np.minimum)):
+        first = absx if op == "Pow" else x
+        first_np = np.abs(a) if op == "Pow" else a
+        for second, second_np in ((y, b), (value("v" + op, 1.5), np.float32(1.5))):
+            out = g.binary(op, first, second)
+            g.output(out)
+            wants[out] = ref(first_np.astype(np.float64), second_np)
+        out = g.binary(op, value("w" + op, 1.25), y)
+        g.output(out)
+        wants[out] = ref(np.float64(1.25), b)
+    clipped = g.variable("clipped")
+    g.node("math.Clip", [x, value("lo", -0.75), value("hi", 1.0)], [clipped])
+    g.output(clipped)
+    wants[clipped] = np.clip(a, -0.75, 1.0)
+    leaky = g.unary("math.LeakyRelu", x, mf.f_bytes(1, mf.value_message(0.2)))
+    g.output(leaky)
+    wants[leaky] = np.where(a > 0, a, a * np.float32(0.2))
+    res = rt.Model(mf.write_model([g], "g")).run({"x": a, "y": b})
+    for name, want in wants.items():
+        assert res[name].shape == np.shape(want), name
+        assert np.allclose(res[name], want, rtol=2e-5, atol=1e-6), name
+    # an axis beyond the rank is an error of the step
+    g = mf.GraphBuilder("g")
+    x = g.input("x", mf.FLOAT, [3, 4])
+    out = g.variable("r")
+    g.node("math.ReduceSum", [x], [out], mf.f_packed(1, [2]))
+    g.output(out)
+    with pytest.raises(rt.RuntimeError_, match="invalid axis"):
+        rt.Model(mf.write_model([g], "g")).run({"x": np.zeros((3, 4), np.float32)})
 
 
 @pytest.mark.gpu

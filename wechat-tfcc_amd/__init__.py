@@ -130,6 +130,9 @@ SYMBOLS = {
     "tfcc_rocm_binary_broadcast_f32": (_I, [_VP, _I, _VP, _VP, _I, C.POINTER(C.c_uint), C.POINTER(_U64),
                                            C.POINTER(_U64), _VP]),
     "tfcc_rocm_lstm_cell_f32": (_I, [_VP, _U, _U, _VP, _VP, _VP, _VP, _F, _VP, _VP]),
+    "tfcc_rocm_reduce_f32": (_I, [_VP, _I, _VP, _U64, _U, _VP]),
+    "tfcc_rocm_clip_f32": (_I, [_VP, _VP, _U64, _F, _F, _VP]),
+    "tfcc_rocm_leaky_relu_f32": (_I, [_VP, _VP, _U64, _F, _VP]),
     "tfcc_rocm_copy2d": (_I, [_VP, _VP, _U64, _VP, _U64, _U64, _U64]),
     "tfcc_rocm_gather_rows": (_I, [_VP, _VP, _U, _U64, _VP, _I, _U64, _VP]),
     "tfcc_rocm_cast": (_I, [_VP, _VP, _I, _VP, _I, _U64]),
@@ -650,7 +653,7 @@ def transform2(a, alpha, beta):
     return out
 
 
-BINARY_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3}
+BINARY_OPS = {"add": 0, "sub": 1, "mul": 2, "div": 3, "pow": 4, "max": 5, "min": 6}
 
 
 def binary(op, a, b):
@@ -746,6 +749,42 @@ def concat(values, axis):
     return out
 
 
+REDUCE_OPS = {"sum": 0, "mean": 1, "prod": 2, "max": 3, "min": 4}
+
+
+def reduce_trailing(op, a, keep):
+    """tfcc::math::reduce_sum / reduce_mean / reduce_prod / reduce_max / reduce_min (tfcc/core/operations/
+    tfcc_math.cpp:464-520): the dimensions from `keep` on are reduced and stay in the shape as 1."""
+    import torch
+    if a.numel() == 0:
+        raise InvalidArgumentError("invalid tensor")
+    if keep >= a.dim():
+        raise InvalidArgumentError("invalid keep dims")
+    a = a.contiguous()
+    cols = 1
+    for d in a.shape[keep:]:
+        cols *= d
+    out = torch.empty(tuple(a.shape[:keep]) + (1,) * (a.dim() - keep), dtype=torch.float32, device=a.device)
+    check(lib().tfcc_rocm_reduce_f32(_stream(), REDUCE_OPS[op], _ptr(a), a.numel() // cols, cols, _ptr(out)))
+    return out
+
+
+def clip(a, lo, hi):
+    import torch
+    a = a.contiguous()
+    out = torch.empty_like(a)
+    check(lib().tfcc_rocm_clip_f32(_stream(), _ptr(a), a.numel(), lo, hi, _ptr(out)))
+    return out
+
+
+def leaky_relu(a, alpha):
+    import torch
+    a = a.contiguous()
+    out = torch.empty_like(a)
+    check(lib().tfcc_rocm_leaky_relu_f32(_stream(), _ptr(a), a.numel(), alpha, _ptr(out)))
+    return out
+
+
 def broadcast_shapes(s1, s2):
     """_get_broadcast_shape of tfcc/core/operations/tfcc_math.cpp:38-86: (result shape, collapsed s1, collapsed s2).
     Right-aligned; extents must be equal or 1; runs of dimensions of the same kind are merged."""
@@ -779,7 +818,7 @@ def broadcast_shapes(s1, s2):
 
 
 def math_binary(op, a, b):
-    """tfcc::math::add / sub / mul / div (op in BINARY_OPS) with the reference's broadcasting."""
+    """tfcc::math::add / sub / mul / div / pow / max / min (op in BINARY_OPS) with the reference's broadcasting."""
     import torch
     shape, ca, cb = broadcast_shapes(a.shape, b.shape)
     out = torch.empty(shape, dtype=torch.float32, device=a.device)

@@ -180,6 +180,62 @@ __global__ __launch_bounds__(256) void binary_kernel(const float* a, const float
   }
 }
 
+// Reductions over the trailing dimensions (rows x cols -> rows): sum, mean, product, maximum, minimum
+// (tfcc/mkl/interfaces/tfcc_mklreduceinterface.cpp:107-230).  A wavefront per row up to 4096 columns, a workgroup
+// per row beyond; partial results meet through lane shuffles (and LDS), in a fixed order.
+template <int OP>
+__device__ __forceinline__ float reduce_identity() {
+  return OP == TFCC_ROCM_REDUCE_PROD ? 1.f : OP == TFCC_ROCM_REDUCE_MAX ? -INFINITY : OP == TFCC_ROCM_REDUCE_MIN ? INFINITY : 0.f;
+}
+template <int OP>
+__device__ __forceinline__ float reduce_join(float a, float b) {
+  return OP == TFCC_ROCM_REDUCE_PROD ? a * b : OP == TFCC_ROCM_REDUCE_MAX ? fmaxf(a, b) : OP == TFCC_ROCM_REDUCE_MIN ? fminf(a, b) : a + b;
+}
+template <int OP>
+__device__ __forceinline__ float wave_join(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = reduce_join<OP>(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+template <int OP, bool BLOCK>
+__global__ __launch_bounds__(256) void reduce_trailing_kernel(const float* in, size_t rows, unsigned cols, float* out) {
+  __shared__ float sh[4];
+  const unsigned lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const size_t row = BLOCK ? blockIdx.x : (size_t)blockIdx.x * 4 + wave;
+  if (!BLOCK && row >= rows) return;
+  const float* a = in + row * cols;
+  float v = reduce_identity<OP>();
+  for (unsigned i = BLOCK ? threadIdx.x : lane; i < cols; i += BLOCK ? 256 : 64) v = reduce_join<OP>(v, a[i]);
+  v = wave_join<OP>(v);
+  if (BLOCK) {
+    if (lane == 0) sh[wave] = v;
+    __syncthreads();
+    v = reduce_join<OP>(reduce_join<OP>(sh[0], sh[1]), reduce_join<OP>(sh[2], sh[3]));
+  }
+  if (OP == TFCC_ROCM_REDUCE_MEAN) v = v / (float)cols;
+  if (BLOCK ? threadIdx.x == 0 : lane == 0) out[row] = v;
+}
+
+// More element-wise functions of two tensors of one shape (op 4 pow, 5 max, 6 min) and of one tensor with scalars
+// (clip to [lo, hi]; leaky relu v > 0 ? v : v * alpha): tfcc/mkl/kernel/tfcc_mklactivationkernel.hpp, tfcc_math.h.
+template <int OP>
+__global__ __launch_bounds__(256) void binary2_kernel(const float* a, const float* b, size_t total, size_t period, float* out) {
+  const size_t step = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += step) {
+    const float x = a[i], y = b[period == total ? i : i % period];
+    out[i] = OP == 4 ? powf(x, y) : OP == 5 ? fmaxf(x, y) : fminf(x, y);
+  }
+}
+template <int OP>
+__global__ __launch_bounds__(256) void scalar2_kernel(const float* a, size_t total, float p0, float p1, float* out) {
+  const size_t step = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += step) {
+    const float v = a[i];
+    out[i] = OP == 0 ? fminf(fmaxf(v, p0), p1) : (v > 0.f ? v : v * p0);
+  }
+}
+
 // The general numpy-style broadcast: every dimension has the output's extent on one side or both, the other side's
 // stride is 0 there.
 struct BroadcastParams {
@@ -202,7 +258,13 @@ __global__ __launch_bounds__(256) void binary_broadcast_kernel(const float* a, c
       ib += c * p.strideB[d];
     }
     const float x = a[ia], y = b[ib];
-    out[i] = OP == 0 ? x + y : OP == 1 ? x - y : OP == 2 ? x * y : x / y;
+    out[i] = OP == 0   ? x + y
+             : OP == 1 ? x - y
+             : OP == 2 ? x * y
+             : OP == 3 ? x / y
+             : OP == 4 ? powf(x, y)
+             : OP == 5 ? fmaxf(x, y)
+                       : fminf(x, y);
   }
 }
 
@@ -342,7 +404,7 @@ int tfcc_rocm_transform2_f32(void* stream, const float* in, uint64_t total, floa
 int tfcc_rocm_binary_f32(void* stream, int op, const float* a, const float* b, uint64_t total, uint64_t period,
                          float* out) {
   TFCC_REQUIRE(a && b && out, "binary: null argument");
-  TFCC_REQUIRE(op >= 0 && op <= 3, "binary: unknown op %d", op);
+  TFCC_REQUIRE(op >= 0 && op <= 6, "binary: unknown op %d", op);
   TFCC_REQUIRE(total > 0 && period > 0 && period <= total && total % period == 0, "binary: bad broadcast period");
   const dim3 grid(grid_for(total)), block(256);
   hipStream_t s = as_stream(stream);
@@ -350,15 +412,57 @@ int tfcc_rocm_binary_f32(void* stream, int op, const float* a, const float* b, u
     case 0: hipLaunchKernelGGL(binary_kernel<0>, grid, block, 0, s, a, b, (size_t)total, (size_t)period, out); break;
     case 1: hipLaunchKernelGGL(binary_kernel<1>, grid, block, 0, s, a, b, (size_t)total, (size_t)period, out); break;
     case 2: hipLaunchKernelGGL(binary_kernel<2>, grid, block, 0, s, a, b, (size_t)total, (size_t)period, out); break;
-    default: hipLaunchKernelGGL(binary_kernel<3>, grid, block, 0, s, a, b, (size_t)total, (size_t)period, out); break;
+    case 3: hipLaunchKernelGGL(binary_kernel<3>, grid, block, 0, s, a, b, (size_t)total, (size_t)period, out); break;
+    case 4: hipLaunchKernelGGL(binary2_kernel<4>, grid, block, 0, s, a, b, (size_t)total, (size_t)period, out); break;
+    case 5: hipLaunchKernelGGL(binary2_kernel<5>, grid, block, 0, s, a, b, (size_t)total, (size_t)period, out); break;
+    default: hipLaunchKernelGGL(binary2_kernel<6>, grid, block, 0, s, a, b, (size_t)total, (size_t)period, out); break;
   }
   return check_launch("binary");
+}
+
+int tfcc_rocm_reduce_f32(void* stream, int op, const float* in, uint64_t rows, unsigned cols, float* out) {
+  TFCC_REQUIRE(in && out, "reduce: null argument");
+  TFCC_REQUIRE(rows > 0 && cols > 0, "reduce: empty tensor");
+  TFCC_REQUIRE(rows < (1ull << 31), "reduce: too many rows");
+  hipStream_t s = as_stream(stream);
+  const bool block = cols > 4096;
+  const dim3 grid(block ? (unsigned)rows : (unsigned)((rows + 3) / 4)), threads(256);
+#define TFCC_REDUCE_CASE(OP)                                                                                        \
+  case OP:                                                                                                          \
+    if (block) hipLaunchKernelGGL((reduce_trailing_kernel<OP, true>), grid, threads, 0, s, in, (size_t)rows, cols, out); \
+    else hipLaunchKernelGGL((reduce_trailing_kernel<OP, false>), grid, threads, 0, s, in, (size_t)rows, cols, out);  \
+    break;
+  switch (op) {
+    TFCC_REDUCE_CASE(TFCC_ROCM_REDUCE_SUM)
+    TFCC_REDUCE_CASE(TFCC_ROCM_REDUCE_MEAN)
+    TFCC_REDUCE_CASE(TFCC_ROCM_REDUCE_PROD)
+    TFCC_REDUCE_CASE(TFCC_ROCM_REDUCE_MAX)
+    TFCC_REDUCE_CASE(TFCC_ROCM_REDUCE_MIN)
+    default: return set_error(TFCC_ROCM_INVALID_ARGUMENT, "reduce: unknown operation %d", op);
+  }
+#undef TFCC_REDUCE_CASE
+  return check_launch("reduce");
+}
+
+int tfcc_rocm_clip_f32(void* stream, const float* in, uint64_t total, float lo, float hi, float* out) {
+  TFCC_REQUIRE(in && out, "clip: null argument");
+  TFCC_REQUIRE(total > 0, "clip: empty tensor");
+  hipLaunchKernelGGL(scalar2_kernel<0>, dim3(grid_for(total)), dim3(256), 0, as_stream(stream), in, (size_t)total, lo, hi, out);
+  return check_launch("clip");
+}
+
+int tfcc_rocm_leaky_relu_f32(void* stream, const float* in, uint64_t total, float alpha, float* out) {
+  TFCC_REQUIRE(in && out, "leaky_relu: null argument");
+  TFCC_REQUIRE(total > 0, "leaky_relu: empty tensor");
+  hipLaunchKernelGGL(scalar2_kernel<1>, dim3(grid_for(total)), dim3(256), 0, as_stream(stream), in, (size_t)total, alpha, 0.f,
+                     out);
+  return check_launch("leaky_relu");
 }
 
 int tfcc_rocm_binary_broadcast_f32(void* stream, int op, const float* a, const float* b, int rank,
                                    const unsigned* dims, const uint64_t* stride_a, const uint64_t* stride_b, float* out) {
   TFCC_REQUIRE(a && b && out && dims && stride_a && stride_b, "binary_broadcast: null argument");
-  TFCC_REQUIRE(op >= 0 && op <= 3, "binary_broadcast: unknown operation %d", op);
+  TFCC_REQUIRE(op >= 0 && op <= 6, "binary_broadcast: unknown operation %d", op);
   TFCC_REQUIRE(rank >= 1 && rank <= 6, "binary_broadcast: rank %d (1..6)", rank);
   BroadcastParams p{};
   p.rank = rank;
@@ -376,7 +480,10 @@ int tfcc_rocm_binary_broadcast_f32(void* stream, int op, const float* a, const f
     case 0: hipLaunchKernelGGL(binary_broadcast_kernel<0>, grid, block, 0, s, a, b, total, p, out); break;
     case 1: hipLaunchKernelGGL(binary_broadcast_kernel<1>, grid, block, 0, s, a, b, total, p, out); break;
     case 2: hipLaunchKernelGGL(binary_broadcast_kernel<2>, grid, block, 0, s, a, b, total, p, out); break;
-    default: hipLaunchKernelGGL(binary_broadcast_kernel<3>, grid, block, 0, s, a, b, total, p, out); break;
+    case 3: hipLaunchKernelGGL(binary_broadcast_kernel<3>, grid, block, 0, s, a, b, total, p, out); break;
+    case 4: hipLaunchKernelGGL(binary_broadcast_kernel<4>, grid, block, 0, s, a, b, total, p, out); break;
+    case 5: hipLaunchKernelGGL(binary_broadcast_kernel<5>, grid, block, 0, s, a, b, total, p, out); break;
+    default: hipLaunchKernelGGL(binary_broadcast_kernel<6>, grid, block, 0, s, a, b, total, p, out); break;
   }
   return check_launch("binary_broadcast");
 }

@@ -3,6 +3,7 @@
 #include <algorithm>
 #include <cstdlib>
 #include <cstring>
+#include <limits>
 #include <type_traits>
 
 #include "tfcc_rocm.h"
@@ -548,6 +549,14 @@ class ROCMActivationInterface : public ActivationInterface<float> {
     check(tfcc_rocm_unary_f32(current_stream(), function, a.data(), a.size(), r.data()));
     return r;
   }
+  Variable<float> leakyRelu(const Tensor<float>& a, float alpha) override {
+    Variable<float> r(a.shape());
+    check(tfcc_rocm_leaky_relu_f32(current_stream(), a.data(), a.size(), alpha, r.data()));
+    return r;
+  }
+  Variable<float> pow(const Tensor<float>& a, float exponent) override;
+  Variable<float> pow(const Tensor<float>& a, const Tensor<float>& exponent) override;
+  Variable<float> pow(float a, const Tensor<float>& exponent) override;
 };
 
 // Checks and error texts of tfcc/mkl/interfaces/tfcc_mklcellinterface.cpp:33-165.
@@ -727,6 +736,15 @@ class ROCMBasicInterface : public BasicInterface<T> {
     }
     return r;
   }
+  Variable<T> clip(const Tensor<T>& a, T minValue, T maxValue) override {
+    if constexpr (std::is_same<T, float>::value) {
+      Variable<T> r(a.shape());
+      check(tfcc_rocm_clip_f32(current_stream(), a.data(), a.size(), minValue, maxValue, r.data()));
+      return r;
+    } else {
+      throw NotImplementedError("clip: float tensors only");
+    }
+  }
   Variable<T> gather(const Tensor<T>& params, const void* indices, int indexCode, const Shape& indexShape) override {
     std::vector<unsigned> shape = indexShape.toVector();
     for (size_t i = 1; i < params.shape().size(); ++i) shape.push_back(params.shape(i));
@@ -739,8 +757,7 @@ class ROCMBasicInterface : public BasicInterface<T> {
 };
 
 // a and b arrive with equal rank, every dimension equal or 1 on one side (tfcc::math merges the rest away).
-class ROCMArithmeticInterface : public ArithmeticInterface<float> {
-  static Variable<float> run(int op, const Tensor<float>& a, const Tensor<float>& b) {
+Variable<float> broadcast_binary_run(int op, const Tensor<float>& a, const Tensor<float>& b) {
     const size_t rank = a.shape().size();
     if (rank == 0 || rank != b.shape().size()) throw InvalidArgumentError("invalid tensor shape");
     std::vector<unsigned> dims(rank);
@@ -771,14 +788,73 @@ class ROCMArithmeticInterface : public ArithmeticInterface<float> {
     check(tfcc_rocm_binary_broadcast_f32(current_stream(), op, a.data(), b.data(), static_cast<int>(rank), dims.data(), sa,
                                          sb, r.data()));
     return r;
+}
+
+class ROCMArithmeticInterface : public ArithmeticInterface<float> {
+ public:
+  Variable<float> add(const Tensor<float>& a, const Tensor<float>& b) override { return broadcast_binary_run(0, a, b); }
+  Variable<float> sub(const Tensor<float>& a, const Tensor<float>& b) override { return broadcast_binary_run(1, a, b); }
+  Variable<float> mul(const Tensor<float>& a, const Tensor<float>& b) override { return broadcast_binary_run(2, a, b); }
+  Variable<float> div(const Tensor<float>& a, const Tensor<float>& b) override { return broadcast_binary_run(3, a, b); }
+};
+
+// a one-element tensor of the rank of `like` holding `value`
+Variable<float> scalar_like(const Tensor<float>& like, float value) {
+  Variable<float> v{Shape(std::vector<unsigned>(like.shape().size(), 1u))};
+  uint64_t bits = 0;
+  std::memcpy(&bits, &value, sizeof(float));
+  check(tfcc_rocm_fill_async(current_stream(), v.data(), bits, sizeof(float), 1));
+  return v;
+}
+
+class ROCMMinMaxInterface : public MinMaxInterface<float> {
+ public:
+  Variable<float> min(const Tensor<float>& a, const Tensor<float>& b) override { return broadcast_binary_run(6, a, b); }
+  Variable<float> max(const Tensor<float>& a, const Tensor<float>& b) override { return broadcast_binary_run(5, a, b); }
+  Variable<float> min(const Tensor<float>& a, float b) override {
+    Variable<float> r(a.shape());
+    check(tfcc_rocm_clip_f32(current_stream(), a.data(), a.size(), -std::numeric_limits<float>::infinity(), b, r.data()));
+    return r;
+  }
+  Variable<float> max(const Tensor<float>& a, float b) override {
+    Variable<float> r(a.shape());
+    check(tfcc_rocm_clip_f32(current_stream(), a.data(), a.size(), b, std::numeric_limits<float>::infinity(), r.data()));
+    return r;
+  }
+};
+
+class ROCMReduceInterface : public ReduceInterface<float> {
+  static Variable<float> run(int op, const Tensor<float>& a, size_t keep) {
+    std::vector<unsigned> s = a.shape().toVector();
+    size_t cols = 1;
+    for (size_t d = keep; d < s.size(); ++d) {
+      cols *= s[d];
+      s[d] = 1;
+    }
+    Variable<float> r{Shape(s)};
+    check(tfcc_rocm_reduce_f32(current_stream(), op, a.data(), a.size() / cols, cols, r.data()));
+    return r;
   }
 
  public:
-  Variable<float> add(const Tensor<float>& a, const Tensor<float>& b) override { return run(0, a, b); }
-  Variable<float> sub(const Tensor<float>& a, const Tensor<float>& b) override { return run(1, a, b); }
-  Variable<float> mul(const Tensor<float>& a, const Tensor<float>& b) override { return run(2, a, b); }
-  Variable<float> div(const Tensor<float>& a, const Tensor<float>& b) override { return run(3, a, b); }
+  Variable<float> reduceSum(const Tensor<float>& a, size_t keep) override { return run(TFCC_ROCM_REDUCE_SUM, a, keep); }
+  Variable<float> reduceMean(const Tensor<float>& a, size_t keep) override { return run(TFCC_ROCM_REDUCE_MEAN, a, keep); }
+  Variable<float> reduceProd(const Tensor<float>& a, size_t keep) override { return run(TFCC_ROCM_REDUCE_PROD, a, keep); }
+  Variable<float> reduceMax(const Tensor<float>& a, size_t keep) override { return run(TFCC_ROCM_REDUCE_MAX, a, keep); }
+  Variable<float> reduceMin(const Tensor<float>& a, size_t keep) override { return run(TFCC_ROCM_REDUCE_MIN, a, keep); }
 };
+
+Variable<float> ROCMActivationInterface::pow(const Tensor<float>& a, float exponent) {
+  Variable<float> e = scalar_like(a, exponent);
+  return broadcast_binary_run(4, a, e);
+}
+Variable<float> ROCMActivationInterface::pow(const Tensor<float>& a, const Tensor<float>& exponent) {
+  return broadcast_binary_run(4, a, exponent);
+}
+Variable<float> ROCMActivationInterface::pow(float a, const Tensor<float>& exponent) {
+  Variable<float> base = scalar_like(exponent, a);
+  return broadcast_binary_run(4, base, exponent);
+}
 
 class ROCMTransformationInterface : public TransformationInterface<float> {
  public:
@@ -856,6 +932,8 @@ ROCMDevice::ROCMDevice(unsigned index, std::unique_ptr<Allocator> allocator)
   _interfaces->f32.setActivationInterface(std::unique_ptr<ActivationInterface<float>>(new ROCMActivationInterface()));
   _interfaces->f32.setNormalizationInterface(std::unique_ptr<NormalizationInterface<float>>(new ROCMNormalizationInterface()));
   _interfaces->f32.setArithmeticInterface(std::unique_ptr<ArithmeticInterface<float>>(new ROCMArithmeticInterface()));
+  _interfaces->f32.setMinMaxInterface(std::unique_ptr<MinMaxInterface<float>>(new ROCMMinMaxInterface()));
+  _interfaces->f32.setReduceInterface(std::unique_ptr<ReduceInterface<float>>(new ROCMReduceInterface()));
   _interfaces->f32.setCellInterface(std::unique_ptr<CellInterface<float>>(new ROCMCellInterface()));
   _interfaces->f32.setTransformationInterface(std::unique_ptr<TransformationInterface<float>>(new ROCMTransformationInterface()));
 }

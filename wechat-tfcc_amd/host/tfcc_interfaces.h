@@ -94,6 +94,11 @@ class ActivationInterface {
   virtual Variable<T> geluAccurate(const Tensor<T>&) { throw NotImplementedError(); }
   // one of the UnaryFunction values below applied to every element
   virtual Variable<T> unary(const Tensor<T>&, int) { throw NotImplementedError(); }
+  // tfcc/core/interfaces/tfcc_activationinterface.h:34-43
+  virtual Variable<T> leakyRelu(const Tensor<T>&, T) { throw NotImplementedError(); }
+  virtual Variable<T> pow(const Tensor<T>&, T) { throw NotImplementedError(); }
+  virtual Variable<T> pow(const Tensor<T>&, const Tensor<T>&) { throw NotImplementedError(); }  // equal rank, broadcast
+  virtual Variable<T> pow(T, const Tensor<T>&) { throw NotImplementedError(); }
 };
 
 // element-wise functions of one tensor (the numbering of the kernel library's TFCC_ROCM_UNARY_* values)
@@ -116,6 +121,7 @@ class BasicInterface {
   virtual Variable<T> slice(const Tensor<T>&, size_t, unsigned, unsigned) { throw NotImplementedError(); }
   virtual Variable<T> concat(const std::vector<const Tensor<T>*>&, size_t) { throw NotImplementedError(); }
   // rows of params by index (tfcc/core/interfaces/tfcc_gatherinterface.h): indices of the type with code indexCode
+  virtual Variable<T> clip(const Tensor<T>&, T, T) { throw NotImplementedError(); }
   virtual Variable<T> gather(const Tensor<T>&, const void* /*indices*/, int /*indexCode*/, const Shape& /*indexShape*/) {
     throw NotImplementedError();
   }
@@ -129,6 +135,30 @@ class ArithmeticInterface {
   virtual Variable<T> sub(const Tensor<T>&, const Tensor<T>&) { throw NotImplementedError(); }
   virtual Variable<T> mul(const Tensor<T>&, const Tensor<T>&) { throw NotImplementedError(); }
   virtual Variable<T> div(const Tensor<T>&, const Tensor<T>&) { throw NotImplementedError(); }
+};
+
+// tfcc/core/interfaces/tfcc_minmaxinterface.h:30-68
+template <class T>
+class MinMaxInterface {
+ public:
+  virtual ~MinMaxInterface() {}
+  virtual Variable<T> min(const Tensor<T>&, const Tensor<T>&) { throw NotImplementedError(); }
+  virtual Variable<T> min(const Tensor<T>&, T) { throw NotImplementedError(); }
+  virtual Variable<T> max(const Tensor<T>&, const Tensor<T>&) { throw NotImplementedError(); }
+  virtual Variable<T> max(const Tensor<T>&, T) { throw NotImplementedError(); }
+};
+
+// tfcc/core/interfaces/tfcc_reduceinterface.h:27-41: the dimensions from `keep` on are reduced and stay in the
+// result's shape with length 1.
+template <class T>
+class ReduceInterface {
+ public:
+  virtual ~ReduceInterface() {}
+  virtual Variable<T> reduceSum(const Tensor<T>&, size_t) { throw NotImplementedError(); }
+  virtual Variable<T> reduceMean(const Tensor<T>&, size_t) { throw NotImplementedError(); }
+  virtual Variable<T> reduceProd(const Tensor<T>&, size_t) { throw NotImplementedError(); }
+  virtual Variable<T> reduceMax(const Tensor<T>&, size_t) { throw NotImplementedError(); }
+  virtual Variable<T> reduceMin(const Tensor<T>&, size_t) { throw NotImplementedError(); }
 };
 
 template <class T>
@@ -193,6 +223,8 @@ class Interface {
   TFCC_SUB_INTERFACE(Arithmetic)
   TFCC_SUB_INTERFACE(Transformation)
   TFCC_SUB_INTERFACE(Cell)
+  TFCC_SUB_INTERFACE(MinMax)
+  TFCC_SUB_INTERFACE(Reduce)
 #undef TFCC_SUB_INTERFACE
 };
 
@@ -442,6 +474,87 @@ template <class T>
 Variable<T> div(const Tensor<T>& a, const Tensor<T>& b) {
   return detail::broadcast_binary(a, b, [](ArithmeticInterface<T>& i, const Tensor<T>& x, const Tensor<T>& y) { return i.div(x, y); });
 }
+// tfcc::math::min / max of two tensors or a tensor and a value (tfcc/core/operations/tfcc_math.cpp:257-320)
+template <class T>
+Variable<T> min(const Tensor<T>& a, const Tensor<T>& b) {
+  Shape resultS, newAS, newBS;
+  std::tie(resultS, newAS, newBS) = detail::broadcast_shapes(a.shape(), b.shape());
+  if (resultS.area() == 0) return Variable<T>(resultS);
+  View<T> aView(a, newAS), bView(b, newBS);
+  Variable<T> result = Operation<T>::getCurrentInterface().getMinMaxInterface().min(aView, bView);
+  result.reshape(std::move(resultS));
+  return result;
+}
+template <class T>
+Variable<T> max(const Tensor<T>& a, const Tensor<T>& b) {
+  Shape resultS, newAS, newBS;
+  std::tie(resultS, newAS, newBS) = detail::broadcast_shapes(a.shape(), b.shape());
+  if (resultS.area() == 0) return Variable<T>(resultS);
+  View<T> aView(a, newAS), bView(b, newBS);
+  Variable<T> result = Operation<T>::getCurrentInterface().getMinMaxInterface().max(aView, bView);
+  result.reshape(std::move(resultS));
+  return result;
+}
+template <class T>
+Variable<T> min(const Tensor<T>& a, T b) {
+  if (a.size() == 0) throw InvalidArgumentError("invalid tensor");
+  return Operation<T>::getCurrentInterface().getMinMaxInterface().min(a, b);
+}
+template <class T>
+Variable<T> min(T a, const Tensor<T>& b) { return min(b, a); }
+template <class T>
+Variable<T> max(const Tensor<T>& a, T b) {
+  if (a.size() == 0) throw InvalidArgumentError("invalid tensor");
+  return Operation<T>::getCurrentInterface().getMinMaxInterface().max(a, b);
+}
+template <class T>
+Variable<T> max(T a, const Tensor<T>& b) { return max(b, a); }
+// tfcc::math::leaky_relu, pow, clip (tfcc/core/operations/tfcc_math.cpp:343-350, :423-452, :536-543).  The reference
+// expands both operands of pow to the result's shape first; here the kernel reads them through their own strides.
+template <class T>
+Variable<T> leaky_relu(const Tensor<T>& a, T alpha) {
+  if (a.size() == 0) throw InvalidArgumentError("invalid tensor");
+  return Operation<T>::getCurrentInterface().getActivationInterface().leakyRelu(a, alpha);
+}
+template <class T>
+Variable<T> pow(const Tensor<T>& a, T exponent) {
+  if (a.size() == 0) throw InvalidArgumentError("invalid tensor");
+  return Operation<T>::getCurrentInterface().getActivationInterface().pow(a, exponent);
+}
+template <class T>
+Variable<T> pow(const Tensor<T>& a, const Tensor<T>& exponent) {
+  if (a.size() == 0 || exponent.size() == 0) throw InvalidArgumentError("invalid tensor");
+  Shape resultS, newAS, newBS;
+  std::tie(resultS, newAS, newBS) = detail::broadcast_shapes(a.shape(), exponent.shape());
+  View<T> aView(a, newAS), bView(exponent, newBS);
+  Variable<T> result = Operation<T>::getCurrentInterface().getActivationInterface().pow(aView, bView);
+  result.reshape(std::move(resultS));
+  return result;
+}
+template <class T>
+Variable<T> pow(T a, const Tensor<T>& exponent) {
+  if (exponent.size() == 0) throw InvalidArgumentError("invalid tensor");
+  return Operation<T>::getCurrentInterface().getActivationInterface().pow(a, exponent);
+}
+template <class T>
+Variable<T> clip(const Tensor<T>& a, T minValue, T maxValue) {
+  if (a.size() == 0) throw InvalidArgumentError("invalid tensor");
+  return Operation<T>::getCurrentInterface().getBasicInterface().clip(a, minValue, maxValue);
+}
+// tfcc::math::reduce_sum / mean / prod / max / min (tfcc/core/operations/tfcc_math.cpp:464-522)
+#define TFCC_REDUCE_FUNCTION(NAME, METHOD)                                                   \
+  template <class T>                                                                         \
+  Variable<T> NAME(const Tensor<T>& a, size_t keep) {                                        \
+    if (a.size() == 0) throw InvalidArgumentError("invalid tensor");                         \
+    if (keep >= a.shape().size()) throw InvalidArgumentError("invalid keep dims");           \
+    return Operation<T>::getCurrentInterface().getReduceInterface().METHOD(a, keep);         \
+  }
+TFCC_REDUCE_FUNCTION(reduce_sum, reduceSum)
+TFCC_REDUCE_FUNCTION(reduce_mean, reduceMean)
+TFCC_REDUCE_FUNCTION(reduce_prod, reduceProd)
+TFCC_REDUCE_FUNCTION(reduce_max, reduceMax)
+TFCC_REDUCE_FUNCTION(reduce_min, reduceMin)
+#undef TFCC_REDUCE_FUNCTION
 template <class T>
 Variable<T> transform(const Tensor<T>& a, T alpha, T beta) {
   return Operation<T>::getCurrentInterface().getTransformationInterface().transform(a, alpha, beta);

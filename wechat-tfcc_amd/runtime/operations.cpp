@@ -87,28 +87,67 @@ class MatmulWithBias : public TypedOperation<T> {
   }
 };
 
-// ---- math.Add / Sub / Mul / Div -------------------------------------------------------------------------
-enum class Arith { ADD, SUB, MUL, DIV };
+// ---- math.Add / Sub / Mul / Div / Pow / Max / Min --------------------------------------------------------
+// tensor (x) tensor, tensor (x) value, value (x) tensor and value (x) value forms, as
+// tfcc_runtime/operations/math/{add,sub,mul,div,pow,max,min}.cpp register them.
+enum class Arith { ADD, SUB, MUL, DIV, POW, MAX, MIN };
 
 template <Arith OP, class T>
 class Arithmetic : public TypedOperation<T> {
   static const char* message() {
-    return OP == Arith::ADD ? "math.Add" : OP == Arith::SUB ? "math.Sub" : OP == Arith::MUL ? "math.Mul" : "math.Div";
+    switch (OP) {
+      case Arith::ADD: return "math.Add";
+      case Arith::SUB: return "math.Sub";
+      case Arith::MUL: return "math.Mul";
+      case Arith::DIV: return "math.Div";
+      case Arith::POW: return "math.Pow";
+      case Arith::MAX: return "math.Max";
+      default: return "math.Min";
+    }
   }
   static Variable<T> tt(const Tensor<T>& a, const Tensor<T>& b) {
-    return OP == Arith::ADD ? a + b : OP == Arith::SUB ? a - b : OP == Arith::MUL ? a * b : a / b;
+    switch (OP) {
+      case Arith::ADD: return a + b;
+      case Arith::SUB: return a - b;
+      case Arith::MUL: return a * b;
+      case Arith::DIV: return a / b;
+      case Arith::POW: return math::pow(a, b);
+      case Arith::MAX: return math::max(a, b);
+      default: return math::min(a, b);
+    }
   }
   static Variable<T> tv(const Tensor<T>& a, T b) {
-    return OP == Arith::ADD ? a + b : OP == Arith::SUB ? a - b : OP == Arith::MUL ? a * b : a / b;
+    switch (OP) {
+      case Arith::ADD: return a + b;
+      case Arith::SUB: return a - b;
+      case Arith::MUL: return a * b;
+      case Arith::DIV: return a / b;
+      case Arith::POW: return math::pow(a, b);
+      case Arith::MAX: return math::max(a, b);
+      default: return math::min(a, b);
+    }
   }
   static Variable<T> vt(T a, const Tensor<T>& b) {
-    if (OP == Arith::ADD) return a + b;
-    if (OP == Arith::SUB) return a - b;
-    if (OP == Arith::MUL) return a * b;
-    throw NotImplementedError("value / tensor");
+    switch (OP) {
+      case Arith::ADD: return a + b;
+      case Arith::SUB: return a - b;
+      case Arith::MUL: return a * b;
+      case Arith::DIV: throw NotImplementedError("value / tensor");
+      case Arith::POW: return math::pow(a, b);
+      case Arith::MAX: return math::max(a, b);
+      default: return math::min(a, b);
+    }
   }
   static T vv(T a, T b) {
-    return OP == Arith::ADD ? a + b : OP == Arith::SUB ? a - b : OP == Arith::MUL ? a * b : a / b;
+    switch (OP) {
+      case Arith::ADD: return a + b;
+      case Arith::SUB: return a - b;
+      case Arith::MUL: return a * b;
+      case Arith::DIV: return a / b;
+      case Arith::POW: return static_cast<T>(std::pow(a, b));
+      case Arith::MAX: return std::max(a, b);
+      default: return std::min(a, b);
+    }
   }
 
  public:
@@ -233,6 +272,119 @@ class Softmax : public TypedOperation<T> {
     const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
     Variable<T>* out = sm.getVariable(node.outputs[0], T());
     graph.addStep([a, out, axis] { *out = math::softmax(*a, axis); });
+    return true;
+  }
+};
+
+// ---- math.ReduceSum / ReduceMean / ReduceProd / ReduceMax / ReduceMin --------------------------------------
+// The axes are sorted and moved behind the others with a transpose when they are not the trailing ones already; the
+// result keeps them with length 1 (tfcc_runtime/operations/math/reducemean.cpp:27-45, utils/reduceutils.h:25-50).
+enum class Reduction { SUM, MEAN, PROD, MAX, MIN };
+
+template <Reduction R, class T>
+class Reduce : public TypedOperation<T> {
+  static const char* message() {
+    switch (R) {
+      case Reduction::SUM: return "math.ReduceSum";
+      case Reduction::MEAN: return "math.ReduceMean";
+      case Reduction::PROD: return "math.ReduceProd";
+      case Reduction::MAX: return "math.ReduceMax";
+      default: return "math.ReduceMin";
+    }
+  }
+  static Variable<T> trailing(const Tensor<T>& a, size_t keep) {
+    switch (R) {
+      case Reduction::SUM: return math::reduce_sum(a, keep);
+      case Reduction::MEAN: return math::reduce_mean(a, keep);
+      case Reduction::PROD: return math::reduce_prod(a, keep);
+      case Reduction::MAX: return math::reduce_max(a, keep);
+      default: return math::reduce_min(a, keep);
+    }
+  }
+
+ public:
+  Reduce() : TypedOperation<T>(message()) {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 1 || node.outputs.size() != 1) return false;
+    if (!same_dtype(graph, node.outputs, this->DTYPE) || !same_dtype(graph, node.inputs, this->DTYPE)) return false;
+    std::vector<size_t> axes;
+    wire::Reader r(node.operation);
+    uint32_t f, t;
+    while (r.next(f, t)) {
+      if (f == 1) r.repeatedVarint(t, axes);
+      else r.skip(t);
+    }
+    std::sort(axes.begin(), axes.end());
+    auto& sm = graph.getSymbolManager();
+    const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+    Variable<T>* out = sm.getVariable(node.outputs[0], T());
+    graph.addStep([a, out, axes] {
+      const size_t rank = a->shape().size();
+      std::vector<unsigned> target = a->shape().toVector();
+      std::vector<bool> reduced(rank, false);
+      for (size_t axis : axes) {
+        if (axis >= rank) throw InvalidArgumentError("invalid axis");
+        target[axis] = 1;
+        reduced[axis] = true;
+      }
+      std::vector<size_t> perm;
+      for (size_t i = 0; i < rank; ++i)
+        if (!reduced[i]) perm.push_back(i);
+      for (size_t axis : axes) perm.push_back(axis);
+      bool inPlace = true;
+      for (size_t i = 0; i < perm.size(); ++i) inPlace = inPlace && perm[i] == i;
+      if (inPlace) {
+        *out = trailing(*a, rank - axes.size());
+      } else {
+        Variable<T> moved = base::transpose(*a, perm);
+        *out = trailing(moved, rank - axes.size());
+        out->reshape(Shape(target));
+      }
+    });
+    return true;
+  }
+};
+
+// ---- math.Clip (tensor, minimum value, maximum value), math.LeakyRelu (alpha in the node) --------------------
+// tfcc_runtime/operations/math/clip.cpp:52-87, leakyrelu.cpp:52-86
+template <class T>
+class Clip : public TypedOperation<T> {
+ public:
+  Clip() : TypedOperation<T>("math.Clip") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 3 || node.outputs.size() != 1) return false;
+    if (!same_dtype(graph, node.outputs, this->DTYPE) || !same_dtype(graph, node.inputs, this->DTYPE)) return false;
+    if (!is_value(stype_of(graph, node.inputs[1])) || !is_value(stype_of(graph, node.inputs[2]))) return false;
+    auto& sm = graph.getSymbolManager();
+    const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+    const T* lo = sm.getValue(node.inputs[1], T());
+    const T* hi = sm.getValue(node.inputs[2], T());
+    Variable<T>* out = sm.getVariable(node.outputs[0], T());
+    graph.addStep([a, lo, hi, out] { *out = math::clip(*a, *lo, *hi); });
+    return true;
+  }
+};
+
+template <class T>
+class LeakyRelu : public TypedOperation<T> {
+ public:
+  LeakyRelu() : TypedOperation<T>("math.LeakyRelu") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 1 || node.outputs.size() != 1) return false;
+    if (!same_dtype(graph, node.outputs, this->DTYPE) || !same_dtype(graph, node.inputs, this->DTYPE)) return false;
+    proto::Value v;
+    wire::Reader r(node.operation);
+    uint32_t f, t;
+    while (r.next(f, t)) {
+      if (f == 1 && t == 2) v = proto::parse_value(r.sub());
+      else r.skip(t);
+    }
+    T alpha = static_cast<T>(0);
+    if (!v.get(alpha)) return false;
+    auto& sm = graph.getSymbolManager();
+    const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+    Variable<T>* out = sm.getVariable(node.outputs[0], T());
+    graph.addStep([a, alpha, out] { *out = math::leaky_relu(*a, alpha); });
     return true;
   }
 };
@@ -954,6 +1106,16 @@ class Collector {
     add(new Arithmetic<Arith::SUB, T>());
     add(new Arithmetic<Arith::MUL, T>());
     add(new Arithmetic<Arith::DIV, T>());
+    add(new Arithmetic<Arith::POW, T>());
+    add(new Arithmetic<Arith::MAX, T>());
+    add(new Arithmetic<Arith::MIN, T>());
+    add(new Reduce<Reduction::SUM, T>());
+    add(new Reduce<Reduction::MEAN, T>());
+    add(new Reduce<Reduction::PROD, T>());
+    add(new Reduce<Reduction::MAX, T>());
+    add(new Reduce<Reduction::MIN, T>());
+    add(new Clip<T>());
+    add(new LeakyRelu<T>());
     add(new Gelu<T>());
     add(new Unary<UnaryFunction::SIGMOID, T>());
     add(new Unary<UnaryFunction::TANH, T>());
