@@ -343,6 +343,26 @@ int tfcc_rocm_reduce_f32(void* stream, int op, const float* in, uint64_t rows, u
 /* min(max(v, lo), hi) (tfcc::math::clip) and v > 0 ? v : v * alpha (tfcc::math::leaky_relu) */
 int tfcc_rocm_clip_f32(void* stream, const float* in, uint64_t total, float lo, float hi, float* out);
 int tfcc_rocm_leaky_relu_f32(void* stream, const float* in, uint64_t total, float alpha, float* out);
+/* Comparisons with byte results (1 where the relation holds, else 0) for every element type (TFCC_ROCM_S8 .. F64).
+ * compare_value: a[i] OP *value, value a host pointer to one element of the tensor's type
+ * (tfcc/core/interfaces/tfcc_comparisoninterface.h:38-83).  compare: (a - b) OP 0 with numpy-style broadcasting given as
+ * for tfcc_rocm_binary_broadcast_f32, the difference taken in the element type as tfcc::relation::equal and its
+ * siblings do for two tensors (tfcc/core/operations/tfcc_relation.cpp:101-115): unsigned differences wrap. */
+enum {
+  TFCC_ROCM_COMPARE_EQUAL = 0,
+  TFCC_ROCM_COMPARE_UNEQUAL = 1,
+  TFCC_ROCM_COMPARE_GREATER = 2,
+  TFCC_ROCM_COMPARE_GREATER_EQUAL = 3,
+  TFCC_ROCM_COMPARE_LESS = 4,
+  TFCC_ROCM_COMPARE_LESS_EQUAL = 5
+};
+int tfcc_rocm_compare_value(void* stream, int op, const void* a, int type, uint64_t total, const void* value,
+                            uint8_t* out);
+int tfcc_rocm_compare(void* stream, int op, const void* a, const void* b, int type, int rank, const unsigned* dims,
+                      const uint64_t* stride_a, const uint64_t* stride_b, uint8_t* out);
+/* out[x, z] = first position y of the largest in[x, y, z], in is [outer, length, inner]
+ * (tfcc/mkl/interfaces/tfcc_mklbasicinterface.cpp:469-485, :757-776). */
+int tfcc_rocm_argmax_f32(void* stream, const float* in, uint64_t outer, unsigned length, uint64_t inner, int64_t* out);
 /* out = a op b with numpy-style broadcasting: dims[rank] is the result's shape, stride_a / stride_b the element strides
  * of each operand per result dimension (0 where the operand's extent is 1).  rank <= 6; callers merge adjacent
  * dimensions of the same kind first, as tfcc::math::add does (tfcc/core/operations/tfcc_math.cpp:38-104). */

@@ -618,6 +618,43 @@ def test_reductions_pow_max_min_clip_leaky_relu(pkg, T):
     assert np.array_equal(T.n(pkg.leaky_relu(T.t(b), 0.1)), np.where(b > 0, b, b * np.float32(0.1)))
 
 
+def test_comparisons_and_argmax(pkg, T):
+    """tfcc::relation's six comparisons: tensor against value (tfcc/core/interfaces/tfcc_comparisoninterface.h:38-83) and
+    tensor against tensor, where the reference compares the difference with 0 in the element type
+    (tfcc/core/operations/tfcc_relation.cpp:101-115): unsigned differences wrap, so `less` never holds for them.
+    tfcc::math::argmax: first position of the largest element (tfcc/mkl/interfaces/tfcc_mklbasicinterface.cpp:469-485)."""
+    rng = np.random.default_rng(47)
+    refs = {"equal": np.equal, "unequal": np.not_equal, "greater": np.greater, "greater_equal": np.greater_equal,
+            "less": np.less, "less_equal": np.less_equal}
+    for dtype in (np.float32, np.int32, np.int64, np.uint8, np.int8, np.float64):
+        a = rng.integers(0, 5, (3, 4, 33)).astype(dtype)
+        b = rng.integers(0, 5, (4, 1)).astype(dtype)
+        for op, ref in refs.items():
+            got = T.n(pkg.compare(op, T.t(a), 2))
+            assert got.dtype == np.uint8 and np.array_equal(got, ref(a, dtype(2)).astype(np.uint8)), (op, dtype)
+            with np.errstate(over="ignore"):
+                diff = (a - b).astype(dtype)
+            got = T.n(pkg.compare(op, T.t(a), T.t(b)))
+            assert np.array_equal(got, ref(diff, dtype(0)).astype(np.uint8)), (op, dtype)
+    inf = np.array([np.inf, 1.0], np.float32)
+    assert T.n(pkg.compare("equal", T.t(inf), T.t(inf))).tolist() == [0, 1]       # inf - inf is not 0
+    assert T.n(pkg.compare("equal", T.t(inf), float("inf"))).tolist() == [1, 0]
+    with pytest.raises(pkg.InvalidArgumentError):
+        pkg.compare("equal", T.t(np.zeros((0, 3), np.float32)), 1.0)
+    for shape, axis in (((5, 7, 9), 0), ((5, 7, 9), 1), ((5, 7, 9), 2), ((6, 300), 1), ((3, 64), 1), ((2, 5000), 1),
+                        ((1, 1), 0)):
+        x = rng.integers(0, 12, shape).astype(np.float32)       # many ties: the first position must win
+        got = T.n(pkg.argmax(T.t(x), axis))
+        assert got.dtype == np.int64 and np.array_equal(got, np.argmax(x, axis=axis, keepdims=True)), (shape, axis)
+    x = rng.normal(size=(4, 200)).astype(np.float32)
+    x[1, 0] = np.nan            # a NaN in the first place stays: nothing is greater
+    x[2, 77] = np.nan           # elsewhere it is never taken
+    want = np.array([np.argmax(x[0]), 0, np.nanargmax(x[2]), np.argmax(x[3])]).reshape(4, 1)
+    assert np.array_equal(T.n(pkg.argmax(T.t(x), 1)), want)
+    with pytest.raises(pkg.InvalidArgumentError, match="invalid axis"):
+        pkg.argmax(T.t(x), 2)
+
+
 BROADCAST_PAIRS = [
     ((2, 4, 8, 8), (2, 1, 1, 8)),        # attention scores + mask
     ((3, 1, 5), (1, 4, 1)),              # both sides broadcast

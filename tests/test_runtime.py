@@ -228,6 +228,25 @@ def test_value_arithmetic_and_vectors_on_host(mf, rt):
     assert [float(res["r_" + op][0]) for op in ops] == [7.5, 4.5, 9.0, 4.0, np.float32(6.0 ** 1.5), 6.0, 1.5]
 
 
+def test_value_comparisons_on_host(mf, rt):
+    """value (x) value forms of the relation nodes and relation.Not of a value run on the host
+    (tfcc_runtime/operations/relation/equal.cpp:123-130, not_.cpp:79-83)."""
+    g = mf.GraphBuilder("g")
+    a = g.value_input("a", mf.INT64)
+    b = g.value_input("b", mf.INT64)
+    ops = ("Equal", "UnEqual", "Greater", "GreaterOrEqual", "Less", "LessOrEqual")
+    for op in ops:
+        out = g._symbol("r_" + op, mf.BOOL, mf.VALUE)
+        g.node("relation." + op, [a, b], [out])
+        g.output(out)
+        inverse = g._symbol("n_" + op, mf.BOOL, mf.VALUE)
+        g.node("relation.Not", [out], [inverse])
+        g.output(inverse)
+    res = rt.Model(mf.write_model([g], "g"), host=True).run({"a": np.array([3], np.int64), "b": np.array([5], np.int64)})
+    assert [int(res["r_" + op][0]) for op in ops] == [0, 1, 0, 0, 1, 1]
+    assert [int(res["n_" + op][0]) for op in ops] == [1, 0, 1, 1, 0, 0]
+
+
 def test_archive_and_graph_errors(mf, rt):
     g = passthrough_graph(mf, mf.FLOAT, [2], [0])
     blob = mf.write_model([g], "g")
@@ -687,6 +706,81 @@ def test_reduce_pow_max_min_clip_leaky_relu_nodes_equal_numpy(mf, rt, dev):
     g.output(out)
     with pytest.raises(rt.RuntimeError_, match="invalid axis"):
         rt.Model(mf.write_model([g], "g")).run({"x": np.zeros((3, 4), np.float32)})
+
+
+@pytest.mark.gpu
+def test_relation_argmax_expand_tile_nodes_equal_numpy(mf, rt, dev):
+    """relation.Equal ... LessOrEqual with tensor and value operands (two tensors: the difference against 0, in the
+    element type), relation.Not, math.ArgMax, base.Expand and base.Tile: tfcc_runtime/operations/relation/*.cpp,
+    math/argmax.cpp, base/expand.cpp, base/tile.cpp.  The attention mask of a converted BERT is built this way:
+    Equal(ids, 0) -> Cast -> Mul by a large negative number."""
+    rng = np.random.default_rng(53)
+    ids = rng.integers(0, 4, (2, 7)).astype(np.int64)
+    a = rng.integers(-3, 4, (2, 3, 7)).astype(np.float32)
+    b = rng.integers(-3, 4, (3, 1)).astype(np.float32)
+    g = mf.GraphBuilder("g")
+    x_ids = g.input("ids", mf.INT64, [2, 7])
+    x = g.input("x", mf.FLOAT, [2, 3, 7])
+    y = g.input("y", mf.FLOAT, [3, 1])
+    wants = {}
+    refs = {"Equal": np.equal, "UnEqual": np.not_equal, "Greater": np.greater, "GreaterOrEqual": np.greater_equal,
+            "Less": np.less, "LessOrEqual": np.less_equal}
+    for op, ref in refs.items():
+        out = g.variable("tt", mf.BOOL)
+        g.node("relation." + op, [x, y], [out])
+        wants[out] = ref(a - b, 0)
+        out = g.variable("tv", mf.BOOL)
+        g.node("relation." + op, [x, g.constant("one" + op, np.array(1, np.float32), mf.CONSTANT_VALUE)], [out])
+        wants[out] = ref(a, 1)
+        out = g.variable("vt", mf.BOOL)
+        g.node("relation." + op, [g.constant("zero" + op, np.array(0, np.float32), mf.CONSTANT_VALUE), y], [out])
+        wants[out] = ref(0, b)
+    is_pad = g.variable("is_pad", mf.BOOL)
+    g.node("relation.Equal", [x_ids, g.constant("pad", np.array(0, np.int64), mf.CONSTANT_VALUE)], [is_pad])
+    wants[is_pad] = ids == 0
+    is_token = g.variable("is_token", mf.BOOL)
+    g.node("relation.Not", [is_pad], [is_token])
+    wants[is_token] = ids != 0
+    mask = g.variable("mask")
+    g.node("base.Cast", [is_pad], [mask], mf.f_varint(1, mf.FLOAT))
+    bias = g.binary("Mul", mask, g.constant("neg", np.array(-10000.0, np.float32), mf.CONSTANT_VALUE))
+    wants[bias] = (ids == 0).astype(np.float32) * np.float32(-10000.0)
+    nonzero = g.variable("nonzero", mf.BOOL)
+    g.node("base.Cast", [x, ], [nonzero], mf.f_varint(1, mf.BOOL))
+    wants[nonzero] = a != 0
+    for axis in range(3):
+        out = g.variable("argmax", mf.INT64)
+        g.node("math.ArgMax", [x], [out], mf.f_varint(1, axis) if axis else b"")
+        wants[out] = np.argmax(a, axis=axis, keepdims=True)
+    vector = lambda name, v, dt: g.constant(name, np.array(v, dt), mf.CONSTANT_VECTOR)  # noqa: E731
+    expanded = g.variable("expanded")
+    g.node("base.Expand", [y, vector("shape", [2, 3, 5], np.int64)], [expanded])
+    wants[expanded] = np.broadcast_to(b, (2, 3, 5))
+    tiled = g.variable("tiled")
+    g.node("base.Tile", [x, vector("repeats", [2, 1, 3], np.int32)], [tiled])
+    wants[tiled] = np.tile(a, (2, 1, 3))
+    for o in wants:
+        g.output(o)
+    res = rt.Model(mf.write_model([g], "g")).run({"ids": ids, "x": a, "y": b})
+    for name, want in wants.items():
+        want = np.asarray(want)
+        assert res[name].shape == want.shape, name
+        assert np.array_equal(res[name], want.astype(res[name].dtype)), name
+    for bad, message in (([2, 0, 5], "Expand: invalid shape"),):
+        g = mf.GraphBuilder("g")
+        y = g.input("y", mf.FLOAT, [3, 1])
+        out = g.variable("o")
+        g.node("base.Expand", [y, g.constant("shape", np.array(bad, np.int64), mf.CONSTANT_VECTOR)], [out])
+        g.output(out)
+        with pytest.raises(rt.RuntimeError_, match=message):
+            rt.Model(mf.write_model([g], "g")).run({"y": b})
+    g = mf.GraphBuilder("g")
+    x = g.input("x", mf.FLOAT, [2, 3, 7])
+    out = g.variable("o")
+    g.node("base.Tile", [x, g.constant("repeats", np.array([2, 2], np.int32), mf.CONSTANT_VECTOR)], [out])
+    g.output(out)
+    with pytest.raises(rt.RuntimeError_, match="Tile: repeated error"):
+        rt.Model(mf.write_model([g], "g")).run({"x": a})
 
 
 @pytest.mark.gpu

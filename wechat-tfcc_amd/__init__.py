@@ -136,6 +136,9 @@ SYMBOLS = {
     "tfcc_rocm_copy2d": (_I, [_VP, _VP, _U64, _VP, _U64, _U64, _U64]),
     "tfcc_rocm_gather_rows": (_I, [_VP, _VP, _U, _U64, _VP, _I, _U64, _VP]),
     "tfcc_rocm_cast": (_I, [_VP, _VP, _I, _VP, _I, _U64]),
+    "tfcc_rocm_compare_value": (_I, [_VP, _I, _VP, _I, _U64, _VP, _VP]),
+    "tfcc_rocm_compare": (_I, [_VP, _I, _VP, _VP, _I, _I, C.POINTER(C.c_uint), C.POINTER(_U64), C.POINTER(_U64), _VP]),
+    "tfcc_rocm_argmax_f32": (_I, [_VP, _VP, _U64, _U, _U64, _VP]),
     "tfcc_rocm_lstm_step_f32": (_I, [_VP, _U, _U, _VP, _VP, _VP, _VP, _F, _VP, _VP, _VP]),
     "tfcc_rocm_gru_cell_gates_f32": (_I, [_VP, _U, _U, _U, _VP, _VP, _VP, _VP, _VP]),
     "tfcc_rocm_gru_cell_candidate_f32": (_I, [_VP, _U, _U, _VP, _VP, _VP, _VP, _VP, _VP]),
@@ -838,6 +841,64 @@ def math_binary(op, a, b):
     n = len(dims)
     check(lib().tfcc_rocm_binary_broadcast_f32(_stream(), BINARY_OPS[op], _ptr(a), _ptr(b), n, (C.c_uint * n)(*dims),
                                                (_U64 * n)(*strides(ca)), (_U64 * n)(*strides(cb)), _ptr(out)))
+    return out
+
+
+COMPARE_OPS = {"equal": 0, "unequal": 1, "greater": 2, "greater_equal": 3, "less": 4, "less_equal": 5}
+_C_TYPES = {S8: C.c_int8, U8: C.c_uint8, S16: C.c_int16, U16: C.c_uint16, S32: C.c_int32, U32: C.c_uint32,
+            S64: C.c_int64, U64: C.c_uint64, F32: C.c_float, F64: C.c_double}
+
+
+def compare(op, a, b):
+    """tfcc::relation::equal / unequal / greater / greater_equal / less / less_equal (op in COMPARE_OPS): a tensor
+    against a Python number (compared directly) or against another tensor of the same element type (the difference,
+    taken in the element type with the reference's broadcasting, against 0).  -> uint8 tensor of 0 / 1."""
+    import torch
+    a = a.contiguous()
+    if not isinstance(b, torch.Tensor):
+        if a.numel() == 0:
+            raise InvalidArgumentError("invalid tensor")
+        out = torch.empty(a.shape, dtype=torch.uint8, device=a.device)
+        code = _type_code(a.dtype)
+        value = _C_TYPES[code](b)
+        check(lib().tfcc_rocm_compare_value(_stream(), COMPARE_OPS[op], _ptr(a), code, a.numel(), C.byref(value), _ptr(out)))
+        return out
+    if a.dtype != b.dtype:
+        raise InvalidArgumentError("compare: element types differ")
+    if a.numel() == 0 or b.numel() == 0:
+        raise InvalidArgumentError("invalid tensor")
+    shape, ca, cb = broadcast_shapes(a.shape, b.shape)
+    if len(ca) > 6:
+        raise NotImplementedError("more than six groups of broadcast dimensions")
+    out = torch.empty(shape, dtype=torch.uint8, device=a.device)
+    b = b.contiguous()
+    dims = [max(x, y) for x, y in zip(ca, cb)]
+
+    def strides(c):
+        st, acc = [0] * len(c), 1
+        for d in range(len(c) - 1, -1, -1):
+            st[d] = 0 if c[d] == 1 and dims[d] != 1 else acc
+            acc *= c[d]
+        return st
+    n = len(dims)
+    check(lib().tfcc_rocm_compare(_stream(), COMPARE_OPS[op], _ptr(a), _ptr(b), _type_code(a.dtype), n, (C.c_uint * n)(*dims),
+                                  (_U64 * n)(*strides(ca)), (_U64 * n)(*strides(cb)), _ptr(out)))
+    return out
+
+
+def argmax(a, axis):
+    """tfcc::math::argmax: int64 positions of the first largest element along axis, which stays with length 1."""
+    import torch
+    if a.numel() == 0:
+        raise InvalidArgumentError("invalid tensor")
+    if not 0 <= axis < a.dim():
+        raise InvalidArgumentError("invalid axis")
+    a = a.contiguous()
+    s1, _, s3 = _split_at(a.shape, axis)
+    shape = list(a.shape)
+    shape[axis] = 1
+    out = torch.empty(shape, dtype=torch.int64, device=a.device)
+    check(lib().tfcc_rocm_argmax_f32(_stream(), _ptr(a), s1, a.shape[axis], s3, _ptr(out)))
     return out
 
 

@@ -1,0 +1,216 @@
+// Comparisons and argmax: byte-valued (0 / 1) results of comparing a tensor with a value or with another tensor, and
+// the position of the largest element along one axis.
+//
+//   tensor (x) value    tfcc/mkl/interfaces/tfcc_mklcomparisoninterface.cpp: result[i] = a[i] OP b ? 1 : 0
+//   tensor (x) tensor   tfcc/core/operations/tfcc_relation.cpp:101-115: the operands are subtracted (with numpy-style
+//                       broadcasting) and the difference is compared with 0, in the element type: unsigned
+//                       differences wrap, and inf - inf is not equal to 0.  The difference is formed here in the
+//                       kernel instead of in memory.
+//   argmax              tfcc/mkl/interfaces/tfcc_mklbasicinterface.cpp:469-485: the first position of the largest
+//                       element (a later element wins only if it is greater).
+#include <type_traits>
+
+#include "common.hpp"
+
+namespace tfcc_rocm {
+namespace {
+
+struct CompareShape {
+  unsigned dims[6];
+  unsigned long long strideA[6], strideB[6];
+  int rank;
+};
+
+template <class T>
+__device__ __forceinline__ unsigned char compare_value(int op, T x, T y) {
+  switch (op) {
+    case TFCC_ROCM_COMPARE_EQUAL: return x == y;
+    case TFCC_ROCM_COMPARE_UNEQUAL: return x != y;
+    case TFCC_ROCM_COMPARE_GREATER: return x > y;
+    case TFCC_ROCM_COMPARE_GREATER_EQUAL: return x >= y;
+    case TFCC_ROCM_COMPARE_LESS: return x < y;
+    default: return x <= y;
+  }
+}
+
+// a - b in T: integers wrap (computed unsigned), floating-point types subtract
+template <class T>
+__device__ __forceinline__ T difference(T x, T y) {
+  if constexpr (std::is_floating_point<T>::value) {
+    return x - y;
+  } else {
+    using U = typename std::make_unsigned<T>::type;
+    return static_cast<T>(static_cast<U>(static_cast<U>(x) - static_cast<U>(y)));
+  }
+}
+
+template <class T>
+__global__ __launch_bounds__(256) void compare_value_kernel(int op, const T* a, size_t total, T value,
+                                                            unsigned char* out) {
+  const size_t step = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += step) out[i] = compare_value<T>(op, a[i], value);
+}
+
+template <class T>
+__global__ __launch_bounds__(256) void compare_tensors_kernel(int op, const T* a, const T* b, size_t total,
+                                                              CompareShape p, unsigned char* out) {
+  const size_t step = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += step) {
+    size_t rem = i, ia = 0, ib = 0;
+    for (int d = p.rank - 1; d >= 0; --d) {
+      const size_t c = rem % p.dims[d];
+      rem /= p.dims[d];
+      ia += c * p.strideA[d];
+      ib += c * p.strideB[d];
+    }
+    out[i] = compare_value<T>(op, difference<T>(a[ia], b[ib]), T(0));
+  }
+}
+
+// one thread per (outer, inner) pair walks the axis; neighbouring threads read neighbouring inner positions
+__global__ __launch_bounds__(256) void argmax_kernel(const float* a, size_t outer, unsigned length, size_t inner,
+                                                     long long* out) {
+  const size_t total = outer * inner;
+  const size_t step = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += step) {
+    const size_t x = i / inner, z = i - x * inner;
+    const float* p = a + x * length * inner + z;
+    float best = p[0];
+    long long index = 0;
+    for (unsigned y = 1; y < length; ++y) {
+      const float v = p[(size_t)y * inner];
+      if (v > best) {
+        best = v;
+        index = y;
+      }
+    }
+    out[i] = index;
+  }
+}
+
+// the last axis: one wavefront per row, lanes stride the row, then the lanes' (value, first index) pairs are joined
+__global__ __launch_bounds__(256) void argmax_rows_kernel(const float* a, size_t rows, unsigned length, long long* out) {
+  const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const unsigned lane = threadIdx.x & 63;
+  const float* p = a + row * length;
+  // every lane starts from the row's first element, as the scalar loop does: a NaN there stays (nothing is greater),
+  // a NaN elsewhere is never taken
+  float best = p[0];
+  unsigned index = 0;
+  for (unsigned y = lane; y < length; y += 64) {
+    const float v = p[y];
+    if (v > best) {
+      best = v;
+      index = y;
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float ob = __shfl_xor(best, off, 64);
+    const unsigned oi = __shfl_xor(index, off, 64);
+    // the greater value wins; of equal values the smaller position
+    if (ob > best || (!(best > ob) && oi < index)) {
+      best = ob;
+      index = oi;
+    }
+  }
+  if (lane == 0) out[row] = index;
+}
+
+unsigned grid_of(size_t total) {
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  return (unsigned)(blocks ? blocks : 1);
+}
+
+template <class T>
+int launch_compare_value(hipStream_t s, int op, const void* a, size_t total, const void* value, unsigned char* out) {
+  hipLaunchKernelGGL(compare_value_kernel<T>, dim3(grid_of(total)), dim3(256), 0, s, op, static_cast<const T*>(a), total,
+                     *static_cast<const T*>(value), out);
+  return check_launch("compare_value");
+}
+
+template <class T>
+int launch_compare_tensors(hipStream_t s, int op, const void* a, const void* b, size_t total, const CompareShape& p,
+                           unsigned char* out) {
+  hipLaunchKernelGGL(compare_tensors_kernel<T>, dim3(grid_of(total)), dim3(256), 0, s, op, static_cast<const T*>(a),
+                     static_cast<const T*>(b), total, p, out);
+  return check_launch("compare");
+}
+
+}  // namespace
+}  // namespace tfcc_rocm
+
+using namespace tfcc_rocm;
+
+#define TFCC_FOR_ELEMENT_TYPES(CALL)          \
+  CALL(TFCC_ROCM_S8, signed char)             \
+  CALL(TFCC_ROCM_U8, unsigned char)           \
+  CALL(TFCC_ROCM_S16, short)                  \
+  CALL(TFCC_ROCM_U16, unsigned short)         \
+  CALL(TFCC_ROCM_S32, int)                    \
+  CALL(TFCC_ROCM_U32, unsigned)               \
+  CALL(TFCC_ROCM_S64, long long)              \
+  CALL(TFCC_ROCM_U64, unsigned long long)     \
+  CALL(TFCC_ROCM_F32, float)                  \
+  CALL(TFCC_ROCM_F64, double)
+
+extern "C" {
+
+int tfcc_rocm_compare_value(void* stream, int op, const void* a, int type, uint64_t total, const void* value,
+                            uint8_t* out) {
+  TFCC_REQUIRE(a && value && out, "compare_value: null argument");
+  TFCC_REQUIRE(total > 0, "compare_value: empty tensor");
+  TFCC_REQUIRE(op >= TFCC_ROCM_COMPARE_EQUAL && op <= TFCC_ROCM_COMPARE_LESS_EQUAL, "compare_value: unknown operation %d", op);
+  hipStream_t s = as_stream(stream);
+#define TFCC_COMPARE_CASE(CODE, T) \
+  case CODE: return launch_compare_value<T>(s, op, a, (size_t)total, value, out);
+  switch (type) {
+    TFCC_FOR_ELEMENT_TYPES(TFCC_COMPARE_CASE)
+    default: return set_error(TFCC_ROCM_INVALID_ARGUMENT, "compare_value: unknown element type %d", type);
+  }
+#undef TFCC_COMPARE_CASE
+}
+
+int tfcc_rocm_compare(void* stream, int op, const void* a, const void* b, int type, int rank, const unsigned* dims,
+                      const uint64_t* stride_a, const uint64_t* stride_b, uint8_t* out) {
+  TFCC_REQUIRE(a && b && out && dims && stride_a && stride_b, "compare: null argument");
+  TFCC_REQUIRE(op >= TFCC_ROCM_COMPARE_EQUAL && op <= TFCC_ROCM_COMPARE_LESS_EQUAL, "compare: unknown operation %d", op);
+  TFCC_REQUIRE(rank >= 1 && rank <= 6, "compare: rank %d (1..6)", rank);
+  CompareShape p{};
+  p.rank = rank;
+  size_t total = 1;
+  for (int d = 0; d < rank; ++d) {
+    TFCC_REQUIRE(dims[d] > 0, "compare: empty tensor");
+    p.dims[d] = dims[d];
+    p.strideA[d] = stride_a[d];
+    p.strideB[d] = stride_b[d];
+    total *= dims[d];
+  }
+  hipStream_t s = as_stream(stream);
+#define TFCC_COMPARE_CASE(CODE, T) \
+  case CODE: return launch_compare_tensors<T>(s, op, a, b, total, p, out);
+  switch (type) {
+    TFCC_FOR_ELEMENT_TYPES(TFCC_COMPARE_CASE)
+    default: return set_error(TFCC_ROCM_INVALID_ARGUMENT, "compare: unknown element type %d", type);
+  }
+#undef TFCC_COMPARE_CASE
+}
+
+int tfcc_rocm_argmax_f32(void* stream, const float* in, uint64_t outer, unsigned length, uint64_t inner, int64_t* out) {
+  TFCC_REQUIRE(in && out, "argmax: null argument");
+  TFCC_REQUIRE(outer > 0 && length > 0 && inner > 0, "argmax: empty tensor");
+  TFCC_REQUIRE(outer * inner < (1ull << 40), "argmax: too many positions");
+  hipStream_t s = as_stream(stream);
+  if (inner == 1 && length >= 64 && outer < (1ull << 31)) {
+    hipLaunchKernelGGL(argmax_rows_kernel, dim3((unsigned)((outer + 3) / 4)), dim3(256), 0, s, in, (size_t)outer, length,
+                       reinterpret_cast<long long*>(out));
+  } else {
+    hipLaunchKernelGGL(argmax_kernel, dim3(grid_of((size_t)(outer * inner))), dim3(256), 0, s, in, (size_t)outer, length,
+                       (size_t)inner, reinterpret_cast<long long*>(out));
+  }
+  return check_launch("argmax");
+}
+
+}  // extern "C"

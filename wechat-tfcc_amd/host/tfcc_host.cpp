@@ -745,6 +745,20 @@ class ROCMBasicInterface : public BasicInterface<T> {
       throw NotImplementedError("clip: float tensors only");
     }
   }
+  Variable<int64_t> argmax(const Tensor<T>& a, size_t axis) override {
+    if constexpr (std::is_same<T, float>::value) {
+      std::vector<unsigned> shape = a.shape().toVector();
+      uint64_t s1, s3;
+      split_at(a.shape(), axis, s1, s3);
+      const unsigned length = shape[axis];
+      shape[axis] = 1;
+      Variable<int64_t> r{Shape(shape)};
+      check(tfcc_rocm_argmax_f32(current_stream(), a.data(), s1, length, s3, r.data()));
+      return r;
+    } else {
+      throw NotImplementedError("argmax: float tensors only");
+    }
+  }
   Variable<T> gather(const Tensor<T>& params, const void* indices, int indexCode, const Shape& indexShape) override {
     std::vector<unsigned> shape = indexShape.toVector();
     for (size_t i = 1; i < params.shape().size(); ++i) shape.push_back(params.shape(i));
@@ -873,7 +887,40 @@ class ROCMTransformationInterface : public TransformationInterface<float> {
 };
 
 template <class T>
+class ROCMComparisonInterface : public ComparisonInterface<T> {
+ public:
+  Variable<uint8_t> compare(const Tensor<T>& a, T b, Relation r) override {
+    Variable<uint8_t> result(a.shape());
+    check(tfcc_rocm_compare_value(current_stream(), static_cast<int>(r), a.data(), ElementCode<T>::value, a.size(), &b,
+                                  result.data()));
+    return result;
+  }
+  Variable<uint8_t> compareDifference(const Tensor<T>& a, const Tensor<T>& b, Relation r) override {
+    const size_t rank = a.shape().size();
+    if (rank == 0 || rank != b.shape().size()) throw InvalidArgumentError("invalid tensor shape");
+    if (rank > 6) throw NotImplementedError("comparison: more than six groups of broadcast dimensions");
+    std::vector<unsigned> dims(rank);
+    for (size_t d = 0; d < rank; ++d) {
+      if (a.shape(d) != b.shape(d) && a.shape(d) != 1 && b.shape(d) != 1) throw InvalidArgumentError("broadcast failed");
+      dims[d] = std::max(a.shape(d), b.shape(d));
+    }
+    Variable<uint8_t> result{Shape(dims)};
+    uint64_t sa[6], sb[6], accA = 1, accB = 1;
+    for (size_t d = rank; d-- > 0;) {
+      sa[d] = a.shape(d) == 1 && dims[d] != 1 ? 0 : accA;
+      sb[d] = b.shape(d) == 1 && dims[d] != 1 ? 0 : accB;
+      accA *= a.shape(d);
+      accB *= b.shape(d);
+    }
+    check(tfcc_rocm_compare(current_stream(), static_cast<int>(r), a.data(), b.data(), ElementCode<T>::value,
+                            static_cast<int>(rank), dims.data(), sa, sb, result.data()));
+    return result;
+  }
+};
+
+template <class T>
 void install_common(Interface<T>& i) {
+  i.setComparisonInterface(std::unique_ptr<ComparisonInterface<T>>(new ROCMComparisonInterface<T>()));
   i.setDataInterface(std::unique_ptr<DataInterface<T>>(new ROCMDataInterface<T>()));
   i.setBasicInterface(std::unique_ptr<BasicInterface<T>>(new ROCMBasicInterface<T>()));
 }

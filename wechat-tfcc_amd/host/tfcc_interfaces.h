@@ -122,6 +122,7 @@ class BasicInterface {
   virtual Variable<T> concat(const std::vector<const Tensor<T>*>&, size_t) { throw NotImplementedError(); }
   // rows of params by index (tfcc/core/interfaces/tfcc_gatherinterface.h): indices of the type with code indexCode
   virtual Variable<T> clip(const Tensor<T>&, T, T) { throw NotImplementedError(); }
+  virtual Variable<int64_t> argmax(const Tensor<T>&, size_t) { throw NotImplementedError(); }
   virtual Variable<T> gather(const Tensor<T>&, const void* /*indices*/, int /*indexCode*/, const Shape& /*indexShape*/) {
     throw NotImplementedError();
   }
@@ -135,6 +136,26 @@ class ArithmeticInterface {
   virtual Variable<T> sub(const Tensor<T>&, const Tensor<T>&) { throw NotImplementedError(); }
   virtual Variable<T> mul(const Tensor<T>&, const Tensor<T>&) { throw NotImplementedError(); }
   virtual Variable<T> div(const Tensor<T>&, const Tensor<T>&) { throw NotImplementedError(); }
+};
+
+// tfcc/core/interfaces/tfcc_comparisoninterface.h:27-83: tensor against value, byte results (1 where the relation
+// holds).  compareDifference is an addition: (a - b) against 0 for two tensors of equal rank with broadcast
+// dimensions, which tfcc::relation's tensor-tensor forms otherwise compose from a subtraction in memory and a
+// comparison with 0 (tfcc/core/operations/tfcc_relation.cpp:101-115).
+enum class Relation { EQUAL = 0, UNEQUAL, GREATER, GREATER_EQUAL, LESS, LESS_EQUAL };
+
+template <class T>
+class ComparisonInterface {
+ public:
+  virtual ~ComparisonInterface() {}
+  virtual Variable<uint8_t> compare(const Tensor<T>&, T, Relation) { throw NotImplementedError(); }
+  virtual Variable<uint8_t> compareDifference(const Tensor<T>&, const Tensor<T>&, Relation) { throw NotImplementedError(); }
+  Variable<uint8_t> equal(const Tensor<T>& a, T b) { return compare(a, b, Relation::EQUAL); }
+  Variable<uint8_t> unequal(const Tensor<T>& a, T b) { return compare(a, b, Relation::UNEQUAL); }
+  Variable<uint8_t> greater(const Tensor<T>& a, T b) { return compare(a, b, Relation::GREATER); }
+  Variable<uint8_t> greaterEqual(const Tensor<T>& a, T b) { return compare(a, b, Relation::GREATER_EQUAL); }
+  Variable<uint8_t> less(const Tensor<T>& a, T b) { return compare(a, b, Relation::LESS); }
+  Variable<uint8_t> lessEqual(const Tensor<T>& a, T b) { return compare(a, b, Relation::LESS_EQUAL); }
 };
 
 // tfcc/core/interfaces/tfcc_minmaxinterface.h:30-68
@@ -225,6 +246,7 @@ class Interface {
   TFCC_SUB_INTERFACE(Cell)
   TFCC_SUB_INTERFACE(MinMax)
   TFCC_SUB_INTERFACE(Reduce)
+  TFCC_SUB_INTERFACE(Comparison)
 #undef TFCC_SUB_INTERFACE
 };
 
@@ -541,6 +563,13 @@ Variable<T> clip(const Tensor<T>& a, T minValue, T maxValue) {
   if (a.size() == 0) throw InvalidArgumentError("invalid tensor");
   return Operation<T>::getCurrentInterface().getBasicInterface().clip(a, minValue, maxValue);
 }
+// tfcc::math::argmax (tfcc/core/operations/tfcc_math.cpp:675-684): the axis stays with length 1
+template <class T>
+Variable<int64_t> argmax(const Tensor<T>& a, size_t axis) {
+  if (a.size() == 0) throw InvalidArgumentError("invalid tensor");
+  if (axis >= a.shape().size()) throw InvalidArgumentError("invalid axis");
+  return Operation<T>::getCurrentInterface().getBasicInterface().argmax(a, axis);
+}
 // tfcc::math::reduce_sum / mean / prod / max / min (tfcc/core/operations/tfcc_math.cpp:464-522)
 #define TFCC_REDUCE_FUNCTION(NAME, METHOD)                                                   \
   template <class T>                                                                         \
@@ -565,6 +594,55 @@ Variable<T> transform2(const Tensor<T>& a, T alpha, T beta) {
 }
 
 }  // namespace math
+
+// tfcc::relation (tfcc/core/operations/tfcc_relation.cpp:81-300): tensor against value, value against tensor (the
+// mirrored relation on the tensor) and tensor against tensor (the difference against 0, with broadcasting).
+namespace relation {
+namespace detail {
+inline Relation mirrored(Relation r) {
+  switch (r) {
+    case Relation::GREATER: return Relation::LESS;
+    case Relation::GREATER_EQUAL: return Relation::LESS_EQUAL;
+    case Relation::LESS: return Relation::GREATER;
+    case Relation::LESS_EQUAL: return Relation::GREATER_EQUAL;
+    default: return r;
+  }
+}
+}  // namespace detail
+template <class T>
+Variable<uint8_t> compare(const Tensor<T>& a, T b, Relation r) {
+  if (a.size() == 0) throw InvalidArgumentError();
+  return Operation<T>::getCurrentInterface().getComparisonInterface().compare(a, b, r);
+}
+template <class T>
+Variable<uint8_t> compare(T a, const Tensor<T>& b, Relation r) {
+  return compare(b, a, detail::mirrored(r));
+}
+template <class T>
+Variable<uint8_t> compare(const Tensor<T>& a, const Tensor<T>& b, Relation r) {
+  if (a.size() == 0 || b.size() == 0) throw InvalidArgumentError();
+  Shape resultS, newAS, newBS;
+  std::tie(resultS, newAS, newBS) = math::detail::broadcast_shapes(a.shape(), b.shape());
+  View<T> aView(a, newAS), bView(b, newBS);
+  Variable<uint8_t> result = Operation<T>::getCurrentInterface().getComparisonInterface().compareDifference(aView, bView, r);
+  result.reshape(std::move(resultS));
+  return result;
+}
+#define TFCC_RELATION_FUNCTION(NAME, VALUE)                                                          \
+  template <class T>                                                                                 \
+  Variable<uint8_t> NAME(const Tensor<T>& a, T b) { return compare(a, b, Relation::VALUE); }         \
+  template <class T>                                                                                 \
+  Variable<uint8_t> NAME(T a, const Tensor<T>& b) { return compare(a, b, Relation::VALUE); }         \
+  template <class T>                                                                                 \
+  Variable<uint8_t> NAME(const Tensor<T>& a, const Tensor<T>& b) { return compare(a, b, Relation::VALUE); }
+TFCC_RELATION_FUNCTION(equal, EQUAL)
+TFCC_RELATION_FUNCTION(unequal, UNEQUAL)
+TFCC_RELATION_FUNCTION(greater, GREATER)
+TFCC_RELATION_FUNCTION(greater_equal, GREATER_EQUAL)
+TFCC_RELATION_FUNCTION(less, LESS)
+TFCC_RELATION_FUNCTION(less_equal, LESS_EQUAL)
+#undef TFCC_RELATION_FUNCTION
+}  // namespace relation
 
 namespace nn {
 

@@ -389,6 +389,188 @@ class LeakyRelu : public TypedOperation<T> {
   }
 };
 
+// ---- relation.Equal / UnEqual / Greater / GreaterOrEqual / Less / LessOrEqual / Not --------------------------
+// Inputs of one element type, a BOOL result; tensor and value operands in the four combinations
+// (tfcc_runtime/operations/relation/equal.cpp:83-133 and its siblings).  Not: BOOL -> BOOL, a tensor or a value
+// (relation/not_.cpp:53-88).
+template <Relation R, class T>
+class Compare : public TypedOperation<T> {
+  static const char* message() {
+    switch (R) {
+      case Relation::EQUAL: return "relation.Equal";
+      case Relation::UNEQUAL: return "relation.UnEqual";
+      case Relation::GREATER: return "relation.Greater";
+      case Relation::GREATER_EQUAL: return "relation.GreaterOrEqual";
+      case Relation::LESS: return "relation.Less";
+      default: return "relation.LessOrEqual";
+    }
+  }
+  static uint8_t vv(T a, T b) {
+    switch (R) {
+      case Relation::EQUAL: return a == b;
+      case Relation::UNEQUAL: return a != b;
+      case Relation::GREATER: return a > b;
+      case Relation::GREATER_EQUAL: return a >= b;
+      case Relation::LESS: return a < b;
+      default: return a <= b;
+    }
+  }
+
+ public:
+  Compare() : TypedOperation<T>(message()) {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 2 || node.outputs.size() != 1) return false;
+    if (!same_dtype(graph, node.outputs, BOOL) || !same_dtype(graph, node.inputs, this->DTYPE)) return false;
+    auto& sm = graph.getSymbolManager();
+    const SymbolType s0 = stype_of(graph, node.inputs[0]), s1 = stype_of(graph, node.inputs[1]);
+    if (is_tensor(s0) && is_tensor(s1)) {
+      const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+      const Tensor<T>* b = sm.getTensor(node.inputs[1], T());
+      Variable<uint8_t>* out = sm.getVariable(node.outputs[0], uint8_t());
+      graph.addStep([a, b, out] { *out = relation::compare(*a, *b, R); });
+    } else if (is_tensor(s0) && is_value(s1)) {
+      const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+      const T* b = sm.getValue(node.inputs[1], T());
+      Variable<uint8_t>* out = sm.getVariable(node.outputs[0], uint8_t());
+      graph.addStep([a, b, out] { *out = relation::compare(*a, *b, R); });
+    } else if (is_value(s0) && is_tensor(s1)) {
+      const T* a = sm.getValue(node.inputs[0], T());
+      const Tensor<T>* b = sm.getTensor(node.inputs[1], T());
+      Variable<uint8_t>* out = sm.getVariable(node.outputs[0], uint8_t());
+      graph.addStep([a, b, out] { *out = relation::compare(*a, *b, R); });
+    } else if (is_value(s0) && is_value(s1)) {
+      const T* a = sm.getValue(node.inputs[0], T());
+      const T* b = sm.getValue(node.inputs[1], T());
+      uint8_t* out = sm.getValue(node.outputs[0], uint8_t());
+      graph.addStep([a, b, out] { *out = vv(*a, *b); });
+    } else {
+      return false;
+    }
+    return true;
+  }
+};
+
+class Not : public Operation {
+ public:
+  std::string getOperationTypeUrl() const override { return type_url("relation.Not"); }
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 1 || node.outputs.size() != 1) return false;
+    if (!same_dtype(graph, node.outputs, BOOL) || !same_dtype(graph, node.inputs, BOOL)) return false;
+    auto& sm = graph.getSymbolManager();
+    const SymbolType si = stype_of(graph, node.inputs[0]);
+    if (is_tensor(si)) {
+      const Tensor<uint8_t>* a = sm.getTensor(node.inputs[0], uint8_t());
+      Variable<uint8_t>* out = sm.getVariable(node.outputs[0], uint8_t());
+      graph.addStep([a, out] { *out = relation::equal(*a, static_cast<uint8_t>(0)); });
+      return true;
+    }
+    if (is_value(si)) {
+      const uint8_t* a = sm.getValue(node.inputs[0], uint8_t());
+      uint8_t* out = sm.getValue(node.outputs[0], uint8_t());
+      graph.addStep([a, out] { *out = *a == 0; });
+      return true;
+    }
+    return false;
+  }
+};
+
+// ---- math.ArgMax: int64 positions along `axis`, which stays with length 1 (math/argmax.cpp:27-38) ----------
+template <class T>
+class ArgMax : public TypedOperation<T> {
+ public:
+  ArgMax() : TypedOperation<T>("math.ArgMax") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 1 || node.outputs.size() != 1) return false;
+    if (!same_dtype(graph, node.outputs, DataTypeOf<int64_t>::value) || !same_dtype(graph, node.inputs, this->DTYPE)) return false;
+    size_t axis = 0;
+    wire::Reader r(node.operation);
+    uint32_t f, t;
+    while (r.next(f, t)) {
+      if (f == 1 && t == 0) axis = static_cast<size_t>(r.varint());
+      else r.skip(t);
+    }
+    auto& sm = graph.getSymbolManager();
+    const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+    Variable<int64_t>* out = sm.getVariable(node.outputs[0], int64_t());
+    graph.addStep([a, out, axis] { *out = math::argmax(*a, axis); });
+    return true;
+  }
+};
+
+// ---- base.Expand (tensor, shape vector) and base.Tile (tensor, repeats vector) ------------------------------
+// Broadcasting does the work: Expand adds zeros of the wanted shape to the input (base/expand.cpp:28-47); Tile views
+// the input as [1, s0, 1, s1, ...], multiplies it by ones of [r0, s0, r1, s1, ...] and views the product as
+// [r0 * s0, r1 * s1, ...] (base/tile.cpp:28-62).
+template <class T, class IDX>
+class Expand : public TypedOperation<T> {
+ public:
+  Expand() : TypedOperation<T>("base.Expand") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if constexpr (!std::is_integral<IDX>::value || sizeof(IDX) < 4) {
+      return false;
+    } else {
+      if (node.inputs.size() != 2 || node.outputs.size() != 1) return false;
+      auto& sm = graph.getSymbolManager();
+      if (sm.getSymbolInfo(node.outputs[0]).dtype != this->DTYPE || sm.getSymbolInfo(node.inputs[0]).dtype != this->DTYPE)
+        return false;
+      if (sm.getSymbolInfo(node.inputs[1]).dtype != DataTypeOf<IDX>::value) return false;
+      const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+      const std::vector<IDX>* shape = sm.getVector(node.inputs[1], IDX());
+      Variable<T>* out = sm.getVariable(node.outputs[0], T());
+      graph.addStep([a, shape, out] {
+        std::vector<unsigned> real(shape->size());
+        for (size_t i = 0; i < shape->size(); ++i) {
+          if ((*shape)[i] <= 0) throw RuntimeError("Expand: invalid shape");
+          real[i] = static_cast<unsigned>((*shape)[i]);
+        }
+        Variable<T> zeros{Shape(real)};
+        data::zeros(zeros);
+        *out = *a + zeros;
+      });
+      return true;
+    }
+  }
+};
+
+template <class T, class IDX>
+class Tile : public TypedOperation<T> {
+ public:
+  Tile() : TypedOperation<T>("base.Tile") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if constexpr (!std::is_integral<IDX>::value || sizeof(IDX) < 4) {
+      return false;
+    } else {
+      if (node.inputs.size() != 2 || node.outputs.size() != 1) return false;
+      auto& sm = graph.getSymbolManager();
+      if (sm.getSymbolInfo(node.outputs[0]).dtype != this->DTYPE || sm.getSymbolInfo(node.inputs[0]).dtype != this->DTYPE)
+        return false;
+      if (sm.getSymbolInfo(node.inputs[1]).dtype != DataTypeOf<IDX>::value) return false;
+      const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+      const std::vector<IDX>* repeats = sm.getVector(node.inputs[1], IDX());
+      Variable<T>* out = sm.getVariable(node.outputs[0], T());
+      graph.addStep([a, repeats, out] {
+        if (repeats->size() != a->shape().size()) throw RuntimeError("Tile: repeated error");
+        std::vector<unsigned> target = a->shape().toVector(), viewed, onesShape;
+        for (size_t i = 0; i < repeats->size(); ++i) {
+          if ((*repeats)[i] <= 0) throw RuntimeError("Tile: repeated error");
+          const unsigned r = static_cast<unsigned>((*repeats)[i]);
+          viewed.push_back(1);
+          viewed.push_back(target[i]);
+          onesShape.push_back(r);
+          onesShape.push_back(target[i]);
+          target[i] *= r;
+        }
+        View<T> spread(*a, Shape(viewed));
+        Variable<T> ones{Shape(onesShape)};
+        data::ones(ones);
+        *out = spread * ones;
+        out->reshape(Shape(target));
+      });
+      return true;
+    }
+  }
+};
+
 // ---- nn.LayerNormalization --------------------------------------------------------------------------------
 template <class T>
 class LayerNormalization : public TypedOperation<T> {
@@ -636,7 +818,12 @@ class Cast : public TypedOperation<SRC> {
     auto& sm = graph.getSymbolManager();
     const SymbolInfo& in = sm.getSymbolInfo(node.inputs[0]);
     const SymbolInfo& outInfo = sm.getSymbolInfo(node.outputs[0]);
-    if (outInfo.dtype != DataTypeOf<DST>::value || in.dtype != this->DTYPE) return false;
+    // BOOL symbols live in bytes: a BOOL source converts like uint8, a BOOL result is 1 where the source is not 0
+    // (tfcc_runtime/operations/base/cast.cpp:58-79)
+    const bool fromBool = std::is_same<SRC, uint8_t>::value && in.dtype == BOOL;
+    const bool toBool = std::is_same<DST, uint8_t>::value && outInfo.dtype == BOOL;
+    if (in.dtype != this->DTYPE && !fromBool) return false;
+    if (outInfo.dtype != DataTypeOf<DST>::value && !toBool) return false;
     uint64_t wanted = 0;
     wire::Reader r(node.operation);
     uint32_t f, t;
@@ -644,7 +831,21 @@ class Cast : public TypedOperation<SRC> {
       if (f == 1 && t == 0) wanted = r.varint();
       else r.skip(t);
     }
-    if (wanted != static_cast<uint64_t>(DataTypeOf<DST>::value)) return false;
+    if (wanted != static_cast<uint64_t>(outInfo.dtype)) return false;
+    if (toBool) {
+      if (is_tensor(in.stype) && is_tensor(outInfo.stype)) {
+        const Tensor<SRC>* a = sm.getTensor(node.inputs[0], SRC());
+        Variable<uint8_t>* out = sm.getVariable(node.outputs[0], uint8_t());
+        graph.addStep([a, out] { *out = relation::unequal(*a, static_cast<SRC>(0)); });
+      } else if (is_value(in.stype) && is_value(outInfo.stype)) {
+        const SRC* a = sm.getValue(node.inputs[0], SRC());
+        uint8_t* out = sm.getValue(node.outputs[0], uint8_t());
+        graph.addStep([a, out] { *out = *a ? 1 : 0; });
+      } else {
+        return false;
+      }
+      return true;
+    }
     if (is_tensor(in.stype) && is_tensor(outInfo.stype)) {
       const Tensor<SRC>* a = sm.getTensor(node.inputs[0], SRC());
       Variable<DST>* out = sm.getVariable(node.outputs[0], DST());
@@ -1115,6 +1316,13 @@ class Collector {
     add(new Reduce<Reduction::MAX, T>());
     add(new Reduce<Reduction::MIN, T>());
     add(new Clip<T>());
+    add(new Compare<Relation::EQUAL, T>());
+    add(new Compare<Relation::UNEQUAL, T>());
+    add(new Compare<Relation::GREATER, T>());
+    add(new Compare<Relation::GREATER_EQUAL, T>());
+    add(new Compare<Relation::LESS, T>());
+    add(new Compare<Relation::LESS_EQUAL, T>());
+    add(new ArgMax<T>());
     add(new LeakyRelu<T>());
     add(new Gelu<T>());
     add(new Unary<UnaryFunction::SIGMOID, T>());
@@ -1159,7 +1367,9 @@ class Collector {
   add(new SliceV1<T, OTHER>());         \
   add(new At<T, OTHER>());              \
   add(new SliceV2<T, OTHER>());         \
-  add(new Pad<T, OTHER>());
+  add(new Pad<T, OTHER>());             \
+  add(new Expand<T, OTHER>());          \
+  add(new Tile<T, OTHER>());
     TFCC_RUNTIME_FOR_ALL_TYPES(TFCC_RUNTIME_ADD_PAIR)
 #undef TFCC_RUNTIME_ADD_PAIR
 #define TFCC_RUNTIME_ADD_DIMENSION(DST, E) add(new GetDimension<T, DST>());
@@ -1172,6 +1382,7 @@ class Collector {
 #define TFCC_RUNTIME_ADD(T, E) addForType<T>();
     TFCC_RUNTIME_FOR_ALL_TYPES(TFCC_RUNTIME_ADD)
 #undef TFCC_RUNTIME_ADD
+    add(new Not());
   }
   const std::vector<std::unique_ptr<Operation>>& get(const std::string& url) const {
     static const std::vector<std::unique_ptr<Operation>> empty;
