@@ -343,6 +343,14 @@ int tfcc_rocm_reduce_f32(void* stream, int op, const float* in, uint64_t rows, u
 /* min(max(v, lo), hi) (tfcc::math::clip) and v > 0 ? v : v * alpha (tfcc::math::leaky_relu) */
 int tfcc_rocm_clip_f32(void* stream, const float* in, uint64_t total, float lo, float hi, float* out);
 int tfcc_rocm_leaky_relu_f32(void* stream, const float* in, uint64_t total, float alpha, float* out);
+/* out[i] = condition[i] != 0 ? x[i] : y[i] on elements of element_bytes (1, 2, 4, 8) bytes; a null x (or y) stands
+ * for one value, the low element_bytes of x_bits (y_bits) (tfcc/mkl/interfaces/tfcc_mklbasicinterface.cpp:398-422). */
+int tfcc_rocm_where(void* stream, const uint8_t* condition, const void* x, uint64_t x_bits, const void* y,
+                    uint64_t y_bits, unsigned element_bytes, uint64_t total, void* out);
+/* tril (upper == 0: row r keeps columns c < r + k + 1) or triu (c >= r + k) of a [rows, cols] matrix, zeros elsewhere
+ * (tfcc/mkl/interfaces/tfcc_mklbasicinterface.cpp:433-466). */
+int tfcc_rocm_triangle(void* stream, const void* in, uint64_t rows, uint64_t cols, int64_t k, int upper,
+                       unsigned element_bytes, void* out);
 /* Comparisons with byte results (1 where the relation holds, else 0) for every element type (TFCC_ROCM_S8 .. F64).
  * compare_value: a[i] OP *value, value a host pointer to one element of the tensor's type
  * (tfcc/core/interfaces/tfcc_comparisoninterface.h:38-83).  compare: (a - b) OP 0 with numpy-style broadcasting given as

@@ -655,6 +655,28 @@ def test_comparisons_and_argmax(pkg, T):
         pkg.argmax(T.t(x), 2)
 
 
+def test_where_and_triangles(pkg, T):
+    """tfcc::nn::where with tensor / value operands and tfcc::base::tril / triu
+    (tfcc/mkl/interfaces/tfcc_mklbasicinterface.cpp:398-466) against numpy, on several element types."""
+    rng = np.random.default_rng(59)
+    for dtype in (np.float32, np.int64, np.uint8, np.int16, np.float64):
+        cond = rng.integers(0, 3, (3, 5, 17)).astype(np.uint8)
+        x = rng.integers(-50, 50, cond.shape).astype(dtype)
+        y = rng.integers(-50, 50, cond.shape).astype(dtype)
+        assert np.array_equal(T.n(pkg.where(T.t(cond), T.t(x), T.t(y))), np.where(cond != 0, x, y))
+        assert np.array_equal(T.n(pkg.where(T.t(cond), 7, T.t(y))), np.where(cond != 0, dtype(7), y))
+        assert np.array_equal(T.n(pkg.where(T.t(cond), T.t(x), 9)), np.where(cond != 0, x, dtype(9)))
+        for rows, cols in ((5, 5), (3, 9), (9, 3), (1, 1)):
+            m = rng.integers(1, 50, (rows, cols)).astype(dtype)
+            for k in (0, 1, -1, 4, -4, 100, -100):
+                assert np.array_equal(T.n(pkg.triangle(T.t(m), k, False)), np.tril(m, k)), (rows, cols, k)
+                assert np.array_equal(T.n(pkg.triangle(T.t(m), k, True)), np.triu(m, k)), (rows, cols, k)
+    with pytest.raises(pkg.InvalidArgumentError, match="different shape"):
+        pkg.where(T.t(np.zeros((2, 3), np.uint8)), T.t(np.zeros((3, 2), np.float32)), 1.0)
+    with pytest.raises(pkg.InvalidArgumentError, match="invalid shape"):
+        pkg.triangle(T.t(np.zeros((2, 3, 4), np.float32)), 0, True)
+
+
 BROADCAST_PAIRS = [
     ((2, 4, 8, 8), (2, 1, 1, 8)),        # attention scores + mask
     ((3, 1, 5), (1, 4, 1)),              # both sides broadcast

@@ -784,6 +784,68 @@ def test_relation_argmax_expand_tile_nodes_equal_numpy(mf, rt, dev):
 
 
 @pytest.mark.gpu
+def test_where_triangle_create_tensor_range_nodes_equal_numpy(mf, rt, dev):
+    """nn.Where with tensor / value operands, base.Tril / Triu with the diagonal in the node, base.CreateTensor (shape
+    vector in, value and type in the node) and base.Range (three values -> a vector, here turned into a tensor):
+    tfcc_runtime/operations/nn/where.cpp, base/tril.cpp, triu.cpp, createtensor.cpp, range.cpp.  A causal mask is
+    built from them: Tril of ones -> Equal 0 -> Where(-10000, 0)."""
+    rng = np.random.default_rng(61)
+    a = rng.normal(size=(6, 6)).astype(np.float32)
+    b = rng.normal(size=(6, 6)).astype(np.float32)
+    g = mf.GraphBuilder("g")
+    x = g.input("x", mf.FLOAT, [6, 6])
+    y = g.input("y", mf.FLOAT, [6, 6])
+    value = lambda name, v, dt=np.float32: g.constant(name, np.array(v, dt), mf.CONSTANT_VALUE)  # noqa: E731
+    wants = {}
+    positive = g.variable("positive", mf.BOOL)
+    g.node("relation.Greater", [x, value("zero", 0.0)], [positive])
+    for name, ins, want in (("tt", [positive, x, y], np.where(a > 0, a, b)),
+                            ("vt", [positive, value("seven", 7.0), y], np.where(a > 0, np.float32(7), b)),
+                            ("tv", [positive, x, value("nine", 9.0)], np.where(a > 0, a, np.float32(9)))):
+        out = g.variable(name)
+        g.node("nn.Where", ins, [out])
+        wants[out] = want
+    for k in (0, 2, -1):
+        for op, ref in (("Tril", np.tril), ("Triu", np.triu)):
+            out = g.variable(op.lower())
+            g.node("base." + op, [x], [out], mf.f_varint(1, k & 0xFFFFFFFFFFFFFFFF) if k else b"")
+            wants[out] = ref(a, k)
+    shape = g.constant("shape", np.array([6, 6], np.int64), mf.CONSTANT_VECTOR)
+    ones = g.variable("ones")
+    g.node("base.CreateTensor", [shape], [ones], mf.f_bytes(1, mf.value_message(1.0)) + mf.f_varint(2, mf.FLOAT))
+    wants[ones] = np.ones((6, 6), np.float32)
+    sevens = g.variable("sevens", mf.INT64)
+    g.node("base.CreateTensor", [shape], [sevens], mf.f_bytes(1, mf.value_message(7, "int64")) + mf.f_varint(2, mf.INT64))
+    wants[sevens] = np.full((6, 6), 7, np.int64)
+    lower = g.variable("lower")
+    g.node("base.Tril", [ones], [lower])
+    hidden = g.variable("hidden", mf.BOOL)
+    g.node("relation.Equal", [lower, value("zero2", 0.0)], [hidden])
+    causal = g.variable("causal")
+    g.node("nn.Where", [hidden, value("neg", -10000.0), value("zero3", 0.0)], [causal])  # both values: nobody takes it
+    steps = g.vector("steps", mf.INT64)
+    g.node("base.Range", [value("start", 2, np.int64), value("limit", 11, np.int64), value("delta", 3, np.int64)], [steps])
+    steps_t = g.variable("steps_t", mf.INT64)
+    g.node("base.ToTensor", [steps], [steps_t])
+    wants[steps_t] = np.arange(2, 11, 3)
+    for o in wants:
+        g.output(o)
+    g.output(causal)
+    with pytest.raises(rt.RuntimeError_, match="(?i)unknow"):
+        rt.Model(mf.write_model([g], "g")).run({"x": a, "y": b})
+    # the same graph with the mask as a tensor-valued Where
+    g.nodes.pop(-3)
+    zeros = g.variable("zeros")
+    g.node("base.CreateTensor", [shape], [zeros], mf.f_bytes(1, mf.value_message(0.0)) + mf.f_varint(2, mf.FLOAT))
+    g.node("nn.Where", [hidden, value("neg2", -10000.0), zeros], [causal])
+    wants[causal] = np.where(np.tril(np.ones((6, 6))) == 0, np.float32(-10000.0), np.float32(0))
+    res = rt.Model(mf.write_model([g], "g")).run({"x": a, "y": b})
+    for name, want in wants.items():
+        assert res[name].shape == np.shape(want), name
+        assert np.array_equal(res[name], np.asarray(want).astype(res[name].dtype)), name
+
+
+@pytest.mark.gpu
 def test_split_stack_slice_pad_nodes_equal_numpy(mf, rt, dev):
     """base.Split (as many equal parts as outputs), base.Stack, base.SliceV2 (negative positions count from the end,
     the end is clipped) and base.Pad: tfcc_runtime/operations/base/split.cpp, stack.cpp, slicev2.cpp, pad.cpp."""

@@ -136,6 +136,8 @@ SYMBOLS = {
     "tfcc_rocm_copy2d": (_I, [_VP, _VP, _U64, _VP, _U64, _U64, _U64]),
     "tfcc_rocm_gather_rows": (_I, [_VP, _VP, _U, _U64, _VP, _I, _U64, _VP]),
     "tfcc_rocm_cast": (_I, [_VP, _VP, _I, _VP, _I, _U64]),
+    "tfcc_rocm_where": (_I, [_VP, _VP, _VP, _U64, _VP, _U64, _U, _U64, _VP]),
+    "tfcc_rocm_triangle": (_I, [_VP, _VP, _U64, _U64, C.c_int64, _I, _U, _VP]),
     "tfcc_rocm_compare_value": (_I, [_VP, _I, _VP, _I, _U64, _VP, _VP]),
     "tfcc_rocm_compare": (_I, [_VP, _I, _VP, _VP, _I, _I, C.POINTER(C.c_uint), C.POINTER(_U64), C.POINTER(_U64), _VP]),
     "tfcc_rocm_argmax_f32": (_I, [_VP, _VP, _U64, _U, _U64, _VP]),
@@ -883,6 +885,45 @@ def compare(op, a, b):
     n = len(dims)
     check(lib().tfcc_rocm_compare(_stream(), COMPARE_OPS[op], _ptr(a), _ptr(b), _type_code(a.dtype), n, (C.c_uint * n)(*dims),
                                   (_U64 * n)(*strides(ca)), (_U64 * n)(*strides(cb)), _ptr(out)))
+    return out
+
+
+def _bits_of(value, dtype):
+    import torch
+    return int.from_bytes(torch.tensor([value], dtype=dtype).numpy().tobytes(), "little")
+
+
+def where(condition, x, y):
+    """tfcc::nn::where: condition (uint8) != 0 ? x : y; x or y (not both) may be a Python number."""
+    import torch
+    tensors = [t for t in (x, y) if isinstance(t, torch.Tensor)]
+    if not tensors:
+        raise InvalidArgumentError("where: x and y are both values")
+    if any(t.shape != condition.shape for t in tensors):
+        raise InvalidArgumentError("condition x and y has different shape")
+    dtype = tensors[0].dtype
+    out = torch.empty(condition.shape, dtype=dtype, device=condition.device)
+    if out.numel() == 0:
+        return out
+    condition = condition.contiguous()
+    xt = x.contiguous() if isinstance(x, torch.Tensor) else None
+    yt = y.contiguous() if isinstance(y, torch.Tensor) else None
+    check(lib().tfcc_rocm_where(_stream(), _ptr(condition), _ptr(xt) if xt is not None else None,
+                                0 if xt is not None else _bits_of(x, dtype), _ptr(yt) if yt is not None else None,
+                                0 if yt is not None else _bits_of(y, dtype), out.element_size(), out.numel(), _ptr(out)))
+    return out
+
+
+def triangle(a, k, upper):
+    """tfcc::base::tril (upper False) / triu (upper True) of a matrix."""
+    import torch
+    if a.dim() != 2:
+        raise InvalidArgumentError("invalid shape")
+    a = a.contiguous()
+    out = torch.empty_like(a)
+    if a.numel():
+        check(lib().tfcc_rocm_triangle(_stream(), _ptr(a), a.shape[0], a.shape[1], k, 1 if upper else 0, a.element_size(),
+                                       _ptr(out)))
     return out
 
 

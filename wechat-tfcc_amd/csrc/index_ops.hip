@@ -7,6 +7,10 @@
 //   slice         tfcc/mkl/interfaces/tfcc_mklbasicinterface.cpp:34-70, 488-515 ([s1, s2, s3] -> [s1, length, s3])
 //   concat        tfcc/core/operations/tfcc_base.cpp:86-106 (every value copied behind the previous ones along axis)
 //   cast          tfcc::data::cast: static_cast element by element
+//   where         tfcc/mkl/interfaces/tfcc_mklbasicinterface.cpp:398-422 (condition[i] != 0 ? x : y, either of x and
+//                 y a tensor or one value)
+//   tril / triu   tfcc/mkl/interfaces/tfcc_mklbasicinterface.cpp:433-466 (row r keeps columns below r + k + 1, or
+//                 from r + k on; the rest is 0)
 #include "common.hpp"
 
 namespace tfcc_rocm {
@@ -47,6 +51,25 @@ template <class IN, class OUT>
 __global__ __launch_bounds__(256) void cast_kernel(const IN* in, size_t total, OUT* out) {
   const size_t stride = (size_t)gridDim.x * 256;
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += stride) out[i] = static_cast<OUT>(in[i]);
+}
+
+// elements of W bytes; x / y null: the value in xBits / yBits instead
+template <class W>
+__global__ __launch_bounds__(256) void where_kernel(const unsigned char* condition, const W* x, W xValue, const W* y,
+                                                    W yValue, size_t total, W* out) {
+  const size_t stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += stride)
+    out[i] = condition[i] != 0 ? (x ? x[i] : xValue) : (y ? y[i] : yValue);
+}
+
+template <class W, bool UPPER>
+__global__ __launch_bounds__(256) void triangle_kernel(const W* in, size_t rows, size_t cols, long long k, W* out) {
+  const size_t total = rows * cols, stride = (size_t)gridDim.x * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += stride) {
+    const long long r = (long long)(i / cols), c = (long long)(i - (size_t)r * cols);
+    const bool keep = UPPER ? c >= r + k : c < r + k + 1;
+    out[i] = keep ? in[i] : W(0);
+  }
 }
 
 struct Word16 { unsigned w[4]; };
@@ -148,6 +171,57 @@ int tfcc_rocm_cast(void* stream, const void* in, int in_type, void* out, int out
     case TFCC_ROCM_F64: return launch_cast_from<double>(s, in, out, out_type, total);
     default: return set_error(TFCC_ROCM_INVALID_ARGUMENT, "cast: unknown source type %d", in_type);
   }
+}
+
+int tfcc_rocm_where(void* stream, const uint8_t* condition, const void* x, uint64_t x_bits, const void* y,
+                    uint64_t y_bits, unsigned element_bytes, uint64_t total, void* out) {
+  TFCC_REQUIRE(condition && out, "where: null argument");
+  TFCC_REQUIRE(x || y, "where: x and y are both values");
+  TFCC_REQUIRE(total > 0, "where: empty tensor");
+  hipStream_t s = as_stream(stream);
+  const dim3 grid(copy_grid((size_t)total)), block(256);
+#define TFCC_WHERE_CASE(BYTES, W)                                                                                  \
+  case BYTES:                                                                                                      \
+    hipLaunchKernelGGL(where_kernel<W>, grid, block, 0, s, condition, static_cast<const W*>(x), (W)x_bits,          \
+                       static_cast<const W*>(y), (W)y_bits, (size_t)total, static_cast<W*>(out));                  \
+    break;
+  switch (element_bytes) {
+    TFCC_WHERE_CASE(1, unsigned char)
+    TFCC_WHERE_CASE(2, unsigned short)
+    TFCC_WHERE_CASE(4, unsigned)
+    TFCC_WHERE_CASE(8, unsigned long long)
+    default: return set_error(TFCC_ROCM_INVALID_ARGUMENT, "where: element size %u (1, 2, 4 or 8)", element_bytes);
+  }
+#undef TFCC_WHERE_CASE
+  return check_launch("where");
+}
+
+int tfcc_rocm_triangle(void* stream, const void* in, uint64_t rows, uint64_t cols, int64_t k, int upper,
+                       unsigned element_bytes, void* out) {
+  TFCC_REQUIRE(in && out, "triangle: null argument");
+  TFCC_REQUIRE(rows > 0 && cols > 0, "triangle: empty matrix");
+  TFCC_REQUIRE(rows < (1ull << 31) && cols < (1ull << 31), "triangle: matrix too large");
+  TFCC_REQUIRE(k > -(1ll << 40) && k < (1ll << 40), "triangle: diagonal out of range");
+  hipStream_t s = as_stream(stream);
+  const dim3 grid(copy_grid((size_t)(rows * cols))), block(256);
+#define TFCC_TRIANGLE_CASE(BYTES, W)                                                                               \
+  case BYTES:                                                                                                      \
+    if (upper)                                                                                                     \
+      hipLaunchKernelGGL((triangle_kernel<W, true>), grid, block, 0, s, static_cast<const W*>(in), (size_t)rows,   \
+                         (size_t)cols, (long long)k, static_cast<W*>(out));                                        \
+    else                                                                                                           \
+      hipLaunchKernelGGL((triangle_kernel<W, false>), grid, block, 0, s, static_cast<const W*>(in), (size_t)rows,  \
+                         (size_t)cols, (long long)k, static_cast<W*>(out));                                        \
+    break;
+  switch (element_bytes) {
+    TFCC_TRIANGLE_CASE(1, unsigned char)
+    TFCC_TRIANGLE_CASE(2, unsigned short)
+    TFCC_TRIANGLE_CASE(4, unsigned)
+    TFCC_TRIANGLE_CASE(8, unsigned long long)
+    default: return set_error(TFCC_ROCM_INVALID_ARGUMENT, "triangle: element size %u (1, 2, 4 or 8)", element_bytes);
+  }
+#undef TFCC_TRIANGLE_CASE
+  return check_launch("triangle");
 }
 
 }  // extern "C"

@@ -376,6 +376,11 @@ class ROCMDataInterface : public DataInterface<T> {
     std::memcpy(&bits, &one, sizeof(T));
     check(tfcc_rocm_fill_async(current_stream(), a.data(), bits, sizeof(T), a.size()));
   }
+  void fill(Variable<T>& a, T value) override {
+    uint64_t bits = 0;
+    std::memcpy(&bits, &value, sizeof(T));
+    check(tfcc_rocm_fill_async(current_stream(), a.data(), bits, sizeof(T), a.size()));
+  }
   void castFrom(const void* source, int sourceCode, Variable<T>& result) override {
     check(tfcc_rocm_cast(current_stream(), source, sourceCode, result.data(), ElementCode<T>::value, result.size()));
   }
@@ -744,6 +749,22 @@ class ROCMBasicInterface : public BasicInterface<T> {
     } else {
       throw NotImplementedError("clip: float tensors only");
     }
+  }
+  Variable<T> where(const Tensor<uint8_t>& condition, const Tensor<T>* x, T xValue, const Tensor<T>* y, T yValue) override {
+    Variable<T> r(condition.shape());
+    if (r.size() == 0) return r;
+    uint64_t xBits = 0, yBits = 0;
+    std::memcpy(&xBits, &xValue, sizeof(T));
+    std::memcpy(&yBits, &yValue, sizeof(T));
+    check(tfcc_rocm_where(current_stream(), condition.data(), x ? x->data() : nullptr, xBits, y ? y->data() : nullptr, yBits,
+                          sizeof(T), r.size(), r.data()));
+    return r;
+  }
+  Variable<T> triangle(const Tensor<T>& a, int64_t k, bool upper) override {
+    if (a.size() == 0) throw InvalidArgumentError("invalid tensor");
+    Variable<T> r(a.shape());
+    check(tfcc_rocm_triangle(current_stream(), a.data(), a.shape(0), a.shape(1), k, upper ? 1 : 0, sizeof(T), r.data()));
+    return r;
   }
   Variable<int64_t> argmax(const Tensor<T>& a, size_t axis) override {
     if constexpr (std::is_same<T, float>::value) {

@@ -81,6 +81,7 @@ class DataInterface {
   virtual void get(const Tensor<T>&, T*) { throw NotImplementedError(); }  // device -> host, synchronises
   virtual void zeros(Variable<T>&) { throw NotImplementedError(); }
   virtual void ones(Variable<T>&) { throw NotImplementedError(); }
+  virtual void fill(Variable<T>&, T) { throw NotImplementedError(); }  // every element = the value (an addition)
   virtual Variable<T> copy(const Tensor<T>&) { throw NotImplementedError(); }
   // static_cast of `total` elements of the type with code `sourceCode` (ElementCode) into a tensor of this type
   virtual void castFrom(const void* /*source*/, int /*sourceCode*/, Variable<T>& /*result*/) { throw NotImplementedError(); }
@@ -123,6 +124,9 @@ class BasicInterface {
   // rows of params by index (tfcc/core/interfaces/tfcc_gatherinterface.h): indices of the type with code indexCode
   virtual Variable<T> clip(const Tensor<T>&, T, T) { throw NotImplementedError(); }
   virtual Variable<int64_t> argmax(const Tensor<T>&, size_t) { throw NotImplementedError(); }
+  // tfcc/core/interfaces/tfcc_basicinterface.h: where with tensor / value operands (x or y null: the value), tril, triu
+  virtual Variable<T> where(const Tensor<uint8_t>&, const Tensor<T>*, T, const Tensor<T>*, T) { throw NotImplementedError(); }
+  virtual Variable<T> triangle(const Tensor<T>&, int64_t, bool /*upper*/) { throw NotImplementedError(); }
   virtual Variable<T> gather(const Tensor<T>&, const void* /*indices*/, int /*indexCode*/, const Shape& /*indexShape*/) {
     throw NotImplementedError();
   }
@@ -367,6 +371,10 @@ void zeros(Variable<T>& a) {
 template <class T>
 void ones(Variable<T>& a) {
   Operation<T>::getCurrentInterface().getDataInterface().ones(a);
+}
+template <class T>
+void fill(Variable<T>& a, T value) {
+  Operation<T>::getCurrentInterface().getDataInterface().fill(a, value);
 }
 template <class T>
 Variable<T> copy(const Tensor<T>& a) {
@@ -744,7 +752,37 @@ Variable<T> pad(const Tensor<T>& a, size_t axis, unsigned paddingHead, unsigned 
 }
 }  // namespace base
 
+namespace base {
+// tfcc::base::tril / triu (tfcc/core/operations/tfcc_base.cpp:249-266)
+template <class T>
+Variable<T> tril(const Tensor<T>& a, int64_t k) {
+  if (a.shape().size() != 2) throw InvalidArgumentError("invalid shape");
+  return Operation<T>::getCurrentInterface().getBasicInterface().triangle(a, k, false);
+}
+template <class T>
+Variable<T> triu(const Tensor<T>& a, int64_t k) {
+  if (a.shape().size() != 2) throw InvalidArgumentError("invalid shape");
+  return Operation<T>::getCurrentInterface().getBasicInterface().triangle(a, k, true);
+}
+}  // namespace base
+
 namespace nn {
+// tfcc::nn::where (tfcc/core/operations/tfcc_nn.cpp:496-523)
+template <class T>
+Variable<T> where(const Tensor<uint8_t>& condition, const Tensor<T>& x, const Tensor<T>& y) {
+  if (condition.shape() != x.shape() || x.shape() != y.shape()) throw InvalidArgumentError("condition x and y has different shape");
+  return Operation<T>::getCurrentInterface().getBasicInterface().where(condition, &x, T(), &y, T());
+}
+template <class T>
+Variable<T> where(const Tensor<uint8_t>& condition, T x, const Tensor<T>& y) {
+  if (condition.shape() != y.shape()) throw InvalidArgumentError("condition x and y has different shape");
+  return Operation<T>::getCurrentInterface().getBasicInterface().where(condition, nullptr, x, &y, T());
+}
+template <class T>
+Variable<T> where(const Tensor<uint8_t>& condition, const Tensor<T>& x, T y) {
+  if (condition.shape() != x.shape()) throw InvalidArgumentError("condition x and y has different shape");
+  return Operation<T>::getCurrentInterface().getBasicInterface().where(condition, &x, T(), nullptr, y);
+}
 // tfcc::nn::gather (tfcc/core/operations/tfcc_nn.cpp:345-385) for int32 / uint32 / int64 / uint64 indices
 template <class T, class IDX>
 Variable<T> gather(const Tensor<T>& params, const Tensor<IDX>& indices) {

@@ -571,6 +571,129 @@ class Tile : public TypedOperation<T> {
   }
 };
 
+// ---- nn.Where (condition, x, y), base.Tril / Triu (k in the node), base.CreateTensor, base.Range -----------
+// Where: a BOOL tensor and two operands of the node's type of which one may be a value (nn/where.cpp:100-125).
+// CreateTensor: zeros of the shape vector plus the value of the node (base/createtensor.cpp:28-45); the sum is formed
+// on the host and written with one fill.  Range: start, limit, delta values -> a vector (base/range.cpp:28-36).
+template <class T>
+class Where : public TypedOperation<T> {
+ public:
+  Where() : TypedOperation<T>("nn.Where") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 3 || node.outputs.size() != 1) return false;
+    auto& sm = graph.getSymbolManager();
+    if (sm.getSymbolInfo(node.inputs[0]).dtype != BOOL || !is_tensor(stype_of(graph, node.inputs[0]))) return false;
+    if (sm.getSymbolInfo(node.inputs[1]).dtype != this->DTYPE || sm.getSymbolInfo(node.inputs[2]).dtype != this->DTYPE ||
+        sm.getSymbolInfo(node.outputs[0]).dtype != this->DTYPE)
+      return false;
+    const SymbolType sx = stype_of(graph, node.inputs[1]), sy = stype_of(graph, node.inputs[2]);
+    const Tensor<uint8_t>* c = sm.getTensor(node.inputs[0], uint8_t());
+    if (is_tensor(sx) && is_tensor(sy)) {
+      const Tensor<T>* x = sm.getTensor(node.inputs[1], T());
+      const Tensor<T>* y = sm.getTensor(node.inputs[2], T());
+      Variable<T>* out = sm.getVariable(node.outputs[0], T());
+      graph.addStep([c, x, y, out] { *out = nn::where(*c, *x, *y); });
+    } else if (is_value(sx) && is_tensor(sy)) {
+      const T* x = sm.getValue(node.inputs[1], T());
+      const Tensor<T>* y = sm.getTensor(node.inputs[2], T());
+      Variable<T>* out = sm.getVariable(node.outputs[0], T());
+      graph.addStep([c, x, y, out] { *out = nn::where(*c, *x, *y); });
+    } else if (is_tensor(sx) && is_value(sy)) {
+      const Tensor<T>* x = sm.getTensor(node.inputs[1], T());
+      const T* y = sm.getValue(node.inputs[2], T());
+      Variable<T>* out = sm.getVariable(node.outputs[0], T());
+      graph.addStep([c, x, y, out] { *out = nn::where(*c, *x, *y); });
+    } else {
+      return false;
+    }
+    return true;
+  }
+};
+
+template <class T, bool UPPER>
+class Triangle : public TypedOperation<T> {
+ public:
+  Triangle() : TypedOperation<T>(UPPER ? "base.Triu" : "base.Tril") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 1 || node.outputs.size() != 1) return false;
+    if (!same_dtype(graph, node.outputs, this->DTYPE) || !same_dtype(graph, node.inputs, this->DTYPE)) return false;
+    int64_t k = 0;
+    wire::Reader r(node.operation);
+    uint32_t f, t;
+    while (r.next(f, t)) {
+      if (f == 1 && t == 0) k = static_cast<int64_t>(r.varint());
+      else r.skip(t);
+    }
+    auto& sm = graph.getSymbolManager();
+    const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+    Variable<T>* out = sm.getVariable(node.outputs[0], T());
+    graph.addStep([a, out, k] { *out = UPPER ? base::triu(*a, k) : base::tril(*a, k); });
+    return true;
+  }
+};
+
+template <class T, class IDX>
+class CreateTensor : public TypedOperation<T> {
+ public:
+  CreateTensor() : TypedOperation<T>("base.CreateTensor") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if constexpr (!std::is_integral<IDX>::value || sizeof(IDX) < 4) {
+      return false;
+    } else {
+      if (node.inputs.size() != 1 || node.outputs.size() != 1) return false;
+      auto& sm = graph.getSymbolManager();
+      if (sm.getSymbolInfo(node.outputs[0]).dtype != this->DTYPE) return false;
+      if (sm.getSymbolInfo(node.inputs[0]).dtype != DataTypeOf<IDX>::value) return false;
+      proto::Value v;
+      uint64_t wanted = 0;
+      wire::Reader r(node.operation);
+      uint32_t f, t;
+      while (r.next(f, t)) {
+        if (f == 1 && t == 2) v = proto::parse_value(r.sub());
+        else if (f == 2 && t == 0) wanted = r.varint();
+        else r.skip(t);
+      }
+      if (wanted != static_cast<uint64_t>(this->DTYPE)) return false;
+      T value = static_cast<T>(0);
+      if (!v.get(value)) return false;
+      value = static_cast<T>(static_cast<T>(0) + value);
+      const std::vector<IDX>* shape = sm.getVector(node.inputs[0], IDX());
+      Variable<T>* out = sm.getVariable(node.outputs[0], T());
+      graph.addStep([shape, value, out] {
+        std::vector<unsigned> real;
+        for (IDX d : *shape) real.push_back(static_cast<unsigned>(d));
+        *out = Variable<T>{Shape(real)};
+        if (out->size() > 0) data::fill(*out, value);
+      });
+      return true;
+    }
+  }
+};
+
+template <class T>
+class Range : public TypedOperation<T> {
+ public:
+  Range() : TypedOperation<T>("base.Range") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 3 || node.outputs.size() != 1) return false;
+    if (!same_dtype(graph, node.outputs, this->DTYPE) || !same_dtype(graph, node.inputs, this->DTYPE)) return false;
+    auto& sm = graph.getSymbolManager();
+    for (const std::string& name : node.inputs)
+      if (!is_value(stype_of(graph, name))) return false;
+    const T* start = sm.getValue(node.inputs[0], T());
+    const T* limit = sm.getValue(node.inputs[1], T());
+    const T* delta = sm.getValue(node.inputs[2], T());
+    std::vector<T>* out = sm.getVector(node.outputs[0], T());
+    graph.addStep([start, limit, delta, out] {
+      out->clear();
+      // the reference's loop does not end for a step that does not move towards the limit
+      if (*start < *limit && !(*delta > static_cast<T>(0))) throw RuntimeError("Range: delta must be positive");
+      for (T x = *start; x < *limit; x += *delta) out->push_back(x);
+    });
+    return true;
+  }
+};
+
 // ---- nn.LayerNormalization --------------------------------------------------------------------------------
 template <class T>
 class LayerNormalization : public TypedOperation<T> {
@@ -1323,6 +1446,10 @@ class Collector {
     add(new Compare<Relation::LESS, T>());
     add(new Compare<Relation::LESS_EQUAL, T>());
     add(new ArgMax<T>());
+    add(new Where<T>());
+    add(new Triangle<T, false>());
+    add(new Triangle<T, true>());
+    add(new Range<T>());
     add(new LeakyRelu<T>());
     add(new Gelu<T>());
     add(new Unary<UnaryFunction::SIGMOID, T>());
@@ -1369,7 +1496,8 @@ class Collector {
   add(new SliceV2<T, OTHER>());         \
   add(new Pad<T, OTHER>());             \
   add(new Expand<T, OTHER>());          \
-  add(new Tile<T, OTHER>());
+  add(new Tile<T, OTHER>());            \
+  add(new CreateTensor<T, OTHER>());
     TFCC_RUNTIME_FOR_ALL_TYPES(TFCC_RUNTIME_ADD_PAIR)
 #undef TFCC_RUNTIME_ADD_PAIR
 #define TFCC_RUNTIME_ADD_DIMENSION(DST, E) add(new GetDimension<T, DST>());
