@@ -1494,12 +1494,18 @@ class Collector {
   add(new SliceV1<T, OTHER>());         \
   add(new At<T, OTHER>());              \
   add(new SliceV2<T, OTHER>());         \
-  add(new Pad<T, OTHER>());             \
-  add(new Expand<T, OTHER>());          \
-  add(new Tile<T, OTHER>());            \
-  add(new CreateTensor<T, OTHER>());
+  add(new Pad<T, OTHER>());
     TFCC_RUNTIME_FOR_ALL_TYPES(TFCC_RUNTIME_ADD_PAIR)
 #undef TFCC_RUNTIME_ADD_PAIR
+#define TFCC_RUNTIME_ADD_SHAPED(IDX) \
+  add(new Expand<T, IDX>());          \
+  add(new Tile<T, IDX>());            \
+  add(new CreateTensor<T, IDX>());
+    TFCC_RUNTIME_ADD_SHAPED(int32_t)
+    TFCC_RUNTIME_ADD_SHAPED(uint32_t)
+    TFCC_RUNTIME_ADD_SHAPED(int64_t)
+    TFCC_RUNTIME_ADD_SHAPED(uint64_t)
+#undef TFCC_RUNTIME_ADD_SHAPED
 #define TFCC_RUNTIME_ADD_DIMENSION(DST, E) add(new GetDimension<T, DST>());
     TFCC_RUNTIME_FOR_ALL_TYPES(TFCC_RUNTIME_ADD_DIMENSION)
 #undef TFCC_RUNTIME_ADD_DIMENSION
