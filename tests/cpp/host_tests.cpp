@@ -827,6 +827,57 @@ static void test_reduce_minmax_pow() {
   CHECK(ok);
 }
 
+// tfcc::relation (tensor against value, value against tensor, tensor against tensor), tfcc::nn::where,
+// tfcc::base::tril / triu, tfcc::math::argmax and data::fill, on float and int64 tensors
+// (tfcc/test/relation.cpp, tfcc/test/nn.cpp's where cases in the reference).
+static void test_relation_where_triangle() {
+  std::vector<int64_t> hv(3 * 5), hw(5);
+  for (size_t i = 0; i < hv.size(); ++i) hv[i] = static_cast<int64_t>((i * 7) % 5) - 2;
+  for (size_t i = 0; i < hw.size(); ++i) hw[i] = static_cast<int64_t>(i) - 2;
+  tfcc::Variable<int64_t> v = tfcc::data::set(hv, {3, 5}), w = tfcc::data::set(hw, {5});
+  std::vector<uint8_t> eq = tfcc::data::get(tfcc::relation::equal(v, int64_t(1))),
+                       lt = tfcc::data::get(tfcc::relation::less(int64_t(0), v)),   // 0 < v
+                       ge = tfcc::data::get(tfcc::relation::greater_equal(v, w)),
+                       ne = tfcc::data::get(tfcc::relation::unequal(w, v));
+  bool ok = eq.size() == hv.size() && ge.size() == hv.size() && ne.size() == hv.size();
+  for (size_t i = 0; ok && i < hv.size(); ++i)
+    ok = eq[i] == (hv[i] == 1) && lt[i] == (0 < hv[i]) && ge[i] == (hv[i] - hw[i % 5] >= 0) && ne[i] == (hw[i % 5] != hv[i]);
+  CHECK(ok);
+  CHECK_THROWS(tfcc::relation::equal(v, tfcc::data::set(std::vector<int64_t>{1, 2}, {2})), tfcc::InvalidArgumentError);
+
+  std::vector<float> hx(4 * 6), hy(4 * 6);
+  for (size_t i = 0; i < hx.size(); ++i) {
+    hx[i] = static_cast<float>((i * 5) % 7) - 3.f;
+    hy[i] = static_cast<float>(i) * 0.5f;
+  }
+  tfcc::Variable<float> x = tfcc::data::set(hx, {4, 6}), y = tfcc::data::set(hy, {4, 6});
+  tfcc::Variable<uint8_t> positive = tfcc::relation::greater(x, 0.f);
+  std::vector<float> w1 = tfcc::data::get(tfcc::nn::where(positive, x, y)), w2 = tfcc::data::get(tfcc::nn::where(positive, 7.f, y)),
+                     w3 = tfcc::data::get(tfcc::nn::where(positive, x, -1.f)), lo = tfcc::data::get(tfcc::base::tril(x, 1)),
+                     up = tfcc::data::get(tfcc::base::triu(x, -1));
+  std::vector<int64_t> am = tfcc::data::get(tfcc::math::argmax(x, 1));
+  ok = w1.size() == hx.size() && am.size() == 4;
+  for (size_t i = 0; ok && i < hx.size(); ++i) {
+    const long r = static_cast<long>(i / 6), c = static_cast<long>(i % 6);
+    ok = w1[i] == (hx[i] > 0 ? hx[i] : hy[i]) && w2[i] == (hx[i] > 0 ? 7.f : hy[i]) && w3[i] == (hx[i] > 0 ? hx[i] : -1.f) &&
+         lo[i] == (c <= r + 1 ? hx[i] : 0.f) && up[i] == (c >= r - 1 ? hx[i] : 0.f);
+  }
+  for (size_t r = 0; ok && r < 4; ++r) {
+    size_t best = 0;
+    for (size_t c = 1; c < 6; ++c)
+      if (hx[r * 6 + c] > hx[r * 6 + best]) best = c;
+    ok = am[r] == static_cast<int64_t>(best);
+  }
+  CHECK(ok);
+  CHECK(tfcc::math::argmax(x, 0).shape() == tfcc::Shape({1, 6}));
+  CHECK_THROWS_MSG(tfcc::nn::where(positive, x, tfcc::data::set(std::vector<float>{1.f}, {1})), tfcc::InvalidArgumentError,
+                   "condition x and y has different shape");
+  CHECK_THROWS_MSG(tfcc::base::tril(tfcc::data::set(std::vector<float>{1.f, 2.f}, {2}), 0), tfcc::InvalidArgumentError, "invalid shape");
+  tfcc::Variable<int16_t> filled(tfcc::Shape({7}));
+  tfcc::data::fill(filled, static_cast<int16_t>(-3));
+  CHECK(tfcc::data::get(filled) == std::vector<int16_t>(7, -3));
+}
+
 // tfcc::math::add / sub / mul / div with the broadcasting of tfcc/core/operations/tfcc_math.cpp:38-104
 // (tfcc/test/math.cpp's broadcast cases): attention mask, both sides broadcast, either operand the larger.
 static void test_broadcast_arithmetic() {
@@ -989,6 +1040,7 @@ int main(int argc, char** argv) {
     run("layer.elementwise", test_layer_ops);
     run("math.broadcast_arithmetic", test_broadcast_arithmetic);
     run("math.reduce_minmax_pow", test_reduce_minmax_pow);
+    run("relation.where_triangle", test_relation_where_triangle);
     run("layer.attention_permuted", test_attention_permuted);
     run("base.data_movement", test_data_movement);
     run("rnn.cells", test_cells);
