@@ -371,6 +371,10 @@ int tfcc_rocm_compare(void* stream, int op, const void* a, const void* b, int ty
 /* out[x, z] = first position y of the largest in[x, y, z], in is [outer, length, inner]
  * (tfcc/mkl/interfaces/tfcc_mklbasicinterface.cpp:469-485, :757-776). */
 int tfcc_rocm_argmax_f32(void* stream, const float* in, uint64_t outer, unsigned length, uint64_t inner, int64_t* out);
+/* The k largest elements of each row of in [rows, length], descending, and their positions; equal values in ascending
+ * position (tfcc/mkl/interfaces/tfcc_mklbasicinterface.cpp:159-260, :779-800 leaves their order open).  1 <= k <= length. */
+int tfcc_rocm_topk_f32(void* stream, const float* in, uint64_t rows, unsigned length, unsigned k, float* values,
+                       uint32_t* positions);
 /* out = a op b with numpy-style broadcasting: dims[rank] is the result's shape, stride_a / stride_b the element strides
  * of each operand per result dimension (0 where the operand's extent is 1).  rank <= 6; callers merge adjacent
  * dimensions of the same kind first, as tfcc::math::add does (tfcc/core/operations/tfcc_math.cpp:38-104). */

@@ -677,6 +677,27 @@ def test_where_and_triangles(pkg, T):
         pkg.triangle(T.t(np.zeros((2, 3, 4), np.float32)), 0, True)
 
 
+def test_top_k(pkg, T):
+    """tfcc::math::top_k (tfcc/mkl/interfaces/tfcc_mklbasicinterface.cpp:159-260, :779-800): the k largest of each row,
+    descending.  Values are checked exactly against a sort; positions against a stable sort (equal values in ascending
+    position: the reference leaves that order to its heaps), also with ties, negative zero and infinities."""
+    rng = np.random.default_rng(67)
+    cases = [((3, 50), 5), ((2, 4, 300), 17), ((1, 30000), 8), ((5, 7), 7), ((4, 1), 1), ((6, 64), 64)]
+    for shape, k in cases:
+        for ties in (False, True):
+            x = (rng.integers(-4, 5, shape) if ties else rng.normal(size=shape)).astype(np.float32)
+            if ties and x.shape[-1] > 3:
+                x[..., 1] = np.inf
+                x[..., 2] = -np.inf
+                x[..., 0] = -0.0
+            values, positions = pkg.top_k(T.t(x), k)
+            order = np.argsort(-x.astype(np.float64), axis=-1, kind="stable")[..., :k]
+            assert np.array_equal(T.n(positions), order), (shape, k, ties)
+            assert np.array_equal(T.n(values).view(np.uint32), np.take_along_axis(x, order, axis=-1).view(np.uint32))
+    with pytest.raises(pkg.InvalidArgumentError, match="invalid k"):
+        pkg.top_k(T.t(np.zeros((2, 3), np.float32)), 4)
+
+
 BROADCAST_PAIRS = [
     ((2, 4, 8, 8), (2, 1, 1, 8)),        # attention scores + mask
     ((3, 1, 5), (1, 4, 1)),              # both sides broadcast

@@ -846,6 +846,28 @@ def test_where_triangle_create_tensor_range_nodes_equal_numpy(mf, rt, dev):
 
 
 @pytest.mark.gpu
+def test_top_k_node(mf, rt, dev):
+    """math.TopK: values and int64 positions of the k largest along the last axis, k a value input clipped to that
+    axis' length (tfcc_runtime/operations/math/topk.cpp:28-135)."""
+    rng = np.random.default_rng(71)
+    a = rng.normal(size=(3, 4, 40)).astype(np.float32)
+    g = mf.GraphBuilder("g")
+    x = g.input("x", mf.FLOAT, [3, 4, 40])
+    wants = {}
+    for name, k, dt in (("five", 5, np.int64), ("all", 100, np.uint32)):
+        values, positions = g.variable("values_" + name), g.variable("positions_" + name, mf.INT64)
+        g.node("math.TopK", [x, g.constant("k_" + name, np.array(k, dt), mf.CONSTANT_VALUE)], [values, positions])
+        g.output(values)
+        g.output(positions)
+        order = np.argsort(-a.astype(np.float64), axis=-1, kind="stable")[..., :min(k, 40)]
+        wants[values] = np.take_along_axis(a, order, axis=-1)
+        wants[positions] = order
+    res = rt.Model(mf.write_model([g], "g")).run({"x": a})
+    for name, want in wants.items():
+        assert res[name].shape == want.shape and np.array_equal(res[name], want.astype(res[name].dtype)), name
+
+
+@pytest.mark.gpu
 def test_split_stack_slice_pad_nodes_equal_numpy(mf, rt, dev):
     """base.Split (as many equal parts as outputs), base.Stack, base.SliceV2 (negative positions count from the end,
     the end is clipped) and base.Pad: tfcc_runtime/operations/base/split.cpp, stack.cpp, slicev2.cpp, pad.cpp."""

@@ -140,6 +140,7 @@ SYMBOLS = {
     "tfcc_rocm_triangle": (_I, [_VP, _VP, _U64, _U64, C.c_int64, _I, _U, _VP]),
     "tfcc_rocm_compare_value": (_I, [_VP, _I, _VP, _I, _U64, _VP, _VP]),
     "tfcc_rocm_compare": (_I, [_VP, _I, _VP, _VP, _I, _I, C.POINTER(C.c_uint), C.POINTER(_U64), C.POINTER(_U64), _VP]),
+    "tfcc_rocm_topk_f32": (_I, [_VP, _VP, _U64, _U, _U, _VP, _VP]),
     "tfcc_rocm_argmax_f32": (_I, [_VP, _VP, _U64, _U, _U64, _VP]),
     "tfcc_rocm_lstm_step_f32": (_I, [_VP, _U, _U, _VP, _VP, _VP, _VP, _F, _VP, _VP, _VP]),
     "tfcc_rocm_gru_cell_gates_f32": (_I, [_VP, _U, _U, _U, _VP, _VP, _VP, _VP, _VP]),
@@ -925,6 +926,22 @@ def triangle(a, k, upper):
         check(lib().tfcc_rocm_triangle(_stream(), _ptr(a), a.shape[0], a.shape[1], k, 1 if upper else 0, a.element_size(),
                                        _ptr(out)))
     return out
+
+
+def top_k(a, k):
+    """tfcc::math::top_k: (values, positions) of the k largest elements along the last axis, descending; positions
+    come back as int64 holding the kernel's uint32 results (torch has no uint32 arithmetic)."""
+    import torch
+    if a.numel() == 0:
+        raise InvalidArgumentError("invalid tensor")
+    if a.shape[-1] < k:
+        raise InvalidArgumentError("invalid k")
+    a = a.contiguous()
+    shape = list(a.shape[:-1]) + [k]
+    values = torch.empty(shape, dtype=torch.float32, device=a.device)
+    positions = torch.empty(shape, dtype=torch.int32, device=a.device)
+    check(lib().tfcc_rocm_topk_f32(_stream(), _ptr(a), a.numel() // a.shape[-1], a.shape[-1], k, _ptr(values), _ptr(positions)))
+    return values, positions.to(torch.int64) & 0xFFFFFFFF
 
 
 def argmax(a, axis):

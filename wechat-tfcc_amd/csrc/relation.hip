@@ -8,6 +8,10 @@
 //                       kernel instead of in memory.
 //   argmax              tfcc/mkl/interfaces/tfcc_mklbasicinterface.cpp:469-485: the first position of the largest
 //                       element (a later element wins only if it is greater).
+//   top k               tfcc/mkl/interfaces/tfcc_mklbasicinterface.cpp:159-260, :779-800: the k largest elements of each
+//                       row in descending order with their positions.  The reference's heaps leave the order of equal
+//                       values to the standard library and to the number of threads; here equal values come in
+//                       ascending position.
 #include <type_traits>
 
 #include "common.hpp"
@@ -118,6 +122,44 @@ __global__ __launch_bounds__(256) void argmax_rows_kernel(const float* a, size_t
   if (lane == 0) out[row] = index;
 }
 
+// Floats as unsigned keys of the same order (negative values reversed, the sign bit flipped for the others), joined
+// with the complement of the position: the larger composite is the larger value or, of equal values, the earlier one.
+__device__ __forceinline__ unsigned long long topk_composite(float v, unsigned position) {
+  unsigned bits = __float_as_uint(v);
+  if (bits == 0x80000000u) bits = 0;  // -0 and +0 are equal values
+  const unsigned key = (bits & 0x80000000u) ? ~bits : (bits | 0x80000000u);
+  return ((unsigned long long)key << 32) | (unsigned)(~position);
+}
+
+// One wavefront per row, k rounds: each round takes the largest composite below the one taken before.  Every round
+// reads the row again (from L2 after the first), which suits the short lists of a decoder: k * length stays small.
+__global__ __launch_bounds__(256) void topk_rows_kernel(const float* a, size_t rows, unsigned length, unsigned k,
+                                                        float* values, unsigned* positions) {
+  const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const unsigned lane = threadIdx.x & 63;
+  const float* p = a + row * length;
+  unsigned long long previous = ~0ull;
+  for (unsigned round = 0; round < k; ++round) {
+    unsigned long long best = 0;  // below the composite of every element: positions stay below 2^32 - 1, so low words are not 0
+    for (unsigned y = lane; y < length; y += 64) {
+      const unsigned long long c = topk_composite(p[y], y);
+      if (c < previous && c > best) best = c;
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const unsigned long long other = __shfl_xor(best, off, 64);
+      if (other > best) best = other;
+    }
+    previous = best;
+    if (lane == 0 && best != 0) {  // k <= length leaves an element for every round
+      const unsigned position = ~(unsigned)(best & 0xffffffffu);
+      values[row * k + round] = p[position];
+      positions[row * k + round] = position;
+    }
+  }
+}
+
 unsigned grid_of(size_t total) {
   size_t blocks = (total + 255) / 256;
   if (blocks > 4096) blocks = 4096;
@@ -211,6 +253,17 @@ int tfcc_rocm_argmax_f32(void* stream, const float* in, uint64_t outer, unsigned
                        (size_t)inner, reinterpret_cast<long long*>(out));
   }
   return check_launch("argmax");
+}
+
+int tfcc_rocm_topk_f32(void* stream, const float* in, uint64_t rows, unsigned length, unsigned k, float* values,
+                       uint32_t* positions) {
+  TFCC_REQUIRE(in && values && positions, "topk: null argument");
+  TFCC_REQUIRE(rows > 0 && length > 0, "topk: empty tensor");
+  TFCC_REQUIRE(k >= 1 && k <= length, "topk: k = %u of %u elements", k, length);
+  TFCC_REQUIRE(rows < (1ull << 31) && length < 0xffffffffu, "topk: tensor too large");
+  hipLaunchKernelGGL(topk_rows_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, as_stream(stream), in, (size_t)rows,
+                     length, k, values, positions);
+  return check_launch("topk");
 }
 
 }  // extern "C"

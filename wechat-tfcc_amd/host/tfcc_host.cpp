@@ -766,6 +766,20 @@ class ROCMBasicInterface : public BasicInterface<T> {
     check(tfcc_rocm_triangle(current_stream(), a.data(), a.shape(0), a.shape(1), k, upper ? 1 : 0, sizeof(T), r.data()));
     return r;
   }
+  std::tuple<Variable<T>, Variable<uint32_t>> topK(const Tensor<T>& a, unsigned k) override {
+    if constexpr (std::is_same<T, float>::value) {
+      if (k == 0) throw InvalidArgumentError("invalid k");
+      std::vector<unsigned> shape = a.shape().toVector();
+      const unsigned length = shape.back();
+      shape.back() = k;
+      Variable<T> values{Shape(shape)};
+      Variable<uint32_t> positions{Shape(shape)};
+      check(tfcc_rocm_topk_f32(current_stream(), a.data(), a.size() / length, length, k, values.data(), positions.data()));
+      return std::make_tuple(std::move(values), std::move(positions));
+    } else {
+      throw NotImplementedError("top_k: float tensors only");
+    }
+  }
   Variable<int64_t> argmax(const Tensor<T>& a, size_t axis) override {
     if constexpr (std::is_same<T, float>::value) {
       std::vector<unsigned> shape = a.shape().toVector();

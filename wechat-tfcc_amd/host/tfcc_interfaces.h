@@ -124,6 +124,7 @@ class BasicInterface {
   // rows of params by index (tfcc/core/interfaces/tfcc_gatherinterface.h): indices of the type with code indexCode
   virtual Variable<T> clip(const Tensor<T>&, T, T) { throw NotImplementedError(); }
   virtual Variable<int64_t> argmax(const Tensor<T>&, size_t) { throw NotImplementedError(); }
+  virtual std::tuple<Variable<T>, Variable<uint32_t>> topK(const Tensor<T>&, unsigned) { throw NotImplementedError(); }
   // tfcc/core/interfaces/tfcc_basicinterface.h: where with tensor / value operands (x or y null: the value), tril, triu
   virtual Variable<T> where(const Tensor<uint8_t>&, const Tensor<T>*, T, const Tensor<T>*, T) { throw NotImplementedError(); }
   virtual Variable<T> triangle(const Tensor<T>&, int64_t, bool /*upper*/) { throw NotImplementedError(); }
@@ -577,6 +578,13 @@ Variable<int64_t> argmax(const Tensor<T>& a, size_t axis) {
   if (a.size() == 0) throw InvalidArgumentError("invalid tensor");
   if (axis >= a.shape().size()) throw InvalidArgumentError("invalid axis");
   return Operation<T>::getCurrentInterface().getBasicInterface().argmax(a, axis);
+}
+// tfcc::math::top_k (tfcc/core/operations/tfcc_math.cpp:546-556): the k largest along the last axis and their positions
+template <class T>
+std::tuple<Variable<T>, Variable<uint32_t>> top_k(const Tensor<T>& a, unsigned k) {
+  if (a.size() == 0) throw InvalidArgumentError("invalid tensor");
+  if (a.shape(a.shape().size() - 1) < k) throw InvalidArgumentError("invalid k");
+  return Operation<T>::getCurrentInterface().getBasicInterface().topK(a, k);
 }
 // tfcc::math::reduce_sum / mean / prod / max / min (tfcc/core/operations/tfcc_math.cpp:464-522)
 #define TFCC_REDUCE_FUNCTION(NAME, METHOD)                                                   \

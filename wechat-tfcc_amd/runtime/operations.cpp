@@ -694,6 +694,38 @@ class Range : public TypedOperation<T> {
   }
 };
 
+// ---- math.TopK (tensor, k value) -> values, int64 positions; k is clipped to the last dimension ---------------
+// tfcc_runtime/operations/math/topk.cpp:28-135 sorts on the host after a read-back; here the rows are searched on the
+// device and the positions converted to int64 there.  Equal values come in ascending position.
+template <class T, class LEN>
+class TopK : public TypedOperation<T> {
+ public:
+  TopK() : TypedOperation<T>("math.TopK") {}
+  bool process(const proto::Node& node, Graph& graph) const override {
+    if (node.inputs.size() != 2 || node.outputs.size() != 2) return false;
+    auto& sm = graph.getSymbolManager();
+    if (sm.getSymbolInfo(node.outputs[0]).dtype != this->DTYPE || sm.getSymbolInfo(node.inputs[0]).dtype != this->DTYPE)
+      return false;
+    if (sm.getSymbolInfo(node.inputs[1]).dtype != DataTypeOf<LEN>::value || !is_value(stype_of(graph, node.inputs[1])))
+      return false;
+    if (sm.getSymbolInfo(node.outputs[1]).dtype != DataTypeOf<int64_t>::value) return false;
+    const Tensor<T>* a = sm.getTensor(node.inputs[0], T());
+    const LEN* k = sm.getValue(node.inputs[1], LEN());
+    Variable<T>* values = sm.getVariable(node.outputs[0], T());
+    Variable<int64_t>* positions = sm.getVariable(node.outputs[1], int64_t());
+    graph.addStep([a, k, values, positions] {
+      if (a->size() == 0) throw InvalidArgumentError("invalid tensor");
+      if (*k <= 0) throw InvalidArgumentError("invalid k");
+      const unsigned length = a->shape(a->shape().size() - 1);
+      const unsigned count = static_cast<unsigned>(std::min<uint64_t>(static_cast<uint64_t>(*k), length));
+      Variable<uint32_t> found;
+      std::tie(*values, found) = math::top_k(*a, count);
+      *positions = data::cast<int64_t>(found);
+    });
+    return true;
+  }
+};
+
 // ---- nn.LayerNormalization --------------------------------------------------------------------------------
 template <class T>
 class LayerNormalization : public TypedOperation<T> {
@@ -1506,6 +1538,14 @@ class Collector {
     TFCC_RUNTIME_ADD_SHAPED(int64_t)
     TFCC_RUNTIME_ADD_SHAPED(uint64_t)
 #undef TFCC_RUNTIME_ADD_SHAPED
+    add(new TopK<T, int8_t>());
+    add(new TopK<T, uint8_t>());
+    add(new TopK<T, int16_t>());
+    add(new TopK<T, uint16_t>());
+    add(new TopK<T, int32_t>());
+    add(new TopK<T, uint32_t>());
+    add(new TopK<T, int64_t>());
+    add(new TopK<T, uint64_t>());
 #define TFCC_RUNTIME_ADD_DIMENSION(DST, E) add(new GetDimension<T, DST>());
     TFCC_RUNTIME_FOR_ALL_TYPES(TFCC_RUNTIME_ADD_DIMENSION)
 #undef TFCC_RUNTIME_ADD_DIMENSION
