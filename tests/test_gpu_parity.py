@@ -651,6 +651,9 @@ def test_comparisons_and_argmax(pkg, T):
     x[2, 77] = np.nan           # elsewhere it is never taken
     want = np.array([np.argmax(x[0]), 0, np.nanargmax(x[2]), np.argmax(x[3])]).reshape(4, 1)
     assert np.array_equal(T.n(pkg.argmax(T.t(x), 1)), want)
+    # the same along the first axis, which is cut into ranges that each start from the axis' first element
+    xt = np.ascontiguousarray(x.T)
+    assert np.array_equal(T.n(pkg.argmax(T.t(xt), 0)), want.reshape(1, 4))
     with pytest.raises(pkg.InvalidArgumentError, match="invalid axis"):
         pkg.argmax(T.t(x), 2)
 

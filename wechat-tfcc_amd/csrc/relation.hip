@@ -71,21 +71,44 @@ __global__ __launch_bounds__(256) void compare_tensors_kernel(int op, const T* a
   }
 }
 
-// one thread per (outer, inner) pair walks the axis; neighbouring threads read neighbouring inner positions
+// 64 neighbouring (outer, inner) positions per workgroup, read coalesced; the axis is cut into four ranges, one per
+// wavefront.  Every range starts from the axis' first element as the scalar loop does (a NaN there stays, a NaN
+// elsewhere is never taken), and the ranges are joined in ascending order: a later one wins only if it is greater.
 __global__ __launch_bounds__(256) void argmax_kernel(const float* a, size_t outer, unsigned length, size_t inner,
                                                      long long* out) {
+  __shared__ float sBest[256];
+  __shared__ unsigned sIndex[256];
   const size_t total = outer * inner;
-  const size_t step = (size_t)gridDim.x * 256;
-  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += step) {
+  const size_t i = (size_t)blockIdx.x * 64 + (threadIdx.x & 63);
+  const unsigned part = threadIdx.x >> 6;
+  const bool valid = i < total;
+  float best = 0.f;
+  unsigned index = 0;
+  const float* p = a;
+  if (valid) {
     const size_t x = i / inner, z = i - x * inner;
-    const float* p = a + x * length * inner + z;
-    float best = p[0];
-    long long index = 0;
-    for (unsigned y = 1; y < length; ++y) {
+    p = a + x * length * inner + z;
+    best = p[0];
+    const unsigned begin = (unsigned)((unsigned long long)length * part / 4);
+    const unsigned end = (unsigned)((unsigned long long)length * (part + 1) / 4);
+    for (unsigned y = begin; y < end; ++y) {
       const float v = p[(size_t)y * inner];
       if (v > best) {
         best = v;
         index = y;
+      }
+    }
+  }
+  sBest[threadIdx.x] = best;
+  sIndex[threadIdx.x] = index;
+  __syncthreads();
+  if (valid && part == 0) {
+#pragma unroll
+    for (int j = 1; j < 4; ++j) {
+      const float ob = sBest[threadIdx.x + 64 * j];
+      if (ob > best) {
+        best = ob;
+        index = sIndex[threadIdx.x + 64 * j];
       }
     }
     out[i] = index;
@@ -131,18 +154,29 @@ __device__ __forceinline__ unsigned long long topk_composite(float v, unsigned p
   return ((unsigned long long)key << 32) | (unsigned)(~position);
 }
 
-// One wavefront per row, k rounds: each round takes the largest composite below the one taken before.  Every round
-// reads the row again (from L2 after the first), which suits the short lists of a decoder: k * length stays small.
-__global__ __launch_bounds__(256) void topk_rows_kernel(const float* a, size_t rows, unsigned length, unsigned k,
-                                                        float* values, unsigned* positions) {
-  const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= rows) return;
-  const unsigned lane = threadIdx.x & 63;
+// One workgroup per row, k rounds: each round takes the largest composite below the one taken before.  Every round
+// reads the row again (from L2 after the first), four independent loads per thread in flight; this suits the short
+// lists of a decoder, where k * length stays small.  The wavefronts' results meet in LDS, two buffers in turn so
+// that one barrier per round is enough.
+__global__ __launch_bounds__(256) void topk_rows_kernel(const float* a, unsigned length, unsigned k, float* values,
+                                                        unsigned* positions) {
+  __shared__ unsigned long long sBest[8];
+  const size_t row = blockIdx.x;
+  const unsigned tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const float* p = a + row * length;
   unsigned long long previous = ~0ull;
   for (unsigned round = 0; round < k; ++round) {
     unsigned long long best = 0;  // below the composite of every element: positions stay below 2^32 - 1, so low words are not 0
-    for (unsigned y = lane; y < length; y += 64) {
+    unsigned y = tid;
+    for (; (unsigned long long)y + 768 < length; y += 1024) {
+      const unsigned long long c0 = topk_composite(p[y], y), c1 = topk_composite(p[y + 256], y + 256),
+                               c2 = topk_composite(p[y + 512], y + 512), c3 = topk_composite(p[y + 768], y + 768);
+      if (c0 < previous && c0 > best) best = c0;
+      if (c1 < previous && c1 > best) best = c1;
+      if (c2 < previous && c2 > best) best = c2;
+      if (c3 < previous && c3 > best) best = c3;
+    }
+    for (; y < length; y += 256) {
       const unsigned long long c = topk_composite(p[y], y);
       if (c < previous && c > best) best = c;
     }
@@ -151,8 +185,15 @@ __global__ __launch_bounds__(256) void topk_rows_kernel(const float* a, size_t r
       const unsigned long long other = __shfl_xor(best, off, 64);
       if (other > best) best = other;
     }
+    unsigned long long* buffer = sBest + (round & 1) * 4;
+    if (lane == 0) buffer[wave] = best;
+    __syncthreads();
+    best = buffer[0];
+#pragma unroll
+    for (int w = 1; w < 4; ++w)
+      if (buffer[w] > best) best = buffer[w];
     previous = best;
-    if (lane == 0 && best != 0) {  // k <= length leaves an element for every round
+    if (tid == 0 && best != 0) {  // k <= length leaves an element for every round
       const unsigned position = ~(unsigned)(best & 0xffffffffu);
       values[row * k + round] = p[position];
       positions[row * k + round] = position;
@@ -243,14 +284,14 @@ int tfcc_rocm_compare(void* stream, int op, const void* a, const void* b, int ty
 int tfcc_rocm_argmax_f32(void* stream, const float* in, uint64_t outer, unsigned length, uint64_t inner, int64_t* out) {
   TFCC_REQUIRE(in && out, "argmax: null argument");
   TFCC_REQUIRE(outer > 0 && length > 0 && inner > 0, "argmax: empty tensor");
-  TFCC_REQUIRE(outer * inner < (1ull << 40), "argmax: too many positions");
+  TFCC_REQUIRE(outer < (1ull << 36) && inner < (1ull << 36) && outer * inner < (1ull << 36), "argmax: too many positions");
   hipStream_t s = as_stream(stream);
   if (inner == 1 && length >= 64 && outer < (1ull << 31)) {
     hipLaunchKernelGGL(argmax_rows_kernel, dim3((unsigned)((outer + 3) / 4)), dim3(256), 0, s, in, (size_t)outer, length,
                        reinterpret_cast<long long*>(out));
   } else {
-    hipLaunchKernelGGL(argmax_kernel, dim3(grid_of((size_t)(outer * inner))), dim3(256), 0, s, in, (size_t)outer, length,
-                       (size_t)inner, reinterpret_cast<long long*>(out));
+    hipLaunchKernelGGL(argmax_kernel, dim3((unsigned)((outer * inner + 63) / 64)), dim3(256), 0, s, in, (size_t)outer,
+                       length, (size_t)inner, reinterpret_cast<long long*>(out));
   }
   return check_launch("argmax");
 }
@@ -260,9 +301,9 @@ int tfcc_rocm_topk_f32(void* stream, const float* in, uint64_t rows, unsigned le
   TFCC_REQUIRE(in && values && positions, "topk: null argument");
   TFCC_REQUIRE(rows > 0 && length > 0, "topk: empty tensor");
   TFCC_REQUIRE(k >= 1 && k <= length, "topk: k = %u of %u elements", k, length);
-  TFCC_REQUIRE(rows < (1ull << 31) && length < 0xffffffffu, "topk: tensor too large");
-  hipLaunchKernelGGL(topk_rows_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0, as_stream(stream), in, (size_t)rows,
-                     length, k, values, positions);
+  TFCC_REQUIRE(rows < (1ull << 31) && length < 0x80000000u, "topk: tensor too large");
+  hipLaunchKernelGGL(topk_rows_kernel, dim3((unsigned)rows), dim3(256), 0, as_stream(stream), in, length, k, values,
+                     positions);
   return check_launch("topk");
 }
 
