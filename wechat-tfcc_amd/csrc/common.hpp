@@ -165,6 +165,26 @@ __device__ static inline int requantize_one_folded(double off, const RequantScal
   return q < lo ? lo : (q > hi ? hi : q);
 }
 
+// The two shortcuts above before the clamp, for callers that clamp while packing (pack_sat_u8).
+__device__ static inline int requantize_one_fast32_unclamped(double off, const RequantScalars& s) {
+  const double y = fma(off, s.inScale, s.inMin) * s.outScale;
+  return (int)(unsigned)__double_as_longlong(y + 6755399441055744.0) - s.offsetMinusLowest32;
+}
+__device__ static inline int requantize_one_folded_unclamped(double off, const RequantScalars& s) {
+  return (int)(unsigned)__double_as_longlong(fma(off, s.inScaleFolded, s.inMinFolded) + s.magicFolded);
+}
+
+// Four int32 clamped to 0..255 and packed into one word, first value in the low byte: int32 -> int16 and
+// int16 -> uint8, both saturating.
+__device__ static inline unsigned pack_sat_u8(int a, int b, int c, int d) {
+  typedef short pack_v2s __attribute__((ext_vector_type(2)));
+  const pack_v2s lo = __builtin_amdgcn_cvt_pk_i16(a, b), hi = __builtin_amdgcn_cvt_pk_i16(c, d);
+  unsigned l, h;
+  asm("v_sat_pk_u8_i16 %0, %1" : "=v"(l) : "v"(lo));
+  asm("v_sat_pk_u8_i16 %0, %1" : "=v"(h) : "v"(hi));
+  return l | (h << 16);
+}
+
 __device__ static inline long long requantize_one_exact(long long x, const RequantScalars& s) {
   double off = (double)x - (double)s.inLowest;
   double real = fma(off, s.inScale, s.inMin);

@@ -424,7 +424,10 @@ int launch_for_outputs(hipStream_t stream, const QGemmParams& p, bool requant) {
 
 int qgemm_dma_launch(hipStream_t stream, const QGemmParams& p, bool requant) {
   const unsigned long long big = (unsigned long long)((p.M + 255) / 256) * ((p.N + 255) / 256) * p.batch;
-  if (big >= 192) return launch_for_outputs<256, 256, 2, 4, 2>(stream, p, requant);
+  if (big >= 192) {
+    if (qgemm_w4_supported(p)) return qgemm_w4_launch(stream, p, requant);
+    return launch_for_outputs<256, 256, 2, 4, 2>(stream, p, requant);
+  }
   // fewer than half a chip of 128x128 tiles: 64x128 tiles (four wavefronts side by side) put twice as many CUs to work
   const unsigned long long mid = (unsigned long long)((p.M + 127) / 128) * ((p.N + 127) / 128) * p.batch;
   if (mid < 128) return launch_for_outputs<64, 128, 1, 4, 2>(stream, p, requant);

@@ -29,6 +29,15 @@ __device__ __forceinline__ void dma16(lds_dma_v4i rsrc, unsigned ldsBase, unsign
                : "memory", "m0");
 }
 
+// The same copy with a scalar byte offset on top of the lane's (the buffer's range check sees the lane offset
+// only) and the LDS address already in a scalar register.
+__device__ __forceinline__ void dma16s(lds_dma_v4i rsrc, unsigned ldsAddr, unsigned voffset, unsigned soffset) {
+  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+               :
+               : "s"(ldsAddr), "v"(voffset), "s"(rsrc), "s"(soffset)
+               : "memory", "m0");
+}
+
 template <int N>
 __device__ __forceinline__ void wait_vmcnt() {
   // s_waitcnt simm16: vmcnt[3:0] | expcnt[6:4] | lgkmcnt[11:8] | vmcnt_hi[15:14]; leave the others at max
