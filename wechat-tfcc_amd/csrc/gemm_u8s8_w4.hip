@@ -74,24 +74,32 @@ __global__ __launch_bounds__(kThreads) void qgemm_w4_kernel(const QGemmParams p)
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept in an SGPR
   const int wm = wave >> 1, wn = wave & 1;
 
+  // Everything this prologue needs of the argument block is read before the first branch (one round trip to
+  // memory instead of one per basic block); the divisions of the tile mapping are multiplications by constants
+  // the launcher worked out.
   unsigned tm, tn, bi;
+  bool inGrid;
   {
     // consecutive workgroup ids go to different XCDs: each XCD gets a contiguous run of tiles,
     // ordered in bands of 4 tile rows
     const unsigned wg = blockIdx.x;
     const unsigned xcd = wg & 7u, slot = wg >> 3;
     const unsigned L = xcd * p.chunk + slot;
-    if (slot >= p.chunk || L >= p.tilesTotal) return;
+    inGrid = slot < p.chunk && L < p.tilesTotal;
     const unsigned perBatch = p.tilesM * p.tilesN;
-    bi = L / perBatch;
+    bi = udiv_apply(L, p.perBatchMagic, p.perBatchShift);
     unsigned t = L - bi * perBatch;
     const unsigned band = 4u * p.tilesN;
-    unsigned gb = t / band;
+    unsigned gb = udiv_apply(t, p.bandMagic, p.bandShift);
     unsigned rowsInBand = min(4u, p.tilesM - gb * 4u);
     unsigned r = t - gb * band;
-    tm = gb * 4u + r % rowsInBand;
-    tn = r / rowsInBand;
+    const unsigned rq = rowsInBand == 4u ? r >> 2 : r / rowsInBand;  // a ragged last band is the rare case
+    tm = gb * 4u + (r - rq * rowsInBand);
+    tn = rq;
   }
+  // (the fields the later blocks read: named here so that their loads leave with the first ones)
+  asm volatile("" ::"s"(p.offsetA), "s"(p.offsetB), "s"(p.minA), "s"(p.minOut), "s"(p.rowsumA), "s"(p.colsumB),
+               "s"(p.strideRA), "s"(p.strideRB), "s"(p.strideC), "s"(p.C), "s"(p.Q));
   const unsigned m0 = tm * BM, n0 = tn * BN;
   const unsigned M = p.M, N = p.N, K = p.K;
   const unsigned char* A = p.A + (size_t)bi * p.strideA;
@@ -131,10 +139,16 @@ __global__ __launch_bounds__(kThreads) void qgemm_w4_kernel(const QGemmParams p)
     soB = __builtin_amdgcn_readfirstlane(sl * BK * N);
   };
 
+  if (!inGrid) return;
   // The first slabs are asked for before anything else: everything up to the main loop runs while they travel.
   constexpr int CPS = (STAGES > 2) ? (COPIES / (BK / 32)) : COPIES;  // copies per step that issues copies
+  // A CU's path into LDS takes 64 bytes a clock: a whole ring is 2000 clocks of it, and a wavefront that has
+  // issued more copies than the path has taken up waits to issue the next.  With four stages of two steps (RAMP)
+  // only slabs 0 and 1 are asked for here; slab 2, the rest of slab 3 and the first half of slab 4 follow between
+  // the matrix ops of slab 0, on top of the copies every step issues anyway.
+  constexpr bool RAMP = STAGES == 4 && (BK / 32) == 2;
 #pragma unroll
-  for (int s = 0; s < STAGES; ++s) {
+  for (int s = 0; s < (RAMP ? 2 : STAGES); ++s) {
     unsigned soA, soB;
     slabOffsets(s, soA, soB);
 #pragma unroll
@@ -171,17 +185,25 @@ __global__ __launch_bounds__(kThreads) void qgemm_w4_kernel(const QGemmParams p)
     } else {
       rq.inScale = p.inScale; rq.inMin = p.inMin; rq.outScale = p.outScale; rq.outOffset = p.outOffset;
       rq.inLowest = -2147483648LL; rq.outLowest = 0; rq.outHighest = 255; rq.mode = 0; rq.fillValue = 0;
-      finish_requant_scalars(rq, 4294967295.0);
+      // finish_requant_scalars, done by the launcher
+      rq.inScaleFolded = p.rqInScaleFolded; rq.inMinFolded = p.rqInMinFolded; rq.magicFolded = p.rqMagicFolded;
+      rq.offsetMinusLowest = p.rqOffsetMinusLowest; rq.offsetMinusLowest32 = p.rqOffsetMinusLowest32;
+      rq.fastOK = p.rqFastOK; rq.fast32OK = p.rqFast32OK; rq.foldedOK = p.rqFoldedOK;
     }
   }
 
+  // 256 accumulator registers set to zero by 16 matrix ops on zero operands (one instruction per block instead
+  // of one per register; the operand is a zero the compiler cannot see through)
   v16i acc[MI][NI];
+  {
+    const int z = (int)(K >> 31);  // K < 2^31
+    const v4i zero4 = {z, z, z, z};
+    const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-  for (int i = 0; i < MI; ++i)
+    for (int i = 0; i < MI; ++i)
 #pragma unroll
-    for (int j = 0; j < NI; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+      for (int j = 0; j < NI; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(zero4, zero4, zero16, 0, 0, 0);
+  }
   // Column sums of B: wavefront row w owns the blocks j = w and w + 2 of its wavefront column.  The bytes of an
   // operand word are summed as unsigned values of b + 128 (v_sad_u8 against zero: the dot-product instructions
   // hold up the matrix pipeline, this one does not); the 512 per word too much come off at the end.
@@ -237,11 +259,13 @@ __global__ __launch_bounds__(kThreads) void qgemm_w4_kernel(const QGemmParams p)
   //   m < 8       one word of this wavefront row's column sums (xor + sad)
   //   some m      one HBM -> LDS copy: copies [copy0, copy0 + ncopy) of dmaSlab into dmaStage
   auto step = [&](auto wrow, v4i (&ua)[MI], v4i (&ub)[NI], v4i (&la)[MI], v4i (&lb)[NI], int ldStage, int ldKs,
-                  auto dma, unsigned dmaSlab, int dmaStage, int copy0) {
+                  auto dma, unsigned dmaSlab, int dmaStage, int copy0, bool ramp = false, unsigned rampSlab = 0,
+                  int rampStage = 0, int rampCopy0 = 0, int rampCopies = 0) {
     constexpr int WROW = decltype(wrow)::value;
     constexpr bool DMA = decltype(dma)::value;
-    unsigned soA = 0, soB = 0;
+    unsigned soA = 0, soB = 0, rsoA = 0, rsoB = 0;
     if constexpr (DMA) slabOffsets(dmaSlab, soA, soB);
+    if (rampCopies > 0) slabOffsets(rampSlab, rsoA, rsoB);
 #pragma unroll
     for (int m = 0; m < 16; ++m) {
       const int i = m / NI, j = m % NI;
@@ -250,6 +274,9 @@ __global__ __launch_bounds__(kThreads) void qgemm_w4_kernel(const QGemmParams p)
       else la[0][j] ^= (int)0x80808080;
       if constexpr (OWN_COLSUM) {
         if (m < 8) csum[m >> 2][m & 3] = __builtin_amdgcn_sad_u8((unsigned)ub[WROW + 2 * (m >> 2)][m & 3] ^ 0x80808080u, 0u, csum[m >> 2][m & 3]);
+      }
+      if (m < rampCopies) {  // the first slab's extra copies, ahead of the step's own in issue order
+        if (ramp) issueCopy(rsoA, rsoB, rampStage, rampCopy0 + m);
       }
       if constexpr (DMA) {
         constexpr int FIRST = CPS >= 16 ? 0 : 16 - 2 * CPS;  // 16 copies: every slot; fewer: odd slots at the end
@@ -269,7 +296,7 @@ __global__ __launch_bounds__(kThreads) void qgemm_w4_kernel(const QGemmParams p)
   //              step with two stages, spread over the KS steps up to the next barrier with more
   static_assert(STAGES == 2 || COPIES % KS == 0, "copies per step");
   const unsigned KTR = KT;  // a multiple of STAGES (the launcher checks)
-  wait_vmcnt<COPIES*(STAGES - 2) + (STAGES > 2 ? CPS : COPIES)>();
+  wait_vmcnt<RAMP ? COPIES : COPIES*(STAGES - 2) + (STAGES > 2 ? CPS : COPIES)>();
   __syncthreads();
   v4i fa[2][MI], fb[2][NI];
 #pragma unroll
@@ -283,15 +310,27 @@ __global__ __launch_bounds__(kThreads) void qgemm_w4_kernel(const QGemmParams p)
         const unsigned kt = kt0 + s;
 #pragma unroll
         for (int ks = 0; ks < KS - 1; ++ks) {
-          if constexpr (STAGES > 2)  // copies (ks+1)*CPS.. of the slab that takes the place of slab kt-1
+          if (RAMP && s == 0)  // slab 0: slab 2 whole, then the step's own copies 4..7 of slab 3
+            step(wrow, fa[0], fb[0], fa[1], fb[1], s, 1, std::true_type{}, kt - 1 + STAGES, STAGES - 1, CPS,
+                 kt0 == 0, 2u, 2, 0, COPIES);
+          else if constexpr (STAGES > 2)  // copies (ks+1)*CPS.. of the slab that takes the place of slab kt-1
             step(wrow, fa[ks & 1], fb[ks & 1], fa[(ks + 1) & 1], fb[(ks + 1) & 1], s, ks + 1, std::true_type{},
                  kt - 1 + STAGES, (s + STAGES - 1) % STAGES, (ks + 1) * CPS);
           else
             step(wrow, fa[ks & 1], fb[ks & 1], fa[(ks + 1) & 1], fb[(ks + 1) & 1], s, ks + 1, std::false_type{}, 0u, 0, 0);
         }
-        wait_vmcnt<COPIES*(STAGES - 2)>();
-        __syncthreads();
-        step(wrow, fa[1], fb[1], fa[0], fb[0], (s + 1) % STAGES, 0, std::true_type{}, kt + STAGES, s, 0);
+        if (RAMP && s == 0) {
+          // slab 0's barrier: after slab 1's copies came slab 2 (8) and copies 4..7 of slab 3
+          if (kt0 == 0) wait_vmcnt<COPIES + CPS>();
+          else wait_vmcnt<COPIES*(STAGES - 2)>();
+          __syncthreads();
+          // copies 0..3 of slab 3, then the step's own
+          step(wrow, fa[1], fb[1], fa[0], fb[0], 1, 0, std::true_type{}, kt + STAGES, s, 0, kt0 == 0, 3u, 3, 0, CPS);
+        } else {
+          wait_vmcnt<COPIES*(STAGES - 2)>();
+          __syncthreads();
+          step(wrow, fa[1], fb[1], fa[0], fb[0], (s + 1) % STAGES, 0, std::true_type{}, kt + STAGES, s, 0);
+        }
       }
     }
   };
@@ -401,6 +440,18 @@ int launch_w4(hipStream_t stream, QGemmParams p) {
   if (total > 0x7fffffffull) return set_error(TFCC_ROCM_INVALID_ARGUMENT, "quantized matmul: too many tiles");
   p.tilesTotal = (unsigned)total;
   p.chunk = (p.tilesTotal + 7) / 8;
+  if (REQUANT && !p.minOut) {
+    RequantScalars rq;
+    rq.inScale = p.inScale; rq.inMin = p.inMin; rq.outScale = p.outScale; rq.outOffset = p.outOffset;
+    rq.inLowest = -2147483648LL; rq.outLowest = 0; rq.outHighest = 255; rq.mode = 0; rq.fillValue = 0;
+    finish_requant_scalars(rq, 4294967295.0);
+    p.rqInScaleFolded = rq.inScaleFolded; p.rqInMinFolded = rq.inMinFolded; p.rqMagicFolded = rq.magicFolded;
+    p.rqOffsetMinusLowest = rq.offsetMinusLowest; p.rqOffsetMinusLowest32 = rq.offsetMinusLowest32;
+    p.rqFastOK = rq.fastOK; p.rqFast32OK = rq.fast32OK; p.rqFoldedOK = rq.foldedOK;
+  }
+  const UDiv perBatch = udiv_prepare(p.tilesM * p.tilesN), band = udiv_prepare(4u * p.tilesN);
+  p.perBatchMagic = perBatch.magic; p.perBatchShift = perBatch.shift;
+  p.bandMagic = band.magic; p.bandShift = band.shift;
   constexpr size_t ring = (size_t)STAGES * (BM + BN) * BK;
   constexpr size_t epi = (size_t)(BM + BN) * 4;
   constexpr size_t lds = ring > epi ? ring : epi;
