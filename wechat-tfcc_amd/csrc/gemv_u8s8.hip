@@ -326,6 +326,17 @@ int gemv_launch(hipStream_t stream, const unsigned char* a, const signed char* b
                 const int* colsumB, int offsetA, int offsetB, const float* const ranges[4],
                 float* const rangeOut[2], unsigned m, unsigned n, unsigned k, int* accOut,
                 float scaleA, const float* scaleB, float* f32Out) {
+  if (gemv_wide_supported(a, b, m, n, k))
+    return gemv_wide_launch(stream, false, a, b, rowsumA, colsumB, offsetA, offsetB, ranges, rangeOut, m, n, k, accOut,
+                            scaleA, scaleB, f32Out);
+  return gemv_onepass_launch(stream, a, b, rowsumA, colsumB, offsetA, offsetB, ranges, rangeOut, m, n, k, accOut, scaleA,
+                             scaleB, f32Out);
+}
+
+int gemv_onepass_launch(hipStream_t stream, const unsigned char* a, const signed char* b, const int* rowsumA,
+                        const int* colsumB, int offsetA, int offsetB, const float* const ranges[4],
+                        float* const rangeOut[2], unsigned m, unsigned n, unsigned k, int* accOut,
+                        float scaleA, const float* scaleB, float* f32Out) {
   GemvParams p{};
   if (ranges && ranges[0]) {
     p.minA = ranges[0]; p.maxA = ranges[1]; p.minB = ranges[2]; p.maxB = ranges[3];
