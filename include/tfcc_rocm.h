@@ -205,6 +205,22 @@ int tfcc_rocm_gemv_u8s8s32(void* stream, const uint8_t* a, const int8_t* b,
                            int32_t offset_b, unsigned m, unsigned n, unsigned k, int32_t* acc_out,
                            float scale_a, const float* scale_b, float* f32_out);
 
+/* The same product through an entry point that allocates nothing.  No counterpart in the reference; it is for
+ * callers that cannot allocate device memory at the point of the call: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid it.  tfcc_rocm_gemv_u8s8s32 keeps the workspace of its K-split kernel in memory it
+ * allocates on first use (one per device and stream); this one uses a fixed array inside the library's image, one per
+ * GPU (1 MiB x 2: 32768 columns x 8 rows of 64-bit words), and therefore
+ *   - takes n <= 32768 where the K-split kernel applies (n % 16 == 0, b aligned to 16 bytes, at least 512 steps of 64
+ *     rows x 256 columns) and fails with TFCC_ROCM_INVALID_ARGUMENT beyond; smaller products run on the kernel without
+ *     a workspace; products that are not skinny (m > 8, unaligned a) are refused, not routed to the general kernel;
+ *   - must not overlap with another call of itself on the same GPU (two streams): both would add into the same
+ *     workspace.  Calls on one stream are ordered and leave the workspace zeroed for the next one.
+ * Same arguments and results as tfcc_rocm_gemv_u8s8s32. */
+int tfcc_rocm_gemv_u8s8s32_noalloc(void* stream, const uint8_t* a, const int8_t* b,
+                                   const int32_t* rowsum_a, const int32_t* colsum_b, int32_t offset_a,
+                                   int32_t offset_b, unsigned m, unsigned n, unsigned k, int32_t* acc_out,
+                                   float scale_a, const float* scale_b, float* f32_out);
+
 /* The same product on a B that was packed once (weights): column slabs of 16, each K x 16 bytes
  * contiguous and already in matrix-core operand order, so that a decode step streams B at the rate
  * of a plain contiguous read.  The reference re-packs its B operand on every call

@@ -395,6 +395,33 @@ extern "C" int tfcc_rocm_gemv_u8s8s32(void* stream, const uint8_t* a, const int8
   return TFCC_ROCM_OK;
 }
 
+// The same product for callers that cannot allocate: the workspace of the kernel that splits K lies inside the
+// library's image, one per GPU.
+extern "C" int tfcc_rocm_gemv_u8s8s32_noalloc(void* stream, const uint8_t* a, const int8_t* b,
+                                              const int32_t* rowsum_a, const int32_t* colsum_b,
+                                              int32_t offset_a, int32_t offset_b, unsigned m, unsigned n,
+                                              unsigned k, int32_t* acc_out, float scale_a,
+                                              const float* scale_b, float* f32_out) {
+  TFCC_REQUIRE(a && b && rowsum_a && colsum_b, "skinny quantized matmul: null operand");
+  TFCC_REQUIRE(m > 0 && n > 0 && k > 0, "skinny quantized matmul: empty operand");
+  TFCC_REQUIRE(acc_out || f32_out, "skinny quantized matmul: no output");
+  TFCC_REQUIRE(!f32_out || scale_b, "skinny quantized matmul: dequantize needs scale_b");
+  hipStream_t s = as_stream(stream);
+  const signed char* bs = reinterpret_cast<const signed char*>(b);
+  if (gemv_wide_supported(a, b, m, n, k)) {
+    TFCC_REQUIRE(n <= gemv_wide_static_max_n(),
+                 "skinny quantized matmul without allocation: n = %u, the workspace inside the library holds %u columns", n,
+                 gemv_wide_static_max_n());
+    return gemv_wide_launch(s, true, a, bs, rowsum_a, colsum_b, offset_a, offset_b, nullptr, nullptr, m, n, k, acc_out,
+                            scale_a, scale_b, f32_out);
+  }
+  // small or narrow products: the kernel that owns its columns over the whole of K uses no workspace at all
+  TFCC_REQUIRE(gemv_supported(a, b, m, n, k),
+               "skinny quantized matmul without allocation: at most 8 rows, n a multiple of 4, k a multiple of 16, a aligned to 16 bytes");
+  return gemv_onepass_launch(s, a, bs, rowsum_a, colsum_b, offset_a, offset_b, nullptr, nullptr, m, n, k, acc_out, scale_a,
+                             scale_b, f32_out);
+}
+
 extern "C" size_t tfcc_rocm_gemv_packed_size(unsigned n, unsigned k) {
   return (size_t)((n + 15) / 16) * ((k + 63) / 64) * 1024;
 }
