@@ -738,6 +738,37 @@ static void test_data_movement() {
   tfcc::Variable<float> fv = tfcc::data::set(std::vector<float>{-2.5f, 0.f, 3.9f, 100.25f}, {4});
   CHECK(tfcc::data::get(tfcc::data::cast<int8_t>(fv)) == (std::vector<int8_t>{-2, 0, 3, 100}));
   CHECK(tfcc::data::get(tfcc::data::cast<uint64_t>(tfcc::data::cast<double>(fv)))[3] == 100u);
+  // The interface itself, as the reference declares it (tfcc/core/interfaces/tfcc_datainterface.h:40-53): one cast
+  // virtual per source type, and cast_to_boolean.  Every source type into float and back out of float.
+  auto& toFloat = tfcc::Operation<float>::getCurrentInterface().getDataInterface();
+#define CAST_ROUND_TRIP(T, ...)                                                                       \
+  {                                                                                                   \
+    const std::vector<T> h{__VA_ARGS__};                                                               \
+    tfcc::Variable<T> src = tfcc::data::set(h, {static_cast<unsigned>(h.size())});                     \
+    std::vector<float> asFloat = tfcc::data::get(toFloat.cast(src));                                   \
+    bool same = asFloat.size() == h.size();                                                           \
+    for (size_t i = 0; same && i < h.size(); ++i) same = asFloat[i] == static_cast<float>(h[i]);       \
+    CHECK(same);                                                                                      \
+    tfcc::Variable<float> f32 = tfcc::data::set(asFloat, {static_cast<unsigned>(h.size())});           \
+    CHECK(tfcc::data::get(tfcc::Operation<T>::getCurrentInterface().getDataInterface().cast(f32)) == h); \
+  }
+  CAST_ROUND_TRIP(float, -1.5f, 0.f, 7.25f)
+  CAST_ROUND_TRIP(double, -1.5, 0.0, 7.25)
+  CAST_ROUND_TRIP(int8_t, -128, 0, 127)
+  CAST_ROUND_TRIP(uint8_t, 0, 1, 255)
+  CAST_ROUND_TRIP(int16_t, -32768, 0, 32767)
+  CAST_ROUND_TRIP(uint16_t, 0, 1, 65535)
+  CAST_ROUND_TRIP(int32_t, -16777216, 0, 16777216)
+  CAST_ROUND_TRIP(uint32_t, 0u, 1u, 16777216u)
+  CAST_ROUND_TRIP(int64_t, -16777216, 0, 16777216)
+  CAST_ROUND_TRIP(uint64_t, 0u, 1u, 16777216u)
+#undef CAST_ROUND_TRIP
+  tfcc::Variable<float> mixed = tfcc::data::set(std::vector<float>{0.f, -0.f, 1e-30f, -3.f, 0.f, 2.f}, {2, 3});
+  tfcc::Variable<uint8_t> flags = tfcc::data::cast_to_boolean(mixed);
+  CHECK(flags.shape() == mixed.shape());
+  CHECK(tfcc::data::get(flags) == (std::vector<uint8_t>{0, 0, 1, 1, 0, 1}));
+  tfcc::Variable<int64_t> wide = tfcc::data::set(std::vector<int64_t>{0, 1ll << 40, -1, 0}, {4});
+  CHECK(tfcc::data::get(tfcc::data::cast_to_boolean(wide)) == (std::vector<uint8_t>{0, 1, 1, 0}));
 }
 
 // tfcc::layer::Dense (tfcc/core/layers/tfcc_denselayer.cpp:47-87) in the style of the reference's layer tests:

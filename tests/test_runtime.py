@@ -373,6 +373,45 @@ def test_replay_reproduces_step_by_step_results(mf, rt, dev):
 
 
 @pytest.mark.gpu
+def test_replay_of_a_graph_that_reads_results_on_the_host(mf, rt, dev):
+    """A step that reads device memory on the host (base.ToVector of a tensor, base.ToValue of a one-element tensor)
+    cannot be part of a recording.  With replay asked for, such a graph runs step by step: every call returns the
+    results of its own inputs (no stale outputs from steps that were only recorded) and none raises."""
+    rng = np.random.default_rng(11)
+    g = mf.GraphBuilder("g")
+    x = g.input("x", mf.FLOAT, [2, 3, 4])
+    w = g.constant("w", rng.normal(size=(4, 5)).astype(np.float32))
+    prod = g.matmul(x, w)
+    shape = g.vector("shape", mf.UINT32)
+    g.node("base.GetShape", [prod], [shape])
+    shape_tensor = g.variable("shape_tensor", mf.UINT32)
+    g.node("base.ToTensor", [shape], [shape_tensor])
+    back = g.vector("back", mf.UINT32)
+    g.node("base.ToVector", [shape_tensor], [back])  # device -> host
+    last = g._symbol("last", mf.UINT32, mf.VALUE)
+    g.node("base.At1", [back], [last], mf.f_varint(1, 2))
+    one_tensor = g.variable("one_tensor", mf.UINT32)
+    g.node("base.ToTensor", [last], [one_tensor])
+    again = g._symbol("again", mf.UINT32, mf.VALUE)
+    g.node("base.ToValue", [one_tensor], [again])  # device -> host
+    doubled = g.binary("Add", prod, prod)
+    for o in (again, doubled):
+        g.output(o)
+    blob = mf.write_model([g], "g")
+    eager, replay = rt.Model(blob), rt.Model(blob)
+    replay.set_replay(True)
+    for i in range(5):
+        a = rng.normal(size=(2, 3, 4)).astype(np.float32)
+        want, got = eager.run({"x": a}), replay.run({"x": a})
+        assert int(got[again][0]) == 5 and int(want[again][0]) == 5
+        assert np.array_equal(got[doubled], want[doubled]), "run %d" % i
+    # released from another session's point of view as well: closing must not throw
+    replay.set_replay(False)
+    replay.close()
+    eager.close()
+
+
+@pytest.mark.gpu
 def test_fused_graph_is_bit_identical_to_the_graph_as_written(mf, rt, dev):
     rng = np.random.default_rng(7)
     for batch, seq, hidden, heads, ffn in ((2, 16, 64, 4, 128), (3, 7, 96, 3, 200), (4, 128, 256, 4, 1024),

@@ -151,7 +151,15 @@ size_t FlexAllocator::bucket(size_t len) {
 }
 
 FlexAllocator::~FlexAllocator() {
-  // blocks still handed out at this point are a bug of the owner; the cache is returned
+  // blocks still handed out at this point are a bug of the owner; the cache is returned, and with it what a
+  // recording left reserved or freed while pinning (its owner may be gone without having given them back)
+  {
+    std::lock_guard<std::mutex> lk(_mtx);
+    for (auto& kv : _reserved) _cached.emplace(kv.second, kv.first);
+    for (auto& kv : _pinnedFree) _cached.emplace(kv.first, kv.second);
+    _reserved.clear();
+    _pinnedFree.clear();
+  }
   releaseDownTo(0);
 }
 
@@ -342,6 +350,14 @@ inline void* current_stream() {
   return s->getStream();
 }
 
+// the stream for an operation the host waits on (copies to and from host memory)
+inline void* current_stream_for_host_transfer(const char* what) {
+  auto* s = dynamic_cast<ROCMSession*>(Session::getThreadDefault());
+  if (s == nullptr) throw RuntimeError("the thread's default session is not a ROCm session");
+  if (s->recording()) throw RuntimeError(std::string(what) + ": not possible while the session's stream records a graph");
+  return s->getStream();
+}
+
 template <class T>
 constexpr int type_code();
 template <> constexpr int type_code<int8_t>() { return TFCC_ROCM_S8; }
@@ -360,12 +376,13 @@ template <class T>
 class ROCMDataInterface : public DataInterface<T> {
  public:
   void set(T* dst, const T* data, size_t len) override {
-    check(tfcc_rocm_memcpy_h2d(current_stream(), dst, data, len * sizeof(T)));
+    check(tfcc_rocm_memcpy_h2d(current_stream_for_host_transfer("data::set"), dst, data, len * sizeof(T)));
   }
   void set(Variable<T>& a, const T* data) override { set(a.data(), data, a.size()); }
   void set(Variable<T>& a, std::vector<T>&& data) override { set(a.data(), data.data(), a.size()); }
   void get(const Tensor<T>& a, T* data) override {
-    check(tfcc_rocm_memcpy_d2h(current_stream(), data, a.data(), static_cast<size_t>(a.size()) * sizeof(T)));
+    check(tfcc_rocm_memcpy_d2h(current_stream_for_host_transfer("data::get"), data, a.data(),
+                               static_cast<size_t>(a.size()) * sizeof(T)));
   }
   void zeros(Variable<T>& a) override {
     check(tfcc_rocm_fill_async(current_stream(), a.data(), 0, sizeof(T), a.size()));
@@ -381,8 +398,32 @@ class ROCMDataInterface : public DataInterface<T> {
     std::memcpy(&bits, &value, sizeof(T));
     check(tfcc_rocm_fill_async(current_stream(), a.data(), bits, sizeof(T), a.size()));
   }
-  void castFrom(const void* source, int sourceCode, Variable<T>& result) override {
-    check(tfcc_rocm_cast(current_stream(), source, sourceCode, result.data(), ElementCode<T>::value, result.size()));
+  // the ten conversions of the reference's interface over the one conversion kernel
+  template <class SRC>
+  Variable<T> castFrom(const Tensor<SRC>& a) {
+    Variable<T> result(a.shape());
+    if (a.size() > 0)
+      check(tfcc_rocm_cast(current_stream(), a.data(), ElementCode<SRC>::value, result.data(), ElementCode<T>::value, result.size()));
+    return result;
+  }
+  Variable<T> cast(const Tensor<float>& a) override { return castFrom(a); }
+  Variable<T> cast(const Tensor<double>& a) override { return castFrom(a); }
+  Variable<T> cast(const Tensor<int8_t>& a) override { return castFrom(a); }
+  Variable<T> cast(const Tensor<uint8_t>& a) override { return castFrom(a); }
+  Variable<T> cast(const Tensor<int16_t>& a) override { return castFrom(a); }
+  Variable<T> cast(const Tensor<uint16_t>& a) override { return castFrom(a); }
+  Variable<T> cast(const Tensor<int32_t>& a) override { return castFrom(a); }
+  Variable<T> cast(const Tensor<uint32_t>& a) override { return castFrom(a); }
+  Variable<T> cast(const Tensor<int64_t>& a) override { return castFrom(a); }
+  Variable<T> cast(const Tensor<uint64_t>& a) override { return castFrom(a); }
+  // b[i] = a[i] ? 1 : 0 (tfcc/mkl/interfaces/tfcc_mkldatainterface.cpp:87-93): the comparison against zero
+  Variable<uint8_t> cast_to_boolean(const Tensor<T>& a) override {
+    Variable<uint8_t> result(a.shape());
+    const T zero = static_cast<T>(0);
+    if (a.size() > 0)
+      check(tfcc_rocm_compare_value(current_stream(), TFCC_ROCM_COMPARE_UNEQUAL, a.data(), ElementCode<T>::value, a.size(), &zero,
+                                    result.data()));
+    return result;
   }
   Variable<T> copy(const Tensor<T>& a) override {
     Variable<T> r(a.shape());
@@ -1046,7 +1087,10 @@ ROCMSession::~ROCMSession() {
   tfcc_rocm_stream_destroy(_stream);
 }
 
-void ROCMSession::sync() const { check(tfcc_rocm_stream_synchronize(_stream)); }
+void ROCMSession::sync() const {
+  if (_recording) throw RuntimeError("Session::sync: not possible while the session's stream records a graph");
+  check(tfcc_rocm_stream_synchronize(_stream));
+}
 
 namespace {
 

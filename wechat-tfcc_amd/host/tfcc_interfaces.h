@@ -83,8 +83,19 @@ class DataInterface {
   virtual void ones(Variable<T>&) { throw NotImplementedError(); }
   virtual void fill(Variable<T>&, T) { throw NotImplementedError(); }  // every element = the value (an addition)
   virtual Variable<T> copy(const Tensor<T>&) { throw NotImplementedError(); }
-  // static_cast of `total` elements of the type with code `sourceCode` (ElementCode) into a tensor of this type
-  virtual void castFrom(const void* /*source*/, int /*sourceCode*/, Variable<T>& /*result*/) { throw NotImplementedError(); }
+  // element-wise static_cast into this interface's type, one virtual per source type, and the conversion to
+  // 0 / 1 bytes (tfcc/core/interfaces/tfcc_datainterface.h:40-53)
+  virtual Variable<T> cast(const Tensor<float>&) { throw NotImplementedError(); }
+  virtual Variable<T> cast(const Tensor<double>&) { throw NotImplementedError(); }
+  virtual Variable<T> cast(const Tensor<int8_t>&) { throw NotImplementedError(); }
+  virtual Variable<T> cast(const Tensor<uint8_t>&) { throw NotImplementedError(); }
+  virtual Variable<T> cast(const Tensor<int16_t>&) { throw NotImplementedError(); }
+  virtual Variable<T> cast(const Tensor<uint16_t>&) { throw NotImplementedError(); }
+  virtual Variable<T> cast(const Tensor<int32_t>&) { throw NotImplementedError(); }
+  virtual Variable<T> cast(const Tensor<uint32_t>&) { throw NotImplementedError(); }
+  virtual Variable<T> cast(const Tensor<int64_t>&) { throw NotImplementedError(); }
+  virtual Variable<T> cast(const Tensor<uint64_t>&) { throw NotImplementedError(); }
+  virtual Variable<uint8_t> cast_to_boolean(const Tensor<T>&) { throw NotImplementedError(); }
 };
 
 template <class T>
@@ -672,13 +683,17 @@ Variable<T> layer_normalization(const Tensor<T>& a, const Tensor<T>& gamma, cons
 }  // namespace nn
 
 namespace data {
-// tfcc::data::cast<DST>(a): element-wise static_cast
+// tfcc::data::cast<DST>(a): element-wise static_cast (tfcc/core/operations/tfcc_data.h)
 template <class DST, class SRC>
 Variable<DST> cast(const Tensor<SRC>& a) {
-  Variable<DST> result(a.shape());
-  if (a.size() == 0) return result;
-  Operation<DST>::getCurrentInterface().getDataInterface().castFrom(a.data(), ElementCode<SRC>::value, result);
-  return result;
+  if (a.size() == 0) return Variable<DST>(a.shape());
+  return Operation<DST>::getCurrentInterface().getDataInterface().cast(a);
+}
+// tfcc::data::cast_to_boolean(a): 1 where the element is not zero, else 0
+template <class T>
+Variable<uint8_t> cast_to_boolean(const Tensor<T>& a) {
+  if (a.size() == 0) return Variable<uint8_t>(a.shape());
+  return Operation<T>::getCurrentInterface().getDataInterface().cast_to_boolean(a);
 }
 }  // namespace data
 

@@ -39,6 +39,7 @@ class ROCMDevice : public Device {
 class ROCMSession : public Session {
   ROCMDevice& _device;
   void* _stream;  // hipStream_t
+  bool _recording = false;  // the stream's launches are being recorded into a graph, not run
 
  public:
   explicit ROCMSession(ROCMDevice& device);
@@ -48,6 +49,11 @@ class ROCMSession : public Session {
   Device& getDevice() override { return _device; }
   const Device& getDevice() const override { return _device; }
   void* getStream() const { return _stream; }
+  // While the stream records (a HIP graph capture), nothing may wait for it or move data between host and device:
+  // sync(), data::get and data::set throw RuntimeError before they touch the stream, so that the recording itself
+  // stays valid and can be ended in the ordinary way by whoever began it.
+  void setRecording(bool recording) { _recording = recording; }
+  bool recording() const { return _recording; }
 };
 
 // Creates (once per process) one ROCMDevice per GPU and gives the calling thread a device and a

@@ -469,61 +469,85 @@ std::string Graph::errorString(const std::string& what, size_t node) {
   return reason;
 }
 
+void Graph::runSteps() {
+  for (const Step& step : _steps) {
+    try {
+      step.run();
+    } catch (std::exception& e) {
+      throw RuntimeError(errorString(e.what(), step.node));
+    }
+  }
+}
+
 void Graph::process() {
   if (!_built) buildGraph();
   if (_captured) {
     rocm_check(tfcc_rocm_graph_launch(_graphExec, session_stream()));
     return;
   }
-  const bool record = _replayWanted && _warm;
+  const bool record = _replayWanted && _warm && !_captureFailed;
+  if (!record) {
+    runSteps();
+    _warm = true;
+    return;
+  }
   Session* session = Session::getThreadDefault();
-  void* stream = nullptr;
-  if (record) {
-    stream = session_stream();
-    session->getAllocator().beginPinning();
+  auto* rocmSession = dynamic_cast<ROCMSession*>(session);
+  void* stream = session_stream();
+  session->getAllocator().beginPinning();
+  try {
     rocm_check(tfcc_rocm_stream_begin_capture(stream));
+  } catch (...) {
+    session->getAllocator().unpin(session->getAllocator().endPinning());
+    throw;
   }
-  std::string failure;
-  for (const Step& step : _steps) {
-    try {
-      step.run();
-    } catch (std::exception& e) {
-      failure = errorString(e.what(), step.node);
-      break;
-    }
+  // From here to the end of the recording the session refuses what a recording cannot hold (waiting for the
+  // stream, copies to and from host memory) before the stream sees it: such a step throws, the recording
+  // stays valid and is ended and dropped below.
+  rocmSession->setRecording(true);
+  bool stepFailed = false;
+  try {
+    runSteps();
+  } catch (std::exception&) {
+    stepFailed = true;  // a step that reads results on the host, or a real error: the step-by-step run below tells
   }
-  if (record) {
-    void* exec = nullptr;
-    const int status = tfcc_rocm_stream_end_capture(stream, &exec);
-    _pinned = session->getAllocator().endPinning();
-    if (status == TFCC_ROCM_OK && failure.empty()) {
-      _graphExec = exec;
-      _captured = true;
-      // the recording only described the work; run it once so this call produces its outputs
-      rocm_check(tfcc_rocm_graph_launch(_graphExec, stream));
-    } else {
-      if (exec) tfcc_rocm_graph_destroy(exec);
-      session->getAllocator().unpin(_pinned);
-      _pinned.clear();
-      if (failure.empty()) throw ROCMRuntimeError(status, tfcc_rocm_last_error_string());
-    }
+  rocmSession->setRecording(false);
+  void* exec = nullptr;
+  const int status = tfcc_rocm_stream_end_capture(stream, &exec);
+  std::vector<void*> pinned = session->getAllocator().endPinning();
+  if (status == TFCC_ROCM_OK && !stepFailed) {
+    _graphExec = exec;
+    _pinned = std::move(pinned);
+    _replaySession = session;
+    _captured = true;
+    // the recording only described the work; run it once so this call produces its outputs
+    rocm_check(tfcc_rocm_graph_launch(_graphExec, stream));
+    return;
   }
-  if (!failure.empty()) throw RuntimeError(failure);
-  _warm = true;
+  // Not recordable.  Nothing has run yet (the steps before the failure were only recorded), so this call still
+  // owes its outputs: give the blocks back, remember not to try again, and run step by step.  An error that is
+  // not about recording shows up again there and is reported as usual.
+  if (exec) tfcc_rocm_graph_destroy(exec);
+  session->getAllocator().unpin(pinned);
+  _captureFailed = true;
+  runSteps();
 }
 
 void Graph::enableReplay(bool enable) {
   _replayWanted = enable;
   if (!enable) {
     if (_graphExec) {
-      Session* session = Session::getThreadDefault();
-      if (session) session->sync();
+      // the stream the recording runs on and the allocator its blocks came from belong to the session it was made
+      // on, whichever thread or session asks for the release
+      if (_replaySession) _replaySession->sync();
       rocm_check(tfcc_rocm_graph_destroy(_graphExec));
-      if (session) session->getAllocator().unpin(_pinned);
+      if (_replaySession) _replaySession->getAllocator().unpin(_pinned);
     }
     _graphExec = nullptr;
+    _replaySession = nullptr;
     _pinned.clear();
     _captured = false;
+    _captureFailed = false;
     _warm = false;
   }
 }
@@ -606,19 +630,22 @@ Model::PerSession& Model::initializeGraphs(Session* session) {
   std::unique_lock<std::mutex> lk(_mutex);
   auto it = _sessions.find(session);
   if (it != _sessions.end()) return it->second;
-  PerSession& data = _sessions[session];
   Device* device = &session->getDevice();
   auto& store = _constants[device];
   if (!store) store.reset(new ConstantStore(*_npz, device));
   ConstantStore& constants = *store;
   lk.unlock();
+  // built aside and entered only when every graph stands: a constructor that throws (a constant that is missing,
+  // a dtype nobody knows) must not leave an entry with no graphs behind for the next call to index
+  PerSession fresh;
+  for (const proto::Graph& g : _proto.graphs) fresh.graphs.emplace_back(new Graph(*this, g, constants));
+  for (auto& g : fresh.graphs) g->buildGraph();
   std::weak_ptr<bool> alive = _alive;
   session->registerReleaseCallback([this, alive](const Session* s) {
     if (!alive.expired()) releaseGraphs(s);
   });
-  for (const proto::Graph& g : _proto.graphs) data.graphs.emplace_back(new Graph(*this, g, constants));
-  for (auto& g : data.graphs) g->buildGraph();
-  return data;
+  lk.lock();
+  return _sessions.emplace(session, std::move(fresh)).first->second;
 }
 
 void Model::releaseGraphs(const Session* session) {

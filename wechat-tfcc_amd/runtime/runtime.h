@@ -308,9 +308,12 @@ class Graph {
   bool _warm = false;            // one step-by-step run has filled the allocator's cache
   void* _graphExec = nullptr;
   bool _captured = false;
+  bool _captureFailed = false;   // a recording was tried and a step could not be recorded: run step by step
+  Session* _replaySession = nullptr;  // the session the recording was made on: its stream and allocator own it
   std::vector<void*> _pinned;    // blocks the recording uses that no symbol owns
   std::set<std::string> _inputOwned;  // tensor inputs held in buffers of the graph's own
   void enableReplayReset();
+  void runSteps();
 
   std::string errorString(const std::string& what, size_t node);
 
