@@ -389,6 +389,37 @@ def test_sgemm_exact_cases(pkg, T):
     assert mm(x, y, np.array([1, 2, 3, 4], np.float32)).tolist() == [[21, 25, 29, 33], [57, 70, 83, 96]]
 
 
+@pytest.mark.parametrize("m,n,k", [(64, 64, 64), (128, 96, 40), (256, 512, 512), (8, 128, 64), (1, 4096, 512),
+                                   (1024, 768, 768)])
+def test_sgemm_keeps_subnormal_operands_and_results(pkg, T, m, n, k):
+    """fp32 values below 2^-126.  The reference's dispatch thread sets flush-to-zero and denormals-are-zero before it
+    runs any kernel (tfcc/mkl/framework/tfcc_mkldevice.cpp:126-128), so on the CPU a subnormal operand counts as 0 and a
+    subnormal result becomes 0.  The fp32 matrix ops and the streaming kernel of this backend follow IEEE gradual
+    underflow instead: operands are taken as they are and subnormal results are produced.  Pinned here on all tile
+    families (register-staged, direct-to-LDS with and without K groups, few-rows streaming kernel) with powers of two,
+    whose products and sums are exact whatever the order; the two oracles differ in exactly the elements named."""
+    a = np.zeros((m, k), np.float32)
+    b = np.zeros((k, n), np.float32)
+    a[0, 0], b[0, :] = np.float32(2.0 ** -130), np.float32(2.0 ** 10)        # subnormal operand, normal product
+    ieee = np.zeros((m, n), np.float64)
+    flushed = np.zeros((m, n), np.float64)
+    ieee[0, :] = 2.0 ** -120                                                   # DAZ: the operand is 0
+    if m > 1:
+        a[1, 1], b[1, :] = np.float32(2.0 ** -70), np.float32(2.0 ** -70)      # normal operands, subnormal product
+        ieee[1, :] = 2.0 ** -140                                               # FTZ: the result is 0
+    if m > 2:
+        a[2, 2:], b[2:, :] = np.float32(2.0 ** -100), np.float32(2.0 ** -30)   # k - 2 subnormal products of 2^-130
+        ieee[2, :] = (k - 2) * 2.0 ** -130
+        flushed[2, :] = np.nan  # depends on where an implementation flushes its partial sums: not compared
+    got = T.n(pkg.blas_matmul(T.t(a), T.t(b))).astype(np.float64)
+    assert np.array_equal(got, ieee)
+    rows = slice(0, min(m, 2))
+    assert np.all(got[rows] != flushed[rows]) and np.all(flushed[rows] == 0.0)
+    # the oracle (fp64 accumulation, one rounding to fp32) is the IEEE flavour too
+    want32, _ = O.sgemm(a, b, None, want64=True)
+    assert np.array_equal(want32.astype(np.float64), ieee)
+
+
 @pytest.mark.parametrize("shape_a,shape_b", [
     ((1, 1), (1, 1)), ((5, 7), (7, 3)), ((33, 65), (65, 31)), ((99, 98), (98, 97)),
     ((3, 50, 20), (3, 20, 30)), ((4, 25, 40), (40, 24)), ((31, 48), (2, 48, 52)), ((2, 3, 17, 9), (2, 3, 9, 33)),
