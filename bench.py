@@ -8,10 +8,14 @@ Headline workload (BASELINE.json configs[2], the one the north-star target is qu
 One step = one such product with inputs resident in HBM.  value = 2*M*N*K / time, in TOP/s.
 
 The same JSON line carries
-  roofline      the dominant kernel against the int8 MFMA peak (5.0 POP/s dense)
+  roofline      the dominant kernel against the int8 MFMA peak (5.0 POP/s dense), next to what the matrix
+                cores sustain alone on this box, and the same kernel after a long warm-up ("settled") and
+                as a short burst after idle ("burst")
   cpu_baseline  the reference's own AVX2 quantized matmul + requantize (oracle/_ref, kind
                 "reference") or, where that library is absent, the scalar C oracle (kind "port"),
-                timed on this host's cores on a bounded sample
+                timed on this host's cores on a bounded sample, with all threads and with the four the
+                reference's test harness uses; an fp32 leg (C1 and the GEMMs of C4) through a plain
+                OpenMP port and through the CPU BLAS torch ships; the CPU model
   other         the remaining BASELINE configs (fp32 GEMM + bias, attention-shaped batched fp32,
                 skinny int8 decode GEMV, int32-writing variant), each with its own roofline figure
 
@@ -32,6 +36,29 @@ sys.path.insert(0, ROOT)
 PEAK_INT8_TOPS = 5000.0   # MI355X dense int8 MFMA
 PEAK_FP32_TFLOPS = 157.3  # MI355X fp32 MFMA
 PEAK_HBM_GBS = 8000.0     # MI355X HBM3E
+
+
+_bench_lib = None
+
+
+def bench_lib():
+    """The benchmark's own measuring aids (wechat-tfcc_amd/csrc/probe.h): not part of the product library."""
+    global _bench_lib
+    if _bench_lib is None:
+        path = os.path.join(ROOT, "wechat-tfcc_amd", "libtfcc_bench.so")
+        if not os.path.exists(path):
+            sys.exit("libtfcc_bench.so is missing: run __graft_entry__.build() first")
+        lib = C.CDLL(path)
+        lib.tfcc_bench_probe_mfma.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_uint, C.c_uint, C.c_void_p]
+        lib.tfcc_bench_probe_read.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_uint, C.c_void_p]
+        lib.tfcc_bench_probe_launch.argtypes = [C.c_void_p, C.c_void_p]
+        _bench_lib = lib
+    return _bench_lib
+
+
+def probe_check(status):
+    if status != 0:
+        sys.exit("measuring probe failed with status %d" % status)
 
 
 def time_launches(torch, fn, steps, warmup, pkg=None, stream=0):
@@ -108,16 +135,39 @@ def make_c3_step(torch, pkg, ta, tb, rs, cs, ranges, out_range, want_acc, colsum
     return step
 
 
+def cpu_model_name():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
 def cpu_baseline(a, b, size):
-    """The reference's CPU path on this host: its AVX2 quantized matmul (offset matrix + kernel) followed
-    by its AVX2 requantize, both from oracle/_ref; falls back to the scalar C oracle on a smaller sample."""
+    """The reference's CPU path on this host's cores, on bounded samples (about 25 s in all).
+    int8 (the headline's workload): the reference's own AVX2 quantized matmul (offset matrix + kernel) followed by its
+    AVX2 requantize, both from oracle/_ref, with every thread the process may use and with the four threads the
+    reference's test harness runs on (tfcc/test/environment.cpp:40); the scalar C oracle on a smaller sample where
+    oracle/_ref has not been built.
+    fp32 (C1 and the six GEMMs of C4's layer): the reference's arithmetic lives in oneDNN 1.8.1, which is not in this
+    image, so two stand-ins are timed: a plain OpenMP port in the oracle library (kind "port") and torch's CPU matmul
+    (the BLAS torch ships: a vendor library, not oneDNN 1.8.1)."""
     sys.path.insert(0, os.path.join(ROOT, "tests"))
     import oracle_lib as O
     cores = len(os.sched_getaffinity(0))
-    threads = int(os.environ.get("OMP_NUM_THREADS", cores))
+    threads = min(int(os.environ.get("OMP_NUM_THREADS", cores)), cores)
+    orc = O.oracle()
+    orc.oracle_set_num_threads.argtypes = [C.c_int]
+    orc.oracle_sgemm_f32_timing.argtypes = [C.c_void_p] * 4 + [C.c_uint] * 3
+    orc.oracle_sgemm_f32_timing.restype = None
     ref = O.ref()
     ranges = (-128.0, 127.0, -128.0, 127.0)
-    if ref is not None:
+    result = {}
+
+    def int8_leg(nthreads, budget):
+        orc.oracle_set_num_threads(nthreads)  # one OpenMP runtime in the process: the reference's kernels follow it
         rs, cs = O.reduce_sum(a, True), O.reduce_sum(b, False)
         oa, ob = O.qmatmul_offsets(*ranges, lib=ref)
         mn_c, mx_c = O.qmatmul_range(*ranges, lib=ref)
@@ -130,20 +180,86 @@ def cpu_baseline(a, b, size):
                                       q.reshape(-1))
             reps += 1
             dt = time.perf_counter() - t0
-            if dt > 10.0 or reps >= 400:
+            if dt > budget or reps >= 400:
                 break
-        tops = 2.0 * size ** 3 * reps / dt / 1e12
-        return {"value": round(tops, 4), "unit": "TOP/s", "cores": min(threads, cores), "kind": "reference",
-                "sample": "%d full %d^3 products + requantize through the reference's AVX2 kernels (oracle/_ref), "
-                          "%.1f s, OMP threads %d" % (reps, size, dt, threads)}
-    sub = 1024
-    sa, sb = np.ascontiguousarray(a[:sub, :sub]), np.ascontiguousarray(b[:sub, :sub])
-    t0 = time.perf_counter()
-    c = O.qgemm(sa, sb, -128, 0)
-    O.requantize_s32_u8(c, -2147483648.0, 2147483648.0, -128.0 * sub * 64.0, 127.0 * sub * 64.0)
-    dt = time.perf_counter() - t0
-    return {"value": round(2.0 * sub ** 3 / dt / 1e12, 5), "unit": "TOP/s", "cores": 1, "kind": "port",
-            "sample": "one %d^3 product + requantize through the scalar C oracle, %.1f s" % (sub, dt)}
+        return 2.0 * size ** 3 * reps / dt / 1e12, reps, dt
+
+    if ref is not None:
+        tops, reps, dt = int8_leg(threads, 8.0)
+        result = {"value": round(tops, 4), "unit": "TOP/s", "cores": threads, "kind": "reference",
+                  "sample": "%d full %d^3 products + requantize through the reference's AVX2 kernels (oracle/_ref), "
+                            "%.1f s, %d OpenMP threads" % (reps, size, dt, threads)}
+        tops4, reps4, dt4 = int8_leg(min(4, threads), 5.0)
+        result["threads_4"] = {"value": round(tops4, 4), "unit": "TOP/s", "cores": min(4, threads),
+                               "sample": "%d products, %.1f s (the thread count of the reference's test harness)" % (reps4, dt4)}
+    else:
+        sub = 1024
+        sa, sb = np.ascontiguousarray(a[:sub, :sub]), np.ascontiguousarray(b[:sub, :sub])
+        t0 = time.perf_counter()
+        c = O.qgemm(sa, sb, -128, 0)
+        O.requantize_s32_u8(c, -2147483648.0, 2147483648.0, -128.0 * sub * 64.0, 127.0 * sub * 64.0)
+        dt = time.perf_counter() - t0
+        result = {"value": round(2.0 * sub ** 3 / dt / 1e12, 5), "unit": "TOP/s", "cores": 1, "kind": "port",
+                  "sample": "one %d^3 product + requantize through the scalar C oracle, %.1f s" % (sub, dt)}
+    result["cpu_model"] = cpu_model_name()
+    result["host_cores"] = cores
+
+    # ---- fp32
+    rng = np.random.default_rng(3)
+    shapes = {"c1_128x768x3072_bias": [(128, 768, 3072)],
+              "c4_layer_gemms_b8_s128": [(1024, 768, 768)] * 4 + [(1024, 768, 3072), (1024, 3072, 768)] +
+                                        [(128, 64, 128)] * 96 + [(128, 128, 64)] * 96}
+    fp32 = {}
+    try:
+        import torch
+    except ImportError:
+        torch = None
+    for name, products in shapes.items():
+        flop = sum(2.0 * m * n * k for m, k, n in products)
+        distinct = sorted(set(products))
+        ops = {sh: (rng.uniform(-1, 1, (sh[0], sh[1])).astype(np.float32), rng.uniform(-1, 1, (sh[1], sh[2])).astype(np.float32),
+                    rng.uniform(-0.1, 0.1, sh[2]).astype(np.float32), np.empty((sh[0], sh[2]), np.float32)) for sh in distinct}
+        entry = {"gflop_per_pass": round(flop / 1e9, 3)}
+        for label, nthreads in (("all_threads", threads), ("threads_4", min(4, threads))):
+            orc.oracle_set_num_threads(nthreads)
+
+            def port_pass():
+                for sh in products:
+                    x, w, bias, out = ops[sh]
+                    orc.oracle_sgemm_f32_timing(x.ctypes.data, w.ctypes.data, bias.ctypes.data, out.ctypes.data, sh[0], sh[2], sh[1])
+            port_pass()
+            reps, t0 = 0, time.perf_counter()
+            while True:
+                port_pass()
+                reps += 1
+                dt = time.perf_counter() - t0
+                if dt > 1.5 or reps >= 200:
+                    break
+            entry["port_%s" % label] = {"gflops": round(flop * reps / dt / 1e9, 1), "cores": nthreads, "kind": "port",
+                                        "sample": "%d passes, %.1f s, OpenMP rows x vectorised inner loop" % (reps, dt)}
+            if torch is not None:
+                torch.set_num_threads(nthreads)
+                tops_ = {sh: (torch.from_numpy(v[0]), torch.from_numpy(v[1]), torch.from_numpy(v[2])) for sh, v in ops.items()}
+
+                def torch_pass():
+                    for sh in products:
+                        x, w, bias = tops_[sh]
+                        torch.addmm(bias, x, w)
+                torch_pass()
+                reps, t0 = 0, time.perf_counter()
+                while True:
+                    torch_pass()
+                    reps += 1
+                    dt = time.perf_counter() - t0
+                    if dt > 1.5 or reps >= 500:
+                        break
+                entry["vendor_blas_%s" % label] = {
+                    "gflops": round(flop * reps / dt / 1e9, 1), "cores": nthreads,
+                    "kind": "torch %s CPU addmm: vendor BLAS, not the reference's oneDNN 1.8.1" % torch.__version__,
+                    "sample": "%d passes, %.1f s" % (reps, dt)}
+        fp32[name] = entry
+    result["fp32"] = fp32
+    return result
 
 
 def bench_other(torch, pkg, dev, steps, warmup, c3):
@@ -154,9 +270,16 @@ def bench_other(torch, pkg, dev, steps, warmup, c3):
     lib = pkg.lib()
     stream = torch.cuda.current_stream().cuda_stream
 
-    def sgemm_case(name, shape_a, shape_b, bias, sets=4):
+    LLC_BYTES = 256 << 20  # last-level cache: a rotation of operand sets must exceed it to measure HBM
+
+    def sets_beyond_llc(bytes_per_set):
+        return max(2, int(1.25 * LLC_BYTES / bytes_per_set) + 1)
+
+    def sgemm_case(name, shape_a, shape_b, bias, sets=None):
         p = pkg.matmul_plan(shape_a, shape_b, None if not bias else (shape_b[-1],))
-        # several buffer sets so that a small working set does not simply sit in the caches
+        # operand sets rotated over more bytes than the last-level cache holds (sets=1: compute-bound, no rotation)
+        per_set = 4 * (int(np.prod(shape_a)) + int(np.prod(shape_b)) + int(np.prod(p["shape"])))
+        sets = sets or sets_beyond_llc(per_set)
         bufs = []
         for _ in range(sets):
             a = torch.randn(shape_a, device=dev, dtype=torch.float32)
@@ -184,12 +307,13 @@ def bench_other(torch, pkg, dev, steps, warmup, c3):
     sgemm_case("c1_fp32_128x768x3072_bias", (128, 768), (768, 3072), True)
     sgemm_case("c2_fp32_qk_16x12x128x64x128", (16, 12, 128, 64), (16, 12, 64, 128), False)
     sgemm_case("c2_fp32_pv_16x12x128x128x64", (16, 12, 128, 128), (16, 12, 128, 64), False)
-    sgemm_case("c4_fp32_ffn_up_1024x768x3072_bias", (8, 128, 768), (768, 3072), True)
+    sgemm_case("c4_fp32_ffn_up_1024x768x3072_bias", (8, 128, 768), (768, 3072), True, sets=4)
 
     # C2, second case: a [1, 12, 64, 64] weight broadcast over the batch of a [16, 12, 128, 64] input
-    def broadcast_case(name, shape_a, shape_b, sets=4):
+    def broadcast_case(name, shape_a, shape_b):
         p = pkg.matmul_plan(shape_a, shape_b)
         g = p["grid"]
+        sets = sets_beyond_llc(4 * (int(np.prod(shape_a)) + int(np.prod(shape_b)) + int(np.prod(p["shape"]))))
         bufs = []
         for _ in range(sets):
             a = torch.randn(shape_a, device=dev, dtype=torch.float32)
@@ -220,7 +344,8 @@ def bench_other(torch, pkg, dev, steps, warmup, c3):
     broadcast_case("c2_fp32_broadcast_16x12x128x64_by_1x12x64x64", (16, 12, 128, 64), (1, 12, 64, 64))
 
     # C2, first product with K used as stored: scores = Q K^T from K [16, 12, 128, 64] (B given transposed)
-    def qkt_case(name, B, H, S, D, sets=4):
+    def qkt_case(name, B, H, S, D):
+        sets = sets_beyond_llc(4 * (2 * B * H * S * D + B * H * S * S))
         bufs = []
         for _ in range(sets):
             q = torch.randn((B, H, S, D), device=dev, dtype=torch.float32)
@@ -251,7 +376,8 @@ def bench_other(torch, pkg, dev, steps, warmup, c3):
     qkt_case("c2_fp32_qkt_k_as_stored_16x12x128x64", 16, 12, 128, 64)
 
     # C2 as one launch: softmax(q k^T / 8) v on [batch, seq, heads, size] tensors, 16 x 12 heads of 128 x 64
-    def attention_case(name, B, H, S, D, sets=4):
+    def attention_case(name, B, H, S, D):
+        sets = sets_beyond_llc(4 * 4 * B * S * H * D)
         bufs = []
         for _ in range(sets):
             q, k, v = (torch.randn((B, S, H, D), device=dev, dtype=torch.float32) for _ in range(3))
@@ -294,14 +420,12 @@ def bench_other(torch, pkg, dev, steps, warmup, c3):
     # up to eight rows of A in fp32 (C5's shape and a square weight): one streaming pass over B
     sgemm_case("fp32_few_rows_m1_4096x11008", (1, 4096), (4096, 11008), False, sets=2)
     sgemm_case("fp32_few_rows_m8_4096x11008", (8, 4096), (4096, 11008), False, sets=2)
-    sgemm_case("fp32_few_rows_m8_4096x4096", (8, 4096), (4096, 4096), False, sets=4)
+    sgemm_case("fp32_few_rows_m8_4096x4096", (8, 4096), (4096, 4096), False)
     # what the fp32 matrix cores sustain alone (register-resident loop of the 4096^3 instruction count)
     probe_out = torch.empty(1024 * 256, dtype=torch.int32, device=dev)
     for label, changing in (("changing", 1),):
         def step():
-            st = lib.tfcc_rocm_probe_mfma(stream, 1, changing, 1024, 2048, probe_out.data_ptr())
-            if st != 0:
-                pkg.check(st)
+            probe_check(bench_lib().tfcc_bench_probe_mfma(stream, 1, changing, 1024, 2048, probe_out.data_ptr()))
         ms = time_launches(torch, step, max(10, steps // 10), max(3, warmup // 10), pkg, stream)
         out["probe_fp32_matrix_cores_alone_%s_operands" % label] = {
             "ms": round(ms, 5), "tflops": round(1024 * 4 * 4 * 2048 * 4096.0 / ms / 1e9, 2)}
@@ -371,17 +495,13 @@ def bench_other(torch, pkg, dev, steps, warmup, c3):
         def step():
             i = idx[0] % sets
             idx[0] += 1
-            st = lib.tfcc_rocm_probe_read(stream, bs[i].data_ptr(), k * n, blocks, probe_word.data_ptr())
-            if st != 0:
-                pkg.check(st)
+            probe_check(bench_lib().tfcc_bench_probe_read(stream, bs[i].data_ptr(), k * n, blocks, probe_word.data_ptr()))
         ms = time_launches(torch, step, max(steps, 50), warmup, pkg, stream)
         out["probe_read_only_45mb_%d_workgroups" % blocks] = {"ms": round(ms, 5), "gbs": round(k * n / ms / 1e6, 1),
                                                                "frac_hbm": round(k * n / ms / 1e6 / PEAK_HBM_GBS, 4)}
 
     def step():
-        st = lib.tfcc_rocm_probe_launch(stream, probe_word.data_ptr())
-        if st != 0:
-            pkg.check(st)
+        probe_check(bench_lib().tfcc_bench_probe_launch(stream, probe_word.data_ptr()))
     out["probe_empty_launch"] = {"ms": round(time_launches(torch, step, max(steps, 50), warmup, pkg, stream), 5)}
 
     # the same decode shapes on weights packed once (column slabs in matrix-core operand order)
@@ -509,8 +629,10 @@ def main():
                    "m": size, "n": size, "k": size},
         "roofline": {"bound": "mfma", "achieved": round(kernel_tops, 2), "peak": PEAK_INT8_TOPS, "unit": "TOP/s",
                      "frac": round(kernel_tops / PEAK_INT8_TOPS, 4), "traffic": None,
-                     "kernel": "qgemm_dma_kernel<256,256,2,4,2,true,false,true>", "kernel_ms": round(kernel_ms, 5),
-                     "algorithmic_ops_per_launch": ops},
+                     "kernel": "qgemm_w4_kernel<64,4,true,false,true>", "kernel_ms": round(kernel_ms, 5),
+                     "algorithmic_ops_per_launch": ops,
+                     "kernel_ms_is": "HIP events around the K timed launches / K: launch to launch, i.e. the kernel's own "
+                                     "duration (what a kernel trace reports) plus the gap between dependent launches"},
     }
     traffic_file = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(traffic_file):
@@ -522,9 +644,20 @@ def main():
     stream0 = torch.cuda.current_stream().cuda_stream
     for label, changing in (("matrix_cores_alone_constant_operands", 0), ("matrix_cores_alone_changing_operands", 1)):
         def probe():
-            pkg.check(pkg.lib().tfcc_rocm_probe_mfma(stream0, 0, changing, 512, 256, probe_out.data_ptr()))
-        ms = time_launches(torch, probe, args.steps, args.warmup)
+            probe_check(bench_lib().tfcc_bench_probe_mfma(stream0, 0, changing, 512, 256, probe_out.data_ptr()))
+        ms = time_launches(torch, probe, max(args.steps, 200), max(args.warmup, 50))
         result["roofline"][label] = round(512 * 4 * 4 * 256 * 65536.0 / ms / 1e9, 2)
+    result["roofline"]["frac_of_matrix_cores_alone_changing_operands"] = round(
+        kernel_tops / result["roofline"]["matrix_cores_alone_changing_operands"], 4)
+    # The two regimes of the same launch: after a long warm-up, when the clocks have settled under the power limit,
+    # and as a burst of a few launches right after the GPU sat idle (the first launches run at the idle clocks).
+    for label, (k_steps, k_warm, idle) in (("settled", (2000, 500, 0.0)), ("burst", (20, 5, 0.5))):
+        torch.cuda.synchronize()
+        if idle:
+            time.sleep(idle)
+        ms = time_launches(torch, step, k_steps, k_warm)
+        result["roofline"][label] = {"steps": k_steps, "warmup": k_warm, "idle_before_s": idle, "kernel_ms": round(ms, 5),
+                                     "achieved": round(ops / ms / 1e9, 2), "frac": round(ops / ms / 1e9 / PEAK_INT8_TOPS, 4)}
     if not args.no_other:
         # on a stream of its own (not the default stream) so that short kernels can be timed as graph replays
         side = torch.cuda.Stream()

@@ -97,6 +97,29 @@ void oracle_sgemm_strided_batched(const float* a, uint64_t strideA, const float*
   free(row);
 }
 
+/* The timing leg of the fp32 path: the same product with fp32 accumulation, rows dealt to OpenMP threads,
+ * the inner loop over a row of B left to the compiler's vectoriser (built for AVX2 where the host has it).
+ * This is what a straightforward CPU port of tfcc_mklblasinterface.cpp:41-118 costs without oneDNN's
+ * JIT kernels; it is measured, never compared bit for bit (its sums run in k order in fp32). */
+#include <omp.h>
+void oracle_set_num_threads(int threads) { if (threads > 0) omp_set_num_threads(threads); }
+int oracle_max_threads(void) { return omp_get_max_threads(); }
+
+__attribute__((target_clones("avx2,fma", "default"), optimize("O3")))
+void oracle_sgemm_f32_timing(const float* a, const float* b, const float* bias, float* c, unsigned m, unsigned n,
+                             unsigned k) {
+#pragma omp parallel for schedule(static)
+  for (unsigned i = 0; i < m; ++i) {
+    float* row = c + (size_t)i * n;
+    for (unsigned j = 0; j < n; ++j) row[j] = bias ? bias[j] : 0.f;
+    for (unsigned p = 0; p < k; ++p) {
+      const float av = a[(size_t)i * k + p];
+      const float* brow = b + (size_t)p * n;
+      for (unsigned j = 0; j < n; ++j) row[j] += av * brow[j];
+    }
+  }
+}
+
 /* ---------------------------------------------------------------------------------------------
  * quantized matmul
  * ------------------------------------------------------------------------------------------- */

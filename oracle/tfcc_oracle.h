@@ -199,6 +199,17 @@ void oracle_pytorch_gru_cell(unsigned batch, unsigned units, const float* state,
                              const float* stateValue, const float* gateBias, const float* candidateIBias,
                              const float* candidateHBias, float* result);
 /*
+ * Timing aids of the benchmark's CPU leg (not part of any parity check): the OpenMP thread count of this process,
+ * and C = A * B (+ bias) in fp32 with rows dealt to the threads - what a plain port of the reference's fp32 path
+ * (tfcc_mklblasinterface.cpp:41-118) costs without oneDNN.  Checked against oracle_sgemm_strided_batched to fp32
+ * tolerance only.
+ */
+void oracle_set_num_threads(int threads);
+int oracle_max_threads(void);
+void oracle_sgemm_f32_timing(const float* a, const float* b, const float* bias, float* c, unsigned m, unsigned n,
+                             unsigned k);
+
+/*
  * tfcc::rnn::lstm_forward / lstm_backward, tfcc/core/operations/tfcc_rnn.cpp:29-81, 83-135:
  * a [seq, batch, length], inputKernel [length, 4 hidden], stateKernel [hidden, 4 hidden], bias [4 hidden],
  * ih / ic [batch, hidden]; per step matmul(x_t, inputKernel), matmul(h, stateKernel), LSTM cell with forget 0.

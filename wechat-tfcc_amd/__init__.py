@@ -119,9 +119,6 @@ SYMBOLS = {
     "tfcc_rocm_sgemm_general": (_I, [_VP, _VP]),
     "tfcc_rocm_sgemm_grouped": (_I, [_VP, _VP, C.POINTER(_VP), C.POINTER(_VP), C.POINTER(_VP), _U, _U, _U, _U]),
     "tfcc_rocm_unary_f32": (_I, [_VP, _I, _VP, _U64, _VP]),
-    "tfcc_rocm_probe_mfma": (_I, [_VP, _I, _I, _U, _U, _VP]),
-    "tfcc_rocm_probe_read": (_I, [_VP, _VP, _U64, _U, _VP]),
-    "tfcc_rocm_probe_launch": (_I, [_VP, _VP]),
     "tfcc_rocm_softmax_div_f32": (_I, [_VP, _VP, _U64, _U, _F, _VP]),
     "tfcc_rocm_attention_f32_supported": (_I, [C.POINTER(AttentionDesc)]),
     "tfcc_rocm_attention_f32": (_I, [_VP, C.POINTER(AttentionDesc)]),

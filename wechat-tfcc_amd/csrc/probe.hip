@@ -2,10 +2,12 @@
 // limits them (no LDS, no memory), with operands that stay the same from one instruction to the next
 // and with operands that change every instruction, as the rows and columns of real matrices do.
 // A measuring aid for the benchmark (it says how far a GEMM kernel is from what the hardware delivers
-// at the clocks its power limit allows); nothing in the library calls it.
-#include "common.hpp"
+// at the clocks its power limit allows).  Built into the benchmark's own library, not the product's.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
 
-namespace tfcc_rocm {
+#include "probe.h"
+
 namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -102,31 +104,31 @@ __global__ void probe_empty_kernel(int* out) {
   if (out == nullptr && threadIdx.x == 1024) __builtin_trap();  // never: keeps the kernel from being dropped
 }
 
+// 0 = ok, 1 = bad argument, 2 = launch failed
+int launched() { return hipGetLastError() == hipSuccess ? 0 : 2; }
+
 }  // namespace
-}  // namespace tfcc_rocm
 
-using namespace tfcc_rocm;
-
-extern "C" int tfcc_rocm_probe_read(void* stream, const void* src, uint64_t bytes, unsigned blocks, int32_t* out) {
-  TFCC_REQUIRE(src && out, "probe: null argument");
-  TFCC_REQUIRE(bytes >= 16 && (uintptr_t)src % 16 == 0 && blocks > 0 && blocks <= 65536, "probe: 16-byte aligned source, 1..65536 blocks");
-  hipLaunchKernelGGL(probe_read_kernel, dim3(blocks), dim3(512), 0, as_stream(stream),
+extern "C" int tfcc_bench_probe_read(void* stream, const void* src, uint64_t bytes, unsigned blocks, int32_t* out) {
+  if (!(src && out)) return 1;
+  if (!(bytes >= 16 && (uintptr_t)src % 16 == 0 && blocks > 0 && blocks <= 65536)) return 1;
+  hipLaunchKernelGGL(probe_read_kernel, dim3(blocks), dim3(512), 0, reinterpret_cast<hipStream_t>(stream),
                      static_cast<const unsigned char*>(src), (unsigned long long)bytes, out);
-  return check_launch("probe");
+  return launched();
 }
 
-extern "C" int tfcc_rocm_probe_launch(void* stream, int32_t* out) {
-  TFCC_REQUIRE(out != nullptr, "probe: null argument");
-  hipLaunchKernelGGL(probe_empty_kernel, dim3(256), dim3(256), 0, as_stream(stream), out);
-  return check_launch("probe");
+extern "C" int tfcc_bench_probe_launch(void* stream, int32_t* out) {
+  if (!(out != nullptr)) return 1;
+  hipLaunchKernelGGL(probe_empty_kernel, dim3(256), dim3(256), 0, reinterpret_cast<hipStream_t>(stream), out);
+  return launched();
 }
 
-extern "C" int tfcc_rocm_probe_mfma(void* stream, int kind, int changing_operands, unsigned blocks, unsigned iters,
+extern "C" int tfcc_bench_probe_mfma(void* stream, int kind, int changing_operands, unsigned blocks, unsigned iters,
                                     int32_t* out) {
-  TFCC_REQUIRE(out != nullptr, "probe: null output (blocks * 256 words)");
-  TFCC_REQUIRE(blocks > 0 && blocks <= 65536 && iters > 0 && iters % 4 == 0, "probe: blocks 1..65536, iters a positive multiple of 4");
-  TFCC_REQUIRE(kind == 0 || kind == 1, "probe: kind 0 (int8 32x32x32) or 1 (fp32 32x32x2)");
-  hipStream_t s = as_stream(stream);
+  if (!(out != nullptr)) return 1;
+  if (!(blocks > 0 && blocks <= 65536 && iters > 0 && iters % 4 == 0)) return 1;
+  if (!(kind == 0 || kind == 1)) return 1;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
   if (kind == 0) {
     if (changing_operands) hipLaunchKernelGGL(probe_i8_kernel<true>, dim3(blocks), dim3(256), 0, s, iters, out);
     else hipLaunchKernelGGL(probe_i8_kernel<false>, dim3(blocks), dim3(256), 0, s, iters, out);
@@ -134,5 +136,5 @@ extern "C" int tfcc_rocm_probe_mfma(void* stream, int kind, int changing_operand
     if (changing_operands) hipLaunchKernelGGL(probe_f32_kernel<true>, dim3(blocks), dim3(256), 0, s, iters, out);
     else hipLaunchKernelGGL(probe_f32_kernel<false>, dim3(blocks), dim3(256), 0, s, iters, out);
   }
-  return check_launch("probe");
+  return launched();
 }
