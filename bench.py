@@ -561,6 +561,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-other", action="store_true", help="skip the secondary configs")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="only the timed launches of the headline kernel (for counter runs): no probes, no settled / "
+                         "burst repeats, no secondary configs, no CPU leg")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="instead of the benchmark, run a plain streaming kernel of known size (reads and writes "
                          "256 MiB each per launch) to calibrate the FETCH_SIZE / WRITE_SIZE counters against")
@@ -640,6 +643,9 @@ def main():
     # What the matrix cores sustain with nothing else in the way: register-resident instruction loops of the
     # headline's op count (2 x 4 wavefronts per CU, 1024 instructions each), with operands that stay the same
     # and with operands that change from one instruction to the next like the rows of real matrices.
+    if args.headline_only:
+        print(json.dumps(result), flush=True)
+        return
     probe_out = torch.empty(512 * 256, dtype=torch.int32, device=dev)
     stream0 = torch.cuda.current_stream().cuda_stream
     for label, changing in (("matrix_cores_alone_constant_operands", 0), ("matrix_cores_alone_changing_operands", 1)):

@@ -119,6 +119,11 @@ struct RequantScalars {
   // first step's constants and the offset into the rounding constant (see requantize_one_folded)
   int foldedOK;
   double inScaleFolded, inMinFolded, magicFolded;
+  // foldedOK and inMinFolded - 2^52 * inScaleFolded is a double without rounding: the first step can take
+  // 2^52 + off (the bits of off under the exponent word of 2^52, no conversion instruction) instead of off
+  // (see requantize_one_biased_unclamped)
+  int biasedOK;
+  double inMinBiased;
 };
 
 // offMax = highest - lowest of the input type (its largest x - inLowest)
@@ -144,6 +149,14 @@ __host__ __device__ static inline void finish_requant_scalars(RequantScalars& s,
   s.inScaleFolded = s.inScale * s.outScale;
   s.inMinFolded = s.inMin * s.outScale;
   s.magicFolded = 6755399441055744.0 - (double)d;
+  // t = inMinFolded - 2^52 * inScaleFolded; the scaling by 2^52 is exact, and the error term of the
+  // subtraction (Knuth's two-sum) is zero exactly when t is the true difference
+  const double big = s.inScaleFolded * 4503599627370496.0;
+  const double t = s.inMinFolded - big;
+  const double bv = t - s.inMinFolded;
+  const double err = (s.inMinFolded - (t - bv)) + (-big - bv);
+  s.biasedOK = (s.foldedOK && err == 0.0 && fabs(big) < 1e300 && fabs(t) < 1e300) ? 1 : 0;
+  s.inMinBiased = t;
 }
 
 // Valid when RequantScalars::fast32OK.  Adding 1.5 * 2^52 rounds y to the nearest integer (ties to
@@ -172,6 +185,15 @@ __device__ static inline int requantize_one_fast32_unclamped(double off, const R
 }
 __device__ static inline int requantize_one_folded_unclamped(double off, const RequantScalars& s) {
   return (int)(unsigned)__double_as_longlong(fma(off, s.inScaleFolded, s.inMinFolded) + s.magicFolded);
+}
+
+// Valid when RequantScalars::biasedOK.  The double whose high word is 0x43300000 and whose low word is off is
+// 2^52 + off exactly, so fma(2^52 + off, inScaleFolded, inMinFolded - 2^52 * inScaleFolded) rounds the same real
+// number off * inScaleFolded + inMinFolded as requantize_one_folded_unclamped does: one rounding, the same value,
+// and no integer-to-double conversion.
+__device__ static inline int requantize_one_biased_unclamped(unsigned off, const RequantScalars& s) {
+  const double d = __hiloint2double(0x43300000, (int)off);
+  return (int)(unsigned)__double_as_longlong(fma(d, s.inScaleFolded, s.inMinBiased) + s.magicFolded);
 }
 
 // Four int32 clamped to 0..255 and packed into one word, first value in the low byte: int32 -> int16 and
@@ -220,6 +242,8 @@ __host__ __device__ static inline RequantScalars make_requant_scalars(int inType
   s.outOffset = 0;
   s.fastOK = 0;
   s.fast32OK = 0;
+  s.foldedOK = 0;
+  s.biasedOK = 0;
   s.offsetMinusLowest32 = 0;
   s.offsetMinusLowest = 0.0;
   if (minOut >= maxOut) {

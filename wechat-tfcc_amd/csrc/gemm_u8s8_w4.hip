@@ -189,7 +189,26 @@ __global__ __launch_bounds__(kThreads) void qgemm_w4_kernel(const QGemmParams p)
       rq.inScaleFolded = p.rqInScaleFolded; rq.inMinFolded = p.rqInMinFolded; rq.magicFolded = p.rqMagicFolded;
       rq.offsetMinusLowest = p.rqOffsetMinusLowest; rq.offsetMinusLowest32 = p.rqOffsetMinusLowest32;
       rq.fastOK = p.rqFastOK; rq.fast32OK = p.rqFast32OK; rq.foldedOK = p.rqFoldedOK;
+      rq.biasedOK = p.rqBiasedOK; rq.inMinBiased = p.rqInMinBiased;
     }
+    // The same in every lane whichever branch made them: kept in scalar registers across the main loop, whose
+    // vector registers are all spoken for.
+    auto uniformInt = [](int x) { return __builtin_amdgcn_readfirstlane(x); };
+    auto uniformDouble = [&](double x) {
+      return __hiloint2double(uniformInt(__double2hiint(x)), uniformInt(__double2loint(x)));
+    };
+    auto uniformLong = [&](long long x) {
+      return (long long)(((unsigned long long)(unsigned)uniformInt((int)(x >> 32)) << 32) |
+                         (unsigned)uniformInt((int)x));
+    };
+    rq.inScale = uniformDouble(rq.inScale); rq.inMin = uniformDouble(rq.inMin);
+    rq.outScale = uniformDouble(rq.outScale); rq.offsetMinusLowest = uniformDouble(rq.offsetMinusLowest);
+    rq.inScaleFolded = uniformDouble(rq.inScaleFolded); rq.inMinFolded = uniformDouble(rq.inMinFolded);
+    rq.magicFolded = uniformDouble(rq.magicFolded); rq.inMinBiased = uniformDouble(rq.inMinBiased);
+    rq.outOffset = uniformLong(rq.outOffset); rq.fillValue = uniformLong(rq.fillValue);
+    rq.offsetMinusLowest32 = uniformInt(rq.offsetMinusLowest32); rq.mode = uniformInt(rq.mode);
+    rq.fastOK = uniformInt(rq.fastOK); rq.fast32OK = uniformInt(rq.fast32OK);
+    rq.foldedOK = uniformInt(rq.foldedOK); rq.biasedOK = uniformInt(rq.biasedOK);
   }
 
   // 256 accumulator registers set to zero by 16 matrix ops on zero operands (one instruction per block instead
@@ -283,7 +302,11 @@ __global__ __launch_bounds__(kThreads) void qgemm_w4_kernel(const QGemmParams p)
         if (CPS >= 16) issueCopy(soA, soB, dmaStage, copy0 + m);
         else if (m >= FIRST && (m & 1)) issueCopy(soA, soB, dmaStage, copy0 + (m - FIRST) / 2);
       }
-      acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ub[j], ua[i], acc[i][j], 0, 0, 0);
+      // odd row blocks run their four column blocks backwards: the B operand of a row block's last matrix op is
+      // the next row block's first, so one operand out of two stays put across the change of row (fewer operand
+      // bits switch; the chip is power-limited on data like this, and the measured gain is half a percent)
+      const int js = (i & 1) ? NI - 1 - j : j;
+      acc[i][js] = __builtin_amdgcn_mfma_i32_32x32x32_i8(ub[js], ua[i], acc[i][js], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -372,8 +395,10 @@ __global__ __launch_bounds__(kThreads) void qgemm_w4_kernel(const QGemmParams p)
   // into a word (two saturating conversions: int32 -> int16 -> uint8, which is the clamp to 0..255), the two
   // half-wavefronts that share a row exchange two of their four words per 32 x 32 block so that each ends up
   // with 16 consecutive columns, and a 128-bit store per block writes 32 bytes of a row per lane pair.
-  auto storeTile = [&](auto flavour) {
-    constexpr int FLAVOUR = decltype(flavour)::value;  // 0 int32 only, 1 double shortcut, 2 exact int64, 3 fill, 4 int32 shortcut, 5 folded
+  auto storeTileChecked = [&](auto flavour, auto inside) __attribute__((always_inline)) {
+    constexpr int FLAVOUR = decltype(flavour)::value;
+    // 0 int32 only, 1 double shortcut, 2 exact int64, 3 fill, 4 int32 shortcut, 5 folded, 6 biased
+    constexpr bool INSIDE = decltype(inside)::value;  // the whole tile lies inside the matrix: no bounds tests
 #pragma unroll
     for (int i = 0; i < MI; ++i) {
       const int trow = wm * 128 + 32 * i + l32;
@@ -393,7 +418,7 @@ __global__ __launch_bounds__(kThreads) void qgemm_w4_kernel(const QGemmParams p)
 #pragma unroll
           for (int e = 0; e < 4; ++e) v[e] = (int)((unsigned)acc[i][j][4 * rq4 + e] + (unsigned)rt + (unsigned)ct[e]);
           if constexpr (WRITE_C) {
-            if (grow < M && n0 + tcol < N)  // N % 16 == 0: the four columns are in or out together
+            if (INSIDE || (grow < M && n0 + tcol < N))  // N % 16 == 0: the four columns are in or out together
               *reinterpret_cast<v4i*>(C + (size_t)grow * N + n0 + tcol) = v4i{v[0], v[1], v[2], v[3]};
           }
           if constexpr (FLAVOUR != 0) {
@@ -405,6 +430,7 @@ __global__ __launch_bounds__(kThreads) void qgemm_w4_kernel(const QGemmParams p)
               else if constexpr (FLAVOUR == 2) q[e] = (int)requantize_one_exact((long long)(int)(off ^ 0x80000000u), rq);
               else if constexpr (FLAVOUR == 4) q[e] = requantize_one_fast32_unclamped((double)off, rq);
               else if constexpr (FLAVOUR == 5) q[e] = requantize_one_folded_unclamped((double)off, rq);
+              else if constexpr (FLAVOUR == 6) q[e] = requantize_one_biased_unclamped(off, rq);
               else q[e] = (int)rq.fillValue;
             }
             packed[rq4] = pack_sat_u8(q[0], q[1], q[2], q[3]);
@@ -415,16 +441,22 @@ __global__ __launch_bounds__(kThreads) void qgemm_w4_kernel(const QGemmParams p)
           const auto s02 = __builtin_amdgcn_permlane32_swap(packed[0], packed[2], false, false);
           const auto s13 = __builtin_amdgcn_permlane32_swap(packed[1], packed[3], false, false);
           const unsigned gcol = n0 + wn * 128 + 32 * j + 16 * g;
-          if (grow < M && gcol < N)
+          if (INSIDE || (grow < M && gcol < N))
             *reinterpret_cast<v4i*>(Q + (size_t)grow * N + gcol) = v4i{(int)s02[0], (int)s02[1], (int)s13[0], (int)s13[1]};
         }
       }
     }
   };
+  const bool tileInside = m0 + BM <= M && n0 + BN <= N;  // the same for the whole workgroup
+  auto storeTile = [&](auto flavour) __attribute__((always_inline)) {
+    if (tileInside) storeTileChecked(flavour, std::true_type{});
+    else storeTileChecked(flavour, std::false_type{});
+  };
   if constexpr (!REQUANT) {
     storeTile(std::integral_constant<int, 0>{});
   } else {
     if (rq.mode) storeTile(std::integral_constant<int, 3>{});
+    else if (rq.biasedOK) storeTile(std::integral_constant<int, 6>{});
     else if (rq.foldedOK) storeTile(std::integral_constant<int, 5>{});
     else if (rq.fast32OK) storeTile(std::integral_constant<int, 4>{});
     else if (rq.fastOK) storeTile(std::integral_constant<int, 1>{});
@@ -448,6 +480,7 @@ int launch_w4(hipStream_t stream, QGemmParams p) {
     p.rqInScaleFolded = rq.inScaleFolded; p.rqInMinFolded = rq.inMinFolded; p.rqMagicFolded = rq.magicFolded;
     p.rqOffsetMinusLowest = rq.offsetMinusLowest; p.rqOffsetMinusLowest32 = rq.offsetMinusLowest32;
     p.rqFastOK = rq.fastOK; p.rqFast32OK = rq.fast32OK; p.rqFoldedOK = rq.foldedOK;
+    p.rqBiasedOK = rq.biasedOK; p.rqInMinBiased = rq.inMinBiased;
   }
   const UDiv perBatch = udiv_prepare(p.tilesM * p.tilesN), band = udiv_prepare(4u * p.tilesN);
   p.perBatchMagic = perBatch.magic; p.perBatchShift = perBatch.shift;

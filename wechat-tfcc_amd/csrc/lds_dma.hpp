@@ -18,6 +18,11 @@ __device__ __forceinline__ lds_dma_v4i make_rsrc(const void* base, unsigned byte
   return r;
 }
 
+// Cache-policy bits appended to the copy instructions (" sc0", " sc1", " nt" or a combination); empty = default.
+#ifndef TFCC_LDS_DMA_CACHE_BITS
+#define TFCC_LDS_DMA_CACHE_BITS ""
+#endif
+
 // One asynchronous 16-byte-per-lane copy HBM -> LDS.  The LDS address of lane i is ldsBase + 16*i
 // (ldsBase wave-uniform, goes through M0); voffset is the lane's byte offset into the buffer.
 // Inline asm on purpose: the outstanding-copy count is managed by hand (s_waitcnt vmcnt) so that
@@ -32,7 +37,7 @@ __device__ __forceinline__ void dma16(lds_dma_v4i rsrc, unsigned ldsBase, unsign
 // The same copy with a scalar byte offset on top of the lane's (the buffer's range check sees the lane offset
 // only) and the LDS address already in a scalar register.
 __device__ __forceinline__ void dma16s(lds_dma_v4i rsrc, unsigned ldsAddr, unsigned voffset, unsigned soffset) {
-  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+  asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen" TFCC_LDS_DMA_CACHE_BITS " lds"
                :
                : "s"(ldsAddr), "v"(voffset), "s"(rsrc), "s"(soffset)
                : "memory", "m0");

@@ -26,8 +26,8 @@ struct QGemmParams {
   unsigned tilesM, tilesN, tilesTotal, chunk;
   // what the requantize step makes of the four immediate scalars above (RequantScalars' derived fields), worked
   // out by launchers whose kernel reads it instead of deriving it per thread; unused with minOut / maxOut
-  double rqInScaleFolded, rqInMinFolded, rqMagicFolded, rqOffsetMinusLowest;
-  int rqOffsetMinusLowest32, rqFastOK, rqFast32OK, rqFoldedOK;
+  double rqInScaleFolded, rqInMinFolded, rqMagicFolded, rqOffsetMinusLowest, rqInMinBiased;
+  int rqOffsetMinusLowest32, rqFastOK, rqFast32OK, rqFoldedOK, rqBiasedOK;
   // division by tilesM * tilesN and by 4 * tilesN as multiply-high and shift (filled by launchers whose kernel uses them)
   unsigned perBatchMagic, perBatchShift, bandMagic, bandShift;
 };
