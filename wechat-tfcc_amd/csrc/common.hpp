@@ -196,6 +196,13 @@ __device__ static inline int requantize_one_biased_unclamped(unsigned off, const
   return (int)(unsigned)__double_as_longlong(fma(d, s.inScaleFolded, s.inMinBiased) + s.magicFolded);
 }
 
+// GELU in its erf form, 0.5 x (1 + erf(x / sqrt 2)) as the reference's scalar template writes it
+// (tfcc/mkl/kernel/tfcc_mklactivationkernel.hpp:213-220: erf in float, the product formed in double): one function
+// for the stand-alone kernel and for every fused tile store, so that fusing changes no bit.
+__device__ static inline float gelu_erf_f32(float v) {
+  return (float)(0.5 * (double)v * (double)(1.0f + erff(v / 1.4142135623730951f)));
+}
+
 // Four int32 clamped to 0..255 and packed into one word, first value in the low byte: int32 -> int16 and
 // int16 -> uint8, both saturating.
 __device__ static inline unsigned pack_sat_u8(int a, int b, int c, int d) {

@@ -461,6 +461,8 @@ int dispatch(hipStream_t s, const SgemmParams& p, bool vec, bool tb, unsigned fi
       // ... and when 128 x 96 tiles over all of them still occupy most of the CUs in one round, twelve wavefronts
       // share each copy of B among four times the rows (44.1 against 46.8 us for three 1024 x 768 x 768 products);
       // the sums are those of the 32 x 96 tiles.
+      // 32 x 96 tiles and four K groups: the four groups as the four hand-scheduled wavefronts of one workgroup
+      if (kTiles[best].config == 1 && ksplit == 4) return sgemm_detail::sgemm_wave96_launch(s, p, 4);
       if (serial && kTiles[best].config == 1) {
         const unsigned long long wide = (unsigned long long)((m + 127) / 128) * ((n + 95) / 96) * p.batch;
         if (wide <= 256 && wide >= 160) return sgemm_detail::sgemm_dma_launch(s, p, 5, ksplit, true);

@@ -45,8 +45,10 @@ __device__ __forceinline__ int row_swizzle(int row) { return (row >> 1) & 7; }
 template <int WGM, int WGN, int NI, int KSPLIT, int STAGES, int VSPLIT = 1>
 __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_dma_kernel(const SgemmParams p) {
   static_assert(VSPLIT == 1 || KSPLIT == 1, "accumulators per would-be group only without real groups");
-  static_assert(NI == 1 || NI == 4, "a lane reads its B operands as one or four consecutive words");
+  static_assert(NI == 1 || NI == 3 || NI == 4, "a lane reads its B operands as one word, three words 32 columns apart or four consecutive words");
+  constexpr bool STRIDED = NI == 3;  // lane lrow owns columns lrow, lrow + 32, lrow + 64 of the wavefront's block
   constexpr int GW = WGM * WGN;
+  constexpr bool PRIVATE_RING = GW == 1;  // one wavefront per group: nobody else reads or fills its ring
   constexpr int WN = 32 * NI;
   constexpr int BM = WGM * 32, BN = WGN * WN;
   constexpr int A_BYTES = BM * BK * 4, B_BYTES = BK * BN * 4, STAGE_BYTES = A_BYTES + B_BYTES;
@@ -103,19 +105,22 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_dma_kernel(cons
   const int lrow = lane & 31, g = lane >> 5;
 
   // values needed only in the tile store are fetched now: at the end their latency would be waited for in full
-  const unsigned gcol = n0 + wn * WN + NI * lrow;  // first of this lane's NI columns
+  const unsigned gcol = n0 + wn * WN + (STRIDED ? lrow : NI * lrow);  // first of this lane's NI columns
+  constexpr unsigned CSTEP = STRIDED ? 32 : 1;                          // from one of them to the next
   float bv[NI];
 #pragma unroll
-  for (int j = 0; j < NI; ++j) bv[j] = (biasPtr && gcol + j < N) ? biasPtr[gcol + j] : 0.f;
-  constexpr bool EARLY_RESIDUAL = NI == 1;  // short launches on small tiles; a large tile fetches it in the store
-  float rv[EARLY_RESIDUAL ? 16 : 1];
+  for (int j = 0; j < NI; ++j) bv[j] = (biasPtr && gcol + j * CSTEP < N) ? biasPtr[gcol + j * CSTEP] : 0.f;
+  constexpr bool EARLY_RESIDUAL = NI != 4;  // short launches on small tiles; a large tile fetches it in the store
+  float rv[EARLY_RESIDUAL ? 16 * NI : 1];
   if constexpr (EARLY_RESIDUAL) {
     if (p.residual && grp == 0) {
       const float* Rp = p.residual + (size_t)bi * p.strideR;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const unsigned grow = m0 + wm * 32 + 8 * (r / 4) + 4 * g + (r & 3);
-        rv[r] = (grow < M && gcol < N) ? Rp[(size_t)grow * N + gcol] : 0.f;
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+          rv[r * NI + j] = (grow < M && gcol + j * CSTEP < N) ? Rp[(size_t)grow * N + gcol + j * CSTEP] : 0.f;
       }
     }
   }
@@ -166,7 +171,7 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_dma_kernel(cons
   struct BOps { float v[4][NI]; };  // [s][j]
   const int arow = wm * 32 + lrow;
   const int aBase = arow * (BK * 4), aSwz = row_swizzle(arow);
-  const int bBase = A_BYTES + (4 * g) * (BN * 4) + (wn * WN + NI * lrow) * 4;
+  const int bBase = A_BYTES + (4 * g) * (BN * 4) + (wn * WN + (STRIDED ? lrow : NI * lrow)) * 4;
   auto readOps = [&](unsigned stage, int kb, v4f& a, BOps& b) {
     const unsigned char* st = gsm + stage * STAGE_BYTES;
     a = *reinterpret_cast<const v4f*>(st + aBase + (((2 * kb + g) ^ aSwz) << 4));
@@ -177,7 +182,9 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_dma_kernel(cons
 #pragma unroll
         for (int j = 0; j < 4; ++j) b.v[s][j] = w[j];
       } else {
-        b.v[s][0] = *reinterpret_cast<const float*>(st + bBase + (8 * kb + s) * (BN * 4));
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+          b.v[s][j] = *reinterpret_cast<const float*>(st + bBase + (8 * kb + s) * (BN * 4) + j * 128);
       }
     }
   };
@@ -196,7 +203,7 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_dma_kernel(cons
 #pragma unroll
   for (int s = 0; s < STAGES; ++s) issueSlab(s);
   wait_vmcnt<COPIES*(STAGES - 1)>();
-  __syncthreads();
+  if constexpr (!PRIVATE_RING) __syncthreads();
   v4f fa[2];
   BOps fb[2];
   readOps(0, 0, fa[0], fb[0]);
@@ -212,7 +219,7 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_dma_kernel(cons
       }
       wait_vmcnt<COPIES*(STAGES - 2)>();
       __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the reads of slab kt have returned
-      __syncthreads();
+      if constexpr (!PRIVATE_RING) __syncthreads();
       readOps(nxt, 0, fa[0], fb[0]);
       issueSlab(kt + STAGES);
       mma(accs[v], fa[(KS - 1) & 1], fb[(KS - 1) & 1]);
@@ -255,7 +262,7 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_dma_kernel(cons
   if (gcol >= N) return;
   const float* R = p.residual ? p.residual + (size_t)bi * p.strideR : nullptr;  // dense, flat batch
   const int act = p.act;
-  const bool whole = gcol + NI <= N;
+  const bool whole = gcol + (NI - 1) * CSTEP < N;
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const unsigned grow = m0 + wm * 32 + 8 * (r / 4) + 4 * g + (r & 3);
@@ -265,11 +272,12 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_dma_kernel(cons
     for (int j = 0; j < NI; ++j) v[j] = acc[j][r] + bv[j];
     if (R) {
       if constexpr (EARLY_RESIDUAL) {
-        v[0] += rv[r];
+#pragma unroll
+        for (int j = 0; j < NI; ++j) v[j] += rv[r * NI + j];
       } else {
 #pragma unroll
         for (int j = 0; j < NI; ++j)
-          if (gcol + j < N) v[j] += R[(size_t)grow * N + gcol + j];
+          if (gcol + j * CSTEP < N) v[j] += R[(size_t)grow * N + gcol + j * CSTEP];
       }
     }
     // same expression as the stand-alone GELU kernel, so that fusing changes no bit
@@ -286,7 +294,7 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_dma_kernel(cons
     }
 #pragma unroll
     for (int j = 0; j < NI; ++j)
-      if (gcol + j < N) dst[j] = v[j];
+      if (gcol + j * CSTEP < N) dst[j * CSTEP] = v[j];
   }
 }
 

@@ -46,6 +46,10 @@ bool sgemm_dma_available(int config, int ksplit);
 // (same additions, same result) - for launches that fill the chip anyway.
 int sgemm_dma_launch(hipStream_t stream, SgemmParams p, int config, int ksplit, bool serialGroups);
 
+// 32 x 96 tiles with the four K groups of ksplit = 4 as the four wavefronts of a workgroup, hand-scheduled
+// (sgemm_wave96.hip).  Same requirements and the same bits as the kernels above for four K groups.
+int sgemm_wave96_launch(hipStream_t stream, SgemmParams p, int ksplit);
+
 // The streaming kernel for up to eight rows of A (sgemv.hip): any K, N, strides and alignment; B not transposed.
 bool sgemv_supported(const SgemmParams& p);
 int sgemv_launch(hipStream_t stream, const SgemmParams& p);
