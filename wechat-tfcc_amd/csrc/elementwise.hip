@@ -150,7 +150,7 @@ __global__ __launch_bounds__(256) void gelu_kernel(const float* in, size_t total
   const size_t step = (size_t)gridDim.x * blockDim.x;
   for (; i < total; i += step) {
     float v = in[i];
-    out[i] = (float)(0.5 * (double)v * (double)(1.0f + erff(v / 1.4142135623730951f)));
+    out[i] = gelu_erf_f32(v);
   }
 }
 

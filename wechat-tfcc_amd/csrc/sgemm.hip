@@ -335,7 +335,7 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_kernel(const Sg
         // same expression as the stand-alone GELU kernel, so that fusing changes no bit
 #pragma unroll
         for (int j = 0; j < NI; ++j)
-          v[j] = (float)(0.5 * (double)v[j] * (double)(1.0f + erff(v[j] / 1.4142135623730951f)));
+          v[j] = gelu_erf_f32(v[j]);
       }
       if (vecOK) {
         if constexpr (NI == 4) *reinterpret_cast<v4f*>(C + off) = v4f{v[0], v[1], v[2], v[3]};

@@ -283,7 +283,7 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_dma_kernel(cons
     // same expression as the stand-alone GELU kernel, so that fusing changes no bit
     if (act == 1) {
 #pragma unroll
-      for (int j = 0; j < NI; ++j) v[j] = (float)(0.5 * (double)v[j] * (double)(1.0f + erff(v[j] / 1.4142135623730951f)));
+      for (int j = 0; j < NI; ++j) v[j] = gelu_erf_f32(v[j]);
     }
     float* dst = Cbase + (size_t)grow * ldc + gcol;
     if constexpr (NI == 4) {

@@ -125,7 +125,7 @@ __global__ __launch_bounds__(kWaves * 64) void sgemv_kernel(SgemmParams p) {
     float v = summed<MR, COLS>(smem, wave, lane);
     if (biasPtr) v += biasPtr[col];
     if (p.residual) v += p.residual[(size_t)bi * p.strideR + (size_t)wave * N + col];
-    if (p.act == 1) v = (float)(0.5 * (double)v * (double)(1.0f + erff(v / 1.4142135623730951f)));
+    if (p.act == 1) v = gelu_erf_f32(v);
     Cbase[(size_t)wave * p.ldc + col] = v;
   }
 }
