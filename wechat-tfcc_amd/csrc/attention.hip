@@ -47,16 +47,6 @@ struct AttentionParams {
   unsigned long long outerM, innerM;
 };
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-  return v;
-}
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
-  return v;
-}
 
 __global__ __launch_bounds__(kThreads, 4) void attention_kernel(const AttentionParams p) {
   extern __shared__ __align__(16) float lds[];

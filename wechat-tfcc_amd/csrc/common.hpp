@@ -196,6 +196,58 @@ __device__ static inline int requantize_one_biased_unclamped(unsigned off, const
   return (int)(unsigned)__double_as_longlong(fma(d, s.inScaleFolded, s.inMinBiased) + s.magicFolded);
 }
 
+// The value of lane i ^ MASK for the six steps of a butterfly over the 64 lanes, without the LDS crossbar that
+// __shfl_xor goes through: the two halves and the rows of 16 lanes are exchanged by the swap instructions (a and b
+// come back as the two members of the pair, in lane order of the lower one), the steps inside a row are data-parallel
+// moves.  wave_sum / wave_max below pair the same lanes in the same order as a __shfl_xor loop from 32 down to 1, and
+// their operations commute, so the results have the same bits.
+template <int MASK>
+__device__ __forceinline__ void butterfly_pair(float v, float& a, float& b) {
+  const unsigned u = __builtin_bit_cast(unsigned, v);
+  if constexpr (MASK == 32) {
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    a = __builtin_bit_cast(float, (unsigned)r[0]); b = __builtin_bit_cast(float, (unsigned)r[1]);
+  } else if constexpr (MASK == 16) {
+    const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    a = __builtin_bit_cast(float, (unsigned)r[0]); b = __builtin_bit_cast(float, (unsigned)r[1]);
+  } else {
+    a = v;
+    unsigned o;
+    if constexpr (MASK == 8) {
+      o = (unsigned)__builtin_amdgcn_update_dpp(0, (int)u, 0x128, 0xf, 0xf, false);  // row_ror:8
+    } else if constexpr (MASK == 4) {
+      o = (unsigned)__builtin_amdgcn_update_dpp(0, (int)u, 0x104, 0xf, 0x5, false);       // row_shl:4, lanes 0-3, 8-11
+      o = (unsigned)__builtin_amdgcn_update_dpp((int)o, (int)u, 0x114, 0xf, 0xa, false);  // row_shr:4, lanes 4-7, 12-15
+    } else if constexpr (MASK == 2) {
+      o = (unsigned)__builtin_amdgcn_update_dpp(0, (int)u, 0x4e, 0xf, 0xf, false);   // quad_perm [2, 3, 0, 1]
+    } else {
+      static_assert(MASK == 1, "a power of two below 64");
+      o = (unsigned)__builtin_amdgcn_update_dpp(0, (int)u, 0xb1, 0xf, 0xf, false);   // quad_perm [1, 0, 3, 2]
+    }
+    b = __builtin_bit_cast(float, o);
+  }
+}
+__device__ __forceinline__ float wave_sum(float v) {
+  float a, b;
+  butterfly_pair<32>(v, a, b); v = a + b;
+  butterfly_pair<16>(v, a, b); v = a + b;
+  butterfly_pair<8>(v, a, b); v = a + b;
+  butterfly_pair<4>(v, a, b); v = a + b;
+  butterfly_pair<2>(v, a, b); v = a + b;
+  butterfly_pair<1>(v, a, b); v = a + b;
+  return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+  float a, b;
+  butterfly_pair<32>(v, a, b); v = fmaxf(a, b);
+  butterfly_pair<16>(v, a, b); v = fmaxf(a, b);
+  butterfly_pair<8>(v, a, b); v = fmaxf(a, b);
+  butterfly_pair<4>(v, a, b); v = fmaxf(a, b);
+  butterfly_pair<2>(v, a, b); v = fmaxf(a, b);
+  butterfly_pair<1>(v, a, b); v = fmaxf(a, b);
+  return v;
+}
+
 // GELU in its erf form, 0.5 x (1 + erf(x / sqrt 2)) as the reference's scalar template writes it
 // (tfcc/mkl/kernel/tfcc_mklactivationkernel.hpp:213-220: erf in float, the product formed in double):
 //   (float)(0.5 * (double)v * (double)(1.0f + erff(v / 1.4142135623730951f)))
