@@ -39,17 +39,17 @@ using sgemm_detail::SgemmParams;
 
 constexpr int BN96 = 96;
 
-// 16-byte chunk c of A row `row` lies at chunk c ^ swizzle: rows of 128 bytes (32 k) and of 64 bytes (16 k)
+// 16-byte chunk c of A row `row` lies at chunk c ^ swizzle: rows of 128 bytes (32 k), 64 bytes (16 k), 32 bytes (8 k)
 template <int BK>
 __device__ __forceinline__ int a_row_swizzle(int row) {
-  return BK == 32 ? (row >> 1) & 7 : (row >> 2) & 3;
+  return BK == 32 ? (row >> 1) & 7 : BK == 16 ? (row >> 2) & 3 : (row >> 2) & 1;
 }
 
 template <int WGM, int KSPLIT, int BK, int STAGES>
 __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const SgemmParams p) {
   static_assert(WGM * KSPLIT == 4, "four wavefronts");
-  static_assert(BK == 32 || BK == 16, "ring slabs of 32 or 16 k");
-  static_assert((STAGES & (STAGES - 1)) == 0 && STAGES >= 2, "ring depth a power of two");
+  static_assert(BK == 32 || BK == 16 || BK == 8, "ring slabs of 32, 16 or 8 k");
+  static_assert(STAGES >= 2, "ring depth");
   constexpr int BM = 32 * WGM;
   constexpr int KS = BK / 8;        // k steps per ring slab
   constexpr int CH = BK / 4;        // 16-byte chunks per A row
@@ -128,12 +128,12 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const SgemmParams p) 
   // Nothing of a copy's set-up runs on the vector unit (a vector instruction between two matrix ops delays the
   // second by some 15 cycles): the lane offsets never change, the slab's k goes into the scalar offset, and a slab
   // past the end of K is read through a descriptor of size zero, which makes every lane read zeros.
-  auto issueCopy = [&](unsigned t, int c) {
+  auto issueCopy = [&](unsigned t, unsigned stage, int c) {
     const unsigned k0 = k0Of(t);
     const bool live = k0 < K;
     const int u = c * WGM + wm;
     const bool isA = u < A_UNITS;
-    const unsigned dst = ldsGroup + (t & (STAGES - 1)) * STAGE_BYTES + u * 1024;
+    const unsigned dst = ldsGroup + stage * STAGE_BYTES + u * 1024;
     const unsigned so = isA ? k0 * 4u : k0 * ldb * 4u;
     w96_v4i rsrc = isA ? rsrcA : rsrcB;
     rsrc[2] = live ? rsrc[2] : 0;
@@ -144,7 +144,7 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const SgemmParams p) 
 #pragma unroll
   for (int s = 0; s < STAGES; ++s)
 #pragma unroll
-    for (int c = 0; c < COPIES; ++c) issueCopy((unsigned)s, c);
+    for (int c = 0; c < COPIES; ++c) issueCopy((unsigned)s, (unsigned)s, c);
 
   // ---- values needed only in the tile store are fetched now.  Rows: lane (lrow, g) stores, for register r of
   // column block j, row 8*(r/4) + 4*g + r%4 of its wavefront's 32 and column 32*j + lrow.  Groups: after the
@@ -182,13 +182,14 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const SgemmParams p) 
 
   // One k step: twelve matrix ops on `cur`; in the issue slots between them the 13 reads of the operands of step
   // (ldStage, ldKb) into `nxt` and, in a slab's last step, the copies of the slab that takes its stage.
-  auto step = [&](const Ops& cur, Ops& nxt, const unsigned char* ldStage, int ldKb, bool dma, unsigned dmaSlab) {
+  auto step = [&](const Ops& cur, Ops& nxt, const unsigned char* ldStage, int ldKb, bool dma, unsigned dmaSlab,
+                  unsigned dmaStage) {
 #pragma unroll
     for (int m = 0; m < 12; ++m) {
       const int s = m / 3, j = m % 3;
       if (m == 0) nxt.a = *reinterpret_cast<const w96_v4f*>(ldStage + aBase + (((2 * ldKb + g) ^ aSwz) << 4));
       nxt.b[s][j] = *reinterpret_cast<const float*>(ldStage + bBase + (8 * ldKb + s) * (BN96 * 4) + j * 128);
-      if (dma && m >= 1 && m <= COPIES) issueCopy(dmaSlab, m - 1);
+      if (dma && m >= 1 && m <= COPIES) issueCopy(dmaSlab, dmaStage, m - 1);
       acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(cur.a[s], cur.b[s][j], acc[j], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -206,15 +207,28 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const SgemmParams p) 
   for (int s = 0; s < 4; ++s)
 #pragma unroll
     for (int j = 0; j < 3; ++j) ops[0].b[s][j] = *reinterpret_cast<const float*>(gsm + bBase + s * (BN96 * 4) + j * 128);
-  for (unsigned t = 0; t < T; ++t) {
-    const unsigned char* stCur = gsm + (t & (STAGES - 1)) * STAGE_BYTES;
-    const unsigned char* stNext = gsm + ((t + 1) & (STAGES - 1)) * STAGE_BYTES;
+  // one ring slab: KS steps starting on the operands in `first`; the next slab's first operands end up in `first`
+  // again when KS is even, in `other` when it is odd (then the loop below alternates the two)
+  unsigned stage = 0;  // of slab t
+  auto slab = [&](unsigned t, Ops& first, Ops& other) {
+    const unsigned next = stage + 1 == STAGES ? 0 : stage + 1;
+    const unsigned char* stCur = gsm + stage * STAGE_BYTES;
+    const unsigned char* stNext = gsm + next * STAGE_BYTES;
 #pragma unroll
-    for (int kb = 0; kb < KS - 1; ++kb) step(ops[kb & 1], ops[(kb + 1) & 1], stCur, kb + 1, false, 0u);
+    for (int kb = 0; kb < KS - 1; ++kb) step(kb & 1 ? other : first, kb & 1 ? first : other, stCur, kb + 1, false, 0u, 0u);
     wait_vmcnt<COPIES*(STAGES - 2)>();
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the reads of slab t have returned
     if constexpr (SHARED) __syncthreads();
-    step(ops[(KS - 1) & 1], ops[0], stNext, 0, true, t + STAGES);
+    step((KS - 1) & 1 ? other : first, (KS - 1) & 1 ? first : other, stNext, 0, true, t + STAGES, stage);
+    stage = next;
+  };
+  if constexpr (KS & 1) {
+    for (unsigned t = 0; t < T; t += 2) {  // T is a multiple of 32 / BK >= 2
+      slab(t, ops[0], ops[1]);
+      slab(t + 1, ops[1], ops[0]);
+    }
+  } else {
+    for (unsigned t = 0; t < T; ++t) slab(t, ops[0], ops[1]);
   }
   wait_vmcnt<0>();
   __syncthreads();
@@ -239,20 +253,33 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const SgemmParams p) 
       }
     }
   } else {
-    // the four partial tiles go through LDS (the rings are idle now); register idx of group q lies at
-    // red[(q * 48 + idx) * 64 + lane], and wavefront w adds the four of its twelve registers in group order
-    float* red = reinterpret_cast<float*>(smem);
+    // the four partial tiles go through LDS (the rings are idle now), four registers per 128-bit access: registers
+    // 4c .. 4c+3 of group q lie at red4[(q * 12 + c) * 64 + lane]; wavefront w adds the four of its twelve registers
+    // (quads 3w .. 3w+2) in group order
+    w96_v4f* red4 = reinterpret_cast<w96_v4f*>(smem);
 #pragma unroll
     for (int j = 0; j < 3; ++j)
 #pragma unroll
-      for (int r = 0; r < 16; ++r) red[((grp * 48 + j * 16 + r) * 64) + lane] = acc[j][r];
+      for (int c = 0; c < 4; ++c)
+        red4[(grp * 12 + j * 4 + c) * 64 + lane] = w96_v4f{acc[j][4 * c], acc[j][4 * c + 1], acc[j][4 * c + 2], acc[j][4 * c + 3]};
     __syncthreads();
+    float sums[12];
+#pragma unroll
+    for (int c = 0; c < 3; ++c) {
+      w96_v4f v = red4[(3 * grp + c) * 64 + lane];
+#pragma unroll
+      for (int o = 1; o < KSPLIT; ++o) {
+        const w96_v4f w = red4[(o * 12 + 3 * grp + c) * 64 + lane];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] += w[e];
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) sums[4 * c + e] = v[e];
+    }
 #pragma unroll
     for (int q = 0; q < 12; ++q) {
       const int idx = firstIdx + q, j = idx >> 4, r = idx & 15;
-      float v = red[(idx * 64) + lane];
-#pragma unroll
-      for (int o = 1; o < KSPLIT; ++o) v += red[((o * 48 + idx) * 64) + lane];
+      const float v = sums[q];
       const unsigned grow = m0 + 8 * (r >> 2) + 4 * g + (r & 3);
       const unsigned gc = gcol0 + 32 * j;
       // bv is indexed by a wave-uniform j: selects keep it in registers
@@ -292,7 +319,14 @@ int launch_wave96(hipStream_t stream, SgemmParams p) {
 namespace sgemm_detail {
 
 int sgemm_wave96_launch(hipStream_t stream, SgemmParams p, int ksplit) {
-  if (ksplit == 4) return launch_wave96<1, 4, 16, 2>(stream, p);
+  if (ksplit == 4) {
+    // Three or more tiles per CU: rings of three slabs of 8 k (12 KB per wavefront) let three workgroups share a CU,
+    // so that all of a CU's tiles overlap (three 1024 x 768 x 768 products in one launch: 33.9 us -> see below).
+    // Fewer: two slabs of 16 k, which leave a slab's copies twice the time to land.
+    const unsigned long long tiles = (unsigned long long)((p.M + 31) / 32) * ((p.N + BN96 - 1) / BN96) * p.batch;
+    if (tiles > 512) return launch_wave96<1, 4, 8, 3>(stream, p);
+    return launch_wave96<1, 4, 16, 2>(stream, p);
+  }
   return set_error(TFCC_ROCM_INVALID_ARGUMENT, "sgemm: no 32 x 96 wavefront kernel for %d K groups", ksplit);
 }
 
