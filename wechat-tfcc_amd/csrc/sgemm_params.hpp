@@ -25,6 +25,14 @@ struct SgemmParams {
   float* groupC[4];
   unsigned M, N, K, batch;
   unsigned tilesM, tilesN, tilesTotal, chunk;
+  // Layer normalisation of every row of the result over its N columns in the same launch (sgemm_wave96.hip only;
+  // lnGamma == nullptr: none).  The sums a * b + bias + residual go to lnSums [M, N] instead of C; lnCounters holds
+  // one word per band of 32 rows, zero when the launch starts and zero again when it ends.
+  const float* lnGamma;
+  const float* lnBeta;
+  float lnEps;
+  float* lnSums;
+  unsigned* lnCounters;
 };
 
 // Fills in the tile counts for BM x BN tiles; false when there are too many tiles for one grid.
@@ -49,6 +57,7 @@ int sgemm_dma_launch(hipStream_t stream, SgemmParams p, int config, int ksplit, 
 // 32 x 96 tiles with the four K groups of ksplit = 4 as the four wavefronts of a workgroup, hand-scheduled
 // (sgemm_wave96.hip).  Same requirements and the same bits as the kernels above for four K groups.
 int sgemm_wave96_launch(hipStream_t stream, SgemmParams p, int ksplit);
+constexpr unsigned kLayerNormMaxColumns = 1024;  // a lane of the normalising wavefront holds 16 values of a row
 
 // The streaming kernel for up to eight rows of A (sgemv.hip): any K, N, strides and alignment; B not transposed.
 bool sgemv_supported(const SgemmParams& p);
