@@ -396,7 +396,9 @@ int tfcc_rocm_compare(void* stream, int op, const void* a, const void* b, int ty
  * (tfcc/mkl/interfaces/tfcc_mklbasicinterface.cpp:469-485, :757-776). */
 int tfcc_rocm_argmax_f32(void* stream, const float* in, uint64_t outer, unsigned length, uint64_t inner, int64_t* out);
 /* The k largest elements of each row of in [rows, length], descending, and their positions; equal values in ascending
- * position (tfcc/mkl/interfaces/tfcc_mklbasicinterface.cpp:159-260, :779-800 leaves their order open).  1 <= k <= length. */
+ * position (tfcc/mkl/interfaces/tfcc_mklbasicinterface.cpp:159-260, :779-800 leaves their order open).  A NaN counts
+ * as larger than every number (the reference's heap comparison v1.value > v2.value leaves its place undefined).
+ * 1 <= k <= min(length, 1024): the selection makes one pass over the row per element, one workgroup per row. */
 int tfcc_rocm_topk_f32(void* stream, const float* in, uint64_t rows, unsigned length, unsigned k, float* values,
                        uint32_t* positions);
 /* out = a op b with numpy-style broadcasting: dims[rank] is the result's shape, stride_a / stride_b the element strides

@@ -730,6 +730,15 @@ def test_top_k(pkg, T):
             assert np.array_equal(T.n(values).view(np.uint32), np.take_along_axis(x, order, axis=-1).view(np.uint32))
     with pytest.raises(pkg.InvalidArgumentError, match="invalid k"):
         pkg.top_k(T.t(np.zeros((2, 3), np.float32)), 4)
+    # a deliberate choice where the reference's heap comparison leaves the order open: a NaN counts as the largest,
+    # several of them in ascending position, +inf next
+    x = np.array([[1.0, np.nan, np.inf, -2.0, np.nan, 7.0]], np.float32)
+    values, positions = pkg.top_k(T.t(x), 4)
+    assert T.n(positions).tolist() == [[1, 4, 2, 5]]
+    assert np.isnan(T.n(values)[0, :2]).all() and T.n(values)[0, 2:].tolist() == [np.inf, 7.0]
+    # the selection makes one pass per element: beyond 1024 it is refused
+    with pytest.raises(pkg.TfccRocmError, match="beyond the 1024"):
+        pkg.top_k(T.t(np.zeros((1, 4096), np.float32)), 1025)
 
 
 BROADCAST_PAIRS = [
@@ -825,3 +834,38 @@ def test_elementwise_against_oracle(pkg, T):
     for perm in ((0, 2, 1, 3), (0, 1, 3, 2), (3, 2, 1, 0), (0, 2, 3, 1)):
         assert np.array_equal(T.n(pkg.transpose(T.t(y), perm)), np.transpose(y, perm))
     assert np.array_equal(T.n(pkg.transpose(T.t(x), (1, 0))), x.T)
+
+
+@pytest.mark.gpu
+def test_max_min_clip_relu_keep_the_reference_comparison_order(pkg, T):
+    """std::max(a, b) = a < b ? b : a and std::min(a, b) = b < a ? b : a, as the reference's kernels call them
+    (tfcc/mkl/interfaces/tfcc_mklminmaxinterface.cpp:37-61, tfcc_mklbasicinterface.cpp:152-153,
+    tfcc/mkl/kernel/tfcc_mklactivationkernel.hpp:67-83): the first argument comes back when either is a NaN, a clip
+    with its bounds the wrong way round gives the lower bound, a leaky relu with alpha > 1 gives max(v, alpha v)."""
+    nan = np.float32(np.nan)
+
+    def std_max(a, b):
+        return np.where(a < b, b, a)
+
+    def std_min(a, b):
+        return np.where(b < a, b, a)
+
+    a = np.array([1.0, nan, -2.0, 0.0, -0.0, 5.0, nan, -3.5], np.float32)
+    b = np.array([nan, 2.0, -1.0, -0.0, 0.0, 4.0, nan, 7.25], np.float32)
+    with np.errstate(invalid="ignore"):
+        for op, ref in (("max", std_max), ("min", std_min)):
+            got = T.n(pkg.binary(op, T.t(a), T.t(b)))
+            want = ref(a, b)
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (op, got, want)
+        v = np.array([-3.0, -1.0, 0.5, 2.0, nan, 9.0], np.float32)
+        for lo, hi in ((-1.0, 2.0), (2.0, -1.0)):  # the second pair: lower bound above the upper one
+            want = std_max(std_min(v, np.float32(hi)), np.float32(lo))
+            got = T.n(pkg.clip(T.t(v), lo, hi))
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (lo, hi, got, want)
+        for alpha in (0.1, 1.5, -0.5):
+            want = std_max(v, np.float32(alpha) * v)
+            got = T.n(pkg.leaky_relu(T.t(v), alpha))
+            assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (alpha, got, want)
+        want = std_max(v, np.float32(0))
+        got = T.n(pkg.unary("relu", T.t(v)))
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))

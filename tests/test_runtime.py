@@ -280,6 +280,81 @@ def test_archive_and_graph_errors(mf, rt):
         rt.Model(mf.write_model([dup], "g"), host=True).run({})
 
 
+def test_crafted_archives_are_refused_not_read_past_their_end(mf, rt):
+    """Offsets and sizes of a zip / npy come from the file.  Every crafted case must end in the runtime's format
+    error (never in a read outside the buffer, an allocation of the size the file claims, or a wrapped sum)."""
+    import struct
+    g = passthrough_graph(mf, mf.FLOAT, [2], [0])
+    good = mf.write_model([g], "g")
+    rt.Model(good, host=True)  # the untouched archive loads
+    eocd = good.rfind(b"PK\x05\x06")
+    entries, = struct.unpack_from("<H", good, eocd + 10)
+    dir_offset, = struct.unpack_from("<I", good, eocd + 16)
+    assert entries >= 2 and good[dir_offset:dir_offset + 4] == b"PK\x01\x02"
+
+    def patched(offset, fmt, value):
+        b = bytearray(good)
+        struct.pack_into(fmt, b, offset, value)
+        return bytes(b)
+
+    cases = {
+        "truncated in the middle": good[:len(good) // 2],
+        "truncated inside the end record": good[:eocd + 10],
+        "central directory offset past the end": patched(eocd + 16, "<I", len(good) + 1000),
+        "central directory offset 0xfffffffe": patched(eocd + 16, "<I", 0xfffffffe),
+        "more entries than there are": patched(eocd + 10, "<H", entries + 7),
+        "local header offset past the end": patched(dir_offset + 42, "<I", 0x7fffffff),
+        "compressed size larger than the file": patched(dir_offset + 20, "<I", 0x7ffffff0),
+        "name length running past the end": patched(dir_offset + 28, "<H", 0xffff),
+    }
+    # a zip64 extra field whose local offset is close to 2^64 (offset + 30 would wrap)
+    b = bytearray(good)
+    name_len, extra_len = struct.unpack_from("<HH", b, dir_offset + 28)
+    if extra_len == 0:
+        entry_end = dir_offset + 46 + name_len
+        extra = struct.pack("<HHQ", 1, 8, 0xffffffffffffffe0)
+        b[entry_end:entry_end] = extra
+        struct.pack_into("<H", b, dir_offset + 30, len(extra))
+        struct.pack_into("<I", b, dir_offset + 42, 0xffffffff)
+        new_eocd = eocd + len(extra)
+        size, = struct.unpack_from("<I", b, new_eocd + 12)
+        struct.pack_into("<I", b, new_eocd + 12, size + len(extra))
+        cases["zip64 local offset near 2^64"] = bytes(b)
+    for what, blob in cases.items():
+        with pytest.raises(rt.RuntimeError_, match="invalid zip|Invalid model data|invalid npy"):
+            rt.Model(blob, host=True)
+    # a deflated member that claims to inflate to 2^32 - 2 bytes: refused before anything of that size is allocated
+    deflated = io.BytesIO()
+    with zipfile.ZipFile(io.BytesIO(good)) as zin, zipfile.ZipFile(deflated, "w", zipfile.ZIP_DEFLATED) as zout:
+        for name in zin.namelist():
+            zout.writestr(name, zin.read(name))
+    d = deflated.getvalue()
+    rt.Model(d, host=True)
+    d_dir, = struct.unpack_from("<I", d, d.rfind(b"PK\x05\x06") + 16)
+    lie = bytearray(d)
+    struct.pack_into("<I", lie, d_dir + 24, 0xfffffffe)
+    with pytest.raises(rt.RuntimeError_, match="invalid zip"):
+        rt.Model(bytes(lie), host=True)
+    # npy members with impossible shapes: a product that wraps 2^64, a dimension beyond 32 bits, more elements than bytes
+    def with_npy_header(shape_text):
+        out = io.BytesIO()
+        with zipfile.ZipFile(io.BytesIO(good)) as zin, zipfile.ZipFile(out, "w") as zout:
+            zout.writestr("model.pb", zin.read("model.pb"))
+            npz = io.BytesIO()
+            with zipfile.ZipFile(io.BytesIO(zin.read("model.npz"))) as nin, zipfile.ZipFile(npz, "w") as nout:
+                names = nin.namelist()
+                for name in names:
+                    nout.writestr(name, nin.read(name))
+                header = ("{'descr': '<f4', 'fortran_order': False, 'shape': %s, }" % shape_text).ljust(117) + "\n"
+                nout.writestr("crafted.npy", b"\x93NUMPY\x01\x00" + struct.pack("<H", len(header)) + header.encode() + b"\0" * 16)
+            zout.writestr("model.npz", npz.getvalue())
+        return out.getvalue()
+    rt.Model(with_npy_header("(4,)"), host=True)  # 16 bytes of body: fits
+    for shape_text in ("(4294967295, 4294967295, 4294967295)", "(99999999999,)", "(5,)", "(65536, 65536, 65536, 65536, 2)"):
+        with pytest.raises(rt.RuntimeError_, match="invalid npy"):
+            rt.Model(with_npy_header(shape_text), host=True)
+
+
 def test_compute_is_not_implemented_on_the_host_device(mf, rt):
     rng = np.random.default_rng(3)
     w = mf.bert_layer_weights(rng, 32, 64)

@@ -196,6 +196,12 @@ __device__ static inline int requantize_one_biased_unclamped(unsigned off, const
   return (int)(unsigned)__double_as_longlong(fma(d, s.inScaleFolded, s.inMinBiased) + s.magicFolded);
 }
 
+// std::max and std::min as the reference's kernels call them (tfcc/mkl/interfaces/tfcc_mklminmaxinterface.cpp:37-61,
+// tfcc_mklbasicinterface.cpp:152-153, tfcc/mkl/kernel/tfcc_mklactivationkernel.hpp:67-83): a comparison that a NaN
+// fails, so the first argument comes back whenever either is a NaN (fmaxf / fminf would drop the NaN).
+__device__ __forceinline__ float ref_max(float a, float b) { return a < b ? b : a; }
+__device__ __forceinline__ float ref_min(float a, float b) { return b < a ? b : a; }
+
 // The value of lane i ^ MASK for the six steps of a butterfly over the 64 lanes, without the LDS crossbar that
 // __shfl_xor goes through: the two halves and the rows of 16 lanes are exchanged by the swap instructions (a and b
 // come back as the two members of the pair, in lane order of the lower one), the steps inside a row are data-parallel

@@ -179,7 +179,7 @@ __device__ __forceinline__ float reduce_identity() {
 }
 template <int OP>
 __device__ __forceinline__ float reduce_join(float a, float b) {
-  return OP == TFCC_ROCM_REDUCE_PROD ? a * b : OP == TFCC_ROCM_REDUCE_MAX ? fmaxf(a, b) : OP == TFCC_ROCM_REDUCE_MIN ? fminf(a, b) : a + b;
+  return OP == TFCC_ROCM_REDUCE_PROD ? a * b : OP == TFCC_ROCM_REDUCE_MAX ? ref_max(a, b) : OP == TFCC_ROCM_REDUCE_MIN ? ref_min(a, b) : a + b;
 }
 template <int OP>
 __device__ __forceinline__ float wave_join(float v) {
@@ -208,13 +208,13 @@ __global__ __launch_bounds__(256) void reduce_trailing_kernel(const float* in, s
 }
 
 // More element-wise functions of two tensors of one shape (op 4 pow, 5 max, 6 min) and of one tensor with scalars
-// (clip to [lo, hi]; leaky relu v > 0 ? v : v * alpha): tfcc/mkl/kernel/tfcc_mklactivationkernel.hpp, tfcc_math.h.
+// (clip: max(min(v, hi), lo); leaky relu: max(v, alpha * v)): tfcc/mkl/kernel/tfcc_mklactivationkernel.hpp, tfcc_math.h.
 template <int OP>
 __global__ __launch_bounds__(256) void binary2_kernel(const float* a, const float* b, size_t total, size_t period, float* out) {
   const size_t step = (size_t)gridDim.x * 256;
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += step) {
     const float x = a[i], y = b[period == total ? i : i % period];
-    out[i] = OP == 4 ? powf(x, y) : OP == 5 ? fmaxf(x, y) : fminf(x, y);
+    out[i] = OP == 4 ? powf(x, y) : OP == 5 ? ref_max(x, y) : ref_min(x, y);
   }
 }
 template <int OP>
@@ -222,7 +222,8 @@ __global__ __launch_bounds__(256) void scalar2_kernel(const float* a, size_t tot
   const size_t step = (size_t)gridDim.x * 256;
   for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += step) {
     const float v = a[i];
-    out[i] = OP == 0 ? fminf(fmaxf(v, p0), p1) : (v > 0.f ? v : v * p0);
+    // clip: min(v, hi) first, then max(., lo), as the reference; leaky relu: max(v, alpha * v)
+    out[i] = OP == 0 ? ref_max(ref_min(v, p1), p0) : ref_max(v, p0 * v);
   }
 }
 
@@ -253,8 +254,8 @@ __global__ __launch_bounds__(256) void binary_broadcast_kernel(const float* a, c
              : OP == 2 ? x * y
              : OP == 3 ? x / y
              : OP == 4 ? powf(x, y)
-             : OP == 5 ? fmaxf(x, y)
-                       : fminf(x, y);
+             : OP == 5 ? ref_max(x, y)
+                       : ref_min(x, y);
   }
 }
 
@@ -307,7 +308,7 @@ template <int OP>
 __device__ __forceinline__ float unary_value(float v) {
   if (OP == TFCC_ROCM_UNARY_SIGMOID) return 1.f / (1.f + expf(0.f - v));
   if (OP == TFCC_ROCM_UNARY_TANH) return tanhf(v);
-  if (OP == TFCC_ROCM_UNARY_RELU) return fmaxf(v, 0.f);
+  if (OP == TFCC_ROCM_UNARY_RELU) return ref_max(v, 0.f);
   if (OP == TFCC_ROCM_UNARY_SOFTPLUS) return logf(expf(v) + 1.f);
   if (OP == TFCC_ROCM_UNARY_LOG) return logf(v);
   if (OP == TFCC_ROCM_UNARY_RSQRT) return 1.f / sqrtf(v);

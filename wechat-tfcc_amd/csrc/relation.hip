@@ -301,6 +301,8 @@ int tfcc_rocm_topk_f32(void* stream, const float* in, uint64_t rows, unsigned le
   TFCC_REQUIRE(in && values && positions, "topk: null argument");
   TFCC_REQUIRE(rows > 0 && length > 0, "topk: empty tensor");
   TFCC_REQUIRE(k >= 1 && k <= length, "topk: k = %u of %u elements", k, length);
+  // one pass over the row per selected element and one workgroup per row: meant for beam-sized k
+  TFCC_REQUIRE(k <= 1024u, "topk: k = %u is beyond the 1024 this selection by repeated passes is meant for", k);
   TFCC_REQUIRE(rows < (1ull << 31) && length < 0x80000000u, "topk: tensor too large");
   hipLaunchKernelGGL(topk_rows_kernel, dim3((unsigned)rows), dim3(256), 0, as_stream(stream), in, length, k, values,
                      positions);

@@ -11,15 +11,20 @@ namespace runtime {
 
 namespace {
 
+// Offsets and sizes come from the file: every test is written so that it cannot wrap (a - b with b <= a, never a + b).
 template <class T>
-T rd(const std::string& s, size_t pos) {
-  if (pos + sizeof(T) > s.size()) throw DataFormatError("invalid zip format");
+T rd(const std::string& s, uint64_t pos) {
+  if (pos > s.size() || s.size() - pos < sizeof(T)) throw DataFormatError("invalid zip format");
   T v;
   std::memcpy(&v, s.data() + pos, sizeof(T));
   return v;
 }
 
-std::string inflate_raw(const char* src, size_t srcLen, size_t dstLen) {
+// deflate expands by at most about 1032 : 1; a stored size beyond that is not a size this stream can have
+constexpr uint64_t kMaxDeflateRatio = 1032;
+
+std::string inflate_raw(const char* src, size_t srcLen, uint64_t dstLen) {
+  if (dstLen / kMaxDeflateRatio > srcLen + 1) throw DataFormatError("invalid zip format: size beyond what the stream can hold");
   std::string out(dstLen, '\0');
   z_stream zs;
   std::memset(&zs, 0, sizeof(zs));
@@ -82,8 +87,7 @@ std::string to_c_order(const std::string& body, const std::vector<unsigned>& sha
   std::string out(body.size(), '\0');
   const size_t rank = shape.size();
   size_t total = 1;
-  for (unsigned d : shape) total *= d;
-  if (body.size() < total * itemSize) throw DataFormatError("invalid npy body");
+  for (unsigned d : shape) total *= d;  // the caller has checked total * itemSize <= body.size()
   std::vector<size_t> fstride(rank);
   size_t acc = 1;
   for (size_t d = 0; d < rank; ++d) {
@@ -141,7 +145,7 @@ std::map<std::string, std::string> unzip(const std::string& data) {
     entries = rd<uint64_t>(data, z64 + 32);
     dirOffset = rd<uint64_t>(data, z64 + 48);
   }
-  size_t pos = dirOffset;
+  uint64_t pos = dirOffset;
   for (uint64_t e = 0; e < entries; ++e) {
     if (rd<uint32_t>(data, pos) != 0x02014b50u) throw DataFormatError("invalid zip format");
     const uint16_t method = rd<uint16_t>(data, pos + 10);
@@ -151,7 +155,7 @@ std::map<std::string, std::string> unzip(const std::string& data) {
     const uint16_t extraLen = rd<uint16_t>(data, pos + 30);
     const uint16_t commentLen = rd<uint16_t>(data, pos + 32);
     uint64_t localOffset = rd<uint32_t>(data, pos + 42);
-    if (pos + 46 + nameLen + extraLen > data.size()) throw DataFormatError("invalid zip format");
+    if (data.size() - pos < 46ull + nameLen + extraLen) throw DataFormatError("invalid zip format");  // pos <= size: read above
     const std::string name = data.substr(pos + 46, nameLen);
     // zip64 extra field (id 1): present values in the order size, compressed size, local offset
     size_t x = pos + 46 + nameLen;
@@ -169,8 +173,10 @@ std::map<std::string, std::string> unzip(const std::string& data) {
     }
     if (method != 0 && method != 8) throw DataFormatError("invalid zip compress type: " + std::to_string(method));
     if (rd<uint32_t>(data, localOffset) != 0x04034b50u) throw DataFormatError("invalid zip format");
-    const size_t body = localOffset + 30 + rd<uint16_t>(data, localOffset + 26) + rd<uint16_t>(data, localOffset + 28);
-    if (body + compressedSize > data.size()) throw DataFormatError("invalid zip format");
+    // localOffset + 30 <= size after the reads below, so `body` cannot wrap
+    const uint64_t body = localOffset + 30 + rd<uint16_t>(data, localOffset + 26) + rd<uint16_t>(data, localOffset + 28);
+    if (body > data.size() || compressedSize > data.size() - body) throw DataFormatError("invalid zip format");
+    if (method == 0 && size != compressedSize) throw DataFormatError("invalid zip format");
     if (!name.empty() && name.back() != '/') {
       result[name] = method == 0 ? data.substr(body, compressedSize)
                                  : inflate_raw(data.data() + body, compressedSize, size);
@@ -190,7 +196,10 @@ std::map<std::string, std::string> unzip_from_path(const std::string& path) {
 
 size_t NpyArray::count() const {
   size_t n = 1;
-  for (unsigned d : shape) n *= d;
+  for (unsigned d : shape) {
+    if (d != 0 && n > static_cast<size_t>(-1) / d) throw DataFormatError("invalid npy shape: too many elements");
+    n *= d;
+  }
   return n;
 }
 
@@ -206,7 +215,7 @@ NpyArray parse_npy(const std::string& data) {
   } else {
     throw DataFormatError("unknow npy version");
   }
-  if (pos + headLength > data.size()) throw DataFormatError("invalid npy header");
+  if (headLength > data.size() - pos) throw DataFormatError("invalid npy header");
   const std::string header = data.substr(pos, headLength);
   const std::string descr = dict_value(header, "descr");  // quoted: '<f4'
   if (descr.size() < 5) throw DataFormatError("invalid npy descr");
@@ -223,7 +232,10 @@ NpyArray parse_npy(const std::string& data) {
     if (strShape[i] >= '0' && strShape[i] <= '9') {
       num += strShape[i];
     } else if (!num.empty()) {
-      a.shape.push_back(static_cast<unsigned>(std::stoull(num)));
+      if (num.size() > 10) throw DataFormatError("invalid npy shape");  // no dimension has more than 10 digits
+      const unsigned long long extent = std::stoull(num);
+      if (extent > 0xffffffffull) throw DataFormatError("invalid npy shape");
+      a.shape.push_back(static_cast<unsigned>(extent));
       num.clear();
     }
   }
@@ -233,7 +245,8 @@ NpyArray parse_npy(const std::string& data) {
   a.type = descr.substr(2, descr.size() - 3);
   const size_t itemSize = std::stoull(a.type.substr(1));
   a.body = data.substr(pos + headLength);
-  if (a.body.size() < a.count() * itemSize) throw DataFormatError("invalid npy body");
+  const size_t count = a.count();
+  if (itemSize == 0 || count > a.body.size() / itemSize) throw DataFormatError("invalid npy body");
   if (order == "True" && a.shape.size() > 1) a.body = to_c_order(a.body, a.shape, itemSize);
   return a;
 }
