@@ -74,25 +74,39 @@ __device__ __forceinline__ void transpose4x4(const unsigned r[4], unsigned c[4])
   c[3] = __builtin_amdgcn_perm(t3, t1, 0x07060302u);
 }
 
-__global__ __launch_bounds__(kThreads) void gemv_wide_kernel(const GemvWideParams p) {
+// The arguments a wavefront needs before it can ask for its first bytes come first and one by one: the build
+// passes -amdgpu-kernarg-preload-count, which has the first arguments of a kernel (scalars and pointers, up to the
+// free user SGPRs) delivered in registers at wavefront start instead of fetched from the argument block, a round trip
+// of about 0.6 us at the head of a 12 us kernel.  The argument block still carries everything (hot.* repeats them).
+struct GemvWideHot {
+  const signed char* B;
+  const unsigned char* A;
+  unsigned M, N, K, colBlocks, kParts, stepsPerWave, chunk;
+};
+__global__ __launch_bounds__(kThreads) void gemv_wide_kernel(const signed char* hotB, const unsigned char* hotA,
+                                                             unsigned hotM, unsigned hotN, unsigned hotK,
+                                                             unsigned hotColBlocks, unsigned hotKParts,
+                                                             unsigned hotStepsPerWave, unsigned hotChunk,
+                                                             const GemvWideParams p) {
   __shared__ int tile[kPartRows * kRowPitch];
+  const GemvWideHot hot = {hotB, hotA, hotM, hotN, hotK, hotColBlocks, hotKParts, hotStepsPerWave, hotChunk};
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   // Consecutive workgroup ids go to different XCDs: each XCD gets a contiguous run of (column block, part) pairs,
   // so that the parts of a block mostly meet on one XCD and every XCD has the same number of pairs to within one
   // (measured: 1.1 us faster than handing the pairs out in the order of the ids).
-  const unsigned L = (blockIdx.x & 7u) * p.chunk + (blockIdx.x >> 3);
-  if ((blockIdx.x >> 3) >= p.chunk || L >= p.colBlocks * p.kParts) return;
-  const unsigned cb = L / p.kParts, part = L - cb * p.kParts;
+  const unsigned L = (blockIdx.x & 7u) * hot.chunk + (blockIdx.x >> 3);
+  if ((blockIdx.x >> 3) >= hot.chunk || L >= hot.colBlocks * hot.kParts) return;
+  const unsigned cb = L / hot.kParts, part = L - cb * hot.kParts;
   const unsigned n0 = cb * kCols;
-  const unsigned M = p.M, N = p.N, K = p.K;
+  const unsigned M = hot.M, N = hot.N, K = hot.K;
   const int j = lane & 15, kg = lane >> 4;
 
   const __amdgpu_buffer_rsrc_t rsrcB =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<signed char*>(p.B), 0, (int)(K * N), 0x00020000);
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<signed char*>(hot.B), 0, (int)(K * N), 0x00020000);
   const __amdgpu_buffer_rsrc_t rsrcA =
-      __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(p.A), 0, (int)(M * K), 0x00020000);
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<unsigned char*>(hot.A), 0, (int)(M * K), 0x00020000);
 
   // What the end of the kernel needs from memory is asked for now: column tid % 256 of every row this thread
   // finishes (rows tid / 256 + kRowsPerPass t), so that the only wait left there is the atomic's own.
@@ -114,7 +128,7 @@ __global__ __launch_bounds__(kThreads) void gemv_wide_kernel(const GemvWideParam
   // columns past N: a lane whose 16 columns lie outside reads nothing (N is a multiple of 16)
   const bool colsInside = n0 + 16u * j < N;
   const unsigned steps = (K + 63) / 64;
-  const unsigned firstStep = (part * kWaves + wave) * p.stepsPerWave;
+  const unsigned firstStep = (part * kWaves + wave) * hot.stepsPerWave;
   v4i raw[16], aRaw;
   // the 16 rows x 16 columns of this lane in step `step` (steps and rows past the end read zeros) and its 16
   // bytes of row j of A
@@ -129,11 +143,12 @@ __global__ __launch_bounds__(kThreads) void gemv_wide_kernel(const GemvWideParam
     }
   };
   // (the tile is cleared before the loads are issued: a barrier waits for all of a wavefront's outstanding
-  // memory operations, and with the loads ahead of it every wavefront would wait for the slowest one's data)
+  // memory operations, and with the loads ahead of it every wavefront would wait for the slowest one's data; a bare
+  // s_barrier after a wait for the LDS stores alone, with the loads issued first, measured 0.6 us slower still)
   for (int i = tid; i < kPartRows * kRowPitch; i += kThreads) tile[i] = 0;
   __syncthreads();
   issueLoads(firstStep);
-  for (unsigned s = 0; s < p.stepsPerWave; ++s) {
+  for (unsigned s = 0; s < hot.stepsPerWave; ++s) {
     const unsigned step = firstStep + s;
     if (step >= steps) break;  // wave-uniform; no barrier inside this loop
     const unsigned k0 = step * 64 + kg * 16;  // this lane's 16 rows
@@ -170,7 +185,7 @@ __global__ __launch_bounds__(kThreads) void gemv_wide_kernel(const GemvWideParam
         }
       }
     }
-    if (s + 1 < p.stepsPerWave) issueLoads(step + 1);
+    if (s + 1 < hot.stepsPerWave) issueLoads(step + 1);
   }
   __syncthreads();
 
@@ -192,12 +207,12 @@ __global__ __launch_bounds__(kThreads) void gemv_wide_kernel(const GemvWideParam
     const unsigned r = er0 + kRowsPerPass * t, idx = r * kCols + ec;
     if (r >= M || egn >= N) continue;
     unsigned sum = (unsigned)tile[tile_slot(r, ec)] + 128u * (unsigned)tile[tile_slot(kMaxM, ec)];
-    if (p.kParts > 1) {
+    if (hot.kParts > 1) {
       // Device scope: the parts of a column block may run anywhere on the chip.  One element after the other: with
       // all of a thread's atomics under way at once the kernel measured 0.5 us slower.
       const unsigned long long before =
           __hip_atomic_fetch_add(ws + idx, ((unsigned long long)sum << 32) | 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if ((unsigned)before != p.kParts - 1) continue;  // others are still to come: one of them finishes the element
+      if ((unsigned)before != hot.kParts - 1) continue;  // others are still to come: one of them finishes the element
       sum += (unsigned)(before >> 32);
       __hip_atomic_store(ws + idx, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
@@ -299,7 +314,8 @@ int gemv_wide_launch(hipStream_t stream, bool staticWorkspace, const unsigned ch
     if (int e = workspace_for(stream, p.colBlocks, &w)) return e;
   }
   p.tiles = w.tiles;
-  hipLaunchKernelGGL(gemv_wide_kernel, dim3(p.chunk * 8), dim3(kThreads), 0, stream, p);
+  hipLaunchKernelGGL(gemv_wide_kernel, dim3(p.chunk * 8), dim3(kThreads), 0, stream, p.B, p.A, p.M, p.N, p.K,
+                     p.colBlocks, p.kParts, p.stepsPerWave, p.chunk, p);
   return check_launch("skinny quantized matmul (split over K)");
 }
 
