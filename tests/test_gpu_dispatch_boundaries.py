@@ -138,3 +138,39 @@ def test_qgemm_around_configuration_thresholds(pkg, T, m, n, k):
     q, _, _, _ = pkg.quantization_matmul_requantize(T.t(a), T.t(rs), T.f1(-128.0), T.f1(127.0), T.t(b), T.t(cs),
                                                     T.f1(-128.0), T.f1(127.0), T.f1(-lim), T.f1(lim), want_acc=False)
     assert np.array_equal(T.n(q), O.requantize_s32_u8(want, mn_c, mx_c, -lim, lim))
+
+
+@pytest.mark.parametrize("m,n,k", [
+    # the products the dispatcher gives 32 x 96 tiles with four K groups: the hand-scheduled kernel with one
+    # wavefront per K group.  Whole tiles; a ragged last row band; a ragged last column block; a K whose 32-k slabs do
+    # not divide by four (one group gets a slab more than the others); a long narrow product; the shortest K it takes
+    (1024, 768, 768), (1000, 768, 3072), (1024, 748, 1024), (1024, 768, 1056), (8192, 96, 2048), (1024, 768, 1024),
+])
+def test_sgemm_on_32x96_tiles_with_four_k_groups(pkg, T, m, n, k):
+    """The same bits as the register-staged kernel (reached through a transposed B, which is summed with the same
+    K groups), the fused bias + residual + GELU equal to the separate kernels, float64 within the fp32 tolerance."""
+    import torch
+    print("sgemm 32x96 / 4 K groups", m, n, k, flush=True)
+    rng = np.random.default_rng(m * 5 + n * 3 + k)
+    a = rng.normal(0, 1, (m, k)).astype(np.float32)
+    b = rng.normal(0, 1, (k, n)).astype(np.float32)
+    bias = rng.uniform(-1, 1, n).astype(np.float32)
+    res = rng.normal(0, 1, (m, n)).astype(np.float32)
+    ta, tb, tbias, tres = T.t(a), T.t(b), T.t(bias), T.t(res)
+    # this shape is one of those the test is about (the predicate of the one-launch layer norm is that of the kernel)
+    assert pkg.sgemm_layer_norm_supported(ta, tb)
+    plain = T.n(pkg.blas_matmul(ta, tb))
+    assert rel_fro(plain, a.astype(np.float64) @ b.astype(np.float64)) <= FP32_TOL
+    c = torch.empty((m, n), dtype=torch.float32, device=ta.device)
+    pkg.sgemm_general(ta, T.t(np.ascontiguousarray(b.T)), c, m, n, k, k, k, n, trans_b=True)
+    assert np.array_equal(T.n(c), plain)
+    out = torch.empty((m, n), dtype=torch.float32, device=ta.device)
+    pkg.check(pkg.lib().tfcc_rocm_sgemm_fused(None, ta.data_ptr(), 0, tb.data_ptr(), 0, tbias.data_ptr(),
+                                              tres.data_ptr(), 0, out.data_ptr(), 0, m, n, k, 1, 1))
+    separate = T.n(pkg.gelu_accurate(pkg.add(pkg.blas_matmul(ta, tb, tbias), tres)))
+    assert np.array_equal(T.n(out), separate)
+    # three products that share A in one launch (more than two tiles per CU: the rings of three 8-k slabs)
+    bs = [tb, T.t(b[:, ::-1].copy()), T.t((b * 0.5).astype(np.float32))]
+    grouped = pkg.sgemm_grouped(ta, bs, [tbias, tbias, tbias])
+    for g, bb in zip(grouped, bs):
+        assert np.array_equal(T.n(g), T.n(pkg.blas_matmul(ta, bb, tbias)))
