@@ -1,24 +1,30 @@
 // fp32 matrix product for mid-sized shapes: one wavefront per SIMD, 32 x 96 outputs per wavefront.
 //
 // A product like 1024 x 3072 x 768 has about one tile per CU, so nothing overlaps a workgroup's stalls except its
-// own instruction order.  The kernels of sgemm_dma.hip leave that order to the compiler, which sinks the LDS reads
-// next to their matrix ops (fewer registers) and waits for each in turn; with one wavefront per SIMD that costs a
-// fifth of the time.  Here the order is written down: a k step is twelve 32x32x2 matrix ops (4 k pairs x 3 column
-// blocks, 64 cycles each), and the 13 LDS reads of the next step's operands and the step's share of the HBM -> LDS
-// copies are dealt out over the issue slots between them, one step ahead, into a second set of registers.
+// own instruction order, and on this hardware nothing overlaps the fp32 matrix ops at all: while one wavefront issues
+// them back to back, vector instructions of every wavefront on the SIMD wait (a vector instruction between two
+// matrix ops costs about 15 cycles, an LDS read 1.5, a copy 2, scalar instructions nothing).  So the order is
+// written down and the loop holds matrix ops, LDS reads, copies and scalar work only: a k step is twelve 32x32x2
+// matrix ops (4 k pairs x 3 column blocks, 64 cycles each); the LDS reads of the next step's operands (one 128-bit
+// read of A, six two-word reads of B) and the step's share of the HBM -> LDS copies are dealt out over the issue
+// slots between them, one step ahead, into a second set of registers; the loop is unrolled over the ring's stages so
+// that every LDS address is a register set up before the loop plus an immediate.  Measured in the loop: 64.3-65.5
+// cycles per matrix op.
 //
 // Two shapes of workgroup, four wavefronts each:
 //   groups (WGM = 1, KSPLIT = 4)  a 32 x 96 tile, wavefront q sums the 32-k slabs q, q + 4, ... in a ring of its
-//                                 own (two half slabs of 16 k, 16 KB per wavefront, so that two workgroups share a
-//                                 CU and one's set-up and tile store run under the other's matrix ops; no barrier
+//                                 own (two half slabs of 16 k, or three of 8 k when three workgroups share a CU, so
+//                                 that one's set-up and tile store run under the others' matrix ops; no barrier
 //                                 in the loop); the four partial tiles meet in LDS and every wavefront finishes a
-//                                 quarter of the tile.  This is the shape the dispatcher uses: 1024 x 768 x 3072
-//                                 39.2 us against 45.9 for the twelve-wavefront kernel of sgemm_dma.hip, three
-//                                 1024 x 768 x 768 products in one launch 33.4 against 39.9.
-//   rows   (WGM = 4, KSPLIT = 1)  a 128 x 96 tile, wavefront w owns rows 32w..32w+31, the ring (slabs of 32 k:
-//                                 A 128 x 32 + B 32 x 96) is shared, one barrier per slab.  Measured no faster than
-//                                 the twelve-wavefront kernel on 1024 x 3072 x 768 (the tile store with its GELU is
-//                                 not hidden by anything) and not dispatched.
+//                                 quarter of the tile.  For products the dispatcher sums in four K groups:
+//                                 1024 x 768 x 3072 36.3 us against 45.9 for the twelve-wavefront kernel of
+//                                 sgemm_dma.hip, three 1024 x 768 x 768 products in one launch 29.5 against 39.9.
+//   rows   (WGM = 4, KSPLIT = 1)  a 128 x 96 tile, wavefront w owns rows 32w..32w+31, the ring (four slabs of 32 k:
+//                                 A 128 x 32 + B 32 x 96) is shared, one barrier per slab.  For products summed in
+//                                 one pass over K whose 128 x 96 tiles fill the CUs: 1024 x 3072 x 768 with GELU
+//                                 40.0 us against 42.4 in 64 x 64 tiles.
+// Whole tiles are stored through a buffer descriptor (a lane offset, a scalar per row, an immediate per column
+// block: no address arithmetic or bounds checks per value); edge tiles take the checked path.
 // The arithmetic is that of sgemm_dma.hip instruction for instruction (k pairs (8kb + s, 8kb + 4 + s) in ascending
 // kb, s; groups added in group order), so a product has the same bits whichever kernel the dispatcher picks for its
 // number of K groups.  Replaces the same oneDNN calls (tfcc/mkl/interfaces/tfcc_mklblasinterface.cpp:41-67, 69-78,
@@ -45,8 +51,16 @@ __device__ __forceinline__ int a_row_swizzle(int row) {
   return BK == 32 ? (row >> 1) & 7 : BK == 16 ? (row >> 2) & 3 : (row >> 2) & 1;
 }
 
-template <int WGM, int KSPLIT, int BK, int STAGES>
-__global__ __launch_bounds__(256) void sgemm_wave96_kernel(const SgemmParams p) {
+template <int WGM, int KSPLIT, int BK, int STAGES, bool PLAIN>
+__global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, const float* hotB, const float* hotB1,
+                                                           const float* hotB2, unsigned hotM, unsigned hotN,
+                                                           unsigned hotK, unsigned hotLda, unsigned hotLdb,
+                                                           unsigned hotBatch, const SgemmParams p) {
+  // The leading arguments repeat what the first copies need: scalar arguments at the front of the list arrive in
+  // registers with the wavefront, the structure has to be fetched from the argument block first, and nothing of it
+  // is looked at before the first slabs are on their way when PLAIN (every batch entry's A starts at hotA, and
+  // either its B at hotB too or the launch is the grouped form with at most three products: hotB, hotB1, hotB2 are
+  // their B).  hotBatch: p.batch, bit 30 set for the grouped form.
   static_assert(WGM * KSPLIT == 4, "four wavefronts");
   static_assert(BK == 32 || BK == 16 || BK == 8, "ring slabs of 32, 16 or 8 k");
   static_assert(STAGES >= 2, "ring depth");
@@ -63,6 +77,7 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const SgemmParams p) 
   constexpr int BCH = BN96 / 4;     // 16-byte chunks per B row
   constexpr bool SHARED = WGM > 1;  // the group's wavefronts read each other's copies
 
+  stagger_by_wave_slot();
   extern __shared__ __align__(16) unsigned char smem[];
   const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int grp = wv / WGM, wm = wv - grp * WGM;  // wave-uniform
@@ -75,31 +90,35 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const SgemmParams p) 
     // consecutive workgroup ids land on different XCDs: hand each XCD a contiguous run of tiles
     const unsigned wg = blockIdx.x;
     const unsigned xcd = wg & 7u, slot = wg >> 3;
-    const unsigned L = xcd * p.chunk + slot;
-    if (slot >= p.chunk || L >= p.tilesTotal) return;
-    const unsigned perBatch = p.tilesM * p.tilesN;
+    const unsigned tilesM = (hotM + BM - 1) / BM, tilesN = (hotN + BN96 - 1) / BN96;
+    const unsigned perBatch = tilesM * tilesN;
+    const unsigned tilesTotal = perBatch * (hotBatch & 0x3fffffffu);  // the launcher checks that this fits
+    const unsigned chunk = (tilesTotal + 7u) / 8u;
+    const unsigned L = xcd * chunk + slot;
+    if (slot >= chunk || L >= tilesTotal) return;
     bi = L / perBatch;
     unsigned t = L - bi * perBatch;
-    const unsigned band = 4u * p.tilesN;
+    const unsigned band = 4u * tilesN;
     unsigned gb = t / band;
-    unsigned rowsInBand = min(4u, p.tilesM - gb * 4u);
+    unsigned rowsInBand = min(4u, tilesM - gb * 4u);
     unsigned r = t - gb * band;
     tm = gb * 4u + r % rowsInBand;
     tn = r / rowsInBand;
   }
   const unsigned m0 = tm * BM, n0 = tn * BN96;
-  const unsigned M = p.M, N = p.N, K = p.K;
-  const unsigned bo = bi / p.batchInner, bn = bi - bo * p.batchInner;
-  const float* A = p.A + (size_t)bo * p.strideA + (size_t)bn * p.innerA;
-  const float* B = p.B + (size_t)bo * p.strideB + (size_t)bn * p.innerB;
-  const float* biasPtr = p.bias;
-  float* Cbase = p.C + (size_t)bo * p.strideC + (size_t)bn * p.innerC;
-  if (p.groups) {  // selects, not indexing: the argument block stays in scalar registers
-    B = bi == 0 ? p.groupB[0] : bi == 1 ? p.groupB[1] : bi == 2 ? p.groupB[2] : p.groupB[3];
-    biasPtr = bi == 0 ? p.groupBias[0] : bi == 1 ? p.groupBias[1] : bi == 2 ? p.groupBias[2] : p.groupBias[3];
-    Cbase = bi == 0 ? p.groupC[0] : bi == 1 ? p.groupC[1] : bi == 2 ? p.groupC[2] : p.groupC[3];
+  const unsigned M = hotM, N = hotN, K = hotK;
+  const bool grouped = (hotBatch >> 30) & 1u;
+  const float* A = hotA;
+  const float* B = hotB;
+  if (grouped) {
+    B = bi == 1 ? hotB1 : bi == 2 ? hotB2 : B;
+    if (!PLAIN) B = bi == 3 ? p.groupB[3] : B;
+  } else if (!PLAIN) {
+    const unsigned bo = bi / p.batchInner, bn = bi - bo * p.batchInner;
+    A += (size_t)bo * p.strideA + (size_t)bn * p.innerA;
+    B += (size_t)bo * p.strideB + (size_t)bn * p.innerB;
   }
-  const unsigned lda = p.lda, ldb = p.ldb, ldc = p.ldc;
+  const unsigned lda = hotLda, ldb = hotLdb;
   const w96_v4i rsrcA = make_rsrc(A, ((M - 1) * lda + K) * 4u);
   const w96_v4i rsrcB = make_rsrc(B, ((K - 1) * ldb + N) * 4u);
 
@@ -146,21 +165,39 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const SgemmParams p) 
 #pragma unroll
     for (int c = 0; c < COPIES; ++c) issueCopy((unsigned)s, (unsigned)s, c);
 
+  // What the tile store needs from the argument block is worked out from here on (the empty statement keeps the
+  // compiler from moving it, and the wait for the block, in front of the copies).
+  unsigned late = 0;
+  asm volatile("" : "+s"(late));
+  const unsigned biL = bi + late;
+  const unsigned ldc = p.ldc;
+  const float* biasPtr = p.bias;
+  float* Cbase;
+  if (grouped) {  // selects, not indexing: the argument block stays in scalar registers
+    biasPtr = biL == 0 ? p.groupBias[0] : biL == 1 ? p.groupBias[1] : biL == 2 ? p.groupBias[2] : p.groupBias[3];
+    Cbase = biL == 0 ? p.groupC[0] : biL == 1 ? p.groupC[1] : biL == 2 ? p.groupC[2] : p.groupC[3];
+  } else {
+    const unsigned bo = biL / p.batchInner, bn = biL - bo * p.batchInner;
+    Cbase = p.C + (size_t)bo * p.strideC + (size_t)bn * p.innerC;
+  }
+
   // ---- values needed only in the tile store are fetched now.  Rows: lane (lrow, g) stores, for register r of
   // column block j, row 8*(r/4) + 4*g + r%4 of its wavefront's 32 and column 32*j + lrow.  Groups: after the
-  // partial tiles met in LDS, wavefront w finishes registers 12w .. 12w+11 of the 48 (j = idx / 16, r = idx % 16).
+  // partial tiles met in LDS, wavefront w finishes registers 4w .. 4w+3 of each column block (rows 8w + 4g + e):
+  // value q = 4j + e of its twelve is register 4w + e of block j.
   constexpr int OWN = KSPLIT == 1 ? 48 : 12;
-  const int firstIdx = KSPLIT == 1 ? 0 : 12 * grp;
+  auto ownBlock = [&](int q) { return KSPLIT == 1 ? q >> 4 : q >> 2; };
+  auto ownRegister = [&](int q) { return KSPLIT == 1 ? q & 15 : 4 * grp + (q & 3); };
   const unsigned gcol0 = n0 + lrow;
   float bv[3];
 #pragma unroll
   for (int j = 0; j < 3; ++j) bv[j] = (biasPtr && gcol0 + 32 * j < N) ? biasPtr[gcol0 + 32 * j] : 0.f;
   float rv[OWN];
-  const float* Rp = p.residual ? p.residual + (size_t)bi * p.strideR : nullptr;  // dense, flat batch
+  const float* Rp = p.residual ? p.residual + (size_t)biL * p.strideR : nullptr;  // dense, flat batch
   if (Rp) {
 #pragma unroll
     for (int q = 0; q < OWN; ++q) {
-      const int idx = firstIdx + q, j = idx >> 4, r = idx & 15;
+      const int j = ownBlock(q), r = ownRegister(q);
       const unsigned grow = m0 + wm * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
       const unsigned gc = gcol0 + 32 * j;
       rv[q] = (grow < M && gc < N) ? Rp[(size_t)grow * N + gc] : 0.f;
@@ -179,16 +216,52 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const SgemmParams p) 
   const int aBase = arow * (BK * 4), aSwz = a_row_swizzle<BK>(arow);
   const int bBase = A_BYTES + (4 * g) * (BN96 * 4) + lrow * 4;
   struct Ops { w96_v4f a; float b[4][3]; };
+  // In the unrolled part of the loop the stage is a constant, and every LDS address is one of a few registers set up
+  // here plus an immediate: no address arithmetic between the matrix ops.  The B operands of a step are then read two
+  // per instruction (two offsets of up to 255 words from one register: a register per stage, k step and half step).
+  typedef const __attribute__((address_space(3))) float* LdsFloats;
+  typedef const __attribute__((address_space(3))) w96_v4f* LdsQuads;
+  constexpr bool PAIRED = STAGES * KS * 2 <= 8;
+  unsigned aAddr[KS], bAddr[PAIRED ? STAGES : 1][KS][2];
+#pragma unroll
+  for (int kb = 0; kb < KS; ++kb) {
+    aAddr[kb] = ldsGroup + aBase + (((2 * kb + g) ^ aSwz) << 4);
+    asm volatile("" : "+v"(aAddr[kb]));
+#pragma unroll
+    for (int st = 0; st < (PAIRED ? STAGES : 1); ++st)
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        bAddr[st][kb][h] = ldsGroup + st * STAGE_BYTES + bBase + (8 * kb + 2 * h) * (BN96 * 4);
+        asm volatile("" : "+v"(bAddr[st][kb][h]));
+      }
+  }
 
-  // One k step: twelve matrix ops on `cur`; in the issue slots between them the 13 reads of the operands of step
-  // (ldStage, ldKb) into `nxt` and, in a slab's last step, the copies of the slab that takes its stage.
-  auto step = [&](const Ops& cur, Ops& nxt, const unsigned char* ldStage, int ldKb, bool dma, unsigned dmaSlab,
-                  unsigned dmaStage) {
+  // One k step: twelve matrix ops on `cur`; in the issue slots between them the reads of the operands of step
+  // (ldStage, ldKb) into `nxt` and, in a slab's last step, the copies of the slab that takes its stage.  fixedStage:
+  // ldStage is a constant where the call is written.
+  auto step = [&](const Ops& cur, Ops& nxt, unsigned ldStage, int ldKb, bool fixedStage, bool dma, unsigned dmaSlab,
+                  unsigned dmaStage) __attribute__((always_inline)) {
+    const unsigned char* st = gsm + ldStage * STAGE_BYTES;
 #pragma unroll
     for (int m = 0; m < 12; ++m) {
       const int s = m / 3, j = m % 3;
-      if (m == 0) nxt.a = *reinterpret_cast<const w96_v4f*>(ldStage + aBase + (((2 * ldKb + g) ^ aSwz) << 4));
-      nxt.b[s][j] = *reinterpret_cast<const float*>(ldStage + bBase + (8 * ldKb + s) * (BN96 * 4) + j * 128);
+      if (fixedStage) {
+        if (m == 0) nxt.a = *reinterpret_cast<LdsQuads>(aAddr[ldKb] + ldStage * STAGE_BYTES);
+        if (PAIRED) {
+          if (m & 1) {  // values 2 * (m / 2) and 2 * (m / 2) + 1 of the twelve, three to a k row
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+              const int v = (m / 2) * 2 + e, vs = v / 3, vj = v % 3;
+              nxt.b[vs][vj] = reinterpret_cast<LdsFloats>(bAddr[PAIRED ? ldStage : 0][ldKb][vs / 2])[(vs & 1) * BN96 + vj * 32];
+            }
+          }
+        } else {
+          nxt.b[s][j] = reinterpret_cast<LdsFloats>(bAddr[0][ldKb][0] + ldStage * STAGE_BYTES)[s * BN96 + j * 32];
+        }
+      } else {
+        if (m == 0) nxt.a = *reinterpret_cast<const w96_v4f*>(st + aBase + (((2 * ldKb + g) ^ aSwz) << 4));
+        nxt.b[s][j] = *reinterpret_cast<const float*>(st + bBase + (8 * ldKb + s) * (BN96 * 4) + j * 128);
+      }
       if (dma && m >= 1 && m <= COPIES) issueCopy(dmaSlab, dmaStage, m - 1);
       acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(cur.a[s], cur.b[s][j], acc[j], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);
@@ -207,28 +280,38 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const SgemmParams p) 
   for (int s = 0; s < 4; ++s)
 #pragma unroll
     for (int j = 0; j < 3; ++j) ops[0].b[s][j] = *reinterpret_cast<const float*>(gsm + bBase + s * (BN96 * 4) + j * 128);
-  // one ring slab: KS steps starting on the operands in `first`; the next slab's first operands end up in `first`
-  // again when KS is even, in `other` when it is odd (then the loop below alternates the two)
-  unsigned stage = 0;  // of slab t
-  auto slab = [&](unsigned t, Ops& first, Ops& other) {
+  // one ring slab in stage `stage`: KS steps starting on the operands in `first`; the next slab's first operands end
+  // up in `first` again when KS is even, in `other` when it is odd (then the loops below alternate the two)
+  auto slab = [&](unsigned t, unsigned stage, bool fixedStage, Ops& first, Ops& other) __attribute__((always_inline)) {
     const unsigned next = stage + 1 == STAGES ? 0 : stage + 1;
-    const unsigned char* stCur = gsm + stage * STAGE_BYTES;
-    const unsigned char* stNext = gsm + next * STAGE_BYTES;
 #pragma unroll
-    for (int kb = 0; kb < KS - 1; ++kb) step(kb & 1 ? other : first, kb & 1 ? first : other, stCur, kb + 1, false, 0u, 0u);
+    for (int kb = 0; kb < KS - 1; ++kb)
+      step(kb & 1 ? other : first, kb & 1 ? first : other, stage, kb + 1, fixedStage, false, 0u, 0u);
     wait_vmcnt<COPIES*(STAGES - 2)>();
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the reads of slab t have returned
     if constexpr (SHARED) __syncthreads();
-    step((KS - 1) & 1 ? other : first, (KS - 1) & 1 ? first : other, stNext, 0, true, t + STAGES, stage);
-    stage = next;
+    step((KS - 1) & 1 ? other : first, (KS - 1) & 1 ? first : other, next, 0, fixedStage, true, t + STAGES, stage);
   };
-  if constexpr (KS & 1) {
-    for (unsigned t = 0; t < T; t += 2) {  // T is a multiple of 32 / BK >= 2
-      slab(t, ops[0], ops[1]);
-      slab(t + 1, ops[1], ops[0]);
+  // U slabs per trip with the stages written out (a multiple of the ring depth, even when the operand sets
+  // alternate); what is left of T after whole trips runs with the stage counted.  T is a multiple of 32 / BK.
+  constexpr int ALT = (KS & 1) ? 2 : 1;
+  constexpr int U = STAGES % ALT == 0 ? STAGES : STAGES * ALT;
+  unsigned t = 0;
+  for (; t + U <= T; t += U) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const bool odd = (KS & 1) && (u & 1);
+      slab(t + u, u % STAGES, true, ops[odd ? 1 : 0], ops[odd ? 0 : 1]);
     }
-  } else {
-    for (unsigned t = 0; t < T; ++t) slab(t, ops[0], ops[1]);
+  }
+  unsigned stage = 0;  // U is a multiple of the ring depth
+  for (; t < T; t += ALT) {
+    slab(t, stage, false, ops[0], ops[1]);
+    stage = stage + 1 == STAGES ? 0 : stage + 1;
+    if constexpr (KS & 1) {
+      slab(t + 1, stage, false, ops[1], ops[0]);
+      stage = stage + 1 == STAGES ? 0 : stage + 1;
+    }
   }
   wait_vmcnt<0>();
   __syncthreads();
@@ -243,6 +326,27 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const SgemmParams p) 
     return v;
   };
   if constexpr (KSPLIT == 1) {
+    if (m0 + wm * 32 + 32 <= M && n0 + BN96 <= N && ldc < (1u << 24)) {
+      // A whole tile: no bounds to check, and the addresses are a register per lane (row 4g, column lrow), a scalar
+      // per row and an immediate per column block.
+      const __amdgpu_buffer_rsrc_t rc =
+          __builtin_amdgcn_make_buffer_rsrc(Cbase + (size_t)(m0 + wm * 32) * ldc + n0, 0, 0x7fffffff, 0x00020000);
+      const unsigned voff = ((4 * g) * ldc + lrow) * 4u;
+      auto store = [&](bool gelu) __attribute__((always_inline)) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+#pragma unroll
+          for (int j = 0; j < 3; ++j) {
+            float out = acc[j][r] + bv[j];
+            if (Rp) out += rv[j * 16 + r];
+            if (gelu) out = gelu_erf_f32(out);
+            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, out), rc, voff + j * 128,
+                                                  (8 * (r >> 2) + (r & 3)) * ldc * 4u, 0);
+          }
+      };
+      if (act == 1) store(true); else store(false);
+      return;
+    }
 #pragma unroll
     for (int j = 0; j < 3; ++j) {
       const unsigned gc = gcol0 + 32 * j;
@@ -254,8 +358,8 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const SgemmParams p) 
     }
   } else {
     // the four partial tiles go through LDS (the rings are idle now), four registers per 128-bit access: registers
-    // 4c .. 4c+3 of group q lie at red4[(q * 12 + c) * 64 + lane]; wavefront w adds the four of its twelve registers
-    // (quads 3w .. 3w+2) in group order
+    // 4c .. 4c+3 of column block j of group q lie at red4[(q * 12 + 4 * j + c) * 64 + lane]; wavefront w adds quad
+    // c = w of every block in group order
     w96_v4f* red4 = reinterpret_cast<w96_v4f*>(smem);
 #pragma unroll
     for (int j = 0; j < 3; ++j)
@@ -265,30 +369,47 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const SgemmParams p) 
     __syncthreads();
     float sums[12];
 #pragma unroll
-    for (int c = 0; c < 3; ++c) {
-      w96_v4f v = red4[(3 * grp + c) * 64 + lane];
+    for (int j = 0; j < 3; ++j) {
+      w96_v4f v = red4[(4 * j + grp) * 64 + lane];
 #pragma unroll
       for (int o = 1; o < KSPLIT; ++o) {
-        const w96_v4f w = red4[(o * 12 + 3 * grp + c) * 64 + lane];
+        const w96_v4f w = red4[(o * 12 + 4 * j + grp) * 64 + lane];
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] += w[e];
       }
 #pragma unroll
-      for (int e = 0; e < 4; ++e) sums[4 * c + e] = v[e];
+      for (int e = 0; e < 4; ++e) sums[4 * j + e] = v[e];
+    }
+    const bool toSums = p.lnGamma != nullptr;
+    if (m0 + 32 <= M && n0 + BN96 <= N && ldc < (1u << 24) && !toSums) {
+      // A whole tile: no bounds to check, and the addresses are a register per lane (row 4g, column lrow of the
+      // wavefront's eight rows), a scalar per row and an immediate per column block.
+      const __amdgpu_buffer_rsrc_t rc =
+          __builtin_amdgcn_make_buffer_rsrc(Cbase + (size_t)(m0 + 8 * grp) * ldc + n0, 0, 0x7fffffff, 0x00020000);
+      const unsigned voff = ((4 * g) * ldc + lrow) * 4u;
+      auto store = [&](bool gelu) __attribute__((always_inline)) {
+#pragma unroll
+        for (int q = 0; q < 12; ++q) {
+          const int j = q >> 2, e = q & 3;
+          float out = sums[q] + bv[j];
+          if (Rp) out += rv[q];
+          if (gelu) out = gelu_erf_f32(out);
+          __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, out), rc, voff + j * 128, e * ldc * 4u, 0);
+        }
+      };
+      if (act == 1) store(true); else store(false);
+      return;
     }
 #pragma unroll
     for (int q = 0; q < 12; ++q) {
-      const int idx = firstIdx + q, j = idx >> 4, r = idx & 15;
-      const float v = sums[q];
+      const int j = q >> 2, r = 4 * grp + (q & 3);
       const unsigned grow = m0 + 8 * (r >> 2) + 4 * g + (r & 3);
       const unsigned gc = gcol0 + 32 * j;
-      // bv is indexed by a wave-uniform j: selects keep it in registers
-      const float b = j == 0 ? bv[0] : j == 1 ? bv[1] : bv[2];
-      float out = v + b;
+      float out = sums[q] + bv[j];
       if (Rp) out += rv[q];
       if (act == 1) out = gelu_erf_f32(out);
       if (grow < M && gc < N) {
-        if (p.lnGamma) {
+        if (toSums) {
           // read back by another workgroup, possibly on another XCD, later in this launch: written through to
           // device scope (the L2 caches of the XCDs do not see each other's plain stores before the launch ends)
           __hip_atomic_store(p.lnSums + (size_t)grow * N + gc, out, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -394,17 +515,24 @@ int launch_wave96(hipStream_t stream, SgemmParams p) {
   constexpr size_t lds = ring > red ? ring : red;
   static_assert(lds <= 160 * 1024, "LDS budget");
   if (!sgemm_detail::set_tiles(p, BM, BN96)) return set_error(TFCC_ROCM_INVALID_ARGUMENT, "sgemm: too many tiles");
-  auto kern = sgemm_wave96_kernel<WGM, KSPLIT, BK, STAGES>;
-  static bool attrSet[16] = {};  // per device: the attribute belongs to the function on one device
+  const bool sameStart = p.batch == 1 || (p.strideA == 0 && p.innerA == 0 && p.strideB == 0 && p.innerB == 0);
+  const bool plain = p.groups ? p.groups <= 3 : sameStart;
+  TFCC_REQUIRE(p.batch < (1u << 30), "sgemm: batch of %u", p.batch);
+  auto kern = plain ? sgemm_wave96_kernel<WGM, KSPLIT, BK, STAGES, true>
+                    : sgemm_wave96_kernel<WGM, KSPLIT, BK, STAGES, false>;
+  static bool attrSet[16][2] = {};  // per device: the attribute belongs to the function on one device
   int dev = 0;
   TFCC_HIP_CHECK(hipGetDevice(&dev));
   TFCC_REQUIRE(dev >= 0 && dev < 16, "device index %d", dev);
-  if (!attrSet[dev]) {
+  if (!attrSet[dev][plain]) {
     TFCC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-    attrSet[dev] = true;
+    attrSet[dev][plain] = true;
   }
-  hipLaunchKernelGGL(kern, dim3(p.chunk * 8), dim3(256), lds, stream, p);
+  const unsigned hotBatch = p.batch | (p.groups ? 1u << 30 : 0u);
+  hipLaunchKernelGGL(kern, dim3(p.chunk * 8), dim3(256), lds, stream, p.A, p.groups ? p.groupB[0] : p.B,
+                     p.groups ? p.groupB[1] : nullptr, p.groups ? p.groupB[2] : nullptr, (unsigned)p.M, (unsigned)p.N,
+                     (unsigned)p.K, (unsigned)p.lda, (unsigned)p.ldb, hotBatch, p);
   return check_launch("sgemm");
 }
 
@@ -421,6 +549,7 @@ int sgemm_wave96_launch(hipStream_t stream, SgemmParams p, int ksplit) {
     if (tiles > 512) return launch_wave96<1, 4, 8, 3>(stream, p);
     return launch_wave96<1, 4, 16, 2>(stream, p);
   }
+  if (ksplit == 1) return launch_wave96<4, 1, 32, 4>(stream, p);
   return set_error(TFCC_ROCM_INVALID_ARGUMENT, "sgemm: no 32 x 96 wavefront kernel for %d K groups", ksplit);
 }
 
