@@ -202,18 +202,6 @@ __device__ static inline int requantize_one_biased_unclamped(unsigned off, const
 __device__ __forceinline__ float ref_max(float a, float b) { return a < b ? b : a; }
 __device__ __forceinline__ float ref_min(float a, float b) { return b < a ? b : a; }
 
-// Wavefronts that share a SIMD and do the same work reach their epilogues together, and the matrix cores idle while
-// all of them store.  Giving them different issue priorities by the wave slot they landed in (hardware id register,
-// bits 3:0) lets the first finish early and store under the others' matrix ops.  Results do not depend on it.
-__device__ __forceinline__ void stagger_by_wave_slot() {
-#ifndef TFCC_NO_STAGGER
-  const unsigned slot = __builtin_amdgcn_s_getreg((3 << 11) | 4);  // 4 bits at offset 0 of HW_ID
-  if (slot == 0) __builtin_amdgcn_s_setprio(3);
-  else if (slot == 1) __builtin_amdgcn_s_setprio(2);
-  else if (slot == 2) __builtin_amdgcn_s_setprio(1);
-#endif
-}
-
 // The value of lane i ^ MASK for the six steps of a butterfly over the 64 lanes, without the LDS crossbar that
 // __shfl_xor goes through: the two halves and the rows of 16 lanes are exchanged by the swap instructions (a and b
 // come back as the two members of the pair, in lane order of the lower one), the steps inside a row are data-parallel

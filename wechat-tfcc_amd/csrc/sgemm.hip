@@ -464,7 +464,7 @@ int dispatch(hipStream_t s, const SgemmParams& p, bool vec, bool tb, unsigned fi
       // 32 x 96 tiles and four K groups: the four groups as the four hand-scheduled wavefronts of one workgroup
       if (kTiles[best].config == 1 && ksplit == 4) return sgemm_detail::sgemm_wave96_launch(s, p, 4);
       // No K groups, and 128 x 96 tiles fill at least 70 % of the CUs in each of their rounds: four hand-scheduled
-      // wavefronts of 32 x 96 share each copy of B (1024 x 3072 x 768 with GELU: 40.0 against 42.4 us in 64 x 64
+      // wavefronts of 32 x 96 share each copy of B (1024 x 3072 x 768 with GELU: 39.3 against 42.4 us in 64 x 64
       // tiles, 1536^3: 69 against 80 us; below that fill, or with a short K, the tiles of the table win).  The sums
       // are the same: one ascending pass over K.
       if (ksplit == 1 && k >= 512) {

@@ -61,7 +61,6 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_dma_kernel(cons
   static_assert(COPIES * STAGES < 64, "vmcnt range");
   static_assert(STAGES >= 2 && KS % 2 == 0, "ring depth; the operand registers alternate per step");
 
-  stagger_by_wave_slot();
   extern __shared__ __align__(16) unsigned char smem[];
   const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int grp = wv / GW, wave = wv - grp * GW;  // wave-uniform

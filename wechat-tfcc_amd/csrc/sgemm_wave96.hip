@@ -19,10 +19,10 @@
 //                                 quarter of the tile.  For products the dispatcher sums in four K groups:
 //                                 1024 x 768 x 3072 36.3 us against 45.9 for the twelve-wavefront kernel of
 //                                 sgemm_dma.hip, three 1024 x 768 x 768 products in one launch 29.5 against 39.9.
-//   rows   (WGM = 4, KSPLIT = 1)  a 128 x 96 tile, wavefront w owns rows 32w..32w+31, the ring (four slabs of 32 k:
+//   rows   (WGM = 4, KSPLIT = 1)  a 128 x 96 tile, wavefront w owns rows 32w..32w+31, the ring (two slabs of 32 k:
 //                                 A 128 x 32 + B 32 x 96) is shared, one barrier per slab.  For products summed in
 //                                 one pass over K whose 128 x 96 tiles fill the CUs: 1024 x 3072 x 768 with GELU
-//                                 40.0 us against 42.4 in 64 x 64 tiles.
+//                                 39.3 us against 42.4 in 64 x 64 tiles.
 // Whole tiles are stored through a buffer descriptor (a lane offset, a scalar per row, an immediate per column
 // block: no address arithmetic or bounds checks per value); edge tiles take the checked path.
 // The arithmetic is that of sgemm_dma.hip instruction for instruction (k pairs (8kb + s, 8kb + 4 + s) in ascending
@@ -77,7 +77,6 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, co
   constexpr int BCH = BN96 / 4;     // 16-byte chunks per B row
   constexpr bool SHARED = WGM > 1;  // the group's wavefronts read each other's copies
 
-  stagger_by_wave_slot();
   extern __shared__ __align__(16) unsigned char smem[];
   const int wv = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int grp = wv / WGM, wm = wv - grp * WGM;  // wave-uniform
@@ -549,7 +548,7 @@ int sgemm_wave96_launch(hipStream_t stream, SgemmParams p, int ksplit) {
     if (tiles > 512) return launch_wave96<1, 4, 8, 3>(stream, p);
     return launch_wave96<1, 4, 16, 2>(stream, p);
   }
-  if (ksplit == 1) return launch_wave96<4, 1, 32, 4>(stream, p);
+  if (ksplit == 1) return launch_wave96<4, 1, 32, 2>(stream, p);
   return set_error(TFCC_ROCM_INVALID_ARGUMENT, "sgemm: no 32 x 96 wavefront kernel for %d K groups", ksplit);
 }
 
