@@ -262,13 +262,15 @@ def cpu_baseline(a, b, size):
     return result
 
 
-def bench_other(torch, pkg, dev, steps, warmup, c3):
+def bench_other(torch, pkg, dev, steps, warmup, c3, short_legs=False):
     """Remaining BASELINE configs; each entry: ms, achieved rate, bound, fraction of the bounding peak."""
     out = {}
     # These launches take microseconds: a handful of them after the host-side set-up of a case measures the clock
     # ramp and the first touch of the rotated buffers, not the kernel.  Whatever --steps / --warmup say, every case
-    # here runs at least 300 untimed and 500 timed launches (the counts used are part of the output).
-    steps, warmup = max(steps, 500), max(warmup, 300)
+    # here runs at least 300 untimed and 500 timed launches (the counts used are part of the output), unless
+    # --short-legs asks for the given counts (counter collection, where every launch is slow).
+    if not short_legs:
+        steps, warmup = max(steps, 500), max(warmup, 300)
     out["launch_counts"] = {"timed": steps, "warmup": warmup}
     rng = np.random.default_rng(1)
     t = lambda x: torch.from_numpy(np.ascontiguousarray(x)).to(dev)
@@ -566,6 +568,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=500)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-other", action="store_true", help="skip the secondary configs")
+    ap.add_argument("--short-legs", action="store_true",
+                    help="secondary configs with the --steps / --warmup given instead of at least 500 / 300 launches "
+                         "(for counter collection; the figures then include the clock ramp)")
     ap.add_argument("--headline-only", action="store_true",
                     help="only the timed launches of the headline kernel (for counter runs): no probes, no settled / "
                          "burst repeats, no secondary configs, no CPU leg")
@@ -674,7 +679,7 @@ def main():
         side = torch.cuda.Stream()
         torch.cuda.synchronize()
         with torch.cuda.stream(side):
-            result["other"] = bench_other(torch, pkg, dev, max(10, args.steps // 2), args.warmup, c3)
+            result["other"] = bench_other(torch, pkg, dev, max(10, args.steps // 2), args.warmup, c3, args.short_legs)
         torch.cuda.synchronize()
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(a, b, size)

@@ -340,7 +340,9 @@ enum {
   TFCC_ROCM_UNARY_SIGN = 8, TFCC_ROCM_UNARY_NEG = 9, TFCC_ROCM_UNARY_RECIPROCAL = 10, TFCC_ROCM_UNARY_SQRT = 11
 };
 int tfcc_rocm_unary_f32(void* stream, int op, const float* in, uint64_t total, float* out);
-/* _MKLActivationKernel::geluAccurate, tfcc/mkl/kernel/tfcc_mklactivationkernel.hpp:213-220 */
+/* _MKLActivationKernel::geluAccurate, tfcc/mkl/kernel/tfcc_mklactivationkernel.hpp:213-220: 0.5 x (1 + erf(x / sqrt 2)).
+ * erf is evaluated through a polynomial fit of log2 erfc (the reference calls the C library's erff): results differ
+ * from the reference's in the last bits, by at most 1e-7 + 1e-6 |x'| of the exact value x'. */
 int tfcc_rocm_gelu_accurate_f32(void* stream, const float* in, uint64_t total, float* out);
 /* out = a * alpha + beta: TransformationInterface::transform, tfcc/core/operations/tfcc_operator.cpp:78-95 */
 int tfcc_rocm_transform_f32(void* stream, const float* in, uint64_t total, float alpha, float beta,
