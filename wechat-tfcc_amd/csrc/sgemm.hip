@@ -309,6 +309,59 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_kernel(const Sg
   const float* __restrict__ R = p.residual ? p.residual + (size_t)bi * p.strideR : nullptr;  // dense, flat batch
   const int act = p.act;
   const unsigned gcol = n0 + wn * WN + NI * lrow;
+  const bool residualByLanes = EARLY_RESIDUAL || !R || (VEC && reinterpret_cast<uintptr_t>(R) % 16 == 0 && N % 4 == 0);
+  if (m0 + wm * WM + WM <= M && n0 + wn * WN + WN <= N && ldc < (1u << 24) && residualByLanes) {
+    // A whole WM x WN block: no bounds to check, and the addresses are a register per lane (row 4g, the lane's first
+    // column), a scalar per row and an immediate per column - no address arithmetic per value.
+    const unsigned blockCol = n0 + wn * WN;
+    const __amdgpu_buffer_rsrc_t rc =
+        __builtin_amdgcn_make_buffer_rsrc(C + (size_t)(m0 + wm * WM) * ldc + blockCol, 0, 0x7fffffff, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rr = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(R ? R + (size_t)(m0 + wm * WM) * N + blockCol : C), 0, 0x7fffffff, 0x00020000);
+    const unsigned voff = ((4 * g) * ldc + NI * lrow) * 4u, voffR = ((4 * g) * N + NI * lrow) * 4u;
+    auto store = [&](bool gelu) __attribute__((always_inline)) {
+#pragma unroll
+      for (int i = 0; i < MI; ++i) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const unsigned rowInBlock = i * 32 + 8 * (r / 4) + (r & 3);
+          float v[NI];
+#pragma unroll
+          for (int j = 0; j < NI; ++j) v[j] = acc[i][j][r] + bv[j];
+          if (R) {
+            if constexpr (EARLY_RESIDUAL) {
+#pragma unroll
+              for (int j = 0; j < NI; ++j) v[j] += rv[i][j][r];
+            } else if constexpr (NI == 4) {
+              const v4f w = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rr, voffR, rowInBlock * N * 4u, 0));
+#pragma unroll
+              for (int j = 0; j < NI; ++j) v[j] += w[j];
+            } else {
+#pragma unroll
+              for (int j = 0; j < NI; ++j)
+                v[j] += __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rr, voffR + j * 4u, rowInBlock * N * 4u, 0));
+            }
+          }
+          if (gelu) {
+#pragma unroll
+            for (int j = 0; j < NI; ++j) v[j] = gelu_erf_f32(v[j]);
+          }
+          if constexpr (NI == 4 && VEC) {
+            typedef unsigned v4u __attribute__((ext_vector_type(4)));
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v4f{v[0], v[1], v[2], v[3]}), rc, voff,
+                                                   rowInBlock * ldc * 4u, 0);
+          } else {
+#pragma unroll
+            for (int j = 0; j < NI; ++j)
+              __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v[j]), rc, voff + j * 4u,
+                                                    rowInBlock * ldc * 4u, 0);
+          }
+        }
+      }
+    };
+    if (act == 1) store(true); else store(false);
+    return;
+  }
   const bool vecOK = VEC && (gcol + NI <= N);
 #pragma unroll
   for (int i = 0; i < MI; ++i) {

@@ -259,9 +259,57 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_dma_kernel(cons
 
   // ---- tile store: + bias, + residual, GELU.  Lane (lrow, g) owns columns NI*lrow .. of the wavefront's
   // block and rows 8*(r/4) + 4*g + r%4.
-  if (gcol >= N) return;
   const float* R = p.residual ? p.residual + (size_t)bi * p.strideR : nullptr;  // dense, flat batch
   const int act = p.act;
+  const bool residualByQuads = EARLY_RESIDUAL || !R || reinterpret_cast<uintptr_t>(R) % 16 == 0;
+  if (m0 + wm * 32 + 32 <= M && n0 + wn * WN + WN <= N && ldc < (1u << 24) && residualByQuads) {
+    // A whole 32 x WN block: no bounds to check, and the addresses are a register per lane (row 4g, the lane's first
+    // column), a scalar per row and an immediate per column - no address arithmetic per value (vector instructions
+    // are what a tile store costs: they do not run under another wavefront's fp32 matrix ops).
+    const unsigned blockCol = n0 + wn * WN;
+    const __amdgpu_buffer_rsrc_t rc =
+        __builtin_amdgcn_make_buffer_rsrc(Cbase + (size_t)(m0 + wm * 32) * ldc + blockCol, 0, 0x7fffffff, 0x00020000);
+    const __amdgpu_buffer_rsrc_t rr = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(R ? R + (size_t)(m0 + wm * 32) * N + blockCol : Cbase), 0, 0x7fffffff, 0x00020000);
+    const unsigned laneCol = STRIDED ? lrow : NI * lrow;
+    const unsigned voff = ((4 * g) * ldc + laneCol) * 4u, voffR = ((4 * g) * N + laneCol) * 4u;
+    auto store = [&](bool gelu) __attribute__((always_inline)) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const unsigned rowInBlock = 8 * (r / 4) + (r & 3);
+        float v[NI];
+#pragma unroll
+        for (int j = 0; j < NI; ++j) v[j] = acc[j][r] + bv[j];
+        if (R) {
+          if constexpr (EARLY_RESIDUAL) {
+#pragma unroll
+            for (int j = 0; j < NI; ++j) v[j] += rv[r * NI + j];
+          } else {
+            const v4f w = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rr, voffR, rowInBlock * N * 4u, 0));
+#pragma unroll
+            for (int j = 0; j < NI; ++j) v[j] += w[j];
+          }
+        }
+        if (gelu) {
+#pragma unroll
+          for (int j = 0; j < NI; ++j) v[j] = gelu_erf_f32(v[j]);
+        }
+        if constexpr (NI == 4) {
+          typedef unsigned v4u __attribute__((ext_vector_type(4)));
+          __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(v4u, v4f{v[0], v[1], v[2], v[3]}), rc, voff,
+                                                 rowInBlock * ldc * 4u, 0);
+        } else {
+#pragma unroll
+          for (int j = 0; j < NI; ++j)
+            __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, v[j]), rc, voff + j * CSTEP * 4u,
+                                                  rowInBlock * ldc * 4u, 0);
+        }
+      }
+    };
+    if (act == 1) store(true); else store(false);
+    return;
+  }
+  if (gcol >= N) return;
   const bool whole = gcol + (NI - 1) * CSTEP < N;
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
