@@ -184,7 +184,7 @@ __global__ __launch_bounds__(kThreads, 4) void attention_kernel(const AttentionP
   // the next product reads
   {
     const unsigned rows = min((unsigned)kRows, S - s0);
-    constexpr int R = 8, W = kThreads / 64;
+    constexpr int R = 8, W = kThreads / 64;  // R is the eight of wave_reduce8
     for (unsigned base = wave; base < rows; base += W * R) {
       float v[R][2], mx[R], sum[R];
 #pragma unroll
@@ -199,29 +199,28 @@ __global__ __launch_bounds__(kThreads, 4) void attention_kernel(const AttentionP
           mx[u] = fmaxf(mx[u], v[u][q]);
         }
       }
-#pragma unroll
-      for (int u = 0; u < R; ++u) mx[u] = wave_max(mx[u]);
+      wave_reduce8<true>(mx, lane);
 #pragma unroll
       for (int u = 0; u < R; ++u) {
         sum[u] = 0.f;
 #pragma unroll
         for (int q = 0; q < 2; ++q) {
           const unsigned i = lane + 64 * q;
-          v[u][q] = i < T ? expf(v[u][q] - mx[u]) : 0.f;
+          v[u][q] = i < T ? softmax_exp(v[u][q] - mx[u]) : 0.f;
           sum[u] += v[u][q];
         }
       }
-#pragma unroll
-      for (int u = 0; u < R; ++u) sum[u] = wave_sum(sum[u]);
+      wave_reduce8<false>(sum, lane);
 #pragma unroll
       for (int u = 0; u < R; ++u) {
         const unsigned row = base + W * u;
         if (row < rows) {
           float* sc = Sc + row * kPitchS;
+          const float inverse = 1.0f / sum[u];  // as the stand-alone softmax: one division per row
 #pragma unroll
           for (int q = 0; q < 2; ++q) {
             const unsigned i = lane + 64 * q;
-            sc[i] = i < T ? v[u][q] / sum[u] : 0.f;
+            sc[i] = i < T ? v[u][q] * inverse : 0.f;
           }
         }
       }

@@ -40,12 +40,13 @@ __global__ __launch_bounds__(256) void softmax_kernel(const float* in, unsigned 
   mx = block_reduce<true>(mx, sh);
   float s = 0.f;
   for (unsigned i = threadIdx.x; i < cols; i += 256) {
-    float e = expf((divide ? a[i] / divisor : a[i]) - mx);
+    float e = softmax_exp((divide ? a[i] / divisor : a[i]) - mx);
     o[i] = e;
     s += e;
   }
   s = block_reduce<false>(s, sh);
-  for (unsigned i = threadIdx.x; i < cols; i += 256) o[i] = o[i] / s;
+  const float inverse = 1.0f / s;  // one division per row, a multiplication per value
+  for (unsigned i = threadIdx.x; i < cols; i += 256) o[i] = o[i] * inverse;
 }
 
 // rows of at most 256 columns: one wavefront per row, values stay in registers
@@ -69,14 +70,15 @@ __global__ __launch_bounds__(256) void softmax_small_kernel(const float* in, siz
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
     unsigned i = lane + 64 * q;
-    v[q] = i < cols ? expf(v[q] - mx) : 0.f;
+    v[q] = i < cols ? softmax_exp(v[q] - mx) : 0.f;
     s += v[q];
   }
   s = wave_sum(s);
+  const float inverse = 1.0f / s;  // one division per row, a multiplication per value
 #pragma unroll
   for (int q = 0; q < 4; ++q) {
     unsigned i = lane + 64 * q;
-    if (i < cols) o[i] = v[q] / s;
+    if (i < cols) o[i] = v[q] * inverse;
   }
 }
 
