@@ -174,3 +174,36 @@ def test_sgemm_on_32x96_tiles_with_four_k_groups(pkg, T, m, n, k):
     grouped = pkg.sgemm_grouped(ta, bs, [tbias, tbias, tbias])
     for g, bb in zip(grouped, bs):
         assert np.array_equal(T.n(g), T.n(pkg.blas_matmul(ta, bb, tbias)))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("m,n,k,batch", [
+    # products summed in one pass over K whose 128 x 96 tiles fill the CUs: four hand-scheduled wavefronts of 32 x 96 on
+    # a shared ring.  Whole tiles; ragged last row band and column block; 192 tiles (three quarters of the CUs); the
+    # shortest K it takes; an odd number of 32-k slabs (the unrolled loop leaves one over); two batch entries with
+    # their own operands (the kernel variant that reads the batch strides before its first copies)
+    (1024, 3072, 768, 1), (1000, 3000, 768, 1), (1536, 1536, 1536, 1), (1024, 3072, 512, 1), (1024, 3072, 544, 1),
+    (512, 3072, 768, 2),
+])
+def test_sgemm_on_128x96_workgroups(pkg, T, m, n, k, batch):
+    """The same bits as the register-staged kernel (reached through a transposed B: also one pass over K), the fused
+    bias + residual + GELU equal to the separate kernels, float64 within the fp32 tolerance."""
+    import torch
+    print("sgemm 128x96 workgroups", m, n, k, batch, flush=True)
+    rng = np.random.default_rng(m * 7 + n * 3 + k + batch)
+    a = rng.normal(0, 1, (batch, m, k)).astype(np.float32)
+    b = rng.normal(0, 1, (batch, k, n)).astype(np.float32)
+    bias = rng.uniform(-1, 1, n).astype(np.float32)
+    res = rng.normal(0, 1, (batch, m, n)).astype(np.float32)
+    ta, tb, tbias, tres = T.t(a), T.t(b), T.t(bias), T.t(res)
+    plain = T.n(pkg.blas_matmul(ta, tb))
+    assert rel_fro(plain, a.astype(np.float64) @ b.astype(np.float64)) <= FP32_TOL
+    c = torch.empty((batch, m, n), dtype=torch.float32, device=ta.device)
+    bt = T.t(np.ascontiguousarray(np.swapaxes(b, 1, 2)))
+    pkg.sgemm_general(ta, bt, c, m, n, k, k, k, n, trans_b=True, batch_outer=batch, strides=(m * k, n * k, m * n))
+    assert np.array_equal(T.n(c), plain)
+    out = torch.empty((batch, m, n), dtype=torch.float32, device=ta.device)
+    pkg.check(pkg.lib().tfcc_rocm_sgemm_fused(None, ta.data_ptr(), m * k, tb.data_ptr(), k * n, tbias.data_ptr(),
+                                              tres.data_ptr(), m * n, out.data_ptr(), m * n, m, n, k, batch, 1))
+    separate = T.n(pkg.gelu_accurate(pkg.add(pkg.blas_matmul(ta, tb, tbias), tres)))
+    assert np.array_equal(T.n(out), separate)
