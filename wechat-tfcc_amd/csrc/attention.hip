@@ -229,8 +229,7 @@ __global__ __launch_bounds__(kThreads, 4) void attention_kernel(const AttentionP
   __syncthreads();
 
   // ---- probabilities x V: the first four wavefronts, (wm, wn) owning rows 32*wm.. and columns 32*wn.. of the
-  // 64 x D result (one accumulator per element over all of T, as in a product of its own); operands are
-  // fetched from LDS for eight steps at a time
+  // 64 x D result (one accumulator per element over all of T, as in a product of its own)
   const int wm = wave >> 1, wn = wave & 1;
   if (wave < 4 && (unsigned)(32 * wn) < D) {
     constexpr int KB = kMaxT / 8, HALF = KB / 2;
@@ -240,7 +239,7 @@ __global__ __launch_bounds__(kThreads, 4) void attention_kernel(const AttentionP
     const float* pa = Sc + (32 * wm + lrow) * kPitchS + 4 * g;
     const float* vb = KVs + (4 * g) * kPitchV + 32 * wn + lrow;
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
+    for (int h = 0; h < 2; ++h) {  // operands are fetched from LDS for eight steps at a time
       v4f af[HALF], bf[HALF];
 #pragma unroll
       for (int q = 0; q < HALF; ++q) {
@@ -262,7 +261,18 @@ __global__ __launch_bounds__(kThreads, 4) void attention_kernel(const AttentionP
       }
     }
     const unsigned col = 32 * wn + lrow;
-    if (col < D) {
+    if (s0 + 32 * wm + 32 <= S && 32u * wn + 32 <= D && p.ldo < (1u << 24)) {
+      // a whole 32 x 32 block: a register per lane (row 4g, column lrow), a scalar per row, no checks
+      const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(
+          O + (size_t)(s0 + 32 * wm) * p.ldo + 32 * wn, 0, 0x7fffffff, 0x00020000);
+      const unsigned voff = ((4 * g) * p.ldo + lrow) * 4u;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float value = acc[r];  // a copy: __builtin_bit_cast applied to a vector element reads element 0
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, value), ro, voff,
+                                              (8 * (r / 4) + (r & 3)) * p.ldo * 4u, 0);
+      }
+    } else if (col < D) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const unsigned row = s0 + 32 * wm + 8 * (r / 4) + 4 * g + (r & 3);
