@@ -810,6 +810,33 @@ def test_lstm_step_in_one_launch(pkg, T, seq, batch, length, hidden):
                                                     dbias.data_ptr(), 0.0, c.data_ptr(), out.data_ptr(), c.data_ptr()))
 
 
+def test_gelu_and_softmax_at_the_edges_of_their_ranges(pkg, T):
+    """GELU goes through a fit of erfc and softmax through the hardware's exp2 where the reference calls erff / exp:
+    the oracle's values at the ends of the ranges, where an approximation would go wrong first."""
+    x = np.array([0.0, -0.0, 1e-40, -1e-40, 1e-10, -1e-10, 0.5, -0.5, 1.0, -1.0, 3.0, -3.0, 5.5, -5.5, 7.0, -7.0, 7.1, -7.1,
+                  10.0, -10.0, 14.0, -14.0, 100.0, -100.0, 1e30, -1e30, 3e38, -3e38, np.inf, -np.inf, np.nan],
+                 dtype=np.float32)
+    x = np.concatenate([x, np.linspace(-8, 8, 4001, dtype=np.float32)])
+    got, want = T.n(pkg.gelu_accurate(T.t(x))), O.gelu_accurate(x)
+    assert np.array_equal(np.isnan(got), np.isnan(want))
+    ok = ~np.isnan(want)
+    assert np.array_equal(np.signbit(got[ok]), np.signbit(want[ok]))
+    assert np.allclose(got[ok], want[ok], rtol=1e-6, atol=1e-7)
+    rows = np.stack([
+        np.linspace(-200, 0, 128), np.linspace(0, 88, 128), np.full(128, -3e38), np.full(128, 3e38),
+        np.concatenate([np.full(64, -np.inf), np.linspace(-5, 5, 64)]), np.full(128, -np.inf),
+        np.concatenate([[np.nan], np.zeros(127)]), np.concatenate([[0.0], np.full(127, -104.5)]),
+    ]).astype(np.float32)
+    for cols in (128, 100, 300, 1500):  # one wavefront per row with the row in registers; a workgroup per long row
+        r = np.ascontiguousarray(np.resize(rows, (rows.shape[0], cols))) if cols != 128 else rows
+        with np.errstate(invalid="ignore", over="ignore"):
+            want = O.softmax(r)
+        got = T.n(pkg.softmax(T.t(r)))
+        assert np.array_equal(np.isnan(got), np.isnan(want)), cols
+        ok = ~np.isnan(want)
+        assert np.allclose(got[ok], want[ok], rtol=2e-6, atol=1e-8), cols
+
+
 def test_elementwise_against_oracle(pkg, T):
     rng = np.random.default_rng(50)
     for shape in ((8, 12, 128, 128), (7, 33), (5, 1000)):
