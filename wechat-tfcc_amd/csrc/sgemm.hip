@@ -496,7 +496,9 @@ int dispatch(hipStream_t s, const SgemmParams& p, bool vec, bool tb, unsigned fi
   // 128x128 tiles once there are enough of them to fill the 256 CUs twice over, else 64x64
   const unsigned long long big = (unsigned long long)((m + 127) / 128) * ((n + 127) / 128) * fillBatch;
   if (vec) {
-    if (big >= 512) return k % 32 == 0 ? sgemm_detail::sgemm_dma_launch(s, p, 4, 1, false) : launch<4, 1, 1, 4, true>(s, p);
+    // (whole slabs of K: four hand-scheduled wavefronts of 32 x 128 on a shared ring, two workgroups per CU -
+    // 4096^3: 150 TFLOP/s against 141 for the same tiles scheduled by the compiler)
+    if (big >= 512) return k % 32 == 0 ? sgemm_detail::sgemm_wave96_launch(s, p, 1, 4) : launch<4, 1, 1, 4, true>(s, p);
     // few 64x64 tiles and a long K: several K groups per workgroup keep the CUs that have a tile busy
     const unsigned long long small = (unsigned long long)((m + 63) / 64) * ((n + 63) / 64) * fillBatch;
     // 32x96 tiles when they cover the 256 CUs in fewer tile-area rounds than 64x64 tiles would
@@ -516,6 +518,10 @@ int dispatch(hipStream_t s, const SgemmParams& p, bool vec, bool tb, unsigned fi
       // the sums are those of the 32 x 96 tiles.
       // 32 x 96 tiles and four K groups: the four groups as the four hand-scheduled wavefronts of one workgroup
       if (kTiles[best].config == 1 && ksplit == 4) return sgemm_detail::sgemm_wave96_launch(s, p, 4);
+      // ... and the same kernel with two column blocks or one per wavefront for 32 x 64 and 32 x 32 tiles
+      // (128 x 768 x 3072: 8.6 against 11.4 us with the operands in cache, 512^3: 5.0 against 6.0)
+      if (ksplit == 4 && (kTiles[best].config == 2 || kTiles[best].config == 3))
+        return sgemm_detail::sgemm_wave96_launch(s, p, 4, kTiles[best].config == 2 ? 2 : 1);
       // No K groups, and 128 x 96 tiles fill at least 70 % of the CUs in each of their rounds: four hand-scheduled
       // wavefronts of 32 x 96 share each copy of B (1024 x 3072 x 768 with GELU: 39.3 against 42.4 us in 64 x 64
       // tiles, 1536^3: 69 against 80 us; below that fill, or with a short K, the tiles of the table win).  The sums

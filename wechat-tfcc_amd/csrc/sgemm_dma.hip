@@ -373,7 +373,7 @@ int launch(hipStream_t stream, SgemmParams p) {
 namespace sgemm_detail {
 
 bool sgemm_dma_available(int config, int ksplit) {
-  return (config >= 0 && config <= 3 && (ksplit == 1 || ksplit == 2 || ksplit == 4)) || (config == 4 && ksplit == 1) ||
+  return (config >= 0 && config <= 3 && (ksplit == 1 || ksplit == 2 || ksplit == 4)) ||
          (config == 5 && (ksplit == 2 || ksplit == 4));
 }
 
@@ -393,7 +393,6 @@ int sgemm_dma_launch(hipStream_t stream, SgemmParams p, int config, int ksplit, 
   TFCC_DMA_CASE(2, 1, 2)  // 32 x 64
   TFCC_DMA_CASE(3, 1, 1)  // 32 x 32
 #undef TFCC_DMA_CASE
-  if (config == 4 && ksplit == 1) return launch<4, 1, 4, 1, 2>(stream, p);  // 128 x 128: four wavefronts of 32 x 128
   // 128 x 96, twelve wavefronts, one group doing the work of `ksplit` groups: four times the rows of A per copy of B
   if (config == 5 && ksplit == 4 && serialGroups) return launch<4, 3, 1, 1, 2, 4>(stream, p);
   if (config == 5 && ksplit == 2 && serialGroups) return launch<4, 3, 1, 1, 2, 2>(stream, p);

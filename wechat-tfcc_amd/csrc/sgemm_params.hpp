@@ -46,17 +46,19 @@ inline bool set_tiles(SgemmParams& p, unsigned bm, unsigned bn) {
   return true;
 }
 
-// The direct-to-LDS kernels (sgemm_dma.hip).  `config`: 0 = 64x64 tiles, 1 = 32x96, 2 = 32x64, 3 = 32x32, 4 = 128x128
-// (ksplit 1 only), 5 = 128x96 (serial groups only); ksplit 1, 2 or 4 groups of wavefronts on one tile.
+// The direct-to-LDS kernels (sgemm_dma.hip).  `config`: 0 = 64x64 tiles, 1 = 32x96, 2 = 32x64, 3 = 32x32,
+// 5 = 128x96 (serial groups only); ksplit 1, 2 or 4 groups of wavefronts on one tile.
 // Requires 16-byte aligned operands and strides, K a multiple of 32 and B not transposed.
 bool sgemm_dma_available(int config, int ksplit);
 // serialGroups: one group of wavefronts per tile does the work of the `ksplit` groups one slab after the other
 // (same additions, same result) - for launches that fill the chip anyway.
 int sgemm_dma_launch(hipStream_t stream, SgemmParams p, int config, int ksplit, bool serialGroups);
 
-// 32 x 96 tiles with the four K groups of ksplit = 4 as the four wavefronts of a workgroup, hand-scheduled
-// (sgemm_wave96.hip).  Same requirements and the same bits as the kernels above for four K groups.
-int sgemm_wave96_launch(hipStream_t stream, SgemmParams p, int ksplit);
+// The hand-scheduled kernels with one wavefront per SIMD (sgemm_wave96.hip), a wavefront owning 32 rows x `blocks`
+// column blocks of 32: ksplit = 4 - tiles of 32 x 32 blocks with the four K groups as the four wavefronts of a
+// workgroup (blocks 1, 2 or 3); ksplit = 1 - tiles of 128 x 32 blocks, four wavefronts on a shared ring (blocks 3 or
+// 4).  Same requirements and the same bits as the kernels above for the same number of K groups.
+int sgemm_wave96_launch(hipStream_t stream, SgemmParams p, int ksplit, int blocks = 3);
 constexpr unsigned kLayerNormMaxColumns = 1024;  // a lane of the normalising wavefront holds 16 values of a row
 
 // The streaming kernel for up to eight rows of A (sgemv.hip): any K, N, strides and alignment; B not transposed.

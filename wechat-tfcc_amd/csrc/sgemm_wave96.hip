@@ -43,15 +43,13 @@ namespace {
 
 using sgemm_detail::SgemmParams;
 
-constexpr int BN96 = 96;
-
 // 16-byte chunk c of A row `row` lies at chunk c ^ swizzle: rows of 128 bytes (32 k), 64 bytes (16 k), 32 bytes (8 k)
 template <int BK>
 __device__ __forceinline__ int a_row_swizzle(int row) {
   return BK == 32 ? (row >> 1) & 7 : BK == 16 ? (row >> 2) & 3 : (row >> 2) & 1;
 }
 
-template <int WGM, int KSPLIT, int BK, int STAGES, bool PLAIN>
+template <int WGM, int KSPLIT, int BK, int STAGES, bool PLAIN, int NI>
 __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, const float* hotB, const float* hotB1,
                                                            const float* hotB2, unsigned hotM, unsigned hotN,
                                                            unsigned hotK, unsigned hotLda, unsigned hotLdb,
@@ -62,19 +60,21 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, co
   // either its B at hotB too or the launch is the grouped form with at most three products: hotB, hotB1, hotB2 are
   // their B).  hotBatch: p.batch, bit 30 set for the grouped form.
   static_assert(WGM * KSPLIT == 4, "four wavefronts");
+  static_assert(NI >= 1 && NI <= 4, "one to four column blocks of 32 per wavefront");
+  constexpr int BN = 32 * NI;       // columns of a tile
   static_assert(BK == 32 || BK == 16 || BK == 8, "ring slabs of 32, 16 or 8 k");
   static_assert(STAGES >= 2, "ring depth");
   constexpr int BM = 32 * WGM;
   constexpr int KS = BK / 8;        // k steps per ring slab
   constexpr int CH = BK / 4;        // 16-byte chunks per A row
   constexpr int SUB = 32 / BK;      // ring slabs per 32-k slab of the product
-  constexpr int A_BYTES = BM * BK * 4, B_BYTES = BK * BN96 * 4, STAGE_BYTES = A_BYTES + B_BYTES;
+  constexpr int A_BYTES = BM * BK * 4, B_BYTES = BK * BN * 4, STAGE_BYTES = A_BYTES + B_BYTES;
   constexpr int A_UNITS = A_BYTES / 1024, UNITS = STAGE_BYTES / 1024;  // 1 KB copies per ring slab
   static_assert(UNITS % WGM == 0, "every wavefront of a group issues the same number of copies");
   constexpr int COPIES = UNITS / WGM;
-  static_assert(COPIES <= 11 && COPIES * STAGES < 64, "copies fit the slots of one step and the vmcnt range");
+  static_assert(COPIES <= 4 * NI - 1 && COPIES * STAGES < 64, "copies fit the slots of one step and the vmcnt range");
   constexpr int GROUP_BYTES = STAGES * STAGE_BYTES;
-  constexpr int BCH = BN96 / 4;     // 16-byte chunks per B row
+  constexpr int BCH = BN / 4;     // 16-byte chunks per B row
   constexpr bool SHARED = WGM > 1;  // the group's wavefronts read each other's copies
 
   extern __shared__ __align__(16) unsigned char smem[];
@@ -89,7 +89,7 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, co
     // consecutive workgroup ids land on different XCDs: hand each XCD a contiguous run of tiles
     const unsigned wg = blockIdx.x;
     const unsigned xcd = wg & 7u, slot = wg >> 3;
-    const unsigned tilesM = (hotM + BM - 1) / BM, tilesN = (hotN + BN96 - 1) / BN96;
+    const unsigned tilesM = (hotM + BM - 1) / BM, tilesN = (hotN + BN - 1) / BN;
     const unsigned perBatch = tilesM * tilesN;
     const unsigned tilesTotal = perBatch * (hotBatch & 0x3fffffffu);  // the launcher checks that this fits
     const unsigned chunk = (tilesTotal + 7u) / 8u;
@@ -104,7 +104,7 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, co
     tm = gb * 4u + r % rowsInBand;
     tn = r / rowsInBand;
   }
-  const unsigned m0 = tm * BM, n0 = tn * BN96;
+  const unsigned m0 = tm * BM, n0 = tn * BN;
   const unsigned M = hotM, N = hotN, K = hotK;
   const bool grouped = (hotBatch >> 30) & 1u;
   const float* A = hotA;
@@ -184,13 +184,13 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, co
   // column block j, row 8*(r/4) + 4*g + r%4 of its wavefront's 32 and column 32*j + lrow.  Groups: after the
   // partial tiles met in LDS, wavefront w finishes registers 4w .. 4w+3 of each column block (rows 8w + 4g + e):
   // value q = 4j + e of its twelve is register 4w + e of block j.
-  constexpr int OWN = KSPLIT == 1 ? 48 : 12;
+  constexpr int OWN = KSPLIT == 1 ? 16 * NI : 4 * NI;
   auto ownBlock = [&](int q) { return KSPLIT == 1 ? q >> 4 : q >> 2; };
   auto ownRegister = [&](int q) { return KSPLIT == 1 ? q & 15 : 4 * grp + (q & 3); };
   const unsigned gcol0 = n0 + lrow;
-  float bv[3];
+  float bv[NI];
 #pragma unroll
-  for (int j = 0; j < 3; ++j) bv[j] = (biasPtr && gcol0 + 32 * j < N) ? biasPtr[gcol0 + 32 * j] : 0.f;
+  for (int j = 0; j < NI; ++j) bv[j] = (biasPtr && gcol0 + 32 * j < N) ? biasPtr[gcol0 + 32 * j] : 0.f;
   float rv[OWN];
   const float* Rp = p.residual ? p.residual + (size_t)biL * p.strideR : nullptr;  // dense, flat batch
   if (Rp) {
@@ -203,9 +203,9 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, co
     }
   }
 
-  w96_v16f acc[3];
+  w96_v16f acc[NI];
 #pragma unroll
-  for (int j = 0; j < 3; ++j)
+  for (int j = 0; j < NI; ++j)
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[j][r] = 0.f;
 
@@ -213,8 +213,8 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, co
   // k rows 8*kb + 4*g + s
   const int arow = wm * 32 + lrow;
   const int aBase = arow * (BK * 4), aSwz = a_row_swizzle<BK>(arow);
-  const int bBase = A_BYTES + (4 * g) * (BN96 * 4) + lrow * 4;
-  struct Ops { w96_v4f a; float b[4][3]; };
+  const int bBase = A_BYTES + (4 * g) * (BN * 4) + lrow * 4;
+  struct Ops { w96_v4f a; float b[4][NI]; };
   // In the unrolled part of the loop the stage is a constant, and every LDS address is one of a few registers set up
   // here plus an immediate: no address arithmetic between the matrix ops.  The B operands of a step are then read two
   // per instruction (two offsets of up to 255 words from one register: a register per stage, k step and half step).
@@ -230,7 +230,7 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, co
     for (int st = 0; st < (PAIRED ? STAGES : 1); ++st)
 #pragma unroll
       for (int h = 0; h < 2; ++h) {
-        bAddr[st][kb][h] = ldsGroup + st * STAGE_BYTES + bBase + (8 * kb + 2 * h) * (BN96 * 4);
+        bAddr[st][kb][h] = ldsGroup + st * STAGE_BYTES + bBase + (8 * kb + 2 * h) * (BN * 4);
         asm volatile("" : "+v"(bAddr[st][kb][h]));
       }
   }
@@ -242,24 +242,24 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, co
                   unsigned dmaStage) __attribute__((always_inline)) {
     const unsigned char* st = gsm + ldStage * STAGE_BYTES;
 #pragma unroll
-    for (int m = 0; m < 12; ++m) {
-      const int s = m / 3, j = m % 3;
+    for (int m = 0; m < 4 * NI; ++m) {
+      const int s = m / NI, j = m % NI;
       if (fixedStage) {
         if (m == 0) nxt.a = *reinterpret_cast<LdsQuads>(aAddr[ldKb] + ldStage * STAGE_BYTES);
         if (PAIRED) {
-          if (m & 1) {  // values 2 * (m / 2) and 2 * (m / 2) + 1 of the twelve, three to a k row
+          if (m & 1) {  // values 2 * (m / 2) and 2 * (m / 2) + 1 of the step's 4 NI, NI to a k row
 #pragma unroll
             for (int e = 0; e < 2; ++e) {
-              const int v = (m / 2) * 2 + e, vs = v / 3, vj = v % 3;
-              nxt.b[vs][vj] = reinterpret_cast<LdsFloats>(bAddr[PAIRED ? ldStage : 0][ldKb][vs / 2])[(vs & 1) * BN96 + vj * 32];
+              const int v = (m / 2) * 2 + e, vs = v / NI, vj = v % NI;
+              nxt.b[vs][vj] = reinterpret_cast<LdsFloats>(bAddr[PAIRED ? ldStage : 0][ldKb][vs / 2])[(vs & 1) * BN + vj * 32];
             }
           }
         } else {
-          nxt.b[s][j] = reinterpret_cast<LdsFloats>(bAddr[0][ldKb][0] + ldStage * STAGE_BYTES)[s * BN96 + j * 32];
+          nxt.b[s][j] = reinterpret_cast<LdsFloats>(bAddr[0][ldKb][0] + ldStage * STAGE_BYTES)[s * BN + j * 32];
         }
       } else {
         if (m == 0) nxt.a = *reinterpret_cast<const w96_v4f*>(st + aBase + (((2 * ldKb + g) ^ aSwz) << 4));
-        nxt.b[s][j] = *reinterpret_cast<const float*>(st + bBase + (8 * ldKb + s) * (BN96 * 4) + j * 128);
+        nxt.b[s][j] = *reinterpret_cast<const float*>(st + bBase + (8 * ldKb + s) * (BN * 4) + j * 128);
       }
       if (dma && m >= 1 && m <= COPIES) issueCopy(dmaSlab, dmaStage, m - 1);
       acc[j] = __builtin_amdgcn_mfma_f32_32x32x2f32(cur.a[s], cur.b[s][j], acc[j], 0, 0, 0);
@@ -278,7 +278,7 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, co
 #pragma unroll
   for (int s = 0; s < 4; ++s)
 #pragma unroll
-    for (int j = 0; j < 3; ++j) ops[0].b[s][j] = *reinterpret_cast<const float*>(gsm + bBase + s * (BN96 * 4) + j * 128);
+    for (int j = 0; j < NI; ++j) ops[0].b[s][j] = *reinterpret_cast<const float*>(gsm + bBase + s * (BN * 4) + j * 128);
   // one ring slab in stage `stage`: KS steps starting on the operands in `first`; the next slab's first operands end
   // up in `first` again when KS is even, in `other` when it is odd (then the loops below alternate the two)
   auto slab = [&](unsigned t, unsigned stage, bool fixedStage, Ops& first, Ops& other) __attribute__((always_inline)) {
@@ -325,7 +325,7 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, co
     return v;
   };
   if constexpr (KSPLIT == 1) {
-    if (m0 + wm * 32 + 32 <= M && n0 + BN96 <= N && ldc < (1u << 24)) {
+    if (m0 + wm * 32 + 32 <= M && n0 + BN <= N && ldc < (1u << 24)) {
       // A whole tile: no bounds to check, and the addresses are a register per lane (row 4g, column lrow), a scalar
       // per row and an immediate per column block.
       const __amdgpu_buffer_rsrc_t rc =
@@ -335,7 +335,7 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, co
 #pragma unroll
         for (int r = 0; r < 16; ++r)
 #pragma unroll
-          for (int j = 0; j < 3; ++j) {
+          for (int j = 0; j < NI; ++j) {
             float out = acc[j][r] + bv[j];
             if (Rp) out += rv[j * 16 + r];
             if (gelu) out = gelu_erf_f32(out);
@@ -347,7 +347,7 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, co
       return;
     }
 #pragma unroll
-    for (int j = 0; j < 3; ++j) {
+    for (int j = 0; j < NI; ++j) {
       const unsigned gc = gcol0 + 32 * j;
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
@@ -357,22 +357,22 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, co
     }
   } else {
     // the four partial tiles go through LDS (the rings are idle now), four registers per 128-bit access: registers
-    // 4c .. 4c+3 of column block j of group q lie at red4[(q * 12 + 4 * j + c) * 64 + lane]; wavefront w adds quad
+    // 4c .. 4c+3 of column block j of group q lie at red4[(q * 4 * NI + 4 * j + c) * 64 + lane]; wavefront w adds quad
     // c = w of every block in group order
     w96_v4f* red4 = reinterpret_cast<w96_v4f*>(smem);
 #pragma unroll
-    for (int j = 0; j < 3; ++j)
+    for (int j = 0; j < NI; ++j)
 #pragma unroll
       for (int c = 0; c < 4; ++c)
-        red4[(grp * 12 + j * 4 + c) * 64 + lane] = w96_v4f{acc[j][4 * c], acc[j][4 * c + 1], acc[j][4 * c + 2], acc[j][4 * c + 3]};
+        red4[(grp * 4 * NI + j * 4 + c) * 64 + lane] = w96_v4f{acc[j][4 * c], acc[j][4 * c + 1], acc[j][4 * c + 2], acc[j][4 * c + 3]};
     __syncthreads();
-    float sums[12];
+    float sums[4 * NI];
 #pragma unroll
-    for (int j = 0; j < 3; ++j) {
+    for (int j = 0; j < NI; ++j) {
       w96_v4f v = red4[(4 * j + grp) * 64 + lane];
 #pragma unroll
       for (int o = 1; o < KSPLIT; ++o) {
-        const w96_v4f w = red4[(o * 12 + 4 * j + grp) * 64 + lane];
+        const w96_v4f w = red4[(o * 4 * NI + 4 * j + grp) * 64 + lane];
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] += w[e];
       }
@@ -380,7 +380,7 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, co
       for (int e = 0; e < 4; ++e) sums[4 * j + e] = v[e];
     }
     const bool toSums = p.lnGamma != nullptr;
-    if (m0 + 32 <= M && n0 + BN96 <= N && ldc < (1u << 24) && !toSums) {
+    if (m0 + 32 <= M && n0 + BN <= N && ldc < (1u << 24) && !toSums) {
       // A whole tile: no bounds to check, and the addresses are a register per lane (row 4g, column lrow of the
       // wavefront's eight rows), a scalar per row and an immediate per column block.
       const __amdgpu_buffer_rsrc_t rc =
@@ -388,7 +388,7 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, co
       const unsigned voff = ((4 * g) * ldc + lrow) * 4u;
       auto store = [&](bool gelu) __attribute__((always_inline)) {
 #pragma unroll
-        for (int q = 0; q < 12; ++q) {
+        for (int q = 0; q < 4 * NI; ++q) {
           const int j = q >> 2, e = q & 3;
           float out = sums[q] + bv[j];
           if (Rp) out += rv[q];
@@ -400,7 +400,7 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, co
       return;
     }
 #pragma unroll
-    for (int q = 0; q < 12; ++q) {
+    for (int q = 0; q < 4 * NI; ++q) {
       const int j = q >> 2, r = 4 * grp + (q & 3);
       const unsigned grow = m0 + 8 * (r >> 2) + 4 * g + (r & 3);
       const unsigned gc = gcol0 + 32 * j;
@@ -506,19 +506,19 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, co
   }
 }
 
-template <int WGM, int KSPLIT, int BK, int STAGES>
+template <int WGM, int KSPLIT, int BK, int STAGES, int NI = 3>
 int launch_wave96(hipStream_t stream, SgemmParams p) {
-  constexpr int BM = 32 * WGM;
-  constexpr size_t ring = (size_t)KSPLIT * STAGES * (BM + BN96) * BK * 4;
-  constexpr size_t red = KSPLIT > 1 ? (size_t)KSPLIT * 48 * 64 * 4 : 0;
+  constexpr int BM = 32 * WGM, BN = 32 * NI;
+  constexpr size_t ring = (size_t)KSPLIT * STAGES * (BM + BN) * BK * 4;
+  constexpr size_t red = KSPLIT > 1 ? (size_t)KSPLIT * 16 * NI * 64 * 4 : 0;
   constexpr size_t lds = ring > red ? ring : red;
   static_assert(lds <= 160 * 1024, "LDS budget");
-  if (!sgemm_detail::set_tiles(p, BM, BN96)) return set_error(TFCC_ROCM_INVALID_ARGUMENT, "sgemm: too many tiles");
+  if (!sgemm_detail::set_tiles(p, BM, BN)) return set_error(TFCC_ROCM_INVALID_ARGUMENT, "sgemm: too many tiles");
   const bool sameStart = p.batch == 1 || (p.strideA == 0 && p.innerA == 0 && p.strideB == 0 && p.innerB == 0);
   const bool plain = p.groups ? p.groups <= 3 : sameStart;
   TFCC_REQUIRE(p.batch < (1u << 30), "sgemm: batch of %u", p.batch);
-  auto kern = plain ? sgemm_wave96_kernel<WGM, KSPLIT, BK, STAGES, true>
-                    : sgemm_wave96_kernel<WGM, KSPLIT, BK, STAGES, false>;
+  auto kern = plain ? sgemm_wave96_kernel<WGM, KSPLIT, BK, STAGES, true, NI>
+                    : sgemm_wave96_kernel<WGM, KSPLIT, BK, STAGES, false, NI>;
   static bool attrSet[16][2] = {};  // per device: the attribute belongs to the function on one device
   int dev = 0;
   TFCC_HIP_CHECK(hipGetDevice(&dev));
@@ -539,17 +539,20 @@ int launch_wave96(hipStream_t stream, SgemmParams p) {
 
 namespace sgemm_detail {
 
-int sgemm_wave96_launch(hipStream_t stream, SgemmParams p, int ksplit) {
+int sgemm_wave96_launch(hipStream_t stream, SgemmParams p, int ksplit, int blocks) {
   if (ksplit == 4) {
-    // Three or more tiles per CU: rings of three slabs of 8 k (12 KB per wavefront) let three workgroups share a CU,
-    // so that all of a CU's tiles overlap (three 1024 x 768 x 768 products in one launch: 33.9 us -> see below).
-    // Fewer: two slabs of 16 k, which leave a slab's copies twice the time to land.
-    const unsigned long long tiles = (unsigned long long)((p.M + 31) / 32) * ((p.N + BN96 - 1) / BN96) * p.batch;
-    if (tiles > 512) return launch_wave96<1, 4, 8, 3>(stream, p);
-    return launch_wave96<1, 4, 16, 2>(stream, p);
+    // Three or more tiles per CU: rings of three slabs of 8 k (12 KB per wavefront with 96 columns) let three
+    // workgroups share a CU, so that all of a CU's tiles overlap.  Fewer: two slabs of 16 k, which leave a slab's
+    // copies twice the time to land.  (With 32 columns a slab of 16 k would be more copies than a step has slots.)
+    const unsigned long long tiles =
+        (unsigned long long)((p.M + 31) / 32) * ((p.N + 32 * blocks - 1) / (32 * blocks)) * p.batch;
+    if (blocks == 3) return tiles > 512 ? launch_wave96<1, 4, 8, 3, 3>(stream, p) : launch_wave96<1, 4, 16, 2, 3>(stream, p);
+    if (blocks == 2) return tiles > 512 ? launch_wave96<1, 4, 8, 3, 2>(stream, p) : launch_wave96<1, 4, 16, 2, 2>(stream, p);
+    if (blocks == 1) return launch_wave96<1, 4, 8, 3, 1>(stream, p);
   }
-  if (ksplit == 1) return launch_wave96<4, 1, 32, 2>(stream, p);
-  return set_error(TFCC_ROCM_INVALID_ARGUMENT, "sgemm: no 32 x 96 wavefront kernel for %d K groups", ksplit);
+  if (ksplit == 1 && blocks == 3) return launch_wave96<4, 1, 32, 2, 3>(stream, p);
+  if (ksplit == 1 && blocks == 4) return launch_wave96<4, 1, 32, 2, 4>(stream, p);
+  return set_error(TFCC_ROCM_INVALID_ARGUMENT, "sgemm: no wavefront kernel for %d K groups and %d column blocks", ksplit, blocks);
 }
 
 }  // namespace sgemm_detail
