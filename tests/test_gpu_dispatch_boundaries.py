@@ -207,3 +207,34 @@ def test_sgemm_on_128x96_workgroups(pkg, T, m, n, k, batch):
                                               tres.data_ptr(), m * n, out.data_ptr(), m * n, m, n, k, batch, 1))
     separate = T.n(pkg.gelu_accurate(pkg.add(pkg.blas_matmul(ta, tb, tbias), tres)))
     assert np.array_equal(T.n(out), separate)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("m,n,k", [
+    # the same hand-scheduled kernel with other numbers of 32-column blocks per wavefront: 32 x 64 tiles and four K
+    # groups (the first BASELINE config; ragged), 32 x 32 tiles and four K groups (whole and ragged), 128 x 128 tiles
+    # for products of 512 tiles and more (whole; ragged rows and columns; a single 32-k slab)
+    (128, 3072, 768), (100, 3000, 800), (512, 512, 512), (500, 500, 544), (2048, 4096, 256), (2050, 4100, 320),
+    (4096, 2048, 32),
+])
+def test_sgemm_wavefront_kernel_with_one_two_and_four_column_blocks(pkg, T, m, n, k):
+    """The same bits as the register-staged kernel (reached through a transposed B, summed with the same K groups), the
+    fused bias + residual + GELU equal to the separate kernels, float64 within the fp32 tolerance."""
+    import torch
+    print("sgemm wavefront kernel, other block counts", m, n, k, flush=True)
+    rng = np.random.default_rng(m * 11 + n * 3 + k)
+    a = rng.normal(0, 1, (m, k)).astype(np.float32)
+    b = rng.normal(0, 1, (k, n)).astype(np.float32)
+    bias = rng.uniform(-1, 1, n).astype(np.float32)
+    res = rng.normal(0, 1, (m, n)).astype(np.float32)
+    ta, tb, tbias, tres = T.t(a), T.t(b), T.t(bias), T.t(res)
+    plain = T.n(pkg.blas_matmul(ta, tb))
+    assert rel_fro(plain, a.astype(np.float64) @ b.astype(np.float64)) <= FP32_TOL
+    c = torch.empty((m, n), dtype=torch.float32, device=ta.device)
+    pkg.sgemm_general(ta, T.t(np.ascontiguousarray(b.T)), c, m, n, k, k, k, n, trans_b=True)
+    assert np.array_equal(T.n(c), plain)
+    out = torch.empty((m, n), dtype=torch.float32, device=ta.device)
+    pkg.check(pkg.lib().tfcc_rocm_sgemm_fused(None, ta.data_ptr(), 0, tb.data_ptr(), 0, tbias.data_ptr(),
+                                              tres.data_ptr(), 0, out.data_ptr(), 0, m, n, k, 1, 1))
+    separate = T.n(pkg.gelu_accurate(pkg.add(pkg.blas_matmul(ta, tb, tbias), tres)))
+    assert np.array_equal(T.n(out), separate)
