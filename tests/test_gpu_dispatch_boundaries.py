@@ -216,6 +216,9 @@ def test_sgemm_on_128x96_workgroups(pkg, T, m, n, k, batch):
     # for products of 512 tiles and more (whole; ragged rows and columns; a single 32-k slab)
     (128, 3072, 768), (100, 3000, 800), (512, 512, 512), (500, 500, 544), (2048, 4096, 256), (2050, 4100, 320),
     (4096, 2048, 32),
+    # two K groups: two pairs of wavefronts on 64 x 64 tiles (whole; ragged, an odd number of 32-k slabs), two
+    # wavefronts on 32 x 32 tiles
+    (1024, 1024, 1024), (1000, 1000, 992), (400, 400, 256), (1111, 996, 320),
 ])
 def test_sgemm_wavefront_kernel_with_one_two_and_four_column_blocks(pkg, T, m, n, k):
     """The same bits as the register-staged kernel (reached through a transposed B, summed with the same K groups), the

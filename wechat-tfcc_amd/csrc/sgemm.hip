@@ -526,6 +526,11 @@ int dispatch(hipStream_t s, const SgemmParams& p, bool vec, bool tb, unsigned fi
       // wavefronts of 32 x 96 share each copy of B (1024 x 3072 x 768 with GELU: 39.3 against 42.4 us in 64 x 64
       // tiles, 1536^3: 69 against 80 us; below that fill, or with a short K, the tiles of the table win).  The sums
       // are the same: one ascending pass over K.
+      // Two K groups: two pairs of wavefronts on a 64 x 64 tile, two wavefronts on a 32 x 32 tile (1024^3: 20.1
+      // against 24.2 us, 400 x 400 x 256: 5.3 against 7.3; on 32 x 96 and 32 x 64 tiles the table's kernels are as
+      // fast or faster and keep the product)
+      if (ksplit == 2 && kTiles[best].config == 0) return sgemm_detail::sgemm_wave96_launch(s, p, 2, 2, 2);
+      if (ksplit == 2 && kTiles[best].config == 3) return sgemm_detail::sgemm_wave96_launch(s, p, 2, 1, 1);
       if (ksplit == 1 && k >= 512) {
         const unsigned long long wide = (unsigned long long)((m + 127) / 128) * ((n + 95) / 96) * fillBatch;
         if (wide * 100 >= 70 * 256 * ((wide + 255) / 256)) return sgemm_detail::sgemm_wave96_launch(s, p, 1);

@@ -20,6 +20,8 @@
 //                                 quarter of the tile.  For products the dispatcher sums in four K groups:
 //                                 1024 x 768 x 3072 36.3 us against 45.9 for the twelve-wavefront kernel of
 //                                 sgemm_dma.hip, three 1024 x 768 x 768 products in one launch 29.5 against 39.9.
+//   (WGM = 2, KSPLIT = 2 and WGM = 1, KSPLIT = 2: the same with two K groups - two pairs of wavefronts on a 64 x 64
+//   tile, each pair sharing its ring, or two wavefronts on a 32 x 32 tile; a wavefront finishes two quarters.)
 //   rows   (WGM = 4, KSPLIT = 1)  a 128 x 96 tile, wavefront w owns rows 32w..32w+31, the ring (two slabs of 32 k:
 //                                 A 128 x 32 + B 32 x 96) is shared, one barrier per slab.  For products summed in
 //                                 one pass over K whose 128 x 96 tiles fill the CUs: 1024 x 3072 x 768 with GELU
@@ -63,7 +65,8 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, co
   // is looked at before the first slabs are on their way when PLAIN (every batch entry's A starts at hotA, and
   // either its B at hotB too or the launch is the grouped form with at most three products: hotB, hotB1, hotB2 are
   // their B).  hotBatch: p.batch, bit 30 set for the grouped form.
-  static_assert(WGM * KSPLIT == 4, "four wavefronts");
+  static_assert(WGM * KSPLIT == 4 || WGM * KSPLIT == 2, "four wavefronts (one per SIMD), or two");
+  static_assert(KSPLIT == 1 || KSPLIT == 2 || KSPLIT == 4, "the quads of a column block divide among the K groups");
   static_assert(NI >= 1 && NI <= 4, "one to four column blocks of 32 per wavefront");
   constexpr int BN = 32 * NI;       // columns of a tile
   static_assert(BK == 32 || BK == 16 || BK == 8, "ring slabs of 32, 16 or 8 k");
@@ -188,9 +191,11 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, co
   // column block j, row 8*(r/4) + 4*g + r%4 of its wavefront's 32 and column 32*j + lrow.  Groups: after the
   // partial tiles met in LDS, wavefront w finishes registers 4w .. 4w+3 of each column block (rows 8w + 4g + e):
   // value q = 4j + e of its twelve is register 4w + e of block j.
-  constexpr int OWN = KSPLIT == 1 ? 16 * NI : 4 * NI;
-  auto ownBlock = [&](int q) { return KSPLIT == 1 ? q >> 4 : q >> 2; };
-  auto ownRegister = [&](int q) { return KSPLIT == 1 ? q & 15 : 4 * grp + (q & 3); };
+  constexpr int QPW = 4 / KSPLIT;   // quads of four registers of each column block that a wavefront finishes
+  constexpr int OWN = 4 * QPW * NI; // values a lane finishes: value q is register 4 (grp QPW + q / 4 % QPW) + q % 4 of
+                                    // block q / (4 QPW)
+  auto ownBlock = [&](int q) { return q / (4 * QPW); };
+  auto ownRegister = [&](int q) { return 4 * ((KSPLIT == 1 ? 0 : grp * QPW) + (q >> 2) % QPW) + (q & 3); };
   const unsigned gcol0 = n0 + lrow;
   float bv[NI];
 #pragma unroll
@@ -360,53 +365,60 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, co
       }
     }
   } else {
-    // the four partial tiles go through LDS (the rings are idle now), four registers per 128-bit access: registers
-    // 4c .. 4c+3 of column block j of group q lie at red4[(q * 4 * NI + 4 * j + c) * 64 + lane]; wavefront w adds quad
-    // c = w of every block in group order
+    // the partial tiles of the K groups go through LDS (the rings are idle now), four registers per 128-bit access:
+    // registers 4c .. 4c+3 of column block j of the wavefront (group q, rows wm) lie at
+    // red4[(((q * WGM + wm) * NI + j) * 4 + c) * 64 + lane]; wavefront (grp, wm) adds the quads c = grp QPW .. of every
+    // block in group order
     w96_v4f* red4 = reinterpret_cast<w96_v4f*>(smem);
 #pragma unroll
     for (int j = 0; j < NI; ++j)
 #pragma unroll
       for (int c = 0; c < 4; ++c)
-        red4[(grp * 4 * NI + j * 4 + c) * 64 + lane] = w96_v4f{acc[j][4 * c], acc[j][4 * c + 1], acc[j][4 * c + 2], acc[j][4 * c + 3]};
+        red4[(((grp * WGM + wm) * NI + j) * 4 + c) * 64 + lane] =
+            w96_v4f{acc[j][4 * c], acc[j][4 * c + 1], acc[j][4 * c + 2], acc[j][4 * c + 3]};
     __syncthreads();
-    float sums[4 * NI];
+    float sums[OWN];
 #pragma unroll
-    for (int j = 0; j < NI; ++j) {
-      w96_v4f v = red4[(4 * j + grp) * 64 + lane];
+    for (int j = 0; j < NI; ++j)
 #pragma unroll
-      for (int o = 1; o < KSPLIT; ++o) {
-        const w96_v4f w = red4[(o * 4 * NI + 4 * j + grp) * 64 + lane];
+      for (int cq = 0; cq < QPW; ++cq) {
+        const int c = grp * QPW + cq;
+        w96_v4f v = red4[((wm * NI + j) * 4 + c) * 64 + lane];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] += w[e];
+        for (int o = 1; o < KSPLIT; ++o) {
+          const w96_v4f w = red4[(((o * WGM + wm) * NI + j) * 4 + c) * 64 + lane];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] += w[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) sums[(j * QPW + cq) * 4 + e] = v[e];
       }
-#pragma unroll
-      for (int e = 0; e < 4; ++e) sums[4 * j + e] = v[e];
-    }
-    const bool toSums = p.lnGamma != nullptr;
-    if (m0 + 32 <= M && n0 + BN <= N && ldc < (1u << 24) && !toSums) {
+    bool toSums = false;
+    if constexpr (WGM == 1 && KSPLIT == 4) toSums = p.lnGamma != nullptr;
+    if (m0 + wm * 32 + 32 <= M && n0 + BN <= N && ldc < (1u << 24) && !toSums) {
       // A whole tile: no bounds to check, and the addresses are a register per lane (row 4g, column lrow of the
-      // wavefront's eight rows), a scalar per row and an immediate per column block.
-      const __amdgpu_buffer_rsrc_t rc =
-          __builtin_amdgcn_make_buffer_rsrc(Cbase + (size_t)(m0 + 8 * grp) * ldc + n0, 0, 0x7fffffff, 0x00020000);
+      // wavefront's 8 QPW rows), a scalar per row and an immediate per column block.
+      const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc(
+          Cbase + (size_t)(m0 + wm * 32 + 8 * grp * QPW) * ldc + n0, 0, 0x7fffffff, 0x00020000);
       const unsigned voff = ((4 * g) * ldc + lrow) * 4u;
       auto store = [&](bool gelu) __attribute__((always_inline)) {
 #pragma unroll
-        for (int q = 0; q < 4 * NI; ++q) {
-          const int j = q >> 2, e = q & 3;
+        for (int q = 0; q < OWN; ++q) {
+          const int j = q / (4 * QPW), cq = (q >> 2) % QPW, e = q & 3;
           float out = sums[q] + bv[j];
           if (Rp) out += rv[q];
           if (gelu) out = gelu_erf_f32(out);
-          __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, out), rc, voff + j * 128, e * ldc * 4u, 0);
+          __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, out), rc, voff + j * 128,
+                                                (8 * cq + e) * ldc * 4u, 0);
         }
       };
       if (act == 1) store(true); else store(false);
       return;
     }
 #pragma unroll
-    for (int q = 0; q < 4 * NI; ++q) {
-      const int j = q >> 2, r = 4 * grp + (q & 3);
-      const unsigned grow = m0 + 8 * (r >> 2) + 4 * g + (r & 3);
+    for (int q = 0; q < OWN; ++q) {
+      const int j = ownBlock(q), r = ownRegister(q);
+      const unsigned grow = m0 + wm * 32 + 8 * (r >> 2) + 4 * g + (r & 3);
       const unsigned gc = gcol0 + 32 * j;
       float out = sums[q] + bv[j];
       if (Rp) out += rv[q];
@@ -421,7 +433,7 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, co
         }
       }
     }
-    if (p.lnGamma) {
+    if constexpr (WGM == 1 && KSPLIT == 4) if (p.lnGamma) {
       // ---- layer normalisation of the band's 32 rows by whichever of its workgroups stores its tile last.
       // Every store above has been acknowledged at device scope before this wavefront reaches the barrier, and
       // the band's counter is incremented after the barrier: the workgroup that reads tilesN - 1 from it sees all
@@ -514,7 +526,7 @@ template <int WGM, int KSPLIT, int BK, int STAGES, int NI = 3>
 int launch_wave96(hipStream_t stream, SgemmParams p) {
   constexpr int BM = 32 * WGM, BN = 32 * NI;
   constexpr size_t ring = (size_t)KSPLIT * STAGES * (BM + BN) * BK * 4;
-  constexpr size_t red = KSPLIT > 1 ? (size_t)KSPLIT * 16 * NI * 64 * 4 : 0;
+  constexpr size_t red = KSPLIT > 1 ? (size_t)KSPLIT * WGM * 16 * NI * 64 * 4 : 0;
   constexpr size_t lds = ring > red ? ring : red;
   static_assert(lds <= 160 * 1024, "LDS budget");
   if (!sgemm_detail::set_tiles(p, BM, BN)) return set_error(TFCC_ROCM_INVALID_ARGUMENT, "sgemm: too many tiles");
@@ -533,7 +545,7 @@ int launch_wave96(hipStream_t stream, SgemmParams p) {
     attrSet[dev][plain] = true;
   }
   const unsigned hotBatch = p.batch | (p.groups ? 1u << 30 : 0u);
-  hipLaunchKernelGGL(kern, dim3(p.chunk * 8), dim3(256), lds, stream, p.A, p.groups ? p.groupB[0] : p.B,
+  hipLaunchKernelGGL(kern, dim3(p.chunk * 8), dim3(64 * WGM * KSPLIT), lds, stream, p.A, p.groups ? p.groupB[0] : p.B,
                      p.groups ? p.groupB[1] : nullptr, p.groups ? p.groupB[2] : nullptr, (unsigned)p.M, (unsigned)p.N,
                      (unsigned)p.K, (unsigned)p.lda, (unsigned)p.ldb, hotBatch, p);
   return check_launch("sgemm");
@@ -543,7 +555,14 @@ int launch_wave96(hipStream_t stream, SgemmParams p) {
 
 namespace sgemm_detail {
 
-int sgemm_wave96_launch(hipStream_t stream, SgemmParams p, int ksplit, int blocks) {
+int sgemm_wave96_launch(hipStream_t stream, SgemmParams p, int ksplit, int blocks, int rowBlocks) {
+  if (ksplit == 2) {
+    // two K groups: two wavefronts on a 32-row tile, or two pairs of wavefronts on a 64 x 64 tile
+    if (rowBlocks == 2 && blocks == 2) return launch_wave96<2, 2, 16, 2, 2>(stream, p);
+    if (rowBlocks == 1 && blocks == 1) return launch_wave96<1, 2, 8, 3, 1>(stream, p);
+  }
+  if (rowBlocks != 0 && rowBlocks != (ksplit == 1 ? 4 : 1))
+    return set_error(TFCC_ROCM_INVALID_ARGUMENT, "sgemm: no wavefront kernel for %d K groups and %d row blocks", ksplit, rowBlocks);
   if (ksplit == 4) {
     // Three or more tiles per CU: rings of three slabs of 8 k (12 KB per wavefront with 96 columns) let three
     // workgroups share a CU, so that all of a CU's tiles overlap.  Fewer: two slabs of 16 k, which leave a slab's
