@@ -394,7 +394,7 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, co
         for (int e = 0; e < 4; ++e) sums[(j * QPW + cq) * 4 + e] = v[e];
       }
     bool toSums = false;
-    if constexpr (WGM == 1 && KSPLIT == 4) toSums = p.lnGamma != nullptr;
+    if constexpr (WGM == 1 && KSPLIT == 4 && NI == 3) toSums = p.lnGamma != nullptr;
     if (m0 + wm * 32 + 32 <= M && n0 + BN <= N && ldc < (1u << 24) && !toSums) {
       // A whole tile: no bounds to check, and the addresses are a register per lane (row 4g, column lrow of the
       // wavefront's 8 QPW rows), a scalar per row and an immediate per column block.
@@ -433,7 +433,7 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, co
         }
       }
     }
-    if constexpr (WGM == 1 && KSPLIT == 4) if (p.lnGamma) {
+    if constexpr (WGM == 1 && KSPLIT == 4 && NI == 3) if (p.lnGamma) {
       // ---- layer normalisation of the band's 32 rows by whichever of its workgroups stores its tile last.
       // Every store above has been acknowledged at device scope before this wavefront reaches the barrier, and
       // the band's counter is incremented after the barrier: the workgroup that reads tilesN - 1 from it sees all
