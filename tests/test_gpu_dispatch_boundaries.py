@@ -221,6 +221,8 @@ def test_sgemm_on_128x96_workgroups(pkg, T, m, n, k, batch):
     (1024, 1024, 1024), (1000, 1000, 992), (400, 400, 256), (1111, 996, 320),
     # 128 x 128 workgroups below 512 tiles, where they fill the CUs and 128 x 96 tiles do not
     (2048, 2048, 512), (1920, 2040, 544),
+    # 64 x 64 tiles with four K groups: four pairs of wavefronts
+    (960, 1024, 2048), (1270, 636, 544),
 ])
 def test_sgemm_wavefront_kernel_with_one_two_and_four_column_blocks(pkg, T, m, n, k):
     """The same bits as the register-staged kernel (reached through a transposed B, summed with the same K groups), the

@@ -522,6 +522,13 @@ int dispatch(hipStream_t s, const SgemmParams& p, bool vec, bool tb, unsigned fi
       // (128 x 768 x 3072: 8.6 against 11.4 us with the operands in cache, 512^3: 5.0 against 6.0)
       if (ksplit == 4 && (kTiles[best].config == 2 || kTiles[best].config == 3))
         return sgemm_detail::sgemm_wave96_launch(s, p, 4, kTiles[best].config == 2 ? 2 : 1);
+      // Two K groups: two pairs of wavefronts on a 64 x 64 tile, two wavefronts on a 32 x 32 tile (1024^3: 20.1
+      // against 24.2 us, 400 x 400 x 256: 5.3 against 7.3; on 32 x 96 and 32 x 64 tiles the table's kernels are as
+      // fast or faster and keep the product)
+      // (and four pairs with four K groups, two wavefronts per SIMD: 960 x 1024 x 2048 34.4 against 41.9 us)
+      if (ksplit == 4 && kTiles[best].config == 0) return sgemm_detail::sgemm_wave96_launch(s, p, 4, 2, 2);
+      if (ksplit == 2 && kTiles[best].config == 0) return sgemm_detail::sgemm_wave96_launch(s, p, 2, 2, 2);
+      if (ksplit == 2 && kTiles[best].config == 3) return sgemm_detail::sgemm_wave96_launch(s, p, 2, 1, 1);
       // No K groups, and 128 x 96 tiles fill at least 70 % of the CUs in each of their rounds (or 128 x 128 tiles
       // 85 %): four hand-scheduled wavefronts of 32 x 96 (32 x 128) share each copy of B (1024 x 3072 x 768 with GELU:
       // 39.3 against 42.4 us in 64 x 64 tiles, 1536^3: 69 against 80 us, 2048^3 in 128 x 128 tiles: 120 against 136;

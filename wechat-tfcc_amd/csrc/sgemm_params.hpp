@@ -56,7 +56,7 @@ int sgemm_dma_launch(hipStream_t stream, SgemmParams p, int config, int ksplit, 
 
 // The hand-scheduled kernels with one wavefront per SIMD (sgemm_wave96.hip), a wavefront owning 32 rows x `blocks`
 // column blocks of 32: ksplit = 4 - tiles of 32 x 32 blocks with the four K groups as the four wavefronts of a
-// workgroup (blocks 1, 2 or 3); ksplit = 2 - 64 x 64 tiles (blocks 2, rowBlocks 2: two pairs of wavefronts) or 32 x 32
+// workgroup (blocks 1, 2 or 3), or 64 x 64 tiles with eight wavefronts (blocks 2, rowBlocks 2); ksplit = 2 - 64 x 64 tiles (blocks 2, rowBlocks 2: two pairs of wavefronts) or 32 x 32
 // (blocks 1, rowBlocks 1: two wavefronts); ksplit = 1 - tiles of 128 x 32 blocks, four wavefronts on a shared ring
 // (blocks 3 or 4).  Same requirements and the same bits as the kernels above for the same number of K groups.
 int sgemm_wave96_launch(hipStream_t stream, SgemmParams p, int ksplit, int blocks = 3, int rowBlocks = 0);

@@ -56,7 +56,7 @@ __device__ __forceinline__ int a_row_swizzle(int row) {
 }
 
 template <int WGM, int KSPLIT, int BK, int STAGES, bool PLAIN, int NI>
-__global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, const float* hotB, const float* hotB1,
+__global__ __launch_bounds__(64 * WGM * KSPLIT > 256 ? 64 * WGM * KSPLIT : 256) void sgemm_wave96_kernel(const float* hotA, const float* hotB, const float* hotB1,
                                                            const float* hotB2, unsigned hotM, unsigned hotN,
                                                            unsigned hotK, unsigned hotLda, unsigned hotLdb,
                                                            unsigned hotBatch, const SgemmParams p) {
@@ -65,7 +65,7 @@ __global__ __launch_bounds__(256) void sgemm_wave96_kernel(const float* hotA, co
   // is looked at before the first slabs are on their way when PLAIN (every batch entry's A starts at hotA, and
   // either its B at hotB too or the launch is the grouped form with at most three products: hotB, hotB1, hotB2 are
   // their B).  hotBatch: p.batch, bit 30 set for the grouped form.
-  static_assert(WGM * KSPLIT == 4 || WGM * KSPLIT == 2, "four wavefronts (one per SIMD), or two");
+  static_assert(WGM * KSPLIT == 4 || WGM * KSPLIT == 2 || WGM * KSPLIT == 8, "four wavefronts (one per SIMD), two, or eight");
   static_assert(KSPLIT == 1 || KSPLIT == 2 || KSPLIT == 4, "the quads of a column block divide among the K groups");
   static_assert(NI >= 1 && NI <= 4, "one to four column blocks of 32 per wavefront");
   constexpr int BN = 32 * NI;       // columns of a tile
@@ -556,6 +556,7 @@ int launch_wave96(hipStream_t stream, SgemmParams p) {
 namespace sgemm_detail {
 
 int sgemm_wave96_launch(hipStream_t stream, SgemmParams p, int ksplit, int blocks, int rowBlocks) {
+  if (ksplit == 4 && rowBlocks == 2 && blocks == 2) return launch_wave96<2, 4, 16, 2, 2>(stream, p);  // 64 x 64, eight wavefronts
   if (ksplit == 2) {
     // two K groups: two wavefronts on a 32-row tile, or two pairs of wavefronts on a 64 x 64 tile
     if (rowBlocks == 2 && blocks == 2) return launch_wave96<2, 2, 16, 2, 2>(stream, p);
