@@ -509,31 +509,25 @@ int dispatch(hipStream_t s, const SgemmParams& p, bool vec, bool tb, unsigned fi
       int best, ksplit;
       unsigned long long bestTiles;
       choose_dma_tiles(m, n, k, fillBatch, best, bestTiles, ksplit);
-      // Several products in one launch (p.batch counts them; fillBatch = 1 chose the configuration of a single
-      // one so that each is summed exactly as on its own): when they fill the chip without the K groups, one
-      // group per tile plays all of them.
-      const bool serial = ksplit > 1 && bestTiles * (p.batch / fillBatch) * kTiles[best].waves >= 256ull * 8;
-      // ... and when 128 x 96 tiles over all of them still occupy most of the CUs in one round, twelve wavefronts
-      // share each copy of B among four times the rows (44.1 against 46.8 us for three 1024 x 768 x 768 products);
-      // the sums are those of the 32 x 96 tiles.
-      // 32 x 96 tiles and four K groups: the four groups as the four hand-scheduled wavefronts of one workgroup
-      if (kTiles[best].config == 1 && ksplit == 4) return sgemm_detail::sgemm_wave96_launch(s, p, 4);
-      // ... and the same kernel with two column blocks or one per wavefront for 32 x 64 and 32 x 32 tiles
-      // (128 x 768 x 3072: 8.6 against 11.4 us with the operands in cache, 512^3: 5.0 against 6.0)
-      if (ksplit == 4 && (kTiles[best].config == 2 || kTiles[best].config == 3))
-        return sgemm_detail::sgemm_wave96_launch(s, p, 4, kTiles[best].config == 2 ? 2 : 1);
-      // Two K groups: two pairs of wavefronts on a 64 x 64 tile, two wavefronts on a 32 x 32 tile (1024^3: 20.1
-      // against 24.2 us, 400 x 400 x 256: 5.3 against 7.3; on 32 x 96 and 32 x 64 tiles the table's kernels are as
-      // fast or faster and keep the product)
-      // (and four pairs with four K groups, two wavefronts per SIMD: 960 x 1024 x 2048 34.4 against 41.9 us)
-      if (ksplit == 4 && kTiles[best].config == 0) return sgemm_detail::sgemm_wave96_launch(s, p, 4, 2, 2);
+      // The hand-scheduled kernel of sgemm_wave96.hip (one wavefront per SIMD, no vector instruction between its
+      // matrix ops) takes every product with four K groups - the groups as the four wavefronts of a workgroup on
+      // 32 x 96, 32 x 64 and 32 x 32 tiles, four pairs of wavefronts on 64 x 64 tiles (1024 x 768 x 3072: 36.3
+      // against 45.9 us for the kernels of sgemm_dma.hip, 128 x 768 x 3072: 8.6 against 11.4 with the operands in
+      // cache, 960 x 1024 x 2048: 34.4 against 41.9) ...
+      if (ksplit == 4) {
+        const int c = kTiles[best].config;
+        return sgemm_detail::sgemm_wave96_launch(s, p, 4, c == 0 ? 2 : c == 1 ? 3 : c == 2 ? 2 : 1, c == 0 ? 2 : 1);
+      }
+      // ... with two K groups the 64 x 64 tiles (two pairs of wavefronts) and the 32 x 32 tiles (two wavefronts):
+      // 1024^3 20.1 against 24.2 us, 400 x 400 x 256 5.3 against 7.3; on 32 x 96 and 32 x 64 tiles the kernels of
+      // sgemm_dma.hip are as fast or faster and keep the product ...
       if (ksplit == 2 && kTiles[best].config == 0) return sgemm_detail::sgemm_wave96_launch(s, p, 2, 2, 2);
       if (ksplit == 2 && kTiles[best].config == 3) return sgemm_detail::sgemm_wave96_launch(s, p, 2, 1, 1);
-      // No K groups, and 128 x 96 tiles fill at least 70 % of the CUs in each of their rounds (or 128 x 128 tiles
-      // 85 %): four hand-scheduled wavefronts of 32 x 96 (32 x 128) share each copy of B (1024 x 3072 x 768 with GELU:
-      // 39.3 against 42.4 us in 64 x 64 tiles, 1536^3: 69 against 80 us, 2048^3 in 128 x 128 tiles: 120 against 136;
-      // below those fills, or with a short K, the tiles of the table win).  The sums are the same: one ascending pass
-      // over K.
+      // ... and without K groups the products whose 128 x 96 tiles fill at least 70 % of the CUs in each of their
+      // rounds (or 128 x 128 tiles 85 %), K >= 512: four wavefronts of 32 x 96 (32 x 128) share each copy of B
+      // (1024 x 3072 x 768 with GELU: 39.3 against 42.4 us in 64 x 64 tiles, 1536^3: 69 against 80, 2048^3 in
+      // 128 x 128 tiles: 120 against 136; below those fills, or with a short K, the tiles of the table win).  The
+      // sums are the same in every case: the K groups of the table, ascending k inside a group.
       if (ksplit == 1 && k >= 512) {
         const unsigned long long wide = (unsigned long long)((m + 127) / 128) * ((n + 95) / 96) * fillBatch;
         const unsigned long long wide4 = (unsigned long long)((m + 127) / 128) * ((n + 127) / 128) * fillBatch;
@@ -542,6 +536,12 @@ int dispatch(hipStream_t s, const SgemmParams& p, bool vec, bool tb, unsigned fi
         if (ok4 && (!ok3 || cost4 < cost3)) return sgemm_detail::sgemm_wave96_launch(s, p, 1, 4);
         if (ok3) return sgemm_detail::sgemm_wave96_launch(s, p, 1);
       }
+      // What is left runs on the kernels of sgemm_dma.hip.  Several products in one launch (p.batch counts them;
+      // fillBatch = 1 chose the configuration of a single one so that each is summed exactly as on its own): when
+      // they fill the chip without the K groups, one group per tile plays all of them; and when 128 x 96 tiles over
+      // all of them still occupy most of the CUs in one round, twelve wavefronts share each copy of B among four
+      // times the rows (the sums are those of the 32 x 96 tiles).
+      const bool serial = ksplit > 1 && bestTiles * (p.batch / fillBatch) * kTiles[best].waves >= 256ull * 8;
       if (serial && kTiles[best].config == 1) {
         const unsigned long long wide = (unsigned long long)((m + 127) / 128) * ((n + 95) / 96) * p.batch;
         if (wide <= 256 && wide >= 160) return sgemm_detail::sgemm_dma_launch(s, p, 5, ksplit, true);

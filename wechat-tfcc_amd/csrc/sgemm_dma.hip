@@ -373,8 +373,7 @@ int launch(hipStream_t stream, SgemmParams p) {
 namespace sgemm_detail {
 
 bool sgemm_dma_available(int config, int ksplit) {
-  return (config >= 0 && config <= 3 && (ksplit == 1 || ksplit == 2 || ksplit == 4)) ||
-         (config == 5 && (ksplit == 2 || ksplit == 4));
+  return (config >= 0 && config <= 3 && (ksplit == 1 || ksplit == 2)) || (config == 5 && ksplit == 2);
 }
 
 // Two stages everywhere: more workgroups per CU beat a deeper ring (measured 42.3 against 43.9 us with
@@ -384,9 +383,7 @@ int sgemm_dma_launch(hipStream_t stream, SgemmParams p, int config, int ksplit, 
   if (config == C) {                                                                \
     if (ksplit == 1) return launch<WGM, WGN, 1, 1, 2>(stream, p);                      \
     if (ksplit == 2 && serialGroups) return launch<WGM, WGN, 1, 1, 2, 2>(stream, p);   \
-    if (ksplit == 4 && serialGroups) return launch<WGM, WGN, 1, 1, 2, 4>(stream, p);   \
     if (ksplit == 2) return launch<WGM, WGN, 1, 2, 2>(stream, p);                      \
-    if (ksplit == 4) return launch<WGM, WGN, 1, 4, 2>(stream, p);                      \
   }
   TFCC_DMA_CASE(0, 2, 2)  // 64 x 64
   TFCC_DMA_CASE(1, 1, 3)  // 32 x 96
@@ -394,7 +391,6 @@ int sgemm_dma_launch(hipStream_t stream, SgemmParams p, int config, int ksplit, 
   TFCC_DMA_CASE(3, 1, 1)  // 32 x 32
 #undef TFCC_DMA_CASE
   // 128 x 96, twelve wavefronts, one group doing the work of `ksplit` groups: four times the rows of A per copy of B
-  if (config == 5 && ksplit == 4 && serialGroups) return launch<4, 3, 1, 1, 2, 4>(stream, p);
   if (config == 5 && ksplit == 2 && serialGroups) return launch<4, 3, 1, 1, 2, 2>(stream, p);
   return set_error(TFCC_ROCM_INVALID_ARGUMENT, "sgemm: no direct-to-LDS kernel for this configuration");
 }

@@ -47,7 +47,8 @@ inline bool set_tiles(SgemmParams& p, unsigned bm, unsigned bn) {
 }
 
 // The direct-to-LDS kernels (sgemm_dma.hip).  `config`: 0 = 64x64 tiles, 1 = 32x96, 2 = 32x64, 3 = 32x32,
-// 5 = 128x96 (serial groups only); ksplit 1, 2 or 4 groups of wavefronts on one tile.
+// 5 = 128x96 (serial groups only); ksplit 1 or 2 groups of wavefronts on one tile (four K groups run on the
+// kernels of sgemm_wave96.hip).
 // Requires 16-byte aligned operands and strides, K a multiple of 32 and B not transposed.
 bool sgemm_dma_available(int config, int ksplit);
 // serialGroups: one group of wavefronts per tile does the work of the `ksplit` groups one slab after the other
