@@ -12,23 +12,23 @@
 // that every LDS address is a register set up before the loop plus an immediate.  Measured in the loop: 64.3-65.5
 // cycles per matrix op.
 //
-// Two shapes of workgroup, four wavefronts each:
-//   groups (WGM = 1, KSPLIT = 4)  a 32 x 96 tile, wavefront q sums the 32-k slabs q, q + 4, ... in a ring of its
+// Shapes of workgroup (WGM row blocks of 32 x KSPLIT K groups wavefronts, NI column blocks of 32 per wavefront):
+//   groups (WGM = 1, KSPLIT = 4)  a 32 x 32 NI tile, wavefront q sums the 32-k slabs q, q + 4, ... in a ring of its
 //                                 own (two half slabs of 16 k, or three of 8 k when three workgroups share a CU, so
 //                                 that one's set-up and tile store run under the others' matrix ops; no barrier
 //                                 in the loop); the four partial tiles meet in LDS and every wavefront finishes a
 //                                 quarter of the tile.  For products the dispatcher sums in four K groups:
 //                                 1024 x 768 x 3072 36.3 us against 45.9 for the twelve-wavefront kernel of
-//                                 sgemm_dma.hip, three 1024 x 768 x 768 products in one launch 29.5 against 39.9.
-//   (WGM = 2, KSPLIT = 2 and WGM = 1, KSPLIT = 2: the same with two K groups - two pairs of wavefronts on a 64 x 64
-//   tile, each pair sharing its ring, or two wavefronts on a 32 x 32 tile; a wavefront finishes two quarters.)
-//   rows   (WGM = 4, KSPLIT = 1)  a 128 x 96 tile, wavefront w owns rows 32w..32w+31, the ring (two slabs of 32 k:
-//                                 A 128 x 32 + B 32 x 96) is shared, one barrier per slab.  For products summed in
-//                                 one pass over K whose 128 x 96 tiles fill the CUs: 1024 x 3072 x 768 with GELU
-//                                 39.3 us against 42.4 in 64 x 64 tiles.
-// NI = 2 and NI = 1 give the groups shape the table's 32 x 64 and 32 x 32 tiles (128 x 768 x 3072: 8.6 against 11.4 us
-// with the operands in cache), NI = 4 gives the rows shape 128 x 128 tiles for products of 512 tiles and more
-// (4096^3: 150 against 141 TFLOP/s).
+//                                 sgemm_dma.hip, three 1024 x 768 x 768 products in one launch 29.5 against 39.9;
+//                                 with NI = 2 and NI = 1 the 32 x 64 and 32 x 32 tiles (128 x 768 x 3072: 8.6
+//                                 against 11.4 us with the operands in cache).
+//          (WGM = 2, KSPLIT = 4)  the same on a 64 x 64 tile: four pairs of wavefronts, a pair sharing its ring.
+//          (WGM = 2 or 1, KSPLIT = 2)  two K groups: two pairs of wavefronts on a 64 x 64 tile, or two wavefronts on
+//                                 a 32 x 32 tile; a wavefront finishes two quarters of its rows.
+//   rows   (WGM = 4, KSPLIT = 1)  a 128 x 32 NI tile, wavefront w owns rows 32w..32w+31, the ring (two slabs of 32 k)
+//                                 is shared, one barrier per slab.  For products summed in one pass over K whose
+//                                 tiles fill the CUs: 1024 x 3072 x 768 with GELU 39.3 us against 42.4 in 64 x 64
+//                                 tiles (NI = 3); 4096^3 150 against 141 TFLOP/s (NI = 4, two workgroups per CU).
 // Whole tiles are stored through a buffer descriptor (a lane offset, a scalar per row, an immediate per column
 // block: no address arithmetic or bounds checks per value); edge tiles take the checked path.
 // The arithmetic is that of sgemm_dma.hip instruction for instruction (k pairs (8kb + s, 8kb + 4 + s) in ascending
@@ -56,16 +56,16 @@ __device__ __forceinline__ int a_row_swizzle(int row) {
 }
 
 template <int WGM, int KSPLIT, int BK, int STAGES, bool PLAIN, int NI>
-__global__ __launch_bounds__(64 * WGM * KSPLIT > 256 ? 64 * WGM * KSPLIT : 256) void sgemm_wave96_kernel(const float* hotA, const float* hotB, const float* hotB1,
-                                                           const float* hotB2, unsigned hotM, unsigned hotN,
-                                                           unsigned hotK, unsigned hotLda, unsigned hotLdb,
-                                                           unsigned hotBatch, const SgemmParams p) {
+__global__ __launch_bounds__(64 * WGM * KSPLIT > 256 ? 64 * WGM * KSPLIT : 256) void sgemm_wave96_kernel(
+    const float* hotA, const float* hotB, const float* hotB1, const float* hotB2, unsigned hotM, unsigned hotN,
+    unsigned hotK, unsigned hotLda, unsigned hotLdb, unsigned hotBatch, const SgemmParams p) {
   // The leading arguments repeat what the first copies need: scalar arguments at the front of the list arrive in
   // registers with the wavefront, the structure has to be fetched from the argument block first, and nothing of it
   // is looked at before the first slabs are on their way when PLAIN (every batch entry's A starts at hotA, and
   // either its B at hotB too or the launch is the grouped form with at most three products: hotB, hotB1, hotB2 are
   // their B).  hotBatch: p.batch, bit 30 set for the grouped form.
-  static_assert(WGM * KSPLIT == 4 || WGM * KSPLIT == 2 || WGM * KSPLIT == 8, "four wavefronts (one per SIMD), two, or eight");
+  static_assert(WGM * KSPLIT == 4 || WGM * KSPLIT == 2 || WGM * KSPLIT == 8,
+                "four wavefronts (one per SIMD), two, or eight");
   static_assert(KSPLIT == 1 || KSPLIT == 2 || KSPLIT == 4, "the quads of a column block divide among the K groups");
   static_assert(NI >= 1 && NI <= 4, "one to four column blocks of 32 per wavefront");
   constexpr int BN = 32 * NI;       // columns of a tile
