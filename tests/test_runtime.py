@@ -398,7 +398,8 @@ def test_oracle_encoder_layer_against_numpy_float64(mf):
 
 # ---- GPU ----------------------------------------------------------------------------------------------
 @pytest.mark.gpu
-@pytest.mark.parametrize("batch,seq,hidden,heads,ffn", [(2, 16, 64, 4, 128), (3, 7, 96, 3, 200), (8, 128, 768, 12, 3072)])
+@pytest.mark.parametrize("batch,seq,hidden,heads,ffn", [(2, 16, 64, 4, 128), (3, 7, 96, 3, 200), (8, 128, 768, 12, 3072), (2, 128, 1024, 16, 4096),
+                                                     (1, 384, 768, 12, 3072), (5, 100, 768, 12, 3072)])
 def test_encoder_layer_matches_oracle(mf, rt, dev, batch, seq, hidden, heads, ffn):
     """fp32 tolerance: relative Frobenius error <= 1e-5 against the double-accumulating oracle"""
     rng = np.random.default_rng(5)
