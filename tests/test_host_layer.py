@@ -96,3 +96,14 @@ def test_host_layer_framework_cpu(tmp_path):
 def test_host_layer_gpu(tmp_path):
     write_named_test_data(str(tmp_path / "named.npz"))
     _run("gpu", str(tmp_path / "named.npz"))
+
+
+def test_copy_offsets_stay_inside_their_operands():
+    """The HBM -> LDS copies that carry a slab's offset in the unchecked scalar offset: every (lane offset, scalar
+    offset) pair the int8 256 x 256 kernel and the fp32 one-wavefront-per-SIMD kernel can issue on ragged shapes,
+    enumerated on the host with the kernels' own offset functions (tests/cpp/copy_offset_tests.cpp)."""
+    exe = os.path.join(ROOT, "wechat-tfcc_amd", "host", "build", "copy_offset_tests")
+    if not os.path.exists(exe):
+        subprocess.check_call(["make", "-C", os.path.join(ROOT, "wechat-tfcc_amd", "host"), "build/copy_offset_tests"])
+    res = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    assert res.returncode == 0 and "copy offsets ok" in res.stdout, res.stdout[-2000:]

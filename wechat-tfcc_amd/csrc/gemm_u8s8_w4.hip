@@ -30,6 +30,7 @@
 #include <type_traits>
 
 #include "common.hpp"
+#include "copy_offsets.hpp"
 #include "lds_dma.hpp"
 #include "qgemm_dma.hpp"
 
@@ -61,7 +62,6 @@ __global__ __launch_bounds__(kThreads) void qgemm_w4_kernel(const QGemmParams p)
   constexpr int A_BYTES = BM * BK, B_BYTES = BK * BN, STAGE_BYTES = A_BYTES + B_BYTES;
   constexpr int A_COPIES = A_BYTES / 16 / kThreads, B_COPIES = B_BYTES / 16 / kThreads;
   constexpr int COPIES = A_COPIES + B_COPIES;  // per thread per slab
-  constexpr int A_ROWS_PER_COPY = kThreads / CH, B_ROWS_PER_COPY = kThreads / 16;
   static_assert(KS >= 2 && KS % 2 == 0, "the operand registers alternate per step");
   static_assert(COPIES * STAGES < 64, "vmcnt range");
   static_assert(COPIES <= 16, "one copy per matrix op of a step");
@@ -111,20 +111,14 @@ __global__ __launch_bounds__(kThreads) void qgemm_w4_kernel(const QGemmParams p)
   // physical chunk s % CH; B slot s holds k row s / 16, physical chunk s % 16.  From one copy to the next the row
   // advances by a multiple of 16, which leaves both swizzles alone.  The lane offsets (one per copy, first slab)
   // go through the range check of the buffer descriptor, so rows past the end of A read zeros; the slab's offset
-  // is the same for all lanes and rides in the scalar offset, which is not checked: K is a multiple of BK here
-  // and slabs past the end are redirected to the last one (into a stage nobody reads any more).
+  // is the same for all lanes and rides in the scalar offset, which is not checked: K is a multiple of BK here,
+  // slabs past the end are redirected to the last one (into a stage nobody reads any more), and a lane whose
+  // columns of B lie past N carries an offset that fails the check whatever the slab (copy_offsets.hpp).
   unsigned aOff[A_COPIES], bOff[B_COPIES];
-  {
-    const int row = tid / CH, phys = tid % CH;
-    const unsigned a0 = (m0 + row) * K + ((phys ^ swz_a<BK>(row)) << 4);
 #pragma unroll
-    for (int c = 0; c < A_COPIES; ++c) aOff[c] = a0 + (unsigned)c * A_ROWS_PER_COPY * K;
-    const int k = tid >> 4, ph = tid & 15;
-    const int chunk = ((((ph & 7) ^ k) & 7) << 1) | (ph >> 3);  // inverse of phys_b
-    const unsigned b0 = k * N + n0 + (chunk << 4);
+  for (int c = 0; c < A_COPIES; ++c) aOff[c] = copy_offsets::w4_a_lane_offset(tid, c, m0, K, BK);
 #pragma unroll
-    for (int c = 0; c < B_COPIES; ++c) bOff[c] = b0 + (unsigned)c * B_ROWS_PER_COPY * N;
-  }
+  for (int c = 0; c < B_COPIES; ++c) bOff[c] = copy_offsets::w4_b_lane_offset(tid, c, n0, N);
   const unsigned KT = K / BK;
   const unsigned ldsWave = __builtin_amdgcn_readfirstlane(ldsBase + wave * 1024);
   // copy c of `slab` into stage `stage` (a compile-time constant wherever this is called)
@@ -136,7 +130,7 @@ __global__ __launch_bounds__(kThreads) void qgemm_w4_kernel(const QGemmParams p)
   auto slabOffsets = [&](unsigned slab, unsigned& soA, unsigned& soB) {
     const unsigned sl = min(slab, KT - 1);
     soA = __builtin_amdgcn_readfirstlane(sl * BK);
-    soB = __builtin_amdgcn_readfirstlane(sl * BK * N);
+    soB = __builtin_amdgcn_readfirstlane(copy_offsets::w4_b_slab_offset(slab, KT, BK, N));
   };
 
   if (!inGrid) return;

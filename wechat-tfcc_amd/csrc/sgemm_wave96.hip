@@ -36,6 +36,7 @@
 // number of K groups.  Replaces the same oneDNN calls (tfcc/mkl/interfaces/tfcc_mklblasinterface.cpp:41-67, 69-78,
 // 87-118).  Taken for 16-byte aligned operands and strides, K a multiple of 32, B not transposed.
 #include "common.hpp"
+#include "copy_offsets.hpp"
 #include "lds_dma.hpp"
 #include "sgemm_params.hpp"
 
@@ -142,8 +143,8 @@ __global__ __launch_bounds__(64 * WGM * KSPLIT > 256 ? 64 * WGM * KSPLIT : 256) 
       const int s = u * 64 + lane, row = s / CH, phys = s % CH;
       off[c] = ((m0 + row) * lda + ((phys ^ a_row_swizzle<BK>(row)) << 2)) * 4u;
     } else {
-      const int s = (u - A_UNITS) * 64 + lane, k = s / BCH, ch = s % BCH;
-      off[c] = (k * ldb + n0 + ch * 4) * 4u;
+      // (columns past N: an offset that fails the range check whatever the slab's scalar offset, copy_offsets.hpp)
+      off[c] = copy_offsets::w96_b_lane_offset((u - A_UNITS) * 64 + lane, BCH, n0, N, ldb);
     }
   }
   // ring slab t of this group covers k0(t) .. k0(t) + BK - 1; past the end of K it is all zeros
