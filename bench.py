@@ -61,6 +61,113 @@ def probe_check(status):
         sys.exit("measuring probe failed with status %d" % status)
 
 
+# ---- clock and power of the GPU while a leg runs ---------------------------------------------------------------
+# A child process, started before this process makes its first GPU call, samples what the driver publishes in
+# sysfs - the shader clock (the level marked current in pp_dpm_sclk, what rocm-smi --showclocks prints) and the
+# socket power (hwmon power1_input, what rocm-smi --showpower / amd-smi metric --power print) - every few
+# milliseconds, with CLOCK_MONOTONIC stamps; the parent brackets a leg with the same clock and reads the samples
+# that fall inside it.  The child only reads files: it never touches the GPU runtime.
+_SAMPLER_CODE = r"""
+import glob, os, sys, time
+out, period = sys.argv[1], float(sys.argv[2])
+dev = None
+for d in sorted(glob.glob('/sys/class/drm/card*/device')):
+    if os.path.exists(os.path.join(d, 'pp_dpm_sclk')):
+        dev = d
+        break
+power = None
+cap = None
+if dev:
+    for h in sorted(glob.glob(os.path.join(dev, 'hwmon', 'hwmon*'))):
+        for name in ('power1_input', 'power1_average'):
+            if os.path.exists(os.path.join(h, name)):
+                power = os.path.join(h, name)
+                break
+        if power:
+            if os.path.exists(os.path.join(h, 'power1_cap')):
+                cap = open(os.path.join(h, 'power1_cap')).read().strip()
+            break
+f = open(out, 'w')
+f.write('# source %s power %s cap_uW %s\n' % (dev, power, cap))
+f.flush()
+if not dev:
+    sys.exit(0)
+sclk = os.path.join(dev, 'pp_dpm_sclk')
+while not os.path.exists(out + '.stop'):
+    t = time.monotonic()
+    mhz = -1
+    try:
+        for line in open(sclk):
+            if '*' in line:
+                mhz = int(''.join(ch for ch in line.split(':')[1] if ch.isdigit()))
+    except (OSError, ValueError, IndexError):
+        pass
+    uw = -1
+    if power:
+        try:
+            uw = int(open(power).read())
+        except (OSError, ValueError):
+            pass
+    f.write('%.6f %d %d\n' % (t, mhz, uw))
+    f.flush()
+    rest = period - (time.monotonic() - t)
+    if rest > 0:
+        time.sleep(rest)
+"""
+
+
+class GpuSampler:
+    def __init__(self, period_s=0.002):
+        import subprocess
+        import tempfile
+        self.path = os.path.join(tempfile.mkdtemp(prefix="tfcc_bench_"), "samples.txt")
+        self.proc = None
+        self.error = None
+        try:
+            self.proc = subprocess.Popen([sys.executable, "-c", _SAMPLER_CODE, self.path, str(period_s)],
+                                         stdin=subprocess.DEVNULL, stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+        except OSError as e:
+            self.error = "sampler did not start: %s" % e
+
+    def window(self, t0, t1):
+        """Clock and power over the samples stamped inside [t0, t1] (time.monotonic() of this process)."""
+        if self.proc is None:
+            return {"available": False, "why": self.error}
+        header, rows = "", []
+        try:
+            for line in open(self.path):
+                if line.startswith("#"):
+                    header = line[1:].strip()
+                    continue
+                parts = line.split()
+                if len(parts) == 3 and t0 <= float(parts[0]) <= t1:
+                    rows.append((int(parts[1]), int(parts[2])))
+        except OSError as e:
+            return {"available": False, "why": "no samples: %s" % e}
+        mhz = [r[0] for r in rows if r[0] > 0]
+        watts = [r[1] / 1e6 for r in rows if r[1] > 0]
+        if not mhz and not watts:
+            return {"available": False, "why": "neither pp_dpm_sclk nor hwmon power answered on this box (%s)" % header,
+                    "samples": len(rows)}
+        med = lambda v: round(sorted(v)[len(v) // 2], 1) if v else None  # noqa: E731
+        res = {"available": True, "samples": len(rows), "sclk_mhz": med(mhz), "sclk_mhz_min": min(mhz) if mhz else None,
+               "sclk_mhz_max": max(mhz) if mhz else None, "power_w": med(watts),
+               "power_w_max": round(max(watts), 1) if watts else None, "source": header}
+        cap = header.split("cap_uW")[-1].strip() if "cap_uW" in header else ""
+        if cap.isdigit():
+            res["power_cap_w"] = int(cap) / 1e6
+        return res
+
+    def close(self):
+        if self.proc is not None:
+            try:
+                open(self.path + ".stop", "w").close()
+                self.proc.wait(timeout=5)
+            except Exception:
+                self.proc.kill()
+            self.proc = None
+
+
 def time_launches(torch, fn, steps, warmup, pkg=None, stream=0):
     """Average duration of one call in ms, measured with HIP events on the stream fn launches on.
     With pkg and a (non-default) stream the timed launches are recorded once into a HIP graph and the graph
@@ -473,7 +580,9 @@ def bench_other(torch, pkg, dev, steps, warmup, c3, short_legs=False):
     bs = [t(rng.integers(-127, 128, (k, n), dtype=np.int8)) for _ in range(sets)]
     css = [pkg.reduce_sum(x, False) for x in bs]
     scale_b = t(rng.uniform(0.001, 0.01, n).astype(np.float32))
-    for m in (1, 4, 8):
+    # (flags 1: the caller's promise that colsum_b holds the true column sums of b - reduce_sum made them here -, as a
+    # weight matrix prepared once declares; the kernel then forms no column sums of its own)
+    for m, flags in ((1, 0), (4, 0), (8, 0), (1, 1), (4, 1), (8, 1)):
         am = t(rng.integers(0, 256, (m, k), dtype=np.uint8))
         rsm = pkg.reduce_sum(am, True)
         acc = torch.empty((m, n), dtype=torch.int32, device=dev)
@@ -483,16 +592,17 @@ def bench_other(torch, pkg, dev, steps, warmup, c3, short_legs=False):
         def step():
             i = idx[0] % sets
             idx[0] += 1
-            st = lib.tfcc_rocm_gemv_u8s8s32(stream, am.data_ptr(), bs[i].data_ptr(), rsm.data_ptr(), css[i].data_ptr(),
-                                            -128, 0, m, n, k, acc.data_ptr(), 0.02, scale_b.data_ptr(), f32.data_ptr())
+            st = lib.tfcc_rocm_gemv_u8s8s32_flags(stream, am.data_ptr(), bs[i].data_ptr(), rsm.data_ptr(), css[i].data_ptr(),
+                                                  -128, 0, m, n, k, acc.data_ptr(), 0.02, scale_b.data_ptr(), f32.data_ptr(),
+                                                  flags)
             if st != 0:
                 pkg.check(st)
         ms = time_launches(torch, step, max(steps, 50), warmup, pkg, stream)
         nbytes = k * n + m * k + 4 * n + 4 * m * n  # B + A + scales + fp32 out (algorithmic)
         gbs = nbytes / ms / 1e6
-        out["c5_int8_gemv_m%d_4096x11008" % m] = {"ms": round(ms, 5), "gbs": round(gbs, 1),
-                                                   "frac_hbm": round(gbs / PEAK_HBM_GBS, 4),
-                                                   "gops": round(2.0 * m * n * k / ms / 1e6, 1)}
+        name = "c5_int8_gemv_m%d_4096x11008" % m + ("_colsum_declared_exact" if flags else "")
+        out[name] = {"ms": round(ms, 5), "gbs": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4),
+                     "gops": round(2.0 * m * n * k / ms / 1e6, 1)}
     # what bounds those launches on this part: a launch that only reads the same 45 MB (same rotation of
     # buffers), and a launch of workgroups that do nothing
     probe_word = torch.zeros(16, dtype=torch.int32, device=dev)

@@ -63,6 +63,12 @@ int tfcc_rocm_malloc(void** ptr, size_t bytes);
 int tfcc_rocm_free(void* ptr);
 int tfcc_rocm_stream_create(void** stream);
 int tfcc_rocm_stream_destroy(void* stream);
+/* Gives back what the library keeps for `stream` on the current device: the workspace the skinny quantized product
+ * allocates per stream on first use (tfcc_rocm_gemv_u8s8s32; blocks it outgrew included - they stay allocated until
+ * here, because launches recorded earlier may still use them).  The stream must be idle and no graph recorded on it
+ * may be replayed afterwards.  tfcc_rocm_stream_destroy does this itself; call it for streams the library did not
+ * create (a framework's own) before they go away.  No counterpart in the reference (its sessions own no such state). */
+int tfcc_rocm_stream_release(void* stream);
 int tfcc_rocm_stream_synchronize(void* stream);
 /* events on a stream, for timing (cf. tfcc::Coster around Session::sync, tfcc_runtime/framework/model.cpp:191-226) */
 int tfcc_rocm_event_create(void** event);
@@ -227,14 +233,27 @@ int tfcc_rocm_gemv_u8s8s32(void* stream, const uint8_t* a, const int8_t* b,
                            int32_t offset_b, unsigned m, unsigned n, unsigned k, int32_t* acc_out,
                            float scale_a, const float* scale_b, float* f32_out);
 
+/* The same product with the caller's promises about its operands (flags, 0 = none: tfcc_rocm_gemv_u8s8s32).
+ * TFCC_ROCM_GEMV_COLSUM_B_IS_EXACT: colsum_b holds the true column sums of b (e.g. it was made by
+ * tfcc_rocm_reduce_sum_cols from this b, as a weight matrix prepared once has it).  The reference takes the sums as the
+ * caller gives them (tfcc/mkl/operations/tfcc_mklquantization.cpp:33-69) and so does this library; what the promise
+ * spares is the kernel's own column sums, which it needs in addition to turn its uint8 operand into int8.  With a
+ * colsum_b that does not hold the true sums and this flag set, the result is wrong. */
+enum { TFCC_ROCM_GEMV_COLSUM_B_IS_EXACT = 1 };
+int tfcc_rocm_gemv_u8s8s32_flags(void* stream, const uint8_t* a, const int8_t* b,
+                                 const int32_t* rowsum_a, const int32_t* colsum_b, int32_t offset_a,
+                                 int32_t offset_b, unsigned m, unsigned n, unsigned k, int32_t* acc_out,
+                                 float scale_a, const float* scale_b, float* f32_out, unsigned flags);
+
 /* The same product through an entry point that allocates nothing.  No counterpart in the reference; it is for
  * callers that cannot allocate device memory at the point of the call: code under HIP graph capture, tight serving
  * loops, harnesses that forbid it.  tfcc_rocm_gemv_u8s8s32 keeps the workspace of its K-split kernel in memory it
  * allocates on first use (one per device and stream); this one uses a fixed array inside the library's image, one per
  * GPU (1 MiB x 2: 32768 columns x 8 rows of 64-bit words), and therefore
- *   - takes n <= 32768 where the K-split kernel applies (n % 16 == 0, b aligned to 16 bytes, at least 512 steps of 64
- *     rows x 256 columns) and fails with TFCC_ROCM_INVALID_ARGUMENT beyond; smaller products run on the kernel without
- *     a workspace; products that are not skinny (m > 8, unaligned a) are refused, not routed to the general kernel;
+ *   - takes n <= 32768 on the K-split kernel where that applies (n % 16 == 0, b aligned to 16 bytes, at least 512 steps
+ *     of 64 rows x 256 columns); wider products and smaller ones run on the kernel that owns its columns over the whole
+ *     of K and needs no workspace (slower on a decode-sized b); what neither kernel takes fails with
+ *     TFCC_ROCM_INVALID_ARGUMENT (n * k beyond 2^31, m > 8, unaligned a: not routed to the general kernel);
  *   - must not overlap with another call of itself on the same GPU (two streams): both would add into the same
  *     workspace.  Calls on one stream are ordered and leave the workspace zeroed for the next one.
  * Same arguments and results as tfcc_rocm_gemv_u8s8s32. */

@@ -175,6 +175,96 @@ def test_gemv_against_oracle(pkg, T, m, n, k):
     assert np.array_equal(T.n(got), O.qgemm(a, b, -128, 0, rs, cs))
 
 
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 5, 7, 8])
+@pytest.mark.parametrize("n,k", [(11008, 4096), (4096, 4000), (1024, 8192), (2048, 16448)])
+def test_gemv_with_column_sums_declared_exact(pkg, T, m, n, k):
+    """Every row count of the K-split kernel (rows padded to 1, 4 or 8; one or several parts of K; two rows per
+    workspace word or one), with the kernel's own column sums and with the caller's promise that colsum_b holds them."""
+    print("gemv exact", m, n, k, flush=True)
+    rng = np.random.default_rng(1000 * m + n + k)
+    a = rng.integers(0, 256, (m, k), dtype=np.uint8)
+    b = rng.integers(-128, 128, (k, n), dtype=np.int8)
+    if m == 8:  # extreme operands: every partial sum at its bound
+        a[:4] = 255
+        b[:, ::2] = -128
+        b[:, 1::4] = 127
+    rs, cs = O.reduce_sum(a, True), O.reduce_sum(b, False)
+    scale_b = rng.uniform(0.001, 0.01, n).astype(np.float32)
+    want = O.qgemm(a, b, -57, 93, rs, cs)
+    for exact in (False, True):
+        for rep in range(2):  # the second call finds the workspace as the first one left it
+            out, acc = pkg.gemv_dequant(T.t(a), T.t(b), T.t(rs), T.t(cs), -57, 93, 0.02, T.t(scale_b), colsum_exact=exact)
+            assert np.array_equal(T.n(acc), want), (exact, rep)
+            assert np.array_equal(T.n(out), O.dequant_per_channel(want, float(np.float32(0.02)), scale_b))
+    # without the promise the caller's sums are used as given, as the reference uses them
+    wrong = (cs - 5).astype(np.int32)
+    _, acc = pkg.gemv_dequant(T.t(a), T.t(b), T.t(rs), T.t(wrong), -57, 93, 1.0, None)
+    assert np.array_equal(T.n(acc), O.qgemm(a, b, -57, 93, rs, wrong))
+
+
+def test_gemv_beyond_one_round_of_workgroups(pkg, T):
+    """A B so wide that sixteen-wavefront workgroups of one step each would be more than a thousand: the kernel of
+    four wavefronts that walk several steps takes it."""
+    m, n, k = 3, 69632, 4096
+    rng = np.random.default_rng(5)
+    a = rng.integers(0, 256, (m, k), dtype=np.uint8)
+    b = rng.integers(-128, 128, (k, n), dtype=np.int8)
+    rs, cs = O.reduce_sum(a, True), O.reduce_sum(b, False)
+    want = O.qgemm(a, b, -128, 0, rs, cs)
+    for exact in (False, True):
+        _, acc = pkg.gemv_dequant(T.t(a), T.t(b), T.t(rs), T.t(cs), -128, 0, 1.0, None, colsum_exact=exact)
+        assert np.array_equal(T.n(acc), want), exact
+
+
+def test_gemv_recorded_into_a_graph(pkg, T):
+    """A skinny product recorded into a HIP graph: with a workspace from an earlier call the K-split kernel is
+    recorded; on a stream that has none yet nothing may be allocated while recording, and the kernel without a
+    workspace takes the launch.  Either way every replay gives the oracle's sums, also after a wider product on the
+    same stream has outgrown the workspace the graph was recorded with."""
+    import ctypes
+    import torch
+    lib = pkg.lib()
+    m, n, k = 4, 4096, 4096
+    rng = np.random.default_rng(9)
+    a = rng.integers(0, 256, (m, k), dtype=np.uint8)
+    b = rng.integers(-127, 128, (k, n), dtype=np.int8)
+    rs, cs = O.reduce_sum(a, True), O.reduce_sum(b, False)
+    want = O.qgemm(a, b, -57, 93, rs, cs)
+    ta, tb, trs, tcs = T.t(a), T.t(b), T.t(rs), T.t(cs)
+    for warm in (False, True):
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            stream = side.cuda_stream
+            acc = torch.zeros((m, n), dtype=torch.int32, device=ta.device)
+            call = lambda: pkg.check(lib.tfcc_rocm_gemv_u8s8s32(stream, ta.data_ptr(), tb.data_ptr(), trs.data_ptr(),  # noqa: E731
+                                                                tcs.data_ptr(), -57, 93, m, n, k, acc.data_ptr(), 1.0, None, None))
+            if warm:
+                call()
+                torch.cuda.synchronize()
+            graph = ctypes.c_void_p()
+            pkg.check(lib.tfcc_rocm_stream_begin_capture(stream))
+            call()
+            pkg.check(lib.tfcc_rocm_stream_end_capture(stream, ctypes.byref(graph)))
+            for replay in range(3):
+                acc.zero_()
+                torch.cuda.synchronize()
+                pkg.check(lib.tfcc_rocm_graph_launch(graph, stream))
+                torch.cuda.synchronize()
+                assert np.array_equal(T.n(acc), want), (warm, replay)
+                if replay == 0:
+                    # a wider product on the same stream: the workspace grows, the one recorded stays valid
+                    n2 = 8192
+                    b2 = torch.zeros((k, n2), dtype=torch.int8, device=ta.device)
+                    cs2 = torch.zeros((n2,), dtype=torch.int32, device=ta.device)
+                    acc2 = torch.empty((m, n2), dtype=torch.int32, device=ta.device)
+                    pkg.check(lib.tfcc_rocm_gemv_u8s8s32(stream, ta.data_ptr(), b2.data_ptr(), trs.data_ptr(), cs2.data_ptr(),
+                                                         0, 0, m, n2, k, acc2.data_ptr(), 1.0, None, None))
+                    torch.cuda.synchronize()
+                    assert int(acc2.abs().max()) == 0
+            pkg.check(lib.tfcc_rocm_graph_destroy(graph))
+            pkg.check(lib.tfcc_rocm_stream_release(stream))
+
+
 @pytest.mark.parametrize("m", [1, 5, 8])
 @pytest.mark.parametrize("n,k", [(11008, 4096), (16, 16), (100, 80), (260, 4000), (4096, 8320), (64, 12352)])
 def test_gemv_on_packed_weights(pkg, T, m, n, k):

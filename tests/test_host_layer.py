@@ -107,3 +107,14 @@ def test_copy_offsets_stay_inside_their_operands():
         subprocess.check_call(["make", "-C", os.path.join(ROOT, "wechat-tfcc_amd", "host"), "build/copy_offset_tests"])
     res = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
     assert res.returncode == 0 and "copy offsets ok" in res.stdout, res.stdout[-2000:]
+
+
+def test_gemv_workspace_bookkeeping():
+    """Per-stream workspaces of the skinny quantized matmul: kept across calls, never freed while a recorded launch
+    may use them, no growth while allocation is not allowed, cleared after a failed launch, released per stream
+    (tests/cpp/gemv_workspace_tests.cpp with a counting allocator)."""
+    exe = os.path.join(ROOT, "wechat-tfcc_amd", "host", "build", "gemv_workspace_tests")
+    if not os.path.exists(exe):
+        subprocess.check_call(["make", "-C", os.path.join(ROOT, "wechat-tfcc_amd", "host"), "build/gemv_workspace_tests"])
+    res = subprocess.run([exe], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True, timeout=120)
+    assert res.returncode == 0 and "bookkeeping ok" in res.stdout, res.stdout[-2000:]

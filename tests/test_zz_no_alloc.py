@@ -47,16 +47,20 @@ def test_no_alloc_entry_point_matches_the_ordinary_one(pkg, T):
         assert np.array_equal(T.n(out).view(np.uint32), T.n(want_out).view(np.uint32))
 
 
-def test_no_alloc_entry_point_rejects_what_its_workspace_cannot_hold(pkg, T):
+def test_no_alloc_entry_point_beyond_its_workspace(pkg, T):
+    """Wider than the workspace inside the library: the kernel that needs no workspace takes the product (same sums);
+    what neither kernel takes is refused with a clear error instead of being routed to a path that allocates."""
     import torch
-    m, n, k = 1, 32768 + 256, 1024  # wider than the workspace inside the library
-    a = torch.zeros((m, k), dtype=torch.uint8, device="cuda")
-    b = torch.zeros((k, n), dtype=torch.int8, device="cuda")
-    rs = torch.zeros((m,), dtype=torch.int32, device="cuda")
-    cs = torch.zeros((n,), dtype=torch.int32, device="cuda")
+    rng = np.random.default_rng(78)
+    m, n, k = 2, 32768 + 256, 1024
+    a, b, rs, cs, scale_b = _case(rng, m, n, k)
+    ta, tb, trs, tcs = T.t(a), T.t(b), T.t(rs), T.t(cs)
     acc = torch.empty((m, n), dtype=torch.int32, device="cuda")
-    with pytest.raises(Exception, match="workspace inside the library"):
-        pkg.gemv_dequant(a, b, rs, cs, 0, 0, 1.0, None, acc=acc, no_alloc=True)
-    # the ordinary entry point takes the same product
-    _, got = pkg.gemv_dequant(a, b, rs, cs, 0, 0, 1.0, None)
-    assert int(got.abs().max()) == 0
+    pkg.gemv_dequant(ta, tb, trs, tcs, -57, 93, 1.0, None, acc=acc, no_alloc=True)
+    assert np.array_equal(T.n(acc), O.qgemm(a, b, -57, 93, rs, cs))
+    # nine rows: not a skinny product
+    a9 = torch.zeros((9, k), dtype=torch.uint8, device="cuda")
+    rs9 = torch.zeros((9,), dtype=torch.int32, device="cuda")
+    acc9 = torch.empty((9, n), dtype=torch.int32, device="cuda")
+    with pytest.raises(Exception, match="without allocation"):
+        pkg.gemv_dequant(a9, tb, rs9, tcs, 0, 0, 1.0, None, acc=acc9, no_alloc=True)

@@ -83,6 +83,7 @@ SYMBOLS = {
     "tfcc_rocm_free": (_I, [_VP]),
     "tfcc_rocm_stream_create": (_I, [C.POINTER(C.c_void_p)]),
     "tfcc_rocm_stream_destroy": (_I, [_VP]),
+    "tfcc_rocm_stream_release": (_I, [_VP]),
     "tfcc_rocm_stream_synchronize": (_I, [_VP]),
     "tfcc_rocm_memcpy_h2d": (_I, [_VP, _VP, _VP, C.c_size_t]),
     "tfcc_rocm_memcpy_d2h": (_I, [_VP, _VP, _VP, C.c_size_t]),
@@ -96,6 +97,7 @@ SYMBOLS = {
     "tfcc_rocm_gemv_u8s8s32_packed": (_I, [_VP, _VP, _VP, _VP, _VP, C.c_int32, C.c_int32, _U, _U, _U, _VP, _F, _VP, _VP]),
     "tfcc_rocm_gemv_u8s8s32": (_I, [_VP, _VP, _VP, _VP, _VP, C.c_int32, C.c_int32, _U, _U, _U, _VP, _F, _VP, _VP]),
     "tfcc_rocm_gemv_u8s8s32_noalloc": (_I, [_VP, _VP, _VP, _VP, _VP, C.c_int32, C.c_int32, _U, _U, _U, _VP, _F, _VP, _VP]),
+    "tfcc_rocm_gemv_u8s8s32_flags": (_I, [_VP, _VP, _VP, _VP, _VP, C.c_int32, C.c_int32, _U, _U, _U, _VP, _F, _VP, _VP, _U]),
     "tfcc_rocm_reduce_sum_rows": (_I, [_VP, _VP, _I, _U, _U, _U, _VP]),
     "tfcc_rocm_reduce_sum_cols": (_I, [_VP, _VP, _I, _U, _U, _U, _VP]),
     "tfcc_rocm_requantize": (_I, [_VP, _VP, _I, _VP, _I, _U64, _VP, _VP, _VP, _VP]),
@@ -430,10 +432,14 @@ def quantization_matmul_requantize(a, reduce_a, min_a, max_a, b, reduce_b, min_b
     return q, c, min_c, max_c
 
 
+GEMV_COLSUM_B_IS_EXACT = 1
+
+
 def gemv_dequant(a, b, reduce_a, reduce_b, offset_a, offset_b, scale_a, scale_b, want_acc=True, out=None, acc=None,
-                 no_alloc=False):
+                 no_alloc=False, colsum_exact=False):
     """Skinny (M <= 8) product with optional fused per-channel dequantize.  Returns (f32 or None, int32 or None).
-    no_alloc: through the entry point that allocates nothing (the caller then passes `out` / `acc` too)."""
+    no_alloc: through the entry point that allocates nothing (the caller then passes `out` / `acc` too).
+    colsum_exact: the caller vouches that reduce_b holds the true column sums of b."""
     import torch
     a, b = a.contiguous(), b.contiguous()
     m, k, n = a.shape[0], a.shape[1], b.shape[1]
@@ -441,6 +447,12 @@ def gemv_dequant(a, b, reduce_a, reduce_b, offset_a, offset_b, scale_a, scale_b,
         acc = torch.empty((m, n), dtype=torch.int32, device=a.device)
     if out is None and scale_b is not None:
         out = torch.empty((m, n), dtype=torch.float32, device=a.device)
+    if colsum_exact:
+        assert not no_alloc
+        check(lib().tfcc_rocm_gemv_u8s8s32_flags(_stream(), _ptr(a), _ptr(b), _ptr(reduce_a), _ptr(reduce_b), offset_a,
+                                                 offset_b, m, n, k, _ptr(acc), float(scale_a), _ptr(scale_b), _ptr(out),
+                                                 GEMV_COLSUM_B_IS_EXACT))
+        return out, acc
     fn = lib().tfcc_rocm_gemv_u8s8s32_noalloc if no_alloc else lib().tfcc_rocm_gemv_u8s8s32
     check(fn(_stream(), _ptr(a), _ptr(b), _ptr(reduce_a), _ptr(reduce_b), offset_a, offset_b, m, n, k, _ptr(acc),
              float(scale_a), _ptr(scale_b), _ptr(out)))

@@ -4,6 +4,7 @@
 #include <string.h>
 
 #include "common.hpp"
+#include "gemv.hpp"
 
 namespace tfcc_rocm {
 
@@ -96,7 +97,14 @@ int tfcc_rocm_stream_create(void** stream) {
   return TFCC_ROCM_OK;
 }
 
+int tfcc_rocm_stream_release(void* stream) {
+  // the stream's pending work may still use what is given back
+  TFCC_HIP_CHECK(hipStreamSynchronize(as_stream(stream)));
+  return tfcc_rocm::gemv_wide_release_stream(as_stream(stream));
+}
+
 int tfcc_rocm_stream_destroy(void* stream) {
+  if (int e = tfcc_rocm_stream_release(stream)) return e;
   TFCC_HIP_CHECK(hipStreamDestroy(as_stream(stream)));
   return TFCC_ROCM_OK;
 }

@@ -449,7 +449,7 @@ extern "C" int tfcc_rocm_gemm_u8s8s32(void* stream, const tfcc_rocm_qgemm_desc* 
     const float* ranges[4] = {p.minA, p.maxA, p.minB, p.maxB};
     float* rangeOut[2] = {p.minC, p.maxC};
     return gemv_launch(as_stream(stream), p.A, p.B, p.rowsumA, p.colsumB, p.offsetA, p.offsetB, ranges, rangeOut,
-                       p.M, p.N, p.K, c, 0.f, nullptr, nullptr);
+                       p.M, p.N, p.K, c, 0.f, nullptr, nullptr, p.colsumExact != 0);
   }
   return dispatch<false>(as_stream(stream), p);
 }

@@ -325,10 +325,10 @@ bool gemv_supported(const void* a, const void* b, unsigned m, unsigned n, unsign
 int gemv_launch(hipStream_t stream, const unsigned char* a, const signed char* b, const int* rowsumA,
                 const int* colsumB, int offsetA, int offsetB, const float* const ranges[4],
                 float* const rangeOut[2], unsigned m, unsigned n, unsigned k, int* accOut,
-                float scaleA, const float* scaleB, float* f32Out) {
+                float scaleA, const float* scaleB, float* f32Out, bool colsumExact) {
   if (gemv_wide_supported(a, b, m, n, k))
     return gemv_wide_launch(stream, false, a, b, rowsumA, colsumB, offsetA, offsetB, ranges, rangeOut, m, n, k, accOut,
-                            scaleA, scaleB, f32Out);
+                            scaleA, scaleB, f32Out, colsumExact);
   return gemv_onepass_launch(stream, a, b, rowsumA, colsumB, offsetA, offsetB, ranges, rangeOut, m, n, k, accOut, scaleA,
                              scaleB, f32Out);
 }
@@ -371,6 +371,17 @@ extern "C" int tfcc_rocm_gemv_u8s8s32(void* stream, const uint8_t* a, const int8
                                       int32_t offset_a, int32_t offset_b, unsigned m, unsigned n,
                                       unsigned k, int32_t* acc_out, float scale_a,
                                       const float* scale_b, float* f32_out) {
+  return tfcc_rocm_gemv_u8s8s32_flags(stream, a, b, rowsum_a, colsum_b, offset_a, offset_b, m, n, k, acc_out, scale_a,
+                                      scale_b, f32_out, 0u);
+}
+
+extern "C" int tfcc_rocm_gemv_u8s8s32_flags(void* stream, const uint8_t* a, const int8_t* b,
+                                            const int32_t* rowsum_a, const int32_t* colsum_b,
+                                            int32_t offset_a, int32_t offset_b, unsigned m, unsigned n,
+                                            unsigned k, int32_t* acc_out, float scale_a,
+                                            const float* scale_b, float* f32_out, unsigned flags) {
+  TFCC_REQUIRE((flags & ~(unsigned)TFCC_ROCM_GEMV_COLSUM_B_IS_EXACT) == 0, "skinny quantized matmul: unknown flags %#x", flags);
+  const bool colsumExact = (flags & TFCC_ROCM_GEMV_COLSUM_B_IS_EXACT) != 0;
   TFCC_REQUIRE(a && b && rowsum_a && colsum_b, "skinny quantized matmul: null operand");
   TFCC_REQUIRE(m > 0 && n > 0 && k > 0, "skinny quantized matmul: empty operand");
   TFCC_REQUIRE(acc_out || f32_out, "skinny quantized matmul: no output");
@@ -378,13 +389,14 @@ extern "C" int tfcc_rocm_gemv_u8s8s32(void* stream, const uint8_t* a, const int8
   hipStream_t s = as_stream(stream);
   if (gemv_supported(a, b, m, n, k))
     return gemv_launch(s, a, reinterpret_cast<const signed char*>(b), rowsum_a, colsum_b, offset_a,
-                       offset_b, nullptr, nullptr, m, n, k, acc_out, scale_a, scale_b, f32_out);
+                       offset_b, nullptr, nullptr, m, n, k, acc_out, scale_a, scale_b, f32_out, colsumExact);
   // shapes the skinny kernel does not take (m > 8, unaligned): general kernel, then dequantize
   TFCC_REQUIRE(acc_out != nullptr, "skinny quantized matmul: this shape needs acc_out (m > 8 or unaligned operands)");
   tfcc_rocm_qgemm_desc d{};
   d.a = a; d.b = b; d.rowsum_a = rowsum_a; d.colsum_b = colsum_b;
   d.m = m; d.n = n; d.k = k; d.batch = 1; d.stride_c = (uint64_t)m * n;
   d.offset_a = offset_a; d.offset_b = offset_b;
+  d.colsum_b_is_exact = colsumExact ? 1 : 0;
   if (int e = tfcc_rocm_gemm_u8s8s32(stream, &d, acc_out)) return e;
   if (f32_out) {
     size_t total = (size_t)m * n;
@@ -408,16 +420,15 @@ extern "C" int tfcc_rocm_gemv_u8s8s32_noalloc(void* stream, const uint8_t* a, co
   TFCC_REQUIRE(!f32_out || scale_b, "skinny quantized matmul: dequantize needs scale_b");
   hipStream_t s = as_stream(stream);
   const signed char* bs = reinterpret_cast<const signed char*>(b);
-  if (gemv_wide_supported(a, b, m, n, k)) {
-    TFCC_REQUIRE(n <= gemv_wide_static_max_n(),
-                 "skinny quantized matmul without allocation: n = %u, the workspace inside the library holds %u columns", n,
-                 gemv_wide_static_max_n());
+  if (gemv_wide_supported(a, b, m, n, k) && n <= gemv_wide_static_max_n())
     return gemv_wide_launch(s, true, a, bs, rowsum_a, colsum_b, offset_a, offset_b, nullptr, nullptr, m, n, k, acc_out,
                             scale_a, scale_b, f32_out);
-  }
-  // small or narrow products: the kernel that owns its columns over the whole of K uses no workspace at all
+  // small or narrow products, and those wider than the workspace inside the library: the kernel that owns its columns
+  // over the whole of K uses no workspace at all
   TFCC_REQUIRE(gemv_supported(a, b, m, n, k),
-               "skinny quantized matmul without allocation: at most 8 rows, n a multiple of 4, k a multiple of 16, a aligned to 16 bytes");
+               "skinny quantized matmul without allocation: at most 8 rows, n a multiple of 4, k a multiple of 16, a aligned "
+               "to 16 bytes, n * k below 2^31 (beyond the %u columns of the workspace inside the library only the kernel "
+               "without a workspace applies)", gemv_wide_static_max_n());
   return gemv_onepass_launch(s, a, bs, rowsum_a, colsum_b, offset_a, offset_b, nullptr, nullptr, m, n, k, acc_out, scale_a,
                              scale_b, f32_out);
 }

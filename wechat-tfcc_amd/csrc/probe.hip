@@ -52,6 +52,120 @@ __global__ __launch_bounds__(256) void probe_i8_kernel(unsigned iters, int* out)
   out[id] = s;
 }
 
+// The same instruction (kind 0) and the 16x16x64 one (kind 2) issued the way a GEMM kernel issues them: a wavefront
+// owns 128 x 128 outputs (all 256 accumulation registers), holds the operands of one k step in registers (4 + 4
+// quads for 32x32x32, 8 + 8 for 16x16x64) and walks the blocks row by row, every other row backwards, so that one
+// operand stays put for a whole row of blocks and the other changes with every instruction.  HOLD_SRC0 says which
+// source of the instruction is the one that stays.  After every k step all operand registers are xored with a
+// per-lane constant: half of their bits flip, as they do when the next step's data arrives.
+// SLEEP > 0: after every k step the wavefront sleeps 64 * SLEEP cycles, which sets the share of time the matrix
+// cores are busy (16 instructions of 32 cycles per step): 1 -> 0.89, 2 -> 0.80, 4 -> 0.67, 8 -> 0.50.
+template <bool HOLD_SRC0, int SLEEP = 0>
+__global__ __launch_bounds__(256) void probe_i8_tile32_kernel(unsigned ksteps, int* out) {
+  const unsigned id = blockIdx.x * 256 + threadIdx.x;
+  v4i ua[4], ub[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      ua[q][e] = (int)hash32(id * 64 + q * 4 + e);
+      ub[q][e] = (int)hash32(id * 64 + 32 + q * 4 + e);
+    }
+  const int flipA = (int)hash32(id + 0x51ed270bu), flipB = (int)hash32(id + 0x2545f491u);
+  v16i acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0;
+  for (unsigned s = 0; s < ksteps; ++s) {
+#pragma unroll
+    for (int m = 0; m < 16; ++m) {
+      const int i = m / 4, j = m % 4, js = (i & 1) ? 3 - j : j;
+      acc[i][js] = HOLD_SRC0 ? __builtin_amdgcn_mfma_i32_32x32x32_i8(ua[i], ub[js], acc[i][js], 0, 0, 0)
+                             : __builtin_amdgcn_mfma_i32_32x32x32_i8(ub[js], ua[i], acc[i][js], 0, 0, 0);
+    }
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { ua[q][e] ^= flipA; ub[q][e] ^= flipB; }
+    if (SLEEP > 0) __builtin_amdgcn_s_sleep(SLEEP);
+  }
+  int t = 0;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) t += acc[i][j][r];
+  out[id] = t;
+}
+
+template <bool HOLD_SRC0>
+__global__ __launch_bounds__(256) void probe_i8_tile16_kernel(unsigned ksteps, int* out) {
+  const unsigned id = blockIdx.x * 256 + threadIdx.x;
+  v4i ua[8], ub[8];
+#pragma unroll
+  for (int q = 0; q < 8; ++q)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      ua[q][e] = (int)hash32(id * 64 + q * 4 + e);
+      ub[q][e] = (int)hash32(id * 64 + 32 + q * 4 + e);
+    }
+  const int flipA = (int)hash32(id + 0x51ed270bu), flipB = (int)hash32(id + 0x2545f491u);
+  v4i acc[8][8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[i][j] = v4i{0, 0, 0, 0};
+  for (unsigned s = 0; s < ksteps; ++s) {
+#pragma unroll
+    for (int m = 0; m < 64; ++m) {
+      const int i = m / 8, j = m % 8, js = (i & 1) ? 7 - j : j;
+      acc[i][js] = HOLD_SRC0 ? __builtin_amdgcn_mfma_i32_16x16x64_i8(ua[i], ub[js], acc[i][js], 0, 0, 0)
+                             : __builtin_amdgcn_mfma_i32_16x16x64_i8(ub[js], ua[i], acc[i][js], 0, 0, 0);
+    }
+#pragma unroll
+    for (int q = 0; q < 8; ++q)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) { ua[q][e] ^= flipA; ub[q][e] ^= flipB; }
+  }
+  int t = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) t += acc[i][j][0] + acc[i][j][1] + acc[i][j][2] + acc[i][j][3];
+  out[id] = t;
+}
+
+// 16x16x64 with the operand pattern of probe_i8_kernel: four accumulators, both operands change every instruction
+template <bool CHANGING>
+__global__ __launch_bounds__(256) void probe_i8_16_kernel(unsigned iters, int* out) {
+  const unsigned id = blockIdx.x * 256 + threadIdx.x;
+  v4i a[4], b[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    const unsigned s = CHANGING ? id * 8 + q : 0x01020304u;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      a[q][e] = (int)(CHANGING ? hash32(s * 4 + e) : s);
+      b[q][e] = (int)(CHANGING ? hash32(s * 4 + e + 0x9e3779b9u) : s);
+    }
+  }
+  v4i c[4] = {v4i{0, 0, 0, 0}, v4i{0, 0, 0, 0}, v4i{0, 0, 0, 0}, v4i{0, 0, 0, 0}};
+  for (unsigned i = 0; i < iters; i += 4) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) c[j] = __builtin_amdgcn_mfma_i32_16x16x64_i8(a[j], b[(j + q) & 3], c[j], 0, 0, 0);
+  }
+  int s = 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) s += c[j][0] + c[j][1] + c[j][2] + c[j][3];
+  out[id] = s;
+}
+
 template <bool CHANGING>
 __global__ __launch_bounds__(256) void probe_f32_kernel(unsigned iters, int* out) {
   const unsigned id = blockIdx.x * 256 + threadIdx.x;
@@ -123,18 +237,42 @@ extern "C" int tfcc_bench_probe_launch(void* stream, int32_t* out) {
   return launched();
 }
 
+extern "C" int tfcc_bench_probe_mfma_duty(void* stream, int sleep, unsigned blocks, unsigned ksteps, int32_t* out) {
+  if (!(out != nullptr && blocks > 0 && blocks <= 65536 && ksteps > 0)) return 1;
+  hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const dim3 g(blocks), b(256);
+  switch (sleep) {
+    case 0: hipLaunchKernelGGL((probe_i8_tile32_kernel<false, 0>), g, b, 0, s, ksteps, out); break;
+    case 1: hipLaunchKernelGGL((probe_i8_tile32_kernel<false, 1>), g, b, 0, s, ksteps, out); break;
+    case 2: hipLaunchKernelGGL((probe_i8_tile32_kernel<false, 2>), g, b, 0, s, ksteps, out); break;
+    case 4: hipLaunchKernelGGL((probe_i8_tile32_kernel<false, 4>), g, b, 0, s, ksteps, out); break;
+    case 8: hipLaunchKernelGGL((probe_i8_tile32_kernel<false, 8>), g, b, 0, s, ksteps, out); break;
+    default: return 1;
+  }
+  return launched();
+}
+
 extern "C" int tfcc_bench_probe_mfma(void* stream, int kind, int changing_operands, unsigned blocks, unsigned iters,
                                     int32_t* out) {
   if (!(out != nullptr)) return 1;
   if (!(blocks > 0 && blocks <= 65536 && iters > 0 && iters % 4 == 0)) return 1;
-  if (!(kind == 0 || kind == 1)) return 1;
+  if (!(kind == 0 || kind == 1 || kind == 2)) return 1;
+  if (!(changing_operands >= 0 && changing_operands <= (kind == 1 ? 1 : 3))) return 1;
   hipStream_t s = reinterpret_cast<hipStream_t>(stream);
+  const dim3 g(blocks), b(256);
   if (kind == 0) {
-    if (changing_operands) hipLaunchKernelGGL(probe_i8_kernel<true>, dim3(blocks), dim3(256), 0, s, iters, out);
-    else hipLaunchKernelGGL(probe_i8_kernel<false>, dim3(blocks), dim3(256), 0, s, iters, out);
+    if (changing_operands == 3) hipLaunchKernelGGL(probe_i8_tile32_kernel<true>, g, b, 0, s, iters, out);
+    else if (changing_operands == 2) hipLaunchKernelGGL(probe_i8_tile32_kernel<false>, g, b, 0, s, iters, out);
+    else if (changing_operands) hipLaunchKernelGGL(probe_i8_kernel<true>, g, b, 0, s, iters, out);
+    else hipLaunchKernelGGL(probe_i8_kernel<false>, g, b, 0, s, iters, out);
+  } else if (kind == 2) {
+    if (changing_operands == 3) hipLaunchKernelGGL(probe_i8_tile16_kernel<true>, g, b, 0, s, iters, out);
+    else if (changing_operands == 2) hipLaunchKernelGGL(probe_i8_tile16_kernel<false>, g, b, 0, s, iters, out);
+    else if (changing_operands) hipLaunchKernelGGL(probe_i8_16_kernel<true>, g, b, 0, s, iters, out);
+    else hipLaunchKernelGGL(probe_i8_16_kernel<false>, g, b, 0, s, iters, out);
   } else {
-    if (changing_operands) hipLaunchKernelGGL(probe_f32_kernel<true>, dim3(blocks), dim3(256), 0, s, iters, out);
-    else hipLaunchKernelGGL(probe_f32_kernel<false>, dim3(blocks), dim3(256), 0, s, iters, out);
+    if (changing_operands) hipLaunchKernelGGL(probe_f32_kernel<true>, g, b, 0, s, iters, out);
+    else hipLaunchKernelGGL(probe_f32_kernel<false>, g, b, 0, s, iters, out);
   }
   return launched();
 }
