@@ -50,6 +50,7 @@ def bench_lib():
             sys.exit("libtfcc_bench.so is missing: run __graft_entry__.build() first")
         lib = C.CDLL(path)
         lib.tfcc_bench_probe_mfma.argtypes = [C.c_void_p, C.c_int, C.c_int, C.c_uint, C.c_uint, C.c_void_p]
+        lib.tfcc_bench_probe_mfma_duty.argtypes = [C.c_void_p, C.c_int, C.c_uint, C.c_uint, C.c_void_p]
         lib.tfcc_bench_probe_read.argtypes = [C.c_void_p, C.c_void_p, C.c_uint64, C.c_uint, C.c_void_p]
         lib.tfcc_bench_probe_launch.argtypes = [C.c_void_p, C.c_void_p]
         _bench_lib = lib
@@ -544,8 +545,26 @@ def bench_other(torch, pkg, dev, steps, warmup, c3, short_legs=False):
         out["probe_fp32_matrix_cores_alone_%s_operands" % label] = {
             "ms": round(ms, 5), "tflops": round(1024 * 4 * 4 * 2048 * 4096.0 / ms / 1e9, 2)}
 
-    # C3 with the int32 accumulators also written (67 MB more traffic)
+    # C3 as the reference's quantization::matmul returns it (tfcc/mkl/operations/tfcc_mklquantization.cpp:71-203): the
+    # int32 tensor alone (67 MB written), no requantize
     a, b, ta, tb, rs, cs, ranges, out_range = c3
+    d32 = pkg.QGemmDesc()
+    d32.a, d32.b, d32.rowsum_a, d32.colsum_b = ta.data_ptr(), tb.data_ptr(), rs.data_ptr(), cs.data_ptr()
+    d32.m, d32.n, d32.k, d32.batch, d32.stride_c = 4096, 4096, 4096, 1, 4096 * 4096
+    d32.min_a, d32.max_a, d32.min_b, d32.max_b = [r.data_ptr() for r in ranges]
+    range_c = torch.empty(2, dtype=torch.float32, device=dev)
+    d32.min_c, d32.max_c = range_c.data_ptr(), range_c.data_ptr() + 4
+    acc32 = torch.empty((4096, 4096), dtype=torch.int32, device=dev)
+
+    def step32():
+        st = lib.tfcc_rocm_gemm_u8s8s32(stream, C.byref(d32), acc32.data_ptr())
+        if st != 0:
+            pkg.check(st)
+    ms = time_launches(torch, step32, steps, warmup)
+    tops = 2.0 * 4096 ** 3 / ms / 1e9
+    out["c3_int8_4096_int32_only"] = {"ms": round(ms, 5), "tops": round(tops, 2), "frac_int8_mfma": round(tops / PEAK_INT8_TOPS, 4)}
+    del acc32
+    # C3 with the int32 accumulators also written (67 MB more traffic)
     step = make_c3_step(torch, pkg, ta, tb, rs, cs, ranges, out_range, want_acc=True)
     ms = time_launches(torch, step, steps, warmup)
     tops = 2.0 * 4096 ** 3 / ms / 1e9
@@ -650,23 +669,27 @@ def bench_other(torch, pkg, dev, steps, warmup, c3, short_legs=False):
     import importlib
     mf = importlib.import_module("wechat_tfcc_amd.modelfile")
     rt = importlib.import_module("wechat_tfcc_amd.runtime_api")
-    batch, seq, hidden, heads, ffn = 8, 128, 768, 12, 3072
+    hidden, heads, ffn = 768, 12, 3072
     w = mf.bert_layer_weights(rng, hidden, ffn)
-    graph = mf.bert_encoder_layer(w, batch, seq, heads)
-    model = rt.Model(mf.write_model([graph], graph.name))
-    x = {"hidden_states": rng.normal(size=(batch, seq, hidden)).astype(np.float32)}
-    rows = batch * seq
-    gemm_flop = 2.0 * rows * hidden * (4 * hidden + 2 * ffn) + 2 * 2.0 * batch * heads * seq * seq * (hidden // heads)
-    entry = {"gemm_flop": gemm_flop, "nodes": len(graph.nodes)}
-    for label, replay in (("step_by_step", False), ("graph_replay", True)):
-        model.set_replay(replay)
-        us = model.time(x, warmup=warmup, iters=steps)
-        entry[label + "_us"] = round(us, 2)
-        entry[label + "_tflops"] = round(gemm_flop / us / 1e6, 2)
-        entry[label + "_frac_fp32_mfma"] = round(gemm_flop / us / 1e6 / PEAK_FP32_TFLOPS, 4)
-    model.set_replay(False)
-    model.close()
-    out["c4_bert_base_layer_b8_s128_runtime"] = entry
+    # batch 8 x 128 positions (BASELINE configs[3]), and one sequence of 384 positions: the length of the
+    # question-answering model the reference documents (samples/ConvertONNXModel.md:16), whose attention walks the
+    # keys in three blocks of 128
+    for name, batch, seq in (("c4_bert_base_layer_b8_s128_runtime", 8, 128), ("bert_base_layer_b1_s384_runtime", 1, 384)):
+        graph = mf.bert_encoder_layer(w, batch, seq, heads)
+        model = rt.Model(mf.write_model([graph], graph.name))
+        x = {"hidden_states": rng.normal(size=(batch, seq, hidden)).astype(np.float32)}
+        rows = batch * seq
+        gemm_flop = 2.0 * rows * hidden * (4 * hidden + 2 * ffn) + 2 * 2.0 * batch * heads * seq * seq * (hidden // heads)
+        entry = {"gemm_flop": gemm_flop, "nodes": len(graph.nodes)}
+        for label, replay in (("step_by_step", False), ("graph_replay", True)):
+            model.set_replay(replay)
+            us = model.time(x, warmup=warmup, iters=steps)
+            entry[label + "_us"] = round(us, 2)
+            entry[label + "_tflops"] = round(gemm_flop / us / 1e6, 2)
+            entry[label + "_frac_fp32_mfma"] = round(gemm_flop / us / 1e6 / PEAK_FP32_TFLOPS, 4)
+        model.set_replay(False)
+        model.close()
+        out[name] = entry
     return out
 
 
@@ -691,6 +714,8 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the matmul path has no multi-GPU part (run with --gpus 1)")
 
+    # the clock / power sampler is a child process and starts before this process makes its first GPU call
+    sampler = None if (args.headline_only or args.copy_calibration) else GpuSampler()
     import torch
     from __graft_entry__ import load_package
     pkg = load_package()
@@ -760,30 +785,85 @@ def main():
     traffic_file = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(traffic_file):
         result["roofline"]["traffic"] = json.load(open(traffic_file)).get("qgemm_c3_bytes_per_launch")
-    # What the matrix cores sustain with nothing else in the way: register-resident instruction loops of the
-    # headline's op count (2 x 4 wavefronts per CU, 1024 instructions each), with operands that stay the same
-    # and with operands that change from one instruction to the next like the rows of real matrices.
+        result["roofline"]["traffic_is"] = ("from profiles/traffic.json (FETCH_SIZE + WRITE_SIZE counter runs of this "
+                                            "command with --headline-only, scaled by a copy kernel of known size), "
+                                            "not measured in this run")
     if args.headline_only:
         print(json.dumps(result), flush=True)
         return
+
+    def timed_with_power(fn, launches, warm):
+        """ms per launch (HIP events) and the sampler's clock / power over the timed launches (first 30 ms left out)."""
+        for _ in range(warm):
+            fn()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        m0 = time.monotonic()
+        e0.record()
+        for _ in range(launches):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        m1 = time.monotonic()
+        w = sampler.window(m0 + 0.03, m1)
+        keep = {k: w[k] for k in ("sclk_mhz", "power_w", "power_w_max", "samples") if k in w} if w.get("available") else w
+        return e0.elapsed_time(e1) / launches, keep
+
+    # The two regimes of the same launch: after a long warm-up, when the clocks have settled under the power limit
+    # (with the shader clock and the socket power the driver reports meanwhile), and as a burst of a few launches
+    # right after the GPU sat idle (the first launches run at the idle clocks).
+    ms, watt = timed_with_power(step, 4000, 500)
+    result["roofline"]["settled"] = {"steps": 4000, "warmup": 500, "idle_before_s": 0.0, "kernel_ms": round(ms, 5),
+                                     "achieved": round(ops / ms / 1e9, 2), "frac": round(ops / ms / 1e9 / PEAK_INT8_TOPS, 4)}
+    settled_tops = ops / ms / 1e9
+    if watt.get("available") is False:
+        result["roofline"]["sclk_mhz"] = result["roofline"]["power_w"] = None
+        result["roofline"]["clock_power_unavailable"] = watt.get("why")
+    else:
+        result["roofline"]["sclk_mhz"], result["roofline"]["power_w"] = watt.get("sclk_mhz"), watt.get("power_w")
+        result["roofline"]["clock_power_is"] = (
+            "median over the settled leg of the shader clock (pp_dpm_sclk, what rocm-smi --showclocks prints) and the "
+            "socket power (hwmon power1_input), sampled every 2 ms by a child process; nominal peak is quoted at 2400 MHz")
+        result["roofline"]["clock_power_detail"] = watt
+        full = sampler.window(0, time.monotonic())
+        if "power_cap_w" in full:
+            result["roofline"]["power_cap_w"] = full["power_cap_w"]
+    torch.cuda.synchronize()
+    time.sleep(0.5)
+    ms = time_launches(torch, step, 20, 5)
+    result["roofline"]["burst"] = {"steps": 20, "warmup": 5, "idle_before_s": 0.5, "kernel_ms": round(ms, 5),
+                                   "achieved": round(ops / ms / 1e9, 2), "frac": round(ops / ms / 1e9 / PEAK_INT8_TOPS, 4)}
+
+    # What the matrix cores sustain with nothing else in the way: register-resident instruction loops of the
+    # headline's op count, each with the clock and power read while it runs.
+    #   constant / changing operands   four accumulators per wavefront, 2 x 4 wavefronts per CU
+    #   gemm_order                     the product kernel's issue order (a wavefront owns 128 x 128 outputs in all 256
+    #                                  accumulation registers, one operand stays for a row of blocks, half of every
+    #                                  operand's bits flip per k step), with 32x32x32 and with 16x16x64 instructions
+    #   busy_share                     the same with the wavefronts asleep part of the time: what a kernel whose
+    #                                  matrix cores are busy that share of its cycles could reach under the power limit
     probe_out = torch.empty(512 * 256, dtype=torch.int32, device=dev)
     stream0 = torch.cuda.current_stream().cuda_stream
-    for label, changing in (("matrix_cores_alone_constant_operands", 0), ("matrix_cores_alone_changing_operands", 1)):
+    probes = {}
+    for label, kind, pattern, blocks, iters in (
+            ("int8_32x32x32_constant_operands", 0, 0, 512, 256), ("int8_32x32x32_changing_operands", 0, 1, 512, 256),
+            ("int8_32x32x32_gemm_order", 0, 2, 256, 128), ("int8_16x16x64_changing_operands", 2, 1, 512, 512),
+            ("int8_16x16x64_gemm_order", 2, 2, 256, 64)):
         def probe():
-            probe_check(bench_lib().tfcc_bench_probe_mfma(stream0, 0, changing, 512, 256, probe_out.data_ptr()))
-        ms = time_launches(torch, probe, max(args.steps, 200), max(args.warmup, 50))
-        result["roofline"][label] = round(512 * 4 * 4 * 256 * 65536.0 / ms / 1e9, 2)
+            probe_check(bench_lib().tfcc_bench_probe_mfma(stream0, kind, pattern, blocks, iters, probe_out.data_ptr()))
+        ms, watt = timed_with_power(probe, 4000, 300)
+        probes[label] = {"tops": round(ops / ms / 1e9, 2), "frac_of_peak": round(ops / ms / 1e9 / PEAK_INT8_TOPS, 4), **watt}
+    for sleep, share in ((1, 0.89), (2, 0.80), (4, 0.67), (8, 0.50)):
+        def probe():
+            probe_check(bench_lib().tfcc_bench_probe_mfma_duty(stream0, sleep, 256, 128, probe_out.data_ptr()))
+        ms, watt = timed_with_power(probe, 3000, 300)
+        probes["int8_32x32x32_gemm_order_busy_share_%.2f" % share] = {"tops": round(ops / ms / 1e9, 2), **watt}
+    result["roofline"]["matrix_cores_alone"] = probes
+    result["roofline"]["matrix_cores_alone_constant_operands"] = probes["int8_32x32x32_constant_operands"]["tops"]
+    result["roofline"]["matrix_cores_alone_changing_operands"] = probes["int8_32x32x32_changing_operands"]["tops"]
     result["roofline"]["frac_of_matrix_cores_alone_changing_operands"] = round(
-        kernel_tops / result["roofline"]["matrix_cores_alone_changing_operands"], 4)
-    # The two regimes of the same launch: after a long warm-up, when the clocks have settled under the power limit,
-    # and as a burst of a few launches right after the GPU sat idle (the first launches run at the idle clocks).
-    for label, (k_steps, k_warm, idle) in (("settled", (2000, 500, 0.0)), ("burst", (20, 5, 0.5))):
-        torch.cuda.synchronize()
-        if idle:
-            time.sleep(idle)
-        ms = time_launches(torch, step, k_steps, k_warm)
-        result["roofline"][label] = {"steps": k_steps, "warmup": k_warm, "idle_before_s": idle, "kernel_ms": round(ms, 5),
-                                     "achieved": round(ops / ms / 1e9, 2), "frac": round(ops / ms / 1e9 / PEAK_INT8_TOPS, 4)}
+        settled_tops / probes["int8_32x32x32_changing_operands"]["tops"], 4)
+    result["roofline"]["frac_of_matrix_cores_alone_gemm_order"] = round(settled_tops / probes["int8_32x32x32_gemm_order"]["tops"], 4)
     if not args.no_other:
         # on a stream of its own (not the default stream) so that short kernels can be timed as graph replays
         side = torch.cuda.Stream()
@@ -791,6 +871,8 @@ def main():
         with torch.cuda.stream(side):
             result["other"] = bench_other(torch, pkg, dev, max(10, args.steps // 2), args.warmup, c3, args.short_legs)
         torch.cuda.synchronize()
+    if sampler is not None:
+        sampler.close()
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline(a, b, size)
     print(json.dumps(result), flush=True)

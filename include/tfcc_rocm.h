@@ -321,7 +321,12 @@ int tfcc_rocm_softmax_div_f32(void* stream, const float* in, uint64_t rows, unsi
  * Transpose that the reference's runtime runs one operation at a time
  * (tfcc_runtime/operations/math/matmul.cpp:27-41, softmax.cpp, base/transpose.cpp) and returns what
  * tfcc_rocm_sgemm_general (trans_b) + tfcc_rocm_softmax_div_f32 (or division, mask addition and softmax one after
- * the other) + tfcc_rocm_sgemm_general return, bit for bit.  Limits: t <= 128, d <= 64 and a multiple of 4, input strides multiples of 4, inputs 16-byte
+ * the other) + tfcc_rocm_sgemm_general return: bit for bit up to t = 128 keys.  Longer key sequences (the reference's
+ * path has no limit: tfcc/mkl/kernel/tfcc_mklactivationkernel.hpp:137-155 between two batched products,
+ * tfcc/mkl/interfaces/tfcc_mklblasinterface.cpp:127-151) are walked in blocks of 128 keys with a running row maximum
+ * and sum: the same function summed in another order, within a few units in the last place of the separate kernels
+ * and inside the fp32 tolerance of the path (relative Frobenius error <= 1e-5 against double precision).
+ * Limits: d <= 64 and a multiple of 4, input strides multiples of 4, inputs 16-byte
  * aligned, and not a single head (batch_outer * batch_inner == 1) of s <= 8 rows, whose separate product
  * runs on the streaming kernel for short A and sums in another order;
  * tfcc_rocm_attention_f32_supported() tells (1 / 0) whether a descriptor is within them.

@@ -141,12 +141,74 @@ def test_attention_with_mask_equals_separate_kernels(pkg, gpu, B, H, S, Tk, D, d
     assert rel_fro(got, ref) <= 1e-5
 
 
+LONG_CASES = [
+    # B, H, S, T, D, divisor, layout: key sequences beyond one block of 128
+    (1, 12, 384, 384, 64, 8.0, "bshd"),     # the sequence length of the question-answering model the reference documents
+    (2, 3, 70, 129, 64, 8.0, "bshd"),       # one key into the second block
+    (1, 2, 100, 512, 36, 6.0, "bhsd"),      # four whole blocks, head width not a multiple of 8
+    (2, 2, 9, 300, 8, None, "bhsd"),        # ragged last block, no divisor
+    (1, 1, 200, 1000, 64, 8.0, "bshd"),     # eight blocks
+]
+
+
+@pytest.mark.parametrize("B,H,S,Tk,D,divisor,layout", LONG_CASES)
+@pytest.mark.parametrize("masked", [False, True])
+def test_attention_over_blocks_of_keys(pkg, gpu, B, H, S, Tk, D, divisor, layout, masked):
+    """Beyond 128 keys the kernel walks the keys in blocks with a running row maximum and sum: the same real
+    function as the separate kernels, summed in another order, so the check is the fp32 contract (relative Frobenius
+    error <= 1e-5 against float64), and closeness - not equality - to the separate kernels."""
+    import torch
+    print("attention over key blocks", B, H, S, Tk, D, divisor, layout, masked, flush=True)
+    rng = np.random.default_rng(B * 1000 + S + Tk + D)
+    shape_q = (B, S, H, D) if layout == "bshd" else (B, H, S, D)
+    shape_k = (B, Tk, H, D) if layout == "bshd" else (B, H, Tk, D)
+    q, k, v = (rng.normal(size=sh).astype(np.float32) for sh in (shape_q, shape_k, shape_k))
+    # scores large enough that the running maximum moves from block to block
+    q *= 3.0
+    mask = None
+    if masked:
+        mask = np.where(rng.random((B, 1, 1, Tk)) < 0.3, -10000.0, 0.0).astype(np.float32)
+        mask[..., Tk // 2] = 0.0
+    tq, tk, tv = gpu.t(q), gpu.t(k), gpu.t(v)
+    out = torch.empty(shape_q, dtype=torch.float32, device=tq.device)
+    if layout == "bshd":
+        kw = dict(batch_outer=B, batch_inner=H, strides=(S * H * D, Tk * H * D, Tk * H * D, S * H * D), inner_strides=(D,) * 4)
+        lds = (H * D,) * 4
+    else:
+        kw = dict(batch_outer=B, batch_inner=H, strides=(H * S * D, H * Tk * D, H * Tk * D, H * S * D),
+                  inner_strides=(S * D, Tk * D, Tk * D, S * D))
+        lds = (D,) * 4
+    tm = None
+    if masked:
+        tm = gpu.t(mask)
+        kw.update(mask=tm, mask_strides=(Tk, 0))
+    desc = pkg.attention_desc(tq, tk, tv, out, S, Tk, D, lds, divisor=divisor, **kw)
+    assert pkg.attention_supported(desc)
+    pkg.attention(desc)
+    got = gpu.n(out).astype(np.float64)
+    to_bhsd = (lambda x: x.transpose(0, 2, 1, 3)) if layout == "bshd" else (lambda x: x)
+    s = np.einsum("bhsd,bhtd->bhst", to_bhsd(q).astype(np.float64), to_bhsd(k).astype(np.float64))
+    if divisor is not None:
+        s = s / divisor
+    if masked:
+        s = s + mask.astype(np.float64)
+    s = s - s.max(axis=-1, keepdims=True)
+    e = np.exp(s)
+    ref = np.einsum("bhst,bhtd->bhsd", e / e.sum(-1, keepdims=True), to_bhsd(v).astype(np.float64))
+    assert rel_fro(to_bhsd(got), ref) <= 1e-5
+    assert np.all(np.isfinite(got))
+    if not masked:
+        sep = gpu.n(separate_kernels(pkg, torch, tq, tk, tv, B, H, S, Tk, D, divisor, layout)).astype(np.float64)
+        assert rel_fro(got, sep) <= 2e-6
+
+
 def test_attention_limits_are_reported(pkg, gpu):
     import torch
     x = torch.zeros(256 * 256, dtype=torch.float32, device=gpu.t(np.zeros(1, np.float32)).device)
     ok = pkg.attention_desc(x, x, x, x, 16, 128, 64, (64,) * 4)
     assert pkg.attention_supported(ok)
-    for s, t, d, ld in [(16, 129, 64, 64), (16, 16, 68, 68), (16, 16, 6, 8), (16, 16, 8, 10)]:
+    assert pkg.attention_supported(pkg.attention_desc(x, x, x, x, 16, 129, 64, (64,) * 4))  # blocks of 128 keys
+    for s, t, d, ld in [(16, 16, 68, 68), (16, 16, 6, 8), (16, 16, 8, 10)]:
         bad = pkg.attention_desc(x, x, x, x, s, t, d, (ld,) * 4)
         assert not pkg.attention_supported(bad)
         with pytest.raises(pkg.TfccRocmError):

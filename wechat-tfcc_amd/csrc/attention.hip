@@ -1,4 +1,5 @@
-// softmax(Q K^T [/ divisor]) V per batch entry in one launch, for key sequences that fit in LDS.
+// softmax(Q K^T [/ divisor]) V per batch entry in one launch: key sequences of up to 128 rows with the scores of a
+// row block in LDS in one piece (attention_kernel), longer ones in blocks of 128 keys (attention_stream_kernel).
 //
 // Stands where the reference's runtime runs the attention core of an encoder layer as separate
 // operations on tensors in HBM: Matmul (tfcc_runtime/operations/math/matmul.cpp:27-41), Div by a
@@ -282,8 +283,245 @@ __global__ __launch_bounds__(kThreads, 4) void attention_kernel(const AttentionP
   }
 }
 
+// ---- the same for key sequences of any length: the keys are walked in blocks of 128 with a running row maximum and
+// row sum (m, l).  Per block: scores as above; p = exp(score - m_new) with m_new = max(m, block maximum);
+// l = l * exp(m - m_new) + sum(p); the output accumulator of the earlier blocks is scaled by exp(m - m_new) before the
+// block's p V is added; at the end every row is divided by its l.  The same real function as the three separate
+// kernels, summed in a different order (a row's exponentials are taken against the running maximum and rescaled,
+// not against the final one): results agree with them to a few units in the last place, not bit for bit; the
+// contract checked is the relative error against double precision.  Blocks of 128 keep the LDS footprint of the
+// kernel above (two workgroups per CU) whatever the length.
+__global__ __launch_bounds__(kThreads) void attention_stream_kernel(const AttentionParams p) {
+  extern __shared__ __align__(16) float lds[];
+  float* KVs = lds;                       // the block's K as [128][kPitchK], then its V as [128][kPitchV]
+  float* Sc = KVs + kMaxT * kPitchV;      // [64][kPitchS]  scores, then probabilities of the block
+  float* rowScale = Sc + kRows * kPitchS; // [64] what the accumulated rows are multiplied by before the block is added
+                                          //      (after the last block: 1 / l)
+
+  const unsigned wg = blockIdx.x;
+  const unsigned L = (wg & 7u) * p.chunk + (wg >> 3);
+  if ((wg >> 3) >= p.chunk || L >= p.total) return;
+  const unsigned bi = L / p.blocksS, blk = L - bi * p.blocksS;
+  const unsigned bo = bi / p.batchInner, bn = bi - bo * p.batchInner;
+  const unsigned s0 = blk * kRows;
+  const unsigned S = p.S, T = p.T, D = p.D;
+  const float* __restrict__ Q = p.Q + (size_t)bo * p.outerQ + (size_t)bn * p.innerQ;
+  const float* __restrict__ K = p.K + (size_t)bo * p.outerK + (size_t)bn * p.innerK;
+  const float* __restrict__ V = p.V + (size_t)bo * p.outerV + (size_t)bn * p.innerV;
+  float* __restrict__ O = p.O + (size_t)bo * p.outerO + (size_t)bn * p.innerO;
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const bool masked = p.mask != nullptr;
+  const float* __restrict__ mrow = masked ? p.mask + (size_t)bo * p.outerM + (size_t)bn * p.innerM : nullptr;
+  const int lrow = lane & 31, g = lane >> 5;
+  const unsigned Dp = (D + 7u) & ~7u;
+  const int wmS = wave >> 2, wnS = wave & 3;  // scores: 2 x 4 wavefronts, one 32 x 32 block each
+  const int wm = wave >> 1, wn = wave & 1;    // second product: the first four wavefronts, 2 x 2 blocks of 32 x 32
+  constexpr int CH = kMaxD / 4;
+  constexpr int KV_ITEMS = kMaxT * CH / kThreads, Q_ITEMS = kRows * CH / kThreads, KBQ = kMaxD / 8;
+  constexpr unsigned kPastEnd = 0xfffffff0u;
+  const __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float*>(K), 0, (int)(((T - 1) * p.ldk + D) * 4u), 0x00020000);
+  const __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc(
+      const_cast<float*>(V), 0, (int)(((T - 1) * p.ldv + D) * 4u), 0x00020000);
+
+  // ---- Q: through the region of the scores into the registers the score product takes it from, once
+  v4f qf[KBQ];
+  {
+    const __amdgpu_buffer_rsrc_t rq = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<float*>(Q), 0, (int)(((S - 1) * p.ldq + D) * 4u), 0x00020000);
+#pragma unroll
+    for (int it = 0; it < Q_ITEMS; ++it) {
+      const unsigned w = tid + it * kThreads, row = w / CH, ch = w % CH;
+      const v4f q = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(
+                                                rq, (s0 + row < S && ch * 4 < D) ? ((s0 + row) * p.ldq + ch * 4) * 4u : kPastEnd, 0, 0));
+      *reinterpret_cast<v4f*>(Sc + row * kPitchK + ch * 4) = q;
+    }
+    __syncthreads();
+    const float* qa = Sc + (32 * wmS + lrow) * kPitchK + 4 * g;
+#pragma unroll
+    for (int kb = 0; kb < KBQ; ++kb) {
+      qf[kb] = v4f{0.f, 0.f, 0.f, 0.f};
+      if ((unsigned)kb * 8 < Dp) qf[kb] = *reinterpret_cast<const v4f*>(qa + kb * 8);
+    }
+  }
+
+  // running maximum and sum of the eight rows this wavefront owns in the softmax step (rows wave + 8 u)
+  constexpr int R = 8, W = kThreads / 64;
+  static_assert(W * R == kRows, "every row of the block has its wavefront");
+  float mrun[R], lrun[R];
+#pragma unroll
+  for (int u = 0; u < R; ++u) { mrun[u] = -FLT_MAX; lrun[u] = 0.f; }
+  v16f acc;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+
+  const float divisor = p.divisor;
+  const unsigned dbits = __builtin_bit_cast(unsigned, divisor), dexpo = (dbits >> 23) & 0xffu;
+  const bool divideByMul = (dbits & 0x007fffffu) == 0 && dexpo >= 2 && dexpo <= 252;  // a power of two: exact
+  const float inverseDivisor = 1.0f / divisor;
+
+  for (unsigned t0 = 0; t0 < T; t0 += kMaxT) {
+    const unsigned Tb = min((unsigned)kMaxT, T - t0);   // keys of this block
+    const unsigned Tbp = (Tb + 7u) & ~7u;                // k extent of the block's second product
+    v4f kreg[KV_ITEMS], vreg[KV_ITEMS];
+#pragma unroll
+    for (int it = 0; it < KV_ITEMS; ++it) {
+      const unsigned w = tid + it * kThreads, row = w / CH, ch = w % CH;
+      const bool in = row < Tb && ch * 4 < D;
+      kreg[it] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rk, in ? ((t0 + row) * p.ldk + ch * 4) * 4u : kPastEnd, 0, 0));
+    }
+    float mk[2] = {0.f, 0.f};
+    if (masked) {
+#pragma unroll
+      for (int q = 0; q < 2; ++q)
+        if ((unsigned)lane + 64u * q < Tb) mk[q] = mrow[t0 + lane + 64 * q];
+    }
+    __syncthreads();  // the block before is done with K / V and with the probabilities (first block: with Q's staging)
+#pragma unroll
+    for (int it = 0; it < KV_ITEMS; ++it) {
+      const int w = tid + it * kThreads, row = w / CH, ch = w % CH;
+      *reinterpret_cast<v4f*>(KVs + row * kPitchK + ch * 4) = kreg[it];
+    }
+    // (V is asked for once K's registers are free: it travels while the scores are computed)
+#pragma unroll
+    for (int it = 0; it < KV_ITEMS; ++it) {
+      const unsigned w = tid + it * kThreads, row = w / CH, ch = w % CH;
+      const bool in = row < Tb && ch * 4 < D;
+      vreg[it] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rv, in ? ((t0 + row) * p.ldv + ch * 4) * 4u : kPastEnd, 0, 0));
+    }
+    __syncthreads();
+
+    // ---- scores of the block
+    const bool liveS = (unsigned)(32 * wnS) < Tb;
+    if (liveS) {
+      v4f bf[KBQ];
+      const float* ka = KVs + (32 * wnS + lrow) * kPitchK + 4 * g;
+#pragma unroll
+      for (int kb = 0; kb < KBQ; ++kb) {
+        bf[kb] = v4f{0.f, 0.f, 0.f, 0.f};
+        if ((unsigned)kb * 8 < Dp) bf[kb] = *reinterpret_cast<const v4f*>(ka + kb * 8);
+      }
+      v16f sacc;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) sacc[r] = 0.f;
+#pragma unroll
+      for (int kb = 0; kb < KBQ; ++kb) {
+        if ((unsigned)kb * 8 < Dp) {
+#pragma unroll
+          for (int s = 0; s < 4; ++s) sacc = __builtin_amdgcn_mfma_f32_32x32x2f32(qf[kb][s], bf[kb][s], sacc, 0, 0, 0);
+        }
+      }
+      float* sc = Sc + (32 * wmS + 4 * g) * kPitchS + 32 * wnS + lrow;
+      if (!p.divide) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sc[(8 * (r / 4) + (r & 3)) * kPitchS] = sacc[r];
+      } else if (divideByMul) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sc[(8 * (r / 4) + (r & 3)) * kPitchS] = sacc[r] * inverseDivisor;
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sc[(8 * (r / 4) + (r & 3)) * kPitchS] = sacc[r] / divisor;
+      }
+    }
+    __syncthreads();
+
+    // ---- K is done with: V takes its place
+#pragma unroll
+    for (int it = 0; it < KV_ITEMS; ++it) {
+      const int w = tid + it * kThreads, row = w / CH, ch = w % CH;
+      *reinterpret_cast<v4f*>(KVs + row * kPitchV + ch * 4) = vreg[it];
+    }
+
+    // ---- the block's share of the softmax: rows wave + 8 u, columns lane and lane + 64
+    {
+      float v[R][2], mb[R], sum[R];
+#pragma unroll
+      for (int u = 0; u < R; ++u) {
+        const float* sc = Sc + (wave + W * u) * kPitchS;
+        mb[u] = -FLT_MAX;
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+          const unsigned i = lane + 64 * q;
+          v[u][q] = i < Tb ? (masked ? sc[i] + mk[q] : sc[i]) : -FLT_MAX;
+          mb[u] = fmaxf(mb[u], v[u][q]);
+        }
+      }
+      wave_reduce8<true>(mb, lane);
+      float scale[R];
+#pragma unroll
+      for (int u = 0; u < R; ++u) {
+        const float mnew = fmaxf(mrun[u], mb[u]);
+        scale[u] = t0 == 0 ? 0.f : softmax_exp(mrun[u] - mnew);  // nothing is accumulated before the first block
+        mrun[u] = mnew;
+        sum[u] = 0.f;
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+          const unsigned i = lane + 64 * q;
+          v[u][q] = i < Tb ? softmax_exp(v[u][q] - mnew) : 0.f;
+          sum[u] += v[u][q];
+        }
+      }
+      wave_reduce8<false>(sum, lane);
+#pragma unroll
+      for (int u = 0; u < R; ++u) {
+        lrun[u] = lrun[u] * scale[u] + sum[u];
+        float* sc = Sc + (wave + W * u) * kPitchS;
+#pragma unroll
+        for (int q = 0; q < 2; ++q) sc[lane + 64 * q] = v[u][q];  // zeros past the block's keys
+        const bool lastBlock = t0 + kMaxT >= T;
+        if (lane == 0) rowScale[wave + W * u] = scale[u];
+        if (lastBlock && lane == 1) rowScale[kRows + wave + W * u] = 1.0f / lrun[u];
+      }
+    }
+    __syncthreads();
+
+    // ---- accumulated rows scaled, then the block's probabilities x V
+    if (wave < 4 && (unsigned)(32 * wn) < D) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[r] *= rowScale[32 * wm + 8 * (r / 4) + 4 * g + (r & 3)];
+      constexpr int KB = kMaxT / 8, HALF = KB / 2;
+      const float* pa = Sc + (32 * wm + lrow) * kPitchS + 4 * g;
+      const float* vb = KVs + (4 * g) * kPitchV + 32 * wn + lrow;
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        v4f af[HALF], bfv[HALF];
+#pragma unroll
+        for (int q = 0; q < HALF; ++q) {
+          const int kb = h * HALF + q;
+          af[q] = v4f{0.f, 0.f, 0.f, 0.f};
+          bfv[q] = v4f{0.f, 0.f, 0.f, 0.f};
+          if ((unsigned)kb * 8 < Tbp) {
+            af[q] = *reinterpret_cast<const v4f*>(pa + kb * 8);
+#pragma unroll
+            for (int s = 0; s < 4; ++s) bfv[q][s] = vb[(kb * 8 + s) * kPitchV];
+          }
+        }
+#pragma unroll
+        for (int q = 0; q < HALF; ++q) {
+          if ((unsigned)(h * HALF + q) * 8 < Tbp) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[q][s], bfv[q][s], acc, 0, 0, 0);
+          }
+        }
+      }
+    }
+  }
+
+  // ---- rows divided by their sums and stored (the reciprocals were left behind the scales by the last block)
+  if (wave < 4 && (unsigned)(32 * wn) < D) {
+    const unsigned col = 32 * wn + lrow;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int trow = 32 * wm + 8 * (r / 4) + 4 * g + (r & 3);
+      const unsigned row = s0 + trow;
+      if (row < S && col < D) O[(size_t)row * p.ldo + col] = acc[r] * rowScale[kRows + trow];
+    }
+  }
+}
+
 const char* unsupported(const tfcc_rocm_attention_desc* d) {
-  if (d->t > (unsigned)kMaxT) return "more than 128 key rows";
   // a lone product of at most eight rows runs on the streaming kernel (sgemv.hip), whose sums are ordered differently
   if (d->s <= 8 && (unsigned long long)d->batch_outer * d->batch_inner == 1) return "a single head of at most eight query rows";
   if (d->d > (unsigned)kMaxD) return "head width above 64";
@@ -333,7 +571,9 @@ extern "C" int tfcc_rocm_attention_f32(void* stream, const tfcc_rocm_attention_d
   p.mask = d->mask;
   p.outerM = d->stride_mask;
   p.innerM = d->inner_stride_mask;
-  constexpr size_t ldsBytes = (size_t)kLdsFloats * sizeof(float);
+  // up to 128 keys: the scores of a row block in one piece; beyond: blocks of 128 keys with a running maximum and sum
+  const bool stream128 = d->t > (unsigned)kMaxT;
+  constexpr size_t ldsBytes = (size_t)(kLdsFloats + 2 * kRows) * sizeof(float);
   static_assert(ldsBytes <= 80 * 1024, "two workgroups per CU");
   static bool attrSet[16] = {};
   int dev = 0;
@@ -342,8 +582,11 @@ extern "C" int tfcc_rocm_attention_f32(void* stream, const tfcc_rocm_attention_d
   if (!attrSet[dev]) {
     TFCC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes));
+    TFCC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_stream_kernel),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes));
     attrSet[dev] = true;
   }
-  hipLaunchKernelGGL(attention_kernel, dim3(p.chunk * 8), dim3(kThreads), ldsBytes, as_stream(stream), p);
+  if (stream128) hipLaunchKernelGGL(attention_stream_kernel, dim3(p.chunk * 8), dim3(kThreads), ldsBytes, as_stream(stream), p);
+  else hipLaunchKernelGGL(attention_kernel, dim3(p.chunk * 8), dim3(kThreads), ldsBytes, as_stream(stream), p);
   return check_launch("attention");
 }
