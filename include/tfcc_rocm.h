@@ -137,27 +137,6 @@ typedef struct tfcc_rocm_sgemm_desc {
 } tfcc_rocm_sgemm_desc;
 int tfcc_rocm_sgemm_general(void* stream, const tfcc_rocm_sgemm_desc* desc);
 
-/* out = layer_norm(a * b + bias + residual) over the n columns of every row, in one launch: the MatmulWithBias,
- * Add and nn.LayerNormalization that follow each other twice in an encoder layer
- * (tfcc_runtime/operations/math/matmulwithbias.cpp:29-40, tfcc/core/operations/tfcc_math.cpp:38-104,
- * _mkl_layer_normalize, tfcc/mkl/interfaces/tfcc_mklnormalizationinterface.cpp:29-62).  Dense row-major operands:
- * a [m, k], b [k, n], bias [n] or NULL, residual [m, n] or NULL, gamma and beta [n].  The result has the bits of
- * tfcc_rocm_sgemm_fused followed by tfcc_rocm_layer_norm_f32.  Only for the shapes tfcc_rocm_sgemm_layer_norm_supported
- * accepts (16-byte aligned operands, k a multiple of 32, n <= 1024, a product the dispatcher runs on 32 x 96 tiles
- * with four K groups); others are an error.  Workspace of the caller: `sums`, m * n floats (16-byte aligned, contents
- * irrelevant before, the sums before normalisation after), and `counters`,
- * tfcc_rocm_sgemm_layer_norm_counters(m) 32-bit words that must be zero when the launch starts and are zero again
- * when it ends (allocate and clear once, reuse for launches that follow each other on one stream).
- * Measured on MI355X it is slower than the two launches it replaces (1024 x 768 x 768: 27.4 us against 13.9 + 4.6;
- * 1024 x 768 x 3072: 51.5 against 39.5 + 4.0): the tiles of a 32-row band meet through device-scope memory, because
- * the L2 caches of the XCDs do not see each other's stores inside a launch, and the workgroup that stores its tile
- * last normalises the band alone.  The host layer and the runtime therefore keep the two launches. */
-int tfcc_rocm_sgemm_layer_norm_supported(const float* a, const float* b, const float* out, unsigned m, unsigned n,
-                                         unsigned k);
-uint64_t tfcc_rocm_sgemm_layer_norm_counters(unsigned m);
-int tfcc_rocm_sgemm_layer_norm(void* stream, const float* a, const float* b, const float* bias, const float* residual,
-                               const float* gamma, const float* beta, float epsilon, float* out, unsigned m,
-                               unsigned n, unsigned k, float* sums, unsigned* counters);
 
 /* Up to four products a * b[g] (+ bias[g]) -> c[g] that share a dense [m, k] operand a and have equal
  * shapes ([k, n] each, dense), in one launch: e.g. the query / key / value projections of an attention

@@ -119,9 +119,6 @@ SYMBOLS = {
     "tfcc_rocm_graph_destroy": (_I, [_VP]),
     "tfcc_rocm_sgemm_fused": (_I, [_VP, _VP, _U64, _VP, _U64, _VP, _VP, _U64, _VP, _U64, _U, _U, _U, _U, _I]),
     "tfcc_rocm_sgemm_general": (_I, [_VP, _VP]),
-    "tfcc_rocm_sgemm_layer_norm_supported": (_I, [_VP, _VP, _VP, _U, _U, _U]),
-    "tfcc_rocm_sgemm_layer_norm_counters": (_U64, [_U]),
-    "tfcc_rocm_sgemm_layer_norm": (_I, [_VP, _VP, _VP, _VP, _VP, _VP, _VP, _F, _VP, _U, _U, _U, _VP, _VP]),
     "tfcc_rocm_sgemm_grouped": (_I, [_VP, _VP, C.POINTER(_VP), C.POINTER(_VP), C.POINTER(_VP), _U, _U, _U, _U]),
     "tfcc_rocm_unary_f32": (_I, [_VP, _I, _VP, _U64, _VP]),
     "tfcc_rocm_softmax_div_f32": (_I, [_VP, _VP, _U64, _U, _F, _VP]),
@@ -547,37 +544,6 @@ def layer_norm(a, gamma, beta, eps):
     check(lib().tfcc_rocm_layer_norm_f32(_stream(), _ptr(a), _ptr(gamma.contiguous()), _ptr(beta.contiguous()),
                                           eps, a.numel() // a.shape[-1], a.shape[-1], _ptr(out)))
     return out
-
-
-def sgemm_layer_norm_supported(a, b, out_like=None):
-    """Whether layer_norm(a @ b + bias + residual) of these 2-D operands has a one-launch form."""
-    m, k = a.shape
-    n = b.shape[1]
-    return bool(lib().tfcc_rocm_sgemm_layer_norm_supported(_ptr(a), _ptr(b), None if out_like is None else _ptr(out_like),
-                                                           m, n, k))
-
-
-def sgemm_layer_norm(a, b, bias, residual, gamma, beta, eps, counters=None):
-    """layer_norm(a @ b + bias + residual) over the last axis in one launch (tfcc_rocm_sgemm_layer_norm): 2-D
-    float32 operands.  Returns (result, sums before normalisation).  `counters`: a zeroed int32 tensor of
-    tfcc_rocm_sgemm_layer_norm_counters(m) words that the launch leaves zeroed (made here when not given)."""
-    import torch
-    a, b = a.contiguous(), b.contiguous()
-    m, k = a.shape
-    n = b.shape[1]
-    out = torch.empty((m, n), dtype=torch.float32, device=a.device)
-    sums = torch.empty((m, n), dtype=torch.float32, device=a.device)
-    if counters is None:
-        counters = torch.zeros(int(lib().tfcc_rocm_sgemm_layer_norm_counters(m)), dtype=torch.int32, device=a.device)
-    check(lib().tfcc_rocm_sgemm_layer_norm(_stream(), _ptr(a), _ptr(b), _ptr(None if bias is None else bias.contiguous()),
-                                            _ptr(None if residual is None else residual.contiguous()),
-                                            _ptr(gamma.contiguous()), _ptr(beta.contiguous()), eps, _ptr(out), m, n, k,
-                                            _ptr(sums), _ptr(counters)))
-    return out, sums
-
-
-UNARY = {"sigmoid": 0, "tanh": 1, "relu": 2, "softplus": 3, "log": 4, "rsqrt": 5, "erf": 6, "abs": 7, "sign": 8,
-         "neg": 9, "reciprocal": 10, "sqrt": 11}
 
 
 def unary(name, a):

@@ -307,7 +307,7 @@ __device__ static inline float softmax_exp(float x) {
 // GELU in its erf form, 0.5 x (1 + erf(x / sqrt 2)), the function of the reference's scalar template
 // (tfcc/mkl/kernel/tfcc_mklactivationkernel.hpp:213-220, which calls the C library's erff).  One function for the
 // stand-alone kernel and for every fused tile store, so that fusing changes no bit.  1 + erf(q) is erfc(-q), and
-// erfc(t) = 2^(t P(t)) for t >= 0 with P a degree-8 fit of log2(erfc(t)) / t (fit_gelu_erfc.py beside this file
+// erfc(t) = 2^(t P(t)) for t >= 0 with P a degree-8 fit of log2(erfc(t)) / t (tests/golden/fit_gelu_erfc.py
 // makes the coefficients: minimax in the error of erfc, 4e-9): for q < 0 the small factor keeps its relative
 // accuracy, for q > 0 it is 2 - erfc(q).  Past t = 5 erfc is below 2e-12 and taken as 0, which also gives the
 // reference's values at the infinities (NaN at -inf, +inf at +inf) and for NaN.  Eighteen vector instructions

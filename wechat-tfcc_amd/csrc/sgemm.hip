@@ -558,24 +558,6 @@ int dispatch(hipStream_t s, const SgemmParams& p, bool vec, bool tb, unsigned fi
   return launch<2, 2, 1, 1, false>(s, p);
 }
 
-
-// The product + layer norm in one launch exists for the shapes the dispatcher above gives to the 32 x 96 wavefront
-// kernel with four K groups (so that the sums keep their bits), rows of at most kLayerNormMaxColumns.
-bool layer_norm_fusable(const float* a, const float* b, const float* out, unsigned m, unsigned n, unsigned k) {
-  if (m == 0 || n == 0 || k == 0 || k % 32 != 0 || n % 4 != 0 || n > sgemm_detail::kLayerNormMaxColumns) return false;
-  if ((uintptr_t)a % 16 || (uintptr_t)b % 16 || (uintptr_t)out % 16) return false;
-  if (((unsigned long long)m + 256) * k + k + 256 >= (1ull << 30) || ((unsigned long long)k + 256) * n + n + 1024 >= (1ull << 30))
-    return false;
-  SgemmParams probe{};
-  probe.M = m; probe.N = n; probe.K = k; probe.batch = 1; probe.batchInner = 1;
-  if (sgemm_detail::sgemv_supported(probe)) return false;
-  if ((unsigned long long)((m + 127) / 128) * ((n + 127) / 128) >= 512) return false;
-  int best, ksplit;
-  unsigned long long tiles;
-  choose_dma_tiles(m, n, k, 1, best, tiles, ksplit);
-  return kTiles[best].config == 1 && ksplit == 4;
-}
-
 }  // namespace
 }  // namespace tfcc_rocm
 
@@ -662,28 +644,3 @@ extern "C" int tfcc_rocm_sgemm_grouped(void* stream, const float* a, const float
   return dispatch(as_stream(stream), p, vec, false, 1, k, n, n);
 }
 
-extern "C" int tfcc_rocm_sgemm_layer_norm_supported(const float* a, const float* b, const float* out, unsigned m,
-                                                    unsigned n, unsigned k) {
-  return layer_norm_fusable(a, b, out, m, n, k) ? 1 : 0;
-}
-
-extern "C" uint64_t tfcc_rocm_sgemm_layer_norm_counters(unsigned m) { return ((uint64_t)m + 31) / 32; }
-
-extern "C" int tfcc_rocm_sgemm_layer_norm(void* stream, const float* a, const float* b, const float* bias,
-                                          const float* residual, const float* gamma, const float* beta, float epsilon,
-                                          float* out, unsigned m, unsigned n, unsigned k, float* sums,
-                                          unsigned* counters) {
-  TFCC_REQUIRE(a && b && gamma && beta && out && sums && counters, "sgemm + layer norm: null argument");
-  TFCC_REQUIRE(layer_norm_fusable(a, b, out, m, n, k),
-               "sgemm + layer norm: no one-launch form for %u x %u x %u with these operands (ask "
-               "tfcc_rocm_sgemm_layer_norm_supported; use the product and the layer norm)", m, n, k);
-  TFCC_REQUIRE((uintptr_t)sums % 16 == 0, "sgemm + layer norm: workspace not 16-byte aligned");
-  SgemmParams p{};
-  p.A = a; p.B = b; p.bias = bias; p.C = out; p.residual = residual;
-  p.strideR = (unsigned long long)m * n;
-  p.batchInner = 1;
-  p.lda = k; p.ldb = n; p.ldc = n;
-  p.M = m; p.N = n; p.K = k; p.batch = 1;
-  p.lnGamma = gamma; p.lnBeta = beta; p.lnEps = epsilon; p.lnSums = sums; p.lnCounters = counters;
-  return sgemm_detail::sgemm_wave96_launch(as_stream(stream), p, 4);
-}

@@ -25,14 +25,6 @@ struct SgemmParams {
   float* groupC[4];
   unsigned M, N, K, batch;
   unsigned tilesM, tilesN, tilesTotal, chunk;
-  // Layer normalisation of every row of the result over its N columns in the same launch (sgemm_wave96.hip only;
-  // lnGamma == nullptr: none).  The sums a * b + bias + residual go to lnSums [M, N] instead of C; lnCounters holds
-  // one word per band of 32 rows, zero when the launch starts and zero again when it ends.
-  const float* lnGamma;
-  const float* lnBeta;
-  float lnEps;
-  float* lnSums;
-  unsigned* lnCounters;
 };
 
 // Fills in the tile counts for BM x BN tiles; false when there are too many tiles for one grid.
@@ -61,7 +53,6 @@ int sgemm_dma_launch(hipStream_t stream, SgemmParams p, int config, int ksplit, 
 // (blocks 1, rowBlocks 1: two wavefronts); ksplit = 1 - tiles of 128 x 32 blocks, four wavefronts on a shared ring
 // (blocks 3 or 4).  Same requirements and the same bits as the kernels above for the same number of K groups.
 int sgemm_wave96_launch(hipStream_t stream, SgemmParams p, int ksplit, int blocks = 3, int rowBlocks = 0);
-constexpr unsigned kLayerNormMaxColumns = 1024;  // a lane of the normalising wavefront holds 16 values of a row
 
 // The streaming kernel for up to eight rows of A (sgemv.hip): any K, N, strides and alignment; B not transposed.
 bool sgemv_supported(const SgemmParams& p);

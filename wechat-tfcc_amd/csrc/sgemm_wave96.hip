@@ -394,9 +394,7 @@ __global__ __launch_bounds__(64 * WGM * KSPLIT > 256 ? 64 * WGM * KSPLIT : 256) 
 #pragma unroll
         for (int e = 0; e < 4; ++e) sums[(j * QPW + cq) * 4 + e] = v[e];
       }
-    bool toSums = false;
-    if constexpr (WGM == 1 && KSPLIT == 4 && NI == 3) toSums = p.lnGamma != nullptr;
-    if (m0 + wm * 32 + 32 <= M && n0 + BN <= N && ldc < (1u << 24) && !toSums) {
+    if (m0 + wm * 32 + 32 <= M && n0 + BN <= N && ldc < (1u << 24)) {
       // A whole tile: no bounds to check, and the addresses are a register per lane (row 4g, column lrow of the
       // wavefront's 8 QPW rows), a scalar per row and an immediate per column block.
       const __amdgpu_buffer_rsrc_t rc = __builtin_amdgcn_make_buffer_rsrc(
@@ -425,99 +423,7 @@ __global__ __launch_bounds__(64 * WGM * KSPLIT > 256 ? 64 * WGM * KSPLIT : 256) 
       if (Rp) out += rv[q];
       if (act == 1) out = gelu_erf_f32(out);
       if (grow < M && gc < N) {
-        if (toSums) {
-          // read back by another workgroup, possibly on another XCD, later in this launch: written through to
-          // device scope (the L2 caches of the XCDs do not see each other's plain stores before the launch ends)
-          __hip_atomic_store(p.lnSums + (size_t)grow * N + gc, out, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        } else {
-          Cbase[(size_t)grow * ldc + gc] = out;
-        }
-      }
-    }
-    if constexpr (WGM == 1 && KSPLIT == 4 && NI == 3) if (p.lnGamma) {
-      // ---- layer normalisation of the band's 32 rows by whichever of its workgroups stores its tile last.
-      // Every store above has been acknowledged at device scope before this wavefront reaches the barrier, and
-      // the band's counter is incremented after the barrier: the workgroup that reads tilesN - 1 from it sees all
-      // tiles of the band complete.  It resets the counter, so that the next launch finds zeros.
-      wait_vmcnt<0>();
-      __syncthreads();
-      unsigned* flag = reinterpret_cast<unsigned*>(smem);
-      if (threadIdx.x == 0) {
-        unsigned* counter = p.lnCounters + tm;
-        const unsigned before = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const bool last = before == p.tilesN - 1;
-        if (last) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        *flag = last ? 1u : 0u;
-      }
-      __syncthreads();
-      if (*flag == 0u) return;
-      // One wavefront per row, eight rows each.  The stand-alone kernel (layer_norm_reg_kernel in elementwise.hip)
-      // gives a row to 256 threads: thread t holds columns t, t + 256, ..., adds them in that order, the four
-      // wavefronts reduce by butterfly and their sums are added in wavefront order.  Lane l plays threads l,
-      // l + 64, l + 128, l + 192 of that kernel with the same additions in the same order: the same bits.
-      constexpr int PER = (int)(sgemm_detail::kLayerNormMaxColumns / 256);
-      float gm[4][PER], bt[4][PER];
-#pragma unroll
-      for (int w = 0; w < 4; ++w)
-#pragma unroll
-        for (int q = 0; q < PER; ++q) {
-          const unsigned c = lane + 64 * w + 256 * q;
-          gm[w][q] = c < N ? p.lnGamma[c] : 0.f;
-          bt[w][q] = c < N ? p.lnBeta[c] : 0.f;
-        }
-      const float eps = p.lnEps;
-      // four rows at a time: their 64 loads are all under way before the first is waited for (one row after the
-      // other the tail costs a memory round trip per row)
-      for (int u0 = 0; u0 < 8; u0 += 4) {
-        float x[4][4][PER];
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const unsigned row = m0 + 8 * wv + u0 + u;
-          const float* src = p.lnSums + (size_t)row * N;
-#pragma unroll
-          for (int w = 0; w < 4; ++w)
-#pragma unroll
-            for (int q = 0; q < PER; ++q) {
-              const unsigned c = lane + 64 * w + 256 * q;
-              x[u][w][q] = (row < M && c < N) ? __hip_atomic_load(src + c, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0.f;
-            }
-        }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const unsigned row = m0 + 8 * wv + u0 + u;
-          if (row >= M) break;  // wave-uniform
-          float S[4];
-#pragma unroll
-          for (int w = 0; w < 4; ++w) {
-            float t = 0.f;
-#pragma unroll
-            for (int q = 0; q < PER; ++q)
-              if (lane + 64 * w + 256 * q < N) t += x[u][w][q];
-            S[w] = wave_sum(t);
-          }
-          const float mean = (((S[0] + S[1]) + S[2]) + S[3]) / (float)N;
-#pragma unroll
-          for (int w = 0; w < 4; ++w) {
-            float t = 0.f;
-#pragma unroll
-            for (int q = 0; q < PER; ++q)
-              if (lane + 64 * w + 256 * q < N) {
-                const float d = x[u][w][q] - mean;
-                t += d * d;
-              }
-            S[w] = wave_sum(t);
-          }
-          const float var = (((S[0] + S[1]) + S[2]) + S[3]) / (float)N;
-          const float inv = 1.0f / sqrtf(var + eps);
-          float* dst = Cbase + (size_t)row * ldc;
-#pragma unroll
-          for (int w = 0; w < 4; ++w)
-#pragma unroll
-            for (int q = 0; q < PER; ++q) {
-              const unsigned c = lane + 64 * w + 256 * q;
-              if (c < N) dst[c] = (x[u][w][q] - mean) * (inv * gm[w][q]) + bt[w][q];
-            }
-        }
+        Cbase[(size_t)grow * ldc + gc] = out;
       }
     }
   }
