@@ -8,9 +8,12 @@ Headline workload (BASELINE.json configs[2], the one the north-star target is qu
 One step = one such product with inputs resident in HBM.  value = 2*M*N*K / time, in TOP/s.
 
 The same JSON line carries
-  roofline      the dominant kernel against the int8 MFMA peak (5.0 POP/s dense), next to what the matrix
-                cores sustain alone on this box, and the same kernel after a long warm-up ("settled") and
-                as a short burst after idle ("burst")
+  roofline      the dominant kernel against the int8 MFMA peak (5.0 POP/s dense); the same kernel after a long
+                warm-up ("settled", with the shader clock and socket power the driver reports meanwhile: sclk_mhz,
+                power_w) and as a short burst after idle ("burst"); what the matrix cores sustain alone on this box
+                (matrix_cores_alone: register-resident loops with constant and with changing operands, in the
+                kernel's own issue order with 32x32x32 and 16x16x64 instructions, and with the matrix cores busy only
+                part of the time), each with its clock and power
   cpu_baseline  the reference's own AVX2 quantized matmul + requantize (oracle/_ref, kind
                 "reference") or, where that library is absent, the scalar C oracle (kind "port"),
                 timed on this host's cores on a bounded sample, with all threads and with the four the
@@ -19,7 +22,7 @@ The same JSON line carries
   other         the remaining BASELINE configs (fp32 GEMM + bias, attention-shaped batched fp32,
                 skinny int8 decode GEMV, int32-writing variant), each with its own roofline figure
 
-usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-other]
+usage: python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-other] [--no-sampler]
 """
 import argparse
 import ctypes as C
@@ -707,6 +710,9 @@ def main():
     ap.add_argument("--headline-only", action="store_true",
                     help="only the timed launches of the headline kernel (for counter runs): no probes, no settled / "
                          "burst repeats, no secondary configs, no CPU leg")
+    ap.add_argument("--no-sampler", action="store_true",
+                    help="do not start the child process that samples clock and power (for runs under a profiler, whose "
+                         "preloaded library has initialised the GPU before this program starts: nothing may be spawned then)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="instead of the benchmark, run a plain streaming kernel of known size (reads and writes "
                          "256 MiB each per launch) to calibrate the FETCH_SIZE / WRITE_SIZE counters against")
@@ -715,7 +721,7 @@ def main():
         sys.exit("bench.py measures one GPU: the matmul path has no multi-GPU part (run with --gpus 1)")
 
     # the clock / power sampler is a child process and starts before this process makes its first GPU call
-    sampler = None if (args.headline_only or args.copy_calibration) else GpuSampler()
+    sampler = None if (args.headline_only or args.copy_calibration or args.no_sampler) else GpuSampler()
     import torch
     from __graft_entry__ import load_package
     pkg = load_package()
@@ -805,7 +811,7 @@ def main():
         e1.record()
         torch.cuda.synchronize()
         m1 = time.monotonic()
-        w = sampler.window(m0 + 0.03, m1)
+        w = sampler.window(m0 + 0.03, m1) if sampler is not None else {"available": False, "why": "--no-sampler"}
         keep = {k: w[k] for k in ("sclk_mhz", "power_w", "power_w_max", "samples") if k in w} if w.get("available") else w
         return e0.elapsed_time(e1) / launches, keep
 
@@ -825,7 +831,7 @@ def main():
             "median over the settled leg of the shader clock (pp_dpm_sclk, what rocm-smi --showclocks prints) and the "
             "socket power (hwmon power1_input), sampled every 2 ms by a child process; nominal peak is quoted at 2400 MHz")
         result["roofline"]["clock_power_detail"] = watt
-        full = sampler.window(0, time.monotonic())
+        full = sampler.window(0, time.monotonic()) if sampler is not None else {}
         if "power_cap_w" in full:
             result["roofline"]["power_cap_w"] = full["power_cap_w"]
     torch.cuda.synchronize()

@@ -634,6 +634,26 @@ static bool all_similar(const tfcc::Tensor<float>& a, const tfcc::Tensor<float>&
   return true;
 }
 
+// Sequence lengths of the cell classes (tfcc/core/rnn/tfcc_lstmcell.cpp:81-91): at `step`, a row whose length is
+// at most `step` keeps the state it came with, the others take the new one.
+static std::vector<unsigned> alternating_lengths(unsigned batch, unsigned step) {
+  std::vector<unsigned> lengths(batch);
+  for (unsigned r = 0; r < batch; ++r) lengths[r] = r % 2 == 0 ? step : step + 1;  // even rows have ended
+  return lengths;
+}
+static bool rows_follow_lengths(const tfcc::Tensor<float>& got, const tfcc::Tensor<float>& kept,
+                                const tfcc::Tensor<float>& fresh, const std::vector<unsigned>& lengths, unsigned step) {
+  if (got.shape() != kept.shape() || got.shape() != fresh.shape() || got.shape().size() != 2) return false;
+  std::vector<float> g = tfcc::data::get(got), k = tfcc::data::get(kept), f = tfcc::data::get(fresh);
+  const unsigned cols = got.shape(1);
+  for (unsigned r = 0; r < got.shape(0); ++r)
+    for (unsigned c = 0; c < cols; ++c) {
+      const size_t i = static_cast<size_t>(r) * cols + c;
+      if (step >= lengths[r] ? g[i] != k[i] : !is_similar(g[i], f[i])) return false;
+    }
+  return true;
+}
+
 // tfcc/test/rnn.cpp:81-104, data named as tfcc/test/python/createtestdata.py names it
 // ("rnn/lstmcell/<i>/..."), generated by the Python side of this test with the formulas of
 // tfcc/test/python/testcase/rnn/lstmcell.py:31-44.
@@ -659,6 +679,15 @@ static void test_lstmcell_from_constants() {
     CHECK(all_similar(nextState.h, expect));
     CHECK(all_similar(nextState.cs, expectCs));
     CHECK_THROWS(cell(inputs, state, 0, {1u, 2u, 3u, 4u, 5u, 6u, 7u}), tfcc::InvalidArgumentError);
+    {
+      const std::vector<unsigned> lengths = alternating_lengths(inputs.shape(0), 3);
+      std::tie(result, nextState) = cell(inputs, state, 3, lengths);
+      CHECK(rows_follow_lengths(result, state.h, expect, lengths, 3));
+      CHECK(rows_follow_lengths(nextState.h, state.h, expect, lengths, 3));
+      CHECK(rows_follow_lengths(nextState.cs, state.cs, expectCs, lengths, 3));
+      std::tie(result, nextState) = cell(inputs, state, 2, lengths);  // one step earlier every row is still running
+      CHECK(all_similar(nextState.cs, expectCs));
+    }
     // the same constant asked for again is the same object; under another scope it is looked up anew
     CHECK(&tfcc::Constant<float>::getConstant("inputs") == &inputs);
     auto other = tfcc::Scope::scope("nowhere");
@@ -685,6 +714,11 @@ static void test_grucells_from_constants() {
       std::tie(result, nextState) = cell(inputs, state, 0, {});
       CHECK(all_similar(result, tfcc::Constant<float>::getConstant("expect")));
       CHECK(all_similar(nextState, tfcc::Constant<float>::getConstant("expect")));
+      const std::vector<unsigned> lengths = alternating_lengths(inputs.shape(0), 5);
+      std::tie(result, nextState) = cell(inputs, state, 5, lengths);
+      CHECK(rows_follow_lengths(nextState, state, tfcc::Constant<float>::getConstant("expect"), lengths, 5));
+      CHECK(rows_follow_lengths(result, state, tfcc::Constant<float>::getConstant("expect"), lengths, 5));
+      CHECK_THROWS(cell(inputs, state, 0, std::vector<unsigned>(inputs.shape(0) + 1, 1u)), tfcc::InvalidArgumentError);
     }
   }
   {
@@ -702,6 +736,9 @@ static void test_grucells_from_constants() {
       CHECK(all_similar(result, tfcc::Constant<float>::getConstant("expect")));
       std::tie(result, nextState) = cell(inputs, state, 0, {});  // the joined kernels are kept
       CHECK(all_similar(nextState, tfcc::Constant<float>::getConstant("expect")));
+      const std::vector<unsigned> lengths = alternating_lengths(inputs.shape(0), 1);
+      std::tie(result, nextState) = cell(inputs, state, 1, lengths);
+      CHECK(rows_follow_lengths(nextState, state, tfcc::Constant<float>::getConstant("expect"), lengths, 1));
     }
   }
 }
@@ -718,6 +755,20 @@ static void test_data_movement() {
     for (unsigned c = 0; c < 3; ++c) ok = ok && s[r * 3 + c] == hv[r * 6 + 2 + c];
   CHECK(ok);
   CHECK(tfcc::base::slice(v, 0, 3, 99).shape() == tfcc::Shape({1, 6}));
+  {
+    // tfcc::base::assign_to (tfcc/core/operations/tfcc_base.cpp:162-181): columns 1..2 of every row replaced
+    std::vector<int32_t> pv = {100, 101, 102, 103, 104, 105, 106, 107};
+    tfcc::Variable<int32_t> patch = tfcc::data::set(pv, {4, 2});
+    tfcc::Variable<int32_t> target = tfcc::data::copy(v);
+    tfcc::base::assign_to(patch, 1, 1, target);
+    std::vector<int32_t> t = tfcc::data::get(target);
+    bool same = true;
+    for (unsigned r = 0; r < 4; ++r)
+      for (unsigned c = 0; c < 6; ++c) same = same && t[r * 6 + c] == ((c == 1 || c == 2) ? pv[r * 2 + c - 1] : hv[r * 6 + c]);
+    CHECK(same);
+    CHECK_THROWS(tfcc::base::assign_to(patch, 1, 5, target), tfcc::InvalidArgumentError);
+    CHECK_THROWS(tfcc::base::assign_to(patch, 2, 0, target), tfcc::InvalidArgumentError);
+  }
   CHECK_THROWS_MSG(tfcc::base::slice(v, 2, 0, 1), tfcc::InvalidArgumentError, "invalid axis");
   CHECK_THROWS_MSG(tfcc::base::slice(v, 1, 3, 3), tfcc::InvalidArgumentError, "start large than end");
   CHECK_THROWS_MSG(tfcc::base::slice(v, 1, 6, 7), tfcc::InvalidArgumentError, "invalid start");

@@ -504,14 +504,17 @@ def test_fused_graph_is_bit_identical_to_the_graph_as_written(mf, rt, dev):
         got = fused.run({"hidden_states": x})["layer_output"]
         # matmul+gelu and 2 x matmul+add each save one step, query / key / value projections share one launch,
         # the four transposes, the two batched products, the division and the softmax between them are one
-        # step (one launch up to 128 keys and head size 64, three launches in the last two cases)
+        # step (one launch up to head size 64, three launches in the last case).  Up to 128 keys the one launch
+        # has the bits of the graph as written; beyond, it walks the keys in blocks with a running maximum and sum:
+        # the same function summed in another order, equal to a few units in the last place
         assert plain.step_count() - fused.step_count() == 12
-        assert np.array_equal(got, want)
+        same = np.array_equal if seq <= 128 else (lambda p, q: rel_frobenius(p, q) <= 2e-6)
+        assert same(got, want)
         fused.set_replay(True)
         for _ in range(3):
-            assert np.array_equal(fused.run({"hidden_states": x})["layer_output"], want)
+            assert np.array_equal(fused.run({"hidden_states": x})["layer_output"], got)
     # the same layer with an attention mask added between the division and the softmax (one more node in the
-    # one-launch step; with 160 keys the fallback runs division, addition and softmax one after the other)
+    # one-launch step; 160 keys are two blocks of keys)
     for batch, seq, hidden, heads, ffn in ((2, 16, 64, 4, 128), (3, 40, 96, 3, 200), (1, 160, 64, 2, 128)):
         w = mf.bert_layer_weights(rng, hidden, ffn)
         g = mf.bert_encoder_layer(w, batch, seq, heads, with_mask=True)
@@ -525,7 +528,8 @@ def test_fused_graph_is_bit_identical_to_the_graph_as_written(mf, rt, dev):
         rt.set_fusion(True)
         fused = rt.Model(blob)
         assert plain.step_count() - fused.step_count() == 13
-        assert np.array_equal(fused.run(feeds)["layer_output"], want)
+        same = np.array_equal if seq <= 128 else (lambda p, q: rel_frobenius(p, q) <= 2e-6)
+        assert same(fused.run(feeds)["layer_output"], want)
         # the mask matters: without the masked keys the output differs
         other = dict(feeds, attention_mask=np.zeros_like(feeds["attention_mask"]))
         assert not np.array_equal(fused.run(other)["layer_output"], want)

@@ -21,14 +21,29 @@ def test_no_alloc_entry_point_matches_the_ordinary_one(pkg, T):
     rng = np.random.default_rng(77)
     # K-split kernel (workspace in use) at the decode size, then a smaller product of the same kind, then one
     # small enough for the kernel without a workspace
+    # What the entry point cannot help is the HIP runtime loading a kernel's code onto the GPU at that kernel's first
+    # launch in the process, so one call per kernel involved comes first, on operands of zeros (callers that must not
+    # allocate - a stream being recorded, for one - warm up the same way); from then on nothing may be allocated.
+    for m, n, k in ((1, 4096, 2048), (4, 4096, 2048), (8, 4096, 2048), (1, 64, 64)):
+        za = torch.zeros((m, k), dtype=torch.uint8, device="cuda")
+        zb = torch.zeros((k, n), dtype=torch.int8, device="cuda")
+        zr, zc = torch.zeros((m,), dtype=torch.int32, device="cuda"), torch.zeros((n,), dtype=torch.int32, device="cuda")
+        zacc = torch.empty((m, n), dtype=torch.int32, device="cuda")
+        pkg.gemv_dequant(za, zb, zr, zc, 0, 0, 1.0, None, acc=zacc, no_alloc=True)
+        assert int(zacc.abs().max()) == 0
     for m, n, k in ((8, 11008, 4096), (3, 4096, 2048), (5, 260, 80)):
         print("no-alloc gemv", m, n, k, flush=True)
         a, b, rs, cs, scale_b = _case(rng, m, n, k)
         ta, tb, trs, tcs, tsb = T.t(a), T.t(b), T.t(rs), T.t(cs), T.t(scale_b)
         out = torch.empty((m, n), dtype=torch.float32, device=ta.device)
         acc = torch.empty((m, n), dtype=torch.int32, device=ta.device)
-        # the new entry point first: in a fresh process this is the library's first launch
+        # The new entry point before the ordinary one has run on this product: the free device memory is read on
+        # both sides of the call (it drops with any allocation, the library's own included).
+        torch.cuda.synchronize()
+        before_first = torch.cuda.mem_get_info()[0]
         pkg.gemv_dequant(ta, tb, trs, tcs, -57, 93, 0.02, tsb, out=out, acc=acc, no_alloc=True)
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == before_first
         got_out, got_acc = T.n(out).copy(), T.n(acc).copy()
         want_out, want_acc = pkg.gemv_dequant(ta, tb, trs, tcs, -57, 93, 0.02, tsb)
         assert np.array_equal(got_acc, T.n(want_acc))

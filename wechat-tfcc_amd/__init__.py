@@ -546,6 +546,10 @@ def layer_norm(a, gamma, beta, eps):
     return out
 
 
+UNARY = {"sigmoid": 0, "tanh": 1, "relu": 2, "softplus": 3, "log": 4, "rsqrt": 5, "erf": 6, "abs": 7, "sign": 8,
+         "neg": 9, "reciprocal": 10, "sqrt": 11}
+
+
 def unary(name, a):
     """tfcc_rocm_unary_f32: one of UNARY applied element-wise."""
     import torch

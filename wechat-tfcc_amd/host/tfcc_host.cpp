@@ -782,6 +782,15 @@ class ROCMBasicInterface : public BasicInterface<T> {
     }
     return r;
   }
+  // tfcc/mkl/interfaces/tfcc_mklbasicinterface.cpp:518-537: one strided copy
+  void assignTo(const Tensor<T>& a, size_t axis, unsigned start, Variable<T>& b) override {
+    if (a.size() == 0) return;
+    uint64_t s1, s3;
+    split_at(a.shape(), axis, s1, s3);
+    const uint64_t width = static_cast<uint64_t>(a.shape(axis)) * s3 * sizeof(T);
+    check(tfcc_rocm_copy2d(current_stream(), a.data(), width, b.data() + static_cast<size_t>(start) * s3,
+                           static_cast<uint64_t>(b.shape(axis)) * s3 * sizeof(T), s1, width));
+  }
   Variable<T> clip(const Tensor<T>& a, T minValue, T maxValue) override {
     if constexpr (std::is_same<T, float>::value) {
       Variable<T> r(a.shape());

@@ -132,6 +132,7 @@ class BasicInterface {
   virtual Variable<T> transpose(const Tensor<T>&, const std::vector<size_t>&) { throw NotImplementedError(); }
   virtual Variable<T> slice(const Tensor<T>&, size_t, unsigned, unsigned) { throw NotImplementedError(); }
   virtual Variable<T> concat(const std::vector<const Tensor<T>*>&, size_t) { throw NotImplementedError(); }
+  virtual void assignTo(const Tensor<T>&, size_t, unsigned, Variable<T>&) { throw NotImplementedError(); }
   // rows of params by index (tfcc/core/interfaces/tfcc_gatherinterface.h): indices of the type with code indexCode
   virtual Variable<T> clip(const Tensor<T>&, T, T) { throw NotImplementedError(); }
   virtual Variable<int64_t> argmax(const Tensor<T>&, size_t) { throw NotImplementedError(); }
@@ -721,6 +722,16 @@ Variable<T> concat(const std::vector<const Tensor<T>*>& values, size_t axis) {
 template <class T>
 Variable<T> concat(std::initializer_list<const Tensor<T>*> values, size_t axis) {
   return concat(std::vector<const Tensor<T>*>(values), axis);
+}
+// tfcc/core/operations/tfcc_base.cpp:162-181: a written into b at position `start` along `axis`
+template <class T>
+void assign_to(const Tensor<T>& a, size_t axis, unsigned start, Variable<T>& b) {
+  if (a.shape().size() != b.shape().size()) throw InvalidArgumentError("dimensions not match");
+  if (axis >= a.shape().size()) throw InvalidArgumentError("invalid axis");
+  for (size_t i = 0; i < a.shape().size(); ++i)
+    if (i != axis && a.shape(i) != b.shape(i)) throw InvalidArgumentError("shape not match");
+  if (b.shape(axis) < start + a.shape(axis)) throw InvalidArgumentError("b is too small to assign");
+  Operation<T>::getCurrentInterface().getBasicInterface().assignTo(a, axis, start, b);
 }
 // tfcc/core/operations/tfcc_base.cpp:43-59: num equal parts along axis
 template <class T>

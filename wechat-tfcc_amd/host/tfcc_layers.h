@@ -251,8 +251,8 @@ Variable<T> dense(const Tensor<T>& inputs, unsigned units, bool useBias, std::st
 namespace rnn {
 
 // One step of an LSTM whose kernel is [inputSize + units, 4 units] (rows of the inputs first, then of h) under
-// "<name>/kernel" and "<name>/bias"; forget bias 1.  Sequence lengths (state frozen past a row's length) are not
-// implemented on this device.
+// "<name>/kernel" and "<name>/bias"; forget bias 1.  With sequence lengths a row whose length is at most `step` keeps
+// the state it came with (tfcc/core/rnn/tfcc_lstmcell.cpp:81-91).
 template <class T>
 class LSTMCell {
   bool _initialized = false;
@@ -280,11 +280,9 @@ class LSTMCell {
 
   std::pair<Variable<T>, State> operator()(const Tensor<T>& inputs, const State& state, size_t step = 0,
                                            const std::vector<unsigned>& lengths = {}) {
-    (void)step;
     if (inputs.shape().size() != 2) throw InvalidArgumentError("invalid inputs");
     if (inputs.shape(0) != state.cs.shape(0)) throw InvalidArgumentError("state and inputs don't match");
     if (lengths.size() != 0 && lengths.size() != inputs.shape(0)) throw InvalidArgumentError("invalid lengths");
-    if (lengths.size() != 0) throw NotImplementedError("LSTMCell with sequence lengths");
     auto scopeG = Scope::scope(_name);
     if (!_initialized) {
       _kernel = &Constant<T>::getConstant("kernel");
@@ -297,6 +295,14 @@ class LSTMCell {
     std::tie(next.h, next.cs) = interface.getCellInterface().processLSTMCell(
         state.cs, blas::matmul(inputs, View<T>(*_kernel, _kernel->shape(), 0, inputs.shape(1))),
         blas::matmul(state.h, View<T>(*_kernel, _kernel->shape(), inputs.shape(1))), *_bias, static_cast<T>(1));
+    // a sequence that has ended keeps its state (tfcc/core/rnn/tfcc_lstmcell.cpp:81-91)
+    for (unsigned i = 0; i < lengths.size(); ++i) {
+      if (step < lengths[i]) continue;
+      View<T> vcs(state.cs, state.cs.shape(), i, i + 1);
+      base::assign_to(vcs, 0, i, next.cs);
+      View<T> vh(state.h, state.h.shape(), i, i + 1);
+      base::assign_to(vh, 0, i, next.h);
+    }
     Variable<T> output = data::copy(next.h);
     return std::make_pair(std::move(output), std::move(next));
   }
@@ -304,7 +310,7 @@ class LSTMCell {
 
 // One step of a GRU in TensorFlow's layout (tfcc/core/rnn/tfcc_grucell.cpp:46-105): "<name>/gates/kernel"
 // [inputSize + units, 2 units] with "gates/bias", "<name>/candidate/kernel" [inputSize + units, units] with
-// "candidate/bias".  Sequence lengths are not implemented on this device.
+// "candidate/bias".
 template <class T>
 class GRUCell {
   bool _initialized = false;
@@ -329,11 +335,9 @@ class GRUCell {
 
   std::pair<Variable<T>, State> operator()(const Tensor<T>& input, const State& state, size_t step = 0,
                                            const std::vector<unsigned>& lengths = {}) {
-    (void)step;
     if (input.shape().size() != 2) throw InvalidArgumentError("invalid inputs");
     if (input.shape(0) != state.shape(0)) throw InvalidArgumentError("state and inputs don't match");
     if (lengths.size() != 0 && lengths.size() != input.shape(0)) throw InvalidArgumentError("invalid lengths");
-    if (lengths.size() != 0) throw NotImplementedError("GRUCell with sequence lengths");
     auto scopeG = Scope::scope(_name);
     if (!_initialized) {
       {
@@ -354,6 +358,11 @@ class GRUCell {
     Variable<T> ci = interface.getCellInterface().processGRUCellGates(state, input, value, *_gatesBias);
     State h = interface.getCellInterface().processGRUCellCandidate(state, value, *_gatesBias,
                                                                    blas::matmul(ci, *_candidateKernel), *_candidateBias);
+    for (unsigned i = 0; i < lengths.size(); ++i) {  // tfcc/core/rnn/tfcc_grucell.cpp:94-102
+      if (step < lengths[i]) continue;
+      View<T> vs(state, state.shape(), i, i + 1);
+      base::assign_to(vs, 0, i, h);
+    }
     Variable<T> output = data::copy(h);
     return std::make_pair(std::move(output), std::move(h));
   }
@@ -387,11 +396,9 @@ class PyTorchGRUCell {
 
   std::pair<Variable<T>, State> operator()(const Tensor<T>& input, const State& state, size_t step = 0,
                                            const std::vector<unsigned>& lengths = {}) {
-    (void)step;
     if (input.shape().size() != 2) throw InvalidArgumentError("invalid inputs");
     if (input.shape(0) != state.shape(0)) throw InvalidArgumentError("state and inputs don't match");
     if (lengths.size() != 0 && lengths.size() != input.shape(0)) throw InvalidArgumentError("invalid lengths");
-    if (lengths.size() != 0) throw NotImplementedError("PyTorchGRUCell with sequence lengths");
     auto scopeG = Scope::scope(_name);
     if (!_initialized) {
       _gatesBias = &Constant<T>::getConstant("bias_gates");
@@ -411,6 +418,11 @@ class PyTorchGRUCell {
     Variable<T> stateValue = blas::matmul(state, _stateKernel);
     State hy = Operation<T>::getCurrentInterface().getCellInterface().processPyTorchGRUCell(
         state, inputValue, stateValue, *_gatesBias, *_candidateIBias, *_candidateHBias);
+    for (unsigned i = 0; i < lengths.size(); ++i) {  // tfcc/core/rnn/tfcc_pytorchgrucell.cpp:103-111
+      if (step < lengths[i]) continue;
+      View<T> vs(state, state.shape(), i, i + 1);
+      base::assign_to(vs, 0, i, hy);
+    }
     Variable<T> output = data::copy(hy);
     return std::make_pair(std::move(output), std::move(hy));
   }
