@@ -393,7 +393,7 @@ def bench_other(torch, pkg, dev, steps, warmup, c3, short_legs=False):
     def sets_beyond_llc(bytes_per_set):
         return max(2, int(1.25 * LLC_BYTES / bytes_per_set) + 1)
 
-    def sgemm_case(name, shape_a, shape_b, bias, sets=None):
+    def sgemm_case(name, shape_a, shape_b, bias, sets=None, step_by_step=False):
         p = pkg.matmul_plan(shape_a, shape_b, None if not bias else (shape_b[-1],))
         # operand sets rotated over more bytes than the last-level cache holds (sets=1: compute-bound, no rotation)
         per_set = 4 * (int(np.prod(shape_a)) + int(np.prod(shape_b)) + int(np.prod(p["shape"])))
@@ -421,11 +421,15 @@ def bench_other(torch, pkg, dev, steps, warmup, c3, short_legs=False):
         tflops, gbs = flop / ms / 1e9, nbytes / ms / 1e6
         out[name] = {"ms": round(ms, 5), "tflops": round(tflops, 3), "frac_fp32_mfma": round(tflops / PEAK_FP32_TFLOPS, 4),
                      "gbs": round(gbs, 1), "frac_hbm": round(gbs / PEAK_HBM_GBS, 4)}
+        if step_by_step:
+            # The same launches issued one by one instead of replayed from a recorded graph: the difference is what a
+            # graph node costs over a plain launch on this runtime (the kernel is long enough to hide the host's launch cost).
+            out[name]["ms_step_by_step"] = round(time_launches(torch, step, max(steps, 300), warmup), 5)
 
     sgemm_case("c1_fp32_128x768x3072_bias", (128, 768), (768, 3072), True)
     sgemm_case("c2_fp32_qk_16x12x128x64x128", (16, 12, 128, 64), (16, 12, 64, 128), False)
     sgemm_case("c2_fp32_pv_16x12x128x128x64", (16, 12, 128, 128), (16, 12, 128, 64), False)
-    sgemm_case("c4_fp32_ffn_up_1024x768x3072_bias", (8, 128, 768), (768, 3072), True, sets=4)
+    sgemm_case("c4_fp32_ffn_up_1024x768x3072_bias", (8, 128, 768), (768, 3072), True, sets=4, step_by_step=True)
 
     # C2, second case: a [1, 12, 64, 64] weight broadcast over the batch of a [16, 12, 128, 64] input
     def broadcast_case(name, shape_a, shape_b):
