@@ -69,6 +69,10 @@ CASES = [
     (3, 5, 64, 5, 4, 0.5, "bshd"),
     (1, 4, 65, 64, 32, 5.656854, "bhsd"),   # one row past a block; only the first column half is live
     (1, 2, 31, 97, 60, 7.75, "bshd"),
+    # more blocks of 64 query rows than the GPU has CUs: blocks of 32 rows, three workgroups per CU
+    (16, 12, 128, 128, 64, 8.0, "bshd"),    # the attention shape of the benchmark
+    (6, 12, 200, 100, 64, 8.0, "bshd"),     # a ragged last block of 8 rows, ragged keys
+    (5, 13, 261, 77, 36, None, "bhsd"),     # a last block of 5 rows, head width not a multiple of 8
 ]
 
 
@@ -111,6 +115,7 @@ def test_attention_equals_separate_kernels(pkg, gpu, B, H, S, Tk, D, divisor, la
     (2, 12, 128, 128, 64, 8.0, False),   # the encoder layer's attention core with a [B, 1, 1, T] mask
     (3, 2, 70, 100, 36, 6.0, False), (2, 3, 33, 65, 16, None, False), (2, 4, 40, 24, 32, 5.0, True),
     (1, 2, 5, 7, 8, 3.0, False),
+    (9, 8, 250, 128, 64, 8.0, False), (4, 17, 250, 90, 40, 6.5, True),   # blocks of 32 query rows
 ])
 def test_attention_with_mask_equals_separate_kernels(pkg, gpu, B, H, S, Tk, D, divisor, per_head):
     """A mask [B, 1, 1, T] (or [B, H, 1, T]) added between the division and the softmax, as BERT graphs do:

@@ -49,7 +49,14 @@ struct AttentionParams {
 };
 
 
-__global__ __launch_bounds__(kThreads, 4) void attention_kernel(const AttentionParams p) {
+// ROWS query rows per workgroup, a wavefront per eight of them: 64 rows (eight wavefronts, 70.7 KB, two workgroups per
+// CU) when every CU gets at most one workgroup that way, 32 rows (four wavefronts, 53.8 KB, three per CU) when the
+// 64-row blocks would pile up two on some CUs and one or none on others (16 x 12 heads of 128 rows: 384 blocks of 64
+// on 256 CUs against 768 blocks of 32, three on every CU).  The arithmetic per element is the same.
+template <int ROWS>
+__global__ __launch_bounds__(8 * ROWS, ROWS == 64 ? 4 : 3) void attention_kernel(const AttentionParams p) {
+  constexpr int kRows = ROWS, kThreads = 8 * ROWS;
+  static_assert(ROWS == 64 || ROWS == 32, "two or one row blocks of 32");
   extern __shared__ __align__(16) float lds[];
   float* KVs = lds;                       // K as [128][kPitchK], later V as [128][kPitchV]
   float* Sc = KVs + kMaxT * kPitchV;      // [64][kPitchS]  scores, then probabilities
@@ -86,7 +93,7 @@ __global__ __launch_bounds__(kThreads, 4) void attention_kernel(const AttentionP
   // the score product takes it from; V waits in registers until K is no longer needed.  A buffer load whose
   // offset lies past the end of its operand returns zero: that is how everything past the operands' extents
   // that a matrix op will read becomes zero.
-  const int wmS = wave >> 2, wnS = wave & 3;  // scores: 2 x 4 wavefronts, one 32 x 32 block each
+  const int wmS = wave >> 2, wnS = wave & 3;  // scores: ROWS / 32 x 4 wavefronts, one 32 x 32 block each
   constexpr int CH = kMaxD / 4;               // 16-byte chunks per row
   constexpr int KV_ITEMS = kMaxT * CH / kThreads, Q_ITEMS = kRows * CH / kThreads, KBQ = kMaxD / 8;
   constexpr unsigned kPastEnd = 0xfffffff0u;
@@ -229,55 +236,125 @@ __global__ __launch_bounds__(kThreads, 4) void attention_kernel(const AttentionP
   }
   __syncthreads();
 
-  // ---- probabilities x V: the first four wavefronts, (wm, wn) owning rows 32*wm.. and columns 32*wn.. of the
-  // 64 x D result (one accumulator per element over all of T, as in a product of its own)
-  const int wm = wave >> 1, wn = wave & 1;
-  if (wave < 4 && (unsigned)(32 * wn) < D) {
-    constexpr int KB = kMaxT / 8, HALF = KB / 2;
-    v16f acc;
+  if constexpr (ROWS == 64) {
+    // ---- probabilities x V: the first four wavefronts, (wm, wn) owning rows 32*wm.. and columns 32*wn.. of the
+    // 64 x D result (one accumulator per element over all of T, as in a product of its own)
+    const int wm = wave >> 1, wn = wave & 1;
+    if (wave < 4 && (unsigned)(32 * wn) < D) {
+      constexpr int KB = kMaxT / 8, HALF = KB / 2;
+      v16f acc;
 #pragma unroll
-    for (int r = 0; r < 16; ++r) acc[r] = 0.f;
-    const float* pa = Sc + (32 * wm + lrow) * kPitchS + 4 * g;
-    const float* vb = KVs + (4 * g) * kPitchV + 32 * wn + lrow;
+      for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+      const float* pa = Sc + (32 * wm + lrow) * kPitchS + 4 * g;
+      const float* vb = KVs + (4 * g) * kPitchV + 32 * wn + lrow;
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {  // operands are fetched from LDS for eight steps at a time
-      v4f af[HALF], bf[HALF];
+      for (int h = 0; h < 2; ++h) {  // operands are fetched from LDS for eight steps at a time
+        v4f af[HALF], bf[HALF];
 #pragma unroll
-      for (int q = 0; q < HALF; ++q) {
-        const int kb = h * HALF + q;
-        af[q] = v4f{0.f, 0.f, 0.f, 0.f};
-        bf[q] = v4f{0.f, 0.f, 0.f, 0.f};
-        if ((unsigned)kb * 8 < Tp) {
-          af[q] = *reinterpret_cast<const v4f*>(pa + kb * 8);
+        for (int q = 0; q < HALF; ++q) {
+          const int kb = h * HALF + q;
+          af[q] = v4f{0.f, 0.f, 0.f, 0.f};
+          bf[q] = v4f{0.f, 0.f, 0.f, 0.f};
+          if ((unsigned)kb * 8 < Tp) {
+            af[q] = *reinterpret_cast<const v4f*>(pa + kb * 8);
 #pragma unroll
-          for (int s = 0; s < 4; ++s) bf[q][s] = vb[(kb * 8 + s) * kPitchV];
+            for (int s = 0; s < 4; ++s) bf[q][s] = vb[(kb * 8 + s) * kPitchV];
+          }
+        }
+#pragma unroll
+        for (int q = 0; q < HALF; ++q) {
+          if ((unsigned)(h * HALF + q) * 8 < Tp) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[q][s], bf[q][s], acc, 0, 0, 0);
+          }
         }
       }
+      const unsigned col = 32 * wn + lrow;
+      if (s0 + 32 * wm + 32 <= S && 32u * wn + 32 <= D && p.ldo < (1u << 24)) {
+        // a whole 32 x 32 block: a register per lane (row 4g, column lrow), a scalar per row, no checks
+        const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(
+            O + (size_t)(s0 + 32 * wm) * p.ldo + 32 * wn, 0, 0x7fffffff, 0x00020000);
+        const unsigned voff = ((4 * g) * p.ldo + lrow) * 4u;
 #pragma unroll
-      for (int q = 0; q < HALF; ++q) {
-        if ((unsigned)(h * HALF + q) * 8 < Tp) {
+        for (int r = 0; r < 16; ++r) {
+          const float value = acc[r];  // a copy: __builtin_bit_cast applied to a vector element reads element 0
+          __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, value), ro, voff,
+                                                (8 * (r / 4) + (r & 3)) * p.ldo * 4u, 0);
+        }
+      } else if (col < D) {
 #pragma unroll
-          for (int s = 0; s < 4; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(af[q][s], bf[q][s], acc, 0, 0, 0);
+        for (int r = 0; r < 16; ++r) {
+          const unsigned row = s0 + 32 * wm + 8 * (r / 4) + 4 * g + (r & 3);
+          if (row < S) O[(size_t)row * p.ldo + col] = acc[r];
         }
       }
     }
-    const unsigned col = 32 * wn + lrow;
-    if (s0 + 32 * wm + 32 <= S && 32u * wn + 32 <= D && p.ldo < (1u << 24)) {
-      // a whole 32 x 32 block: a register per lane (row 4g, column lrow), a scalar per row, no checks
-      const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(
-          O + (size_t)(s0 + 32 * wm) * p.ldo + 32 * wn, 0, 0x7fffffff, 0x00020000);
-      const unsigned voff = ((4 * g) * p.ldo + lrow) * 4u;
+  } else {
+    // ---- probabilities x V.  A product of its own sums each element in one accumulator over k in the order
+    // 8kb + s, 8kb + 4 + s (s = 0..3) with 32x32x2 matrix ops; the 16x16x4 op adds its four k values to the accumulator
+    // one after the other in lane-group order, so feeding lane groups 0..3 the k values 8kb + 2h, 8kb + 4 + 2h,
+    // 8kb + 2h + 1, 8kb + 5 + 2h in ops h = 0, 1 gives the same bits - and blocks of 16 x 16 divide the ROWS x D
+    // result evenly among all wavefronts: wavefront w owns rows 16 (w / 2).. and the column blocks 2 (w & 1), 2 (w & 1) + 1.
+  // With 32 rows this keeps all four SIMDs busy (two 32 x 32 blocks would occupy two); with 64 rows it measured a
+  // microsecond slower than the four 32 x 32 blocks above (twice the LDS operand reads, two-way bank conflicts).
+    {
+      constexpr int KB = kMaxT / 8;
+      const int l16 = lane & 15, q = lane >> 4;
+      const int rb = wave >> 1, cb0 = 2 * (wave & 1);
+      const int kq = (q >> 1) + 4 * (q & 1);  // this lane group's k inside a block of eight, op 0 (op 1: + 2)
+      const float* pa = Sc + (16 * rb + l16) * kPitchS + kq;
+      const float* vb = KVs + kq * kPitchV + 16 * cb0 + l16;
+      const bool live[2] = {(unsigned)(16 * cb0) < D, (unsigned)(16 * cb0 + 16) < D};
+      v4f acc[2] = {v4f{0.f, 0.f, 0.f, 0.f}, v4f{0.f, 0.f, 0.f, 0.f}};
+      if (live[0]) {
+        float af[KB][2], bf[2][KB][2];
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const float value = acc[r];  // a copy: __builtin_bit_cast applied to a vector element reads element 0
-        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, value), ro, voff,
-                                              (8 * (r / 4) + (r & 3)) * p.ldo * 4u, 0);
-      }
-    } else if (col < D) {
+        for (int kb = 0; kb < KB; ++kb) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const unsigned row = s0 + 32 * wm + 8 * (r / 4) + 4 * g + (r & 3);
-        if (row < S) O[(size_t)row * p.ldo + col] = acc[r];
+          for (int h = 0; h < 2; ++h) {
+            af[kb][h] = 0.f; bf[0][kb][h] = 0.f; bf[1][kb][h] = 0.f;
+          }
+          if ((unsigned)kb * 8 < Tp) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+              af[kb][h] = pa[kb * 8 + 2 * h];
+              bf[0][kb][h] = vb[(kb * 8 + 2 * h) * kPitchV];
+              bf[1][kb][h] = vb[(kb * 8 + 2 * h) * kPitchV + 16];  // columns past D hold zeros
+            }
+          }
+        }
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+          if ((unsigned)kb * 8 < Tp) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+              acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[kb][h], bf[0][kb][h], acc[0], 0, 0, 0);
+              acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[kb][h], bf[1][kb][h], acc[1], 0, 0, 0);
+            }
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+          if (!live[j]) continue;
+          const unsigned c0 = 16 * (cb0 + j), r0 = s0 + 16 * rb;
+          if (r0 + 16 <= S && c0 + 16 <= D && p.ldo < (1u << 24)) {
+            // a whole 16 x 16 block: a register per lane (row 4q, column l16), a scalar per row, no checks
+            const __amdgpu_buffer_rsrc_t ro =
+                __builtin_amdgcn_make_buffer_rsrc(O + (size_t)r0 * p.ldo + c0, 0, 0x7fffffff, 0x00020000);
+            const unsigned voff = ((4 * q) * p.ldo + l16) * 4u;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const float value = acc[j][r];  // a copy: __builtin_bit_cast applied to a vector element reads element 0
+              __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(unsigned, value), ro, voff, r * p.ldo * 4u, 0);
+            }
+          } else if (c0 + l16 < D) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const unsigned row = r0 + 4 * q + r;
+              if (row < S) O[(size_t)row * p.ldo + c0 + l16] = acc[j][r];
+            }
+          }
+        }
       }
     }
   }
@@ -561,7 +638,27 @@ extern "C" int tfcc_rocm_attention_f32(void* stream, const tfcc_rocm_attention_d
   p.outerQ = d->stride_q; p.outerK = d->stride_k; p.outerV = d->stride_v; p.outerO = d->stride_out;
   p.innerQ = d->inner_stride_q; p.innerK = d->inner_stride_k; p.innerV = d->inner_stride_v; p.innerO = d->inner_stride_out;
   p.batchInner = d->batch_inner;
-  p.blocksS = (d->s + kRows - 1) / kRows;
+  // up to 128 keys: the scores of a row block in one piece; beyond: blocks of 128 keys with a running maximum and sum
+  const bool stream128 = d->t > (unsigned)kMaxT;
+  int cus = 0;
+  {
+    int dev = 0;
+    TFCC_HIP_CHECK(hipGetDevice(&dev));
+    static int cuCount[16] = {};
+    TFCC_REQUIRE(dev >= 0 && dev < 16, "device index %d", dev);
+    if (!cuCount[dev]) TFCC_HIP_CHECK(hipDeviceGetAttribute(&cuCount[dev], hipDeviceAttributeMultiprocessorCount, dev));
+    cus = cuCount[dev];
+  }
+  // A CU works through its blocks roughly one after the other (two resident workgroups overlap little: 19.1 us for
+  // 384 blocks of 64 rows against 12.7 for 192), so what counts is the largest number of rows any CU gets; a block of
+  // 32 rows costs about 0.55 of a block of 64 (K and V are loaded per block).  16 x 12 heads of 128 rows: 17.8 against
+  // 19.1 us with 32 rows; 32 x 12 heads: 30.5 against 27.7, so those keep 64.
+  const unsigned long long heads = (unsigned long long)d->batch_outer * d->batch_inner;
+  const unsigned long long blocks64 = (d->s + 63) / 64 * heads, blocks32 = (d->s + 31) / 32 * heads;
+  const unsigned long long perCu64 = (blocks64 + cus - 1) / cus, perCu32 = (blocks32 + cus - 1) / cus;
+  const bool rows32 = !stream128 && perCu32 * 55 < perCu64 * 100;
+  const unsigned rowsPerBlock = rows32 ? 32 : kRows;
+  p.blocksS = (d->s + rowsPerBlock - 1) / rowsPerBlock;
   const unsigned long long total = (unsigned long long)p.blocksS * d->batch_outer * d->batch_inner;
   TFCC_REQUIRE(total < (1ull << 31) - 8, "attention: too many blocks");
   p.total = (unsigned)total;
@@ -571,22 +668,25 @@ extern "C" int tfcc_rocm_attention_f32(void* stream, const tfcc_rocm_attention_d
   p.mask = d->mask;
   p.outerM = d->stride_mask;
   p.innerM = d->inner_stride_mask;
-  // up to 128 keys: the scores of a row block in one piece; beyond: blocks of 128 keys with a running maximum and sum
-  const bool stream128 = d->t > (unsigned)kMaxT;
   constexpr size_t ldsBytes = (size_t)(kLdsFloats + 2 * kRows) * sizeof(float);
   static_assert(ldsBytes <= 80 * 1024, "two workgroups per CU");
+  constexpr size_t ldsBytes32 = (size_t)(kMaxT * kPitchV + 32 * kPitchS) * sizeof(float);
+  static_assert(3 * ldsBytes32 <= 160 * 1024, "three workgroups per CU");
   static bool attrSet[16] = {};
   int dev = 0;
   TFCC_HIP_CHECK(hipGetDevice(&dev));
   TFCC_REQUIRE(dev >= 0 && dev < 16, "device index %d", dev);
   if (!attrSet[dev]) {
-    TFCC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_kernel),
+    TFCC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_kernel<64>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes));
+    TFCC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_kernel<32>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes32));
     TFCC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_stream_kernel),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes));
     attrSet[dev] = true;
   }
   if (stream128) hipLaunchKernelGGL(attention_stream_kernel, dim3(p.chunk * 8), dim3(kThreads), ldsBytes, as_stream(stream), p);
-  else hipLaunchKernelGGL(attention_kernel, dim3(p.chunk * 8), dim3(kThreads), ldsBytes, as_stream(stream), p);
+  else if (rows32) hipLaunchKernelGGL(attention_kernel<32>, dim3(p.chunk * 8), dim3(256), ldsBytes32, as_stream(stream), p);
+  else hipLaunchKernelGGL(attention_kernel<64>, dim3(p.chunk * 8), dim3(kThreads), ldsBytes, as_stream(stream), p);
   return check_launch("attention");
 }

@@ -230,7 +230,7 @@ __global__ __launch_bounds__(64 * WGM * KSPLIT > 256 ? 64 * WGM * KSPLIT : 256) 
   // per instruction (two offsets of up to 255 words from one register: a register per stage, k step and half step).
   typedef const __attribute__((address_space(3))) float* LdsFloats;
   typedef const __attribute__((address_space(3))) w96_v4f* LdsQuads;
-  constexpr bool PAIRED = STAGES * KS * 2 <= 8;
+  constexpr bool PAIRED = STAGES * KS * 2 <= (NI <= 2 ? 12 : 8);
   unsigned aAddr[KS], bAddr[PAIRED ? STAGES : 1][KS][2];
 #pragma unroll
   for (int kb = 0; kb < KS; ++kb) {
@@ -478,7 +478,13 @@ int sgemm_wave96_launch(hipStream_t stream, SgemmParams p, int ksplit, int block
     const unsigned long long tiles =
         (unsigned long long)((p.M + 31) / 32) * ((p.N + 32 * blocks - 1) / (32 * blocks)) * p.batch;
     if (blocks == 3) return tiles > 512 ? launch_wave96<1, 4, 8, 3, 3>(stream, p) : launch_wave96<1, 4, 16, 2, 3>(stream, p);
-    if (blocks == 2) return tiles > 512 ? launch_wave96<1, 4, 8, 3, 2>(stream, p) : launch_wave96<1, 4, 16, 2, 2>(stream, p);
+    // 64 columns, at most one tile per CU (128 x 768 x 3072): a third slab in the ring.  Two leave a slab's copies
+    // one slab of matrix ops (0.4 us) to land, less than a trip to HBM: 11.1 -> 9.8 us with operands that come from
+    // HBM, 8.1 -> 8.3 us with operands in cache; four and six slabs ask for so much at once that the first slab
+    // lands later (10.2, 11.1 us), and slabs of 8 k read A in 32-byte pieces (12.2 us).  No gain with 96 columns.
+    if (blocks == 2)
+      return tiles > 512 ? launch_wave96<1, 4, 8, 3, 2>(stream, p)
+                         : tiles <= 256 ? launch_wave96<1, 4, 16, 3, 2>(stream, p) : launch_wave96<1, 4, 16, 2, 2>(stream, p);
     if (blocks == 1) return launch_wave96<1, 4, 8, 3, 1>(stream, p);
   }
   if (ksplit == 1 && blocks == 3) return launch_wave96<4, 1, 32, 2, 3>(stream, p);
