@@ -844,6 +844,28 @@ def main():
     result["roofline"]["burst"] = {"steps": 20, "warmup": 5, "idle_before_s": 0.5, "kernel_ms": round(ms, 5),
                                    "achieved": round(ops / ms / 1e9, 2), "frac": round(ops / ms / 1e9 / PEAK_INT8_TOPS, 4)}
 
+    # The same kernel, the same launch and the same instruction stream on operands of other statistics: what it does
+    # per second depends on how many operand bits change from one matrix op to the next, i.e. on power.  The
+    # headline keeps the uniform operands its configuration prescribes; these legs are evidence, not results.
+    rng_alt = np.random.default_rng(7)
+    alt_sets = {
+        # a quantized bell curve: activations around the zero point 128, weights around 0 (sigma 12 codes each)
+        "quantized_normal_sigma12": (np.clip(np.rint(rng_alt.normal(128.0, 12.0, (size, size))), 0, 255).astype(np.uint8),
+                                     np.clip(np.rint(rng_alt.normal(0.0, 12.0, (size, size))), -127, 127).astype(np.int8)),
+        # every element the same: no operand bit ever changes
+        "constant": (np.full((size, size), 131, dtype=np.uint8), np.full((size, size), 3, dtype=np.int8)),
+    }
+    alt_out = {}
+    for label, (a_alt, b_alt) in alt_sets.items():
+        ta_alt, tb_alt = torch.from_numpy(a_alt).to(dev), torch.from_numpy(b_alt).to(dev)
+        rs_alt, cs_alt = pkg.reduce_sum(ta_alt, True), pkg.reduce_sum(tb_alt, False)
+        step_alt = make_c3_step(torch, pkg, ta_alt, tb_alt, rs_alt, cs_alt, ranges, out_range, want_acc=False)
+        ms, watt = timed_with_power(step_alt, 3000, 500)
+        alt_out[label] = {"kernel_ms": round(ms, 5), "tops": round(ops / ms / 1e9, 2),
+                          "frac_of_peak": round(ops / ms / 1e9 / PEAK_INT8_TOPS, 4), **watt}
+        del step_alt, ta_alt, tb_alt
+    result["roofline"]["same_kernel_other_operands"] = alt_out
+
     # What the matrix cores sustain with nothing else in the way: register-resident instruction loops of the
     # headline's op count, each with the clock and power read while it runs.
     #   constant / changing operands   four accumulators per wavefront, 2 x 4 wavefronts per CU

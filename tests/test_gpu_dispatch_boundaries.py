@@ -243,3 +243,24 @@ def test_sgemm_wavefront_kernel_with_one_two_and_four_column_blocks(pkg, T, m, n
                                               tres.data_ptr(), 0, out.data_ptr(), 0, m, n, k, 1, 1))
     separate = T.n(pkg.gelu_accurate(pkg.add(pkg.blas_matmul(ta, tb, tbias), tres)))
     assert np.array_equal(T.n(out), separate)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("batch,m,n,k", [
+    # many small products: 128 x 128 tiles only where they would be mostly result (512 of them and three quarters full)
+    (768, 64, 64, 64), (512, 64, 128, 64), (600, 100, 100, 96), (512, 112, 112, 32), (520, 128, 128, 64), (130, 250, 250, 64),
+])
+def test_batched_small_products_pick_tiles_that_they_fill(pkg, T, batch, m, n, k):
+    print("batched sgemm", batch, m, n, k, flush=True)
+    rng = np.random.default_rng(batch + m * 3 + n * 5 + k)
+    a = rng.normal(0, 1, (batch, m, k)).astype(np.float32)
+    b = rng.normal(0, 1, (batch, k, n)).astype(np.float32)
+    want = np.matmul(a.astype(np.float64), b.astype(np.float64))
+    got = T.n(pkg.blas_matmul(T.t(a), T.t(b)))
+    assert got.shape == want.shape and rel_fro(got, want) <= FP32_TOL
+    assert np.abs(got - want).max() <= 1e-4 * max(1.0, np.abs(want).max())
+    # the same bits as each product on its own: with K this short every kernel sums an element in one group over
+    # ascending k, whatever its tiles
+    for i in (0, batch // 2, batch - 1):
+        alone = T.n(pkg.blas_matmul(T.t(a[i]), T.t(b[i])))
+        assert np.array_equal(alone, got[i])

@@ -454,9 +454,16 @@ void choose_dma_tiles(unsigned m, unsigned n, unsigned k, unsigned fillBatch, in
 // The number of K groups the kernels for B as stored [k, n] would sum this product with (the sums of an element
 // are defined by it, not by the tile shape): B given transposed must use the same, so that transposing B first
 // and multiplying give the same bits as multiplying the transposed view.
-int k_groups_of_plain_product(unsigned m, unsigned n, unsigned k, unsigned fillBatch) {
+// 128 x 128 tiles: once there are enough of them to fill the 256 CUs twice over, and only when they are mostly
+// result (a batch of 768 products of 64 x 64 x 64 counts 768 such tiles, each three quarters empty: 23 us in them
+// against 11 in 64 x 64 tiles).
+bool takes_128_tiles(unsigned m, unsigned n, unsigned fillBatch) {
   const unsigned long long big = (unsigned long long)((m + 127) / 128) * ((n + 127) / 128) * fillBatch;
-  if (big >= 512) return 1;
+  return big >= 512 && (unsigned long long)m * n * fillBatch * 100 >= big * (128 * 128) * 75;
+}
+
+int k_groups_of_plain_product(unsigned m, unsigned n, unsigned k, unsigned fillBatch) {
+  if (takes_128_tiles(m, n, fillBatch)) return 1;
   if (k % 32 == 0) {
     int best, ksplit;
     unsigned long long tiles;
@@ -494,11 +501,10 @@ int dispatch(hipStream_t s, const SgemmParams& p, bool vec, bool tb, unsigned fi
   // kernel reproduces bit for bit.
   if (fillBatch == 1 && sgemm_detail::sgemv_supported(p)) return sgemm_detail::sgemv_launch(s, p);
   // 128x128 tiles once there are enough of them to fill the 256 CUs twice over, else 64x64
-  const unsigned long long big = (unsigned long long)((m + 127) / 128) * ((n + 127) / 128) * fillBatch;
   if (vec) {
     // (whole slabs of K: four hand-scheduled wavefronts of 32 x 128 on a shared ring, two workgroups per CU -
     // 4096^3: 150 TFLOP/s against 141 for the same tiles scheduled by the compiler)
-    if (big >= 512) return k % 32 == 0 ? sgemm_detail::sgemm_wave96_launch(s, p, 1, 4) : launch<4, 1, 1, 4, true>(s, p);
+    if (takes_128_tiles(m, n, fillBatch)) return k % 32 == 0 ? sgemm_detail::sgemm_wave96_launch(s, p, 1, 4) : launch<4, 1, 1, 4, true>(s, p);
     // few 64x64 tiles and a long K: several K groups per workgroup keep the CUs that have a tile busy
     const unsigned long long small = (unsigned long long)((m + 63) / 64) * ((n + 63) / 64) * fillBatch;
     // 32x96 tiles when they cover the 256 CUs in fewer tile-area rounds than 64x64 tiles would
