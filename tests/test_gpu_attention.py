@@ -153,6 +153,7 @@ LONG_CASES = [
     (1, 2, 100, 512, 36, 6.0, "bhsd"),      # four whole blocks, head width not a multiple of 8
     (2, 2, 9, 300, 8, None, "bhsd"),        # ragged last block, no divisor
     (1, 1, 200, 1000, 64, 8.0, "bshd"),     # eight blocks
+    (5, 10, 256, 200, 64, 8.0, "bshd"),     # 400 blocks of 32 query rows are more than the GPU has CUs: blocks of 64 (the cases above run as blocks of 32)
 ]
 
 

@@ -368,7 +368,10 @@ __global__ __launch_bounds__(8 * ROWS, ROWS == 64 ? 4 : 3) void attention_kernel
 // not against the final one): results agree with them to a few units in the last place, not bit for bit; the
 // contract checked is the relative error against double precision.  Blocks of 128 keep the LDS footprint of the
 // kernel above (two workgroups per CU) whatever the length.
-__global__ __launch_bounds__(kThreads) void attention_stream_kernel(const AttentionParams p) {
+template <int ROWS>
+__global__ __launch_bounds__(8 * ROWS) void attention_stream_kernel(const AttentionParams p) {
+  constexpr int kRows = ROWS, kThreads = 8 * ROWS;  // blocks of 64 or 32 query rows, as in attention_kernel
+  static_assert(ROWS == 64 || ROWS == 32, "two or one row blocks of 32");
   extern __shared__ __align__(16) float lds[];
   float* KVs = lds;                       // the block's K as [128][kPitchK], then its V as [128][kPitchV]
   float* Sc = KVs + kMaxT * kPitchV;      // [64][kPitchS]  scores, then probabilities of the block
@@ -393,8 +396,8 @@ __global__ __launch_bounds__(kThreads) void attention_stream_kernel(const Attent
   const float* __restrict__ mrow = masked ? p.mask + (size_t)bo * p.outerM + (size_t)bn * p.innerM : nullptr;
   const int lrow = lane & 31, g = lane >> 5;
   const unsigned Dp = (D + 7u) & ~7u;
-  const int wmS = wave >> 2, wnS = wave & 3;  // scores: 2 x 4 wavefronts, one 32 x 32 block each
-  const int wm = wave >> 1, wn = wave & 1;    // second product: the first four wavefronts, 2 x 2 blocks of 32 x 32
+  const int wmS = wave >> 2, wnS = wave & 3;  // scores: ROWS / 32 x 4 wavefronts, one 32 x 32 block each
+  const int wm = wave >> 1, wn = wave & 1;    // second product: the first half of the wavefronts, ROWS / 32 x 2 blocks of 32 x 32
   constexpr int CH = kMaxD / 4;
   constexpr int KV_ITEMS = kMaxT * CH / kThreads, Q_ITEMS = kRows * CH / kThreads, KBQ = kMaxD / 8;
   constexpr unsigned kPastEnd = 0xfffffff0u;
@@ -430,25 +433,41 @@ __global__ __launch_bounds__(kThreads) void attention_stream_kernel(const Attent
   float mrun[R], lrun[R];
 #pragma unroll
   for (int u = 0; u < R; ++u) { mrun[u] = -FLT_MAX; lrun[u] = 0.f; }
+  // context accumulators: one 32 x 32 block per wavefront of the first half (ROWS = 64), or two 16 x 16 blocks per
+  // wavefront of all four (ROWS = 32: rows 16 (wave / 2).., column blocks 2 (wave & 1) and 2 (wave & 1) + 1; see
+  // attention_kernel for the order the k values are fed in)
   v16f acc;
 #pragma unroll
   for (int r = 0; r < 16; ++r) acc[r] = 0.f;
+  v4f acc16[2] = {v4f{0.f, 0.f, 0.f, 0.f}, v4f{0.f, 0.f, 0.f, 0.f}};
+  const int l16 = lane & 15, q16 = lane >> 4, rb16 = wave >> 1, cb16 = 2 * (wave & 1);
+  const int kq16 = (q16 >> 1) + 4 * (q16 & 1);
 
   const float divisor = p.divisor;
   const unsigned dbits = __builtin_bit_cast(unsigned, divisor), dexpo = (dbits >> 23) & 0xffu;
   const bool divideByMul = (dbits & 0x007fffffu) == 0 && dexpo >= 2 && dexpo <= 252;  // a power of two: exact
   const float inverseDivisor = 1.0f / divisor;
 
-  for (unsigned t0 = 0; t0 < T; t0 += kMaxT) {
-    const unsigned Tb = min((unsigned)kMaxT, T - t0);   // keys of this block
-    const unsigned Tbp = (Tb + 7u) & ~7u;                // k extent of the block's second product
-    v4f kreg[KV_ITEMS], vreg[KV_ITEMS];
+  // With blocks of 32 rows (every workgroup alone on its CU) K of a block is asked for one block ahead, into the
+  // registers that the block before has just emptied into LDS, so that only the first block waits for its keys; with
+  // blocks of 64 rows two workgroups per CU cover each other's waits and the registers are worth more (1 % slower).
+  constexpr bool kAhead = ROWS == 32;
+  v4f kreg[KV_ITEMS];
+  auto fetchK = [&](unsigned t0) {
+    const unsigned Tb = min((unsigned)kMaxT, T - t0);
 #pragma unroll
     for (int it = 0; it < KV_ITEMS; ++it) {
       const unsigned w = tid + it * kThreads, row = w / CH, ch = w % CH;
       const bool in = row < Tb && ch * 4 < D;
       kreg[it] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rk, in ? ((t0 + row) * p.ldk + ch * 4) * 4u : kPastEnd, 0, 0));
     }
+  };
+  if constexpr (kAhead) fetchK(0);
+  for (unsigned t0 = 0; t0 < T; t0 += kMaxT) {
+    const unsigned Tb = min((unsigned)kMaxT, T - t0);   // keys of this block
+    const unsigned Tbp = (Tb + 7u) & ~7u;                // k extent of the block's second product
+    v4f vreg[KV_ITEMS];
+    if constexpr (!kAhead) fetchK(t0);
     float mk[2] = {0.f, 0.f};
     if (masked) {
 #pragma unroll
@@ -467,6 +486,9 @@ __global__ __launch_bounds__(kThreads) void attention_stream_kernel(const Attent
       const unsigned w = tid + it * kThreads, row = w / CH, ch = w % CH;
       const bool in = row < Tb && ch * 4 < D;
       vreg[it] = __builtin_bit_cast(v4f, __builtin_amdgcn_raw_buffer_load_b128(rv, in ? ((t0 + row) * p.ldv + ch * 4) * 4u : kPastEnd, 0, 0));
+    }
+    if constexpr (kAhead) {
+      if (t0 + kMaxT < T) fetchK(t0 + kMaxT);
     }
     __syncthreads();
 
@@ -555,7 +577,43 @@ __global__ __launch_bounds__(kThreads) void attention_stream_kernel(const Attent
     __syncthreads();
 
     // ---- accumulated rows scaled, then the block's probabilities x V
-    if (wave < 4 && (unsigned)(32 * wn) < D) {
+    if constexpr (ROWS == 32) {
+      if ((unsigned)(16 * cb16) < D) {
+        constexpr int KB = kMaxT / 8;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) acc16[j][r] *= rowScale[16 * rb16 + 4 * q16 + r];
+        const float* pa = Sc + (16 * rb16 + l16) * kPitchS + kq16;
+        const float* vb = KVs + kq16 * kPitchV + 16 * cb16 + l16;
+        float af[KB][2], bfv[2][KB][2];
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+#pragma unroll
+          for (int h = 0; h < 2; ++h) {
+            af[kb][h] = 0.f; bfv[0][kb][h] = 0.f; bfv[1][kb][h] = 0.f;
+          }
+          if ((unsigned)kb * 8 < Tbp) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+              af[kb][h] = pa[kb * 8 + 2 * h];
+              bfv[0][kb][h] = vb[(kb * 8 + 2 * h) * kPitchV];
+              bfv[1][kb][h] = vb[(kb * 8 + 2 * h) * kPitchV + 16];  // columns past D hold zeros
+            }
+          }
+        }
+#pragma unroll
+        for (int kb = 0; kb < KB; ++kb) {
+          if ((unsigned)kb * 8 < Tbp) {
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+              acc16[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[kb][h], bfv[0][kb][h], acc16[0], 0, 0, 0);
+              acc16[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[kb][h], bfv[1][kb][h], acc16[1], 0, 0, 0);
+            }
+          }
+        }
+      }
+    } else if (wave < ROWS / 16 && (unsigned)(32 * wn) < D) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[r] *= rowScale[32 * wm + 8 * (r / 4) + 4 * g + (r & 3)];
       constexpr int KB = kMaxT / 8, HALF = KB / 2;
@@ -587,7 +645,18 @@ __global__ __launch_bounds__(kThreads) void attention_stream_kernel(const Attent
   }
 
   // ---- rows divided by their sums and stored (the reciprocals were left behind the scales by the last block)
-  if (wave < 4 && (unsigned)(32 * wn) < D) {
+  if constexpr (ROWS == 32) {
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+      const unsigned col = 16 * (cb16 + j) + l16;
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const int trow = 16 * rb16 + 4 * q16 + r;
+        const unsigned row = s0 + trow;
+        if (row < S && col < D) O[(size_t)row * p.ldo + col] = acc16[j][r] * rowScale[kRows + trow];
+      }
+    }
+  } else if (wave < ROWS / 16 && (unsigned)(32 * wn) < D) {
     const unsigned col = 32 * wn + lrow;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
@@ -656,7 +725,9 @@ extern "C" int tfcc_rocm_attention_f32(void* stream, const tfcc_rocm_attention_d
   const unsigned long long heads = (unsigned long long)d->batch_outer * d->batch_inner;
   const unsigned long long blocks64 = (d->s + 63) / 64 * heads, blocks32 = (d->s + 31) / 32 * heads;
   const unsigned long long perCu64 = (blocks64 + cus - 1) / cus, perCu32 = (blocks32 + cus - 1) / cus;
-  const bool rows32 = !stream128 && perCu32 * 55 < perCu64 * 100;
+  // (Beyond 128 keys a block of 32 rows walks all the keys again and holds one workgroup per SIMD's registers: it
+  // pays only while every block has a CU to itself - 12 heads of 384 rows 25.3 against 28.4 us, 48 heads 70.5 against 54.4.)
+  const bool rows32 = stream128 ? blocks32 <= (unsigned long long)cus : perCu32 * 55 < perCu64 * 100;
   const unsigned rowsPerBlock = rows32 ? 32 : kRows;
   p.blocksS = (d->s + rowsPerBlock - 1) / rowsPerBlock;
   const unsigned long long total = (unsigned long long)p.blocksS * d->batch_outer * d->batch_inner;
@@ -672,6 +743,7 @@ extern "C" int tfcc_rocm_attention_f32(void* stream, const tfcc_rocm_attention_d
   static_assert(ldsBytes <= 80 * 1024, "two workgroups per CU");
   constexpr size_t ldsBytes32 = (size_t)(kMaxT * kPitchV + 32 * kPitchS) * sizeof(float);
   static_assert(3 * ldsBytes32 <= 160 * 1024, "three workgroups per CU");
+  constexpr size_t ldsStream32 = ldsBytes32 + 2 * 32 * sizeof(float);
   static bool attrSet[16] = {};
   int dev = 0;
   TFCC_HIP_CHECK(hipGetDevice(&dev));
@@ -681,11 +753,14 @@ extern "C" int tfcc_rocm_attention_f32(void* stream, const tfcc_rocm_attention_d
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes));
     TFCC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_kernel<32>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes32));
-    TFCC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_stream_kernel),
+    TFCC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_stream_kernel<64>),
                                        hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsBytes));
+    TFCC_HIP_CHECK(hipFuncSetAttribute(reinterpret_cast<const void*>(attention_stream_kernel<32>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, (int)ldsStream32));
     attrSet[dev] = true;
   }
-  if (stream128) hipLaunchKernelGGL(attention_stream_kernel, dim3(p.chunk * 8), dim3(kThreads), ldsBytes, as_stream(stream), p);
+  if (stream128 && rows32) hipLaunchKernelGGL(attention_stream_kernel<32>, dim3(p.chunk * 8), dim3(256), ldsStream32, as_stream(stream), p);
+  else if (stream128) hipLaunchKernelGGL(attention_stream_kernel<64>, dim3(p.chunk * 8), dim3(kThreads), ldsBytes, as_stream(stream), p);
   else if (rows32) hipLaunchKernelGGL(attention_kernel<32>, dim3(p.chunk * 8), dim3(256), ldsBytes32, as_stream(stream), p);
   else hipLaunchKernelGGL(attention_kernel<64>, dim3(p.chunk * 8), dim3(kThreads), ldsBytes, as_stream(stream), p);
   return check_launch("attention");
