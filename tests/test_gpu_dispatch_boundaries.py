@@ -41,10 +41,10 @@ def test_sgemm_around_configuration_thresholds(pkg, T, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [
-    # up to eight rows of A: the streaming kernel.  32 columns per wavefront below N = 8192, 64 from there on;
+    # up to eight rows of A: the streaming kernel.  32 columns per wavefront below N = 10240, 64 from there on;
     # K below, at and past one 64-row chunk per wavefront (16 * 64 = 1024), ragged chunk tails, ragged N edges
     (1, 1, 1), (1, 64, 64), (2, 65, 63), (3, 31, 1000), (4, 4096, 1024), (5, 100, 1025), (8, 3072, 768),
-    (8, 33, 2049), (7, 8192, 96), (8, 8200, 130), (1, 11008, 512), (6, 8191, 70),
+    (8, 33, 2049), (7, 8192, 96), (8, 8200, 130), (1, 11008, 512), (6, 8191, 70), (5, 10240, 96), (3, 10239, 130),
     # nine rows: back on the tiled kernels
     (9, 3072, 768),
 ])

@@ -201,11 +201,12 @@ namespace sgemm_detail {
 
 bool sgemv_supported(const SgemmParams& p) { return p.M >= 1 && p.M <= 8 && p.batch <= 65535u && p.N < (1u << 30); }
 
-// 64 columns per wavefront read B in the longest runs (5.7 TB/s at N = 11008); below 128 such column blocks too
-// few CUs take part, and 32 columns per wavefront with twice the workgroups are faster (17 against 23 us at
-// 4096 x 4096).  The choice depends on N alone, so that a product is summed the same way alone and in a group.
+// 64 columns per wavefront read B in the longest runs (8 x 4096 x 11008: 37 us against 50 with 32 columns); below
+// 160 such column blocks too few CUs take part, and 32 columns per wavefront with twice the workgroups are faster
+// (8 x 4096 x 8192: 30.8 against 36.2 us, 4096 x 4096: 23.4 against 30.1; 16 columns read B in 64-byte pieces and
+// lose: 25.2).  The choice depends on N alone, so that a product is summed the same way alone and in a group.
 int sgemv_launch(hipStream_t stream, const SgemmParams& p) {
-  return p.N >= 8192 ? launch_width<64>(stream, p) : launch_width<32>(stream, p);
+  return p.N >= 10240 ? launch_width<64>(stream, p) : launch_width<32>(stream, p);
 }
 
 }  // namespace sgemm_detail
