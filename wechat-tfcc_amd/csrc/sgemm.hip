@@ -521,6 +521,10 @@ int dispatch(hipStream_t s, const SgemmParams& p, bool vec, bool tb, unsigned fi
       // against 45.9 us for the kernels of sgemm_dma.hip, 128 x 768 x 3072: 8.6 against 11.4 with the operands in
       // cache, 960 x 1024 x 2048: 34.4 against 41.9) ...
       if (ksplit == 4) {
+        // (Tiles of 16 x 96 from 16x16x4 matrix ops - the same bits, 256 tiles instead of 192 for 128 x 768 x 3072 and
+        // a quarter less matrix time - were built and measured: 7.6 against 8.3 us with the operands in cache, 10.1
+        // against 9.8 with them in HBM, where the wait for the first slab and the bytes in flight decide, not the
+        // matrix ops.  The table's tiles keep the product.)
         const int c = kTiles[best].config;
         return sgemm_detail::sgemm_wave96_launch(s, p, 4, c == 0 ? 2 : c == 1 ? 3 : c == 2 ? 2 : 1, c == 0 ? 2 : 1);
       }
