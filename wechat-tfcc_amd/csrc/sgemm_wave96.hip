@@ -56,7 +56,7 @@ __device__ __forceinline__ int a_row_swizzle(int row) {
   return BK == 32 ? (row >> 1) & 7 : BK == 16 ? (row >> 2) & 3 : (row >> 2) & 1;
 }
 
-template <int WGM, int KSPLIT, int BK, int STAGES, bool PLAIN, int NI>
+template <int WGM, int KSPLIT, int BK, int STAGES, bool PLAIN, int NI, bool RAMP>
 __global__ __launch_bounds__(64 * WGM * KSPLIT > 256 ? 64 * WGM * KSPLIT : 256) void sgemm_wave96_kernel(
     const float* hotA, const float* hotB, const float* hotB1, const float* hotB2, unsigned hotM, unsigned hotN,
     unsigned hotK, unsigned hotLda, unsigned hotLdb, unsigned hotBatch, const SgemmParams p) {
@@ -72,6 +72,7 @@ __global__ __launch_bounds__(64 * WGM * KSPLIT > 256 ? 64 * WGM * KSPLIT : 256) 
   constexpr int BN = 32 * NI;       // columns of a tile
   static_assert(BK == 32 || BK == 16 || BK == 8, "ring slabs of 32, 16 or 8 k");
   static_assert(STAGES >= 2, "ring depth");
+  static_assert(!RAMP || (STAGES >= 3 && BK <= 16 && WGM == 1), "the ramp fills the last stage during slab 0's first step");
   constexpr int BM = 32 * WGM;
   constexpr int KS = BK / 8;        // k steps per ring slab
   constexpr int CH = BK / 4;        // 16-byte chunks per A row
@@ -166,9 +167,11 @@ __global__ __launch_bounds__(64 * WGM * KSPLIT > 256 ? 64 * WGM * KSPLIT : 256) 
     dma16s(rsrc, dst, off[c], live ? so : 0u);
   };
 
-  // the first slabs are on their way before anything else is set up
+  // the first slabs are on their way before anything else is set up (RAMP: all but the last stage's, which is asked
+  // for during the first step of slab 0 - what is asked for at the start delays the first slab, 0.4 us per slab
+  // with operands in HBM)
 #pragma unroll
-  for (int s = 0; s < STAGES; ++s)
+  for (int s = 0; s < (RAMP ? STAGES - 1 : STAGES); ++s)
 #pragma unroll
     for (int c = 0; c < COPIES; ++c) issueCopy((unsigned)s, (unsigned)s, c);
 
@@ -281,7 +284,7 @@ __global__ __launch_bounds__(64 * WGM * KSPLIT > 256 ? 64 * WGM * KSPLIT : 256) 
   // and its reads of slab t have returned; with a shared ring a barrier makes that true of the whole group.  Then
   // slab t+1 is complete and visible, and slab t's stage is free: it is refilled with slab t+STAGES while the last
   // step's matrix ops run on operands already in registers.
-  wait_vmcnt<COPIES*(STAGES - 1)>();
+  wait_vmcnt<COPIES*((RAMP ? STAGES - 1 : STAGES) - 1)>();
   if constexpr (SHARED) __syncthreads();
   Ops ops[2];
   ops[0].a = *reinterpret_cast<const w96_v4f*>(gsm + aBase + ((g ^ aSwz) << 4));
@@ -295,7 +298,8 @@ __global__ __launch_bounds__(64 * WGM * KSPLIT > 256 ? 64 * WGM * KSPLIT : 256) 
     const unsigned next = stage + 1 == STAGES ? 0 : stage + 1;
 #pragma unroll
     for (int kb = 0; kb < KS - 1; ++kb)
-      step(kb & 1 ? other : first, kb & 1 ? first : other, stage, kb + 1, fixedStage, false, 0u, 0u);
+      step(kb & 1 ? other : first, kb & 1 ? first : other, stage, kb + 1, fixedStage, RAMP && kb == 0 && t == 0,
+           (unsigned)(STAGES - 1), (unsigned)(STAGES - 1));
     wait_vmcnt<COPIES*(STAGES - 2)>();
     __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0): the reads of slab t have returned
     if constexpr (SHARED) __syncthreads();
@@ -429,7 +433,7 @@ __global__ __launch_bounds__(64 * WGM * KSPLIT > 256 ? 64 * WGM * KSPLIT : 256) 
   }
 }
 
-template <int WGM, int KSPLIT, int BK, int STAGES, int NI = 3>
+template <int WGM, int KSPLIT, int BK, int STAGES, int NI = 3, bool RAMP = false>
 int launch_wave96(hipStream_t stream, SgemmParams p) {
   constexpr int BM = 32 * WGM, BN = 32 * NI;
   constexpr size_t ring = (size_t)KSPLIT * STAGES * (BM + BN) * BK * 4;
@@ -440,8 +444,8 @@ int launch_wave96(hipStream_t stream, SgemmParams p) {
   const bool sameStart = p.batch == 1 || (p.strideA == 0 && p.innerA == 0 && p.strideB == 0 && p.innerB == 0);
   const bool plain = p.groups ? p.groups <= 3 : sameStart;
   TFCC_REQUIRE(p.batch < (1u << 30), "sgemm: batch of %u", p.batch);
-  auto kern = plain ? sgemm_wave96_kernel<WGM, KSPLIT, BK, STAGES, true, NI>
-                    : sgemm_wave96_kernel<WGM, KSPLIT, BK, STAGES, false, NI>;
+  auto kern = plain ? sgemm_wave96_kernel<WGM, KSPLIT, BK, STAGES, true, NI, RAMP>
+                    : sgemm_wave96_kernel<WGM, KSPLIT, BK, STAGES, false, NI, RAMP>;
   static bool attrSet[16][2] = {};  // per device: the attribute belongs to the function on one device
   int dev = 0;
   TFCC_HIP_CHECK(hipGetDevice(&dev));
@@ -482,9 +486,11 @@ int sgemm_wave96_launch(hipStream_t stream, SgemmParams p, int ksplit, int block
     // one slab of matrix ops (0.4 us) to land, less than a trip to HBM: 11.1 -> 9.8 us with operands that come from
     // HBM, 8.1 -> 8.3 us with operands in cache; four and six slabs ask for so much at once that the first slab
     // lands later (10.2, 11.1 us), and slabs of 8 k read A in 32-byte pieces (12.2 us).  No gain with 96 columns.
+    // The third slab is asked for during slab 0's first step, not at the start (RAMP): 8.3 -> 8.1 us in cache, 9.8 ->
+    // 9.75 from HBM.
     if (blocks == 2)
       return tiles > 512 ? launch_wave96<1, 4, 8, 3, 2>(stream, p)
-                         : tiles <= 256 ? launch_wave96<1, 4, 16, 3, 2>(stream, p) : launch_wave96<1, 4, 16, 2, 2>(stream, p);
+                         : tiles <= 256 ? launch_wave96<1, 4, 16, 3, 2, true>(stream, p) : launch_wave96<1, 4, 16, 2, 2>(stream, p);
     if (blocks == 1) return launch_wave96<1, 4, 8, 3, 1>(stream, p);
   }
   if (ksplit == 1 && blocks == 3) return launch_wave96<4, 1, 32, 2, 3>(stream, p);
