@@ -709,7 +709,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-other", action="store_true", help="skip the secondary configs")
     ap.add_argument("--short-legs", action="store_true",
-                    help="secondary configs with the --steps / --warmup given instead of at least 500 / 300 launches "
+                    help="secondary configs with the --steps / --warmup given instead of at least 500 / 300 launches, the "
+                         "headline's settled and matrix-core legs cut to 40 launches, no operand-statistics legs "
                          "(for counter collection; the figures then include the clock ramp)")
     ap.add_argument("--headline-only", action="store_true",
                     help="only the timed launches of the headline kernel (for counter runs): no probes, no settled / "
@@ -822,8 +823,10 @@ def main():
     # The two regimes of the same launch: after a long warm-up, when the clocks have settled under the power limit
     # (with the shader clock and the socket power the driver reports meanwhile), and as a burst of a few launches
     # right after the GPU sat idle (the first launches run at the idle clocks).
-    ms, watt = timed_with_power(step, 4000, 500)
-    result["roofline"]["settled"] = {"steps": 4000, "warmup": 500, "idle_before_s": 0.0, "kernel_ms": round(ms, 5),
+    # (--short-legs: counter collection, where every launch is slow and only the dispatches' counters matter)
+    long_n, long_w = (4000, 500) if not args.short_legs else (40, 10)
+    ms, watt = timed_with_power(step, long_n, long_w)
+    result["roofline"]["settled"] = {"steps": long_n, "warmup": long_w, "idle_before_s": 0.0, "kernel_ms": round(ms, 5),
                                      "achieved": round(ops / ms / 1e9, 2), "frac": round(ops / ms / 1e9 / PEAK_INT8_TOPS, 4)}
     settled_tops = ops / ms / 1e9
     if watt.get("available") is False:
@@ -848,7 +851,9 @@ def main():
     # per second depends on how many operand bits change from one matrix op to the next, i.e. on power.  The
     # headline keeps the uniform operands its configuration prescribes; these legs are evidence, not results.
     rng_alt = np.random.default_rng(7)
-    alt_sets = {
+    # (Left out with --short-legs and with --no-sampler: without clock and power they say little, and a kernel trace of
+    # the run then averages the headline kernel over its prescribed operands only.)
+    alt_sets = {} if (args.short_legs or sampler is None) else {
         # a quantized bell curve: activations around the zero point 128, weights around 0 (sigma 12 codes each)
         "quantized_normal_sigma12": (np.clip(np.rint(rng_alt.normal(128.0, 12.0, (size, size))), 0, 255).astype(np.uint8),
                                      np.clip(np.rint(rng_alt.normal(0.0, 12.0, (size, size))), -127, 127).astype(np.int8)),
@@ -883,12 +888,12 @@ def main():
             ("int8_16x16x64_gemm_order", 2, 2, 256, 64)):
         def probe():
             probe_check(bench_lib().tfcc_bench_probe_mfma(stream0, kind, pattern, blocks, iters, probe_out.data_ptr()))
-        ms, watt = timed_with_power(probe, 4000, 300)
+        ms, watt = timed_with_power(probe, long_n, 300 if not args.short_legs else 10)
         probes[label] = {"tops": round(ops / ms / 1e9, 2), "frac_of_peak": round(ops / ms / 1e9 / PEAK_INT8_TOPS, 4), **watt}
     for sleep, share in ((1, 0.89), (2, 0.80), (4, 0.67), (8, 0.50)):
         def probe():
             probe_check(bench_lib().tfcc_bench_probe_mfma_duty(stream0, sleep, 256, 128, probe_out.data_ptr()))
-        ms, watt = timed_with_power(probe, 3000, 300)
+        ms, watt = timed_with_power(probe, 3000 if not args.short_legs else 40, 300 if not args.short_legs else 10)
         probes["int8_32x32x32_gemm_order_busy_share_%.2f" % share] = {"tops": round(ops / ms / 1e9, 2), **watt}
     result["roofline"]["matrix_cores_alone"] = probes
     result["roofline"]["matrix_cores_alone_constant_operands"] = probes["int8_32x32x32_constant_operands"]["tops"]
