@@ -151,8 +151,14 @@ __global__ __launch_bounds__(kThreads) void qgemm_w4_kernel(const QGemmParams p)
 
   int offA = p.offsetA, offB = p.offsetB;
   float minC = 0.f, maxC = 0.f;
+  // The ranges are read through the scalar cache (the constant address space: they are inputs, nothing in this launch
+  // writes them).  Read as vector loads they would queue up behind the copies above - memory operations of a
+  // wavefront return in the order they were issued - and everything that is worked out from them below would wait
+  // until the first two slabs have landed instead of running while they travel.
+  typedef const __attribute__((address_space(4))) float* ConstFloats;
+  auto uniformLoad = [](const float* ptr) { return *(ConstFloats)(unsigned long long)ptr; };
   if (p.minA) {
-    float mnA = *p.minA, mxA = *p.maxA, mnB = *p.minB, mxB = *p.maxB;
+    float mnA = uniformLoad(p.minA), mxA = uniformLoad(p.maxA), mnB = uniformLoad(p.minB), mxB = uniformLoad(p.maxB);
     qmatmul_offsets(mnA, mxA, mnB, mxB, &offA, &offB);
     qmatmul_range(mnA, mxA, mnB, mxB, &minC, &maxC);
     if (blockIdx.x == 0 && tid == 0) {
@@ -175,7 +181,7 @@ __global__ __launch_bounds__(kThreads) void qgemm_w4_kernel(const QGemmParams p)
   RequantScalars rq;
   if (REQUANT) {
     if (p.minOut) {
-      rq = make_requant_scalars(TFCC_ROCM_S32, TFCC_ROCM_U8, minC, maxC, *p.minOut, *p.maxOut);
+      rq = make_requant_scalars(TFCC_ROCM_S32, TFCC_ROCM_U8, minC, maxC, uniformLoad(p.minOut), uniformLoad(p.maxOut));
     } else {
       rq.inScale = p.inScale; rq.inMin = p.inMin; rq.outScale = p.outScale; rq.outOffset = p.outOffset;
       rq.inLowest = -2147483648LL; rq.outLowest = 0; rq.outHighest = 255; rq.mode = 0; rq.fillValue = 0;
