@@ -69,6 +69,14 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_dma_kernel(cons
   unsigned char* gsm = smem + grp * GROUP_BYTES;
   const unsigned ldsGroup = (unsigned)(size_t)(__attribute__((address_space(3))) unsigned char*)gsm;
 
+  // A launch of these kernels is a few microseconds, so what stands in front of its first copies counts: everything
+  // they need of the argument block is named before the first branch (one round trip to memory instead of one per
+  // basic block), and the divisions of the tile mapping are multiplications by constants the launcher worked out.
+  asm volatile("" ::"s"(p.chunk), "s"(p.tilesTotal), "s"(p.tilesM), "s"(p.tilesN), "s"(p.perBatchMagic),
+               "s"(p.perBatchShift), "s"(p.bandMagic), "s"(p.bandShift), "s"(p.innerMagic), "s"(p.innerShift),
+               "s"(p.batchInner), "s"(p.M), "s"(p.N), "s"(p.K), "s"(p.lda), "s"(p.ldb), "s"(p.groups), "s"(p.A), "s"(p.B),
+               "s"(p.strideA), "s"(p.strideB), "s"(p.innerA), "s"(p.innerB), "s"(p.groupB[0]), "s"(p.groupB[1]), "s"(p.groupB[2]),
+               "s"(p.groupB[3]));
   unsigned tm, tn, bi;
   {
     // consecutive workgroup ids land on different XCDs: hand each XCD a contiguous run of tiles
@@ -77,53 +85,28 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_dma_kernel(cons
     const unsigned L = xcd * p.chunk + slot;
     if (slot >= p.chunk || L >= p.tilesTotal) return;
     const unsigned perBatch = p.tilesM * p.tilesN;
-    bi = L / perBatch;
+    bi = udiv_apply(L, p.perBatchMagic, p.perBatchShift);
     unsigned t = L - bi * perBatch;
     const unsigned band = 4u * p.tilesN;
-    unsigned g = t / band;
+    unsigned g = udiv_apply(t, p.bandMagic, p.bandShift);
     unsigned rowsInBand = min(4u, p.tilesM - g * 4u);
     unsigned r = t - g * band;
-    tm = g * 4u + r % rowsInBand;
-    tn = r / rowsInBand;
+    const unsigned rq = rowsInBand == 4u ? r >> 2 : r / rowsInBand;  // a ragged last band is the rare case
+    tm = g * 4u + (r - rq * rowsInBand);
+    tn = rq;
   }
   const unsigned m0 = tm * BM, n0 = tn * BN;
   const unsigned M = p.M, N = p.N, K = p.K;
-  const unsigned bo = bi / p.batchInner, bn = bi - bo * p.batchInner;
+  const unsigned bo = udiv_apply(bi, p.innerMagic, p.innerShift), bn = bi - bo * p.batchInner;
   const float* A = p.A + (size_t)bo * p.strideA + (size_t)bn * p.innerA;
   const float* B = p.B + (size_t)bo * p.strideB + (size_t)bn * p.innerB;
-  const float* biasPtr = p.bias;
-  float* Cbase = p.C + (size_t)bo * p.strideC + (size_t)bn * p.innerC;
-  if (p.groups) {  // selects, not indexing: the argument block stays in scalar registers
+  if (p.groups)  // selects, not indexing: the argument block stays in scalar registers
     B = bi == 0 ? p.groupB[0] : bi == 1 ? p.groupB[1] : bi == 2 ? p.groupB[2] : p.groupB[3];
-    biasPtr = bi == 0 ? p.groupBias[0] : bi == 1 ? p.groupBias[1] : bi == 2 ? p.groupBias[2] : p.groupBias[3];
-    Cbase = bi == 0 ? p.groupC[0] : bi == 1 ? p.groupC[1] : bi == 2 ? p.groupC[2] : p.groupC[3];
-  }
-  const unsigned lda = p.lda, ldb = p.ldb, ldc = p.ldc;
+  const unsigned lda = p.lda, ldb = p.ldb;
   const v4i rsrcA = make_rsrc(A, ((M - 1) * lda + K) * 4u);
   const v4i rsrcB = make_rsrc(B, ((K - 1) * ldb + N) * 4u);
 
   const int lrow = lane & 31, g = lane >> 5;
-
-  // values needed only in the tile store are fetched now: at the end their latency would be waited for in full
-  const unsigned gcol = n0 + wn * WN + (STRIDED ? lrow : NI * lrow);  // first of this lane's NI columns
-  constexpr unsigned CSTEP = STRIDED ? 32 : 1;                          // from one of them to the next
-  float bv[NI];
-#pragma unroll
-  for (int j = 0; j < NI; ++j) bv[j] = (biasPtr && gcol + j * CSTEP < N) ? biasPtr[gcol + j * CSTEP] : 0.f;
-  constexpr bool EARLY_RESIDUAL = NI != 4;  // short launches on small tiles; a large tile fetches it in the store
-  float rv[EARLY_RESIDUAL ? 16 * NI : 1];
-  if constexpr (EARLY_RESIDUAL) {
-    if (p.residual && grp == 0) {
-      const float* Rp = p.residual + (size_t)bi * p.strideR;
-#pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const unsigned grow = m0 + wm * 32 + 8 * (r / 4) + 4 * g + (r & 3);
-#pragma unroll
-        for (int j = 0; j < NI; ++j)
-          rv[r * NI + j] = (grow < M && gcol + j * CSTEP < N) ? Rp[(size_t)grow * N + gcol + j * CSTEP] : 0.f;
-      }
-    }
-  }
 
   // ---- copy descriptors.  Copy c of a slab is unit u = c * GW + wave of the stage image; LDS slot s
   // (16 bytes) of the A image holds row s / 8, physical chunk s % 8 = logical chunk ^ row_swizzle(row);
@@ -202,6 +185,37 @@ __global__ __launch_bounds__(WGM * WGN * 64 * KSPLIT) void sgemm_dma_kernel(cons
   const unsigned KT = ((K + BK - 1) / BK + KSPLIT - 1) / KSPLIT;
 #pragma unroll
   for (int s = 0; s < STAGES; ++s) issueSlab(s);
+  // (what the tile store needs of the argument block is read from here on, not in front of the copies)
+  const unsigned ldc = p.ldc;
+  const float* biasPtr = p.bias;
+  float* Cbase = p.C + (size_t)bo * p.strideC + (size_t)bn * p.innerC;
+  if (p.groups) {
+    biasPtr = bi == 0 ? p.groupBias[0] : bi == 1 ? p.groupBias[1] : bi == 2 ? p.groupBias[2] : p.groupBias[3];
+    Cbase = bi == 0 ? p.groupC[0] : bi == 1 ? p.groupC[1] : bi == 2 ? p.groupC[2] : p.groupC[3];
+  }
+  // values needed only in the tile store are fetched now, behind the first slabs: at the end their latency would be
+  // waited for in full (memory operations return in the order they were issued, so the wait below also covers the
+  // part of slab 1 that was asked for before these)
+  const unsigned gcol = n0 + wn * WN + (STRIDED ? lrow : NI * lrow);  // first of this lane's NI columns
+  constexpr unsigned CSTEP = STRIDED ? 32 : 1;                          // from one of them to the next
+  float bv[NI];
+#pragma unroll
+  for (int j = 0; j < NI; ++j) bv[j] = (biasPtr && gcol + j * CSTEP < N) ? biasPtr[gcol + j * CSTEP] : 0.f;
+  constexpr bool EARLY_RESIDUAL = NI != 4;  // short launches on small tiles; a large tile fetches it in the store
+  float rv[EARLY_RESIDUAL ? 16 * NI : 1];
+  if constexpr (EARLY_RESIDUAL) {
+    if (p.residual && grp == 0) {
+      const float* Rp = p.residual + (size_t)bi * p.strideR;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const unsigned grow = m0 + wm * 32 + 8 * (r / 4) + 4 * g + (r & 3);
+#pragma unroll
+        for (int j = 0; j < NI; ++j)
+          rv[r * NI + j] = (grow < M && gcol + j * CSTEP < N) ? Rp[(size_t)grow * N + gcol + j * CSTEP] : 0.f;
+      }
+    }
+  }
+
   wait_vmcnt<COPIES*(STAGES - 1)>();
   if constexpr (!PRIVATE_RING) __syncthreads();
   v4f fa[2];

@@ -3,6 +3,7 @@
 #pragma once
 
 #include "common.hpp"
+#include "qgemm_params.hpp"  // UDiv: division by multiply-high
 
 namespace tfcc_rocm {
 namespace sgemm_detail {
@@ -25,6 +26,8 @@ struct SgemmParams {
   float* groupC[4];
   unsigned M, N, K, batch;
   unsigned tilesM, tilesN, tilesTotal, chunk;
+  // division by tilesM * tilesN, by 4 * tilesN and by batchInner as multiply-high and shift (set_tiles)
+  unsigned perBatchMagic, perBatchShift, bandMagic, bandShift, innerMagic, innerShift;
 };
 
 // Fills in the tile counts for BM x BN tiles; false when there are too many tiles for one grid.
@@ -35,6 +38,11 @@ inline bool set_tiles(SgemmParams& p, unsigned bm, unsigned bn) {
   if (total > 0x7fffffffull) return false;
   p.tilesTotal = (unsigned)total;
   p.chunk = (p.tilesTotal + 7) / 8;
+  const UDiv perBatch = udiv_prepare(p.tilesM * p.tilesN), band = udiv_prepare(4u * p.tilesN),
+             inner = udiv_prepare(p.batchInner);
+  p.perBatchMagic = perBatch.magic; p.perBatchShift = perBatch.shift;
+  p.bandMagic = band.magic; p.bandShift = band.shift;
+  p.innerMagic = inner.magic; p.innerShift = inner.shift;
   return true;
 }
 
