@@ -15,6 +15,7 @@
 #include <float.h>
 
 #include "common.hpp"
+#include "qgemm_params.hpp"  // UDiv: division by multiply-high
 
 namespace tfcc_rocm {
 namespace {
@@ -46,7 +47,17 @@ struct AttentionParams {
   int divide;
   const float* mask;  // optional: one value per key column, added to the (divided) scores of every query row
   unsigned long long outerM, innerM;
+  unsigned blocksMagic, blocksShift, innerMagic, innerShift;  // division by blocksS and by batchInner as multiply-high
 };
+
+// Everything the kernels read of the argument block, named before the first branch: one round trip to memory for it
+// instead of one per basic block, at the head of a launch of ten to twenty microseconds.
+#define TFCC_ATTENTION_FETCH_ARGUMENTS(p)                                                                              \
+  asm volatile("" ::"s"(p.Q), "s"(p.K), "s"(p.V), "s"(p.O), "s"(p.S), "s"(p.T), "s"(p.D), "s"(p.ldq), "s"(p.ldk),      \
+               "s"(p.ldv), "s"(p.ldo), "s"(p.outerQ), "s"(p.outerK), "s"(p.outerV), "s"(p.outerO), "s"(p.innerQ),      \
+               "s"(p.innerK), "s"(p.innerV), "s"(p.innerO), "s"(p.batchInner), "s"(p.blocksS), "s"(p.total),           \
+               "s"(p.chunk), "s"(p.divisor), "s"(p.divide), "s"(p.mask), "s"(p.outerM), "s"(p.innerM),                 \
+               "s"(p.blocksMagic), "s"(p.blocksShift), "s"(p.innerMagic), "s"(p.innerShift))
 
 
 // ROWS query rows per workgroup, a wavefront per eight of them: 64 rows (eight wavefronts, 70.7 KB, two workgroups per
@@ -63,10 +74,11 @@ __global__ __launch_bounds__(8 * ROWS, ROWS == 64 ? 4 : 3) void attention_kernel
 
   // consecutive workgroup ids land on different XCDs: the blocks of one head stay on one XCD
   const unsigned wg = blockIdx.x;
+  TFCC_ATTENTION_FETCH_ARGUMENTS(p);
   const unsigned L = (wg & 7u) * p.chunk + (wg >> 3);
   if ((wg >> 3) >= p.chunk || L >= p.total) return;
-  const unsigned bi = L / p.blocksS, blk = L - bi * p.blocksS;
-  const unsigned bo = bi / p.batchInner, bn = bi - bo * p.batchInner;
+  const unsigned bi = udiv_apply(L, p.blocksMagic, p.blocksShift), blk = L - bi * p.blocksS;
+  const unsigned bo = udiv_apply(bi, p.innerMagic, p.innerShift), bn = bi - bo * p.batchInner;
   const unsigned s0 = blk * kRows;
   const unsigned S = p.S, T = p.T, D = p.D;
   const float* __restrict__ Q = p.Q + (size_t)bo * p.outerQ + (size_t)bn * p.innerQ;
@@ -379,10 +391,11 @@ __global__ __launch_bounds__(8 * ROWS) void attention_stream_kernel(const Attent
                                           //      (after the last block: 1 / l)
 
   const unsigned wg = blockIdx.x;
+  TFCC_ATTENTION_FETCH_ARGUMENTS(p);
   const unsigned L = (wg & 7u) * p.chunk + (wg >> 3);
   if ((wg >> 3) >= p.chunk || L >= p.total) return;
-  const unsigned bi = L / p.blocksS, blk = L - bi * p.blocksS;
-  const unsigned bo = bi / p.batchInner, bn = bi - bo * p.batchInner;
+  const unsigned bi = udiv_apply(L, p.blocksMagic, p.blocksShift), blk = L - bi * p.blocksS;
+  const unsigned bo = udiv_apply(bi, p.innerMagic, p.innerShift), bn = bi - bo * p.batchInner;
   const unsigned s0 = blk * kRows;
   const unsigned S = p.S, T = p.T, D = p.D;
   const float* __restrict__ Q = p.Q + (size_t)bo * p.outerQ + (size_t)bn * p.innerQ;
@@ -734,6 +747,9 @@ extern "C" int tfcc_rocm_attention_f32(void* stream, const tfcc_rocm_attention_d
   TFCC_REQUIRE(total < (1ull << 31) - 8, "attention: too many blocks");
   p.total = (unsigned)total;
   p.chunk = (p.total + 7) / 8;
+  const UDiv blocksDiv = udiv_prepare(p.blocksS), innerDiv = udiv_prepare(p.batchInner);
+  p.blocksMagic = blocksDiv.magic; p.blocksShift = blocksDiv.shift;
+  p.innerMagic = innerDiv.magic; p.innerShift = innerDiv.shift;
   p.divisor = d->divisor;
   p.divide = d->has_divisor ? 1 : 0;
   p.mask = d->mask;

@@ -301,6 +301,9 @@ __global__ __launch_bounds__(kPackThreads) void gemv_packed_kernel(const GemvPar
   }
   const unsigned offA = (unsigned)oA, offB = (unsigned)oB;
   const unsigned global = offA * offB * K;
+  // What was asked for at the start is first looked at here: otherwise the compiler widens this column's scale to
+  // double right behind its load, and the wait for that load would stand in front of the stream of B.
+  asm volatile("" : "+v"(eScale), "+v"(eRowsum), "+v"(eColsum));
   if (eActive) {
     unsigned sum = 0, cs = 0;
 #pragma unroll
