@@ -68,6 +68,12 @@ __global__ __launch_bounds__(WGM * WGN * 64, 2) void qgemm_dma_kernel(const QGem
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform, kept in an SGPR
   const int wm = wave / WGN, wn = wave % WGN;
 
+  // What stands in front of the first copies counts in a launch of ten microseconds: everything they need of the
+  // argument block is named before the first branch (one round trip to memory instead of one per basic block), and
+  // the divisions of the tile mapping are multiplications by constants the launcher worked out.
+  asm volatile("" ::"s"(p.chunk), "s"(p.tilesTotal), "s"(p.tilesM), "s"(p.tilesN), "s"(p.perBatchMagic),
+               "s"(p.perBatchShift), "s"(p.bandMagic), "s"(p.bandShift), "s"(p.M), "s"(p.N), "s"(p.K), "s"(p.A), "s"(p.B),
+               "s"(p.strideA), "s"(p.strideB));
   unsigned tm, tn, bi;
   {
     // consecutive workgroup ids go to different XCDs: each XCD gets a contiguous run of tiles,
@@ -77,14 +83,15 @@ __global__ __launch_bounds__(WGM * WGN * 64, 2) void qgemm_dma_kernel(const QGem
     const unsigned L = xcd * p.chunk + slot;
     if (slot >= p.chunk || L >= p.tilesTotal) return;
     const unsigned perBatch = p.tilesM * p.tilesN;
-    bi = L / perBatch;
+    bi = udiv_apply(L, p.perBatchMagic, p.perBatchShift);
     unsigned t = L - bi * perBatch;
     const unsigned band = 4u * p.tilesN;
-    unsigned g = t / band;
+    unsigned g = udiv_apply(t, p.bandMagic, p.bandShift);
     unsigned rowsInBand = min(4u, p.tilesM - g * 4u);
     unsigned r = t - g * band;
-    tm = g * 4u + r % rowsInBand;
-    tn = r / rowsInBand;
+    const unsigned rq = rowsInBand == 4u ? r >> 2 : r / rowsInBand;  // a ragged last band is the rare case
+    tm = g * 4u + (r - rq * rowsInBand);
+    tn = rq;
   }
   const unsigned m0 = tm * BM, n0 = tn * BN;
   const unsigned M = p.M, N = p.N, K = p.K;
@@ -93,29 +100,6 @@ __global__ __launch_bounds__(WGM * WGN * 64, 2) void qgemm_dma_kernel(const QGem
   // buffer descriptors: base, 0 stride, size in bytes, raw 32-bit format; held in SGPRs
   const v4i rsrcA = make_rsrc(A, M * K);
   const v4i rsrcB = make_rsrc(B, K * N);
-
-  int offA = p.offsetA, offB = p.offsetB;
-  float minC = 0.f, maxC = 0.f;
-  if (p.minA) {
-    float mnA = *p.minA, mxA = *p.maxA, mnB = *p.minB, mxB = *p.maxB;
-    qmatmul_offsets(mnA, mxA, mnB, mxB, &offA, &offB);
-    qmatmul_range(mnA, mxA, mnB, mxB, &minC, &maxC);
-    if (blockIdx.x == 0 && tid == 0) {
-      if (p.minC) *p.minC = minC;
-      if (p.maxC) *p.maxC = maxC;
-    }
-  }
-
-  // The caller's row / column sums this thread turns into offset terms after the main loop are fetched now:
-  // at the end their latency would be waited for in full (one tile per CU, nothing to overlap it with).
-  static_assert(BM <= kThreads && BN <= kThreads, "one row sum and one column sum per thread");
-  unsigned rsPre = 0, csPre = 0;
-  {
-    const int* rsA = p.rowsumA + (size_t)bi * p.strideRA;
-    const int* csB = p.colsumB + (size_t)bi * p.strideRB;
-    if (tid < BM && m0 + tid < M) rsPre = (unsigned)rsA[m0 + tid];
-    if (tid < BN && n0 + tid < N) csPre = (unsigned)csB[n0 + tid];
-  }
 
   // ---- per-thread copy descriptors: which 16 bytes of the slab this lane moves in each copy.
   // LDS slot s (16 bytes) of the A image holds row s/8, physical chunk s%8 = logical chunk ^ swzA(row).
@@ -249,6 +233,30 @@ __global__ __launch_bounds__(WGM * WGN * 64, 2) void qgemm_dma_kernel(const QGem
   const unsigned KT = (K + BK - 1) / BK;
 #pragma unroll
   for (int s = 0; s < STAGES; ++s) issueSlab(s);
+  // (everything the tile store needs is worked out and asked for from here on, with the first slabs on their way)
+  int offA = p.offsetA, offB = p.offsetB;
+  float minC = 0.f, maxC = 0.f;
+  if (p.minA) {
+    float mnA = *p.minA, mxA = *p.maxA, mnB = *p.minB, mxB = *p.maxB;
+    qmatmul_offsets(mnA, mxA, mnB, mxB, &offA, &offB);
+    qmatmul_range(mnA, mxA, mnB, mxB, &minC, &maxC);
+    if (blockIdx.x == 0 && tid == 0) {
+      if (p.minC) *p.minC = minC;
+      if (p.maxC) *p.maxC = maxC;
+    }
+  }
+
+  // The caller's row / column sums this thread turns into offset terms after the main loop are fetched now:
+  // at the end their latency would be waited for in full (one tile per CU, nothing to overlap it with).
+  static_assert(BM <= kThreads && BN <= kThreads, "one row sum and one column sum per thread");
+  unsigned rsPre = 0, csPre = 0;
+  {
+    const int* rsA = p.rowsumA + (size_t)bi * p.strideRA;
+    const int* csB = p.colsumB + (size_t)bi * p.strideRB;
+    if (tid < BM && m0 + tid < M) rsPre = (unsigned)rsA[m0 + tid];
+    if (tid < BN && n0 + tid < N) csPre = (unsigned)csB[n0 + tid];
+  }
+
   wait_vmcnt<COPIES*(STAGES - 1)>();
   __syncthreads();
   v4i fa[2][MI], fb[2][NI];
@@ -380,6 +388,9 @@ int launch(hipStream_t stream, QGemmParams p) {
   if (total > 0x7fffffffull) return set_error(TFCC_ROCM_INVALID_ARGUMENT, "quantized matmul: too many tiles");
   p.tilesTotal = (unsigned)total;
   p.chunk = (p.tilesTotal + 7) / 8;
+  const UDiv perBatch = udiv_prepare(p.tilesM * p.tilesN), band = udiv_prepare(4u * p.tilesN);
+  p.perBatchMagic = perBatch.magic; p.perBatchShift = perBatch.shift;
+  p.bandMagic = band.magic; p.bandShift = band.shift;
   constexpr size_t ring = (size_t)STAGES * (BM + BN) * BK;
   constexpr size_t epi = (size_t)(BM + BN) * 4 + (size_t)BM * (BN + 4);
   constexpr size_t lds = ring > epi ? ring : epi;
