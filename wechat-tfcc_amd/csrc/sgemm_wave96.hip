@@ -104,14 +104,18 @@ __global__ __launch_bounds__(64 * WGM * KSPLIT > 256 ? 64 * WGM * KSPLIT : 256) 
     const unsigned chunk = (tilesTotal + 7u) / 8u;
     const unsigned L = xcd * chunk + slot;
     if (slot >= chunk || L >= tilesTotal) return;
-    bi = L / perBatch;
+    // (a division is some thirty instructions in front of the first copies: the common cases - one product, a band
+    // of a power of two of tiles, whole bands - go without)
+    const bool oneProduct = tilesTotal == perBatch;
+    bi = oneProduct ? 0u : L / perBatch;
     unsigned t = L - bi * perBatch;
     const unsigned band = 4u * tilesN;
-    unsigned gb = t / band;
+    unsigned gb = (band & (band - 1u)) == 0u ? t >> (unsigned)__builtin_ctz(band) : t / band;
     unsigned rowsInBand = min(4u, tilesM - gb * 4u);
     unsigned r = t - gb * band;
-    tm = gb * 4u + r % rowsInBand;
-    tn = r / rowsInBand;
+    const unsigned rq = rowsInBand == 4u ? r >> 2 : r / rowsInBand;
+    tm = gb * 4u + (r - rq * rowsInBand);
+    tn = rq;
   }
   const unsigned m0 = tm * BM, n0 = tn * BN;
   const unsigned M = hotM, N = hotN, K = hotK;
