@@ -77,6 +77,13 @@ __global__ __launch_bounds__(kThreads) void qgemm_w4_kernel(const QGemmParams p)
   // Everything this prologue needs of the argument block is read before the first branch (one round trip to
   // memory instead of one per basic block); the divisions of the tile mapping are multiplications by constants
   // the launcher worked out.
+  // (every field the prologue and the later blocks read, named before anything is computed from one of them: their
+  // loads leave together)
+  asm volatile("" ::"s"(p.chunk), "s"(p.tilesTotal), "s"(p.tilesM), "s"(p.tilesN), "s"(p.perBatchMagic),
+               "s"(p.perBatchShift), "s"(p.bandMagic), "s"(p.bandShift), "s"(p.M), "s"(p.N), "s"(p.K), "s"(p.A), "s"(p.B),
+               "s"(p.strideA), "s"(p.strideB), "s"(p.offsetA), "s"(p.offsetB), "s"(p.minA), "s"(p.maxA), "s"(p.minB),
+               "s"(p.maxB), "s"(p.minOut), "s"(p.maxOut), "s"(p.rowsumA), "s"(p.colsumB), "s"(p.strideRA),
+               "s"(p.strideRB), "s"(p.strideC), "s"(p.C), "s"(p.Q));
   unsigned tm, tn, bi;
   bool inGrid;
   {
@@ -97,9 +104,6 @@ __global__ __launch_bounds__(kThreads) void qgemm_w4_kernel(const QGemmParams p)
     tm = gb * 4u + (r - rq * rowsInBand);
     tn = rq;
   }
-  // (the fields the later blocks read: named here so that their loads leave with the first ones)
-  asm volatile("" ::"s"(p.offsetA), "s"(p.offsetB), "s"(p.minA), "s"(p.minOut), "s"(p.rowsumA), "s"(p.colsumB),
-               "s"(p.strideRA), "s"(p.strideRB), "s"(p.strideC), "s"(p.C), "s"(p.Q));
   const unsigned m0 = tm * BM, n0 = tn * BN;
   const unsigned M = p.M, N = p.N, K = p.K;
   const unsigned char* A = p.A + (size_t)bi * p.strideA;
