@@ -258,6 +258,19 @@ __global__ __launch_bounds__(1024) void gemv_wide16_kernel(const signed char* ho
   } else if (!EXACT && j == kOnesRow) {
     a = v4i{0x01010101, 0x01010101, 0x01010101, 0x01010101};
   }
+  // The offsets that ranges in device memory stand for (two divisions in double precision) are worked out here, with
+  // the loads of B under way, not behind the barrier in front of the finish; the ranges were asked for before B, so
+  // waiting for them waits for nothing else.
+  int oA = p.offsetA, oB = p.offsetB;
+  if (p.minA) {
+    qmatmul_offsets(mnA, mxA, mnB, mxB, &oA, &oB);
+    if (cb == 0 && part == 0 && tid == 0) {
+      float mnC, mxC;
+      qmatmul_range(mnA, mxA, mnB, mxB, &mnC, &mxC);
+      if (p.minC) *p.minC = mnC;
+      if (p.maxC) *p.maxC = mxC;
+    }
+  }
   const v4i bias = {(int)kTileBias, (int)kTileBias, (int)kTileBias, (int)kTileBias};
   // what this lane adds to the tile: registers 0, 1 of its result are pair kg of A's rows (for MR = 1 the second one
   // is the column sums, for MR = 4 lane group 2 holds them in register 0); for MR = 8 lane group 0 holds the column
@@ -294,16 +307,6 @@ __global__ __launch_bounds__(1024) void gemv_wide16_kernel(const signed char* ho
   }
   __syncthreads();
 
-  int oA = p.offsetA, oB = p.offsetB;
-  if (p.minA) {
-    qmatmul_offsets(mnA, mxA, mnB, mxB, &oA, &oB);
-    if (cb == 0 && part == 0 && tid == 0) {
-      float mnC, mxC;
-      qmatmul_range(mnA, mxA, mnB, mxB, &mnC, &mxC);
-      if (p.minC) *p.minC = mnC;
-      if (p.maxC) *p.maxC = mxC;
-    }
-  }
   if (!finisher) return;
   // ---- this thread's rows r0 .. r0 + RPT - 1 of column ec: every one of the sixteen wavefronts added its bias
   unsigned sum[RPT];
